@@ -1,0 +1,115 @@
+"""ctypes binding of libdaphne_hip.so (the C ABI declared in include/daphne_hip.h).
+
+Loading fails loudly when the library has not been built: there is no CPU fallback.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from pathlib import Path
+
+LIB_PATH = Path(__file__).resolve().parent / "libdaphne_hip.so"
+
+DH_OK, DH_ERR_RUNTIME, DH_ERR_INVALID_ARG, DH_ERR_DOMAIN, DH_ERR_HIP, DH_ERR_OOM = range(6)
+
+sz = C.c_size_t
+vp = C.c_void_p
+i32 = C.c_int
+
+
+class DaphneHipError(RuntimeError):
+    """std::runtime_error of the reference (bad shapes, unknown op codes, HIP failures)."""
+
+    def __init__(self, status: int, msg: str):
+        super().__init__(msg)
+        self.status = status
+
+
+class DaphneHipInvalidArgument(DaphneHipError, ValueError):
+    """std::invalid_argument of the reference."""
+
+
+class DaphneHipDomainError(DaphneHipError, ArithmeticError):
+    """std::domain_error of the reference (sqrt/ln/asin/acos outside their domain)."""
+
+
+_lib = None
+
+
+def _signatures(lib: C.CDLL) -> None:
+    ctxp = vp
+    lib.dh_last_error.restype = C.c_char_p
+    lib.dh_last_error.argtypes = []
+    lib.dh_ctx_create.argtypes = [i32, C.POINTER(vp)]
+    lib.dh_ctx_destroy.argtypes = [ctxp]
+    lib.dh_ctx_mem_budget.argtypes = [ctxp]
+    lib.dh_ctx_mem_budget.restype = sz
+    lib.dh_ctx_mem_in_use.argtypes = [ctxp]
+    lib.dh_ctx_mem_in_use.restype = sz
+    lib.dh_ctx_device.argtypes = [ctxp]
+    lib.dh_ctx_props.argtypes = [ctxp, C.POINTER(i32), C.POINTER(i32), C.POINTER(sz), C.c_char_p, sz]
+    lib.dh_ctx_set_stream.argtypes = [ctxp, vp]
+    lib.dh_ctx_get_stream.argtypes = [ctxp]
+    lib.dh_ctx_get_stream.restype = vp
+    lib.dh_sync.argtypes = [ctxp]
+    lib.dh_malloc.argtypes = [ctxp, sz, i32, C.POINTER(vp)]
+    lib.dh_free.argtypes = [ctxp, vp]
+    lib.dh_h2d.argtypes = [ctxp, vp, vp, sz]
+    lib.dh_d2h.argtypes = [ctxp, vp, vp, sz]
+    lib.dh_d2d.argtypes = [ctxp, vp, vp, sz]
+    lib.dh_timer_start.argtypes = [ctxp]
+    lib.dh_timer_stop_ms.argtypes = [ctxp, C.POINTER(C.c_float)]
+    for suf, ct in (("f32", C.c_float), ("f64", C.c_double)):
+        f = lambda name: getattr(lib, f"{name}_{suf}")
+        f("dh_ew_binary").argtypes = [ctxp, i32, vp, sz, vp, sz, sz, sz, vp, sz, sz, sz]
+        f("dh_ew_binary_sca").argtypes = [ctxp, i32, vp, sz, vp, sz, sz, sz, ct]
+        f("dh_ew_unary").argtypes = [ctxp, i32, vp, sz, vp, sz, sz, sz]
+        f("dh_agg_all").argtypes = [ctxp, i32, vp, sz, sz, sz, C.POINTER(ct)]
+        f("dh_agg_all_dev").argtypes = [ctxp, i32, vp, sz, sz, sz, vp]
+        f("dh_agg_row").argtypes = [ctxp, i32, vp, sz, vp, sz, sz, sz]
+        f("dh_agg_row_idx").argtypes = [ctxp, i32, vp, sz, vp, sz, sz, sz]
+        f("dh_agg_col").argtypes = [ctxp, i32, vp, vp, sz, sz, sz]
+        f("dh_agg_col_idx").argtypes = [ctxp, i32, vp, vp, sz, sz, sz]
+        for name, at in _LATE_SIGNATURES.items():
+            fn = getattr(lib, f"{name}_{suf}", None)
+            if fn is not None:
+                fn.argtypes = [ct if a == "T" else a for a in at]
+
+
+# Entry points added after the first kernels; bound when the library exports them.
+_LATE_SIGNATURES: dict[str, list] = {
+    "dh_matmul": [vp, vp, sz, vp, sz, sz, sz, vp, sz, sz, sz, i32, i32],
+    "dh_syrk": [vp, vp, sz, vp, sz, sz, sz, i32],
+    "dh_solve": [vp, vp, vp, sz, sz, vp],
+    "dh_conv2d_forward": [vp, vp, C.POINTER(sz), C.POINTER(sz), vp, vp, sz, sz, vp, sz, sz, sz, sz, sz, sz, sz, sz, sz, sz],
+    "dh_maxpool_forward": [vp, vp, C.POINTER(sz), C.POINTER(sz), vp, sz, sz, sz, sz, sz, sz, sz, sz, sz, sz],
+    "dh_affine_forward": [vp, vp, vp, sz, sz, vp, sz, sz, vp, sz, sz],
+    "dh_bias_add": [vp, vp, vp, sz, sz, vp, sz],
+    "dh_batchnorm_inference": [vp, vp, vp, sz, sz, vp, vp, vp, vp, sz, "T", i32],
+    "dh_softmax": [vp, vp, sz, vp, sz, sz, sz],
+}
+
+
+def lib() -> C.CDLL:
+    """Returns the loaded library; raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not LIB_PATH.exists():
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: build it with `python -m daphne_amd.build` "
+                "(there is no CPU fallback for the device kernels)"
+            )
+        _lib = C.CDLL(str(LIB_PATH))
+        _signatures(_lib)
+    return _lib
+
+
+def check(status: int) -> None:
+    """Turns a dh_status into the exception type the reference would throw."""
+    if status == DH_OK:
+        return
+    msg = lib().dh_last_error().decode("utf-8", "replace")
+    if status == DH_ERR_INVALID_ARG:
+        raise DaphneHipInvalidArgument(status, msg)
+    if status == DH_ERR_DOMAIN:
+        raise DaphneHipDomainError(status, msg)
+    raise DaphneHipError(status, msg)

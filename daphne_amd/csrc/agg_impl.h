@@ -1,0 +1,915 @@
+// Aggregation kernels (full, per row, per column, index of row/column extremum) for
+// DenseMatrix<float|double>; instantiated per value type by agg_f32.hip / agg_f64.hip.
+//
+// Semantics follow the reference's CPU kernels:
+//   AggAll  runtime/local/kernels/AggAll.h:64-96,124-193   (SUM PROD MIN MAX MEAN VAR STDDEV)
+//   AggRow  runtime/local/kernels/AggRow.h:60-161          (+ IDXMIN / IDXMAX at :71-94)
+//   AggCol  runtime/local/kernels/AggCol.h:58-178          (+ IDXMIN / IDXMAX at :70-122)
+// What is kept from them: population variance (divide by N); MIN/MAX built on std::min /
+// std::max, so a NaN never replaces the running value, and the running value of AggRow / AggCol
+// starts at the first element (a NaN there is the result) while AggAll starts at +-inf (NaNs are
+// ignored); IDXMIN / IDXMAX return the first position of the strict extremum and position 0 if
+// the first element is NaN. What differs is only the summation order (trees instead of one
+// sequential chain), which is why floating-point results are compared with a tolerance.
+//
+// Mapping to the hardware: every kernel streams its input once with 16-byte loads, with the
+// lanes of a wavefront on consecutive addresses. Row aggregations give each row to a group of
+// G = 1..64 lanes (a 64-wide f32 row is 16 lanes x float4, four rows per wavefront) and finish
+// with cross-lane shuffles, so a tall-skinny matrix needs neither one block per row nor LDS.
+// Column aggregations give each block a contiguous slab of rows, keep per-column partials in
+// registers, fold the TY row-lanes of the block through LDS and leave one partial row per block
+// for a small second kernel; no atomics, so results are deterministic. Variance per column is
+// computed in the same single pass as (count, mean, M2) triples merged with Chan's formula.
+#pragma once
+
+#include "common.h"
+
+#include <cmath>
+#include <limits>
+
+namespace dh_agg {
+
+constexpr int THREADS = 256;
+constexpr int UNROLL = 4;
+
+template <typename T> struct RSum {
+    static __device__ __forceinline__ T id() { return T(0); }
+    static __device__ __forceinline__ T comb(T a, T b) { return a + b; }
+};
+template <typename T> struct RProd {
+    static __device__ __forceinline__ T id() { return T(1); }
+    static __device__ __forceinline__ T comb(T a, T b) { return a * b; }
+};
+template <typename T> struct RMin {
+    static __device__ __forceinline__ T id() { return std::numeric_limits<T>::infinity(); }
+    static __device__ __forceinline__ T comb(T a, T b) { return (b < a) ? b : a; }
+};
+template <typename T> struct RMax {
+    static __device__ __forceinline__ T id() { return -std::numeric_limits<T>::infinity(); }
+    static __device__ __forceinline__ T comb(T a, T b) { return (a < b) ? b : a; }
+};
+
+template <typename T> __device__ __forceinline__ T dev_sqrt(T a);
+template <> __device__ __forceinline__ float dev_sqrt<float>(float a) { return sqrtf(a); }
+template <> __device__ __forceinline__ double dev_sqrt<double>(double a) { return sqrt(a); }
+template <typename T> __device__ __forceinline__ bool dev_isnan(T a) { return a != a; }
+
+template <typename T, int VEC> __device__ __forceinline__ void load_vec(const T *p, T (&v)[VEC]) {
+    if constexpr (VEC == 1) {
+        v[0] = *p;
+    } else {
+        using V = typename dh_vec<T>::type;
+        V t = *reinterpret_cast<const V *>(p);
+        const T *tp = reinterpret_cast<const T *>(&t);
+#pragma unroll
+        for (int i = 0; i < VEC; i++)
+            v[i] = tp[i];
+    }
+}
+
+template <typename T, class R> __device__ __forceinline__ T wave_reduce(T v) {
+#pragma unroll
+    for (int off = DH_WAVE / 2; off >= 1; off >>= 1)
+        v = R::comb(v, dh_shfl_xor(v, off));
+    return v;
+}
+
+// Reduces over the whole block; the result is valid in thread 0.
+template <typename T, class R> __device__ __forceinline__ T block_reduce(T v) {
+    __shared__ T lds[THREADS / DH_WAVE];
+    const int tid = threadIdx.y * blockDim.x + threadIdx.x;
+    v = wave_reduce<T, R>(v);
+    if ((tid % DH_WAVE) == 0)
+        lds[tid / DH_WAVE] = v;
+    __syncthreads();
+    if (tid == 0) {
+#pragma unroll
+        for (int w = 1; w < THREADS / DH_WAVE; w++)
+            v = R::comb(v, lds[w]);
+    }
+    __syncthreads();
+    return v;
+}
+
+// =======================================================================================
+// AggAll
+// =======================================================================================
+// Stage 1: (TX, TY) walk over rows x cvecs vectors; one partial per block.
+template <typename T, int VEC, class R, bool SQDEV>
+__global__ __launch_bounds__(THREADS) void all_stage1(const T *arg, size_t rows, size_t cvecs, size_t ld,
+                                                      const T *mean_dev, T *partials) {
+    T m = T(0);
+    if constexpr (SQDEV)
+        m = *mean_dev;
+    T acc[VEC];
+#pragma unroll
+    for (int i = 0; i < VEC; i++)
+        acc[i] = R::id();
+    const size_t row_step = static_cast<size_t>(gridDim.x) * blockDim.y;
+    for (size_t cv = static_cast<size_t>(blockIdx.y) * blockDim.x + threadIdx.x; cv < cvecs;
+         cv += static_cast<size_t>(gridDim.y) * blockDim.x) {
+        for (size_t r0 = static_cast<size_t>(blockIdx.x) * blockDim.y + threadIdx.y; r0 < rows;
+             r0 += row_step * UNROLL) {
+            T x[UNROLL][VEC];
+#pragma unroll
+            for (int u = 0; u < UNROLL; u++) {
+                const size_t r = r0 + u * row_step;
+                if (r < rows)
+                    load_vec<T, VEC>(arg + r * ld + cv * VEC, x[u]);
+            }
+#pragma unroll
+            for (int u = 0; u < UNROLL; u++) {
+                const size_t r = r0 + u * row_step;
+                if (r < rows) {
+#pragma unroll
+                    for (int i = 0; i < VEC; i++) {
+                        T v = x[u][i];
+                        if constexpr (SQDEV)
+                            v = (v - m) * (v - m);
+                        acc[i] = R::comb(acc[i], v);
+                    }
+                }
+            }
+        }
+    }
+    T a = acc[0];
+#pragma unroll
+    for (int i = 1; i < VEC; i++)
+        a = R::comb(a, acc[i]);
+    a = block_reduce<T, R>(a);
+    if (threadIdx.x == 0 && threadIdx.y == 0)
+        partials[static_cast<size_t>(blockIdx.y) * gridDim.x + blockIdx.x] = a;
+}
+
+// Stage 2: one block folds the partials. FINAL: 0 as is, 1 divide by count, 2 divide then sqrt.
+template <typename T, class R, int FINAL>
+__global__ __launch_bounds__(THREADS) void all_stage2(const T *partials, size_t np, T *out, T count) {
+    T a = R::id();
+    for (size_t i = threadIdx.x; i < np; i += THREADS)
+        a = R::comb(a, partials[i]);
+    a = block_reduce<T, R>(a);
+    if (threadIdx.x == 0) {
+        if constexpr (FINAL >= 1)
+            a = a / count;
+        if constexpr (FINAL == 2)
+            a = dev_sqrt<T>(a);
+        out[0] = a;
+    }
+}
+
+struct Plan2D {
+    dim3 grid, block;
+    size_t nblocks;
+};
+static inline Plan2D plan2d(const dh_ctx *ctx, size_t rows, size_t cvecs) {
+    unsigned tx = 1;
+    while (tx < THREADS && tx < cvecs)
+        tx <<= 1;
+    unsigned ty = THREADS / tx;
+    size_t gy = dh_ceil_div(cvecs, tx);
+    if (gy > 512)
+        gy = 512;
+    const size_t max_blocks = static_cast<size_t>(ctx->num_cus) * 8;
+    size_t gx = dh_ceil_div(rows, static_cast<size_t>(ty) * UNROLL);
+    size_t cap = max_blocks / gy;
+    if (cap < 1)
+        cap = 1;
+    if (gx > cap)
+        gx = cap;
+    if (gx < 1)
+        gx = 1;
+    Plan2D p;
+    p.grid = dim3(static_cast<unsigned>(gx), static_cast<unsigned>(gy), 1);
+    p.block = dim3(tx, ty, 1);
+    p.nblocks = gx * gy;
+    return p;
+}
+
+// Runs stage 1 over (rows, cols, ld) - flat if contiguous - and returns the number of partials.
+template <typename T, class R, bool SQDEV>
+static inline size_t all_stage1_launch(dh_ctx *ctx, const T *arg, size_t rows, size_t cols, size_t ld,
+                                       const T *mean_dev, T *partials) {
+    constexpr int V = dh_vec<T>::N;
+    size_t np = 0;
+    if (ld == cols || rows == 1) {
+        const size_t n = rows * cols;
+        const size_t width = static_cast<size_t>(THREADS) * V;
+        const size_t body_rows = dh_aligned(arg, 16) ? n / width : 0;
+        if (body_rows) {
+            Plan2D p = plan2d(ctx, body_rows, THREADS);
+            hipLaunchKernelGGL((all_stage1<T, V, R, SQDEV>), p.grid, p.block, 0, ctx->stream, arg, body_rows,
+                               size_t(THREADS), width, mean_dev, partials);
+            np += p.nblocks;
+        }
+        const size_t done = body_rows * width;
+        if (done < n) {
+            Plan2D p = plan2d(ctx, 1, n - done);
+            hipLaunchKernelGGL((all_stage1<T, 1, R, SQDEV>), p.grid, p.block, 0, ctx->stream, arg + done, size_t(1),
+                               n - done, n - done, mean_dev, partials + np);
+            np += p.nblocks;
+        }
+        return np;
+    }
+    const bool vec_ok = (cols % V == 0) && (ld % V == 0) && dh_aligned(arg, 16);
+    if (vec_ok) {
+        Plan2D p = plan2d(ctx, rows, cols / V);
+        hipLaunchKernelGGL((all_stage1<T, V, R, SQDEV>), p.grid, p.block, 0, ctx->stream, arg, rows, cols / V, ld,
+                           mean_dev, partials);
+        np = p.nblocks;
+    } else {
+        Plan2D p = plan2d(ctx, rows, cols);
+        hipLaunchKernelGGL((all_stage1<T, 1, R, SQDEV>), p.grid, p.block, 0, ctx->stream, arg, rows, cols, ld,
+                           mean_dev, partials);
+        np = p.nblocks;
+    }
+    return np;
+}
+
+template <typename T> dh_status agg_all_dev(dh_ctx *ctx, int op, const T *arg, size_t rows, size_t cols, size_t ld, T *out) {
+    DH_REQUIRE_CTX(ctx);
+    if (ld < cols)
+        return dh_fail(DH_ERR_RUNTIME, "AggAll - leading dimension smaller than the column count");
+    if (op == DH_AGG_IDXMIN || op == DH_AGG_IDXMAX || op < 0 || op > DH_AGG_VAR)
+        return dh_fail(DH_ERR_RUNTIME, "unsupported AggOpCode"); // AggAll.h:147,161
+    void *wsv = nullptr;
+    const size_t max_partials = static_cast<size_t>(ctx->num_cus) * 8 * 2 + 1024 + 16;
+    dh_status st = dh_workspace(ctx, (max_partials + 64) * sizeof(T), &wsv);
+    if (st != DH_OK)
+        return st;
+    T *mean_slot = static_cast<T *>(wsv); // first 256 bytes: the mean for the variance pass
+    T *partials = reinterpret_cast<T *>(static_cast<char *>(wsv) + 256);
+    const T count = static_cast<T>(rows * cols);
+    size_t np;
+    switch (op) {
+    case DH_AGG_SUM:
+        np = all_stage1_launch<T, RSum<T>, false>(ctx, arg, rows, cols, ld, nullptr, partials);
+        hipLaunchKernelGGL((all_stage2<T, RSum<T>, 0>), dim3(1), dim3(THREADS), 0, ctx->stream, partials, np, out, count);
+        break;
+    case DH_AGG_PROD:
+        np = all_stage1_launch<T, RProd<T>, false>(ctx, arg, rows, cols, ld, nullptr, partials);
+        hipLaunchKernelGGL((all_stage2<T, RProd<T>, 0>), dim3(1), dim3(THREADS), 0, ctx->stream, partials, np, out, count);
+        break;
+    case DH_AGG_MIN:
+        np = all_stage1_launch<T, RMin<T>, false>(ctx, arg, rows, cols, ld, nullptr, partials);
+        hipLaunchKernelGGL((all_stage2<T, RMin<T>, 0>), dim3(1), dim3(THREADS), 0, ctx->stream, partials, np, out, count);
+        break;
+    case DH_AGG_MAX:
+        np = all_stage1_launch<T, RMax<T>, false>(ctx, arg, rows, cols, ld, nullptr, partials);
+        hipLaunchKernelGGL((all_stage2<T, RMax<T>, 0>), dim3(1), dim3(THREADS), 0, ctx->stream, partials, np, out, count);
+        break;
+    case DH_AGG_MEAN:
+        np = all_stage1_launch<T, RSum<T>, false>(ctx, arg, rows, cols, ld, nullptr, partials);
+        hipLaunchKernelGGL((all_stage2<T, RSum<T>, 1>), dim3(1), dim3(THREADS), 0, ctx->stream, partials, np, out, count);
+        break;
+    case DH_AGG_VAR:
+    case DH_AGG_STDDEV:
+        // Two passes like AggAll.h:165-191: the mean, then the mean squared deviation from it.
+        np = all_stage1_launch<T, RSum<T>, false>(ctx, arg, rows, cols, ld, nullptr, partials);
+        hipLaunchKernelGGL((all_stage2<T, RSum<T>, 1>), dim3(1), dim3(THREADS), 0, ctx->stream, partials, np, mean_slot, count);
+        np = all_stage1_launch<T, RSum<T>, true>(ctx, arg, rows, cols, ld, mean_slot, partials);
+        if (op == DH_AGG_VAR)
+            hipLaunchKernelGGL((all_stage2<T, RSum<T>, 1>), dim3(1), dim3(THREADS), 0, ctx->stream, partials, np, out, count);
+        else
+            hipLaunchKernelGGL((all_stage2<T, RSum<T>, 2>), dim3(1), dim3(THREADS), 0, ctx->stream, partials, np, out, count);
+        break;
+    default:
+        return dh_fail(DH_ERR_RUNTIME, "unsupported AggOpCode");
+    }
+    DH_CHECK_LAUNCH();
+    return DH_OK;
+}
+
+template <typename T> dh_status agg_all(dh_ctx *ctx, int op, const T *arg, size_t rows, size_t cols, size_t ld, T *result_host) {
+    DH_REQUIRE_CTX(ctx);
+    if (result_host == nullptr)
+        return dh_fail(DH_ERR_RUNTIME, "AggAll - result pointer is null");
+    T *slot = reinterpret_cast<T *>(reinterpret_cast<char *>(ctx->flag_dev) + 64);
+    dh_status st = agg_all_dev<T>(ctx, op, arg, rows, cols, ld, slot);
+    if (st != DH_OK)
+        return st;
+    T *host_slot = reinterpret_cast<T *>(reinterpret_cast<char *>(ctx->flag_host) + 64);
+    DH_CHECK_HIP(hipMemcpyAsync(host_slot, slot, sizeof(T), hipMemcpyDeviceToHost, ctx->stream));
+    DH_CHECK_HIP(hipStreamSynchronize(ctx->stream));
+    *result_host = *host_slot;
+    return DH_OK;
+}
+
+// =======================================================================================
+// AggRow
+// =======================================================================================
+// FINAL: 0 plain reduction, 1 mean, 2 var, 3 stddev. G lanes share a row (G a power of two
+// <= 64, G divides 64). NANFIRST: MIN/MAX take a NaN in column 0 as the result (AggRow.h:108).
+template <typename T, int VEC, class R, int FINAL, bool NANFIRST>
+__global__ __launch_bounds__(THREADS) void row_kernel(T *res, size_t ld_res, const T *arg, size_t rows,
+                                                      size_t cols, size_t ld, int G) {
+    const int tid = threadIdx.x;
+    const int lane = tid % G;
+    const size_t rows_per_block = THREADS / G;
+    const size_t cvecs = cols / VEC;
+    for (size_t r = static_cast<size_t>(blockIdx.x) * rows_per_block + tid / G; r < rows;
+         r += static_cast<size_t>(gridDim.x) * rows_per_block) {
+        const T *row = arg + r * ld;
+        T acc = R::id();
+        for (size_t cv = lane; cv < cvecs; cv += G) {
+            T x[VEC];
+            load_vec<T, VEC>(row + cv * VEC, x);
+#pragma unroll
+            for (int i = 0; i < VEC; i++)
+                acc = R::comb(acc, x[i]);
+        }
+        for (int off = G / 2; off >= 1; off >>= 1)
+            acc = R::comb(acc, dh_shfl_xor(acc, off));
+        if constexpr (FINAL >= 1)
+            acc = acc / static_cast<T>(cols);
+        if constexpr (FINAL >= 2) {
+            const T mean = acc;
+            T s = T(0);
+            for (size_t cv = lane; cv < cvecs; cv += G) {
+                T x[VEC];
+                load_vec<T, VEC>(row + cv * VEC, x);
+#pragma unroll
+                for (int i = 0; i < VEC; i++) {
+                    const T d = x[i] - mean;
+                    s = s + d * d;
+                }
+            }
+            for (int off = G / 2; off >= 1; off >>= 1)
+                s = s + dh_shfl_xor(s, off);
+            s = s / static_cast<T>(cols);
+            acc = (FINAL == 3) ? dev_sqrt<T>(s) : s;
+        }
+        if constexpr (NANFIRST) {
+            const T first = row[0];
+            if (dev_isnan(first))
+                acc = first;
+        }
+        if (lane == 0)
+            res[r * ld_res] = acc;
+    }
+}
+
+// IDXMIN / IDXMAX per row: (value, index) pairs; on equal values the lower index wins.
+template <typename T, int VEC, bool IS_MIN>
+__global__ __launch_bounds__(THREADS) void row_idx_kernel(uint64_t *res, size_t ld_res, const T *arg, size_t rows,
+                                                          size_t cols, size_t ld, int G) {
+    const int tid = threadIdx.x;
+    const int lane = tid % G;
+    const size_t rows_per_block = THREADS / G;
+    const size_t cvecs = cols / VEC;
+    const T worst = IS_MIN ? std::numeric_limits<T>::infinity() : -std::numeric_limits<T>::infinity();
+    for (size_t r = static_cast<size_t>(blockIdx.x) * rows_per_block + tid / G; r < rows;
+         r += static_cast<size_t>(gridDim.x) * rows_per_block) {
+        const T *row = arg + r * ld;
+        T best = worst;
+        unsigned long long bi = ~0ull;
+        for (size_t cv = lane; cv < cvecs; cv += G) {
+            T x[VEC];
+            load_vec<T, VEC>(row + cv * VEC, x);
+#pragma unroll
+            for (int i = 0; i < VEC; i++) {
+                const unsigned long long idx = cv * VEC + i;
+                const bool better = IS_MIN ? (x[i] < best) : (x[i] > best);
+                // within a lane indices only grow, so a tie keeps the earlier one, except against
+                // the sentinel (an actual +-inf value must beat "nothing seen yet")
+                const bool first_seen = (bi == ~0ull) && !dev_isnan(x[i]);
+                if (better || first_seen) {
+                    best = x[i];
+                    bi = idx;
+                }
+            }
+        }
+        for (int off = G / 2; off >= 1; off >>= 1) {
+            const T ov = dh_shfl_xor(best, off);
+            const unsigned long long oi = dh_shfl_xor(bi, off);
+            const bool better = IS_MIN ? (ov < best) : (ov > best);
+            if (better || (ov == best && oi < bi)) {
+                best = ov;
+                bi = oi;
+            }
+        }
+        if (lane == 0) {
+            // AggRow.h:73-80: the scan starts from element 0; if that is NaN no later element
+            // compares below/above it, so 0 is returned. An all-NaN tail leaves bi untouched.
+            if (dev_isnan(row[0]) || bi == ~0ull)
+                bi = 0;
+            res[r * ld_res] = bi;
+        }
+    }
+}
+
+static inline int pick_group(size_t cvecs) {
+    int g = 1;
+    while (g < DH_WAVE && static_cast<size_t>(g) < cvecs)
+        g <<= 1;
+    return g;
+}
+
+static inline unsigned row_grid(const dh_ctx *ctx, size_t rows, int G) {
+    const size_t rpb = THREADS / G;
+    size_t g = dh_ceil_div(rows, rpb);
+    const size_t cap = static_cast<size_t>(ctx->num_cus) * 16;
+    if (g > cap)
+        g = cap;
+    if (g < 1)
+        g = 1;
+    return static_cast<unsigned>(g);
+}
+
+template <typename T, class R, int FINAL, bool NANFIRST>
+static inline void row_launch(dh_ctx *ctx, T *res, size_t ld_res, const T *arg, size_t rows, size_t cols, size_t ld) {
+    constexpr int V = dh_vec<T>::N;
+    const bool vec_ok = (cols % V == 0) && (ld % V == 0) && dh_aligned(arg, 16);
+    if (vec_ok) {
+        const int G = pick_group(cols / V);
+        hipLaunchKernelGGL((row_kernel<T, V, R, FINAL, NANFIRST>), dim3(row_grid(ctx, rows, G)), dim3(THREADS), 0,
+                           ctx->stream, res, ld_res, arg, rows, cols, ld, G);
+    } else {
+        const int G = pick_group(cols);
+        hipLaunchKernelGGL((row_kernel<T, 1, R, FINAL, NANFIRST>), dim3(row_grid(ctx, rows, G)), dim3(THREADS), 0,
+                           ctx->stream, res, ld_res, arg, rows, cols, ld, G);
+    }
+}
+
+template <typename T> dh_status agg_row(dh_ctx *ctx, int op, T *res, size_t ld_res, const T *arg, size_t rows, size_t cols, size_t ld) {
+    DH_REQUIRE_CTX(ctx);
+    if (ld < cols || ld_res < 1)
+        return dh_fail(DH_ERR_RUNTIME, "AggRow - leading dimension smaller than the column count");
+    if (rows == 0)
+        return DH_OK;
+    if (cols == 0)
+        return dh_fail(DH_ERR_RUNTIME, "AggRow - the argument has no columns");
+    switch (op) {
+    case DH_AGG_SUM:
+        row_launch<T, RSum<T>, 0, false>(ctx, res, ld_res, arg, rows, cols, ld);
+        break;
+    case DH_AGG_PROD:
+        row_launch<T, RProd<T>, 0, false>(ctx, res, ld_res, arg, rows, cols, ld);
+        break;
+    case DH_AGG_MIN:
+        row_launch<T, RMin<T>, 0, true>(ctx, res, ld_res, arg, rows, cols, ld);
+        break;
+    case DH_AGG_MAX:
+        row_launch<T, RMax<T>, 0, true>(ctx, res, ld_res, arg, rows, cols, ld);
+        break;
+    case DH_AGG_MEAN:
+        row_launch<T, RSum<T>, 1, false>(ctx, res, ld_res, arg, rows, cols, ld);
+        break;
+    case DH_AGG_VAR:
+        row_launch<T, RSum<T>, 2, false>(ctx, res, ld_res, arg, rows, cols, ld);
+        break;
+    case DH_AGG_STDDEV:
+        row_launch<T, RSum<T>, 3, false>(ctx, res, ld_res, arg, rows, cols, ld);
+        break;
+    default:
+        return dh_fail(DH_ERR_RUNTIME, "unsupported AggOpCode"); // AggOpCode.h:48
+    }
+    DH_CHECK_LAUNCH();
+    return DH_OK;
+}
+
+template <typename T>
+dh_status agg_row_idx(dh_ctx *ctx, int op, uint64_t *res, size_t ld_res, const T *arg, size_t rows, size_t cols, size_t ld) {
+    DH_REQUIRE_CTX(ctx);
+    if (ld < cols || ld_res < 1)
+        return dh_fail(DH_ERR_RUNTIME, "AggRow - leading dimension smaller than the column count");
+    if (op != DH_AGG_IDXMIN && op != DH_AGG_IDXMAX)
+        return dh_fail(DH_ERR_RUNTIME, "unsupported AggOpCode");
+    if (rows == 0)
+        return DH_OK;
+    if (cols == 0)
+        return dh_fail(DH_ERR_RUNTIME, "AggRow - the argument has no columns");
+    constexpr int V = dh_vec<T>::N;
+    const bool vec_ok = (cols % V == 0) && (ld % V == 0) && dh_aligned(arg, 16);
+    const int G = pick_group(vec_ok ? cols / V : cols);
+    const dim3 grid(row_grid(ctx, rows, G)), block(THREADS);
+    if (vec_ok) {
+        if (op == DH_AGG_IDXMIN)
+            hipLaunchKernelGGL((row_idx_kernel<T, V, true>), grid, block, 0, ctx->stream, res, ld_res, arg, rows, cols, ld, G);
+        else
+            hipLaunchKernelGGL((row_idx_kernel<T, V, false>), grid, block, 0, ctx->stream, res, ld_res, arg, rows, cols, ld, G);
+    } else {
+        if (op == DH_AGG_IDXMIN)
+            hipLaunchKernelGGL((row_idx_kernel<T, 1, true>), grid, block, 0, ctx->stream, res, ld_res, arg, rows, cols, ld, G);
+        else
+            hipLaunchKernelGGL((row_idx_kernel<T, 1, false>), grid, block, 0, ctx->stream, res, ld_res, arg, rows, cols, ld, G);
+    }
+    DH_CHECK_LAUNCH();
+    return DH_OK;
+}
+
+// =======================================================================================
+// AggCol
+// =======================================================================================
+// Block b owns rows [b*slab, (b+1)*slab). Threads (tx, ty): tx walks column vectors (grid.y
+// covers wider matrices), ty interleaves the slab's rows.
+template <typename T, int VEC, class R>
+__global__ __launch_bounds__(THREADS) void col_stage1(const T *arg, size_t rows, size_t cvecs, size_t ld, size_t slab,
+                                                      T *partials /* [gridDim.x][cvecs*VEC] */) {
+    extern __shared__ unsigned char lds_raw[];
+    T *lds = reinterpret_cast<T *>(lds_raw); // [blockDim.y][blockDim.x * VEC]
+    const size_t cv = static_cast<size_t>(blockIdx.y) * blockDim.x + threadIdx.x;
+    const size_t r_begin = static_cast<size_t>(blockIdx.x) * slab;
+    const size_t r_end = (r_begin + slab < rows) ? r_begin + slab : rows;
+    T acc[VEC];
+#pragma unroll
+    for (int i = 0; i < VEC; i++)
+        acc[i] = R::id();
+    if (cv < cvecs) {
+        const size_t step = blockDim.y;
+        for (size_t r0 = r_begin + threadIdx.y; r0 < r_end; r0 += step * UNROLL) {
+            T x[UNROLL][VEC];
+#pragma unroll
+            for (int u = 0; u < UNROLL; u++) {
+                const size_t r = r0 + u * step;
+                if (r < r_end)
+                    load_vec<T, VEC>(arg + r * ld + cv * VEC, x[u]);
+            }
+#pragma unroll
+            for (int u = 0; u < UNROLL; u++) {
+                const size_t r = r0 + u * step;
+                if (r < r_end) {
+#pragma unroll
+                    for (int i = 0; i < VEC; i++)
+                        acc[i] = R::comb(acc[i], x[u][i]);
+                }
+            }
+        }
+    }
+    const int w = blockDim.x * VEC;
+#pragma unroll
+    for (int i = 0; i < VEC; i++)
+        lds[threadIdx.y * w + threadIdx.x * VEC + i] = acc[i];
+    __syncthreads();
+    if (threadIdx.y == 0 && cv < cvecs) {
+#pragma unroll
+        for (int i = 0; i < VEC; i++) {
+            T a = acc[i];
+            for (unsigned y = 1; y < blockDim.y; y++)
+                a = R::comb(a, lds[y * w + threadIdx.x * VEC + i]);
+            partials[static_cast<size_t>(blockIdx.x) * cvecs * VEC + cv * VEC + i] = a;
+        }
+    }
+}
+
+// FINAL: 0 as is, 1 mean. NANFIRST as for rows (AggCol.h:135-141: row 0 seeds the result).
+template <typename T, class R, int FINAL, bool NANFIRST>
+__global__ __launch_bounds__(THREADS) void col_stage2(const T *partials, size_t nparts, size_t cols, T *res,
+                                                      const T *arg, T count) {
+    const size_t c = static_cast<size_t>(blockIdx.x) * THREADS + threadIdx.x;
+    if (c >= cols)
+        return;
+    T a = R::id();
+    for (size_t p = 0; p < nparts; p++)
+        a = R::comb(a, partials[p * cols + c]);
+    if constexpr (FINAL == 1)
+        a = a / count;
+    if constexpr (NANFIRST) {
+        const T first = arg[c];
+        if (dev_isnan(first))
+            a = first;
+    }
+    res[c] = a;
+}
+
+// Single-pass variance: per thread shifted sums around the first value it sees, converted to
+// (n, mean, M2); the TY row-lanes are merged through LDS, blocks are merged in stage 2.
+template <typename T, int VEC>
+__global__ __launch_bounds__(THREADS) void col_var_stage1(const T *arg, size_t rows, size_t cvecs, size_t ld,
+                                                          size_t slab, T *part_mean, T *part_m2) {
+    extern __shared__ unsigned char lds_raw[];
+    T *lds_mean = reinterpret_cast<T *>(lds_raw);             // [TY][TX*VEC]
+    T *lds_m2 = lds_mean + blockDim.y * blockDim.x * VEC;     // [TY][TX*VEC]
+    const size_t cv = static_cast<size_t>(blockIdx.y) * blockDim.x + threadIdx.x;
+    const size_t r_begin = static_cast<size_t>(blockIdx.x) * slab;
+    const size_t r_end = (r_begin + slab < rows) ? r_begin + slab : rows;
+    const size_t step = blockDim.y;
+    T shift[VEC], s1[VEC], s2[VEC];
+#pragma unroll
+    for (int i = 0; i < VEC; i++) {
+        shift[i] = T(0);
+        s1[i] = T(0);
+        s2[i] = T(0);
+    }
+    size_t n = 0;
+    if (cv < cvecs && r_begin + threadIdx.y < r_end) {
+        load_vec<T, VEC>(arg + (r_begin + threadIdx.y) * ld + cv * VEC, shift);
+        n = (r_end - r_begin - threadIdx.y + step - 1) / step;
+        for (size_t r0 = r_begin + threadIdx.y; r0 < r_end; r0 += step * UNROLL) {
+            T x[UNROLL][VEC];
+#pragma unroll
+            for (int u = 0; u < UNROLL; u++) {
+                const size_t r = r0 + u * step;
+                if (r < r_end)
+                    load_vec<T, VEC>(arg + r * ld + cv * VEC, x[u]);
+            }
+#pragma unroll
+            for (int u = 0; u < UNROLL; u++) {
+                const size_t r = r0 + u * step;
+                if (r < r_end) {
+#pragma unroll
+                    for (int i = 0; i < VEC; i++) {
+                        const T d = x[u][i] - shift[i];
+                        s1[i] += d;
+                        s2[i] += d * d;
+                    }
+                }
+            }
+        }
+    }
+    const int w = blockDim.x * VEC;
+#pragma unroll
+    for (int i = 0; i < VEC; i++) {
+        T mean = T(0), m2 = T(0);
+        if (n) {
+            const T nn = static_cast<T>(n);
+            mean = shift[i] + s1[i] / nn;
+            m2 = s2[i] - s1[i] * s1[i] / nn;
+            if (m2 < T(0))
+                m2 = T(0);
+        }
+        lds_mean[threadIdx.y * w + threadIdx.x * VEC + i] = mean;
+        lds_m2[threadIdx.y * w + threadIdx.x * VEC + i] = m2;
+    }
+    __syncthreads();
+    if (threadIdx.y == 0 && cv < cvecs) {
+        const size_t total = (r_end > r_begin) ? r_end - r_begin : 0;
+#pragma unroll
+        for (int i = 0; i < VEC; i++) {
+            double cn = 0.0, cmean = 0.0, cm2 = 0.0;
+            for (unsigned y = 0; y < blockDim.y; y++) {
+                if (y >= total)
+                    break;
+                const double ny = static_cast<double>((total - y + step - 1) / step);
+                const double my = static_cast<double>(lds_mean[y * w + threadIdx.x * VEC + i]);
+                const double qy = static_cast<double>(lds_m2[y * w + threadIdx.x * VEC + i]);
+                const double delta = my - cmean;
+                const double nt = cn + ny;
+                cmean += delta * ny / nt;
+                cm2 += qy + delta * delta * cn * ny / nt;
+                cn = nt;
+            }
+            part_mean[static_cast<size_t>(blockIdx.x) * cvecs * VEC + cv * VEC + i] = static_cast<T>(cmean);
+            part_m2[static_cast<size_t>(blockIdx.x) * cvecs * VEC + cv * VEC + i] = static_cast<T>(cm2);
+        }
+    }
+}
+
+// OUT: 0 variance, 1 stddev, 2 mean (unused by the public API but kept for pipelines).
+template <typename T, int OUT>
+__global__ __launch_bounds__(THREADS) void col_var_stage2(const T *part_mean, const T *part_m2, size_t nparts,
+                                                          size_t cols, size_t rows, size_t slab, T *res) {
+    const size_t c = static_cast<size_t>(blockIdx.x) * THREADS + threadIdx.x;
+    if (c >= cols)
+        return;
+    double cn = 0.0, cmean = 0.0, cm2 = 0.0;
+    for (size_t p = 0; p < nparts; p++) {
+        const size_t r_begin = p * slab;
+        if (r_begin >= rows)
+            break;
+        const size_t r_end = (r_begin + slab < rows) ? r_begin + slab : rows;
+        const double np_ = static_cast<double>(r_end - r_begin);
+        const double mp = static_cast<double>(part_mean[p * cols + c]);
+        const double qp = static_cast<double>(part_m2[p * cols + c]);
+        const double delta = mp - cmean;
+        const double nt = cn + np_;
+        cmean += delta * np_ / nt;
+        cm2 += qp + delta * delta * cn * np_ / nt;
+        cn = nt;
+    }
+    double v = cm2 / static_cast<double>(rows);
+    if constexpr (OUT == 1)
+        v = sqrt(v);
+    if constexpr (OUT == 2)
+        v = cmean;
+    res[c] = static_cast<T>(v);
+}
+
+// IDXMIN / IDXMAX per column.
+template <typename T, int VEC, bool IS_MIN>
+__global__ __launch_bounds__(THREADS) void col_idx_stage1(const T *arg, size_t rows, size_t cvecs, size_t ld, size_t slab,
+                                                          T *part_val, unsigned long long *part_idx) {
+    extern __shared__ unsigned char lds_raw[];
+    unsigned long long *lds_idx = reinterpret_cast<unsigned long long *>(lds_raw);        // [TY][TX*VEC]
+    T *lds_val = reinterpret_cast<T *>(lds_idx + blockDim.y * blockDim.x * VEC);          // [TY][TX*VEC]
+    const T worst = IS_MIN ? std::numeric_limits<T>::infinity() : -std::numeric_limits<T>::infinity();
+    const size_t cv = static_cast<size_t>(blockIdx.y) * blockDim.x + threadIdx.x;
+    const size_t r_begin = static_cast<size_t>(blockIdx.x) * slab;
+    const size_t r_end = (r_begin + slab < rows) ? r_begin + slab : rows;
+    T best[VEC];
+    unsigned long long bi[VEC];
+#pragma unroll
+    for (int i = 0; i < VEC; i++) {
+        best[i] = worst;
+        bi[i] = ~0ull;
+    }
+    if (cv < cvecs) {
+        for (size_t r = r_begin + threadIdx.y; r < r_end; r += blockDim.y) {
+            T x[VEC];
+            load_vec<T, VEC>(arg + r * ld + cv * VEC, x);
+#pragma unroll
+            for (int i = 0; i < VEC; i++) {
+                const bool better = IS_MIN ? (x[i] < best[i]) : (x[i] > best[i]);
+                const bool first_seen = (bi[i] == ~0ull) && !dev_isnan(x[i]);
+                if (better || first_seen) {
+                    best[i] = x[i];
+                    bi[i] = r;
+                }
+            }
+        }
+    }
+    const int w = blockDim.x * VEC;
+#pragma unroll
+    for (int i = 0; i < VEC; i++) {
+        lds_val[threadIdx.y * w + threadIdx.x * VEC + i] = best[i];
+        lds_idx[threadIdx.y * w + threadIdx.x * VEC + i] = bi[i];
+    }
+    __syncthreads();
+    if (threadIdx.y == 0 && cv < cvecs) {
+#pragma unroll
+        for (int i = 0; i < VEC; i++) {
+            T b = best[i];
+            unsigned long long k = bi[i];
+            for (unsigned y = 1; y < blockDim.y; y++) {
+                const T ov = lds_val[y * w + threadIdx.x * VEC + i];
+                const unsigned long long oi = lds_idx[y * w + threadIdx.x * VEC + i];
+                const bool better = IS_MIN ? (ov < b) : (ov > b);
+                if (better || (ov == b && oi < k)) {
+                    b = ov;
+                    k = oi;
+                }
+            }
+            part_val[static_cast<size_t>(blockIdx.x) * cvecs * VEC + cv * VEC + i] = b;
+            part_idx[static_cast<size_t>(blockIdx.x) * cvecs * VEC + cv * VEC + i] = k;
+        }
+    }
+}
+
+template <typename T, bool IS_MIN>
+__global__ __launch_bounds__(THREADS) void col_idx_stage2(const T *part_val, const unsigned long long *part_idx,
+                                                          size_t nparts, size_t cols, const T *arg, uint64_t *res) {
+    const size_t c = static_cast<size_t>(blockIdx.x) * THREADS + threadIdx.x;
+    if (c >= cols)
+        return;
+    T b = part_val[c];
+    unsigned long long k = part_idx[c];
+    for (size_t p = 1; p < nparts; p++) {
+        const T ov = part_val[p * cols + c];
+        const unsigned long long oi = part_idx[p * cols + c];
+        const bool better = IS_MIN ? (ov < b) : (ov > b);
+        if (better || (ov == b && oi < k)) {
+            b = ov;
+            k = oi;
+        }
+    }
+    // AggCol.h:75-91: row 0 seeds the running extremum; a NaN there is never displaced.
+    if (dev_isnan(arg[c]) || k == ~0ull)
+        k = 0;
+    res[c] = k;
+}
+
+struct ColPlan {
+    dim3 grid, block;
+    size_t slab, nparts, cvecs;
+    int vec;
+};
+template <typename T> static inline ColPlan col_plan(const dh_ctx *ctx, const T *arg, size_t rows, size_t cols, size_t ld) {
+    constexpr int V = dh_vec<T>::N;
+    ColPlan p;
+    const bool vec_ok = (cols % V == 0) && (ld % V == 0) && dh_aligned(arg, 16);
+    p.vec = vec_ok ? V : 1;
+    p.cvecs = cols / p.vec;
+    unsigned tx = 1;
+    while (tx < THREADS && tx < p.cvecs)
+        tx <<= 1;
+    unsigned ty = THREADS / tx;
+    size_t gy = dh_ceil_div(p.cvecs, tx);
+    size_t max_blocks = static_cast<size_t>(ctx->num_cus) * 8;
+    size_t gx = max_blocks / gy;
+    if (gx < 1)
+        gx = 1;
+    const size_t min_slab = static_cast<size_t>(ty) * UNROLL;
+    size_t slab = dh_ceil_div(rows, gx);
+    slab = dh_ceil_div(slab, min_slab) * min_slab;
+    gx = dh_ceil_div(rows, slab);
+    if (gx < 1)
+        gx = 1;
+    p.grid = dim3(static_cast<unsigned>(gx), static_cast<unsigned>(gy), 1);
+    p.block = dim3(tx, ty, 1);
+    p.slab = slab;
+    p.nparts = gx;
+    return p;
+}
+
+template <typename T, class R, int FINAL, bool NANFIRST>
+static inline dh_status col_launch(dh_ctx *ctx, T *res, const T *arg, size_t rows, size_t cols, size_t ld) {
+    constexpr int V = dh_vec<T>::N;
+    ColPlan p = col_plan<T>(ctx, arg, rows, cols, ld);
+    void *wsv = nullptr;
+    dh_status st = dh_workspace(ctx, p.nparts * cols * sizeof(T), &wsv);
+    if (st != DH_OK)
+        return st;
+    T *partials = static_cast<T *>(wsv);
+    const size_t lds = static_cast<size_t>(THREADS) * p.vec * sizeof(T);
+    if (p.vec == V)
+        hipLaunchKernelGGL((col_stage1<T, V, R>), p.grid, p.block, lds, ctx->stream, arg, rows, p.cvecs, ld, p.slab, partials);
+    else
+        hipLaunchKernelGGL((col_stage1<T, 1, R>), p.grid, p.block, lds, ctx->stream, arg, rows, p.cvecs, ld, p.slab, partials);
+    hipLaunchKernelGGL((col_stage2<T, R, FINAL, NANFIRST>), dim3(static_cast<unsigned>(dh_ceil_div(cols, THREADS))),
+                       dim3(THREADS), 0, ctx->stream, partials, p.nparts, cols, res, arg, static_cast<T>(rows));
+    return DH_OK;
+}
+
+template <typename T> dh_status agg_col(dh_ctx *ctx, int op, T *res, const T *arg, size_t rows, size_t cols, size_t ld) {
+    DH_REQUIRE_CTX(ctx);
+    if (ld < cols)
+        return dh_fail(DH_ERR_RUNTIME, "AggCol - leading dimension smaller than the column count");
+    if (cols == 0)
+        return DH_OK;
+    if (rows == 0)
+        return dh_fail(DH_ERR_RUNTIME, "AggCol - the argument has no rows");
+    dh_status st = DH_OK;
+    switch (op) {
+    case DH_AGG_SUM:
+        st = col_launch<T, RSum<T>, 0, false>(ctx, res, arg, rows, cols, ld);
+        break;
+    case DH_AGG_PROD:
+        st = col_launch<T, RProd<T>, 0, false>(ctx, res, arg, rows, cols, ld);
+        break;
+    case DH_AGG_MIN:
+        st = col_launch<T, RMin<T>, 0, true>(ctx, res, arg, rows, cols, ld);
+        break;
+    case DH_AGG_MAX:
+        st = col_launch<T, RMax<T>, 0, true>(ctx, res, arg, rows, cols, ld);
+        break;
+    case DH_AGG_MEAN:
+        st = col_launch<T, RSum<T>, 1, false>(ctx, res, arg, rows, cols, ld);
+        break;
+    case DH_AGG_VAR:
+    case DH_AGG_STDDEV: {
+        constexpr int V = dh_vec<T>::N;
+        ColPlan p = col_plan<T>(ctx, arg, rows, cols, ld);
+        void *wsv = nullptr;
+        st = dh_workspace(ctx, 2 * p.nparts * cols * sizeof(T), &wsv);
+        if (st != DH_OK)
+            return st;
+        T *pm = static_cast<T *>(wsv);
+        T *pq = pm + p.nparts * cols;
+        const size_t lds = 2 * static_cast<size_t>(THREADS) * p.vec * sizeof(T);
+        if (p.vec == V)
+            hipLaunchKernelGGL((col_var_stage1<T, V>), p.grid, p.block, lds, ctx->stream, arg, rows, p.cvecs, ld, p.slab, pm, pq);
+        else
+            hipLaunchKernelGGL((col_var_stage1<T, 1>), p.grid, p.block, lds, ctx->stream, arg, rows, p.cvecs, ld, p.slab, pm, pq);
+        const dim3 g2(static_cast<unsigned>(dh_ceil_div(cols, THREADS)));
+        if (op == DH_AGG_VAR)
+            hipLaunchKernelGGL((col_var_stage2<T, 0>), g2, dim3(THREADS), 0, ctx->stream, pm, pq, p.nparts, cols, rows, p.slab, res);
+        else
+            hipLaunchKernelGGL((col_var_stage2<T, 1>), g2, dim3(THREADS), 0, ctx->stream, pm, pq, p.nparts, cols, rows, p.slab, res);
+        break;
+    }
+    default:
+        return dh_fail(DH_ERR_RUNTIME, "unsupported AggOpCode");
+    }
+    if (st != DH_OK)
+        return st;
+    DH_CHECK_LAUNCH();
+    return DH_OK;
+}
+
+template <typename T> dh_status agg_col_idx(dh_ctx *ctx, int op, uint64_t *res, const T *arg, size_t rows, size_t cols, size_t ld) {
+    DH_REQUIRE_CTX(ctx);
+    if (ld < cols)
+        return dh_fail(DH_ERR_RUNTIME, "AggCol - leading dimension smaller than the column count");
+    if (op != DH_AGG_IDXMIN && op != DH_AGG_IDXMAX)
+        return dh_fail(DH_ERR_RUNTIME, "unsupported AggOpCode");
+    if (cols == 0)
+        return DH_OK;
+    if (rows == 0)
+        return dh_fail(DH_ERR_RUNTIME, "AggCol - the argument has no rows");
+    constexpr int V = dh_vec<T>::N;
+    ColPlan p = col_plan<T>(ctx, arg, rows, cols, ld);
+    void *wsv = nullptr;
+    dh_status st = dh_workspace(ctx, p.nparts * cols * (sizeof(T) + sizeof(unsigned long long)) + 256, &wsv);
+    if (st != DH_OK)
+        return st;
+    unsigned long long *pidx = static_cast<unsigned long long *>(wsv);
+    T *pval = reinterpret_cast<T *>(pidx + p.nparts * cols);
+    const size_t lds = static_cast<size_t>(THREADS) * p.vec * (sizeof(T) + sizeof(unsigned long long));
+    const dim3 g2(static_cast<unsigned>(dh_ceil_div(cols, THREADS)));
+    if (op == DH_AGG_IDXMIN) {
+        if (p.vec == V)
+            hipLaunchKernelGGL((col_idx_stage1<T, V, true>), p.grid, p.block, lds, ctx->stream, arg, rows, p.cvecs, ld, p.slab, pval, pidx);
+        else
+            hipLaunchKernelGGL((col_idx_stage1<T, 1, true>), p.grid, p.block, lds, ctx->stream, arg, rows, p.cvecs, ld, p.slab, pval, pidx);
+        hipLaunchKernelGGL((col_idx_stage2<T, true>), g2, dim3(THREADS), 0, ctx->stream, pval, pidx, p.nparts, cols, arg, res);
+    } else {
+        if (p.vec == V)
+            hipLaunchKernelGGL((col_idx_stage1<T, V, false>), p.grid, p.block, lds, ctx->stream, arg, rows, p.cvecs, ld, p.slab, pval, pidx);
+        else
+            hipLaunchKernelGGL((col_idx_stage1<T, 1, false>), p.grid, p.block, lds, ctx->stream, arg, rows, p.cvecs, ld, p.slab, pval, pidx);
+        hipLaunchKernelGGL((col_idx_stage2<T, false>), g2, dim3(THREADS), 0, ctx->stream, pval, pidx, p.nparts, cols, arg, res);
+    }
+    DH_CHECK_LAUNCH();
+    return DH_OK;
+}
+
+} // namespace dh_agg

@@ -1,0 +1,240 @@
+// Device context and allocator of libdaphne_hip.so.
+//
+// Stands in for the reference's CUDAContext (runtime/local/context/CUDAContext.cpp:41-135):
+// device selection, property query, a memory budget of 90 % of the device total, and a
+// registry of allocations that are released when the context is destroyed. There are no
+// library handles: every kernel in this library is hand-written.
+#include "common.h"
+
+#include <cstring>
+
+namespace {
+thread_local std::string g_last_error;
+}
+
+void dh_set_error(const char *fmt, ...) {
+    char buf[1024];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof(buf), fmt, ap);
+    va_end(ap);
+    g_last_error = buf;
+}
+
+dh_status dh_fail(dh_status st, const char *fmt, ...) {
+    char buf[1024];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof(buf), fmt, ap);
+    va_end(ap);
+    g_last_error = buf;
+    return st;
+}
+
+extern "C" const char *dh_last_error(void) { return g_last_error.c_str(); }
+
+extern "C" dh_status dh_ctx_create(int device, dh_ctx **out) {
+    if (out == nullptr)
+        return dh_fail(DH_ERR_RUNTIME, "dh_ctx_create: out is null");
+    *out = nullptr;
+    int count = 0;
+    DH_CHECK_HIP(hipGetDeviceCount(&count));
+    if (device < 0 || device >= count)
+        return dh_fail(DH_ERR_RUNTIME, "dh_ctx_create: requested device %d but only %d device(s) are visible",
+                       device, count);
+    DH_CHECK_HIP(hipSetDevice(device));
+    auto *ctx = new dh_ctx();
+    ctx->device = device;
+    hipError_t e = hipGetDeviceProperties(&ctx->props, device);
+    if (e != hipSuccess) {
+        delete ctx;
+        return dh_fail(DH_ERR_HIP, "hipGetDeviceProperties: %s", hipGetErrorString(e));
+    }
+    if (strncmp(ctx->props.gcnArchName, "gfx950", 6) != 0) {
+        std::string arch = ctx->props.gcnArchName;
+        delete ctx;
+        return dh_fail(DH_ERR_RUNTIME, "dh_ctx_create: this library holds gfx950 code only, device %d is %s", device,
+                       arch.c_str());
+    }
+    size_t free_b = 0, total_b = 0;
+    e = hipMemGetInfo(&free_b, &total_b);
+    if (e != hipSuccess) {
+        delete ctx;
+        return dh_fail(DH_ERR_HIP, "hipMemGetInfo: %s", hipGetErrorString(e));
+    }
+    // 90 % of the device total, like CUDAContext.cpp:49-50.
+    ctx->mem_budget = static_cast<size_t>(static_cast<double>(total_b) * 0.9);
+    ctx->num_cus = ctx->props.multiProcessorCount;
+    bool ok = hipMalloc(reinterpret_cast<void **>(&ctx->flag_dev), 256) == hipSuccess &&
+              hipHostMalloc(reinterpret_cast<void **>(&ctx->flag_host), 256, hipHostMallocDefault) == hipSuccess &&
+              hipEventCreate(&ctx->ev_start) == hipSuccess && hipEventCreate(&ctx->ev_stop) == hipSuccess;
+    if (!ok) {
+        dh_ctx_destroy(ctx);
+        return dh_fail(DH_ERR_HIP, "dh_ctx_create: could not allocate the context's flag words / events");
+    }
+    *out = ctx;
+    return DH_OK;
+}
+
+extern "C" dh_status dh_ctx_destroy(dh_ctx *ctx) {
+    if (ctx == nullptr)
+        return DH_OK;
+    (void)hipSetDevice(ctx->device);
+    (void)hipDeviceSynchronize();
+    for (auto &kv : ctx->allocations)
+        (void)hipFree(kv.first);
+    ctx->allocations.clear();
+    if (ctx->ws)
+        (void)hipFree(ctx->ws);
+    if (ctx->flag_dev)
+        (void)hipFree(ctx->flag_dev);
+    if (ctx->flag_host)
+        (void)hipHostFree(ctx->flag_host);
+    if (ctx->ev_start)
+        (void)hipEventDestroy(ctx->ev_start);
+    if (ctx->ev_stop)
+        (void)hipEventDestroy(ctx->ev_stop);
+    delete ctx;
+    return DH_OK;
+}
+
+extern "C" size_t dh_ctx_mem_budget(const dh_ctx *ctx) { return ctx ? ctx->mem_budget : 0; }
+extern "C" size_t dh_ctx_mem_in_use(const dh_ctx *ctx) { return ctx ? ctx->mem_in_use : 0; }
+extern "C" int dh_ctx_device(const dh_ctx *ctx) { return ctx ? ctx->device : -1; }
+
+extern "C" dh_status dh_ctx_props(const dh_ctx *ctx, int *compute_units, int *clock_khz, size_t *total_mem,
+                                  char *name, size_t name_cap) {
+    if (ctx == nullptr)
+        return dh_fail(DH_ERR_RUNTIME, "dh_ctx_props: context is null");
+    if (compute_units)
+        *compute_units = ctx->props.multiProcessorCount;
+    if (clock_khz)
+        *clock_khz = ctx->props.clockRate;
+    if (total_mem)
+        *total_mem = ctx->props.totalGlobalMem;
+    if (name && name_cap) {
+        snprintf(name, name_cap, "%s (%s)", ctx->props.name, ctx->props.gcnArchName);
+    }
+    return DH_OK;
+}
+
+extern "C" dh_status dh_ctx_set_stream(dh_ctx *ctx, void *hip_stream) {
+    if (ctx == nullptr)
+        return dh_fail(DH_ERR_RUNTIME, "dh_ctx_set_stream: context is null");
+    ctx->stream = static_cast<hipStream_t>(hip_stream);
+    return DH_OK;
+}
+
+extern "C" void *dh_ctx_get_stream(const dh_ctx *ctx) { return ctx ? static_cast<void *>(ctx->stream) : nullptr; }
+
+extern "C" dh_status dh_sync(dh_ctx *ctx) {
+    DH_REQUIRE_CTX(ctx);
+    DH_CHECK_HIP(hipStreamSynchronize(ctx->stream));
+    return DH_OK;
+}
+
+extern "C" dh_status dh_malloc(dh_ctx *ctx, size_t bytes, int zero, void **out) {
+    DH_REQUIRE_CTX(ctx);
+    if (out == nullptr)
+        return dh_fail(DH_ERR_RUNTIME, "dh_malloc: out is null");
+    *out = nullptr;
+    std::lock_guard<std::mutex> g(ctx->lock);
+    if (ctx->mem_in_use + bytes > ctx->mem_budget)
+        return dh_fail(DH_ERR_OOM, "dh_malloc: %zu bytes requested, %zu in use, budget %zu", bytes, ctx->mem_in_use,
+                       ctx->mem_budget);
+    void *p = nullptr;
+    // A zero-size request still gets a distinct pointer so it can serve as a registry key.
+    hipError_t e = hipMalloc(&p, bytes ? bytes : 1);
+    if (e != hipSuccess)
+        return dh_fail(e == hipErrorOutOfMemory ? DH_ERR_OOM : DH_ERR_HIP, "hipMalloc(%zu): %s", bytes,
+                       hipGetErrorString(e));
+    if (zero && bytes) {
+        e = hipMemsetAsync(p, 0, bytes, ctx->stream);
+        if (e != hipSuccess) {
+            (void)hipFree(p);
+            return dh_fail(DH_ERR_HIP, "hipMemsetAsync: %s", hipGetErrorString(e));
+        }
+    }
+    ctx->allocations[p] = bytes;
+    ctx->mem_in_use += bytes;
+    *out = p;
+    return DH_OK;
+}
+
+extern "C" dh_status dh_free(dh_ctx *ctx, void *ptr) {
+    DH_REQUIRE_CTX(ctx);
+    if (ptr == nullptr)
+        return DH_OK;
+    std::lock_guard<std::mutex> g(ctx->lock);
+    auto it = ctx->allocations.find(ptr);
+    if (it == ctx->allocations.end())
+        return dh_fail(DH_ERR_RUNTIME, "dh_free: pointer %p was not allocated by this context", ptr);
+    // hipFree waits for outstanding work that may still use the buffer.
+    DH_CHECK_HIP(hipFree(ptr));
+    ctx->mem_in_use -= it->second;
+    ctx->allocations.erase(it);
+    return DH_OK;
+}
+
+extern "C" dh_status dh_h2d(dh_ctx *ctx, void *dst_dev, const void *src_host, size_t bytes) {
+    DH_REQUIRE_CTX(ctx);
+    if (bytes == 0)
+        return DH_OK;
+    DH_CHECK_HIP(hipMemcpyAsync(dst_dev, src_host, bytes, hipMemcpyHostToDevice, ctx->stream));
+    DH_CHECK_HIP(hipStreamSynchronize(ctx->stream));
+    return DH_OK;
+}
+
+extern "C" dh_status dh_d2h(dh_ctx *ctx, void *dst_host, const void *src_dev, size_t bytes) {
+    DH_REQUIRE_CTX(ctx);
+    if (bytes == 0)
+        return DH_OK;
+    DH_CHECK_HIP(hipMemcpyAsync(dst_host, src_dev, bytes, hipMemcpyDeviceToHost, ctx->stream));
+    DH_CHECK_HIP(hipStreamSynchronize(ctx->stream));
+    return DH_OK;
+}
+
+extern "C" dh_status dh_d2d(dh_ctx *ctx, void *dst_dev, const void *src_dev, size_t bytes) {
+    DH_REQUIRE_CTX(ctx);
+    if (bytes == 0)
+        return DH_OK;
+    DH_CHECK_HIP(hipMemcpyAsync(dst_dev, src_dev, bytes, hipMemcpyDeviceToDevice, ctx->stream));
+    return DH_OK;
+}
+
+extern "C" dh_status dh_timer_start(dh_ctx *ctx) {
+    DH_REQUIRE_CTX(ctx);
+    DH_CHECK_HIP(hipEventRecord(ctx->ev_start, ctx->stream));
+    return DH_OK;
+}
+
+extern "C" dh_status dh_timer_stop_ms(dh_ctx *ctx, float *ms) {
+    DH_REQUIRE_CTX(ctx);
+    DH_CHECK_HIP(hipEventRecord(ctx->ev_stop, ctx->stream));
+    DH_CHECK_HIP(hipEventSynchronize(ctx->ev_stop));
+    float t = 0.f;
+    DH_CHECK_HIP(hipEventElapsedTime(&t, ctx->ev_start, ctx->ev_stop));
+    if (ms)
+        *ms = t;
+    return DH_OK;
+}
+
+dh_status dh_workspace(dh_ctx *ctx, size_t bytes, void **out) {
+    std::lock_guard<std::mutex> g(ctx->ws_lock);
+    if (bytes > ctx->ws_bytes) {
+        size_t want = bytes < (size_t(8) << 20) ? (size_t(8) << 20) : bytes;
+        if (ctx->ws) {
+            DH_CHECK_HIP(hipStreamSynchronize(ctx->stream));
+            DH_CHECK_HIP(hipFree(ctx->ws));
+            ctx->ws = nullptr;
+            ctx->ws_bytes = 0;
+        }
+        hipError_t e = hipMalloc(&ctx->ws, want);
+        if (e != hipSuccess)
+            return dh_fail(e == hipErrorOutOfMemory ? DH_ERR_OOM : DH_ERR_HIP, "workspace hipMalloc(%zu): %s", want,
+                           hipGetErrorString(e));
+        ctx->ws_bytes = want;
+    }
+    *out = ctx->ws;
+    return DH_OK;
+}

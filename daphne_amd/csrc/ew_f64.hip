@@ -1,0 +1,19 @@
+// Elementwise kernels, double instantiation. See ew_impl.h for the design and reference citations.
+#include "ew_impl.h"
+
+extern "C" dh_status dh_ew_binary_f64(dh_ctx *ctx, int op, double *res, size_t ld_res, const double *lhs, size_t lhs_rows,
+                                     size_t lhs_cols, size_t ld_lhs, const double *rhs, size_t rhs_rows,
+                                     size_t rhs_cols, size_t ld_rhs) {
+    return dh_ew::ew_binary<double>(ctx, op, res, ld_res, lhs, lhs_rows, lhs_cols, ld_lhs, rhs, rhs_rows, rhs_cols,
+                                ld_rhs);
+}
+
+extern "C" dh_status dh_ew_binary_sca_f64(dh_ctx *ctx, int op, double *res, size_t ld_res, const double *lhs, size_t rows,
+                                         size_t cols, size_t ld_lhs, double rhs) {
+    return dh_ew::ew_binary_sca<double>(ctx, op, res, ld_res, lhs, rows, cols, ld_lhs, rhs);
+}
+
+extern "C" dh_status dh_ew_unary_f64(dh_ctx *ctx, int op, double *res, size_t ld_res, const double *arg, size_t rows,
+                                    size_t cols, size_t ld_arg) {
+    return dh_ew::ew_unary<double>(ctx, op, res, ld_res, arg, rows, cols, ld_arg);
+}

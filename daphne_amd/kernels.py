@@ -1,0 +1,382 @@
+"""Python mirror of the reference's kernel interface for the device path.
+
+Function names, argument order and error behaviour follow the reference's kernel convenience
+functions (``ewBinaryMat(opCode, res, lhs, rhs, ctx)``, ``aggRow(opCode, res, arg, ctx)``,
+``matMul(res, lhs, rhs, transa, transb, ctx)`` ...; reference: src/runtime/local/kernels/*.h and
+src/runtime/local/kernels/CUDA/*.h). ``res=None`` makes the kernel allocate the result, a
+``DenseMatrix`` passed as ``res`` is written in place - like ``DT *&res`` in the reference.
+
+Everything here only marshals pointers and shapes into the C ABI of libdaphne_hip.so; all
+arithmetic happens in the HIP kernels. There is no CPU fallback.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import enum
+from typing import Optional
+
+import numpy as np
+
+from . import capi
+
+
+class BinaryOpCode(enum.IntEnum):  # runtime/local/kernels/BinaryOpCode.h:29-55
+    ADD = 0; SUB = 1; MUL = 2; DIV = 3; POW = 4; MOD = 5; LOG = 6; EQ = 7; NEQ = 8; LT = 9; LE = 10
+    GT = 11; GE = 12; MIN = 13; MAX = 14; AND = 15; OR = 16; BITWISE_AND = 17; CONCAT = 18
+
+
+class UnaryOpCode(enum.IntEnum):  # runtime/local/kernels/UnaryOpCode.h:28-55
+    MINUS = 0; ABS = 1; SIGN = 2; SQRT = 3; EXP = 4; LN = 5; SIN = 6; COS = 7; TAN = 8; ASIN = 9
+    ACOS = 10; ATAN = 11; SINH = 12; COSH = 13; TANH = 14; FLOOR = 15; CEIL = 16; ROUND = 17
+    ISNAN = 18; UPPER = 19; LOWER = 20
+
+
+class AggOpCode(enum.IntEnum):  # runtime/local/kernels/AggOpCode.h:25-35
+    SUM = 0; PROD = 1; MIN = 2; MAX = 3; IDXMIN = 4; IDXMAX = 5; MEAN = 6; STDDEV = 7; VAR = 8
+
+
+_SUFFIX = {np.dtype(np.float32): "f32", np.dtype(np.float64): "f64"}
+
+
+class HIPContext:
+    """Device context + allocator; the counterpart of the reference's CUDAContext
+    (src/runtime/local/context/CUDAContext.h:29-114)."""
+
+    def __init__(self, device: int = 0):
+        self._h = C.c_void_p()
+        capi.check(capi.lib().dh_ctx_create(device, C.byref(self._h)))
+
+    # CUDAContext::getMemBudget
+    def getMemBudget(self) -> int:
+        return capi.lib().dh_ctx_mem_budget(self._h)
+
+    def memInUse(self) -> int:
+        return capi.lib().dh_ctx_mem_in_use(self._h)
+
+    def props(self) -> dict:
+        cus, khz, total = C.c_int(), C.c_int(), C.c_size_t()
+        name = C.create_string_buffer(256)
+        capi.check(capi.lib().dh_ctx_props(self._h, C.byref(cus), C.byref(khz), C.byref(total), name, 256))
+        return {"compute_units": cus.value, "clock_khz": khz.value, "total_mem": total.value,
+                "name": name.value.decode()}
+
+    def malloc(self, nbytes: int, zero: bool = False) -> int:
+        p = C.c_void_p()
+        capi.check(capi.lib().dh_malloc(self._h, nbytes, int(zero), C.byref(p)))
+        return p.value or 0
+
+    def free(self, ptr: int) -> None:
+        capi.check(capi.lib().dh_free(self._h, ptr))
+
+    def set_stream(self, stream_handle: int) -> None:
+        capi.check(capi.lib().dh_ctx_set_stream(self._h, stream_handle))
+
+    def sync(self) -> None:
+        capi.check(capi.lib().dh_sync(self._h))
+
+    def timer_start(self) -> None:
+        capi.check(capi.lib().dh_timer_start(self._h))
+
+    def timer_stop_ms(self) -> float:
+        ms = C.c_float()
+        capi.check(capi.lib().dh_timer_stop_ms(self._h, C.byref(ms)))
+        return ms.value
+
+    def destroy(self) -> None:
+        if self._h:
+            capi.lib().dh_ctx_destroy(self._h)
+            self._h = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.destroy()
+        except Exception:
+            pass
+
+
+class DenseMatrix:
+    """Row-major dense matrix resident in device memory: pointer, numRows, numCols, rowSkip
+    (reference: src/runtime/local/datastructures/DenseMatrix.h:42-56). Views share the buffer."""
+
+    def __init__(self, ctx: HIPContext, rows: int, cols: int, dtype, ptr: Optional[int] = None,
+                 row_skip: Optional[int] = None, zero: bool = False, keepalive=None):
+        self.ctx = ctx
+        self.rows, self.cols = int(rows), int(cols)
+        self.dtype = np.dtype(dtype)
+        self.row_skip = int(row_skip if row_skip is not None else cols)
+        self._owned = ptr is None
+        self._keepalive = keepalive
+        if ptr is None:
+            ptr = ctx.malloc(max(1, self.rows * self.row_skip) * self.dtype.itemsize, zero)
+        self.ptr = ptr
+
+    # -- construction -------------------------------------------------------------------
+    @staticmethod
+    def from_numpy(ctx: HIPContext, a) -> "DenseMatrix":
+        a = np.ascontiguousarray(a)
+        if a.ndim == 1:
+            a = a.reshape(-1, 1)
+        m = DenseMatrix(ctx, a.shape[0], a.shape[1], a.dtype)
+        if a.size:
+            capi.check(capi.lib().dh_h2d(ctx._h, m.ptr, a.ctypes.data, a.nbytes))
+        return m
+
+    @staticmethod
+    def from_torch(ctx: HIPContext, t) -> "DenseMatrix":
+        """Wraps a 2-D row-major torch tensor already resident on the device (no copy)."""
+        import torch
+
+        assert t.is_cuda and t.dim() == 2 and t.stride(1) == 1
+        dt = {torch.float32: np.float32, torch.float64: np.float64, torch.int64: np.int64,
+              torch.uint64: np.uint64}[t.dtype]
+        return DenseMatrix(ctx, t.shape[0], t.shape[1], dt, ptr=t.data_ptr(), row_skip=t.stride(0) if t.shape[0] > 1 else t.shape[1],
+                           keepalive=t)
+
+    # -- reference accessors --------------------------------------------------------------
+    def getNumRows(self) -> int:
+        return self.rows
+
+    def getNumCols(self) -> int:
+        return self.cols
+
+    def getRowSkip(self) -> int:
+        return self.row_skip
+
+    def getNumItems(self) -> int:
+        return self.rows * self.cols
+
+    def to_numpy(self) -> np.ndarray:
+        buf = np.empty((self.rows, self.row_skip), dtype=self.dtype)
+        if buf.size:
+            n = ((self.rows - 1) * self.row_skip + self.cols) * self.dtype.itemsize
+            capi.check(capi.lib().dh_d2h(self.ctx._h, buf.ctypes.data, self.ptr, n))
+        return np.ascontiguousarray(buf[:, : self.cols])
+
+    def slice(self, r0: int, r1: int, c0: int = 0, c1: Optional[int] = None) -> "DenseMatrix":
+        """View of rows [r0, r1) and columns [c0, c1) (DenseMatrix::slice of the reference)."""
+        c1 = self.cols if c1 is None else c1
+        off = (r0 * self.row_skip + c0) * self.dtype.itemsize
+        return DenseMatrix(self.ctx, r1 - r0, c1 - c0, self.dtype, ptr=self.ptr + off, row_skip=self.row_skip,
+                           keepalive=self)
+
+    def destroy(self) -> None:
+        if self._owned and self.ptr:
+            self.ctx.free(self.ptr)
+            self.ptr = 0
+
+    def __del__(self):
+        try:
+            if self._owned and self.ptr and self.ctx._h:
+                self.destroy()
+        except Exception:
+            pass
+
+
+def _fn(name: str, dtype):
+    try:
+        suf = _SUFFIX[np.dtype(dtype)]
+    except KeyError:
+        raise capi.DaphneHipError(capi.DH_ERR_RUNTIME, f"{name}: unsupported value type {dtype}")
+    return getattr(capi.lib(), f"{name}_{suf}")
+
+
+def _same_dtype(*ms):
+    d = ms[0].dtype
+    for m in ms[1:]:
+        if m is not None and m.dtype != d:
+            raise capi.DaphneHipError(capi.DH_ERR_RUNTIME, "mixed value types are not instantiated for the device kernels")
+    return d
+
+
+# ------------------------------------------------------------------------------------------
+# elementwise
+# ------------------------------------------------------------------------------------------
+def ewBinaryMat(opCode, res, lhs: DenseMatrix, rhs: DenseMatrix, ctx: HIPContext) -> DenseMatrix:
+    """CUDA::ewBinaryMat (kernels/CUDA/EwBinaryMat.h:40-47)."""
+    dt = _same_dtype(lhs, rhs, res)
+    if res is None:
+        res = DenseMatrix(ctx, lhs.rows, lhs.cols, dt)
+    capi.check(_fn("dh_ew_binary", dt)(ctx._h, int(opCode), res.ptr, res.row_skip, lhs.ptr, lhs.rows, lhs.cols,
+                                       lhs.row_skip, rhs.ptr, rhs.rows, rhs.cols, rhs.row_skip))
+    return res
+
+
+def ewBinaryObjSca(opCode, res, lhs: DenseMatrix, rhs: float, ctx: HIPContext) -> DenseMatrix:
+    """CUDA::ewBinaryObjSca (kernels/CUDA/EwBinaryObjSca.h:52-60)."""
+    dt = _same_dtype(lhs, res)
+    if res is None:
+        res = DenseMatrix(ctx, lhs.rows, lhs.cols, dt)
+    capi.check(_fn("dh_ew_binary_sca", dt)(ctx._h, int(opCode), res.ptr, res.row_skip, lhs.ptr, lhs.rows, lhs.cols,
+                                           lhs.row_skip, float(rhs)))
+    return res
+
+
+def ewUnaryMat(opCode, res, arg: DenseMatrix, ctx: HIPContext) -> DenseMatrix:
+    """ewUnaryMat (kernels/EwUnaryMat.h:43-45)."""
+    dt = _same_dtype(arg, res)
+    if res is None:
+        res = DenseMatrix(ctx, arg.rows, arg.cols, dt)
+    capi.check(_fn("dh_ew_unary", dt)(ctx._h, int(opCode), res.ptr, res.row_skip, arg.ptr, arg.rows, arg.cols,
+                                      arg.row_skip))
+    return res
+
+
+# ------------------------------------------------------------------------------------------
+# aggregations
+# ------------------------------------------------------------------------------------------
+def aggAll(opCode, arg: DenseMatrix, ctx: HIPContext) -> float:
+    """CUDA::aggAll (kernels/CUDA/AggAll.h:44-50): returns the scalar."""
+    ct = C.c_float if arg.dtype == np.float32 else C.c_double
+    out = ct()
+    capi.check(_fn("dh_agg_all", arg.dtype)(ctx._h, int(opCode), arg.ptr, arg.rows, arg.cols, arg.row_skip,
+                                            C.byref(out)))
+    return arg.dtype.type(out.value)
+
+
+def aggRow(opCode, res, arg: DenseMatrix, ctx: HIPContext) -> DenseMatrix:
+    """CUDA::aggRow (kernels/CUDA/AggRow.h:46-52); IDXMIN / IDXMAX give a DenseMatrix<size_t>
+    (kernels/AggRow.h:71-94)."""
+    if int(opCode) in (AggOpCode.IDXMIN, AggOpCode.IDXMAX):
+        if res is None:
+            res = DenseMatrix(ctx, arg.rows, 1, np.uint64)
+        capi.check(_fn("dh_agg_row_idx", arg.dtype)(ctx._h, int(opCode), res.ptr, res.row_skip, arg.ptr, arg.rows,
+                                                    arg.cols, arg.row_skip))
+        return res
+    if res is None:
+        res = DenseMatrix(ctx, arg.rows, 1, arg.dtype)
+    capi.check(_fn("dh_agg_row", arg.dtype)(ctx._h, int(opCode), res.ptr, res.row_skip, arg.ptr, arg.rows, arg.cols,
+                                            arg.row_skip))
+    return res
+
+
+def aggCol(opCode, res, arg: DenseMatrix, ctx: HIPContext) -> DenseMatrix:
+    """CUDA::aggCol (kernels/CUDA/AggCol.h:46-52)."""
+    if int(opCode) in (AggOpCode.IDXMIN, AggOpCode.IDXMAX):
+        if res is None:
+            res = DenseMatrix(ctx, 1, arg.cols, np.uint64)
+        capi.check(_fn("dh_agg_col_idx", arg.dtype)(ctx._h, int(opCode), res.ptr, arg.ptr, arg.rows, arg.cols,
+                                                    arg.row_skip))
+        return res
+    if res is None:
+        res = DenseMatrix(ctx, 1, arg.cols, arg.dtype)
+    capi.check(_fn("dh_agg_col", arg.dtype)(ctx._h, int(opCode), res.ptr, arg.ptr, arg.rows, arg.cols, arg.row_skip))
+    return res
+
+
+# ------------------------------------------------------------------------------------------
+# contractions
+# ------------------------------------------------------------------------------------------
+def matMul(res, lhs: DenseMatrix, rhs: DenseMatrix, transa: bool, transb: bool, ctx: HIPContext) -> DenseMatrix:
+    """CUDA::matMul (kernels/CUDA/MatMul.h:45-51)."""
+    dt = _same_dtype(lhs, rhs, res)
+    nr1 = lhs.cols if transa else lhs.rows
+    nc2 = rhs.rows if transb else rhs.cols
+    if res is None:
+        res = DenseMatrix(ctx, nr1, nc2, dt)
+    capi.check(_fn("dh_matmul", dt)(ctx._h, res.ptr, res.row_skip, lhs.ptr, lhs.rows, lhs.cols, lhs.row_skip,
+                                    rhs.ptr, rhs.rows, rhs.cols, rhs.row_skip, int(transa), int(transb)))
+    return res
+
+
+def syrk(res, arg: DenseMatrix, transLeft: bool, ctx: HIPContext) -> DenseMatrix:
+    """syrk (kernels/Syrk.h:38-40; device version kernels/CUDA/Syrk.h:40-46)."""
+    n = arg.cols if transLeft else arg.rows
+    if res is None:
+        res = DenseMatrix(ctx, n, n, arg.dtype)
+    capi.check(_fn("dh_syrk", arg.dtype)(ctx._h, res.ptr, res.row_skip, arg.ptr, arg.rows, arg.cols, arg.row_skip,
+                                         int(transLeft)))
+    return res
+
+
+def solve(res, lhs: DenseMatrix, rhs: DenseMatrix, ctx: HIPContext) -> DenseMatrix:
+    """CUDA::solve (kernels/CUDA/Solve.h; CPU kernels/Solve.h:86-116): A x = b by LU."""
+    dt = _same_dtype(lhs, rhs, res)
+    if lhs.rows != rhs.rows:
+        raise capi.DaphneHipError(1, "#rows of lhs and #rows of rhs must be the same")
+    if lhs.rows != lhs.cols:
+        raise capi.DaphneHipError(1, "#rows and #cols of lhs must be the same")
+    if lhs.row_skip != lhs.cols:
+        raise capi.DaphneHipError(1, "#cols of lhs must match row skip")
+    if rhs.cols != 1:
+        raise capi.DaphneHipError(1, "#cols of rhs must be 1")
+    if res is None:
+        res = DenseMatrix(ctx, lhs.rows, 1, dt)
+    capi.check(_fn("dh_solve", dt)(ctx._h, res.ptr, lhs.ptr, lhs.rows, lhs.row_skip, rhs.ptr))
+    return res
+
+
+# ------------------------------------------------------------------------------------------
+# DNN
+# ------------------------------------------------------------------------------------------
+def conv2dForward(res, data: DenseMatrix, filter: DenseMatrix, bias, batch_size, num_channels, img_h, img_w,
+                  filter_h, filter_w, stride_h, stride_w, pad_h, pad_w, ctx: HIPContext):
+    """CUDA::Convolution::Forward::apply (kernels/CUDA/Convolution.h:33-38). Returns
+    (res, res_h, res_w)."""
+    dt = _same_dtype(data, filter, bias, res)
+    F = filter.rows
+    P = (img_h + 2 * pad_h - filter_h) // stride_h + 1 if img_h + 2 * pad_h >= filter_h else 0
+    Q = (img_w + 2 * pad_w - filter_w) // stride_w + 1 if img_w + 2 * pad_w >= filter_w else 0
+    if res is None:
+        res = DenseMatrix(ctx, batch_size, F * P * Q, dt)
+    rh, rw = C.c_size_t(), C.c_size_t()
+    capi.check(_fn("dh_conv2d_forward", dt)(ctx._h, res.ptr, C.byref(rh), C.byref(rw), data.ptr, filter.ptr,
+                                            filter.rows, filter.cols, bias.ptr if bias is not None else None,
+                                            batch_size, num_channels, img_h, img_w, filter_h, filter_w, stride_h,
+                                            stride_w, pad_h, pad_w))
+    return res, rh.value, rw.value
+
+
+def maxPoolForward(res, data: DenseMatrix, batch_size, num_channels, img_h, img_w, pool_h, pool_w, stride_h,
+                   stride_w, pad_h, pad_w, ctx: HIPContext):
+    """CUDA::NN::Pooling::Forward<MAX>::apply (kernels/CUDA/Pooling.h:31-35; CPU
+    kernels/MaxPoolForward.h:35-44). Returns (res, res_h, res_w)."""
+    dt = data.dtype
+    P = (img_h + 2 * pad_h - pool_h) // stride_w + 1 if img_h + 2 * pad_h >= pool_h else 0
+    Q = (img_w + 2 * pad_w - pool_w) // stride_h + 1 if img_w + 2 * pad_w >= pool_w else 0
+    if res is None:
+        res = DenseMatrix(ctx, batch_size, num_channels * P * Q, dt)
+    rh, rw = C.c_size_t(), C.c_size_t()
+    capi.check(_fn("dh_maxpool_forward", dt)(ctx._h, res.ptr, C.byref(rh), C.byref(rw), data.ptr, batch_size,
+                                             num_channels, img_h, img_w, pool_h, pool_w, stride_h, stride_w, pad_h,
+                                             pad_w))
+    return res, rh.value, rw.value
+
+
+def affineForward(res, data: DenseMatrix, weights: DenseMatrix, bias, ctx: HIPContext) -> DenseMatrix:
+    """CUDA::NN::Affine::Forward::apply (kernels/CUDA/Affine.h:24-26)."""
+    dt = _same_dtype(data, weights, bias, res)
+    if res is None:
+        res = DenseMatrix(ctx, data.rows, weights.cols, dt)
+    capi.check(_fn("dh_affine_forward", dt)(ctx._h, res.ptr, data.ptr, data.rows, data.cols, weights.ptr,
+                                            weights.rows, weights.cols, bias.ptr if bias is not None else None,
+                                            bias.rows if bias is not None else 0,
+                                            bias.cols if bias is not None else 0))
+    return res
+
+
+def biasAdd(res, data: DenseMatrix, bias: DenseMatrix, ctx: HIPContext) -> DenseMatrix:
+    """CUDA::BiasAdd::apply (kernels/CUDA/BiasAdd.h:26-28; CPU kernels/BiasAdd.h:34-52)."""
+    dt = _same_dtype(data, bias, res)
+    if res is None:
+        res = DenseMatrix(ctx, data.rows, data.cols, dt)
+    capi.check(_fn("dh_bias_add", dt)(ctx._h, res.ptr, data.ptr, data.rows, data.cols, bias.ptr, bias.getNumItems()))
+    return res
+
+
+def batchNormInferenceForward(res, data, gamma, beta, ema_mean, ema_var, eps, ctx: HIPContext,
+                              stat_index: int = 0) -> DenseMatrix:
+    """CUDA::BatchNormInferenceForward::apply (kernels/CUDA/BatchNorm.h:26-29)."""
+    dt = _same_dtype(data, gamma, beta, ema_mean, ema_var, res)
+    if res is None:
+        res = DenseMatrix(ctx, data.rows, data.cols, dt)
+    capi.check(_fn("dh_batchnorm_inference", dt)(ctx._h, res.ptr, data.ptr, data.rows, data.cols, gamma.ptr, beta.ptr,
+                                                 ema_mean.ptr, ema_var.ptr, gamma.rows, float(eps), stat_index))
+    return res
+
+
+def softmax(res, arg: DenseMatrix, ctx: HIPContext) -> DenseMatrix:
+    """CUDA::Softmax::apply (kernels/CUDA/Softmax.h:32-34; CPU kernels/Softmax.h:22-58)."""
+    if res is None:
+        res = DenseMatrix(ctx, arg.rows, arg.cols, arg.dtype)
+    capi.check(_fn("dh_softmax", arg.dtype)(ctx._h, res.ptr, res.row_skip, arg.ptr, arg.rows, arg.cols, arg.row_skip))
+    return res

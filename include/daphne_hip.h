@@ -1,0 +1,302 @@
+/*
+ * daphne_hip.h - C ABI of libdaphne_hip.so: the gfx950 (MI355X) device kernel set for
+ * DenseMatrix<float/double> that DAPHNE's run-time dispatches to an accelerator.
+ *
+ * Every entry point takes plain device pointers, element counts and leading dimensions
+ * (the reference's DenseMatrix::getRowSkip(), in elements). All matrices are row-major.
+ * No C++ or torch type crosses this boundary. Each entry point names the reference
+ * interface it stands in for (paths relative to the reference checkout, src/ omitted
+ * where unambiguous).
+ *
+ * Error model: every function returns a dh_status. On failure a thread-local message is
+ * available from dh_last_error(). The status selects the C++ exception type the reference
+ * would have thrown (see the enum), so a C++ caller can re-throw it unchanged.
+ *
+ * Threading: a dh_ctx may be used from several host threads; allocation bookkeeping is
+ * mutex-guarded and kernels are enqueued on the context's stream. Kernels that return a
+ * value to the host (dh_agg_all_*, domain checks of dh_ew_unary_*) synchronise that stream.
+ */
+#ifndef DAPHNE_HIP_H
+#define DAPHNE_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ------------------------------------------------------------------------------------ */
+/* status codes                                                                          */
+/* ------------------------------------------------------------------------------------ */
+typedef enum dh_status {
+    DH_OK = 0,
+    DH_ERR_RUNTIME = 1,      /* std::runtime_error: bad shapes, unknown/unsupported op code  */
+    DH_ERR_INVALID_ARG = 2,  /* std::invalid_argument: e.g. conv filter larger than image    */
+    DH_ERR_DOMAIN = 3,       /* std::domain_error: sqrt/ln/asin/acos outside their domain    */
+    DH_ERR_HIP = 4,          /* std::runtime_error carrying the HIP error string             */
+    DH_ERR_OOM = 5           /* std::runtime_error: device allocation beyond the budget      */
+} dh_status;
+
+/* Thread-local text of the last failure on the calling thread ("" if none). */
+const char *dh_last_error(void);
+
+/* ------------------------------------------------------------------------------------ */
+/* op codes - numeric values equal the reference enums, so they pass through unchanged   */
+/* ------------------------------------------------------------------------------------ */
+/* runtime/local/kernels/BinaryOpCode.h:29-55 */
+typedef enum dh_binary_op {
+    DH_BIN_ADD = 0, DH_BIN_SUB = 1, DH_BIN_MUL = 2, DH_BIN_DIV = 3, DH_BIN_POW = 4,
+    DH_BIN_MOD = 5, DH_BIN_LOG = 6, DH_BIN_EQ = 7, DH_BIN_NEQ = 8, DH_BIN_LT = 9,
+    DH_BIN_LE = 10, DH_BIN_GT = 11, DH_BIN_GE = 12, DH_BIN_MIN = 13, DH_BIN_MAX = 14,
+    DH_BIN_AND = 15, DH_BIN_OR = 16,
+    DH_BIN_BITWISE_AND = 17, /* integer only in the reference: rejected for float/double */
+    DH_BIN_CONCAT = 18       /* strings only: rejected */
+} dh_binary_op;
+
+/* runtime/local/kernels/UnaryOpCode.h:28-55 */
+typedef enum dh_unary_op {
+    DH_UN_MINUS = 0, DH_UN_ABS = 1, DH_UN_SIGN = 2, DH_UN_SQRT = 3, DH_UN_EXP = 4,
+    DH_UN_LN = 5, DH_UN_SIN = 6, DH_UN_COS = 7, DH_UN_TAN = 8, DH_UN_ASIN = 9,
+    DH_UN_ACOS = 10, DH_UN_ATAN = 11, DH_UN_SINH = 12, DH_UN_COSH = 13, DH_UN_TANH = 14,
+    DH_UN_FLOOR = 15, DH_UN_CEIL = 16, DH_UN_ROUND = 17, DH_UN_ISNAN = 18,
+    DH_UN_UPPER = 19, DH_UN_LOWER = 20 /* strings only: rejected */
+} dh_unary_op;
+
+/* runtime/local/kernels/AggOpCode.h:25-35 */
+typedef enum dh_agg_op {
+    DH_AGG_SUM = 0, DH_AGG_PROD = 1, DH_AGG_MIN = 2, DH_AGG_MAX = 3, DH_AGG_IDXMIN = 4,
+    DH_AGG_IDXMAX = 5, DH_AGG_MEAN = 6, DH_AGG_STDDEV = 7, DH_AGG_VAR = 8
+} dh_agg_op;
+
+/* ------------------------------------------------------------------------------------ */
+/* device context and allocator                                                          */
+/* replaces runtime/local/context/CUDAContext.h:29-114, CUDAContext.cpp:41-135 and       */
+/* runtime/local/kernels/CUDA/CreateCUDAContext.cpp:5-10                                 */
+/* ------------------------------------------------------------------------------------ */
+typedef struct dh_ctx dh_ctx;
+
+/* Select `device`, read its properties, set the memory budget to 90 % of total device
+ * memory (CUDAContext.cpp:49-50) and create the reduction workspace. */
+dh_status dh_ctx_create(int device, dh_ctx **out);
+/* Frees every allocation still registered, the workspace and the context. */
+dh_status dh_ctx_destroy(dh_ctx *ctx);
+/* CUDAContext::getMemBudget() (CUDAContext.h:83). */
+size_t dh_ctx_mem_budget(const dh_ctx *ctx);
+/* Bytes currently handed out by dh_malloc on this context. */
+size_t dh_ctx_mem_in_use(const dh_ctx *ctx);
+int dh_ctx_device(const dh_ctx *ctx);
+/* Number of compute units and the max engine clock in kHz (for roofline print-outs). */
+dh_status dh_ctx_props(const dh_ctx *ctx, int *compute_units, int *clock_khz, size_t *total_mem,
+                       char *name, size_t name_cap);
+/* Enqueue kernels of this context on `hip_stream` (a hipStream_t; NULL = the default
+ * stream, which is also the initial setting). The context never owns the stream. */
+dh_status dh_ctx_set_stream(dh_ctx *ctx, void *hip_stream);
+void *dh_ctx_get_stream(const dh_ctx *ctx);
+/* Blocks until all work enqueued on the context's stream has finished. */
+dh_status dh_sync(dh_ctx *ctx);
+
+/* CUDAContext::malloc(size, zero, id) / free(id) (CUDAContext.cpp:120-135). The device
+ * pointer itself is the registry key. Fails with DH_ERR_OOM past the budget. */
+dh_status dh_malloc(dh_ctx *ctx, size_t bytes, int zero, void **out);
+dh_status dh_free(dh_ctx *ctx, void *ptr);
+/* AllocationDescriptorCUDA::transferTo / transferFrom
+ * (runtime/local/datastructures/AllocationDescriptorCUDA.h:56-68): synchronous copies. */
+dh_status dh_h2d(dh_ctx *ctx, void *dst_dev, const void *src_host, size_t bytes);
+dh_status dh_d2h(dh_ctx *ctx, void *dst_host, const void *src_dev, size_t bytes);
+dh_status dh_d2d(dh_ctx *ctx, void *dst_dev, const void *src_dev, size_t bytes);
+
+/* Stream-ordered stopwatch on the context's stream (hipEvent pair). dh_timer_stop_ms
+ * synchronises on the stop event and returns the elapsed milliseconds. */
+dh_status dh_timer_start(dh_ctx *ctx);
+dh_status dh_timer_stop_ms(dh_ctx *ctx, float *ms);
+
+/* ------------------------------------------------------------------------------------ */
+/* elementwise                                                                           */
+/* ------------------------------------------------------------------------------------ */
+/* CUDA::EwBinaryMat<DenseMatrix<VT>,...>::apply (kernels/CUDA/EwBinaryMat.h:31-47,
+ * EwBinaryMat.cu:97-263) with the CPU kernel's semantics (kernels/EwBinaryMat.h:54-108,
+ * EwBinarySca.h:143-167): res has the shape of lhs; rhs is the same shape, a 1 x cols
+ * row vector, or a rows x 1 column vector, else DH_ERR_RUNTIME. All 17 floating-point op
+ * codes are supported. res may alias lhs (or rhs of the same shape). */
+dh_status dh_ew_binary_f32(dh_ctx *ctx, int op, float *res, size_t ld_res, const float *lhs,
+                           size_t lhs_rows, size_t lhs_cols, size_t ld_lhs, const float *rhs,
+                           size_t rhs_rows, size_t rhs_cols, size_t ld_rhs);
+dh_status dh_ew_binary_f64(dh_ctx *ctx, int op, double *res, size_t ld_res, const double *lhs,
+                           size_t lhs_rows, size_t lhs_cols, size_t ld_lhs, const double *rhs,
+                           size_t rhs_rows, size_t rhs_cols, size_t ld_rhs);
+
+/* CUDA::EwBinaryObjSca<DenseMatrix<VT>,DenseMatrix<VT>,VT>::apply
+ * (kernels/CUDA/EwBinaryObjSca.h:37-60, .cu:31-88; CPU kernels/EwBinaryObjSca.h:57-79). */
+dh_status dh_ew_binary_sca_f32(dh_ctx *ctx, int op, float *res, size_t ld_res, const float *lhs,
+                               size_t rows, size_t cols, size_t ld_lhs, float rhs);
+dh_status dh_ew_binary_sca_f64(dh_ctx *ctx, int op, double *res, size_t ld_res, const double *lhs,
+                               size_t rows, size_t cols, size_t ld_lhs, double rhs);
+
+/* EwUnaryMat<DenseMatrix<VT>,DenseMatrix<VT>>::apply (kernels/EwUnaryMat.h:57-77,
+ * EwUnarySca.h:182-206); no device version exists in the reference. SQRT/LN with an
+ * argument below zero and ASIN/ACOS outside [-1,1] return DH_ERR_DOMAIN
+ * (EwUnarySca.h:134-157); res then holds what libm produced (NaN at the offending items).
+ * Only these four op codes synchronise the stream. */
+dh_status dh_ew_unary_f32(dh_ctx *ctx, int op, float *res, size_t ld_res, const float *arg,
+                          size_t rows, size_t cols, size_t ld_arg);
+dh_status dh_ew_unary_f64(dh_ctx *ctx, int op, double *res, size_t ld_res, const double *arg,
+                          size_t rows, size_t cols, size_t ld_arg);
+
+/* ------------------------------------------------------------------------------------ */
+/* aggregations                                                                          */
+/* ------------------------------------------------------------------------------------ */
+/* CUDA::AggAll<VT,DenseMatrix<VT>>::apply (kernels/CUDA/AggAll.h:28-50, .cu:109-151; CPU
+ * kernels/AggAll.h:124-193): SUM PROD MIN MAX MEAN VAR STDDEV (population variance).
+ * The scalar is written to *result_host after a stream synchronise. */
+dh_status dh_agg_all_f32(dh_ctx *ctx, int op, const float *arg, size_t rows, size_t cols,
+                         size_t ld, float *result_host);
+dh_status dh_agg_all_f64(dh_ctx *ctx, int op, const double *arg, size_t rows, size_t cols,
+                         size_t ld, double *result_host);
+/* Same, but the scalar stays on the device (result_dev[0]); no synchronisation. */
+dh_status dh_agg_all_dev_f32(dh_ctx *ctx, int op, const float *arg, size_t rows, size_t cols,
+                             size_t ld, float *result_dev);
+dh_status dh_agg_all_dev_f64(dh_ctx *ctx, int op, const double *arg, size_t rows, size_t cols,
+                             size_t ld, double *result_dev);
+
+/* CUDA::AggRow<DenseMatrix<VT>,DenseMatrix<VT>>::apply (kernels/CUDA/AggRow.h:30-52,
+ * .cu:108-143; CPU kernels/AggRow.h:60-161): res is rows x 1 with leading dimension
+ * ld_res. SUM PROD MIN MAX MEAN VAR STDDEV. */
+dh_status dh_agg_row_f32(dh_ctx *ctx, int op, float *res, size_t ld_res, const float *arg,
+                         size_t rows, size_t cols, size_t ld);
+dh_status dh_agg_row_f64(dh_ctx *ctx, int op, double *res, size_t ld_res, const double *arg,
+                         size_t rows, size_t cols, size_t ld);
+/* RowIdxMin / RowIdxMax = AggRow<DenseMatrix<size_t>,DenseMatrix<VT>> with IDXMIN / IDXMAX
+ * (kernels/AggRow.h:71-94; op idxminRow, ir/daphneir/DaphneOps.td:544): first index of the
+ * strict extremum, 64-bit unsigned output. No device version exists in the reference. */
+dh_status dh_agg_row_idx_f32(dh_ctx *ctx, int op, uint64_t *res, size_t ld_res, const float *arg,
+                             size_t rows, size_t cols, size_t ld);
+dh_status dh_agg_row_idx_f64(dh_ctx *ctx, int op, uint64_t *res, size_t ld_res,
+                             const double *arg, size_t rows, size_t cols, size_t ld);
+
+/* CUDA::AggCol<DenseMatrix<VT>,DenseMatrix<VT>>::apply (kernels/CUDA/AggCol.h:30-52,
+ * .cu:45-86; CPU kernels/AggCol.h:58-178): res is 1 x cols. */
+dh_status dh_agg_col_f32(dh_ctx *ctx, int op, float *res, const float *arg, size_t rows,
+                         size_t cols, size_t ld);
+dh_status dh_agg_col_f64(dh_ctx *ctx, int op, double *res, const double *arg, size_t rows,
+                         size_t cols, size_t ld);
+/* AggCol with IDXMIN / IDXMAX (kernels/AggCol.h:70-122): first row of the strict extremum
+ * per column. */
+dh_status dh_agg_col_idx_f32(dh_ctx *ctx, int op, uint64_t *res, const float *arg, size_t rows,
+                             size_t cols, size_t ld);
+dh_status dh_agg_col_idx_f64(dh_ctx *ctx, int op, uint64_t *res, const double *arg, size_t rows,
+                             size_t cols, size_t ld);
+
+/* ------------------------------------------------------------------------------------ */
+/* contractions                                                                          */
+/* ------------------------------------------------------------------------------------ */
+/* CUDA::MatMul<DenseMatrix<T>,...>::apply (kernels/CUDA/MatMul.h:31-51, MatMul.cpp:45-91;
+ * CPU kernels/MatMul.cpp:248-290): res = op(lhs) * op(rhs), alpha = 1, beta = 0. The shapes
+ * are those of the stored matrices; the transposes are applied by the kernel. Returns
+ * DH_ERR_RUNTIME if the inner dimensions differ (MatMul.cpp:256-259). Matrix-vector and
+ * vector-vector shapes take streaming paths (MatMul.cpp:277-283). */
+dh_status dh_matmul_f32(dh_ctx *ctx, float *res, size_t ld_res, const float *lhs, size_t lhs_rows,
+                        size_t lhs_cols, size_t ld_lhs, const float *rhs, size_t rhs_rows,
+                        size_t rhs_cols, size_t ld_rhs, int transa, int transb);
+dh_status dh_matmul_f64(dh_ctx *ctx, double *res, size_t ld_res, const double *lhs,
+                        size_t lhs_rows, size_t lhs_cols, size_t ld_lhs, const double *rhs,
+                        size_t rhs_rows, size_t rhs_cols, size_t ld_rhs, int transa, int transb);
+
+/* CUDA::Syrk<DenseMatrix<VT>,DenseMatrix<VT>>::apply (kernels/CUDA/Syrk.h:29-46,
+ * Syrk.cu:54-87) with the CPU signature that carries transLeft (kernels/Syrk.h:51-93):
+ * res = transLeft ? arg^T * arg : arg * arg^T, full symmetric n x n (both triangles). */
+dh_status dh_syrk_f32(dh_ctx *ctx, float *res, size_t ld_res, const float *arg, size_t rows,
+                      size_t cols, size_t ld, int trans_left);
+dh_status dh_syrk_f64(dh_ctx *ctx, double *res, size_t ld_res, const double *arg, size_t rows,
+                      size_t cols, size_t ld, int trans_left);
+
+/* CUDA::Solve<DenseMatrix<VT>,...>::apply (kernels/CUDA/Solve.cpp:75-151, cuSOLVER getrf/getrs;
+ * CPU kernels/Solve.h:86-116, LAPACKE_?gesv): solves A x = b for one right-hand side by LU with
+ * partial pivoting. A is n x n with leading dimension lda and is left untouched; x and b hold n
+ * values. DH_ERR_RUNTIME if a pivot is exactly zero (Solve.h:113-115). Synchronises the stream. */
+dh_status dh_solve_f32(dh_ctx *ctx, float *x, const float *A, size_t n, size_t lda, const float *b);
+dh_status dh_solve_f64(dh_ctx *ctx, double *x, const double *A, size_t n, size_t lda, const double *b);
+
+/* ------------------------------------------------------------------------------------ */
+/* DNN inference ops (NCHW images flattened to rows: one image per matrix row)           */
+/* ------------------------------------------------------------------------------------ */
+/* CUDA::Convolution::Forward<...>::apply (kernels/CUDA/Convolution.h:33-38, .cpp:21-135;
+ * CPU kernels/Conv2DForward.h:77-140): cross-correlation, data N x (C*H*W), filter
+ * filter_rows x filter_cols = F x (C*Hf*Wf), res N x (F*P*Q) with
+ * P = (H + 2*pad_h - Hf)/stride_h + 1. bias is F values or NULL (no bias, as the CUDA kernel
+ * allows). *res_h / *res_w receive P / Q. DH_ERR_INVALID_ARG if the filter does not hold
+ * F*C*Hf*Wf items (Convolution.cpp:32-39) or exceeds the padded image. */
+dh_status dh_conv2d_forward_f32(dh_ctx *ctx, float *res, size_t *res_h, size_t *res_w,
+                                const float *data, const float *filter, size_t filter_rows,
+                                size_t filter_cols, const float *bias, size_t batch,
+                                size_t channels, size_t img_h, size_t img_w, size_t filter_h,
+                                size_t filter_w, size_t stride_h, size_t stride_w, size_t pad_h,
+                                size_t pad_w);
+dh_status dh_conv2d_forward_f64(dh_ctx *ctx, double *res, size_t *res_h, size_t *res_w,
+                                const double *data, const double *filter, size_t filter_rows,
+                                size_t filter_cols, const double *bias, size_t batch,
+                                size_t channels, size_t img_h, size_t img_w, size_t filter_h,
+                                size_t filter_w, size_t stride_h, size_t stride_w, size_t pad_h,
+                                size_t pad_w);
+
+/* CUDA::NN::Pooling::Forward<MAX,...>::apply (kernels/CUDA/Pooling.h:31-35, .cpp:22-65) with
+ * the CPU kernel's arithmetic (kernels/Pooling.cpp:28-107, Pooling.h:46-54,
+ * MaxPoolForward.h:35-44): the result is max(0, window) because the CPU kernel folds the
+ * window into a zero-initialised output; P is derived with stride_w and Q with stride_h
+ * (Pooling.cpp:38-39); windows are clipped at the image border. */
+dh_status dh_maxpool_forward_f32(dh_ctx *ctx, float *res, size_t *res_h, size_t *res_w,
+                                 const float *data, size_t batch, size_t channels, size_t img_h,
+                                 size_t img_w, size_t pool_h, size_t pool_w, size_t stride_h,
+                                 size_t stride_w, size_t pad_h, size_t pad_w);
+dh_status dh_maxpool_forward_f64(dh_ctx *ctx, double *res, size_t *res_h, size_t *res_w,
+                                 const double *data, size_t batch, size_t channels, size_t img_h,
+                                 size_t img_w, size_t pool_h, size_t pool_w, size_t stride_h,
+                                 size_t stride_w, size_t pad_h, size_t pad_w);
+
+/* CUDA::NN::Affine::Forward<...>::apply (kernels/CUDA/Affine.h:24-26, Affine.cpp:42-83):
+ * res = data * weights (+ bias broadcast over rows). bias may be NULL. DH_ERR_RUNTIME if
+ * data_cols != w_rows or bias is not 1 x w_cols (Affine.cpp:50-60). */
+dh_status dh_affine_forward_f32(dh_ctx *ctx, float *res, const float *data, size_t data_rows,
+                                size_t data_cols, const float *weights, size_t w_rows,
+                                size_t w_cols, const float *bias, size_t bias_rows,
+                                size_t bias_cols);
+dh_status dh_affine_forward_f64(dh_ctx *ctx, double *res, const double *data, size_t data_rows,
+                                size_t data_cols, const double *weights, size_t w_rows,
+                                size_t w_cols, const double *bias, size_t bias_rows,
+                                size_t bias_cols);
+
+/* CUDA::BiasAdd<...>::apply (kernels/CUDA/BiasAdd.h:26-28, BiasAdd.cpp:20-55; CPU
+ * kernels/BiasAdd.h:34-52): res[i, c*HW + j] = data[i, c*HW + j] + bias[c], HW = cols /
+ * num_bias. num_bias is the bias item count (rows for the CPU test's C x 1 bias, cols for
+ * the CUDA test's 1 x C bias). */
+dh_status dh_bias_add_f32(dh_ctx *ctx, float *res, const float *data, size_t rows, size_t cols,
+                          const float *bias, size_t num_bias);
+dh_status dh_bias_add_f64(dh_ctx *ctx, double *res, const double *data, size_t rows, size_t cols,
+                          const double *bias, size_t num_bias);
+
+/* CUDA::BatchNormInferenceForward<...>::apply (kernels/CUDA/BatchNorm.h:26-29, .cpp:21-55;
+ * CPU kernels/BatchNorm2DTestForward.h:77-101):
+ *   res = gamma_s * (x - mean_s) / sqrt(var_s + eps) + beta_s.
+ * stat_index = 0: s is the channel of the element, channels = rows of gamma (the cuDNN
+ * spatial mode of the CUDA kernel); stat_index = 1: s is the row (image) index, which is
+ * what the CPU kernel does (BatchNorm2DTestForward.h:96-97). */
+dh_status dh_batchnorm_inference_f32(dh_ctx *ctx, float *res, const float *data, size_t rows,
+                                     size_t cols, const float *gamma, const float *beta,
+                                     const float *ema_mean, const float *ema_var,
+                                     size_t channels, float eps, int stat_index);
+dh_status dh_batchnorm_inference_f64(dh_ctx *ctx, double *res, const double *data, size_t rows,
+                                     size_t cols, const double *gamma, const double *beta,
+                                     const double *ema_mean, const double *ema_var,
+                                     size_t channels, double eps, int stat_index);
+
+/* CUDA::Softmax<...>::apply (kernels/CUDA/Softmax.h:32-34, Softmax.cpp:22-48; CPU
+ * kernels/Softmax.h:22-58): row-wise exp(x - max) / sum. */
+dh_status dh_softmax_f32(dh_ctx *ctx, float *res, size_t ld_res, const float *arg, size_t rows,
+                         size_t cols, size_t ld);
+dh_status dh_softmax_f64(dh_ctx *ctx, double *res, size_t ld_res, const double *arg, size_t rows,
+                         size_t cols, size_t ld);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DAPHNE_HIP_H */

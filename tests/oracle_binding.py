@@ -1,0 +1,162 @@
+"""ctypes binding of oracle/liboracle.so - the CPU restatement of the reference's kernels.
+
+Test infrastructure only. Builds the library with `make -C oracle` if it is missing.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import subprocess
+from pathlib import Path
+
+import numpy as np
+
+ORACLE_DIR = Path(__file__).resolve().parent.parent / "oracle"
+LIB = ORACLE_DIR / "liboracle.so"
+
+ST_OK, ST_RUNTIME, ST_INVALID, ST_DOMAIN = 0, 1, 2, 3
+_SUF = {np.dtype(np.float32): "f32", np.dtype(np.float64): "f64"}
+_lib = None
+
+
+def lib() -> C.CDLL:
+    global _lib
+    if _lib is None:
+        if not LIB.exists():
+            subprocess.run(["make", "-C", str(ORACLE_DIR)], check=True, capture_output=True)
+        _lib = C.CDLL(str(LIB))
+    return _lib
+
+
+def _p(a):
+    return C.c_void_p(a.ctypes.data) if a is not None else None
+
+
+def _f(name, dt):
+    return getattr(lib(), f"oracle_{name}_{_SUF[np.dtype(dt)]}")
+
+
+def _sc(dt, v):
+    return C.c_float(v) if np.dtype(dt) == np.float32 else C.c_double(v)
+
+
+def _ld(a):
+    """Leading dimension (elements) of a 2-D row-major array or view."""
+    assert a.ndim == 2 and (a.shape[1] <= 1 or a.strides[1] == a.itemsize)
+    return a.strides[0] // a.itemsize if a.shape[0] > 1 else max(a.shape[1], 1)
+
+
+sz = C.c_size_t
+
+
+def ew_binary(op, lhs, rhs):
+    res = np.empty(lhs.shape, lhs.dtype)
+    st = _f("ew_binary", lhs.dtype)(int(op), _p(res), sz(_ld(res)), _p(lhs), sz(lhs.shape[0]), sz(lhs.shape[1]),
+                                    sz(_ld(lhs)), _p(rhs), sz(rhs.shape[0]), sz(rhs.shape[1]), sz(_ld(rhs)))
+    return st, res
+
+
+def ew_binary_sca(op, lhs, s):
+    res = np.empty(lhs.shape, lhs.dtype)
+    st = _f("ew_binary_sca", lhs.dtype)(int(op), _p(res), sz(_ld(res)), _p(lhs), sz(lhs.shape[0]), sz(lhs.shape[1]),
+                                        sz(_ld(lhs)), _sc(lhs.dtype, s))
+    return st, res
+
+
+def ew_unary(op, arg):
+    res = np.empty(arg.shape, arg.dtype)
+    st = _f("ew_unary", arg.dtype)(int(op), _p(res), sz(_ld(res)), _p(arg), sz(arg.shape[0]), sz(arg.shape[1]),
+                                   sz(_ld(arg)))
+    return st, res
+
+
+def agg_all(op, arg):
+    out = np.empty(1, arg.dtype)
+    st = _f("agg_all", arg.dtype)(int(op), _p(arg), sz(arg.shape[0]), sz(arg.shape[1]), sz(_ld(arg)), _p(out))
+    return st, out[0]
+
+
+def agg_row(op, arg):
+    if int(op) in (4, 5):
+        res = np.empty((arg.shape[0], 1), np.uint64)
+        st = _f("agg_row_idx", arg.dtype)(int(op), _p(res), sz(1), _p(arg), sz(arg.shape[0]), sz(arg.shape[1]),
+                                          sz(_ld(arg)))
+        return st, res
+    res = np.empty((arg.shape[0], 1), arg.dtype)
+    st = _f("agg_row", arg.dtype)(int(op), _p(res), sz(1), _p(arg), sz(arg.shape[0]), sz(arg.shape[1]), sz(_ld(arg)))
+    return st, res
+
+
+def agg_col(op, arg):
+    if int(op) in (4, 5):
+        res = np.empty((1, arg.shape[1]), np.uint64)
+        st = _f("agg_col_idx", arg.dtype)(int(op), _p(res), _p(arg), sz(arg.shape[0]), sz(arg.shape[1]), sz(_ld(arg)))
+        return st, res
+    res = np.empty((1, arg.shape[1]), arg.dtype)
+    st = _f("agg_col", arg.dtype)(int(op), _p(res), _p(arg), sz(arg.shape[0]), sz(arg.shape[1]), sz(_ld(arg)))
+    return st, res
+
+
+def matmul(lhs, rhs, ta=False, tb=False):
+    nr1 = lhs.shape[1] if ta else lhs.shape[0]
+    nc2 = rhs.shape[0] if tb else rhs.shape[1]
+    res = np.empty((nr1, nc2), lhs.dtype)
+    st = _f("matmul", lhs.dtype)(_p(res), sz(max(nc2, 1)), _p(lhs), sz(lhs.shape[0]), sz(lhs.shape[1]), sz(_ld(lhs)),
+                                 _p(rhs), sz(rhs.shape[0]), sz(rhs.shape[1]), sz(_ld(rhs)), int(ta), int(tb))
+    return st, res
+
+
+def syrk(arg, trans_left=True):
+    n = arg.shape[1] if trans_left else arg.shape[0]
+    res = np.empty((n, n), arg.dtype)
+    st = _f("syrk", arg.dtype)(_p(res), sz(n), _p(arg), sz(arg.shape[0]), sz(arg.shape[1]), sz(_ld(arg)),
+                               int(trans_left))
+    return st, res
+
+
+def solve(A, b):
+    A = np.ascontiguousarray(A)
+    b = np.ascontiguousarray(b).reshape(-1)
+    x = np.empty(b.shape, A.dtype)
+    st = _f("solve", A.dtype)(_p(x), _p(A), sz(A.shape[0]), _p(b))
+    return st, x.reshape(-1, 1)
+
+
+def conv2d(data, filt, bias, N, Cc, H, W, Hf, Wf, sh, sw, ph, pw):
+    F = filt.shape[0]
+    P = (H + 2 * ph - Hf) // sh + 1
+    Q = (W + 2 * pw - Wf) // sw + 1
+    res = np.empty((N, F * P * Q), data.dtype)
+    rh, rw = sz(), sz()
+    st = _f("conv2d_forward", data.dtype)(_p(res), C.byref(rh), C.byref(rw), _p(data), _p(filt), _p(bias), sz(N),
+                                          sz(Cc), sz(H), sz(W), sz(F), sz(Hf), sz(Wf), sz(sh), sz(sw), sz(ph), sz(pw))
+    return st, res, rh.value, rw.value
+
+
+def maxpool(data, N, Cc, H, W, ph, pw, sh, sw, padh, padw):
+    P = (H + 2 * padh - ph) // sw + 1
+    Q = (W + 2 * padw - pw) // sh + 1
+    res = np.empty((N, Cc * P * Q), data.dtype)
+    rh, rw = sz(), sz()
+    st = _f("maxpool_forward", data.dtype)(_p(res), C.byref(rh), C.byref(rw), _p(data), sz(N), sz(Cc), sz(H), sz(W),
+                                           sz(ph), sz(pw), sz(sh), sz(sw), sz(padh), sz(padw))
+    return st, res, rh.value, rw.value
+
+
+def bias_add(data, bias):
+    res = np.empty(data.shape, data.dtype)
+    st = _f("bias_add", data.dtype)(_p(res), _p(data), sz(data.shape[0]), sz(data.shape[1]), _p(bias), sz(bias.size))
+    return st, res
+
+
+def batchnorm(data, gamma, beta, mean, var, eps, stat_index=0):
+    res = np.empty(data.shape, data.dtype)
+    st = _f("batchnorm_inference", data.dtype)(_p(res), _p(data), sz(data.shape[0]), sz(data.shape[1]), _p(gamma),
+                                               _p(beta), _p(mean), _p(var), sz(gamma.shape[0]), _sc(data.dtype, eps),
+                                               int(stat_index))
+    return st, res
+
+
+def softmax(arg):
+    res = np.empty(arg.shape, arg.dtype)
+    st = _f("softmax", arg.dtype)(_p(res), sz(_ld(res)), _p(arg), sz(arg.shape[0]), sz(arg.shape[1]), sz(_ld(arg)))
+    return st, res
