@@ -98,3 +98,30 @@ template <> struct dh_vec<double> {
 
 template <typename T> __device__ __forceinline__ T dh_shfl_xor(T v, int mask) { return __shfl_xor(v, mask, DH_WAVE); }
 template <typename T> __device__ __forceinline__ T dh_shfl_down(T v, int d) { return __shfl_down(v, d, DH_WAVE); }
+
+// 16-byte (VEC = 16 / sizeof(T)) or scalar (VEC = 1) global load / store into a register array.
+template <typename T, int VEC> __device__ __forceinline__ void dh_load_vec(const T *p, T (&v)[VEC]) {
+    if constexpr (VEC == 1) {
+        v[0] = *p;
+    } else {
+        using V = typename dh_vec<T>::type;
+        const V t = *reinterpret_cast<const V *>(p);
+        const T *tp = reinterpret_cast<const T *>(&t);
+#pragma unroll
+        for (int i = 0; i < VEC; i++)
+            v[i] = tp[i];
+    }
+}
+template <typename T, int VEC> __device__ __forceinline__ void dh_store_vec(T *p, const T (&v)[VEC]) {
+    if constexpr (VEC == 1) {
+        *p = v[0];
+    } else {
+        using V = typename dh_vec<T>::type;
+        V t;
+        T *tp = reinterpret_cast<T *>(&t);
+#pragma unroll
+        for (int i = 0; i < VEC; i++)
+            tp[i] = v[i];
+        *reinterpret_cast<V *>(p) = t;
+    }
+}

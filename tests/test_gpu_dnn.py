@@ -1,0 +1,133 @@
+"""GPU parity: Conv2D / MaxPool / BiasAdd / BatchNorm / Softmax (through the C ABI) vs the CPU oracle."""
+import numpy as np
+import pytest
+
+import oracle_binding as orc
+from parity import assert_close, assert_exact
+
+pytestmark = pytest.mark.gpu
+
+from daphne_amd import capi
+from daphne_amd.kernels import (DenseMatrix, batchNormInferenceForward, biasAdd, conv2dForward, maxPoolForward,
+                                softmax)
+
+DTYPES = [np.float32, np.float64]
+
+CONV_CASES = [  # N, C, H, W, F, Hf, Wf, sh, sw, ph, pw
+    (2, 3, 3, 3, 1, 2, 2, 2, 2, 1, 1),
+    (1, 1, 3, 3, 1, 2, 2, 1, 1, 0, 0),
+    (5, 1, 28, 28, 32, 5, 5, 1, 1, 2, 2),
+    (3, 32, 14, 14, 64, 5, 5, 1, 1, 2, 2),
+    (4, 3, 17, 13, 70, 3, 5, 2, 1, 1, 2),
+    (2, 8, 9, 9, 130, 3, 3, 1, 2, 0, 1),
+    (130, 2, 5, 6, 5, 1, 1, 1, 1, 0, 0),
+    (1, 4, 7, 7, 3, 7, 7, 1, 1, 0, 0),
+]
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("case", CONV_CASES)
+def test_conv2d(ctx, dt, case):
+    N, C, H, W, F, Hf, Wf, sh, sw, ph, pw = case
+    rng = np.random.default_rng(sum(case))
+    x = rng.random((N, C * H * W)).astype(dt)
+    w = (rng.standard_normal((F, C * Hf * Wf)) * np.sqrt(2.0 / (C * Hf * Wf))).astype(dt)
+    b = (rng.standard_normal((F, 1)) * 0.1).astype(dt)
+    st, exp, eh, ew_ = orc.conv2d(x, w, b, N, C, H, W, Hf, Wf, sh, sw, ph, pw)
+    assert st == 0
+    X, Wd, B = DenseMatrix.from_numpy(ctx, x), DenseMatrix.from_numpy(ctx, w), DenseMatrix.from_numpy(ctx, b)
+    got, gh, gw = conv2dForward(None, X, Wd, B, N, C, H, W, Hf, Wf, sh, sw, ph, pw, ctx)
+    assert (gh, gw) == (eh, ew_)
+    assert_close(got.to_numpy(), exp, elementwise=False)
+    # without bias (allowed by the reference's CUDA kernel)
+    st, exp0, _, _ = orc.conv2d(x, w, None, N, C, H, W, Hf, Wf, sh, sw, ph, pw)
+    got0, _, _ = conv2dForward(None, X, Wd, None, N, C, H, W, Hf, Wf, sh, sw, ph, pw, ctx)
+    assert_close(got0.to_numpy(), exp0, elementwise=False)
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+def test_conv2d_integer_valued_exact(ctx, dt):
+    rng = np.random.default_rng(4)
+    N, C, H, W, F, Hf, Wf = 3, 5, 11, 12, 40, 3, 3
+    x = rng.integers(-3, 4, (N, C * H * W)).astype(dt)
+    w = rng.integers(-3, 4, (F, C * Hf * Wf)).astype(dt)
+    b = rng.integers(-3, 4, (F, 1)).astype(dt)
+    st, exp, _, _ = orc.conv2d(x, w, b, N, C, H, W, Hf, Wf, 1, 1, 1, 1)
+    got, _, _ = conv2dForward(None, DenseMatrix.from_numpy(ctx, x), DenseMatrix.from_numpy(ctx, w),
+                              DenseMatrix.from_numpy(ctx, b), N, C, H, W, Hf, Wf, 1, 1, 1, 1, ctx)
+    assert_exact(got.to_numpy(), exp)
+
+
+def test_conv2d_filter_mismatch(ctx):
+    x = DenseMatrix.from_numpy(ctx, np.ones((1, 9), np.float32))
+    w = DenseMatrix.from_numpy(ctx, np.ones((1, 5), np.float32))
+    with pytest.raises(capi.DaphneHipInvalidArgument, match="Convolution kernel dimension mismatch"):
+        conv2dForward(None, x, w, None, 1, 1, 3, 3, 2, 2, 1, 1, 0, 0, ctx)
+
+
+POOL_CASES = [  # N, C, H, W, ph, pw, sh, sw, padh, padw
+    (2, 3, 5, 5, 2, 2, 2, 2, 1, 1),
+    (2, 3, 5, 5, 2, 2, 1, 1, 0, 0),
+    (3, 32, 28, 28, 2, 2, 2, 2, 0, 0),
+    (3, 64, 14, 14, 2, 2, 2, 2, 0, 0),
+    (2, 2, 9, 7, 3, 3, 2, 2, 1, 1),
+    (2, 2, 9, 7, 3, 2, 3, 3, 0, 0),
+    (4, 5, 6, 1, 6, 1, 1, 1, 0, 0),   # P == Q == 1 and W == 1: the reference's quick path
+    (1, 1, 4, 4, 4, 4, 1, 1, 0, 0),
+]
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("case", POOL_CASES)
+def test_maxpool(ctx, dt, case):
+    N, C, H, W, ph, pw, sh, sw, padh, padw = case
+    rng = np.random.default_rng(sum(case))
+    x = (rng.standard_normal((N, C * H * W))).astype(dt)  # negative values: the result is max(0, window)
+    st, exp, eh, ew_ = orc.maxpool(x, N, C, H, W, ph, pw, sh, sw, padh, padw)
+    assert st == 0
+    got, gh, gw = maxPoolForward(None, DenseMatrix.from_numpy(ctx, x), N, C, H, W, ph, pw, sh, sw, padh, padw, ctx)
+    assert (gh, gw) == (eh, ew_)
+    assert_exact(got.to_numpy(), exp)
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("rows,C,HW", [(2, 3, 9), (7, 32, 784), (5, 64, 196), (9, 10, 1), (3, 5, 7), (100, 1, 33)])
+def test_bias_add(ctx, dt, rows, C, HW):
+    rng = np.random.default_rng(rows + C + HW)
+    x = rng.standard_normal((rows, C * HW)).astype(dt)
+    for bshape in ((C, 1), (1, C)):  # CPU test uses C x 1, the CUDA test 1 x C
+        b = rng.standard_normal(bshape).astype(dt)
+        st, exp = orc.bias_add(x, b)
+        got = biasAdd(None, DenseMatrix.from_numpy(ctx, x), DenseMatrix.from_numpy(ctx, b), ctx).to_numpy()
+        assert_exact(got, exp)
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("rows,C,HW", [(1, 1, 9), (2, 3, 9), (6, 16, 49), (5, 7, 3)])
+def test_batchnorm_inference(ctx, dt, rows, C, HW):
+    rng = np.random.default_rng(rows * 7 + C)
+    x = rng.standard_normal((rows, C * HW)).astype(dt)
+    eps = 1e-5
+    for stat_index, S in ((0, C), (1, rows)):
+        gamma = (rng.random((S, 1)) + 0.5).astype(dt)
+        beta = rng.standard_normal((S, 1)).astype(dt)
+        mean = rng.standard_normal((S, 1)).astype(dt)
+        var = (rng.random((S, 1)) + 0.1).astype(dt)
+        st, exp = orc.batchnorm(x, gamma, beta, mean, var, eps, stat_index)
+        assert st == 0
+        d = lambda a: DenseMatrix.from_numpy(ctx, a)
+        got = batchNormInferenceForward(None, d(x), d(gamma), d(beta), d(mean), d(var), eps, ctx, stat_index).to_numpy()
+        assert_close(got, exp, rtol=2e-5 if dt == np.float32 else 1e-12, elementwise=False)
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("rows,cols", [(3, 3), (1, 9), (4096, 10), (7, 1), (33, 1000), (5, 64)])
+def test_softmax(ctx, dt, rows, cols):
+    rng = np.random.default_rng(rows + cols)
+    x = (rng.standard_normal((rows, cols)) * 4).astype(dt)
+    if rows > 2 and cols > 2:
+        x[1, 1] = np.nan
+        x[2, 0] = np.inf
+    st, exp = orc.softmax(x)
+    got = softmax(None, DenseMatrix.from_numpy(ctx, x), ctx).to_numpy()
+    assert_close(got, exp)

@@ -1,0 +1,192 @@
+"""GPU parity: MatMul / Syrk / Solve / Affine (through the C ABI) against the CPU oracle.
+
+Tolerance: norm-wise relative error max|got - exp| / max|exp| <= 1e-4 (float) / 1e-10 (double):
+the reference's BLAS and the MFMA kernels sum in different orders, so single entries that are
+sums with heavy cancellation cannot be compared relative to themselves. Integer-valued inputs
+(every partial sum exactly representable) must match bit for bit in any order.
+"""
+import numpy as np
+import pytest
+
+import oracle_binding as orc
+from parity import assert_close, assert_exact
+
+pytestmark = pytest.mark.gpu
+
+from daphne_amd import capi
+from daphne_amd.kernels import DenseMatrix, affineForward, matMul, solve, syrk
+
+DTYPES = [np.float32, np.float64]
+
+SHAPES = [  # (m, n, k)
+    (1, 1, 1), (3, 5, 7), (16, 16, 16), (33, 17, 65), (128, 128, 128), (129, 127, 130), (200, 300, 50),
+    (256, 32, 64), (1000, 16, 64), (16, 64, 3000), (20, 300, 40), (5, 5, 20000), (260, 7, 9), (384, 512, 640),
+]
+
+
+def _stored(rng, r, c, dt, trans):
+    a = (rng.random((c, r) if trans else (r, c)) * 2 - 1).astype(dt)
+    return a
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False), (True, True)])
+@pytest.mark.parametrize("m,n,k", SHAPES)
+def test_matmul_random(ctx, dt, ta, tb, m, n, k):
+    rng = np.random.default_rng(m * 1000003 + n * 1009 + k)
+    a, b = _stored(rng, m, k, dt, ta), _stored(rng, k, n, dt, tb)
+    st, exp = orc.matmul(a, b, ta, tb)
+    assert st == 0
+    truth = (a.T if ta else a).astype(np.float64) @ (b.T if tb else b).astype(np.float64)
+    got = matMul(None, DenseMatrix.from_numpy(ctx, a), DenseMatrix.from_numpy(ctx, b), ta, tb, ctx).to_numpy()
+    assert got.shape == (m, n)
+    assert_close(got, exp, elementwise=False)
+    assert_close(got, truth.astype(dt), elementwise=False)
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False), (True, True)])
+def test_matmul_integer_valued_exact(ctx, dt, ta, tb):
+    rng = np.random.default_rng(1)
+    for (m, n, k) in [(37, 41, 53), (130, 140, 300), (8, 8, 5000), (300, 20, 64)]:
+        a = rng.integers(-4, 5, (k, m) if ta else (m, k)).astype(dt)
+        b = rng.integers(-4, 5, (n, k) if tb else (k, n)).astype(dt)
+        exp = ((a.T if ta else a).astype(np.int64) @ (b.T if tb else b).astype(np.int64)).astype(dt)
+        got = matMul(None, DenseMatrix.from_numpy(ctx, a), DenseMatrix.from_numpy(ctx, b), ta, tb, ctx).to_numpy()
+        assert_exact(got, exp)
+        assert_exact(orc.matmul(a, b, ta, tb)[1], exp)
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+def test_matmul_views(ctx, dt):
+    """rowSkip > numCols on lhs, rhs and res (kernels/MatMul.cpp:269-271 passes rowSkip as ld)."""
+    rng = np.random.default_rng(2)
+    A = (rng.random((90, 77)) - 0.5).astype(dt)
+    B = (rng.random((80, 66)) - 0.5).astype(dt)
+    dA, dB = DenseMatrix.from_numpy(ctx, A), DenseMatrix.from_numpy(ctx, B)
+    va, vb = A[5:70, 3:60], B[10:67, 1:50]  # 65x57 @ 57x49
+    res = DenseMatrix(ctx, 100, 60, dt, zero=True)
+    matMul(res.slice(7, 72, 2, 51), dA.slice(5, 70, 3, 60), dB.slice(10, 67, 1, 50), False, False, ctx)
+    full = res.to_numpy()
+    assert_close(full[7:72, 2:51], orc.matmul(va, vb)[1], elementwise=False)
+    full[7:72, 2:51] = 0
+    assert (full == 0).all(), "wrote outside the result view"
+    # unaligned leading dimensions / odd offsets with transposes
+    got = matMul(None, dA.slice(5, 62, 3, 68), dB.slice(10, 67, 1, 50), True, False, ctx).to_numpy()
+    assert_close(got, orc.matmul(A[5:62, 3:68], vb, True, False)[1], elementwise=False)
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+def test_matmul_vectors(ctx, dt):
+    """matrix-vector and vector-vector shapes (kernels/MatMul.cpp:277-283)."""
+    rng = np.random.default_rng(3)
+    A = (rng.random((500, 70)) - 0.5).astype(dt)
+    x = (rng.random((70, 1)) - 0.5).astype(dt)
+    y = (rng.random((500, 1)) - 0.5).astype(dt)
+    dA = DenseMatrix.from_numpy(ctx, A)
+    assert_close(matMul(None, dA, DenseMatrix.from_numpy(ctx, x), False, False, ctx).to_numpy(), orc.matmul(A, x)[1],
+                 elementwise=False)
+    assert_close(matMul(None, dA, DenseMatrix.from_numpy(ctx, y), True, False, ctx).to_numpy(),
+                 orc.matmul(A, y, True, False)[1], elementwise=False)
+    xr = np.ascontiguousarray(x.T)
+    assert_close(matMul(None, dA, DenseMatrix.from_numpy(ctx, xr), False, True, ctx).to_numpy(),
+                 orc.matmul(A, xr, False, True)[1], elementwise=False)
+    # dot products
+    u = (rng.random((1, 3000)) - 0.5).astype(dt)
+    v = (rng.random((3000, 1)) - 0.5).astype(dt)
+    got = matMul(None, DenseMatrix.from_numpy(ctx, u), DenseMatrix.from_numpy(ctx, v), False, False, ctx).to_numpy()
+    assert got.shape == (1, 1)
+    assert_close(got, (u.astype(np.float64) @ v.astype(np.float64)).astype(dt), rtol=1e-4 if dt == np.float32 else 1e-10,
+                 elementwise=False)
+    got = matMul(None, DenseMatrix.from_numpy(ctx, v), DenseMatrix.from_numpy(ctx, v), True, False, ctx).to_numpy()
+    assert_close(got, (v.T.astype(np.float64) @ v.astype(np.float64)).astype(dt), elementwise=False)
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+def test_matmul_shape_error(ctx, dt):
+    a = DenseMatrix.from_numpy(ctx, np.ones((4, 5), dt))
+    b = DenseMatrix.from_numpy(ctx, np.ones((4, 5), dt))
+    with pytest.raises(capi.DaphneHipError, match="#cols of lhs and #rows of rhs must be the same"):
+        matMul(None, a, b, False, False, ctx)
+    matMul(None, a, b, True, False, ctx)
+    matMul(None, a, b, False, True, ctx)
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("trans_left", [True, False])
+@pytest.mark.parametrize("rows,cols", [(7, 3), (100, 100), (1000, 100), (5000, 130), (64, 257), (20000, 16)])
+def test_syrk(ctx, dt, trans_left, rows, cols):
+    rng = np.random.default_rng(rows + cols)
+    if not trans_left:
+        rows, cols = cols, rows
+    x = (rng.random((rows, cols)) * 2 - 1).astype(dt)
+    st, exp = orc.syrk(x, trans_left)
+    got = syrk(None, DenseMatrix.from_numpy(ctx, x), trans_left, ctx).to_numpy()
+    assert_close(got, exp, elementwise=False)
+    assert_exact(got, got.T)  # the lower triangle is a copy of the upper one (Syrk.h:65-69)
+    # syrk(X) == matMul(t(X), X) (test/runtime/local/kernels/SyrkTest.cpp:32-58)
+    X = DenseMatrix.from_numpy(ctx, x)
+    mm = matMul(None, X, X, trans_left, not trans_left, ctx).to_numpy()
+    assert_close(got, mm, elementwise=False)
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+def test_syrk_integer_valued_exact(ctx, dt):
+    rng = np.random.default_rng(9)
+    x = rng.integers(-3, 4, (3000, 150)).astype(dt)
+    exp = (x.T.astype(np.int64) @ x.astype(np.int64)).astype(dt)
+    assert_exact(syrk(None, DenseMatrix.from_numpy(ctx, x), True, ctx).to_numpy(), exp)
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("n", [1, 3, 10, 100, 257])
+def test_solve(ctx, dt, n):
+    rng = np.random.default_rng(n)
+    A = (rng.random((n, n)) - 0.5).astype(dt) + np.eye(n, dtype=dt) * dt(0.1)
+    b = (rng.random((n, 1)) - 0.5).astype(dt)
+    st, exp = orc.solve(A, b)
+    assert st == 0
+    got = solve(None, DenseMatrix.from_numpy(ctx, A), DenseMatrix.from_numpy(ctx, b), ctx).to_numpy()
+    tol = (1e-3 if dt == np.float32 else 1e-9) if n > 50 else (1e-4 if dt == np.float32 else 1e-10)
+    assert_close(got, exp, rtol=tol, elementwise=False)
+    # residual against the definition
+    r = A.astype(np.float64) @ got.astype(np.float64) - b
+    assert np.abs(r).max() <= (5e-4 if dt == np.float32 else 1e-11) * max(1.0, np.abs(got).max()) * n
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+def test_solve_errors(ctx, dt):
+    A = DenseMatrix.from_numpy(ctx, np.zeros((3, 3), dt))
+    b = DenseMatrix.from_numpy(ctx, np.ones((3, 1), dt))
+    with pytest.raises(capi.DaphneHipError, match="exactly singular"):
+        solve(None, A, b, ctx)
+    with pytest.raises(capi.DaphneHipError, match="#rows and #cols of lhs must be the same"):
+        solve(None, DenseMatrix.from_numpy(ctx, np.ones((3, 2), dt)), b, ctx)
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("m,k,n", [(1, 9, 2), (64, 100, 10), (300, 3136, 512), (257, 512, 10)])
+def test_affine(ctx, dt, m, k, n):
+    """Affine = MatMul then row-vector add (the reference has no CPU affine kernel)."""
+    rng = np.random.default_rng(m + k + n)
+    x = (rng.random((m, k)) - 0.5).astype(dt)
+    w = (rng.standard_normal((k, n)) * np.sqrt(2.0 / k)).astype(dt)
+    b = (rng.standard_normal((1, n)) * 0.1).astype(dt)
+    st, mm = orc.matmul(x, w)
+    st, exp = orc.ew_binary(0, mm, b)
+    got = affineForward(None, DenseMatrix.from_numpy(ctx, x), DenseMatrix.from_numpy(ctx, w),
+                        DenseMatrix.from_numpy(ctx, b), ctx).to_numpy()
+    assert_close(got, exp, elementwise=False)
+    got = affineForward(None, DenseMatrix.from_numpy(ctx, x), DenseMatrix.from_numpy(ctx, w), None, ctx).to_numpy()
+    assert_close(got, mm, elementwise=False)
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+def test_affine_errors(ctx, dt):
+    x = DenseMatrix.from_numpy(ctx, np.ones((4, 5), dt))
+    w = DenseMatrix.from_numpy(ctx, np.ones((6, 3), dt))
+    with pytest.raises(capi.DaphneHipError, match="#cols of lhs and #rows of rhs must be the same"):
+        affineForward(None, x, w, None, ctx)
+    w = DenseMatrix.from_numpy(ctx, np.ones((5, 3), dt))
+    with pytest.raises(capi.DaphneHipError, match="bias dimensions not matching"):
+        affineForward(None, x, w, DenseMatrix.from_numpy(ctx, np.ones((3, 1), dt)), ctx)
