@@ -44,7 +44,7 @@ template <> struct Mfma<double> {
         return __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c, 0, 0, 0);
     }
     // accumulator register v of lane l holds C[row(l, v)][col(l)]
-    static __device__ __forceinline__ int row(int lane, int v) { return 4 * (lane / 16) + v; }
+    static __device__ __forceinline__ int row(int lane, int v) { return 4 * v + (lane / 16); }
     static __device__ __forceinline__ int col(int lane) { return lane % 16; }
 };
 template <> struct Mfma<float> {
