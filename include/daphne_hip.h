@@ -296,6 +296,81 @@ dh_status dh_softmax_f32(dh_ctx *ctx, float *res, size_t ld_res, const float *ar
 dh_status dh_softmax_f64(dh_ctx *ctx, double *res, size_t ld_res, const double *arg, size_t rows,
                          size_t cols, size_t ld);
 
+
+/* ------------------------------------------------------------------------------------ */
+/* fused vectorized pipeline                                                             */
+/* ------------------------------------------------------------------------------------ */
+/* Device side of VectorizedPipeline<DenseMatrix<VT>>::apply
+ * (runtime/local/kernels/VectorizedPipeline.h:35-69) and of the device worker that runs a
+ * pipeline body operator by operator on row chunks (runtime/local/vectorized/TasksCUDA.cpp:21-63,
+ * MTWrapper_dense.cpp:203-336). Here the body is given as a short instruction list and runs as
+ * one kernel over all rows: inputs split by ROWS, outputs combined by ROWS (tile / row
+ * stores) or ADD / MIN / MAX (REDUCE_ALL), the split/combine kinds of
+ * ir/daphneir/DaphneVectorizableOpInterface.td:23-34.
+ *
+ * Two implicit values per row: t, the row tile (cols values) which starts as the row of the
+ * primary input x, and r, the row scalar set by ROW_AGG. `domain` selects which of them an
+ * elementwise instruction works on (0 = t, 1 = r). */
+#define DH_PIPE_MAX_INSTR 16
+#define DH_PIPE_MAX_OPERANDS 4
+
+typedef enum dh_pipe_kind {
+    DH_PIPE_EW_BINARY = 0,     /* t|r = op(t|r, operand); swap != 0: op(operand, t|r); op: dh_binary_op */
+    DH_PIPE_EW_UNARY = 1,      /* t|r = op(t|r); op: dh_unary_op                                        */
+    DH_PIPE_ROW_AGG = 2,       /* r = agg(t); op: dh_agg_op (IDXMIN / IDXMAX give the index as a value)   */
+    DH_PIPE_STORE_TILE = 3,    /* out_tile[index] row = t                                                 */
+    DH_PIPE_STORE_ROW = 4,     /* out_row[index][row] = r (value type)                                    */
+    DH_PIPE_STORE_ROW_IDX = 5, /* out_row[index][row] = (uint64_t) r                                      */
+    DH_PIPE_REDUCE_ALL = 6     /* out_all[index] = combine over all rows of r (domain 1) or of every item
+                                  of t (domain 0); op: DH_AGG_SUM / MIN / MAX; index 0 or 1               */
+} dh_pipe_kind;
+
+typedef enum dh_pipe_operand {
+    DH_OPD_SCALAR = 0, /* the immediate `scalar`                                  */
+    DH_OPD_SELF = 1,   /* t (or r) itself, e.g. t * t                             */
+    DH_OPD_ROWVEC = 2, /* rowvec[index], 1 x cols, broadcast over rows (domain 0) */
+    DH_OPD_COLVEC = 3, /* colvec[index], rows x 1, broadcast over columns         */
+    DH_OPD_MATRIX = 4, /* matrix[index], rows x cols (domain 0)                   */
+    DH_OPD_ROWREG = 5  /* r broadcast over the row (domain 0)                     */
+} dh_pipe_operand;
+
+typedef struct dh_pipe_instr {
+    int32_t kind;    /* dh_pipe_kind */
+    int32_t op;      /* op code of the kind's enum */
+    int32_t domain;  /* 0: row tile t, 1: row scalar r */
+    int32_t operand; /* dh_pipe_operand (EW_BINARY only) */
+    int32_t index;   /* operand / output slot */
+    int32_t swap;    /* EW_BINARY: operand on the left-hand side */
+    double scalar;   /* DH_OPD_SCALAR immediate */
+} dh_pipe_instr;
+
+#define DH_PIPE_IO(SUF, T)                                                                         \
+    typedef struct dh_pipe_io_##SUF {                                                              \
+        const T *x;                 /* primary input, rows x cols */                               \
+        size_t ld_x;                                                                               \
+        const T *matrix[DH_PIPE_MAX_OPERANDS];                                                     \
+        size_t ld_matrix[DH_PIPE_MAX_OPERANDS];                                                    \
+        const T *rowvec[DH_PIPE_MAX_OPERANDS];                                                     \
+        const T *colvec[DH_PIPE_MAX_OPERANDS];                                                     \
+        size_t ld_colvec[DH_PIPE_MAX_OPERANDS];                                                    \
+        T *out_tile[DH_PIPE_MAX_OPERANDS];                                                         \
+        size_t ld_out_tile[DH_PIPE_MAX_OPERANDS];                                                  \
+        void *out_row[DH_PIPE_MAX_OPERANDS]; /* T or uint64_t per row */                           \
+        size_t ld_out_row[DH_PIPE_MAX_OPERANDS];                                                   \
+        T *out_all[2];              /* device scalars */                                           \
+    } dh_pipe_io_##SUF;
+DH_PIPE_IO(f32, float)
+DH_PIPE_IO(f64, double)
+#undef DH_PIPE_IO
+
+/* Runs `num_instr` instructions over every row. Unbound slots are NULL. Rows wider than
+ * 1024 floats / 512 doubles do not fit the register tile: DH_ERR_RUNTIME, and the caller runs
+ * the operators one by one. Unary domain errors are reported as for dh_ew_unary_*. */
+dh_status dh_vectorized_pipeline_f32(dh_ctx *ctx, const dh_pipe_instr *program, int num_instr,
+                                     const dh_pipe_io_f32 *io, size_t rows, size_t cols);
+dh_status dh_vectorized_pipeline_f64(dh_ctx *ctx, const dh_pipe_instr *program, int num_instr,
+                                     const dh_pipe_io_f64 *io, size_t rows, size_t cols);
+
 #ifdef __cplusplus
 }
 #endif

@@ -160,3 +160,16 @@ def softmax(arg):
     res = np.empty(arg.shape, arg.dtype)
     st = _f("softmax", arg.dtype)(_p(res), sz(_ld(res)), _p(arg), sz(arg.shape[0]), sz(arg.shape[1]), sz(_ld(arg)))
     return st, res
+
+
+def zscore_pipeline(X, threads=4, thr=64.0):
+    """Reference-style execution of the z-score / row-sum / threshold-count pipeline (float32):
+    column statistics as single kernel calls, the row-split body on `threads` workers."""
+    assert X.dtype == np.float32 and X.flags.c_contiguous
+    rows, cols = X.shape
+    mu, sd = np.empty((1, cols), np.float32), np.empty((1, cols), np.float32)
+    r, s = np.empty((rows, 1), np.float32), np.empty(1, np.float32)
+    secs = np.zeros(2, np.float64)
+    st = lib().oracle_zscore_pipeline_f32(_p(X), sz(rows), sz(cols), C.c_int(threads), C.c_float(thr), _p(mu), _p(sd),
+                                          _p(r), _p(s), _p(secs))
+    return st, mu, sd, r, s[0], secs

@@ -1,0 +1,171 @@
+"""GPU parity: the fused vectorized pipeline against (a) the same operators run one by one through
+the stand-alone device kernels and (b) the CPU oracle's restatement of the reference's engine."""
+import numpy as np
+import pytest
+
+import oracle_binding as orc
+from parity import assert_close, assert_exact
+
+pytestmark = pytest.mark.gpu
+
+from daphne_amd import capi
+from daphne_amd.kernels import (AggOpCode, BinaryOpCode, DenseMatrix, UnaryOpCode, aggAll, aggCol, aggRow, ewBinaryMat,
+                                ewBinaryObjSca, ewUnaryMat)
+from daphne_amd.pipeline import ROWREG, SELF, VectorizedPipeline
+
+DTYPES = [np.float32, np.float64]
+
+
+def zscore_device(ctx, X, thr=64.0):
+    """Config-2 style pipeline on the device: two column statistics + one fused kernel."""
+    mu = aggCol(AggOpCode.MEAN, None, X, ctx)
+    sd = ewUnaryMat(UnaryOpCode.SQRT, None, aggCol(AggOpCode.VAR, None, X, ctx), ctx)
+    p = VectorizedPipeline(ctx, X)
+    p.ewBinary(BinaryOpCode.SUB, mu).ewBinary(BinaryOpCode.DIV, sd).ewBinary(BinaryOpCode.MUL, SELF)
+    p.rowAgg(AggOpCode.SUM)
+    r = p.storeRow()
+    p.ewBinary(BinaryOpCode.GT, thr)
+    s = p.reduceAll(AggOpCode.SUM)
+    p.run()
+    return mu, sd, r, s
+
+
+@pytest.mark.parametrize("rows,cols", [(1000, 64), (50001, 64), (777, 16), (513, 40), (300, 7), (64, 256), (5, 1000)])
+def test_zscore_pipeline_vs_oracle_engine(ctx, rows, cols):
+    rng = np.random.default_rng(rows + cols)
+    x = (rng.standard_normal((rows, cols)) * 2 + 5).astype(np.float32)
+    thr = float(cols)
+    st, mu_e, sd_e, r_e, s_e, _ = orc.zscore_pipeline(x, threads=3, thr=thr)
+    mu, sd, r, s = zscore_device(ctx, DenseMatrix.from_numpy(ctx, x), thr)
+    assert_close(mu.to_numpy(), mu_e)
+    assert_close(sd.to_numpy(), sd_e)
+    assert_close(r.to_numpy(), r_e)
+    # the count may differ only by rows whose r is within tolerance of the threshold
+    amb = int((np.abs(r_e - thr) <= 1e-4 * thr).sum())
+    assert abs(float(s.to_numpy()[0, 0]) - float(s_e)) <= amb
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("rows,cols", [(1000, 64), (333, 16), (129, 36), (70, 5), (40, 512), (9, 130)])
+def test_pipeline_equals_op_by_op(ctx, dt, rows, cols):
+    """Same body, fused vs one kernel per operator (how the reference's device worker runs it)."""
+    rng = np.random.default_rng(rows * 3 + cols)
+    x = (rng.standard_normal((rows, cols)) + 3).astype(dt)
+    y = rng.standard_normal((rows, cols)).astype(dt)
+    rv = (rng.random((1, cols)) + 0.5).astype(dt)
+    cv = (rng.random((rows, 1)) + 0.5).astype(dt)
+    X, Y, RV, CV = (DenseMatrix.from_numpy(ctx, a) for a in (x, y, rv, cv))
+    # fused
+    p = VectorizedPipeline(ctx, X)
+    p.ewBinary(BinaryOpCode.ADD, Y).ewBinary(BinaryOpCode.MUL, RV).ewBinary(BinaryOpCode.DIV, CV)
+    p.ewBinary(BinaryOpCode.SUB, 0.25).ewUnary(UnaryOpCode.ABS).ewBinary(BinaryOpCode.SUB, 1.0, swap=True)
+    tile = p.storeTile()
+    p.rowAgg(AggOpCode.MAX)
+    rmax = p.storeRow()
+    p.toTile().ewBinary(BinaryOpCode.SUB, ROWREG).ewUnary(UnaryOpCode.EXP)
+    p.rowAgg(AggOpCode.SUM)
+    rsum = p.storeRow()
+    tot = p.reduceAll(AggOpCode.SUM)
+    p.toTile().ewBinary(BinaryOpCode.DIV, ROWREG)
+    soft = p.storeTile()
+    p.run()
+    # one by one
+    t = ewBinaryMat(BinaryOpCode.ADD, None, X, Y, ctx)
+    t = ewBinaryMat(BinaryOpCode.MUL, None, t, RV, ctx)
+    t = ewBinaryMat(BinaryOpCode.DIV, None, t, CV, ctx)
+    t = ewBinaryObjSca(BinaryOpCode.SUB, None, t, 0.25, ctx)
+    t = ewUnaryMat(UnaryOpCode.ABS, None, t, ctx)
+    t = ewBinaryObjSca(BinaryOpCode.MUL, None, ewBinaryObjSca(BinaryOpCode.SUB, None, t, 1.0, ctx), -1.0, ctx)
+    assert_exact(tile.to_numpy(), t.to_numpy())
+    m = aggRow(AggOpCode.MAX, None, t, ctx)
+    assert_exact(rmax.to_numpy(), m.to_numpy())
+    e = ewUnaryMat(UnaryOpCode.EXP, None, ewBinaryMat(BinaryOpCode.SUB, None, t, m, ctx), ctx)
+    ssum = aggRow(AggOpCode.SUM, None, e, ctx)
+    assert_close(rsum.to_numpy(), ssum.to_numpy())
+    assert_close(tot.to_numpy(), np.array([[aggAll(AggOpCode.SUM, ssum, ctx)]], dt), rtol=1e-5 if dt == np.float32 else 1e-12)
+    assert_close(soft.to_numpy(), ewBinaryMat(BinaryOpCode.DIV, None, e, ssum, ctx).to_numpy())
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("op", [AggOpCode.SUM, AggOpCode.PROD, AggOpCode.MIN, AggOpCode.MAX, AggOpCode.MEAN,
+                                AggOpCode.STDDEV, AggOpCode.VAR, AggOpCode.IDXMIN, AggOpCode.IDXMAX])
+@pytest.mark.parametrize("rows,cols", [(2000, 16), (50, 64), (33, 24), (7, 300)])
+def test_pipeline_row_aggs_vs_oracle(ctx, dt, op, rows, cols):
+    rng = np.random.default_rng(rows + cols + int(op))
+    if op in (AggOpCode.IDXMIN, AggOpCode.IDXMAX):
+        x = rng.integers(0, 5, (rows, cols)).astype(dt)
+        x[0, :] = np.nan
+        x[1, 0] = np.nan
+        x[2, 1:] = np.nan
+        x[3, :] = np.inf
+    elif op == AggOpCode.PROD:
+        x = (1 + 0.01 * rng.standard_normal((rows, cols))).astype(dt)
+    else:
+        x = (rng.standard_normal((rows, cols)) * 2 + 5).astype(dt)
+        if op in (AggOpCode.MIN, AggOpCode.MAX):
+            x[1, 0] = np.nan
+            x[2, 3] = np.nan
+    p = VectorizedPipeline(ctx, DenseMatrix.from_numpy(ctx, x))
+    p.rowAgg(op)
+    is_idx = op in (AggOpCode.IDXMIN, AggOpCode.IDXMAX)
+    out = p.storeRow(as_index=is_idx)
+    p.run()
+    st, exp = orc.agg_row(op, x)
+    if is_idx or op in (AggOpCode.MIN, AggOpCode.MAX):
+        assert_exact(out.to_numpy(), exp)
+    else:
+        assert_close(out.to_numpy(), exp, elementwise=op not in (AggOpCode.VAR, AggOpCode.STDDEV))
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+def test_pipeline_kmeans_distance_idxmin(ctx, dt):
+    """D = xx - 2*XC + cc ; idx = idxminRow(D) as one fused body (k-means assignment step)."""
+    rng = np.random.default_rng(8)
+    rows, k = 5000, 16
+    xc = rng.standard_normal((rows, k)).astype(dt)
+    xx = (rng.random((rows, 1)) * 3).astype(dt)
+    cc = (rng.random((1, k)) * 3).astype(dt)
+    p = VectorizedPipeline(ctx, DenseMatrix.from_numpy(ctx, xc))
+    p.ewBinary(BinaryOpCode.MUL, -2.0).ewBinary(BinaryOpCode.ADD, DenseMatrix.from_numpy(ctx, xx))
+    p.ewBinary(BinaryOpCode.ADD, DenseMatrix.from_numpy(ctx, cc))
+    p.rowAgg(AggOpCode.IDXMIN)
+    idx = p.storeRow(as_index=True)
+    p.run()
+    d = orc.ew_binary(0, orc.ew_binary(0, orc.ew_binary_sca(2, xc, -2.0)[1], xx)[1], cc)[1]
+    assert_exact(idx.to_numpy(), orc.agg_row(AggOpCode.IDXMIN, d)[1])
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+def test_pipeline_reduce_min_max_and_views(ctx, dt):
+    rng = np.random.default_rng(9)
+    big = rng.standard_normal((400, 96)).astype(dt)
+    B = DenseMatrix.from_numpy(ctx, big)
+    v, V = big[10:390, 8:72], B.slice(10, 390, 8, 72)
+    p = VectorizedPipeline(ctx, V)
+    p.ewBinary(BinaryOpCode.MUL, 2.0)
+    mn = p.reduceAll(AggOpCode.MIN)
+    mx = p.reduceAll(AggOpCode.MAX)
+    p.run()
+    assert_exact(mn.to_numpy(), np.array([[v.min() * 2]], dt))
+    assert_exact(mx.to_numpy(), np.array([[v.max() * 2]], dt))
+
+
+def test_pipeline_errors(ctx):
+    x = DenseMatrix.from_numpy(ctx, np.ones((10, 8), np.float32))
+    p = VectorizedPipeline(ctx, x)
+    p.ewBinary(999, 1.0)
+    with pytest.raises(capi.DaphneHipError, match="unknown BinaryOpCode"):
+        p.run()
+    p = VectorizedPipeline(ctx, DenseMatrix.from_numpy(ctx, -np.ones((10, 8), np.float32)))
+    p.ewUnary(UnaryOpCode.SQRT)
+    p.storeTile()
+    with pytest.raises(capi.DaphneHipDomainError):
+        p.run()
+    wide = DenseMatrix.from_numpy(ctx, np.ones((2, 5000), np.float32))
+    p = VectorizedPipeline(ctx, wide)
+    p.ewUnary(UnaryOpCode.ABS)
+    p.storeTile()
+    with pytest.raises(capi.DaphneHipError, match="do not fit the register tile"):
+        p.run()
+    with pytest.raises(capi.DaphneHipError, match="row/column vector"):
+        VectorizedPipeline(ctx, x).ewBinary(BinaryOpCode.ADD, DenseMatrix.from_numpy(ctx, np.ones((3, 3), np.float32)))
