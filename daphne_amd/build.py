@@ -45,6 +45,37 @@ def _compile(src: Path) -> Path:
     return obj
 
 
+JIT_PRELUDE = """// generated: sources compiled at run time (hiprtc) for fused pipeline bodies
+typedef __SIZE_TYPE__ size_t;
+typedef __INT32_TYPE__ int32_t;
+typedef __UINT32_TYPE__ uint32_t;
+typedef __INT64_TYPE__ int64_t;
+typedef __UINT64_TYPE__ uint64_t;
+"""
+
+
+def generate_jit_sources() -> Path:
+    """Embeds the public header and the device headers of the pipeline kernel as one string."""
+    parts = [JIT_PRELUDE]
+    for f in (PKG_DIR.parent / "include" / "daphne_hip.h", CSRC / "dev_common.h", CSRC / "ew_ops.h",
+              CSRC / "pipeline_kernel.h"):
+        for line in f.read_text().splitlines():
+            if line.startswith("#include") or line.startswith("#pragma once"):
+                continue
+            parts.append(line)
+    text = "\n".join(parts)
+    if ')DHJIT"' in text:
+        raise RuntimeError("embedded source contains the raw-string delimiter")
+    # split into chunks: some compilers cap the length of a single literal
+    chunks, step = [], 12000
+    for i in range(0, len(text), step):
+        chunks.append('R"DHJIT(' + text[i:i + step] + ')DHJIT"')
+    out = OBJ_DIR / "jit_sources.inc"
+    OBJ_DIR.mkdir(parents=True, exist_ok=True)
+    out.write_text("static const char kJitEmbeddedSource[] =\n" + "\n".join(chunks) + ";\n")
+    return out
+
+
 def sources() -> list[Path]:
     return sorted(CSRC.glob("*.hip"))
 
@@ -52,13 +83,14 @@ def sources() -> list[Path]:
 def build_all(jobs: int | None = None, verbose: bool = True) -> Path:
     """Compiles every translation unit and links the shared library. Always recompiles."""
     OBJ_DIR.mkdir(parents=True, exist_ok=True)
+    generate_jit_sources()
     srcs = sources()
     jobs = jobs or min(len(srcs), max(1, (os.cpu_count() or 2)), 16)
     if verbose:
         print(f"[daphne_amd.build] compiling {len(srcs)} files with hipcc for gfx950 ({jobs} jobs)", flush=True)
     with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as pool:
         objs = list(pool.map(_compile, srcs))
-    cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(LIB_PATH), *map(str, objs)]
+    cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(LIB_PATH), *map(str, objs), "-lhiprtc"]
     proc = subprocess.run(cmd, capture_output=True, text=True)
     if proc.returncode != 0:
         raise RuntimeError(f"link failed:\n{proc.stderr}")

@@ -108,27 +108,33 @@ __global__ __launch_bounds__(THREADS) void all_stage1(const T *arg, size_t rows,
     const size_t row_step = static_cast<size_t>(gridDim.x) * blockDim.y;
     for (size_t cv = static_cast<size_t>(blockIdx.y) * blockDim.x + threadIdx.x; cv < cvecs;
          cv += static_cast<size_t>(gridDim.y) * blockDim.x) {
-        for (size_t r0 = static_cast<size_t>(blockIdx.x) * blockDim.y + threadIdx.y; r0 < rows;
-             r0 += row_step * UNROLL) {
+        // main loop: UNROLL independent, unguarded loads in flight; then a guarded tail
+        size_t r0 = static_cast<size_t>(blockIdx.x) * blockDim.y + threadIdx.y;
+        for (; r0 + (UNROLL - 1) * row_step < rows; r0 += row_step * UNROLL) {
             T x[UNROLL][VEC];
 #pragma unroll
-            for (int u = 0; u < UNROLL; u++) {
-                const size_t r = r0 + u * row_step;
-                if (r < rows)
-                    load_vec<T, VEC>(arg + r * ld + cv * VEC, x[u]);
-            }
+            for (int u = 0; u < UNROLL; u++)
+                dh_load_vec_stream<T, VEC>(arg + (r0 + u * row_step) * ld + cv * VEC, x[u]);
 #pragma unroll
             for (int u = 0; u < UNROLL; u++) {
-                const size_t r = r0 + u * row_step;
-                if (r < rows) {
 #pragma unroll
-                    for (int i = 0; i < VEC; i++) {
-                        T v = x[u][i];
-                        if constexpr (SQDEV)
-                            v = (v - m) * (v - m);
-                        acc[i] = R::comb(acc[i], v);
-                    }
+                for (int i = 0; i < VEC; i++) {
+                    T v = x[u][i];
+                    if constexpr (SQDEV)
+                        v = (v - m) * (v - m);
+                    acc[i] = R::comb(acc[i], v);
                 }
+            }
+        }
+        for (; r0 < rows; r0 += row_step) {
+            T x[VEC];
+            dh_load_vec_stream<T, VEC>(arg + r0 * ld + cv * VEC, x);
+#pragma unroll
+            for (int i = 0; i < VEC; i++) {
+                T v = x[i];
+                if constexpr (SQDEV)
+                    v = (v - m) * (v - m);
+                acc[i] = R::comb(acc[i], v);
             }
         }
     }
@@ -302,49 +308,105 @@ template <typename T> dh_status agg_all(dh_ctx *ctx, int op, const T *arg, size_
 template <typename T, int VEC, class R, int FINAL, bool NANFIRST>
 __global__ __launch_bounds__(THREADS) void row_kernel(T *res, size_t ld_res, const T *arg, size_t rows,
                                                       size_t cols, size_t ld, int G) {
+    // UR rows per lane group are processed together so that UR independent loads are in flight;
+    // rows past the end are clamped to the last row for loading and dropped at the store.
+    // Per step a wavefront owns GPW * UR consecutive rows (row (u, g) = base + u * GPW + g for
+    // lane group g): load u covers GPW whole rows back to back, and the step's results are one
+    // contiguous run stored by the first GPW * UR lanes.
+    constexpr int UR = 4;
     const int tid = threadIdx.x;
     const int lane = tid % G;
-    const size_t rows_per_block = THREADS / G;
+    const int wlane = tid % DH_WAVE;
+    const int GPW = DH_WAVE / G;
+    const int g_in_wave = wlane / G;
     const size_t cvecs = cols / VEC;
-    for (size_t r = static_cast<size_t>(blockIdx.x) * rows_per_block + tid / G; r < rows;
-         r += static_cast<size_t>(gridDim.x) * rows_per_block) {
-        const T *row = arg + r * ld;
-        T acc = R::id();
+    const size_t rows_per_step = static_cast<size_t>(GPW) * UR;
+    const size_t wave_id = static_cast<size_t>(blockIdx.x) * (THREADS / DH_WAVE) + tid / DH_WAVE;
+    const size_t wave_stride = static_cast<size_t>(gridDim.x) * (THREADS / DH_WAVE) * rows_per_step;
+    for (size_t base = wave_id * rows_per_step; base < rows; base += wave_stride) {
+        const T *row[UR];
+#pragma unroll
+        for (int u = 0; u < UR; u++) {
+            const size_t r = base + static_cast<size_t>(u * GPW + g_in_wave);
+            row[u] = arg + (r < rows ? r : rows - 1) * ld;
+        }
+        T acc[UR];
+#pragma unroll
+        for (int u = 0; u < UR; u++)
+            acc[u] = R::id();
         for (size_t cv = lane; cv < cvecs; cv += G) {
-            T x[VEC];
-            load_vec<T, VEC>(row + cv * VEC, x);
+            T x[UR][VEC];
 #pragma unroll
-            for (int i = 0; i < VEC; i++)
-                acc = R::comb(acc, x[i]);
+            for (int u = 0; u < UR; u++)
+                dh_load_vec_stream<T, VEC>(row[u] + cv * VEC, x[u]);
+#pragma unroll
+            for (int u = 0; u < UR; u++)
+#pragma unroll
+                for (int i = 0; i < VEC; i++)
+                    acc[u] = R::comb(acc[u], x[u][i]);
         }
-        for (int off = G / 2; off >= 1; off >>= 1)
-            acc = R::comb(acc, dh_shfl_xor(acc, off));
-        if constexpr (FINAL >= 1)
-            acc = acc / static_cast<T>(cols);
-        if constexpr (FINAL >= 2) {
-            const T mean = acc;
-            T s = T(0);
-            for (size_t cv = lane; cv < cvecs; cv += G) {
-                T x[VEC];
-                load_vec<T, VEC>(row + cv * VEC, x);
 #pragma unroll
-                for (int i = 0; i < VEC; i++) {
-                    const T d = x[i] - mean;
-                    s = s + d * d;
-                }
-            }
+        for (int u = 0; u < UR; u++) {
             for (int off = G / 2; off >= 1; off >>= 1)
-                s = s + dh_shfl_xor(s, off);
-            s = s / static_cast<T>(cols);
-            acc = (FINAL == 3) ? dev_sqrt<T>(s) : s;
+                acc[u] = R::comb(acc[u], dh_shfl_xor(acc[u], off));
+            if constexpr (FINAL >= 1)
+                acc[u] = acc[u] / static_cast<T>(cols);
         }
-        if constexpr (NANFIRST) {
-            const T first = row[0];
-            if (dev_isnan(first))
-                acc = first;
+        if constexpr (FINAL >= 2) {
+            T s[UR];
+#pragma unroll
+            for (int u = 0; u < UR; u++)
+                s[u] = T(0);
+            for (size_t cv = lane; cv < cvecs; cv += G) {
+                T x[UR][VEC];
+#pragma unroll
+                for (int u = 0; u < UR; u++)
+                    load_vec<T, VEC>(row[u] + cv * VEC, x[u]);
+#pragma unroll
+                for (int u = 0; u < UR; u++)
+#pragma unroll
+                    for (int i = 0; i < VEC; i++) {
+                        const T d = x[u][i] - acc[u];
+                        s[u] = s[u] + d * d;
+                    }
+            }
+#pragma unroll
+            for (int u = 0; u < UR; u++) {
+                for (int off = G / 2; off >= 1; off >>= 1)
+                    s[u] = s[u] + dh_shfl_xor(s[u], off);
+                s[u] = s[u] / static_cast<T>(cols);
+                acc[u] = (FINAL == 3) ? dev_sqrt<T>(s[u]) : s[u];
+            }
         }
-        if (lane == 0)
-            res[r * ld_res] = acc;
+#pragma unroll
+        for (int u = 0; u < UR; u++) {
+            if constexpr (NANFIRST) {
+                const T first = row[u][0];
+                if (dev_isnan(first))
+                    acc[u] = first;
+            }
+        }
+        if (GPW * UR <= DH_WAVE) {
+            // lane j takes the result of row base + j: it sits in group j % GPW as acc[j / GPW]
+            T mine = T(0);
+#pragma unroll
+            for (int u = 0; u < UR; u++) {
+                const T v = __shfl(acc[u], (wlane % GPW) * G, DH_WAVE);
+                if (wlane / GPW == u)
+                    mine = v;
+            }
+            const size_t orow = base + static_cast<size_t>(wlane);
+            if (wlane < GPW * UR && orow < rows)
+                res[orow * ld_res] = mine;
+        } else {
+            // fewer than 4 lanes per row: more rows per step than lanes, every group stores its own
+#pragma unroll
+            for (int u = 0; u < UR; u++) {
+                const size_t r = base + static_cast<size_t>(u * GPW + g_in_wave);
+                if (lane == 0 && r < rows)
+                    res[r * ld_res] = acc[u];
+            }
+        }
     }
 }
 
@@ -352,47 +414,63 @@ __global__ __launch_bounds__(THREADS) void row_kernel(T *res, size_t ld_res, con
 template <typename T, int VEC, bool IS_MIN>
 __global__ __launch_bounds__(THREADS) void row_idx_kernel(uint64_t *res, size_t ld_res, const T *arg, size_t rows,
                                                           size_t cols, size_t ld, int G) {
+    constexpr int UR = 4; // rows in flight per lane group (clamped past the end, dropped at the store)
     const int tid = threadIdx.x;
     const int lane = tid % G;
     const size_t rows_per_block = THREADS / G;
     const size_t cvecs = cols / VEC;
+    const size_t stride = static_cast<size_t>(gridDim.x) * rows_per_block;
     const T worst = IS_MIN ? std::numeric_limits<T>::infinity() : -std::numeric_limits<T>::infinity();
-    for (size_t r = static_cast<size_t>(blockIdx.x) * rows_per_block + tid / G; r < rows;
-         r += static_cast<size_t>(gridDim.x) * rows_per_block) {
-        const T *row = arg + r * ld;
-        T best = worst;
-        unsigned long long bi = ~0ull;
-        for (size_t cv = lane; cv < cvecs; cv += G) {
-            T x[VEC];
-            load_vec<T, VEC>(row + cv * VEC, x);
+    for (size_t r0 = static_cast<size_t>(blockIdx.x) * rows_per_block + tid / G; r0 < rows; r0 += stride * UR) {
+        const T *row[UR];
+        T best[UR];
+        unsigned long long bi[UR];
 #pragma unroll
-            for (int i = 0; i < VEC; i++) {
-                const unsigned long long idx = cv * VEC + i;
-                const bool better = IS_MIN ? (x[i] < best) : (x[i] > best);
-                // within a lane indices only grow, so a tie keeps the earlier one, except against
-                // the sentinel (an actual +-inf value must beat "nothing seen yet")
-                const bool first_seen = (bi == ~0ull) && !dev_isnan(x[i]);
-                if (better || first_seen) {
-                    best = x[i];
-                    bi = idx;
+        for (int u = 0; u < UR; u++) {
+            const size_t r = r0 + u * stride;
+            row[u] = arg + (r < rows ? r : rows - 1) * ld;
+            best[u] = worst;
+            bi[u] = ~0ull;
+        }
+        for (size_t cv = lane; cv < cvecs; cv += G) {
+            T x[UR][VEC];
+#pragma unroll
+            for (int u = 0; u < UR; u++)
+                dh_load_vec_stream<T, VEC>(row[u] + cv * VEC, x[u]);
+#pragma unroll
+            for (int u = 0; u < UR; u++)
+#pragma unroll
+                for (int i = 0; i < VEC; i++) {
+                    const unsigned long long idx = cv * VEC + i;
+                    const bool better = IS_MIN ? (x[u][i] < best[u]) : (x[u][i] > best[u]);
+                    // within a lane indices only grow, so a tie keeps the earlier one, except
+                    // against the sentinel (an actual +-inf value must beat "nothing seen yet")
+                    const bool first_seen = (bi[u] == ~0ull) && !dev_isnan(x[u][i]);
+                    if (better || first_seen) {
+                        best[u] = x[u][i];
+                        bi[u] = idx;
+                    }
+                }
+        }
+#pragma unroll
+        for (int u = 0; u < UR; u++) {
+            for (int off = G / 2; off >= 1; off >>= 1) {
+                const T ov = dh_shfl_xor(best[u], off);
+                const unsigned long long oi = dh_shfl_xor(bi[u], off);
+                const bool better = IS_MIN ? (ov < best[u]) : (ov > best[u]);
+                if (better || (ov == best[u] && oi < bi[u])) {
+                    best[u] = ov;
+                    bi[u] = oi;
                 }
             }
-        }
-        for (int off = G / 2; off >= 1; off >>= 1) {
-            const T ov = dh_shfl_xor(best, off);
-            const unsigned long long oi = dh_shfl_xor(bi, off);
-            const bool better = IS_MIN ? (ov < best) : (ov > best);
-            if (better || (ov == best && oi < bi)) {
-                best = ov;
-                bi = oi;
+            const size_t r = r0 + u * stride;
+            if (lane == 0 && r < rows) {
+                // AggRow.h:73-80: the scan starts from element 0; if that is NaN no later element
+                // compares below/above it, so 0 is returned. An all-NaN tail leaves bi untouched.
+                if (dev_isnan(row[u][0]) || bi[u] == ~0ull)
+                    bi[u] = 0;
+                res[r * ld_res] = bi[u];
             }
-        }
-        if (lane == 0) {
-            // AggRow.h:73-80: the scan starts from element 0; if that is NaN no later element
-            // compares below/above it, so 0 is returned. An all-NaN tail leaves bi untouched.
-            if (dev_isnan(row[0]) || bi == ~0ull)
-                bi = 0;
-            res[r * ld_res] = bi;
         }
     }
 }
@@ -405,9 +483,9 @@ static inline int pick_group(size_t cvecs) {
 }
 
 static inline unsigned row_grid(const dh_ctx *ctx, size_t rows, int G) {
-    const size_t rpb = THREADS / G;
+    const size_t rpb = static_cast<size_t>(THREADS / G) * 4; // rows per block and step (4 per lane group)
     size_t g = dh_ceil_div(rows, rpb);
-    const size_t cap = static_cast<size_t>(ctx->num_cus) * 16;
+    const size_t cap = static_cast<size_t>(ctx->num_cus) * 64;
     if (g > cap)
         g = cap;
     if (g < 1)
@@ -497,6 +575,8 @@ dh_status agg_row_idx(dh_ctx *ctx, int op, uint64_t *res, size_t ld_res, const T
     return DH_OK;
 }
 
+constexpr int S2_TX = 16, S2_TY = 16; // second-stage block: columns x partial lanes
+
 // =======================================================================================
 // AggCol
 // =======================================================================================
@@ -516,23 +596,24 @@ __global__ __launch_bounds__(THREADS) void col_stage1(const T *arg, size_t rows,
         acc[i] = R::id();
     if (cv < cvecs) {
         const size_t step = blockDim.y;
-        for (size_t r0 = r_begin + threadIdx.y; r0 < r_end; r0 += step * UNROLL) {
+        size_t r0 = r_begin + threadIdx.y;
+        for (; r0 + (UNROLL - 1) * step < r_end; r0 += step * UNROLL) {
             T x[UNROLL][VEC];
 #pragma unroll
-            for (int u = 0; u < UNROLL; u++) {
-                const size_t r = r0 + u * step;
-                if (r < r_end)
-                    load_vec<T, VEC>(arg + r * ld + cv * VEC, x[u]);
-            }
+            for (int u = 0; u < UNROLL; u++)
+                dh_load_vec_stream<T, VEC>(arg + (r0 + u * step) * ld + cv * VEC, x[u]);
 #pragma unroll
-            for (int u = 0; u < UNROLL; u++) {
-                const size_t r = r0 + u * step;
-                if (r < r_end) {
+            for (int u = 0; u < UNROLL; u++)
 #pragma unroll
-                    for (int i = 0; i < VEC; i++)
-                        acc[i] = R::comb(acc[i], x[u][i]);
-                }
-            }
+                for (int i = 0; i < VEC; i++)
+                    acc[i] = R::comb(acc[i], x[u][i]);
+        }
+        for (; r0 < r_end; r0 += step) {
+            T x[VEC];
+            dh_load_vec_stream<T, VEC>(arg + r0 * ld + cv * VEC, x);
+#pragma unroll
+            for (int i = 0; i < VEC; i++)
+                acc[i] = R::comb(acc[i], x[i]);
         }
     }
     const int w = blockDim.x * VEC;
@@ -555,12 +636,29 @@ __global__ __launch_bounds__(THREADS) void col_stage1(const T *arg, size_t rows,
 template <typename T, class R, int FINAL, bool NANFIRST>
 __global__ __launch_bounds__(THREADS) void col_stage2(const T *partials, size_t nparts, size_t cols, T *res,
                                                       const T *arg, T count) {
-    const size_t c = static_cast<size_t>(blockIdx.x) * THREADS + threadIdx.x;
-    if (c >= cols)
+    // block = (S2_TX columns, S2_TY partial lanes): the partial rows are split over the TY lanes
+    // (4 independent loads in flight each) and folded through LDS in a fixed order.
+    __shared__ T lds[S2_TY][S2_TX];
+    const size_t c = static_cast<size_t>(blockIdx.x) * S2_TX + threadIdx.x;
+    T a0 = R::id(), a1 = R::id(), a2 = R::id(), a3 = R::id();
+    if (c < cols) {
+        size_t p = threadIdx.y;
+        for (; p + 3 * S2_TY < nparts; p += 4 * S2_TY) {
+            a0 = R::comb(a0, partials[p * cols + c]);
+            a1 = R::comb(a1, partials[(p + S2_TY) * cols + c]);
+            a2 = R::comb(a2, partials[(p + 2 * S2_TY) * cols + c]);
+            a3 = R::comb(a3, partials[(p + 3 * S2_TY) * cols + c]);
+        }
+        for (; p < nparts; p += S2_TY)
+            a0 = R::comb(a0, partials[p * cols + c]);
+    }
+    lds[threadIdx.y][threadIdx.x] = R::comb(R::comb(a0, a1), R::comb(a2, a3));
+    __syncthreads();
+    if (threadIdx.y != 0 || c >= cols)
         return;
-    T a = R::id();
-    for (size_t p = 0; p < nparts; p++)
-        a = R::comb(a, partials[p * cols + c]);
+    T a = lds[0][threadIdx.x];
+    for (int y = 1; y < S2_TY; y++)
+        a = R::comb(a, lds[y][threadIdx.x]);
     if constexpr (FINAL == 1)
         a = a / count;
     if constexpr (NANFIRST) {
@@ -594,25 +692,29 @@ __global__ __launch_bounds__(THREADS) void col_var_stage1(const T *arg, size_t r
     if (cv < cvecs && r_begin + threadIdx.y < r_end) {
         load_vec<T, VEC>(arg + (r_begin + threadIdx.y) * ld + cv * VEC, shift);
         n = (r_end - r_begin - threadIdx.y + step - 1) / step;
-        for (size_t r0 = r_begin + threadIdx.y; r0 < r_end; r0 += step * UNROLL) {
+        size_t r0 = r_begin + threadIdx.y;
+        for (; r0 + (UNROLL - 1) * step < r_end; r0 += step * UNROLL) {
             T x[UNROLL][VEC];
 #pragma unroll
-            for (int u = 0; u < UNROLL; u++) {
-                const size_t r = r0 + u * step;
-                if (r < r_end)
-                    load_vec<T, VEC>(arg + r * ld + cv * VEC, x[u]);
-            }
+            for (int u = 0; u < UNROLL; u++)
+                dh_load_vec_stream<T, VEC>(arg + (r0 + u * step) * ld + cv * VEC, x[u]);
 #pragma unroll
-            for (int u = 0; u < UNROLL; u++) {
-                const size_t r = r0 + u * step;
-                if (r < r_end) {
+            for (int u = 0; u < UNROLL; u++)
 #pragma unroll
-                    for (int i = 0; i < VEC; i++) {
-                        const T d = x[u][i] - shift[i];
-                        s1[i] += d;
-                        s2[i] += d * d;
-                    }
+                for (int i = 0; i < VEC; i++) {
+                    const T d = x[u][i] - shift[i];
+                    s1[i] += d;
+                    s2[i] += d * d;
                 }
+        }
+        for (; r0 < r_end; r0 += step) {
+            T x[VEC];
+            dh_load_vec_stream<T, VEC>(arg + r0 * ld + cv * VEC, x);
+#pragma unroll
+            for (int i = 0; i < VEC; i++) {
+                const T d = x[i] - shift[i];
+                s1[i] += d;
+                s2[i] += d * d;
             }
         }
     }
@@ -658,22 +760,41 @@ __global__ __launch_bounds__(THREADS) void col_var_stage1(const T *arg, size_t r
 template <typename T, int OUT>
 __global__ __launch_bounds__(THREADS) void col_var_stage2(const T *part_mean, const T *part_m2, size_t nparts,
                                                           size_t cols, size_t rows, size_t slab, T *res) {
-    const size_t c = static_cast<size_t>(blockIdx.x) * THREADS + threadIdx.x;
-    if (c >= cols)
-        return;
+    // (S2_TX columns, S2_TY partial lanes): every lane merges its share of the per-block
+    // (count, mean, M2) triples with Chan's formula in double, lane 0 then merges the lanes.
+    __shared__ double lds_n[S2_TY][S2_TX], lds_mean[S2_TY][S2_TX], lds_m2[S2_TY][S2_TX];
+    const size_t c = static_cast<size_t>(blockIdx.x) * S2_TX + threadIdx.x;
     double cn = 0.0, cmean = 0.0, cm2 = 0.0;
-    for (size_t p = 0; p < nparts; p++) {
-        const size_t r_begin = p * slab;
-        if (r_begin >= rows)
-            break;
-        const size_t r_end = (r_begin + slab < rows) ? r_begin + slab : rows;
-        const double np_ = static_cast<double>(r_end - r_begin);
-        const double mp = static_cast<double>(part_mean[p * cols + c]);
-        const double qp = static_cast<double>(part_m2[p * cols + c]);
-        const double delta = mp - cmean;
+    if (c < cols) {
+        for (size_t p = threadIdx.y; p < nparts; p += S2_TY) {
+            const size_t r_begin = p * slab;
+            if (r_begin >= rows)
+                break;
+            const size_t r_end = (r_begin + slab < rows) ? r_begin + slab : rows;
+            const double np_ = static_cast<double>(r_end - r_begin);
+            const double mp = static_cast<double>(part_mean[p * cols + c]);
+            const double qp = static_cast<double>(part_m2[p * cols + c]);
+            const double delta = mp - cmean;
+            const double nt = cn + np_;
+            cmean += delta * np_ / nt;
+            cm2 += qp + delta * delta * cn * np_ / nt;
+            cn = nt;
+        }
+    }
+    lds_n[threadIdx.y][threadIdx.x] = cn;
+    lds_mean[threadIdx.y][threadIdx.x] = cmean;
+    lds_m2[threadIdx.y][threadIdx.x] = cm2;
+    __syncthreads();
+    if (threadIdx.y != 0 || c >= cols)
+        return;
+    for (int y = 1; y < S2_TY; y++) {
+        const double np_ = lds_n[y][threadIdx.x];
+        if (np_ == 0.0)
+            continue;
+        const double delta = lds_mean[y][threadIdx.x] - cmean;
         const double nt = cn + np_;
         cmean += delta * np_ / nt;
-        cm2 += qp + delta * delta * cn * np_ / nt;
+        cm2 += lds_m2[y][threadIdx.x] + delta * delta * cn * np_ / nt;
         cn = nt;
     }
     double v = cm2 / static_cast<double>(rows);
@@ -783,7 +904,7 @@ template <typename T> static inline ColPlan col_plan(const dh_ctx *ctx, const T 
         tx <<= 1;
     unsigned ty = THREADS / tx;
     size_t gy = dh_ceil_div(p.cvecs, tx);
-    size_t max_blocks = static_cast<size_t>(ctx->num_cus) * 8;
+    size_t max_blocks = static_cast<size_t>(ctx->num_cus) * 4; // few, fat blocks: short second stage
     size_t gx = max_blocks / gy;
     if (gx < 1)
         gx = 1;
@@ -814,8 +935,8 @@ static inline dh_status col_launch(dh_ctx *ctx, T *res, const T *arg, size_t row
         hipLaunchKernelGGL((col_stage1<T, V, R>), p.grid, p.block, lds, ctx->stream, arg, rows, p.cvecs, ld, p.slab, partials);
     else
         hipLaunchKernelGGL((col_stage1<T, 1, R>), p.grid, p.block, lds, ctx->stream, arg, rows, p.cvecs, ld, p.slab, partials);
-    hipLaunchKernelGGL((col_stage2<T, R, FINAL, NANFIRST>), dim3(static_cast<unsigned>(dh_ceil_div(cols, THREADS))),
-                       dim3(THREADS), 0, ctx->stream, partials, p.nparts, cols, res, arg, static_cast<T>(rows));
+    hipLaunchKernelGGL((col_stage2<T, R, FINAL, NANFIRST>), dim3(static_cast<unsigned>(dh_ceil_div(cols, S2_TX))),
+                       dim3(S2_TX, S2_TY), 0, ctx->stream, partials, p.nparts, cols, res, arg, static_cast<T>(rows));
     return DH_OK;
 }
 
@@ -859,11 +980,11 @@ template <typename T> dh_status agg_col(dh_ctx *ctx, int op, T *res, const T *ar
             hipLaunchKernelGGL((col_var_stage1<T, V>), p.grid, p.block, lds, ctx->stream, arg, rows, p.cvecs, ld, p.slab, pm, pq);
         else
             hipLaunchKernelGGL((col_var_stage1<T, 1>), p.grid, p.block, lds, ctx->stream, arg, rows, p.cvecs, ld, p.slab, pm, pq);
-        const dim3 g2(static_cast<unsigned>(dh_ceil_div(cols, THREADS)));
+        const dim3 g2(static_cast<unsigned>(dh_ceil_div(cols, S2_TX)));
         if (op == DH_AGG_VAR)
-            hipLaunchKernelGGL((col_var_stage2<T, 0>), g2, dim3(THREADS), 0, ctx->stream, pm, pq, p.nparts, cols, rows, p.slab, res);
+            hipLaunchKernelGGL((col_var_stage2<T, 0>), g2, dim3(S2_TX, S2_TY), 0, ctx->stream, pm, pq, p.nparts, cols, rows, p.slab, res);
         else
-            hipLaunchKernelGGL((col_var_stage2<T, 1>), g2, dim3(THREADS), 0, ctx->stream, pm, pq, p.nparts, cols, rows, p.slab, res);
+            hipLaunchKernelGGL((col_var_stage2<T, 1>), g2, dim3(S2_TX, S2_TY), 0, ctx->stream, pm, pq, p.nparts, cols, rows, p.slab, res);
         break;
     }
     default:

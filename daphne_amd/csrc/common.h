@@ -81,47 +81,4 @@ dh_status dh_workspace(dh_ctx *ctx, size_t bytes, void **out);
 static inline size_t dh_ceil_div(size_t a, size_t b) { return (a + b - 1) / b; }
 static inline bool dh_aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
 
-// ---------------------------------------------------------------------------------------
-// device helpers
-// ---------------------------------------------------------------------------------------
-constexpr int DH_WAVE = 64;
-
-template <typename T> struct dh_vec; // 16-byte vector of T
-template <> struct dh_vec<float> {
-    using type = float4;
-    static constexpr int N = 4;
-};
-template <> struct dh_vec<double> {
-    using type = double2;
-    static constexpr int N = 2;
-};
-
-template <typename T> __device__ __forceinline__ T dh_shfl_xor(T v, int mask) { return __shfl_xor(v, mask, DH_WAVE); }
-template <typename T> __device__ __forceinline__ T dh_shfl_down(T v, int d) { return __shfl_down(v, d, DH_WAVE); }
-
-// 16-byte (VEC = 16 / sizeof(T)) or scalar (VEC = 1) global load / store into a register array.
-template <typename T, int VEC> __device__ __forceinline__ void dh_load_vec(const T *p, T (&v)[VEC]) {
-    if constexpr (VEC == 1) {
-        v[0] = *p;
-    } else {
-        using V = typename dh_vec<T>::type;
-        const V t = *reinterpret_cast<const V *>(p);
-        const T *tp = reinterpret_cast<const T *>(&t);
-#pragma unroll
-        for (int i = 0; i < VEC; i++)
-            v[i] = tp[i];
-    }
-}
-template <typename T, int VEC> __device__ __forceinline__ void dh_store_vec(T *p, const T (&v)[VEC]) {
-    if constexpr (VEC == 1) {
-        *p = v[0];
-    } else {
-        using V = typename dh_vec<T>::type;
-        V t;
-        T *tp = reinterpret_cast<T *>(&t);
-#pragma unroll
-        for (int i = 0; i < VEC; i++)
-            tp[i] = v[i];
-        *reinterpret_cast<V *>(p) = t;
-    }
-}
+#include "dev_common.h"

@@ -371,6 +371,17 @@ dh_status dh_vectorized_pipeline_f32(dh_ctx *ctx, const dh_pipe_instr *program, 
 dh_status dh_vectorized_pipeline_f64(dh_ctx *ctx, const dh_pipe_instr *program, int num_instr,
                                      const dh_pipe_io_f64 *io, size_t rows, size_t cols);
 
+/* A pipeline body is specialised at run time: the kernel source is compiled once per distinct
+ * instruction list (hiprtc) and cached, the counterpart of the reference JIT-compiling every
+ * VectorizedPipelineOp body (compiler/lowering/LowerToLLVMPass.cpp:654-726). If that is
+ * switched off (environment DH_PIPELINE_JIT=0) or fails, a generic kernel interprets the list.
+ * Returns how the calling thread's last pipeline ran: 1 specialised, 0 interpreted. */
+int dh_vectorized_pipeline_last_mode(void);
+/* Compiles the specialised kernel of a body without loading or running it (no device needed).
+ * value_type 0 = float, 1 = double; vec = items per 16-byte vector or 1; kv = 1, 2 or 4. */
+dh_status dh_vectorized_pipeline_compile_check(int value_type, int vec, int kv,
+                                               const dh_pipe_instr *program, int num_instr);
+
 #ifdef __cplusplus
 }
 #endif
