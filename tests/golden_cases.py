@@ -1,0 +1,224 @@
+"""Replays the reference's own kernel unit tests (tests/golden/reference_kernel_tests.json, written
+by tests/golden/extract_reference_vectors.py) against a backend: the CPU oracle or the HIP kernels.
+
+Every check call of the reference's tests is mapped onto the backend's kernel of the same name; the
+comparison is the one the reference's test uses (operator== -> exact; checkEqApprox -> its epsilon).
+"""
+from __future__ import annotations
+
+import json
+import re
+from pathlib import Path
+
+import numpy as np
+
+GOLDEN = Path(__file__).resolve().parent / "golden" / "reference_kernel_tests.json"
+
+BIN = {n: i for i, n in enumerate(["ADD", "SUB", "MUL", "DIV", "POW", "MOD", "LOG", "EQ", "NEQ", "LT", "LE", "GT", "GE",
+                                   "MIN", "MAX", "AND", "OR", "BITWISE_AND", "CONCAT"])}
+UN = {n: i for i, n in enumerate(["MINUS", "ABS", "SIGN", "SQRT", "EXP", "LN", "SIN", "COS", "TAN", "ASIN", "ACOS",
+                                  "ATAN", "SINH", "COSH", "TANH", "FLOOR", "CEIL", "ROUND", "ISNAN", "UPPER", "LOWER"])}
+AGG = {n: i for i, n in enumerate(["SUM", "PROD", "MIN", "MAX", "IDXMIN", "IDXMAX", "MEAN", "STDDEV", "VAR"])}
+
+
+class Skip(Exception):
+    pass
+
+
+class DomainError(Exception):
+    pass
+
+
+class KernelError(Exception):
+    pass
+
+
+def load():
+    return json.loads(GOLDEN.read_text())
+
+
+def _num(v):
+    return {"nan": np.nan, "inf": np.inf, "-inf": -np.inf}.get(v, v) if isinstance(v, str) else v
+
+
+def matrix(spec, dt):
+    vals = np.array([_num(v) for v in spec["values"]], dtype=np.float64)
+    rows = spec["rows"]
+    if rows == 0 or vals.size % rows:
+        raise Skip("ragged literal")
+    return np.ascontiguousarray(vals.reshape(rows, vals.size // rows).astype(dt))
+
+
+def _scalar(tok):
+    t = re.sub(r"\(\s*(typename\s+)?[\w:]+\s*\)", "", tok).strip()
+    m = re.match(r"^\w+\((.*)\)$", t)
+    if m:
+        t = m.group(1)
+    try:
+        return float(t.rstrip("fFlL"))
+    except ValueError:
+        raise Skip(f"scalar {tok!r}")
+
+
+def _ints(args):
+    out = []
+    for a in ",".join(args).split(","):
+        if re.fullmatch(r"\d+", a.strip()):
+            out.append(int(a))
+    return out
+
+
+def all_checks():
+    """Yields (id, file, case, check) for every replayable check call."""
+    for f in load():
+        for ci, c in enumerate(f["cases"]):
+            for ki, k in enumerate(c["checks"]):
+                yield f"{f['file']}::{c['name'].strip() or ci}::{ki}:{k['fn']}", f, c, k
+            if not c["checks"]:
+                yield f"{f['file']}::{c['name'].strip() or ci}::direct", f, c, {"fn": "direct", "args": []}
+
+
+def _eq(got, exp):
+    got, exp = np.asarray(got, dtype=np.float64), np.asarray(exp, dtype=np.float64)
+    assert got.shape == exp.shape, (got.shape, exp.shape)
+    same = (got == exp) | (np.isnan(got) & np.isnan(exp))
+    assert same.all(), f"got {got.ravel()[:12]} expected {exp.ravel()[:12]}"
+
+
+def _approx(got, exp, eps):
+    got, exp = np.asarray(got, dtype=np.float64), np.asarray(exp, dtype=np.float64)
+    assert got.shape == exp.shape, (got.shape, exp.shape)
+    both_nan = np.isnan(got) & np.isnan(exp)
+    both_inf = np.isinf(exp) & (got == exp)
+    ok = both_nan | both_inf | (np.abs(got - exp) <= eps)
+    assert ok.all(), f"got {got.ravel()[:12]} expected {exp.ravel()[:12]} eps {eps}"
+
+
+def run(backend, f, c, k, dt):
+    """Replays one check; raises Skip for what is outside the float/double dense path."""
+    fn, args, file = k["fn"], k["args"], f["file"]
+    # a literal may be re-defined inside a test case (per SECTION / per value-type branch): a check
+    # uses the definition that precedes it in the source, else the first one
+    pos = k.get("pos", 1 << 60)
+    mats = dict(f.get("helper_matrices", {}))
+    for name, defs in c["matrices"].items():
+        before = [d for d in defs if d["pos"] < pos]
+        mats[name] = before[-1] if before else defs[0]
+    feps = 1e-5 if dt == np.float32 else 1e-9
+
+    def M(name):
+        name = name.strip()
+        if name not in mats:
+            if name in ("inputs",) and "genInput" in mats:
+                return matrix(mats["genInput"], dt)
+            raise Skip(f"matrix {name} is not a numeric literal")
+        return matrix(mats[name], dt)
+
+    def code(tok, table):
+        name = tok.split("::")[-1].strip()
+        if name not in table:
+            raise Skip(f"op {tok}")
+        return table[name]
+
+    if fn in ("checkEwBinaryMat",):
+        op = code(args[0], BIN)
+        if op >= 17:
+            raise Skip("integer/string op")
+        _eq(backend.ew_binary(op, M(args[1]), M(args[2])), M(args[3]))
+    elif fn == "checkEwBinaryObjSca":
+        op = code(args[0], BIN)
+        if op >= 17:
+            raise Skip("integer/string op")
+        _eq(backend.ew_binary_sca(op, M(args[1]), _scalar(args[2])), M(args[3]))
+    elif fn == "checkEwUnaryMat":
+        op = code(args[0], UN)
+        if op >= 19:
+            raise Skip("string op")
+        _eq(backend.ew_unary(op, M(args[1])), M(args[2]))
+    elif fn == "checkEwUnaryMatApprox":
+        _approx(backend.ew_unary(code(args[0], UN), M(args[1])), M(args[2]), 1e-2)  # EwUnaryMatTest.cpp: checkEqApprox(..., 1e-2)
+    elif fn == "checkEwUnaryMatThrow":
+        try:
+            backend.ew_unary(code(args[0], UN), M(args[1]))
+        except DomainError:
+            return
+        raise AssertionError("expected std::domain_error")
+    elif fn == "CHECK_THROWS" and "999" in args[0]:
+        a = M("arg") if "arg" in mats else M(next(iter(mats)))
+        try:
+            if "UnaryOpCode" in args[0]:
+                backend.ew_unary(999, a)
+            elif "ObjSca" in args[0]:
+                backend.ew_binary_sca(999, a, 1.0)
+            else:
+                backend.ew_binary(999, a, a)
+        except KernelError:
+            return
+        raise AssertionError("expected an exception for op code 999")
+    elif fn == "checkAggAll":
+        op = code(args[0], AGG)
+        exp = _scalar(args[2])
+        got = backend.agg_all(op, M(args[1]))
+        _approx(np.array([got]), np.array([exp]), max(feps, abs(exp) * (1e-6 if dt == np.float32 else 1e-14)))
+    elif fn in ("checkAggRow", "checkAggCol"):
+        op = code(args[0], AGG)
+        got = (backend.agg_row if fn == "checkAggRow" else backend.agg_col)(op, M(args[1]))
+        exp = M(args[2])
+        if op in (AGG["IDXMIN"], AGG["IDXMAX"]):
+            _eq(got.astype(np.float64), exp)
+        else:
+            _approx(got, exp, 1e-5)  # AggRowTest.cpp / AggColTest.cpp: checkEqApprox(..., 1e-5)
+    elif fn in ("checkMatMul", "checkMatMulCUDA"):
+        flags = [a.strip() for a in args[3:] if a.strip() in ("true", "false")]
+        ta = flags[0] == "true" if flags else False
+        tb = flags[1] == "true" if len(flags) > 1 else False
+        _eq(backend.matmul(M(args[0]), M(args[1]), ta, tb), M(args[2]))
+    elif fn == "checkSyrk":
+        m = M(args[0])
+        # SyrkTest.cpp:32-58: syrk(m) must equal matMul(t(m), m)
+        _eq(backend.syrk(m, True), backend.matmul(m, m, True, False))
+        _eq(backend.syrk(m, True), (m.astype(np.float64).T @ m.astype(np.float64)).astype(dt))
+    elif fn == "checkSolve":
+        # SolveTest.cpp:42-68: normal equations of X w = y, solved for w (eps 1e-6 ... 1e-4 for float)
+        X, w = M("X"), M("w")
+        y = backend.matmul(X, w, False, False)
+        A = backend.matmul(X, X, True, False)
+        b = backend.matmul(X, y, True, False)
+        _approx(backend.solve(A, b), w, 1e-3 if dt == np.float32 else 1e-6)
+    elif file.endswith("DNNConv2DForwardTest.cpp") and fn == "checkConv2DForward":
+        p = _ints(f["helper_calls"][0]["args"])  # C H W Hf Wf sh sw ph pw
+        inp, flt = M(args[0]), M(args[1])
+        bias = np.zeros((1, 1), dt)
+        res, oh, ow = backend.conv2d(inp, flt, bias, inp.shape[0], *p)
+        _eq(res, M(args[2]))
+    elif file.endswith("CUDA/DNNConvolutionTest.cpp") and fn == "direct":
+        p = _ints(f["helper_calls"][0]["args"])
+        inp, flt = M("input"), M("filter")
+        res, oh, ow = backend.conv2d(inp, flt, None, inp.shape[0], *p)
+        _eq(res, M("result"))
+    elif "Pooling" in file and fn == "checkPoolingForward":
+        if "AVG" in c["name"]:
+            raise Skip("average pooling is outside the kernel set")
+        if file.startswith("CUDA/"):
+            raise Skip("CUDA/DNNPoolingTest.cpp is not part of the reference's test build and its expectation "
+                       "belongs to other parameters than its call")
+        p = _ints(f["helper_calls"][0]["args"])  # C H W ph pw sh sw padh padw
+        inp = M(args[0])
+        res, oh, ow = backend.maxpool(inp, inp.shape[0], *p)
+        _eq(res, M(args[1]))
+    elif fn in ("checkBiasAddForward", "checkBiasAdd"):
+        _eq(backend.bias_add(M(args[0]), M(args[1])), M(args[2]))
+    elif "BatchNorm" in file and ("Inference" in fn or (fn == "direct" and "BatchNorm::Forward" in c["name"])):
+        x = M("input")
+        got = backend.batchnorm(x, M("gamma"), M("beta"), M("ema_mean"), M("ema_var"), 1e-5)
+        _approx(got, M("result"), 1e-4)  # the reference compares with Approx().epsilon(1e-5) on ~unit values
+    elif "Softmax" in file and fn == "direct":
+        got = backend.softmax(M("input"))
+        _approx(got, M("result"), 1e-6 if (dt == np.float32 or file.startswith("CUDA/")) else 1e-12)
+    elif file.endswith("CUDA/DNNAffineTest.cpp") and fn == "direct":
+        _eq(backend.affine(M("input"), M("weights"), M("bias")), M("result"))
+    elif file.endswith("CUDA/DNNActivationTest.cpp") and fn == "direct":
+        # ReLU == ewBinaryObjSca(MAX, x, 0): the reference has no CPU activation kernel
+        _eq(backend.ew_binary_sca(BIN["MAX"], M("input"), 0.0), M("result"))
+    else:
+        raise Skip(f"{fn} is outside the dense float/double kernel set")
