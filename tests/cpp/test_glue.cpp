@@ -1,0 +1,234 @@
+// Exercises the C++ kernel interface (daphne_amd/cpp/daphne_hip_kernels.h) the way the reference's
+// Catch2 unit tests exercise its device kernels: contexts built by hand, Kernel<...>::apply called
+// directly (reference: test/run_tests.cpp:28-49, test/runtime/local/kernels/CUDA/*.cpp). The
+// literals are the reference's own test vectors. Built with a plain host compiler.
+#include <cmath>
+#include <cstdio>
+#include <memory>
+#include <stdexcept>
+#include <vector>
+
+#include "../../daphne_amd/cpp/daphne_hip_kernels.h"
+
+static int g_fail = 0, g_checks = 0;
+#define CHECK(cond)                                                                                 \
+    do {                                                                                            \
+        g_checks++;                                                                                 \
+        if (!(cond)) {                                                                              \
+            g_fail++;                                                                               \
+            std::printf("FAILED %s:%d: %s\n", __FILE__, __LINE__, #cond);                           \
+        }                                                                                           \
+    } while (0)
+#define CHECK_THROWS_AS(expr, EX)                                                                   \
+    do {                                                                                            \
+        g_checks++;                                                                                 \
+        bool ok__ = false;                                                                          \
+        try {                                                                                       \
+            expr;                                                                                   \
+        } catch (const EX &) {                                                                      \
+            ok__ = true;                                                                            \
+        } catch (...) {                                                                             \
+        }                                                                                           \
+        if (!ok__) {                                                                                \
+            g_fail++;                                                                               \
+            std::printf("FAILED %s:%d: %s did not throw %s\n", __FILE__, __LINE__, #expr, #EX);     \
+        }                                                                                           \
+    } while (0)
+
+template <class DT> bool equals(const DT *m, const std::vector<typename DT::VT> &exp) { return m->toHost() == exp; }
+template <class DT> bool approx(const DT *m, const std::vector<typename DT::VT> &exp, double eps) {
+    auto v = m->toHost();
+    if (v.size() != exp.size())
+        return false;
+    for (size_t i = 0; i < v.size(); i++)
+        if (!(std::fabs(double(v[i]) - double(exp[i])) <= eps))
+            return false;
+    return true;
+}
+
+template <typename VT> void run_all(DaphneContext *dctx) {
+    using DT = DenseMatrix<VT>;
+    auto G = [&](size_t rows, std::vector<VT> v) { return genGivenVals<DT>(rows, v, dctx); };
+
+    // CUDA/MatMulTest.cpp:37-123
+    {
+        auto m1 = G(3, {1, 2, 3, 3, 1, 2, 2, 3, 1}), m2v = G(3, {13, 13, 10, 10, 13, 13, 13, 10, 13});
+        auto m3 = G(2, {1, 0, 3, 0, 0, 0, 2, 0}), m4 = G(4, {0, 1, 2, 0, 1, 1, 0, 0});
+        auto v2 = G(3, {1, 2, 3});
+        DT *res = nullptr;
+        HIP::matMul(res, m1, m1, false, false, dctx);
+        CHECK(equals(res, m2v->toHost()));
+        DataObjectFactory::destroy(res);
+        res = nullptr;
+        HIP::matMul(res, m3, m4, false, false, dctx);
+        CHECK(equals(res, {3, 4, 2, 2}));
+        DataObjectFactory::destroy(res);
+        res = nullptr;
+        HIP::matMul(res, m1, v2, false, false, dctx);
+        CHECK(equals(res, {14, 11, 11}));
+        DataObjectFactory::destroy(res);
+        // CUDA/MatMulTest.cpp:125-228 (transposed): m3 * m3^T
+        res = nullptr;
+        HIP::matMul(res, m3, m3, false, true, dctx);
+        CHECK(res->getNumRows() == 2 && res->getNumCols() == 2 && equals(res, {10, 6, 6, 4}));
+        DataObjectFactory::destroy(res);
+        res = nullptr;
+        CHECK_THROWS_AS(HIP::matMul(res, m3, m3, false, false, dctx), std::runtime_error);
+        CHECK(res == nullptr);
+        for (auto *m : {m1, m2v, m3, m4, v2})
+            DataObjectFactory::destroy(m);
+    }
+    // AggRowTest.cpp:221-277 (idxmin incl. ties), result type size_t
+    {
+        auto m1 = G(3, {4, 6, 3, 9, 2, 5, 0, 1, 7, 4, 5, 4});
+        DenseMatrix<size_t> *idx = nullptr;
+        HIP::aggRow(AggOpCode::IDXMIN, idx, m1, dctx);
+        CHECK(equals(idx, {2, 2, 1}));
+        DT *sum = nullptr;
+        HIP::aggRow(AggOpCode::SUM, sum, m1, dctx);
+        CHECK(equals(sum, {22, 8, 20}));
+        DT *cs = nullptr;
+        HIP::aggCol(AggOpCode::MAX, cs, m1, dctx);
+        CHECK(equals(cs, {7, 6, 5, 9}));
+        CHECK((HIP::aggAll<VT, DT>(AggOpCode::SUM, m1, dctx) == VT(50)));
+        CHECK_THROWS_AS(HIP::aggRow(static_cast<AggOpCode>(99), sum, m1, dctx), std::runtime_error);
+        DataObjectFactory::destroy(idx);
+        DataObjectFactory::destroy(sum);
+        DataObjectFactory::destroy(cs);
+        DataObjectFactory::destroy(m1);
+    }
+    // EwBinaryMatTest.cpp: add, broadcasting, invalid op code (:611), shape mismatch (EwBinaryMat.h:98-106)
+    {
+        auto m = G(2, {1, 2, 3, 4, 5, 6}), rv = G(1, {10, 20, 30}), cv = G(2, {100, 200}), bad = G(3, {1, 2, 3});
+        DT *res = nullptr;
+        HIP::ewBinaryMat(BinaryOpCode::ADD, res, m, rv, dctx);
+        CHECK(equals(res, {11, 22, 33, 14, 25, 36}));
+        HIP::ewBinaryMat(BinaryOpCode::ADD, res, res, cv, dctx); // in place, res aliases lhs (TasksCUDA.cpp:109)
+        CHECK(equals(res, {111, 122, 133, 214, 225, 236}));
+        DT *sca = nullptr;
+        HIP::ewBinaryObjSca(BinaryOpCode::GT, sca, m, VT(3), dctx);
+        CHECK(equals(sca, {0, 0, 0, 1, 1, 1}));
+        CHECK_THROWS_AS(HIP::ewBinaryMat(static_cast<BinaryOpCode>(999), res, m, m, dctx), std::runtime_error);
+        CHECK_THROWS_AS(HIP::ewBinaryMat(BinaryOpCode::ADD, res, m, bad, dctx), std::runtime_error);
+        // a view with rowSkip > numCols
+        std::unique_ptr<DT> view(m->slice(0, 2, 1, 3));
+        DT *vres = nullptr;
+        HIP::ewBinaryObjSca(BinaryOpCode::MUL, vres, view.get(), VT(2), dctx);
+        CHECK(equals(vres, {4, 6, 10, 12}));
+        for (auto *x : {m, rv, cv, bad, res, sca, vres})
+            DataObjectFactory::destroy(x);
+    }
+    // EwUnaryMatTest.cpp:148 sqrt domain_error, :62 abs
+    {
+        auto a = G(1, {-1, 4, 9}), b = G(1, {1, 4, 9});
+        DT *res = nullptr;
+        CHECK_THROWS_AS(HIP::ewUnaryMat(UnaryOpCode::SQRT, res, a, dctx), std::domain_error);
+        DataObjectFactory::destroy(res);
+        res = nullptr;
+        HIP::ewUnaryMat(UnaryOpCode::SQRT, res, b, dctx);
+        CHECK(equals(res, {1, 2, 3}));
+        HIP::ewUnaryMat(UnaryOpCode::ABS, res, a, dctx);
+        CHECK(equals(res, {1, 4, 9}));
+        CHECK_THROWS_AS(HIP::ewUnaryMat(static_cast<UnaryOpCode>(999), res, a, dctx), std::runtime_error);
+        for (auto *x : {a, b, res})
+            DataObjectFactory::destroy(x);
+    }
+    // DNNConv2DForwardTest.cpp:32-65 and CUDA/DNNConvolutionTest.cpp:36-43
+    {
+        std::vector<VT> img;
+        for (int r = 0; r < 2; r++)
+            for (int i = 1; i <= 27; i++)
+                img.push_back(VT(i));
+        auto input = G(2, img), filter = G(1, {1, 0, 0, 1, 1, 0, 0, 1, 1, 0, 0, 1}), bias = G(1, {0});
+        DT *res = nullptr;
+        size_t oh = 0, ow = 0;
+        HIP::Convolution::Forward<DT, DT>::apply(res, &oh, &ow, input, filter, bias, 2, 3, 3, 3, 2, 2, 2, 2, 1, 1, dctx);
+        CHECK(oh == 2 && ow == 2 && equals(res, {30, 36, 48, 96, 30, 36, 48, 96}));
+        auto in1 = G(1, {1, 2, 3, 4, 5, 6, 7, 8, 9}), f1 = G(1, {1, 0, 0, 1});
+        DT *res1 = nullptr;
+        HIP::Convolution::Forward<DT, DT>::apply(res1, &oh, &ow, in1, f1, nullptr, 1, 1, 3, 3, 2, 2, 1, 1, 0, 0, dctx);
+        CHECK(equals(res1, {6, 8, 12, 14}));
+        DT *res2 = nullptr;
+        CHECK_THROWS_AS((HIP::Convolution::Forward<DT, DT>::apply(res2, &oh, &ow, in1, f1, nullptr, 1, 1, 3, 3, 3, 3, 1, 1,
+                                                                  0, 0, dctx)),
+                        std::invalid_argument);
+        for (auto *x : {input, filter, bias, res, in1, f1, res1, res2})
+            DataObjectFactory::destroy(x);
+    }
+    // DNNPoolingTestForward.cpp:74-123 (2x2, stride 2, pad 1 on two 3x5x5 images)
+    {
+        std::vector<VT> v;
+        for (int i = 1; i <= 150; i++)
+            v.push_back(VT(i));
+        auto in = G(2, v);
+        DT *res = nullptr;
+        size_t oh = 0, ow = 0;
+        HIP::NN::Pooling::Forward<HIP::NN::Pooling::MAX, DT, DT>::apply(res, oh, ow, in, 2, 3, 5, 5, 2, 2, 2, 2, 1, 1, dctx);
+        std::vector<VT> exp;
+        for (int img = 0; img < 2; img++)
+            for (int c = 0; c < 3; c++)
+                for (int p : {0, 2, 4})
+                    for (int q : {0, 2, 4})
+                        exp.push_back(VT(img * 75 + c * 25 + p * 5 + q + 1));
+        CHECK(oh == 3 && ow == 3 && equals(res, exp));
+        DataObjectFactory::destroy(in);
+        DataObjectFactory::destroy(res);
+    }
+    // DNNBiasAddForwardTest.cpp:32-50, SoftmaxTest.cpp:17-34, CUDA/DNNAffineTest.cpp:28-45,
+    // DNNBatchNorm2DForwardTest.cpp:32-49
+    {
+        auto x = G(2, {1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12}), b = G(3, {1, 2, 3});
+        DT *res = nullptr;
+        HIP::BiasAdd<DT, DT>::apply(res, x, b, dctx);
+        CHECK(equals(res, {2, 3, 4, 5, 7, 8, 9, 10, 12, 13, 14, 15, 2, 3, 4, 5, 7, 8, 9, 10, 12, 13, 14, 15}));
+        auto s = G(3, {-3, -2, -1, 0, 1, 2, 3, 4, 5});
+        DT *sm = nullptr;
+        HIP::Softmax<DT, DT>::apply(sm, s, dctx);
+        CHECK(approx(sm, {VT(0.09003057317038046), VT(0.24472847105479764), VT(0.6652409557748218), VT(0.09003057317038046),
+                          VT(0.24472847105479764), VT(0.6652409557748218), VT(0.09003057317038046), VT(0.24472847105479764),
+                          VT(0.6652409557748218)},
+                     1e-6));
+        auto in = G(1, {-3, -2, -1, 0, 1, 2, 3, 4, 5}), w = G(9, {1, 1, 2, 2, 3, 3, 4, 4, 5, 5, 6, 6, 7, 7, 8, 8, 9, 9}),
+             b0 = G(1, {0});
+        DT *aff = nullptr;
+        HIP::NN::Affine::Forward<DT, DT>::apply(aff, in, w, b0, dctx);
+        CHECK(equals(aff, {105, 105}));
+        auto one = G(1, {1}), zero = G(1, {0});
+        DT *bn = nullptr;
+        HIP::BatchNormInferenceForward<DT, DT>::apply(bn, in, one, zero, zero, one, VT(1e-5), dctx);
+        CHECK(approx(bn, {-3, -2, -1, 0, 1, 2, 3, 4, 5}, 1e-4));
+        for (auto *m : {x, b, res, s, sm, in, w, b0, aff, one, zero, bn})
+            DataObjectFactory::destroy(m);
+    }
+    // SyrkTest.cpp:32-58 (syrk == t(X) X) and SolveTest.cpp:42-68 (normal equations)
+    {
+        auto X = G(7, {1, 4, 5, 3, 7, 1, 2, 3, 5, 9, 8, 1, 1, 2, 3, 5, 1, 9, 2, 3, 1}), w = G(3, {1, 2, 3});
+        DT *y = nullptr, *A = nullptr, *A2 = nullptr, *b = nullptr, *sol = nullptr;
+        HIP::matMul(y, X, w, false, false, dctx);
+        HIP::syrk(A, X, true, dctx);
+        HIP::matMul(A2, X, X, true, false, dctx);
+        CHECK(equals(A, A2->toHost()));
+        HIP::matMul(b, X, y, true, false, dctx);
+        HIP::solve(sol, A, b, dctx);
+        CHECK(approx(sol, {1, 2, 3}, sizeof(VT) == 4 ? 1e-3 : 1e-6));
+        for (auto *m : {X, w, y, A, A2, b, sol})
+            DataObjectFactory::destroy(m);
+    }
+}
+
+int main() {
+    // test/runtime/local/kernels/CUDA_ContextTest.cpp:25-30
+    auto dctx = std::make_unique<DaphneContext>();
+    try {
+        HIP::createHIPContext(dctx.get());
+    } catch (const std::exception &e) {
+        std::printf("FAILED to create the HIP context: %s\n", e.what());
+        return 2;
+    }
+    CHECK(dctx->useHIP());
+    CHECK(HIPContext::get(dctx.get(), 0)->getMemBudget() > 0);
+    run_all<float>(dctx.get());
+    run_all<double>(dctx.get());
+    std::printf("%s: %d checks, %d failed\n", g_fail ? "FAILED" : "PASSED", g_checks, g_fail);
+    return g_fail ? 1 : 0;
+}

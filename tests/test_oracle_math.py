@@ -1,0 +1,189 @@
+"""CPU: pins the oracle by what the mathematics fixes, independently of its own formulas: numpy /
+scipy library routines, closed forms, brute force on small inputs. Each check is chosen so that a
+plausible slip (dropped term, wrong sign or index, transposed operand, wrong divisor) fails it."""
+import numpy as np
+import pytest
+import scipy.special
+
+import oracle_binding as orc
+
+DT = [np.float32, np.float64]
+
+
+def tol(dt):
+    return 2e-6 if dt == np.float32 else 1e-13
+
+
+@pytest.mark.parametrize("dt", DT)
+def test_ew_single_ieee_ops_equal_numpy_bitwise(dt):
+    rng = np.random.default_rng(0)
+    a, b = rng.standard_normal((31, 17)).astype(dt), rng.standard_normal((31, 17)).astype(dt)
+    with np.errstate(all="ignore"):
+        for op, f in {0: np.add, 1: np.subtract, 2: np.multiply, 3: np.divide, 5: np.fmod}.items():
+            assert np.array_equal(orc.ew_binary(op, a, b)[1], f(a, b))
+        for op, f in {7: np.equal, 8: np.not_equal, 9: np.less, 10: np.less_equal, 11: np.greater, 12: np.greater_equal}.items():
+            assert np.array_equal(orc.ew_binary(op, a, b)[1], f(a, b).astype(dt))
+        assert np.array_equal(orc.ew_binary(13, a, b)[1], np.minimum(a, b))
+        assert np.array_equal(orc.ew_binary(14, a, b)[1], np.maximum(a, b))
+        assert np.allclose(orc.ew_binary(4, np.abs(a), b)[1], np.power(np.abs(a), b), rtol=tol(dt) * 10)
+        assert np.allclose(orc.ew_binary(6, np.abs(a) + 1, np.abs(b) + 2)[1], np.log(np.abs(a) + 1) / np.log(np.abs(b) + 2), rtol=tol(dt) * 10)
+    # broadcasting: result has lhs' shape, row vector over rows, column vector over columns
+    rv, cv = b[:1], b[:, :1]
+    assert np.array_equal(orc.ew_binary(1, a, rv)[1], a - rv)
+    assert np.array_equal(orc.ew_binary(1, a, cv)[1], a - cv)
+    assert orc.ew_binary(0, a, b[:5])[0] == orc.ST_RUNTIME
+    # std::min / std::max NaN rule: NaN on the right is ignored, NaN on the left stays
+    x, y = np.array([[np.nan, 1.0]], dt), np.array([[1.0, np.nan]], dt)
+    r = orc.ew_binary(13, x, y)[1]
+    assert np.isnan(r[0, 0]) and r[0, 1] == 1.0
+
+
+@pytest.mark.parametrize("dt", DT)
+def test_unary_against_numpy(dt):
+    rng = np.random.default_rng(1)
+    a = rng.standard_normal((9, 13)).astype(dt) * 2
+    fns = {0: np.negative, 1: np.abs, 2: np.sign, 4: np.exp, 6: np.sin, 7: np.cos, 8: np.tan, 11: np.arctan, 12: np.sinh,
+           13: np.cosh, 14: np.tanh, 15: np.floor, 16: np.ceil}
+    for op, f in fns.items():
+        assert np.allclose(orc.ew_unary(op, a)[1], f(a), rtol=tol(dt) * 20, atol=0), op
+    assert np.array_equal(orc.ew_unary(3, np.abs(a))[1], np.sqrt(np.abs(a)))
+    # round: half away from zero (C round), unlike numpy's half-to-even
+    h = np.array([[0.5, 1.5, 2.5, -0.5, -1.5, -2.5]], dt)
+    assert np.array_equal(orc.ew_unary(17, h)[1], np.array([[1, 2, 3, -1, -2, -3]], dt))
+    assert np.array_equal(orc.ew_unary(18, np.array([[np.nan, 1.0]], dt))[1], np.array([[1, 0]], dt))
+    for op, bad in ((3, -1.0), (5, -1.0), (9, 1.01), (10, -1.01)):
+        assert orc.ew_unary(op, np.array([[0.5, bad]], dt))[0] == orc.ST_DOMAIN
+        assert orc.ew_unary(op, np.array([[0.5, 0.25]], dt))[0] == 0
+    assert orc.ew_unary(3, np.array([[-0.0, np.nan]], dt))[0] == 0  # -0 and NaN are inside the domain check
+
+
+@pytest.mark.parametrize("dt", DT)
+def test_aggregations_against_numpy(dt):
+    rng = np.random.default_rng(2)
+    a = (rng.standard_normal((57, 23)) * 3 + 1).astype(dt)
+    a64 = a.astype(np.float64)
+    rt = 1e-5 if dt == np.float32 else 1e-12
+    at = rt * np.abs(a64).sum(axis=1).max()  # sums with cancellation: error relative to the summed magnitudes
+    for op, f in {0: np.sum, 2: np.min, 3: np.max, 6: np.mean, 7: np.std, 8: np.var}.items():
+        assert np.allclose(orc.agg_all(op, a)[1], f(a64), rtol=rt, atol=at)
+        assert np.allclose(orc.agg_row(op, a)[1][:, 0], f(a64, axis=1), rtol=rt, atol=at)
+        assert np.allclose(orc.agg_col(op, a)[1][0], f(a64, axis=0), rtol=rt, atol=at)
+    p = (1 + 0.01 * rng.standard_normal((11, 7))).astype(dt)
+    assert np.allclose(orc.agg_all(1, p)[1], np.prod(p.astype(np.float64)), rtol=rt)
+    # index of the first strict extremum == numpy argmin / argmax (ties: first)
+    t = rng.integers(0, 4, (40, 9)).astype(dt)
+    assert np.array_equal(orc.agg_row(4, t)[1][:, 0], np.argmin(t, axis=1).astype(np.uint64))
+    assert np.array_equal(orc.agg_row(5, t)[1][:, 0], np.argmax(t, axis=1).astype(np.uint64))
+    assert np.array_equal(orc.agg_col(4, t)[1][0], np.argmin(t, axis=0).astype(np.uint64))
+    assert np.array_equal(orc.agg_col(5, t)[1][0], np.argmax(t, axis=0).astype(np.uint64))
+    # views: leading dimension larger than the column count
+    big = rng.standard_normal((20, 30)).astype(dt)
+    v = big[3:17, 4:21]
+    assert np.allclose(orc.agg_all(0, v)[1], v.astype(np.float64).sum(), rtol=rt)
+    assert np.allclose(orc.agg_col(8, v)[1][0], v.astype(np.float64).var(axis=0), rtol=rt)
+
+
+@pytest.mark.parametrize("dt", DT)
+def test_contractions_against_numpy(dt):
+    rng = np.random.default_rng(3)
+    rt = 1e-5 if dt == np.float32 else 1e-12
+    A, B = rng.standard_normal((13, 29)).astype(dt), rng.standard_normal((29, 7)).astype(dt)
+    ref = A.astype(np.float64) @ B.astype(np.float64)
+    for ta, tb in ((0, 0), (1, 0), (0, 1), (1, 1)):
+        a = np.ascontiguousarray(A.T) if ta else A
+        b = np.ascontiguousarray(B.T) if tb else B
+        st, got = orc.matmul(a, b, ta, tb)
+        assert st == 0 and np.allclose(got, ref, rtol=rt, atol=rt * np.abs(ref).max())
+    assert orc.matmul(A, A)[0] == orc.ST_RUNTIME
+    X = rng.standard_normal((50, 6)).astype(dt)
+    for tl in (True, False):
+        st, S = orc.syrk(X, tl)
+        refS = X.astype(np.float64).T @ X.astype(np.float64) if tl else X.astype(np.float64) @ X.astype(np.float64).T
+        assert np.allclose(S, refS, rtol=rt, atol=rt * np.abs(refS).max()) and np.array_equal(S, S.T)
+    M = rng.standard_normal((12, 12)).astype(dt) + 4 * np.eye(12, dtype=dt)
+    b = rng.standard_normal((12, 1)).astype(dt)
+    st, x = orc.solve(M, b)
+    assert st == 0 and np.allclose(x, np.linalg.solve(M.astype(np.float64), b.astype(np.float64)), rtol=1e-3 if dt == np.float32 else 1e-10)
+    assert orc.solve(np.zeros((3, 3), dt), np.ones((3, 1), dt))[0] == orc.ST_RUNTIME
+    # a system that needs the row exchange (zero leading pivot)
+    P = np.array([[0, 2, 1], [1, 1, 1], [2, 0, 3]], dt)
+    assert np.allclose(orc.solve(P, np.array([[3], [3], [5]], dt))[1], np.linalg.solve(P.astype(np.float64), [[3], [3], [5]]), rtol=1e-5)
+
+
+def _conv_brute(x, w, bias, N, C, H, W, F, Hf, Wf, sh, sw, ph, pw):
+    xp = np.zeros((N, C, H + 2 * ph, W + 2 * pw))
+    xp[:, :, ph:ph + H, pw:pw + W] = x.reshape(N, C, H, W)
+    P, Q = (H + 2 * ph - Hf) // sh + 1, (W + 2 * pw - Wf) // sw + 1
+    win = np.lib.stride_tricks.sliding_window_view(xp, (Hf, Wf), axis=(2, 3))[:, :, ::sh, ::sw][:, :, :P, :Q]
+    out = np.einsum("ncpqhw,fchw->nfpq", win, w.reshape(F, C, Hf, Wf).astype(np.float64))
+    if bias is not None:
+        out += bias.reshape(1, F, 1, 1)
+    return out.reshape(N, F * P * Q), P, Q
+
+
+@pytest.mark.parametrize("dt", DT)
+@pytest.mark.parametrize("case", [(2, 3, 7, 6, 4, 3, 2, 1, 1, 1, 0), (1, 2, 9, 9, 5, 3, 3, 2, 2, 1, 1), (3, 1, 5, 5, 2, 5, 5, 1, 1, 2, 2),
+                                  (2, 4, 6, 8, 3, 1, 1, 1, 2, 0, 0)])
+def test_conv_against_brute_force(dt, case):
+    N, C, H, W, F, Hf, Wf, sh, sw, ph, pw = case
+    rng = np.random.default_rng(sum(case))
+    x = rng.standard_normal((N, C * H * W)).astype(dt)
+    w = rng.standard_normal((F, C * Hf * Wf)).astype(dt)
+    b = rng.standard_normal((F, 1)).astype(dt)
+    st, got, oh, ow = orc.conv2d(x, w, b, N, C, H, W, Hf, Wf, sh, sw, ph, pw)
+    exp, P, Q = _conv_brute(x.astype(np.float64), w, b.astype(np.float64), N, C, H, W, F, Hf, Wf, sh, sw, ph, pw)
+    assert st == 0 and (oh, ow) == (P, Q)
+    assert np.allclose(got, exp, rtol=1e-4 if dt == np.float32 else 1e-11, atol=1e-4 if dt == np.float32 else 1e-11)
+
+
+@pytest.mark.parametrize("dt", DT)
+@pytest.mark.parametrize("case", [(2, 3, 6, 6, 2, 2, 2, 2, 0, 0), (1, 2, 7, 5, 3, 3, 1, 1, 1, 1), (2, 1, 8, 8, 3, 2, 2, 2, 1, 1)])
+def test_maxpool_against_brute_force(dt, case):
+    N, C, H, W, ph, pw, sh, sw, padh, padw = case
+    rng = np.random.default_rng(sum(case))
+    x = rng.standard_normal((N, C * H * W)).astype(dt)
+    st, got, oh, ow = orc.maxpool(x, N, C, H, W, ph, pw, sh, sw, padh, padw)
+    xp = np.zeros((N, C, H + 2 * padh, W + 2 * padw), dt)  # zero padding takes part, and the fold starts at 0
+    xp[:, :, padh:padh + H, padw:padw + W] = x.reshape(N, C, H, W)
+    P, Q = (H + 2 * padh - ph) // sw + 1, (W + 2 * padw - pw) // sh + 1  # the reference's swapped strides
+    exp = np.zeros((N, C, P, Q), dt)
+    for p in range(P):
+        for q in range(Q):
+            win = xp[:, :, p * sh:p * sh + ph, q * sw:q * sw + pw]
+            exp[:, :, p, q] = np.maximum(0, win.max(axis=(2, 3)))
+    assert st == 0 and (oh, ow) == (P, Q) and np.array_equal(got, exp.reshape(N, -1))
+
+
+@pytest.mark.parametrize("dt", DT)
+def test_channel_ops_and_softmax_closed_forms(dt):
+    rng = np.random.default_rng(5)
+    N, C, HW = 4, 3, 10
+    x = rng.standard_normal((N, C * HW)).astype(dt)
+    b = rng.standard_normal((C, 1)).astype(dt)
+    assert np.array_equal(orc.bias_add(x, b)[1], (x.reshape(N, C, HW) + b.reshape(1, C, 1)).reshape(N, -1))
+    g, be, mu, var = (rng.random((C, 1)).astype(dt) + 0.5 for _ in range(4))
+    exp = (g.reshape(1, C, 1) * (x.reshape(N, C, HW) - mu.reshape(1, C, 1)) / np.sqrt(var.reshape(1, C, 1) + dt(1e-5))
+           + be.reshape(1, C, 1)).reshape(N, -1)
+    assert np.allclose(orc.batchnorm(x, g, be, mu, var, 1e-5, 0)[1], exp, rtol=1e-5 if dt == np.float32 else 1e-13)
+    gi, bi, mi, vi = (rng.random((N, 1)).astype(dt) + 0.5 for _ in range(4))
+    exp = gi * (x - mi) / np.sqrt(vi + dt(1e-5)) + bi  # statistics per row, the reference's CPU loop
+    assert np.allclose(orc.batchnorm(x, gi, bi, mi, vi, 1e-5, 1)[1], exp, rtol=1e-5 if dt == np.float32 else 1e-13)
+    s = orc.softmax(x * 5)[1]
+    assert np.allclose(s, scipy.special.softmax(x.astype(np.float64) * 5, axis=1), rtol=1e-5 if dt == np.float32 else 1e-13)
+    assert np.allclose(s.sum(axis=1), 1.0, rtol=1e-5)
+
+
+def test_vectorized_engine_equals_plain_kernels():
+    """The multithreaded row-split engine gives what the plain kernels give on the whole matrix
+    (reference: test/runtime/local/vectorized/MultiThreadedKernelTest.cpp:41-154)."""
+    rng = np.random.default_rng(6)
+    x = (rng.standard_normal((5000, 64)) * 2 + 5).astype(np.float32)
+    st, mu, sd, r, s, _ = orc.zscore_pipeline(x, threads=5, thr=64.0)
+    mu1 = orc.agg_col(6, x)[1]
+    sd1 = orc.ew_unary(3, orc.agg_col(8, x)[1])[1]
+    z = orc.ew_binary(3, orc.ew_binary(1, x, mu1)[1], sd1)[1]
+    r1 = orc.agg_row(0, orc.ew_binary(2, z, z)[1])[1]
+    assert np.array_equal(mu, mu1) and np.array_equal(sd, sd1) and np.array_equal(r, r1)
+    assert s == float((r1 > 64.0).sum())
+    for threads in (1, 2, 7):
+        assert np.array_equal(orc.zscore_pipeline(x, threads=threads, thr=64.0)[3], r1)
