@@ -11,7 +11,7 @@
 // self-contained so that it can be built and tested without the DAPHNE source tree: DenseMatrix,
 // DaphneContext, IContext and DataObjectFactory below are minimal device-resident counterparts
 // with the reference's member names (getNumRows / getNumCols / getRowSkip / getValues, ...).
-// Inside DAPHNE the same kernel bodies bind to the real classes; INTEGRATION.md shows that glue.
+// Inside DAPHNE the same kernel bodies bind to the real classes (getValues(&alloc_desc) for the device pointer).
 #pragma once
 
 #include <algorithm>
