@@ -107,6 +107,17 @@ template <typename T, int R, int BK, bool KCONTIG, int THREADS> struct TileMover
             }
         }
     }
+    // Interior tile of an aligned matrix: plain 16-byte loads, no bounds logic.
+    __device__ __forceinline__ void load_full(const T *__restrict__ base, size_t ld, size_t outer0, size_t inner0,
+                                              int tid) {
+        static_assert(NVEC % THREADS == 0, "full tiles only for tile shapes that divide evenly");
+#pragma unroll
+        for (int i = 0; i < PER_THREAD; i++) {
+            const int v = tid + i * THREADS;
+            const int o = v / VPR, iv = v % VPR;
+            dh_load_vec<T, VEC>(base + (outer0 + o) * ld + inner0 + static_cast<size_t>(iv) * VEC, regs[i]);
+        }
+    }
     __device__ __forceinline__ void store(T *lds, int tid) const {
 #pragma unroll
         for (int i = 0; i < PER_THREAD; i++) {
@@ -170,8 +181,11 @@ __device__ __forceinline__ void tile_of_block(const GemmArgs &g, int &tm, int &t
     tn = in_panel / rows_here;
 }
 
-template <typename T, int BM, int BN, int BK, int WM, int WN, bool TA, bool TB, int EPI>
-__global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(GemmArgs g) {
+// FULL: every tile is interior and both operands are 16-byte aligned (checked on the host): no
+// bounds logic in the loads and stores, and the register budget is held to two workgroups per CU
+// so that a second wavefront per SIMD covers the global-load latency of the first.
+template <typename T, int BM, int BN, int BK, int WM, int WN, bool TA, bool TB, int EPI, bool FULL = false>
+__global__ __launch_bounds__(64 * WM * WN, FULL ? 2 : 1) void gemm_kernel(GemmArgs g) {
     using M = Mfma<T>;
     constexpr int THREADS = 64 * WM * WN;
     constexpr int TM = BM / WM, TN = BN / WN;
@@ -207,6 +221,17 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(GemmArgs g) {
     TileMover<T, BM, BK, A_KC, THREADS> mv_a;
     TileMover<T, BN, BK, B_KC, THREADS> mv_b;
     auto fetch = [&](size_t k0) {
+        if constexpr (FULL) {
+            if constexpr (A_KC)
+                mv_a.load_full(A, g.lda, m0, k0, tid);
+            else
+                mv_a.load_full(A, g.lda, k0, m0, tid);
+            if constexpr (B_KC)
+                mv_b.load_full(B, g.ldb, n0, k0, tid);
+            else
+                mv_b.load_full(B, g.ldb, k0, n0, tid);
+            return;
+        }
         if constexpr (A_KC)
             mv_a.load(A, g.lda, m0, k0, g.m, k_end, g.aligned_a, tid);
         else
@@ -263,14 +288,14 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_kernel(GemmArgs g) {
 #pragma unroll
         for (int j = 0; j < FN; j++) {
             const size_t c = n0 + wave_n * TN + j * M::NT + M::col(lane);
-            if (c < g.n) {
+            if (FULL || c < g.n) {
                 T b = T(0);
                 if constexpr (EPI == EPI_BIAS)
                     b = static_cast<const T *>(g.bias)[c * g.bias_stride];
 #pragma unroll
                 for (int v = 0; v < M::ACC; v++) {
                     const size_t r = m0 + wave_m * TM + i * M::MT + M::row(lane, v);
-                    if (r < g.m)
+                    if (FULL || r < g.m)
                         C[r * g.ldc + c] = acc[i][j][v] + b;
                 }
             }
@@ -375,17 +400,17 @@ __global__ __launch_bounds__(256) void gemv_t_stage2(const T *partials, size_t n
 // ---------------------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------------------
-template <typename T, int BM, int BN, int BK, int WM, int WN, int EPI>
+template <typename T, int BM, int BN, int BK, int WM, int WN, int EPI, bool FULL = false>
 static inline void launch_cfg(dh_ctx *ctx, const GemmArgs &g, bool ta, bool tb, dim3 grid) {
     const dim3 block(64 * WM * WN);
     if (!ta && !tb)
-        hipLaunchKernelGGL((gemm_kernel<T, BM, BN, BK, WM, WN, false, false, EPI>), grid, block, 0, ctx->stream, g);
+        hipLaunchKernelGGL((gemm_kernel<T, BM, BN, BK, WM, WN, false, false, EPI, FULL>), grid, block, 0, ctx->stream, g);
     else if (!ta && tb)
-        hipLaunchKernelGGL((gemm_kernel<T, BM, BN, BK, WM, WN, false, true, EPI>), grid, block, 0, ctx->stream, g);
+        hipLaunchKernelGGL((gemm_kernel<T, BM, BN, BK, WM, WN, false, true, EPI, FULL>), grid, block, 0, ctx->stream, g);
     else if (ta && !tb)
-        hipLaunchKernelGGL((gemm_kernel<T, BM, BN, BK, WM, WN, true, false, EPI>), grid, block, 0, ctx->stream, g);
+        hipLaunchKernelGGL((gemm_kernel<T, BM, BN, BK, WM, WN, true, false, EPI, FULL>), grid, block, 0, ctx->stream, g);
     else
-        hipLaunchKernelGGL((gemm_kernel<T, BM, BN, BK, WM, WN, true, true, EPI>), grid, block, 0, ctx->stream, g);
+        hipLaunchKernelGGL((gemm_kernel<T, BM, BN, BK, WM, WN, true, true, EPI, FULL>), grid, block, 0, ctx->stream, g);
 }
 
 // K depth of an LDS tile: 16 floats or 8 doubles (64 bytes per row either way), which keeps the
@@ -478,7 +503,11 @@ dh_status gemm(dh_ctx *ctx, bool ta, bool tb, size_t m, size_t n, size_t k, cons
         else                                                                                       \
             launch_cfg<T, BM_, BN_, GEMM_BK, WM_, WN_, EPI_STORE>(ctx, g, ta, tb, grid);           \
     } while (0)
-    if (bm == 128 && bn == 128)
+    const bool full = bm == 128 && bn == 128 && !fuse_bias && m % 128 == 0 && n % 128 == 0 && k % GEMM_BK == 0 &&
+                      g.aligned_a && g.aligned_b && k > 0;
+    if (full)
+        launch_cfg<T, 128, 128, GEMM_BK, 2, 2, EPI_STORE, true>(ctx, g, ta, tb, grid);
+    else if (bm == 128 && bn == 128)
         DH_LAUNCH(128, 128, 2, 2);
     else if (bm == 256)
         DH_LAUNCH(256, 32, 4, 1);
