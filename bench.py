@@ -33,6 +33,9 @@ HBM_PEAK_GBS = 8000.0
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--config", type=int, default=2, choices=[1, 2, 3, 4, 5],
+                    help="which BASELINE.json configuration to run (1-based); the default 2 is the headline "
+                         "metric, the others print the same kind of line for their own workload")
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--rows", type=int, default=20_000_000)
@@ -48,6 +51,11 @@ def main() -> int:
         print(f"bench.py: this build runs on exactly one GPU; --gpus {args.gpus} is not supported "
               "(the path shards by rows with one small all-reduce, which is documented, not built).", file=sys.stderr)
         return 2
+
+    if args.config != 2:
+        import bench_other_configs
+
+        return bench_other_configs.run(args)
 
     import numpy as np
     import torch

@@ -1,0 +1,220 @@
+"""Benchmark lines for BASELINE.json configurations 1, 3, 4 and 5 (`python bench.py --config N`).
+
+Same conventions as bench.py: inputs resident in HBM before the timed region, K timed steps between
+synchronisations, one JSON line. `value` is the configuration's own figure of merit (GB/s over canonical
+algorithmic bytes for the HBM-bound ones, TFLOP/s for the contractions, images/s for the CNN), next to the
+roofline fraction of the dominant kernel and a bounded CPU baseline from the oracle's restatement."""
+from __future__ import annotations
+
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+HBM_PEAK_GBS = 8000.0
+MFMA_PEAK = {"f32": 157.3, "f64": 78.6}
+
+
+def _timed(torch, fn, steps, warmup):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) * 1e3 / steps
+
+
+def _events(torch, fn, reps=10):
+    """Average duration of one call of fn on the current stream, with device events."""
+    fn()
+    torch.cuda.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(reps):
+        fn()
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) / reps
+
+
+def _line(metric_value, unit, ms, args, dtype, workload, roofline, cpu, extra=None):
+    cfg = {"workload": workload}
+    cfg.update(extra or {})
+    return {"metric": "HBM GB/s (% peak) on fused ew+agg pipelines; MatMul/Syrk TFLOP/s (% MFMA peak)",
+            "value": round(metric_value, 3), "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+            "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": dtype, "data": "synthetic", "config": cfg, "roofline": roofline, "cpu_baseline": cpu}
+
+
+def run(args) -> int:
+    import torch
+
+    sys.path.insert(0, os.path.join(os.path.dirname(os.path.abspath(__file__)), "tests"))
+    from daphne_amd.kernels import DenseMatrix, HIPContext, matMul, syrk
+    from daphne_amd.workloads import KMeans, lenet_forward, lmds
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 1
+    ctx = HIPContext(0)
+    gen = torch.Generator(device="cuda").manual_seed(42)
+    threads = min(os.cpu_count() or 1, 16)
+    orc = None
+    if not args.no_cpu:
+        import oracle_binding as orc
+
+    if args.config == 1:
+        n, m = 100_000, 100
+        Xt = torch.rand(n, m, device="cuda", dtype=torch.float64, generator=gen)
+        w = torch.randn(m, 1, device="cuda", dtype=torch.float64, generator=gen)
+        yt = Xt @ w + 0.1 * torch.randn(n, 1, device="cuda", dtype=torch.float64, generator=gen)
+        X, y = DenseMatrix.from_torch(ctx, Xt), DenseMatrix.from_torch(ctx, yt)
+        eye = DenseMatrix.from_numpy(ctx, np.eye(m))
+        ms = _timed(torch, lambda: lmds(ctx, X, y, 1e-3, eye), args.steps, args.warmup)
+        t_syrk = _events(torch, lambda: syrk(None, X, True, ctx))
+        nbytes = (n * m * 8 + m * m * 8) + (n * m * 8 + n * 8 + m * 8) + 3 * m * m * 8
+        cpu = None
+        if orc:
+            Xh, yh = Xt.cpu().numpy(), yt.cpu().numpy()
+            t0 = time.perf_counter()
+            A = orc.syrk(Xh, True)[1] + np.eye(m) * 1e-3
+            b = orc.matmul(Xh, yh, True, False)[1]
+            orc.solve(A, b)
+            dt = time.perf_counter() - t0
+            cpu = {"value": round(nbytes / dt / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
+                   "sample": f"the whole configuration once, single thread, scalar loops ({dt:.2f} s)"}
+        roof = {"bound": "hbm", "kernel": "gemm_kernel<double,128,128,8,2,2,true,false> split-K (syrk)",
+                "achieved": round((n * m * 8 + m * m * 8) / t_syrk / 1e6, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round((n * m * 8 + m * m * 8) / t_syrk / 1e6 / HBM_PEAK_GBS, 4), "traffic": None}
+        out = _line(nbytes / ms / 1e6, "GB/s", ms, args, "f64",
+                    "lmDS normal equations: X 100000x100 f64; A = syrk(X) + 1e-3 I, b = t(X) y, solve (launch-latency bound)",
+                    roof, cpu, {"canonical_bytes_per_step": nbytes, "syrk_us": round(t_syrk * 1e3, 1)})
+    elif args.config == 3:
+        n, f, k = 2_000_000, 64, 16
+        centres = torch.randn(k, f, device="cuda", generator=gen) * 5
+        Xt = centres[torch.arange(n, device="cuda") % k] + torch.randn(n, f, device="cuda", generator=gen)
+        X = DenseMatrix.from_torch(ctx, Xt)
+        km = KMeans(ctx, X, k)
+        C0 = Xt[torch.arange(k, device="cuda") * 125000].contiguous()
+        state = {"C": DenseMatrix.from_torch(ctx, C0)}
+
+        def step():  # one Lloyd iteration
+            state["C"] = km.iterate(state["C"])
+
+        ms = _timed(torch, step, args.steps, args.warmup)
+        # canonical bytes per iteration: X C^T (read X, write D), D assembly 3 x |D|, idxmin (read D, write idx),
+        # one-hot P, P^T X (read P and X), colSums(P)
+        D = n * k * 4
+        nbytes = (n * f * 4 + D) + 3 * D + (D + n * 8) + D + (D + n * f * 4) + D
+        t_gemm = _events(torch, lambda: matMul(km.XC, X, state["C"], False, True, ctx))
+        cpu = None
+        if orc:
+            ns = 100_000
+            Xh = Xt[:ns].cpu().numpy()
+            Ch = C0.cpu().numpy()
+            t0 = time.perf_counter()
+            xx = orc.agg_row(0, orc.ew_binary(2, Xh, Xh)[1])[1]
+            XC = orc.matmul(Xh, Ch, False, True)[1]
+            cc = orc.agg_row(0, orc.ew_binary(2, Ch, Ch)[1])[1]
+            Dh = orc.ew_binary(0, orc.ew_binary(0, orc.ew_binary_sca(2, XC, -2.0)[1], xx)[1], np.ascontiguousarray(cc.T))[1]
+            idx = orc.agg_row(4, Dh)[1]
+            P = (idx == np.arange(k, dtype=np.uint64)[None, :]).astype(np.float32)
+            orc.matmul(P, Xh, True, False)
+            orc.agg_col(0, P)
+            dt = time.perf_counter() - t0
+            cpu = {"value": round(nbytes * (ns / n) / dt / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
+                   "sample": f"one iteration on the first {ns} of {n} rows, single thread ({dt:.2f} s)"}
+        roof = {"bound": "hbm", "kernel": "gemm_kernel<float,256,32,16,4,1,false,true> (X C^T)",
+                "achieved": round((n * f * 4 + D) / t_gemm / 1e6, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round((n * f * 4 + D) / t_gemm / 1e6 / HBM_PEAK_GBS, 4), "traffic": None}
+        out = _line(nbytes / ms / 1e6, "GB/s", ms, args, "f32",
+                    "k-means Lloyd iteration: X 2000000x64 f32 (16 Gaussians), C 16x64; step = one iteration",
+                    roof, cpu, {"canonical_bytes_per_step": nbytes, "xct_ms": round(t_gemm, 4)})
+    elif args.config == 4:
+        res = {}
+        for name, dt, n in (("matmul_f64_8192", torch.float64, 8192), ("matmul_f32_16384", torch.float32, 16384)):
+            A = torch.rand(n, n, device="cuda", dtype=dt, generator=gen) * 2 - 1
+            B = torch.rand(n, n, device="cuda", dtype=dt, generator=gen) * 2 - 1
+            Cm = torch.empty(n, n, device="cuda", dtype=dt)
+            dA, dB, dC = (DenseMatrix.from_torch(ctx, t) for t in (A, B, Cm))
+            ms = _timed(torch, lambda: matMul(dC, dA, dB, False, False, ctx), args.steps, args.warmup)
+            res[name] = {"ms": round(ms, 3), "tflops": round(2.0 * n ** 3 / ms / 1e9, 2)}
+            del A, B, Cm, dA, dB, dC
+            torch.cuda.empty_cache()
+        Xs = torch.rand(1_000_000, 1024, device="cuda", dtype=torch.float64, generator=gen) * 2 - 1
+        dX, S = DenseMatrix.from_torch(ctx, Xs), DenseMatrix(ctx, 1024, 1024, np.float64)
+        ms_s = _timed(torch, lambda: syrk(S, dX, True, ctx), args.steps, args.warmup)
+        res["syrk_f64_1e6x1024"] = {"ms": round(ms_s, 3), "tflops": round(1024 * 1025 * 1e6 / ms_s / 1e9, 2)}
+        cpu = None
+        if orc:
+            a = np.random.default_rng(0).random((512, 512))
+            t0 = time.perf_counter()
+            orc.matmul(a, a)
+            dt = time.perf_counter() - t0
+            cpu = {"value": round(2 * 512 ** 3 / dt / 1e12, 5), "unit": "TFLOP/s", "cores": 1, "kind": "port",
+                   "sample": f"f64 matMul 512^3 with the oracle's scalar triple loop, single thread ({dt:.2f} s); "
+                             "the reference calls OpenBLAS here, which is not available"}
+        f64 = res["matmul_f64_8192"]["tflops"]
+        roof = {"bound": "mfma", "kernel": "gemm_kernel<double,128,128,8,2,2,false,false,0,true>", "achieved": f64,
+                "peak": MFMA_PEAK["f64"], "unit": "TFLOP/s", "frac": round(f64 / MFMA_PEAK["f64"], 4), "traffic": None}
+        for v, key in ((res["matmul_f64_8192"], "f64"), (res["matmul_f32_16384"], "f32"), (res["syrk_f64_1e6x1024"], "f64")):
+            v["pct_of_mfma_peak"] = round(100 * v["tflops"] / MFMA_PEAK[key], 1)
+        out = _line(f64, "TFLOP/s", res["matmul_f64_8192"]["ms"], args, "f64",
+                    "dense contractions: (a) MatMul f64 8192^3 [value], (b) MatMul f32 16384^3, (c) Syrk f64 1000000x1024",
+                    roof, cpu, res)
+    else:
+        N = 4096
+        rng = np.random.default_rng(42)
+        he = lambda shape, fan: (rng.standard_normal(shape) * np.sqrt(2.0 / fan)).astype(np.float32)
+        small = lambda shape: (rng.standard_normal(shape) * 0.1).astype(np.float32)
+        Wh = {"w1": he((32, 25), 25), "b1": small((32, 1)), "w2": he((64, 800), 800), "b2": small((64, 1)),
+              "w3": he((3136, 512), 3136), "b3": small((1, 512)), "w4": he((512, 10), 512), "b4": small((1, 10))}
+        W = {k_: DenseMatrix.from_numpy(ctx, v) for k_, v in Wh.items()}
+        xt = torch.rand(N, 784, device="cuda", generator=gen)
+        x = DenseMatrix.from_torch(ctx, xt)
+        ms = _timed(torch, lambda: lenet_forward(ctx, x, W, N), args.steps, args.warmup)
+        layers, last = {}, [None]
+
+        def timer(name):
+            e = torch.cuda.Event(enable_timing=True)
+            e.record()
+            if last[0] is not None:
+                layers.setdefault(name, []).append((last[0], e))
+            last[0] = e
+
+        for _ in range(5):
+            last[0] = torch.cuda.Event(enable_timing=True)
+            last[0].record()
+            lenet_forward(ctx, x, W, N, timer)
+        torch.cuda.synchronize()
+        layer_ms = {k_: round(float(np.mean([a.elapsed_time(b) for a, b in v])), 4) for k_, v in layers.items()}
+        flops = {"conv1+bias": 2.0 * N * 32 * 784 * 25, "conv2+bias": 2.0 * N * 64 * 196 * 800, "affine1": 2.0 * N * 3136 * 512,
+                 "affine2": 2.0 * N * 512 * 10}
+        layer_tflops = {k_: round(flops[k_] / layer_ms[k_] / 1e9, 2) for k_ in flops}
+        cpu = None
+        if orc:
+            nb = 8
+            xh = xt[:nb].cpu().numpy()
+            relu = lambda a: orc.ew_binary_sca(14, a, 0.0)[1]
+            t0 = time.perf_counter()
+            h = relu(orc.conv2d(xh, Wh["w1"], Wh["b1"], nb, 1, 28, 28, 5, 5, 1, 1, 2, 2)[1])
+            h = orc.maxpool(h, nb, 32, 28, 28, 2, 2, 2, 2, 0, 0)[1]
+            h = relu(orc.conv2d(h, Wh["w2"], Wh["b2"], nb, 32, 14, 14, 5, 5, 1, 1, 2, 2)[1])
+            h = orc.maxpool(h, nb, 64, 14, 14, 2, 2, 2, 2, 0, 0)[1]
+            h = relu(orc.ew_binary(0, orc.matmul(h, Wh["w3"])[1], Wh["b3"])[1])
+            orc.softmax(orc.ew_binary(0, orc.matmul(h, Wh["w4"])[1], Wh["b4"])[1])
+            dt = time.perf_counter() - t0
+            cpu = {"value": round(nb / dt, 2), "unit": "images/s", "cores": 1, "kind": "port",
+                   "sample": f"batch {nb} of {N}, raw-pointer restatement of the reference loops, single thread ({dt:.2f} s)"}
+        c2 = layer_tflops["conv2+bias"]
+        roof = {"bound": "mfma", "kernel": "conv2d_kernel<float,64,128,16,4> (conv2: 4096x32x14x14, 64 filters 5x5)",
+                "achieved": c2, "peak": MFMA_PEAK["f32"], "unit": "TFLOP/s", "frac": round(c2 / MFMA_PEAK["f32"], 4), "traffic": None}
+        out = _line(N / ms * 1e3, "images/s", ms, args, "f32",
+                    "LeNet-style CNN inference, batch 4096, 1x28x28 input, conv-pool-conv-pool-affine-affine-softmax",
+                    roof, cpu, {"layer_ms": layer_ms, "layer_tflops": layer_tflops, "total_gflop": 100.6})
+    print(json.dumps(out))
+    return 0
