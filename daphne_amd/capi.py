@@ -45,6 +45,9 @@ def _signatures(lib: C.CDLL) -> None:
     lib.dh_ctx_mem_budget.restype = sz
     lib.dh_ctx_mem_in_use.argtypes = [ctxp]
     lib.dh_ctx_mem_in_use.restype = sz
+    lib.dh_ctx_mem_cached.argtypes = [ctxp]
+    lib.dh_ctx_mem_cached.restype = sz
+    lib.dh_ctx_release_cached.argtypes = [ctxp]
     lib.dh_ctx_device.argtypes = [ctxp]
     lib.dh_ctx_props.argtypes = [ctxp, C.POINTER(i32), C.POINTER(i32), C.POINTER(sz), C.c_char_p, sz]
     lib.dh_ctx_set_stream.argtypes = [ctxp, vp]

@@ -23,8 +23,16 @@ struct dh_ctx {
     hipDeviceProp_t props{};
     size_t mem_budget = 0;
     size_t mem_in_use = 0;
-    std::mutex lock;                  // guards allocations / mem_in_use
-    std::map<void *, size_t> allocations;
+    std::mutex lock;                  // guards allocations / mem_in_use / the block cache
+    struct Block {
+        size_t requested, capacity;
+    };
+    std::map<void *, Block> allocations;
+    // Blocks returned by dh_free, kept for reuse (hipMalloc/hipFree cost hundreds of microseconds
+    // and synchronise the device). Reuse is ordered by the context's stream.
+    std::multimap<size_t, void *> cached;
+    size_t cached_bytes = 0;   // sum of the capacities in `cached`
+    size_t reserved_bytes = 0; // capacities of live + cached blocks
 
     // Reduction workspace (partials of the two-stage aggregations, split-K slabs). Grown on
     // demand under ws_lock; kernels using it are serialised by that lock only for the

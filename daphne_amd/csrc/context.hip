@@ -84,6 +84,9 @@ extern "C" dh_status dh_ctx_destroy(dh_ctx *ctx) {
     for (auto &kv : ctx->allocations)
         (void)hipFree(kv.first);
     ctx->allocations.clear();
+    for (auto &kv : ctx->cached)
+        (void)hipFree(kv.second);
+    ctx->cached.clear();
     if (ctx->ws)
         (void)hipFree(ctx->ws);
     if (ctx->flag_dev)
@@ -121,6 +124,11 @@ extern "C" dh_status dh_ctx_props(const dh_ctx *ctx, int *compute_units, int *cl
 extern "C" dh_status dh_ctx_set_stream(dh_ctx *ctx, void *hip_stream) {
     if (ctx == nullptr)
         return dh_fail(DH_ERR_RUNTIME, "dh_ctx_set_stream: context is null");
+    if (ctx->stream != static_cast<hipStream_t>(hip_stream)) {
+        // cached blocks may still be in use by work queued on the old stream
+        (void)hipSetDevice(ctx->device);
+        DH_CHECK_HIP(hipStreamSynchronize(ctx->stream));
+    }
     ctx->stream = static_cast<hipStream_t>(hip_stream);
     return DH_OK;
 }
@@ -133,6 +141,34 @@ extern "C" dh_status dh_sync(dh_ctx *ctx) {
     return DH_OK;
 }
 
+// Capacity class of a request: multiples of 512 B below 64 KiB, above that 1/16 of the largest
+// power of two not above the request (at most 6.25 % slack), so that repeated requests of similar
+// size share cached blocks.
+static size_t block_capacity(size_t bytes) {
+    if (bytes == 0)
+        bytes = 1; // a zero-size request still gets a distinct pointer as its registry key
+    size_t gran = 512;
+    if (bytes >= (size_t(64) << 10)) {
+        size_t p2 = size_t(1) << 16;
+        while ((p2 << 1) != 0 && (p2 << 1) <= bytes)
+            p2 <<= 1;
+        gran = p2 / 16;
+    }
+    return (bytes + gran - 1) / gran * gran;
+}
+
+// Returns every cached block to the driver. Caller holds ctx->lock.
+static void release_cached_locked(dh_ctx *ctx) {
+    if (ctx->cached.empty())
+        return;
+    (void)hipStreamSynchronize(ctx->stream);
+    for (auto &kv : ctx->cached)
+        (void)hipFree(kv.second);
+    ctx->reserved_bytes -= ctx->cached_bytes;
+    ctx->cached_bytes = 0;
+    ctx->cached.clear();
+}
+
 extern "C" dh_status dh_malloc(dh_ctx *ctx, size_t bytes, int zero, void **out) {
     DH_REQUIRE_CTX(ctx);
     if (out == nullptr)
@@ -142,20 +178,38 @@ extern "C" dh_status dh_malloc(dh_ctx *ctx, size_t bytes, int zero, void **out) 
     if (ctx->mem_in_use + bytes > ctx->mem_budget)
         return dh_fail(DH_ERR_OOM, "dh_malloc: %zu bytes requested, %zu in use, budget %zu", bytes, ctx->mem_in_use,
                        ctx->mem_budget);
+    const size_t cap = block_capacity(bytes);
     void *p = nullptr;
-    // A zero-size request still gets a distinct pointer so it can serve as a registry key.
-    hipError_t e = hipMalloc(&p, bytes ? bytes : 1);
-    if (e != hipSuccess)
-        return dh_fail(e == hipErrorOutOfMemory ? DH_ERR_OOM : DH_ERR_HIP, "hipMalloc(%zu): %s", bytes,
-                       hipGetErrorString(e));
+    auto it = ctx->cached.lower_bound(cap);
+    if (it != ctx->cached.end() && it->first == cap) {
+        p = it->second;
+        ctx->cached.erase(it);
+        ctx->cached_bytes -= cap;
+    } else {
+        if (ctx->reserved_bytes + cap > ctx->mem_budget)
+            release_cached_locked(ctx);
+        hipError_t e = hipMalloc(&p, cap);
+        if (e == hipErrorOutOfMemory && !ctx->cached.empty()) {
+            (void)hipGetLastError();
+            release_cached_locked(ctx);
+            e = hipMalloc(&p, cap);
+        }
+        if (e != hipSuccess) {
+            (void)hipGetLastError();
+            return dh_fail(e == hipErrorOutOfMemory ? DH_ERR_OOM : DH_ERR_HIP, "hipMalloc(%zu): %s", cap,
+                           hipGetErrorString(e));
+        }
+        ctx->reserved_bytes += cap;
+    }
     if (zero && bytes) {
-        e = hipMemsetAsync(p, 0, bytes, ctx->stream);
+        hipError_t e = hipMemsetAsync(p, 0, bytes, ctx->stream);
         if (e != hipSuccess) {
             (void)hipFree(p);
+            ctx->reserved_bytes -= cap;
             return dh_fail(DH_ERR_HIP, "hipMemsetAsync: %s", hipGetErrorString(e));
         }
     }
-    ctx->allocations[p] = bytes;
+    ctx->allocations[p] = dh_ctx::Block{bytes, cap};
     ctx->mem_in_use += bytes;
     *out = p;
     return DH_OK;
@@ -169,10 +223,21 @@ extern "C" dh_status dh_free(dh_ctx *ctx, void *ptr) {
     auto it = ctx->allocations.find(ptr);
     if (it == ctx->allocations.end())
         return dh_fail(DH_ERR_RUNTIME, "dh_free: pointer %p was not allocated by this context", ptr);
-    // hipFree waits for outstanding work that may still use the buffer.
-    DH_CHECK_HIP(hipFree(ptr));
-    ctx->mem_in_use -= it->second;
+    // The block goes back to the cache without waiting: whatever still uses it was queued on the
+    // context's stream, and so is whatever will use it next.
+    ctx->mem_in_use -= it->second.requested;
+    ctx->cached.emplace(it->second.capacity, ptr);
+    ctx->cached_bytes += it->second.capacity;
     ctx->allocations.erase(it);
+    return DH_OK;
+}
+
+extern "C" size_t dh_ctx_mem_cached(const dh_ctx *ctx) { return ctx ? ctx->cached_bytes : 0; }
+
+extern "C" dh_status dh_ctx_release_cached(dh_ctx *ctx) {
+    DH_REQUIRE_CTX(ctx);
+    std::lock_guard<std::mutex> g(ctx->lock);
+    release_cached_locked(ctx);
     return DH_OK;
 }
 

@@ -33,7 +33,25 @@ struct ConvArgs {
     unsigned K;          // C*Hf*Wf
     int aligned_w;       // filter rows can be read with 16-byte loads
     size_t pixels;       // N*P*Q
+    const int *ktab;     // per k (padded to a multiple of the K tile): offset of (c, hy, hx) in an image,
+                         // then hy << 16 | hx; entries beyond K are zero
 };
+
+// k = (c, hy, hx) -> { c*H*W + hy*W + hx, hy << 16 | hx }, so that the gather does no divisions.
+static __global__ void conv_table_kernel(int *tab, unsigned K, unsigned Kpad, unsigned HW, unsigned W, unsigned Hf,
+                                         unsigned Wf) {
+    for (unsigned k = blockIdx.x * blockDim.x + threadIdx.x; k < Kpad; k += gridDim.x * blockDim.x) {
+        int off = 0, yx = 0;
+        if (k < K) {
+            const unsigned c = k / (Hf * Wf), hw = k % (Hf * Wf);
+            const unsigned hy = hw / Wf, hx = hw % Wf;
+            off = static_cast<int>(c * HW + hy * W + hx);
+            yx = static_cast<int>(hy << 16 | hx);
+        }
+        tab[k] = off;
+        tab[Kpad + k] = yx;
+    }
+}
 
 template <typename T, int BM, int BN, int BK, int WN>
 __global__ __launch_bounds__(64 * WN) void conv2d_kernel(ConvArgs g) {
@@ -53,7 +71,7 @@ __global__ __launch_bounds__(64 * WN) void conv2d_kernel(ConvArgs g) {
     const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
     const size_t pix0 = static_cast<size_t>(blockIdx.x) * BN;
     const size_t f0 = static_cast<size_t>(blockIdx.y) * BM;
-    const unsigned PQ = g.P * g.Q, HW = g.H * g.W, HfWf = g.Hf * g.Wf;
+    const unsigned PQ = g.P * g.Q, HW = g.H * g.W;
 
     // the pixel this thread gathers for, decoded once
     constexpr int KG = THREADS / BN;      // K groups among the threads
@@ -61,32 +79,42 @@ __global__ __launch_bounds__(64 * WN) void conv2d_kernel(ConvArgs g) {
     const int gj = tid % BN, gkg = tid / BN;
     const size_t gpix = pix0 + gj;
     const bool pix_ok = gpix < g.pixels;
+    const bool small = g.pixels <= 0xffffffffull; // 32-bit divisions suffice (uniform)
     unsigned img = 0, p = 0, q = 0;
     if (pix_ok) {
-        img = static_cast<unsigned>(gpix / PQ);
-        const unsigned pq = static_cast<unsigned>(gpix % PQ);
+        unsigned pq;
+        if (small) {
+            img = static_cast<unsigned>(gpix) / PQ;
+            pq = static_cast<unsigned>(gpix) % PQ;
+        } else {
+            img = static_cast<unsigned>(gpix / PQ);
+            pq = static_cast<unsigned>(gpix % PQ);
+        }
         p = pq / g.Q;
         q = pq % g.Q;
     }
-    const T *ximg = X + static_cast<size_t>(img) * g.C * HW;
     const int y0 = static_cast<int>(p * g.sh) - static_cast<int>(g.ph);
-    const int x0 = static_cast<int>(q * g.sw) - static_cast<int>(g.pw);
+    // a pixel beyond the end gets a row origin that fails every bounds check
+    const int x0 = pix_ok ? static_cast<int>(q * g.sw) - static_cast<int>(g.pw) : -0x10000000;
+    const T *xpix = X + static_cast<size_t>(img) * g.C * HW + static_cast<ptrdiff_t>(y0) * static_cast<int>(g.W) + x0;
+    const unsigned Kpad = (g.K + BK - 1) / BK * BK;
+    const int *tab_off = g.ktab + gkg * KPT, *tab_yx = g.ktab + Kpad + gkg * KPT;
 
     TileMover<T, BM, BK, true, THREADS> mv_a;
     T gb[KPT];
     auto fetch = [&](unsigned k0) {
         mv_a.load(Wt, g.K, f0, k0, g.F, g.K, g.aligned_w != 0, tid);
+        int off[KPT], yx[KPT];
 #pragma unroll
         for (int i = 0; i < KPT; i++) {
-            const unsigned k = k0 + gkg * KPT + i;
-            T v = T(0);
-            if (pix_ok && k < g.K) {
-                const unsigned c = k / HfWf, hw = k % HfWf;
-                const int y = y0 + static_cast<int>(hw / g.Wf), x = x0 + static_cast<int>(hw % g.Wf);
-                if (y >= 0 && y < static_cast<int>(g.H) && x >= 0 && x < static_cast<int>(g.W))
-                    v = ximg[static_cast<size_t>(c) * HW + static_cast<unsigned>(y) * g.W + static_cast<unsigned>(x)];
-            }
-            gb[i] = v;
+            off[i] = tab_off[k0 + i];
+            yx[i] = tab_yx[k0 + i];
+        }
+#pragma unroll
+        for (int i = 0; i < KPT; i++) {
+            // unsigned compares fold the lower bound in: a negative coordinate wraps to a huge value
+            const unsigned y = static_cast<unsigned>(y0 + (yx[i] >> 16)), x = static_cast<unsigned>(x0 + (yx[i] & 0xffff));
+            gb[i] = (y < g.H && x < g.W && k0 + gkg * KPT + i < g.K) ? xpix[off[i]] : T(0);
         }
     };
     auto stash = [&](int buf) {
@@ -142,7 +170,14 @@ __global__ __launch_bounds__(64 * WN) void conv2d_kernel(ConvArgs g) {
     for (int j = 0; j < FN; j++) {
         const size_t pix = pix0 + wave * TN + j * M::NT + M::col(lane);
         if (pix < g.pixels) {
-            const size_t oimg = pix / PQ, opq = pix % PQ;
+            size_t oimg, opq;
+            if (small) {
+                oimg = static_cast<unsigned>(pix) / PQ;
+                opq = static_cast<unsigned>(pix) % PQ;
+            } else {
+                oimg = pix / PQ;
+                opq = pix % PQ;
+            }
             T *obase = out + oimg * g.F * PQ + opq;
 #pragma unroll
             for (int i = 0; i < FM; i++)
@@ -196,6 +231,17 @@ dh_status conv2d_forward(dh_ctx *ctx, T *res, size_t *res_h, size_t *res_w, cons
     const size_t gx = dh_ceil_div(pixels, BN);
     if (gx >= (size_t(1) << 31))
         return dh_fail(DH_ERR_RUNTIME, "Convolution: too many output pixels for one launch");
+    if (Hf >= 0x8000 || Wf >= 0x10000 || H >= (size_t(1) << 28) || W >= (size_t(1) << 28))
+        return dh_fail(DH_ERR_RUNTIME, "Convolution: filter or image side too large");
+    const unsigned Kpad = static_cast<unsigned>(dh_ceil_div(g.K, BK) * BK);
+    void *wsv = nullptr;
+    dh_status st = dh_workspace(ctx, 2 * static_cast<size_t>(Kpad) * sizeof(int), &wsv);
+    if (st != DH_OK)
+        return st;
+    g.ktab = static_cast<const int *>(wsv);
+    hipLaunchKernelGGL(conv_table_kernel, dim3(static_cast<unsigned>(dh_ceil_div(Kpad, 256) > 64 ? 64 : dh_ceil_div(Kpad, 256))),
+                       dim3(256), 0, ctx->stream, static_cast<int *>(wsv), g.K, Kpad, static_cast<unsigned>(H * W),
+                       static_cast<unsigned>(W), static_cast<unsigned>(Hf), static_cast<unsigned>(Wf));
     if (F <= 32) {
         hipLaunchKernelGGL((conv2d_kernel<T, 32, BN, BK, 4>), dim3(static_cast<unsigned>(gx), 1), dim3(256), 0,
                            ctx->stream, g);
@@ -243,6 +289,51 @@ __global__ __launch_bounds__(256) void maxpool_kernel(T *res, const T *data, siz
     }
 }
 
+// Non-overlapping 2x2 windows (stride 2, no padding, even H and W): the tensor is a flat list of row
+// pairs [R][2][W] -> [R][W/2]. Each thread loads VI consecutive values of both rows of a pair and
+// writes VI/2 outputs, all as single vector accesses.
+template <typename T, int VI>
+__global__ __launch_bounds__(256) void maxpool2x2_kernel(T *res, const T *data, size_t items, unsigned W,
+                                                         unsigned wvecs) {
+    const size_t item = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (item >= items)
+        return;
+    size_t r;
+    unsigned j;
+    if (items <= 0xffffffffull) {
+        r = static_cast<unsigned>(item) / wvecs;
+        j = static_cast<unsigned>(item) % wvecs;
+    } else {
+        r = item / wvecs;
+        j = static_cast<unsigned>(item % wvecs);
+    }
+    const T *in = data + r * 2 * W + static_cast<size_t>(j) * VI;
+    T a[VI], b[VI], o[VI / 2];
+    dh_load_vec_stream<T, VI>(in, a);
+    dh_load_vec_stream<T, VI>(in + W, b);
+#pragma unroll
+    for (int i = 0; i < VI / 2; i++) {
+        // window order of Pooling.cpp:77-105 with the accumulator starting at zero
+        T m = T(0);
+        m = (m < a[2 * i]) ? a[2 * i] : m;
+        m = (m < a[2 * i + 1]) ? a[2 * i + 1] : m;
+        m = (m < b[2 * i]) ? b[2 * i] : m;
+        m = (m < b[2 * i + 1]) ? b[2 * i + 1] : m;
+        o[i] = m;
+    }
+    T *out = res + r * (W / 2) + static_cast<size_t>(j) * (VI / 2);
+    if constexpr (VI / 2 == 1) {
+        *out = o[0];
+    } else {
+        typedef T half_vec __attribute__((ext_vector_type(VI / 2)));
+        half_vec t;
+#pragma unroll
+        for (int i = 0; i < VI / 2; i++)
+            t[i] = o[i];
+        *reinterpret_cast<half_vec *>(out) = t;
+    }
+}
+
 template <typename T> __global__ __launch_bounds__(256) void fill_kernel(T *p, size_t n, T v) {
     for (size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x; i < n; i += static_cast<size_t>(gridDim.x) * 256)
         p[i] = v;
@@ -270,7 +361,13 @@ dh_status maxpool_forward(dh_ctx *ctx, T *res, size_t *res_h, size_t *res_w, con
     const size_t cap = static_cast<size_t>(ctx->num_cus) * 32;
     if (grid > cap)
         grid = cap;
-    if (P == 1 && Q == 1 && W == 1) {
+    constexpr int VI = 16 / sizeof(T);
+    if (ph == 2 && pw == 2 && sh == 2 && sw == 2 && padh == 0 && padw == 0 && H % 2 == 0 && W % VI == 0 &&
+        dh_aligned(data, 16) && dh_aligned(res, 8) && total * 2 / VI < (size_t(1) << 39)) {
+        const size_t items = N * C * P * (W / VI);
+        hipLaunchKernelGGL((maxpool2x2_kernel<T, VI>), dim3(static_cast<unsigned>(dh_ceil_div(items, 256))), dim3(256), 0,
+                           ctx->stream, res, data, items, static_cast<unsigned>(W), static_cast<unsigned>(W / VI));
+    } else if (P == 1 && Q == 1 && W == 1) {
         // Pooling.cpp:57-66: this quick path folds the window into numeric_limits::max(), so that
         // value is what the CPU kernel returns for every output.
         hipLaunchKernelGGL((fill_kernel<T>), dim3(static_cast<unsigned>(grid)), dim3(256), 0, ctx->stream, res, total,

@@ -53,6 +53,12 @@ class HIPContext:
     def memInUse(self) -> int:
         return capi.lib().dh_ctx_mem_in_use(self._h)
 
+    def memCached(self) -> int:
+        return capi.lib().dh_ctx_mem_cached(self._h)
+
+    def releaseCached(self) -> None:
+        capi.check(capi.lib().dh_ctx_release_cached(self._h))
+
     def props(self) -> dict:
         cus, khz, total = C.c_int(), C.c_int(), C.c_size_t()
         name = C.create_string_buffer(256)

@@ -97,9 +97,17 @@ void *dh_ctx_get_stream(const dh_ctx *ctx);
 dh_status dh_sync(dh_ctx *ctx);
 
 /* CUDAContext::malloc(size, zero, id) / free(id) (CUDAContext.cpp:120-135). The device
- * pointer itself is the registry key. Fails with DH_ERR_OOM past the budget. */
+ * pointer itself is the registry key. Fails with DH_ERR_OOM past the budget.
+ * Unlike cudaMalloc/cudaFree there, freed blocks are kept by the context and handed out again to
+ * later requests of the same size class, without a device synchronisation: reuse is ordered by the
+ * context's stream, so a caller that used a buffer on another stream waits for that work before
+ * dh_free. Cached blocks are returned to the driver when the budget or the device runs short, by
+ * dh_ctx_release_cached, and by dh_ctx_destroy. */
 dh_status dh_malloc(dh_ctx *ctx, size_t bytes, int zero, void **out);
 dh_status dh_free(dh_ctx *ctx, void *ptr);
+/* Bytes held in freed blocks awaiting reuse / give them back to the driver (synchronises). */
+size_t dh_ctx_mem_cached(const dh_ctx *ctx);
+dh_status dh_ctx_release_cached(dh_ctx *ctx);
 /* AllocationDescriptorCUDA::transferTo / transferFrom
  * (runtime/local/datastructures/AllocationDescriptorCUDA.h:56-68): synchronous copies. */
 dh_status dh_h2d(dh_ctx *ctx, void *dst_dev, const void *src_host, size_t bytes);
