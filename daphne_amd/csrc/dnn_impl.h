@@ -10,9 +10,11 @@
 // Conv2D as a GEMM without materialising im2col:
 //     out_n[f][pixel] = sum_k W[f][k] * patch[k][pixel],   k = (c, h, w), pixel = (n, p, q)
 // The filter matrix (F x K, K contiguous) is the row operand; the patch matrix is never built:
-// each workgroup gathers its BK x BN slice straight from the NCHW input into LDS (zero outside
-// the image), with consecutive lanes on consecutive output pixels so that both the gather and
-// the final store are contiguous along q. Pixels of all images form one long N dimension, so a
+// each workgroup gathers its BK x BN slice from the NCHW input into LDS, with consecutive lanes
+// on consecutive output pixels so that both the gather and the final store are contiguous along q.
+// When the convolution has a border, the input is first copied into a workspace with the zeros
+// written out: the gather then needs no bounds checks, and with a table k -> offset no divisions,
+// which leaves one scalar add and one load per gathered element. Pixels of all images form one long N dimension, so a
 // tile may span image boundaries and small images still fill the 128-pixel tile.
 #pragma once
 
@@ -27,30 +29,58 @@ using dh_gemm::TileLayout;
 using dh_gemm::TileMover;
 
 struct ConvArgs {
-    const void *data, *filter, *bias;
+    const void *xpad;    // input with the zero border materialised: N x C x Hp x Wp
+    const void *wpack;   // filter matrix padded with zeros to Fpad x Kpad
+    const int *ktab;     // k = (c, hy, hx) -> c*Hp*Wp + hy*Wp + hx, Kpad entries (zero beyond K)
+    const void *bias;
     void *res;
-    unsigned N, C, H, W, F, Hf, Wf, sh, sw, ph, pw, P, Q;
-    unsigned K;          // C*Hf*Wf
-    int aligned_w;       // filter rows can be read with 16-byte loads
+    unsigned F, K, Kpad, P, Q, sh, sw, Wp;
+    unsigned CHpWp;      // elements of one padded image
     size_t pixels;       // N*P*Q
-    const int *ktab;     // per k (padded to a multiple of the K tile): offset of (c, hy, hx) in an image,
-                         // then hy << 16 | hx; entries beyond K are zero
 };
 
-// k = (c, hy, hx) -> { c*H*W + hy*W + hx, hy << 16 | hx }, so that the gather does no divisions.
-static __global__ void conv_table_kernel(int *tab, unsigned K, unsigned Kpad, unsigned HW, unsigned W, unsigned Hf,
-                                         unsigned Wf) {
-    for (unsigned k = blockIdx.x * blockDim.x + threadIdx.x; k < Kpad; k += gridDim.x * blockDim.x) {
-        int off = 0, yx = 0;
+// Table of patch offsets and the zero-padded filter matrix, so that the main loop has neither divisions
+// nor bounds checks on the filter side.
+template <typename T>
+__global__ __launch_bounds__(256) void conv_prep_kernel(int *tab, T *wpack, const T *filter, unsigned F, unsigned Fpad,
+                                                        unsigned K, unsigned Kpad, unsigned HpWp, unsigned Wp,
+                                                        unsigned Hf, unsigned Wf) {
+    const unsigned t = blockIdx.x * 256 + threadIdx.x, nt = gridDim.x * 256;
+    for (unsigned k = t; k < Kpad; k += nt) {
+        int off = 0;
         if (k < K) {
             const unsigned c = k / (Hf * Wf), hw = k % (Hf * Wf);
-            const unsigned hy = hw / Wf, hx = hw % Wf;
-            off = static_cast<int>(c * HW + hy * W + hx);
-            yx = static_cast<int>(hy << 16 | hx);
+            off = static_cast<int>(c * HpWp + (hw / Wf) * Wp + hw % Wf);
         }
         tab[k] = off;
-        tab[Kpad + k] = yx;
     }
+    const size_t total = static_cast<size_t>(Fpad) * Kpad;
+    for (size_t i = t; i < total; i += nt) {
+        const unsigned f = static_cast<unsigned>(i / Kpad), k = static_cast<unsigned>(i % Kpad);
+        wpack[i] = (f < F && k < K) ? filter[static_cast<size_t>(f) * K + k] : T(0);
+    }
+}
+
+// Copies the images into a buffer with the zero border of Padding.h:11-22 written out, one thread per
+// padded element (consecutive threads along a padded row).
+template <typename T>
+__global__ __launch_bounds__(256) void conv_pad_kernel(T *xpad, const T *x, size_t total, unsigned H, unsigned W,
+                                                       unsigned Hp, unsigned Wp, unsigned ph, unsigned pw) {
+    const size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (i >= total)
+        return;
+    size_t plane;
+    unsigned r;
+    const unsigned HpWp = Hp * Wp;
+    if (total <= 0xffffffffull) {
+        plane = static_cast<unsigned>(i) / HpWp;
+        r = static_cast<unsigned>(i) % HpWp;
+    } else {
+        plane = i / HpWp;
+        r = static_cast<unsigned>(i % HpWp);
+    }
+    const unsigned y = r / Wp - ph, x_ = r % Wp - pw; // wraps to a huge value inside the border
+    xpad[i] = (y < H && x_ < W) ? x[plane * H * W + static_cast<size_t>(y) * W + x_] : T(0);
 }
 
 template <typename T, int BM, int BN, int BK, int WN>
@@ -60,65 +90,87 @@ __global__ __launch_bounds__(64 * WN) void conv2d_kernel(ConvArgs g) {
     constexpr int TN = BN / WN;
     constexpr int FM = BM / M::MT, FN = TN / M::NT;
     static_assert(BM % M::MT == 0 && TN % M::NT == 0 && BK % M::KT == 0, "tile shape");
-    static_assert(THREADS % BN == 0 && BK % (THREADS / BN) == 0, "gather mapping");
+    static_assert(THREADS % BN == 0 && BK % (THREADS / BN) == 0 && BN % 64 == 0, "gather mapping");
+    constexpr int VEC = 16 / sizeof(T);
+    constexpr int KPL = BK / (64 / M::ROWS); // k values per lane and tile
+    static_assert(KPL % VEC == 0, "fragment reads are whole 16-byte vectors");
     using LA = TileLayout<T, BM, BK, true>;  // filter tile [f][k]
     using LB = TileLayout<T, BN, BK, false>; // patch tile  [k][pixel]
     __shared__ __attribute__((aligned(16))) T lds_a[2][LA::ELEMS];
     __shared__ __attribute__((aligned(16))) T lds_b[2][LB::ELEMS];
 
-    const T *X = static_cast<const T *>(g.data);
-    const T *Wt = static_cast<const T *>(g.filter);
     const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
     const size_t pix0 = static_cast<size_t>(blockIdx.x) * BN;
-    const size_t f0 = static_cast<size_t>(blockIdx.y) * BM;
-    const unsigned PQ = g.P * g.Q, HW = g.H * g.W;
-
-    // the pixel this thread gathers for, decoded once
-    constexpr int KG = THREADS / BN;      // K groups among the threads
-    constexpr int KPT = BK / KG;          // K values per thread and tile
-    const int gj = tid % BN, gkg = tid / BN;
-    const size_t gpix = pix0 + gj;
-    const bool pix_ok = gpix < g.pixels;
+    const unsigned f0 = blockIdx.y * BM;
+    const unsigned PQ = g.P * g.Q;
     const bool small = g.pixels <= 0xffffffffull; // 32-bit divisions suffice (uniform)
-    unsigned img = 0, p = 0, q = 0;
-    if (pix_ok) {
-        unsigned pq;
-        if (small) {
-            img = static_cast<unsigned>(gpix) / PQ;
-            pq = static_cast<unsigned>(gpix) % PQ;
-        } else {
-            img = static_cast<unsigned>(gpix / PQ);
-            pq = static_cast<unsigned>(gpix % PQ);
-        }
-        p = pq / g.Q;
-        q = pq % g.Q;
-    }
-    const int y0 = static_cast<int>(p * g.sh) - static_cast<int>(g.ph);
-    // a pixel beyond the end gets a row origin that fails every bounds check
-    const int x0 = pix_ok ? static_cast<int>(q * g.sw) - static_cast<int>(g.pw) : -0x10000000;
-    const T *xpix = X + static_cast<size_t>(img) * g.C * HW + static_cast<ptrdiff_t>(y0) * static_cast<int>(g.W) + x0;
-    const unsigned Kpad = (g.K + BK - 1) / BK * BK;
-    const int *tab_off = g.ktab + gkg * KPT, *tab_yx = g.ktab + Kpad + gkg * KPT;
 
-    TileMover<T, BM, BK, true, THREADS> mv_a;
-    T gb[KPT];
+    // Gather mapping: thread -> one pixel of the tile and a group of KPT consecutive k. The k group is the
+    // same for a whole wave (BN is a multiple of 64) and kept in a scalar register, so the table entries
+    // come by scalar loads and every gather load is "uniform base + per-lane 32-bit offset".
+    constexpr int KG = THREADS / BN;
+    constexpr int KPT = BK / KG;
+    const int gj = tid % BN, gkg = __builtin_amdgcn_readfirstlane(tid / BN);
+    // pixels past the end repeat the last one; their results are dropped by the epilogue
+    const size_t gpix = pix0 + gj < g.pixels ? pix0 + gj : g.pixels - 1;
+    size_t img0;
+    unsigned img, pq;
+    if (small) {
+        img0 = static_cast<unsigned>(pix0) / PQ;
+        img = static_cast<unsigned>(gpix) / PQ;
+        pq = static_cast<unsigned>(gpix) % PQ;
+    } else {
+        img0 = pix0 / PQ;
+        img = static_cast<unsigned>(gpix / PQ);
+        pq = static_cast<unsigned>(gpix % PQ);
+    }
+    const unsigned p = pq / g.Q, q = pq % g.Q;
+    const char *xblk = reinterpret_cast<const char *>(static_cast<const T *>(g.xpad) + img0 * g.CHpWp);
+    // byte offset of this pixel's window origin from the block's first image (the host checks the range)
+    const unsigned voff = static_cast<unsigned>(((img - static_cast<unsigned>(img0)) * g.CHpWp + p * g.sh * g.Wp + q * g.sw) *
+                                                sizeof(T));
+    const int *tab = g.ktab + gkg * KPT;
+
+    // filter tile: whole 16-byte vectors of the padded matrix
+    constexpr int VPR = BK / VEC, NVEC = BM * VPR, APT = (NVEC + THREADS - 1) / THREADS;
+    const T *wrow[APT];
+    int a_lds[APT];
+#pragma unroll
+    for (int i = 0; i < APT; i++) {
+        const int v = tid + i * THREADS;
+        const int o = (v / VPR) % BM, iv = v % VPR;
+        wrow[i] = static_cast<const T *>(g.wpack) + static_cast<size_t>(f0 + o) * g.Kpad + iv * VEC;
+        a_lds[i] = LA::at(o, iv * VEC);
+    }
+
+    T ga[APT][VEC], gb[KPT];
     auto fetch = [&](unsigned k0) {
-        mv_a.load(Wt, g.K, f0, k0, g.F, g.K, g.aligned_w != 0, tid);
-        int off[KPT], yx[KPT];
 #pragma unroll
-        for (int i = 0; i < KPT; i++) {
-            off[i] = tab_off[k0 + i];
-            yx[i] = tab_yx[k0 + i];
-        }
+        for (int i = 0; i < APT; i++)
+            if ((NVEC % THREADS == 0) || (tid + i * THREADS < NVEC))
+                dh_load_vec<T, VEC>(wrow[i] + k0, ga[i]);
+        int off[KPT];
 #pragma unroll
-        for (int i = 0; i < KPT; i++) {
-            // unsigned compares fold the lower bound in: a negative coordinate wraps to a huge value
-            const unsigned y = static_cast<unsigned>(y0 + (yx[i] >> 16)), x = static_cast<unsigned>(x0 + (yx[i] & 0xffff));
-            gb[i] = (y < g.H && x < g.W && k0 + gkg * KPT + i < g.K) ? xpix[off[i]] : T(0);
+        for (int i = 0; i < KPT; i++)
+            off[i] = tab[k0 + i];
+        if (k0 + BK <= g.K) {
+#pragma unroll
+            for (int i = 0; i < KPT; i++)
+                gb[i] = *reinterpret_cast<const T *>(xblk + static_cast<ptrdiff_t>(off[i]) * static_cast<ptrdiff_t>(sizeof(T)) + voff);
+        } else {
+            // last tile: k beyond K contributes nothing, whatever the image holds there
+#pragma unroll
+            for (int i = 0; i < KPT; i++) {
+                const T v = *reinterpret_cast<const T *>(xblk + static_cast<ptrdiff_t>(off[i]) * static_cast<ptrdiff_t>(sizeof(T)) + voff);
+                gb[i] = (k0 + gkg * KPT + i < g.K) ? v : T(0);
+            }
         }
     };
     auto stash = [&](int buf) {
-        mv_a.store(lds_a[buf], tid);
+#pragma unroll
+        for (int i = 0; i < APT; i++)
+            if ((NVEC % THREADS == 0) || (tid + i * THREADS < NVEC))
+                dh_store_vec<T, VEC>(lds_a[buf] + a_lds[i], ga[i]);
 #pragma unroll
         for (int i = 0; i < KPT; i++)
             lds_b[buf][LB::at(gj, gkg * KPT + i)] = gb[i];
@@ -142,21 +194,32 @@ __global__ __launch_bounds__(64 * WN) void conv2d_kernel(ConvArgs g) {
             fetch(k0 + BK);
         const T *la = lds_a[buf];
         const T *lb = lds_b[buf];
+        // The k index an MFMA step assigns to a lane group is free as long as both operands agree:
+        // lane group h takes the KPL consecutive values k = h*KPL .. h*KPL+KPL-1 of the tile, one per
+        // step, so the filter fragment (contiguous along k in LDS) is read with 16-byte loads.
+        T fa[FM][KPL], fb[FN][KPL];
 #pragma unroll
-        for (int kk = 0; kk < BK; kk += M::KT) {
-            T fa[FM], fb[FN];
+        for (int i = 0; i < FM; i++)
 #pragma unroll
-            for (int i = 0; i < FM; i++)
-                fa[i] = la[LA::at(i * M::MT + frag_row, kk + frag_k)];
+            for (int v = 0; v < KPL; v += VEC) {
+                T t[VEC];
+                dh_load_vec<T, VEC>(la + LA::at(i * M::MT + frag_row, frag_k * KPL + v), t);
 #pragma unroll
-            for (int j = 0; j < FN; j++)
-                fb[j] = lb[LB::at(wave * TN + j * M::NT + frag_row, kk + frag_k)];
+                for (int e = 0; e < VEC; e++)
+                    fa[i][v + e] = t[e];
+            }
+#pragma unroll
+        for (int j = 0; j < FN; j++)
+#pragma unroll
+            for (int s_ = 0; s_ < KPL; s_++)
+                fb[j][s_] = lb[LB::at(wave * TN + j * M::NT + frag_row, frag_k * KPL + s_)];
+#pragma unroll
+        for (int s_ = 0; s_ < KPL; s_++)
 #pragma unroll
             for (int i = 0; i < FM; i++)
 #pragma unroll
                 for (int j = 0; j < FN; j++)
-                    acc[i][j] = M::mma(fa[i], fb[j], acc[i][j]);
-        }
+                    acc[i][j] = M::mma(fa[i][s_], fb[j][s_], acc[i][j]);
         if (more)
             stash(buf ^ 1);
         __syncthreads();
@@ -213,43 +276,74 @@ dh_status conv2d_forward(dh_ctx *ctx, T *res, size_t *res_h, size_t *res_w, cons
     const size_t pixels = N * P * Q;
     if (pixels == 0 || F == 0)
         return DH_OK;
-    if (C * H * W >= (size_t(1) << 31) || C * Hf * Wf >= (size_t(1) << 31) || P * Q >= (size_t(1) << 31) ||
-        N >= (size_t(1) << 31))
-        return dh_fail(DH_ERR_RUNTIME, "Convolution: image or filter extents exceed 2^31 elements");
-    ConvArgs g{};
-    g.data = data;
-    g.filter = filter;
-    g.bias = bias;
-    g.res = res;
-    g.N = N; g.C = C; g.H = H; g.W = W; g.F = F; g.Hf = Hf; g.Wf = Wf;
-    g.sh = sh; g.sw = sw; g.ph = ph; g.pw = pw; g.P = P; g.Q = Q;
-    g.K = static_cast<unsigned>(C * Hf * Wf);
-    g.pixels = pixels;
-    g.aligned_w = dh_aligned(filter, 16) && (g.K % (16 / sizeof(T)) == 0);
     constexpr int BK = dh_gemm::GemmBK<T>::value;
     constexpr int BN = 128;
+    const size_t Hp = H + 2 * ph, Wp = W + 2 * pw, K = C * Hf * Wf;
+    // a workgroup addresses its pixels with 32-bit byte offsets from its first image
+    const size_t images_per_tile = (BN + P * Q - 2) / (P * Q) + 1;
+    if (C * Hp * Wp * images_per_tile * sizeof(T) >= (size_t(1) << 32) || K >= (size_t(1) << 31) ||
+        P * Q >= (size_t(1) << 31) || N >= (size_t(1) << 31) || F >= (size_t(1) << 31))
+        return dh_fail(DH_ERR_RUNTIME, "Convolution: image or filter extents exceed the 32-bit addressing of a tile");
     const size_t gx = dh_ceil_div(pixels, BN);
     if (gx >= (size_t(1) << 31))
         return dh_fail(DH_ERR_RUNTIME, "Convolution: too many output pixels for one launch");
-    if (Hf >= 0x8000 || Wf >= 0x10000 || H >= (size_t(1) << 28) || W >= (size_t(1) << 28))
-        return dh_fail(DH_ERR_RUNTIME, "Convolution: filter or image side too large");
-    const unsigned Kpad = static_cast<unsigned>(dh_ceil_div(g.K, BK) * BK);
+    const int BM = F <= 32 ? 32 : 64;
+    const unsigned gy = static_cast<unsigned>(dh_ceil_div(F, BM));
+    const size_t Kpad = dh_ceil_div(K, BK) * BK, Fpad = static_cast<size_t>(gy) * BM;
+    const bool padded = ph != 0 || pw != 0;
+
+    // workspace: offset table | packed filter | padded images
+    const size_t tab_bytes = dh_ceil_div(Kpad * sizeof(int), 256) * 256;
+    const size_t w_bytes = dh_ceil_div(Fpad * Kpad * sizeof(T), 256) * 256;
+    const size_t x_elems = padded ? N * C * Hp * Wp : 0;
     void *wsv = nullptr;
-    dh_status st = dh_workspace(ctx, 2 * static_cast<size_t>(Kpad) * sizeof(int), &wsv);
+    dh_status st = dh_workspace(ctx, tab_bytes + w_bytes + x_elems * sizeof(T), &wsv);
     if (st != DH_OK)
         return st;
-    g.ktab = static_cast<const int *>(wsv);
-    hipLaunchKernelGGL(conv_table_kernel, dim3(static_cast<unsigned>(dh_ceil_div(Kpad, 256) > 64 ? 64 : dh_ceil_div(Kpad, 256))),
-                       dim3(256), 0, ctx->stream, static_cast<int *>(wsv), g.K, Kpad, static_cast<unsigned>(H * W),
-                       static_cast<unsigned>(W), static_cast<unsigned>(Hf), static_cast<unsigned>(Wf));
-    if (F <= 32) {
-        hipLaunchKernelGGL((conv2d_kernel<T, 32, BN, BK, 4>), dim3(static_cast<unsigned>(gx), 1), dim3(256), 0,
+    char *ws = static_cast<char *>(wsv);
+    int *tab = reinterpret_cast<int *>(ws);
+    T *wpack = reinterpret_cast<T *>(ws + tab_bytes);
+    T *xpad = reinterpret_cast<T *>(ws + tab_bytes + w_bytes);
+    size_t pg = dh_ceil_div(Fpad * Kpad, 256);
+    if (pg > 1024)
+        pg = 1024;
+    hipLaunchKernelGGL((conv_prep_kernel<T>), dim3(static_cast<unsigned>(pg)), dim3(256), 0, ctx->stream, tab, wpack, filter,
+                       static_cast<unsigned>(F), static_cast<unsigned>(Fpad), static_cast<unsigned>(K),
+                       static_cast<unsigned>(Kpad), static_cast<unsigned>(Hp * Wp), static_cast<unsigned>(Wp),
+                       static_cast<unsigned>(Hf), static_cast<unsigned>(Wf));
+    DH_CHECK_LAUNCH();
+    if (padded) {
+        const size_t blocks = dh_ceil_div(x_elems, 256);
+        if (blocks >= (size_t(1) << 31))
+            return dh_fail(DH_ERR_RUNTIME, "Convolution: input too large for one launch");
+        hipLaunchKernelGGL((conv_pad_kernel<T>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0, ctx->stream, xpad, data,
+                           x_elems, static_cast<unsigned>(H), static_cast<unsigned>(W), static_cast<unsigned>(Hp),
+                           static_cast<unsigned>(Wp), static_cast<unsigned>(ph), static_cast<unsigned>(pw));
+        DH_CHECK_LAUNCH();
+    }
+
+    ConvArgs g{};
+    g.xpad = padded ? xpad : data;
+    g.wpack = wpack;
+    g.ktab = tab;
+    g.bias = bias;
+    g.res = res;
+    g.F = static_cast<unsigned>(F);
+    g.K = static_cast<unsigned>(K);
+    g.Kpad = static_cast<unsigned>(Kpad);
+    g.P = static_cast<unsigned>(P);
+    g.Q = static_cast<unsigned>(Q);
+    g.sh = static_cast<unsigned>(sh);
+    g.sw = static_cast<unsigned>(sw);
+    g.Wp = static_cast<unsigned>(Wp);
+    g.CHpWp = static_cast<unsigned>(C * Hp * Wp);
+    g.pixels = pixels;
+    if (BM == 32)
+        hipLaunchKernelGGL((conv2d_kernel<T, 32, BN, BK, 4>), dim3(static_cast<unsigned>(gx), gy), dim3(256), 0,
                            ctx->stream, g);
-    } else {
-        const unsigned gy = static_cast<unsigned>(dh_ceil_div(F, 64));
+    else
         hipLaunchKernelGGL((conv2d_kernel<T, 64, BN, BK, 4>), dim3(static_cast<unsigned>(gx), gy), dim3(256), 0,
                            ctx->stream, g);
-    }
     DH_CHECK_LAUNCH();
     return DH_OK;
 }
