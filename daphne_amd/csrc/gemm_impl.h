@@ -397,6 +397,12 @@ __global__ __launch_bounds__(256) void gemv_t_stage2(const T *partials, size_t n
     y[c * incy] = s;
 }
 
+} // namespace dh_gemm
+
+#include "ts_impl.h"
+
+namespace dh_gemm {
+
 // ---------------------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------------------
@@ -426,6 +432,20 @@ dh_status gemm(dh_ctx *ctx, bool ta, bool tb, size_t m, size_t n, size_t k, cons
                size_t ldb, T *C, size_t ldc, const T *bias, bool triangular, size_t bias_stride = 1) {
     if (m == 0 || n == 0)
         return DH_OK;
+    // tall-and-skinny shapes stream straight from HBM into the matrix cores
+    if (bias == nullptr) {
+        dh_status st = DH_OK;
+        if (ta && !tb && ts_tn<T>(ctx, m, n, k, A, lda, B, ldb, C, ldc, &st)) {
+            if (st == DH_OK)
+                DH_CHECK_LAUNCH();
+            return st;
+        }
+        if (!ta && tb && !triangular && ts_nt<T>(ctx, m, n, k, A, lda, B, ldb, C, ldc, &st)) {
+            if (st == DH_OK)
+                DH_CHECK_LAUNCH();
+            return st;
+        }
+    }
     constexpr int V = 16 / sizeof(T);
     GemmArgs g{};
     g.A = A;
@@ -554,6 +574,15 @@ dh_status gemv(dh_ctx *ctx, bool trans, size_t rows, size_t cols, const T *A, si
     }
     if (cols == 0)
         return DH_OK;
+    {
+        // y = t(A) x as a one-column case of the streaming contraction
+        dh_status st = DH_OK;
+        if (ts_tn<T>(ctx, cols, 1, rows, A, lda, x, incx, y, incy, &st)) {
+            if (st == DH_OK)
+                DH_CHECK_LAUNCH();
+            return st;
+        }
+    }
     unsigned tx = 1;
     while (tx < 256 && tx < cols)
         tx <<= 1;

@@ -1,0 +1,479 @@
+// Streaming contractions for tall-and-skinny operands, the shapes of the reference's ML scripts
+// (t(X) %*% X, t(X) %*% y, t(P) %*% X, X %*% t(C) with X of millions of rows and tens of columns).
+// They are bound by HBM, not by the matrix cores, so nothing is staged through LDS: every
+// wavefront loads its operands from global memory directly in MFMA fragment layout and keeps going
+// without barriers.
+//
+// Both use the 16x16x4 matrix instruction (v_mfma_f32_16x16x4_f32 / v_mfma_f64_16x16x4_f64):
+// lane l supplies A[i = l%16][k = l/16] and B[k = l/16][j = l%16]. Which row of C a lane's "i"
+// stands for, and which k its "k" stands for, is free as long as both operands agree - that is what
+// lets a lane use whole 16-byte vectors:
+//
+//   ts_tn:  C[m x n] = t(A) B,  A: K x m, B: K x n, K huge, m, n <= 128.
+//           The four lane groups take four consecutive rows k; a lane loads a vector of V consecutive
+//           columns of that row, and element e of the vector feeds MFMA number e, which therefore
+//           computes the C rows {V*i + e}. A wave load covers whole contiguous rows. The K range is
+//           cut over workgroups (and over the waves of a workgroup when the output is small); each
+//           workgroup writes one partial slab, and a second kernel adds the slabs in a fixed order.
+//   ts_nt:  C[M x n] = A t(B),  A: M x K, B: n x K, M huge, n <= 32, K small.
+//           Lane group h takes the k values [c*4V + h*V, +V) of chunk c: one vector load per lane and
+//           chunk, V MFMAs. B sits in LDS (a few KB, loaded once per workgroup).
+#pragma once
+
+#include "common.h"
+
+namespace dh_gemm {
+
+typedef float ts_f32x4 __attribute__((ext_vector_type(4)));
+typedef double ts_f64x4 __attribute__((ext_vector_type(4)));
+
+template <typename T> struct Mfma16;
+template <> struct Mfma16<float> {
+    using acc_t = ts_f32x4;
+    static __device__ __forceinline__ acc_t mma(float a, float b, acc_t c) {
+        return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
+    }
+    // accumulator register v of lane l holds C[row(l, v)][l % 16]
+    static __device__ __forceinline__ int row(int lane, int v) { return 4 * (lane / 16) + v; }
+};
+template <> struct Mfma16<double> {
+    using acc_t = ts_f64x4;
+    static __device__ __forceinline__ acc_t mma(double a, double b, acc_t c) {
+        return __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ int row(int lane, int v) { return 4 * v + (lane / 16); }
+};
+
+// V consecutive values; `stream` marks data that no other wave will ask for again
+template <typename T, int V> __device__ __forceinline__ void ts_load(const T *p, T (&v)[V], bool stream) {
+    if constexpr (V == 1) {
+        v[0] = stream ? __builtin_nontemporal_load(p) : *p;
+    } else {
+        typedef T vec_t __attribute__((ext_vector_type(V)));
+        const vec_t t = stream ? __builtin_nontemporal_load(reinterpret_cast<const vec_t *>(p))
+                               : *reinterpret_cast<const vec_t *>(p);
+#pragma unroll
+        for (int e = 0; e < V; e++)
+            v[e] = t[e];
+    }
+}
+
+struct TsTnArgs {
+    const void *A, *B;
+    void *slabs;       // [gridDim.x][m][n]
+    size_t lda, ldb, K;
+    size_t k_chunk;    // rows per workgroup, a multiple of 4 * waves-along-K * unroll
+    unsigned m, n;
+    int stream;        // operands are read once (no reuse between waves or operands)
+};
+
+// Wave tile: TM = 16*VA*RA rows by TN = 16*VB*RB columns of C; WM x WN wave tiles per workgroup,
+// the remaining 4/(WM*WN) waves split K.
+template <typename T, int VA, int RA, int VB, int RB, int WM, int WN>
+__global__ __launch_bounds__(256) void ts_tn_kernel(TsTnArgs g) {
+    using M = Mfma16<T>;
+    constexpr int KW = 4 / (WM * WN);
+    constexpr int TM = 16 * VA * RA, TN = 16 * VB * RB;
+    constexpr int NACC = RA * VA * RB * VB;         // MFMA tiles per wave
+    constexpr int U = NACC >= 16 ? 2 : 4;           // quads (4 rows of K) in flight per wave
+    const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
+    const int wm = wave % WM, wn = (wave / WM) % WN, wk = wave / (WM * WN);
+    const int i = lane % 16, h = lane / 16;
+    const T *A = static_cast<const T *>(g.A);
+    const T *B = static_cast<const T *>(g.B);
+    const bool stream = g.stream != 0;
+
+    // first column of each vector this lane loads; vectors that start beyond the matrix are skipped
+    unsigned ca[RA], cb[RB];
+    bool oka[RA], okb[RB];
+#pragma unroll
+    for (int a = 0; a < RA; a++) {
+        ca[a] = wm * TM + a * 16 * VA + i * VA;
+        oka[a] = ca[a] < g.m;
+    }
+#pragma unroll
+    for (int b = 0; b < RB; b++) {
+        cb[b] = wn * TN + b * 16 * VB + i * VB;
+        okb[b] = cb[b] < g.n;
+    }
+
+    typename M::acc_t acc[RA][VA][RB][VB];
+#pragma unroll
+    for (int a = 0; a < RA; a++)
+#pragma unroll
+        for (int e = 0; e < VA; e++)
+#pragma unroll
+            for (int b = 0; b < RB; b++)
+#pragma unroll
+                for (int f = 0; f < VB; f++)
+                    acc[a][e][b][f] = typename M::acc_t{0, 0, 0, 0};
+
+    const size_t kb = static_cast<size_t>(blockIdx.x) * g.k_chunk;
+    const size_t ke = kb + g.k_chunk < g.K ? kb + g.k_chunk : g.K;
+
+    T fa[U][RA][VA], fb[U][RB][VB];
+    auto load_quad = [&](int u, size_t k, bool guard) {
+        const bool row_ok = !guard || k < ke;
+#pragma unroll
+        for (int a = 0; a < RA; a++) {
+            if (oka[a] && row_ok) {
+                ts_load<T, VA>(A + k * g.lda + ca[a], fa[u][a], stream);
+            } else {
+#pragma unroll
+                for (int e = 0; e < VA; e++)
+                    fa[u][a][e] = T(0);
+            }
+        }
+#pragma unroll
+        for (int b = 0; b < RB; b++) {
+            if (okb[b] && row_ok) {
+                ts_load<T, VB>(B + k * g.ldb + cb[b], fb[u][b], stream);
+            } else {
+#pragma unroll
+                for (int f = 0; f < VB; f++)
+                    fb[u][b][f] = T(0);
+            }
+        }
+    };
+    auto mma_quad = [&](int u) {
+#pragma unroll
+        for (int a = 0; a < RA; a++)
+#pragma unroll
+            for (int e = 0; e < VA; e++)
+#pragma unroll
+                for (int b = 0; b < RB; b++)
+#pragma unroll
+                    for (int f = 0; f < VB; f++)
+                        acc[a][e][b][f] = M::mma(fa[u][a][e], fb[u][b][f], acc[a][e][b][f]);
+    };
+
+    // quad q of this wave covers rows kb + (q*KW + wk)*4 .. +3; lane group h takes row +h
+    size_t k = kb + static_cast<size_t>(wk) * 4 + h;
+    constexpr size_t STEP = static_cast<size_t>(KW) * 4;
+    // full groups of U quads: every row of the last quad is inside the chunk
+    while (k - h + (U - 1) * STEP + 4 <= ke) {
+#pragma unroll
+        for (int u = 0; u < U; u++)
+            load_quad(u, k + u * STEP, false);
+#pragma unroll
+        for (int u = 0; u < U; u++)
+            mma_quad(u);
+        k += U * STEP;
+    }
+    while (k - h < ke) {
+        load_quad(0, k, true);
+        mma_quad(0);
+        k += STEP;
+    }
+
+    // add up the waves that split K: wave 0 of each tile collects the others one at a time (fixed order)
+    if constexpr (KW > 1) {
+        __shared__ __attribute__((aligned(16))) T red[WM * WN][NACC * 4][64];
+        const int tile = wave % (WM * WN);
+        for (int w = 1; w < KW; w++) {
+            if (wk == w) {
+                int r = 0;
+#pragma unroll
+                for (int a = 0; a < RA; a++)
+#pragma unroll
+                    for (int e = 0; e < VA; e++)
+#pragma unroll
+                        for (int b = 0; b < RB; b++)
+#pragma unroll
+                            for (int f = 0; f < VB; f++)
+#pragma unroll
+                                for (int v = 0; v < 4; v++)
+                                    red[tile][r++][lane] = acc[a][e][b][f][v];
+            }
+            __syncthreads();
+            if (wk == 0) {
+                int r = 0;
+#pragma unroll
+                for (int a = 0; a < RA; a++)
+#pragma unroll
+                    for (int e = 0; e < VA; e++)
+#pragma unroll
+                        for (int b = 0; b < RB; b++)
+#pragma unroll
+                            for (int f = 0; f < VB; f++)
+#pragma unroll
+                                for (int v = 0; v < 4; v++)
+                                    acc[a][e][b][f][v] += red[tile][r++][lane];
+            }
+            __syncthreads();
+        }
+    }
+    if (wk != 0)
+        return;
+
+    // slab[row][col], row = wm*TM + a*16*VA + VA*i' + e with i' = the accumulator's row inside its MFMA
+    // tile, col = cb[b] + f: the VB values f of one (a, e, b, v) are neighbours in memory
+    T *slab = static_cast<T *>(g.slabs) + static_cast<size_t>(blockIdx.x) * g.m * g.n;
+#pragma unroll
+    for (int a = 0; a < RA; a++)
+#pragma unroll
+        for (int e = 0; e < VA; e++)
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                const unsigned row = wm * TM + a * 16 * VA + VA * M::row(lane, v) + e;
+                if (row < g.m) {
+#pragma unroll
+                    for (int b = 0; b < RB; b++)
+#pragma unroll
+                        for (int f = 0; f < VB; f++)
+                            if (cb[b] + f < g.n)
+                                slab[static_cast<size_t>(row) * g.n + cb[b] + f] = acc[a][e][b][f][v];
+                }
+            }
+}
+
+// C[e] = sum over slabs, slabs added in index order inside each of GY interleaved groups and the groups in
+// order after that: the same association for the same shapes, whatever the timing.
+template <typename T>
+__global__ __launch_bounds__(256) void ts_slab_reduce_kernel(T *C, size_t ldc, const T *slabs, unsigned nslabs, unsigned m,
+                                                             unsigned n) {
+    constexpr int EX = 32, GY = 8;
+    __shared__ T part[GY][EX];
+    const int ex = threadIdx.x % EX, gy = threadIdx.x / EX;
+    const size_t elems = static_cast<size_t>(m) * n;
+    const size_t e = static_cast<size_t>(blockIdx.x) * EX + ex;
+    T s0 = T(0), s1 = T(0), s2 = T(0), s3 = T(0);
+    if (e < elems) {
+        unsigned z = gy;
+        for (; z + 3 * GY < nslabs; z += 4 * GY) {
+            s0 += slabs[static_cast<size_t>(z) * elems + e];
+            s1 += slabs[static_cast<size_t>(z + GY) * elems + e];
+            s2 += slabs[static_cast<size_t>(z + 2 * GY) * elems + e];
+            s3 += slabs[static_cast<size_t>(z + 3 * GY) * elems + e];
+        }
+        for (; z < nslabs; z += GY)
+            s0 += slabs[static_cast<size_t>(z) * elems + e];
+    }
+    part[gy][ex] = (s0 + s1) + (s2 + s3);
+    __syncthreads();
+    if (gy == 0 && e < elems) {
+        T s = part[0][ex];
+#pragma unroll
+        for (int q = 1; q < GY; q++)
+            s += part[q][ex];
+        C[(e / n) * ldc + e % n] = s;
+    }
+}
+
+// ---------------------------------------------------------------------------------------
+// ts_nt
+// ---------------------------------------------------------------------------------------
+struct TsNtArgs {
+    const void *A, *B;
+    void *C;
+    size_t lda, ldb, ldc, M;
+    unsigned n, K;
+    unsigned kpad;   // K rounded up to whole chunks
+};
+
+// NB column blocks of 16; each wave walks over row blocks of 16, two at a time.
+template <typename T, int NB> __global__ __launch_bounds__(256) void ts_nt_kernel(TsNtArgs g) {
+    using M = Mfma16<T>;
+    constexpr int V = 16 / sizeof(T);
+    constexpr int KC = 4 * V;     // k values per chunk
+    constexpr int RBW = 8;        // row blocks per wave
+    extern __shared__ __attribute__((aligned(16))) unsigned char ts_nt_lds[];
+    T *lb = reinterpret_cast<T *>(ts_nt_lds); // [NB*16][kpad + V], zero padded
+    const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
+    const int i = lane % 16, h = lane / 16;
+    const T *A = static_cast<const T *>(g.A);
+    const T *B = static_cast<const T *>(g.B);
+    T *C = static_cast<T *>(g.C);
+    const unsigned ldl = g.kpad + V;
+
+    for (unsigned idx = tid; idx < NB * 16 * (g.kpad / V); idx += 256) {
+        const unsigned j = idx / (g.kpad / V), kv = (idx % (g.kpad / V)) * V;
+        T t[V];
+        if (j < g.n && kv < g.K) {
+            ts_load<T, V>(B + static_cast<size_t>(j) * g.ldb + kv, t, false);
+        } else {
+#pragma unroll
+            for (int e = 0; e < V; e++)
+                t[e] = T(0);
+        }
+        dh_store_vec<T, V>(lb + j * ldl + kv, t);
+    }
+    __syncthreads();
+
+    const size_t row0 = (static_cast<size_t>(blockIdx.x) * 4 + wave) * (16 * RBW);
+    const unsigned chunks = g.kpad / KC;
+    for (int rb = 0; rb < RBW; rb += 2) {
+        const size_t r0 = row0 + static_cast<size_t>(rb) * 16 + i, r1 = r0 + 16;
+        if (r0 - i >= g.M)
+            break;
+        const bool ok0 = r0 < g.M, ok1 = r1 < g.M;
+        typename M::acc_t acc[2][NB];
+#pragma unroll
+        for (int b = 0; b < NB; b++) {
+            acc[0][b] = typename M::acc_t{0, 0, 0, 0};
+            acc[1][b] = typename M::acc_t{0, 0, 0, 0};
+        }
+        // chunks in groups of 4: eight vector loads in flight per lane
+        for (unsigned c0 = 0; c0 < chunks; c0 += 4) {
+            T fa[2][4][V];
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                const unsigned kv = (c0 + c) * KC + h * V;
+                const bool kok = kv < g.K;
+                if (ok0 && kok) {
+                    ts_load<T, V>(A + r0 * g.lda + kv, fa[0][c], true);
+                } else {
+#pragma unroll
+                    for (int e = 0; e < V; e++)
+                        fa[0][c][e] = T(0);
+                }
+                if (ok1 && kok) {
+                    ts_load<T, V>(A + r1 * g.lda + kv, fa[1][c], true);
+                } else {
+#pragma unroll
+                    for (int e = 0; e < V; e++)
+                        fa[1][c][e] = T(0);
+                }
+            }
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                if (c0 + c < chunks) {
+#pragma unroll
+                    for (int b = 0; b < NB; b++) {
+                        T fb[V];
+                        dh_load_vec<T, V>(lb + (b * 16 + i) * ldl + (c0 + c) * KC + h * V, fb);
+#pragma unroll
+                        for (int e = 0; e < V; e++) {
+                            acc[0][b] = M::mma(fa[0][c][e], fb[e], acc[0][b]);
+                            acc[1][b] = M::mma(fa[1][c][e], fb[e], acc[1][b]);
+                        }
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < 2; t++)
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                const size_t row = row0 + static_cast<size_t>(rb + t) * 16 + M::row(lane, v);
+                if (row < g.M) {
+#pragma unroll
+                    for (int b = 0; b < NB; b++)
+                        if (b * 16 + i < static_cast<int>(g.n))
+                            C[row * g.ldc + b * 16 + i] = acc[t][b][v];
+                }
+            }
+    }
+}
+
+// ---------------------------------------------------------------------------------------
+// host side
+// ---------------------------------------------------------------------------------------
+// side classes of ts_tn: up to 16 columns (scalar loads), up to 64 (one wave), up to 128 (two waves)
+template <typename T> struct TsSide {
+    static constexpr int V = 16 / sizeof(T);          // f32 4, f64 2
+    static constexpr int R64 = 64 / (16 * V);         // loads per lane for a 64-wide wave tile: f32 1, f64 2
+};
+
+template <typename T, int VA, int RA, int WM, int VB, int RB, int WN>
+static inline void ts_tn_launch(dh_ctx *ctx, const TsTnArgs &g, unsigned blocks) {
+    hipLaunchKernelGGL((ts_tn_kernel<T, VA, RA, VB, RB, WM, WN>), dim3(blocks), dim3(256), 0, ctx->stream, g);
+}
+
+// Returns false when the shape or the alignment does not fit (the caller then takes the tiled GEMM).
+template <typename T>
+bool ts_tn(dh_ctx *ctx, size_t m, size_t n, size_t K, const T *A, size_t lda, const T *B, size_t ldb, T *C, size_t ldc,
+           dh_status *status) {
+    constexpr int V = TsSide<T>::V, R64 = TsSide<T>::R64;
+    if (m == 0 || n == 0 || m > 128 || n > 128 || K < 4096)
+        return false;
+    const int cls_a = m <= 16 ? 0 : (m <= 64 ? 1 : 2), cls_b = n <= 16 ? 0 : (n <= 64 ? 1 : 2);
+    // vector loads need aligned rows and must not run past the end of the last row
+    auto vec_ok = [&](const T *p, size_t ld, size_t cols) {
+        return dh_aligned(p, 16) && ld % V == 0 && (cols % V == 0 || ld >= (cols + V - 1) / V * V);
+    };
+    if ((cls_a > 0 && !vec_ok(A, lda, m)) || (cls_b > 0 && !vec_ok(B, ldb, n)))
+        return false;
+    const int wm = cls_a == 2 ? 2 : 1, wn = cls_b == 2 ? 2 : 1, kw = 4 / (wm * wn);
+    const int nacc = (cls_a == 0 ? 1 : V * R64) * (cls_b == 0 ? 1 : V * R64);
+    const int unroll = nacc >= 16 ? 2 : 4;
+    const size_t gran = static_cast<size_t>(4) * kw * unroll;
+    // one or two workgroups per CU; each gets at least 32 row quads per wave
+    size_t blocks = static_cast<size_t>(ctx->num_cus) * (nacc >= 16 ? 1 : 2);
+    size_t k_chunk = dh_ceil_div(dh_ceil_div(K, blocks), gran) * gran;
+    const size_t min_chunk = gran * 16;
+    if (k_chunk < min_chunk)
+        k_chunk = min_chunk;
+    blocks = dh_ceil_div(K, k_chunk);
+    void *wsv = nullptr;
+    *status = dh_workspace(ctx, blocks * m * n * sizeof(T), &wsv);
+    if (*status != DH_OK)
+        return true;
+    TsTnArgs g{};
+    g.A = A;
+    g.B = B;
+    g.slabs = wsv;
+    g.lda = lda;
+    g.ldb = ldb;
+    g.K = K;
+    g.k_chunk = k_chunk;
+    g.m = static_cast<unsigned>(m);
+    g.n = static_cast<unsigned>(n);
+    g.stream = (wm * wn == 1 && static_cast<const void *>(A) != static_cast<const void *>(B)) ? 1 : 0;
+    const unsigned nb = static_cast<unsigned>(blocks);
+#define DH_TS_B(VA_, RA_, WM_)                                                                     \
+    do {                                                                                           \
+        if (cls_b == 0)                                                                            \
+            ts_tn_launch<T, VA_, RA_, WM_, 1, 1, 1>(ctx, g, nb);                                   \
+        else if (cls_b == 1)                                                                       \
+            ts_tn_launch<T, VA_, RA_, WM_, V, R64, 1>(ctx, g, nb);                                 \
+        else                                                                                       \
+            ts_tn_launch<T, VA_, RA_, WM_, V, R64, 2>(ctx, g, nb);                                 \
+    } while (0)
+    if (cls_a == 0)
+        DH_TS_B(1, 1, 1);
+    else if (cls_a == 1)
+        DH_TS_B(V, R64, 1);
+    else
+        DH_TS_B(V, R64, 2);
+#undef DH_TS_B
+    const size_t elems = m * n;
+    hipLaunchKernelGGL((ts_slab_reduce_kernel<T>), dim3(static_cast<unsigned>(dh_ceil_div(elems, 32))), dim3(256), 0,
+                       ctx->stream, C, ldc, static_cast<const T *>(wsv), nb, g.m, g.n);
+    *status = DH_OK;
+    return true;
+}
+
+template <typename T>
+bool ts_nt(dh_ctx *ctx, size_t M, size_t n, size_t K, const T *A, size_t lda, const T *B, size_t ldb, T *C, size_t ldc,
+           dh_status *status) {
+    constexpr int V = 16 / sizeof(T), KC = 4 * V;
+    if (n == 0 || n > 32 || K == 0 || K > 512 || M < 65536)
+        return false;
+    if (!dh_aligned(A, 16) || !dh_aligned(B, 16) || lda % V || ldb % V || K % V)
+        return false;
+    const int nb = n <= 16 ? 1 : 2;
+    TsNtArgs g{};
+    g.A = A;
+    g.B = B;
+    g.C = C;
+    g.lda = lda;
+    g.ldb = ldb;
+    g.ldc = ldc;
+    g.M = M;
+    g.n = static_cast<unsigned>(n);
+    g.K = static_cast<unsigned>(K);
+    g.kpad = static_cast<unsigned>(dh_ceil_div(K, KC) * KC);
+    const size_t lds = static_cast<size_t>(nb) * 16 * (g.kpad + V) * sizeof(T);
+    const size_t blocks = dh_ceil_div(M, 4 * 16 * 8);
+    if (blocks >= (size_t(1) << 31) || lds > (size_t(48) << 10))
+        return false;
+    if (nb == 1)
+        hipLaunchKernelGGL((ts_nt_kernel<T, 1>), dim3(static_cast<unsigned>(blocks)), dim3(256), lds, ctx->stream, g);
+    else
+        hipLaunchKernelGGL((ts_nt_kernel<T, 2>), dim3(static_cast<unsigned>(blocks)), dim3(256), lds, ctx->stream, g);
+    *status = DH_OK;
+    return true;
+}
+
+} // namespace dh_gemm

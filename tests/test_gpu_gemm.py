@@ -190,3 +190,89 @@ def test_affine_errors(ctx, dt):
     w = DenseMatrix.from_numpy(ctx, np.ones((5, 3), dt))
     with pytest.raises(capi.DaphneHipError, match="bias dimensions not matching"):
         affineForward(None, x, w, DenseMatrix.from_numpy(ctx, np.ones((3, 1), dt)), ctx)
+
+
+# ---------------------------------------------------------------------------------------------------
+# tall-and-skinny shapes (the streaming kernels): t(A) B with a long contraction, A t(B) with many rows
+# ---------------------------------------------------------------------------------------------------
+TS_TN = [  # (K, m, n): every side class (<=16, <=64, <=128) on both sides, ragged K
+    (4096, 1, 1), (5000, 16, 64), (4097, 16, 16), (7001, 64, 16), (6000, 40, 40), (9999, 64, 64), (4500, 100, 100),
+    (4100, 128, 128), (8191, 100, 1), (5003, 128, 60), (5003, 30, 120), (4099, 13, 7), (20000, 18, 66),
+]
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("K,m,n", TS_TN)
+def test_matmul_tall_tn(ctx, dt, K, m, n):
+    rng = np.random.default_rng(K + 31 * m + n)
+    a = (rng.random((K, m)) * 2 - 1).astype(dt)
+    b = (rng.random((K, n)) * 2 - 1).astype(dt)
+    truth = (a.T.astype(np.float64) @ b.astype(np.float64)).astype(dt)
+    got = matMul(None, DenseMatrix.from_numpy(ctx, a), DenseMatrix.from_numpy(ctx, b), True, False, ctx).to_numpy()
+    assert got.shape == (m, n)
+    assert_close(got, truth, elementwise=False)
+    if K * m * n <= 5000 * 64 * 64:
+        assert_close(got, orc.matmul(a, b, True, False)[1], elementwise=False)
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+def test_matmul_tall_tn_integer_exact_and_views(ctx, dt):
+    rng = np.random.default_rng(5)
+    K = 6007
+    A = rng.integers(-3, 4, (K, 72)).astype(dt)
+    B = rng.integers(-3, 4, (K, 136)).astype(dt)
+    dA, dB = DenseMatrix.from_numpy(ctx, A), DenseMatrix.from_numpy(ctx, B)
+    # whole matrices, column slices at aligned and unaligned offsets (leading dimension > columns)
+    for (a0, a1, b0, b1) in [(0, 72, 0, 128), (8, 40, 16, 80), (3, 19, 5, 69), (0, 16, 4, 68), (1, 2, 0, 1)]:
+        exp = (A[:, a0:a1].T.astype(np.int64) @ B[:, b0:b1].astype(np.int64)).astype(dt)
+        got = matMul(None, dA.slice(0, K, a0, a1), dB.slice(0, K, b0, b1), True, False, ctx).to_numpy()
+        assert_exact(got, exp)
+    # into a view of a larger result
+    res = DenseMatrix(ctx, 80, 140, dt, zero=True)
+    matMul(res.slice(2, 74, 3, 131), dA, dB.slice(0, K, 0, 128), True, False, ctx)
+    full = res.to_numpy()
+    assert_exact(full[2:74, 3:131], (A.T.astype(np.int64) @ B[:, :128].astype(np.int64)).astype(dt))
+    full[2:74, 3:131] = 0
+    assert (full == 0).all()
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+def test_syrk_and_gemv_tall(ctx, dt):
+    rng = np.random.default_rng(6)
+    X = (rng.random((50000, 100)) * 2 - 1).astype(dt)
+    y = (rng.random((50000, 1)) * 2 - 1).astype(dt)
+    dX, dy = DenseMatrix.from_numpy(ctx, X), DenseMatrix.from_numpy(ctx, y)
+    got = syrk(None, dX, True, ctx).to_numpy()
+    truth = X.T.astype(np.float64) @ X.astype(np.float64)
+    assert_close(got, truth.astype(dt), elementwise=False)
+    assert_exact(got, got.T)  # both triangles come from the same products in the same order
+    gv = matMul(None, dX, dy, True, False, ctx).to_numpy()
+    assert gv.shape == (100, 1)
+    assert_close(gv, (X.T.astype(np.float64) @ y.astype(np.float64)).astype(dt), elementwise=False)
+    # the vector given as a row (transposed rhs) and as a strided column of a wider matrix
+    yr = np.ascontiguousarray(y.T)
+    assert_close(matMul(None, dX, DenseMatrix.from_numpy(ctx, yr), True, True, ctx).to_numpy(), gv, elementwise=False)
+    Y3 = np.repeat(y, 3, axis=1).copy()
+    assert_exact(matMul(None, dX, DenseMatrix.from_numpy(ctx, Y3).slice(0, 50000, 1, 2), True, False, ctx).to_numpy(), gv)
+
+
+TS_NT = [  # (M, n, K)
+    (65536, 16, 64), (70001, 16, 64), (65537, 1, 4), (66000, 7, 20), (65536, 32, 128), (80000, 17, 72), (65536, 16, 512),
+    (100003, 10, 100),
+]
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("M,n,K", TS_NT)
+def test_matmul_tall_nt(ctx, dt, M, n, K):
+    rng = np.random.default_rng(M + 7 * n + K)
+    a = (rng.random((M, K)) * 2 - 1).astype(dt)
+    b = (rng.random((n, K)) * 2 - 1).astype(dt)
+    truth = (a.astype(np.float64) @ b.T.astype(np.float64)).astype(dt)
+    got = matMul(None, DenseMatrix.from_numpy(ctx, a), DenseMatrix.from_numpy(ctx, b), False, True, ctx).to_numpy()
+    assert got.shape == (M, n)
+    assert_close(got, truth, elementwise=False)
+    ai = rng.integers(-3, 4, (M, K)).astype(dt)
+    bi = rng.integers(-3, 4, (n, K)).astype(dt)
+    goti = matMul(None, DenseMatrix.from_numpy(ctx, ai), DenseMatrix.from_numpy(ctx, bi), False, True, ctx).to_numpy()
+    assert_exact(goti, (ai.astype(np.int64) @ bi.T.astype(np.int64)).astype(dt))
