@@ -87,7 +87,7 @@ def run(args) -> int:
             dt = time.perf_counter() - t0
             cpu = {"value": round(nbytes / dt / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
                    "sample": f"the whole configuration once, single thread, scalar loops ({dt:.2f} s)"}
-        roof = {"bound": "hbm", "kernel": "gemm_kernel<double,128,128,8,2,2,true,false> split-K (syrk)",
+        roof = {"bound": "hbm", "kernel": "ts_tn_kernel<double,2,2,2,2,2,2> (syrk, streaming t(X) X)",
                 "achieved": round((n * m * 8 + m * m * 8) / t_syrk / 1e6, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round((n * m * 8 + m * m * 8) / t_syrk / 1e6 / HBM_PEAK_GBS, 4), "traffic": None}
         out = _line(nbytes / ms / 1e6, "GB/s", ms, args, "f64",
@@ -128,7 +128,7 @@ def run(args) -> int:
             dt = time.perf_counter() - t0
             cpu = {"value": round(nbytes * (ns / n) / dt / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
                    "sample": f"one iteration on the first {ns} of {n} rows, single thread ({dt:.2f} s)"}
-        roof = {"bound": "hbm", "kernel": "gemm_kernel<float,256,32,16,4,1,false,true> (X C^T)",
+        roof = {"bound": "hbm", "kernel": "ts_nt_kernel<float,1> (X t(C))",
                 "achieved": round((n * f * 4 + D) / t_gemm / 1e6, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round((n * f * 4 + D) / t_gemm / 1e6 / HBM_PEAK_GBS, 4), "traffic": None}
         out = _line(nbytes / ms / 1e6, "GB/s", ms, args, "f32",

@@ -5,7 +5,8 @@
 // getrf + getrs) with the result of the CPU kernel (src/runtime/local/kernels/Solve.h:86-116,
 // LAPACKE_?gesv): same pivot choice (first row of maximal magnitude), multipliers formed with
 // the reciprocal of the pivot. The systems on this path are small (100 x 100 normal equations),
-// so one workgroup working in a global scratch copy of A is latency-, not throughput-bound.
+// so the work is latency-bound: a system that fits in LDS (up to about 135 doubles / 190 floats a
+// side) is factored there with two barriers per column; larger ones work in a global scratch copy.
 #include "common.h"
 
 namespace {
@@ -106,6 +107,119 @@ __global__ __launch_bounds__(SOLVE_THREADS) void lu_solve_kernel(T *lu, T *x, co
     }
 }
 
+// The whole system in LDS. Per column: wave 0 finds the pivot with shuffles, swaps the rows and
+// publishes the pivot row; after one barrier all 256 threads apply the rank-1 update (16 x 16 thread
+// grid, multipliers recomputed per row instead of stored: only U and the eliminated right-hand side
+// are needed afterwards); a second barrier closes the column. Back substitution runs in wave 0 alone,
+// right-hand side in registers, one shuffle per unknown.
+constexpr int LDS_SOLVE_MAX_SLOTS = 3; // rows per lane in the back substitution: n <= 192
+
+template <typename T>
+__global__ __launch_bounds__(256) void lu_solve_lds_kernel(T *x_out, const T *A, size_t lda, const T *b, unsigned n,
+                                                           int *flag) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char solve_lds[];
+    __shared__ int s_stop;
+    const unsigned ld = n | 1u; // odd stride: column walks spread over the banks
+    T *a = reinterpret_cast<T *>(solve_lds);
+    T *prow = a + static_cast<size_t>(n) * ld;
+    T *xs = prow + n;
+    const unsigned tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
+    const unsigned tx = tid % 16, ty = tid / 16;
+    for (unsigned e = tid; e < n * n; e += 256)
+        a[(e / n) * ld + e % n] = A[static_cast<size_t>(e / n) * lda + e % n];
+    for (unsigned i = tid; i < n; i += 256)
+        xs[i] = b[i];
+    if (tid == 0)
+        s_stop = 0;
+    __syncthreads();
+    for (unsigned j = 0; j < n; j++) {
+        if (wave == 0) {
+            // pivot: first row i >= j with the largest |a[i][j]|
+            T best = T(-1);
+            unsigned bi = j;
+            for (unsigned i = j + lane; i < n; i += 64) {
+                const T v = dev_abs(a[i * ld + j]);
+                if (v > best) {
+                    best = v;
+                    bi = i;
+                }
+            }
+#pragma unroll
+            for (int off = 32; off >= 1; off >>= 1) {
+                const T ov = __shfl_xor(best, off);
+                const unsigned oi = __shfl_xor(bi, off);
+                if (ov > best || (ov == best && oi < bi)) {
+                    best = ov;
+                    bi = oi;
+                }
+            }
+            const unsigned p = bi;
+            if (a[p * ld + j] == T(0)) {
+                if (lane == 0) {
+                    *flag = static_cast<int>(j) + 1; // info > 0 of ?gesv
+                    s_stop = 1;
+                }
+            } else {
+                for (unsigned c = j + lane; c < n; c += 64) {
+                    const T pv = a[p * ld + c];
+                    prow[c] = pv;
+                    if (p != j) {
+                        a[p * ld + c] = a[j * ld + c];
+                        a[j * ld + c] = pv;
+                    }
+                }
+                if (lane == 0 && p != j) {
+                    const T t = xs[j];
+                    xs[j] = xs[p];
+                    xs[p] = t;
+                }
+            }
+        }
+        __syncthreads();
+        if (s_stop)
+            return;
+        const T inv = T(1) / prow[j];
+        const T xj = xs[j];
+        for (unsigned i = j + 1 + ty; i < n; i += 16) {
+            const T l = a[i * ld + j] * inv;
+            for (unsigned c = j + 1 + tx; c < n; c += 16)
+                a[i * ld + c] -= l * prow[c];
+            if (tx == 0)
+                xs[i] -= l * xj;
+        }
+        __syncthreads();
+    }
+    if (wave != 0)
+        return;
+    // back substitution, column oriented: x[j] = rhs[j] / U[j][j]; rhs[r] -= U[r][j] x[j] for r < j
+    T rhs[LDS_SOLVE_MAX_SLOTS], res[LDS_SOLVE_MAX_SLOTS];
+#pragma unroll
+    for (int s_ = 0; s_ < LDS_SOLVE_MAX_SLOTS; s_++) {
+        const unsigned r = lane + 64 * s_;
+        rhs[s_] = r < n ? xs[r] : T(0);
+        res[s_] = T(0);
+    }
+    for (unsigned jj = n; jj-- > 0;) {
+        const unsigned slot = jj / 64, owner = jj % 64;
+        const T mine = slot == 0 ? rhs[0] : (slot == 1 ? rhs[1] : rhs[2]);
+        const T xj = __shfl(mine, owner) / a[jj * ld + jj];
+#pragma unroll
+        for (int s_ = 0; s_ < LDS_SOLVE_MAX_SLOTS; s_++) {
+            const unsigned r = lane + 64 * s_;
+            if (r < jj)
+                rhs[s_] -= a[r * ld + jj] * xj;
+            else if (r == jj)
+                res[s_] = xj;
+        }
+    }
+#pragma unroll
+    for (int s_ = 0; s_ < LDS_SOLVE_MAX_SLOTS; s_++) {
+        const unsigned r = lane + 64 * s_;
+        if (r < n)
+            x_out[r] = res[s_];
+    }
+}
+
 __global__ void clear_flag_kernel(int *flag) { *flag = 0; }
 
 template <typename T> dh_status solve(dh_ctx *ctx, T *x, const T *A, size_t n, size_t lda, const T *b) {
@@ -116,13 +230,29 @@ template <typename T> dh_status solve(dh_ctx *ctx, T *x, const T *A, size_t n, s
         return dh_fail(DH_ERR_RUNTIME, "#cols of lhs must match row skip");
     if (n >= (size_t(1) << 15))
         return dh_fail(DH_ERR_RUNTIME, "Solve: systems beyond 32767 unknowns are not supported by this kernel");
-    void *wsv = nullptr;
-    dh_status st = dh_workspace(ctx, n * n * sizeof(T), &wsv);
-    if (st != DH_OK)
-        return st;
     hipLaunchKernelGGL(clear_flag_kernel, dim3(1), dim3(1), 0, ctx->stream, ctx->flag_dev);
-    hipLaunchKernelGGL((lu_solve_kernel<T>), dim3(1), dim3(SOLVE_THREADS), 0, ctx->stream, static_cast<T *>(wsv), x, A,
-                       lda, b, static_cast<unsigned>(n), ctx->flag_dev);
+    const size_t lds_bytes = (n * (n | 1) + 2 * n) * sizeof(T);
+    if (n <= 64 * LDS_SOLVE_MAX_SLOTS && lds_bytes <= (size_t(150) << 10)) {
+        if (lds_bytes > (size_t(64) << 10)) {
+            static std::mutex attr_lock;
+            static bool attr_set[16] = {};
+            std::lock_guard<std::mutex> guard(attr_lock);
+            if (ctx->device < 16 && !attr_set[ctx->device]) {
+                DH_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&lu_solve_lds_kernel<T>),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, 150 << 10));
+                attr_set[ctx->device] = true;
+            }
+        }
+        hipLaunchKernelGGL((lu_solve_lds_kernel<T>), dim3(1), dim3(256), lds_bytes, ctx->stream, x, A, lda, b,
+                           static_cast<unsigned>(n), ctx->flag_dev);
+    } else {
+        void *wsv = nullptr;
+        dh_status st = dh_workspace(ctx, n * n * sizeof(T), &wsv);
+        if (st != DH_OK)
+            return st;
+        hipLaunchKernelGGL((lu_solve_kernel<T>), dim3(1), dim3(SOLVE_THREADS), 0, ctx->stream, static_cast<T *>(wsv), x,
+                           A, lda, b, static_cast<unsigned>(n), ctx->flag_dev);
+    }
     DH_CHECK_LAUNCH();
     DH_CHECK_HIP(hipMemcpyAsync(ctx->flag_host, ctx->flag_dev, sizeof(int), hipMemcpyDeviceToHost, ctx->stream));
     DH_CHECK_HIP(hipStreamSynchronize(ctx->stream));

@@ -111,31 +111,35 @@ __global__ __launch_bounds__(256) void ts_tn_kernel(TsTnArgs g) {
     const size_t kb = static_cast<size_t>(blockIdx.x) * g.k_chunk;
     const size_t ke = kb + g.k_chunk < g.K ? kb + g.k_chunk : g.K;
 
-    T fa[U][RA][VA], fb[U][RB][VB];
-    auto load_quad = [&](int u, size_t k, bool guard) {
+    // one group = U quads; two register sets so that the loads of the next group are in flight while
+    // the matrix cores work on the current one
+    struct Frag {
+        T a[U][RA][VA], b[U][RB][VB];
+    };
+    auto load_quad = [&](Frag &fr, int u, size_t k, bool guard) {
         const bool row_ok = !guard || k < ke;
 #pragma unroll
         for (int a = 0; a < RA; a++) {
             if (oka[a] && row_ok) {
-                ts_load<T, VA>(A + k * g.lda + ca[a], fa[u][a], stream);
+                ts_load<T, VA>(A + k * g.lda + ca[a], fr.a[u][a], stream);
             } else {
 #pragma unroll
                 for (int e = 0; e < VA; e++)
-                    fa[u][a][e] = T(0);
+                    fr.a[u][a][e] = T(0);
             }
         }
 #pragma unroll
         for (int b = 0; b < RB; b++) {
             if (okb[b] && row_ok) {
-                ts_load<T, VB>(B + k * g.ldb + cb[b], fb[u][b], stream);
+                ts_load<T, VB>(B + k * g.ldb + cb[b], fr.b[u][b], stream);
             } else {
 #pragma unroll
                 for (int f = 0; f < VB; f++)
-                    fb[u][b][f] = T(0);
+                    fr.b[u][b][f] = T(0);
             }
         }
     };
-    auto mma_quad = [&](int u) {
+    auto mma_quad = [&](const Frag &fr, int u) {
 #pragma unroll
         for (int a = 0; a < RA; a++)
 #pragma unroll
@@ -144,25 +148,46 @@ __global__ __launch_bounds__(256) void ts_tn_kernel(TsTnArgs g) {
                 for (int b = 0; b < RB; b++)
 #pragma unroll
                     for (int f = 0; f < VB; f++)
-                        acc[a][e][b][f] = M::mma(fa[u][a][e], fb[u][b][f], acc[a][e][b][f]);
+                        acc[a][e][b][f] = M::mma(fr.a[u][a][e], fr.b[u][b][f], acc[a][e][b][f]);
     };
 
     // quad q of this wave covers rows kb + (q*KW + wk)*4 .. +3; lane group h takes row +h
     size_t k = kb + static_cast<size_t>(wk) * 4 + h;
     constexpr size_t STEP = static_cast<size_t>(KW) * 4;
-    // full groups of U quads: every row of the last quad is inside the chunk
-    while (k - h + (U - 1) * STEP + 4 <= ke) {
+    // a full group: every row of its last quad is inside the chunk
+    auto full = [&]() { return k - h + (U - 1) * STEP + 4 <= ke; };
+    auto load_group = [&](Frag &fr) {
 #pragma unroll
         for (int u = 0; u < U; u++)
-            load_quad(u, k + u * STEP, false);
-#pragma unroll
-        for (int u = 0; u < U; u++)
-            mma_quad(u);
+            load_quad(fr, u, k + u * STEP, false);
         k += U * STEP;
+    };
+    auto mma_group = [&](const Frag &fr) {
+#pragma unroll
+        for (int u = 0; u < U; u++)
+            mma_quad(fr, u);
+    };
+    Frag f0, f1;
+    if (full()) {
+        load_group(f0);
+        while (true) {
+            bool more = full();
+            if (more)
+                load_group(f1);
+            mma_group(f0);
+            if (!more)
+                break;
+            more = full();
+            if (more)
+                load_group(f0);
+            mma_group(f1);
+            if (!more)
+                break;
+        }
     }
     while (k - h < ke) {
-        load_quad(0, k, true);
-        mma_quad(0);
+        load_quad(f0, 0, k, true);
+        mma_quad(f0, 0);
         k += STEP;
     }
 
@@ -398,10 +423,10 @@ bool ts_tn(dh_ctx *ctx, size_t m, size_t n, size_t K, const T *A, size_t lda, co
     const int nacc = (cls_a == 0 ? 1 : V * R64) * (cls_b == 0 ? 1 : V * R64);
     const int unroll = nacc >= 16 ? 2 : 4;
     const size_t gran = static_cast<size_t>(4) * kw * unroll;
-    // one or two workgroups per CU; each gets at least 32 row quads per wave
+    // one or two workgroups per CU (more only add slab traffic), each with at least four load groups per wave
     size_t blocks = static_cast<size_t>(ctx->num_cus) * (nacc >= 16 ? 1 : 2);
     size_t k_chunk = dh_ceil_div(dh_ceil_div(K, blocks), gran) * gran;
-    const size_t min_chunk = gran * 16;
+    const size_t min_chunk = gran * 4;
     if (k_chunk < min_chunk)
         k_chunk = min_chunk;
     blocks = dh_ceil_div(K, k_chunk);

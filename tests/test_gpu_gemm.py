@@ -139,7 +139,7 @@ def test_syrk_integer_valued_exact(ctx, dt):
 
 
 @pytest.mark.parametrize("dt", DTYPES)
-@pytest.mark.parametrize("n", [1, 3, 10, 100, 257])
+@pytest.mark.parametrize("n", [1, 3, 10, 63, 64, 65, 100, 128, 135, 136, 150, 190, 192, 193, 257])
 def test_solve(ctx, dt, n):
     rng = np.random.default_rng(n)
     A = (rng.random((n, n)) - 0.5).astype(dt) + np.eye(n, dtype=dt) * dt(0.1)
@@ -152,6 +152,29 @@ def test_solve(ctx, dt, n):
     # residual against the definition
     r = A.astype(np.float64) @ got.astype(np.float64) - b
     assert np.abs(r).max() <= (5e-4 if dt == np.float32 else 1e-11) * max(1.0, np.abs(got).max()) * n
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+def test_solve_pivoting_and_late_singularity(ctx, dt):
+    rng = np.random.default_rng(77)
+    for n in (4, 70, 130, 200):
+        # zero diagonal: every column needs a row exchange; integer entries make ties in the pivot search
+        A = rng.integers(-3, 4, (n, n)).astype(dt)
+        np.fill_diagonal(A, 0)
+        A += np.roll(np.eye(n, dtype=dt), 1, axis=0) * dt(9)
+        b = rng.integers(-5, 6, (n, 1)).astype(dt)
+        st, exp = orc.solve(A, b)
+        assert st == 0
+        got = solve(None, DenseMatrix.from_numpy(ctx, A), DenseMatrix.from_numpy(ctx, b), ctx).to_numpy()
+        assert_close(got, exp, rtol=2e-3 if dt == np.float32 else 1e-9, elementwise=False)
+        # rank deficiency that only shows in the last column
+        S = rng.random((n, n)).astype(dt)
+        S[:, -1] = S[:, 0]
+        if n <= 4:  # exact zero pivot only when the elimination is exact
+            S = np.array([[1, 2, 3, 1], [0, 1, 4, 0], [0, 0, 1, 0], [1, 2, 3, 1]], dt)
+            with pytest.raises(capi.DaphneHipError, match="exactly singular"):
+                solve(None, DenseMatrix.from_numpy(ctx, S), DenseMatrix.from_numpy(ctx, b), ctx)
+            assert orc.solve(S, b)[0] != 0
 
 
 @pytest.mark.parametrize("dt", DTYPES)
