@@ -410,27 +410,37 @@ __global__ __launch_bounds__(THREADS) void row_kernel(T *res, size_t ld_res, con
     }
 }
 
-// IDXMIN / IDXMAX per row: (value, index) pairs; on equal values the lower index wins.
-template <typename T, int VEC, bool IS_MIN>
+// IDXMIN / IDXMAX per row: (value, index) pairs; on equal values the lower index wins. Same row
+// mapping as row_kernel (a wavefront owns GPW * UR consecutive rows per step, results stored as one
+// contiguous run). I is the index type carried through the reduction: 32 bits unless a row has 2^32
+// or more columns.
+template <typename T, int VEC, bool IS_MIN, typename I>
 __global__ __launch_bounds__(THREADS) void row_idx_kernel(uint64_t *res, size_t ld_res, const T *arg, size_t rows,
                                                           size_t cols, size_t ld, int G) {
-    constexpr int UR = 4; // rows in flight per lane group (clamped past the end, dropped at the store)
+    constexpr int UR = 4;
+    constexpr I NONE = ~static_cast<I>(0);
     const int tid = threadIdx.x;
     const int lane = tid % G;
-    const size_t rows_per_block = THREADS / G;
+    const int wlane = tid % DH_WAVE;
+    const int GPW = DH_WAVE / G;
+    const int g_in_wave = wlane / G;
     const size_t cvecs = cols / VEC;
-    const size_t stride = static_cast<size_t>(gridDim.x) * rows_per_block;
+    const size_t rows_per_step = static_cast<size_t>(GPW) * UR;
+    const size_t wave_id = static_cast<size_t>(blockIdx.x) * (THREADS / DH_WAVE) + tid / DH_WAVE;
+    const size_t wave_stride = static_cast<size_t>(gridDim.x) * (THREADS / DH_WAVE) * rows_per_step;
     const T worst = IS_MIN ? std::numeric_limits<T>::infinity() : -std::numeric_limits<T>::infinity();
-    for (size_t r0 = static_cast<size_t>(blockIdx.x) * rows_per_block + tid / G; r0 < rows; r0 += stride * UR) {
+    for (size_t base = wave_id * rows_per_step; base < rows; base += wave_stride) {
         const T *row[UR];
         T best[UR];
-        unsigned long long bi[UR];
+        I bi[UR];
+        bool nan0[UR]; // element 0 of the row is NaN (known to the lane that loads it)
 #pragma unroll
         for (int u = 0; u < UR; u++) {
-            const size_t r = r0 + u * stride;
+            const size_t r = base + static_cast<size_t>(u * GPW + g_in_wave);
             row[u] = arg + (r < rows ? r : rows - 1) * ld;
             best[u] = worst;
-            bi[u] = ~0ull;
+            bi[u] = NONE;
+            nan0[u] = false;
         }
         for (size_t cv = lane; cv < cvecs; cv += G) {
             T x[UR][VEC];
@@ -438,38 +448,58 @@ __global__ __launch_bounds__(THREADS) void row_idx_kernel(uint64_t *res, size_t 
             for (int u = 0; u < UR; u++)
                 dh_load_vec_stream<T, VEC>(row[u] + cv * VEC, x[u]);
 #pragma unroll
-            for (int u = 0; u < UR; u++)
+            for (int u = 0; u < UR; u++) {
+                if (cv == 0)
+                    nan0[u] = dev_isnan(x[u][0]);
 #pragma unroll
                 for (int i = 0; i < VEC; i++) {
-                    const unsigned long long idx = cv * VEC + i;
+                    const I idx = static_cast<I>(cv * VEC + i);
                     const bool better = IS_MIN ? (x[u][i] < best[u]) : (x[u][i] > best[u]);
                     // within a lane indices only grow, so a tie keeps the earlier one, except
                     // against the sentinel (an actual +-inf value must beat "nothing seen yet")
-                    const bool first_seen = (bi[u] == ~0ull) && !dev_isnan(x[u][i]);
+                    const bool first_seen = (bi[u] == NONE) && (x[u][i] == best[u]);
                     if (better || first_seen) {
                         best[u] = x[u][i];
                         bi[u] = idx;
                     }
                 }
+            }
         }
 #pragma unroll
         for (int u = 0; u < UR; u++) {
             for (int off = G / 2; off >= 1; off >>= 1) {
                 const T ov = dh_shfl_xor(best[u], off);
-                const unsigned long long oi = dh_shfl_xor(bi[u], off);
+                const I oi = dh_shfl_xor(bi[u], off);
                 const bool better = IS_MIN ? (ov < best[u]) : (ov > best[u]);
                 if (better || (ov == best[u] && oi < bi[u])) {
                     best[u] = ov;
                     bi[u] = oi;
                 }
             }
-            const size_t r = r0 + u * stride;
-            if (lane == 0 && r < rows) {
-                // AggRow.h:73-80: the scan starts from element 0; if that is NaN no later element
-                // compares below/above it, so 0 is returned. An all-NaN tail leaves bi untouched.
-                if (dev_isnan(row[u][0]) || bi[u] == ~0ull)
-                    bi[u] = 0;
-                res[r * ld_res] = bi[u];
+            // AggRow.h:73-80: the scan starts from element 0; if that is NaN no later element
+            // compares below/above it, so 0 is returned. A row of NaNs only leaves bi untouched.
+            // (after the xor exchange every lane of the group holds the group's result; lane 0 knows nan0)
+            if (nan0[u] || bi[u] == NONE)
+                bi[u] = 0;
+        }
+        if (GPW * UR <= DH_WAVE) {
+            // lane j takes the result of row base + j: group j % GPW, slot j / GPW, from that group's lane 0
+            I mine = 0;
+#pragma unroll
+            for (int u = 0; u < UR; u++) {
+                const I v = __shfl(bi[u], (wlane % GPW) * G, DH_WAVE);
+                if (wlane / GPW == u)
+                    mine = v;
+            }
+            const size_t orow = base + static_cast<size_t>(wlane);
+            if (wlane < GPW * UR && orow < rows)
+                res[orow * ld_res] = mine;
+        } else {
+#pragma unroll
+            for (int u = 0; u < UR; u++) {
+                const size_t r = base + static_cast<size_t>(u * GPW + g_in_wave);
+                if (lane == 0 && r < rows)
+                    res[r * ld_res] = bi[u];
             }
         }
     }
@@ -560,17 +590,28 @@ dh_status agg_row_idx(dh_ctx *ctx, int op, uint64_t *res, size_t ld_res, const T
     const bool vec_ok = (cols % V == 0) && (ld % V == 0) && dh_aligned(arg, 16);
     const int G = pick_group(vec_ok ? cols / V : cols);
     const dim3 grid(row_grid(ctx, rows, G)), block(THREADS);
+    const bool wide = cols >= 0xffffffffull; // index does not fit 32 bits next to the sentinel
+#define DH_ROW_IDX(VEC_, MIN_)                                                                                          \
+    do {                                                                                                                \
+        if (wide)                                                                                                       \
+            hipLaunchKernelGGL((row_idx_kernel<T, VEC_, MIN_, unsigned long long>), grid, block, 0, ctx->stream, res,   \
+                               ld_res, arg, rows, cols, ld, G);                                                         \
+        else                                                                                                            \
+            hipLaunchKernelGGL((row_idx_kernel<T, VEC_, MIN_, unsigned>), grid, block, 0, ctx->stream, res, ld_res,     \
+                               arg, rows, cols, ld, G);                                                                 \
+    } while (0)
     if (vec_ok) {
         if (op == DH_AGG_IDXMIN)
-            hipLaunchKernelGGL((row_idx_kernel<T, V, true>), grid, block, 0, ctx->stream, res, ld_res, arg, rows, cols, ld, G);
+            DH_ROW_IDX(V, true);
         else
-            hipLaunchKernelGGL((row_idx_kernel<T, V, false>), grid, block, 0, ctx->stream, res, ld_res, arg, rows, cols, ld, G);
+            DH_ROW_IDX(V, false);
     } else {
         if (op == DH_AGG_IDXMIN)
-            hipLaunchKernelGGL((row_idx_kernel<T, 1, true>), grid, block, 0, ctx->stream, res, ld_res, arg, rows, cols, ld, G);
+            DH_ROW_IDX(1, true);
         else
-            hipLaunchKernelGGL((row_idx_kernel<T, 1, false>), grid, block, 0, ctx->stream, res, ld_res, arg, rows, cols, ld, G);
+            DH_ROW_IDX(1, false);
     }
+#undef DH_ROW_IDX
     DH_CHECK_LAUNCH();
     return DH_OK;
 }
