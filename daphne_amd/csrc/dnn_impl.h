@@ -403,8 +403,16 @@ __global__ __launch_bounds__(256) void maxpool2x2_kernel(T *res, const T *data, 
     }
     const T *in = data + r * 2 * W + static_cast<size_t>(j) * VI;
     T a[VI], b[VI], o[VI / 2];
-    dh_load_vec_stream<T, VI>(in, a);
-    dh_load_vec_stream<T, VI>(in + W, b);
+    {
+        typedef T in_vec __attribute__((ext_vector_type(VI)));
+        const in_vec va = __builtin_nontemporal_load(reinterpret_cast<const in_vec *>(in));
+        const in_vec vb = __builtin_nontemporal_load(reinterpret_cast<const in_vec *>(in + W));
+#pragma unroll
+        for (int i = 0; i < VI; i++) {
+            a[i] = va[i];
+            b[i] = vb[i];
+        }
+    }
 #pragma unroll
     for (int i = 0; i < VI / 2; i++) {
         // window order of Pooling.cpp:77-105 with the accumulator starting at zero
@@ -456,11 +464,17 @@ dh_status maxpool_forward(dh_ctx *ctx, T *res, size_t *res_h, size_t *res_w, con
     if (grid > cap)
         grid = cap;
     constexpr int VI = 16 / sizeof(T);
-    if (ph == 2 && pw == 2 && sh == 2 && sw == 2 && padh == 0 && padw == 0 && H % 2 == 0 && W % VI == 0 &&
-        dh_aligned(data, 16) && dh_aligned(res, 8) && total * 2 / VI < (size_t(1) << 39)) {
+    const bool pairs = ph == 2 && pw == 2 && sh == 2 && sw == 2 && padh == 0 && padw == 0 && H % 2 == 0 && W % 2 == 0 &&
+                       total < (size_t(1) << 39);
+    if (pairs && W % VI == 0 && dh_aligned(data, 16) && dh_aligned(res, 8)) {
         const size_t items = N * C * P * (W / VI);
         hipLaunchKernelGGL((maxpool2x2_kernel<T, VI>), dim3(static_cast<unsigned>(dh_ceil_div(items, 256))), dim3(256), 0,
                            ctx->stream, res, data, items, static_cast<unsigned>(W), static_cast<unsigned>(W / VI));
+    } else if (pairs && VI > 2 && dh_aligned(data, 8)) {
+        // rows of an even number of floats that is not a multiple of four: 8-byte loads, one output per thread
+        const size_t items = N * C * P * (W / 2);
+        hipLaunchKernelGGL((maxpool2x2_kernel<T, 2>), dim3(static_cast<unsigned>(dh_ceil_div(items, 256))), dim3(256), 0,
+                           ctx->stream, res, data, items, static_cast<unsigned>(W), static_cast<unsigned>(W / 2));
     } else if (P == 1 && Q == 1 && W == 1) {
         // Pooling.cpp:57-66: this quick path folds the window into numeric_limits::max(), so that
         // value is what the CPU kernel returns for every output.
