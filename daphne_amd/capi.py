@@ -9,7 +9,7 @@ from pathlib import Path
 
 LIB_PATH = Path(__file__).resolve().parent / "libdaphne_hip.so"
 
-DH_OK, DH_ERR_RUNTIME, DH_ERR_INVALID_ARG, DH_ERR_DOMAIN, DH_ERR_HIP, DH_ERR_OOM = range(6)
+DH_OK, DH_ERR_RUNTIME, DH_ERR_INVALID_ARG, DH_ERR_DOMAIN, DH_ERR_HIP, DH_ERR_OOM, DH_ERR_OUT_OF_RANGE = range(7)
 
 sz = C.c_size_t
 vp = C.c_void_p
@@ -30,6 +30,10 @@ class DaphneHipInvalidArgument(DaphneHipError, ValueError):
 
 class DaphneHipDomainError(DaphneHipError, ArithmeticError):
     """std::domain_error of the reference (sqrt/ln/asin/acos outside their domain)."""
+
+
+class DaphneHipOutOfRange(DaphneHipError, IndexError):
+    """std::out_of_range of the reference (ExtractCol position outside the matrix)."""
 
 
 _lib = None
@@ -89,6 +93,13 @@ _LATE_SIGNATURES: dict[str, list] = {
     "dh_bias_add": [vp, vp, vp, sz, sz, vp, sz],
     "dh_batchnorm_inference": [vp, vp, vp, sz, sz, vp, vp, vp, vp, sz, "T", i32],
     "dh_softmax": [vp, vp, sz, vp, sz, sz, sz],
+    "dh_avgpool_forward": [vp, vp, C.POINTER(sz), C.POINTER(sz), vp, sz, sz, sz, sz, sz, sz, sz, sz, sz, sz],
+    "dh_relu_forward": [vp, vp, sz, vp, sz, sz, sz],
+    "dh_fill": [vp, vp, sz, "T", sz, sz],
+    "dh_col_bind": [vp, vp, sz, vp, sz, sz, sz, vp, sz, sz, sz],
+    "dh_extract_col": [vp, vp, sz, vp, sz, sz, sz, vp, sz, sz, sz],
+    "dh_transpose": [vp, vp, sz, vp, sz, sz, sz],
+    "dh_gemv": [vp, vp, sz, vp, sz, sz, sz, vp, sz, sz],
 }
 
 
@@ -113,6 +124,8 @@ def check(status: int) -> None:
     msg = lib().dh_last_error().decode("utf-8", "replace")
     if status == DH_ERR_INVALID_ARG:
         raise DaphneHipInvalidArgument(status, msg)
+    if status == DH_ERR_OUT_OF_RANGE:
+        raise DaphneHipOutOfRange(status, msg)
     if status == DH_ERR_DOMAIN:
         raise DaphneHipDomainError(status, msg)
     raise DaphneHipError(status, msg)

@@ -60,6 +60,8 @@ inline void check(dh_status st) {
         throw std::invalid_argument(msg);
     if (st == DH_ERR_DOMAIN)
         throw std::domain_error(msg);
+    if (st == DH_ERR_OUT_OF_RANGE)
+        throw std::out_of_range(msg);
     throw std::runtime_error(msg);
 }
 } // namespace HIP
@@ -191,6 +193,13 @@ DH_OVERLOAD2(dh_affine_forward)
 DH_OVERLOAD2(dh_bias_add)
 DH_OVERLOAD2(dh_batchnorm_inference)
 DH_OVERLOAD2(dh_softmax)
+DH_OVERLOAD2(dh_avgpool_forward)
+DH_OVERLOAD2(dh_relu_forward)
+DH_OVERLOAD2(dh_fill)
+DH_OVERLOAD2(dh_col_bind)
+DH_OVERLOAD2(dh_extract_col)
+DH_OVERLOAD2(dh_transpose)
+DH_OVERLOAD2(dh_gemv)
 #undef DH_OVERLOAD2
 
 // --- EwBinaryMat (kernels/CUDA/EwBinaryMat.h:31-47) ---------------------------------------
@@ -399,21 +408,27 @@ template <class DTRes, class DTArg> struct Forward {
 };
 } // namespace Convolution
 
-// --- NN::Pooling::Forward<MAX> (kernels/CUDA/Pooling.h:31-35) ------------------------------
+// --- NN::Pooling::Forward<MAX | AVG> (kernels/CUDA/Pooling.h:31-35) ------------------------
 namespace NN::Pooling {
 template <typename VT> struct MAX {};
+template <typename VT> struct AVG {};
 template <template <typename> class OP, class DTRes, class DTArg> struct Forward {
     static void apply(DTRes *&res, size_t &res_h, size_t &res_w, const DTArg *data, const size_t batch_size,
                       const size_t num_channels, const size_t img_h, const size_t img_w, const size_t pool_h,
                       const size_t pool_w, const size_t stride_h, const size_t stride_w, const size_t pad_h,
                       const size_t pad_w, DCTX(ctx)) {
         using VT = typename DTRes::VT;
-        static_assert(std::is_same<OP<VT>, MAX<VT>>::value, "only MAX pooling is part of this kernel set");
         const size_t P = (img_h + 2 * pad_h - pool_h) / stride_w + 1, Q = (img_w + 2 * pad_w - pool_w) / stride_h + 1;
         if (res == nullptr)
             res = DataObjectFactory::create<DTRes>(batch_size, num_channels * P * Q, false, ctx);
-        check(dh_maxpool_forward(VT(), detail::raw(ctx), res->getValues(), &res_h, &res_w, data->getValues(), batch_size,
-                                 num_channels, img_h, img_w, pool_h, pool_w, stride_h, stride_w, pad_h, pad_w));
+        if constexpr (std::is_same<OP<VT>, MAX<VT>>::value)
+            check(dh_maxpool_forward(VT(), detail::raw(ctx), res->getValues(), &res_h, &res_w, data->getValues(),
+                                     batch_size, num_channels, img_h, img_w, pool_h, pool_w, stride_h, stride_w, pad_h,
+                                     pad_w));
+        else
+            check(dh_avgpool_forward(VT(), detail::raw(ctx), res->getValues(), &res_h, &res_w, data->getValues(),
+                                     batch_size, num_channels, img_h, img_w, pool_h, pool_w, stride_h, stride_w, pad_h,
+                                     pad_w));
     }
 };
 } // namespace NN::Pooling
@@ -470,5 +485,96 @@ template <class DTRes, class DTArg> struct Softmax {
                          data->getNumRows(), data->getNumCols(), data->getRowSkip()));
     }
 };
+
+// --- NN::Activation::Forward<ReLU> (kernels/CUDA/Activation.h:24-33) -----------------------
+namespace NN::Activation {
+struct ReLU {};
+template <typename OP, typename DTRes, typename DTArg> struct Forward {
+    static void apply(DTRes *&res, const DTArg *data, DCTX(ctx)) {
+        using VT = typename DTRes::VT;
+        static_assert(std::is_same<OP, ReLU>::value, "ReLU is the only activation of the reference's kernel library");
+        if (res == nullptr)
+            res = DataObjectFactory::create<DTRes>(data->getNumRows(), data->getNumCols(), false, ctx);
+        check(dh_relu_forward(VT(), detail::raw(ctx), res->getValues(), res->getRowSkip(), data->getValues(),
+                              data->getNumRows(), data->getNumCols(), data->getRowSkip()));
+    }
+};
+} // namespace NN::Activation
+
+// --- Fill (kernels/CUDA/Fill.h:30-47) --------------------------------------------------------
+template <class DTRes, typename VTArg> struct Fill {
+    static void apply(DTRes *&res, VTArg arg, size_t numRows, size_t numCols, DCTX(ctx)) {
+        using VT = typename DTRes::VT;
+        if (res == nullptr)
+            res = DataObjectFactory::create<DTRes>(numRows, numCols, false, ctx);
+        check(dh_fill(VT(), detail::raw(ctx), res->getValues(), res->getRowSkip(), static_cast<VT>(arg), numRows, numCols));
+    }
+};
+template <class DTRes, typename VTArg> void fill(DTRes *&res, VTArg arg, size_t numRows, size_t numCols, DCTX(ctx)) {
+    Fill<DTRes, VTArg>::apply(res, arg, numRows, numCols, ctx);
+}
+
+// --- ColBind (kernels/CUDA/ColBind.h:26-44) --------------------------------------------------
+template <class DTRes, class DTLhs, class DTRhs> struct ColBind {
+    static void apply(DTRes *&res, const DTLhs *lhs, const DTRhs *rhs, DCTX(ctx)) {
+        using VT = typename DTRes::VT;
+        if (lhs->getNumRows() != rhs->getNumRows())
+            throw std::runtime_error("ColBind - the two operands must have the same number of rows, but lhs has " +
+                                     std::to_string(lhs->getNumRows()) + " and rhs has " +
+                                     std::to_string(rhs->getNumRows()) + " rows");
+        if (res == nullptr)
+            res = DataObjectFactory::create<DTRes>(lhs->getNumRows(), lhs->getNumCols() + rhs->getNumCols(), false, ctx);
+        check(dh_col_bind(VT(), detail::raw(ctx), res->getValues(), res->getRowSkip(), lhs->getValues(), lhs->getNumRows(),
+                          lhs->getNumCols(), lhs->getRowSkip(), rhs->getValues(), rhs->getNumRows(), rhs->getNumCols(),
+                          rhs->getRowSkip()));
+    }
+};
+template <class DTRes, class DTLhs, class DTRhs> void colBind(DTRes *&res, const DTLhs *lhs, const DTRhs *rhs, DCTX(ctx)) {
+    ColBind<DTRes, DTLhs, DTRhs>::apply(res, lhs, rhs, ctx);
+}
+
+// --- ExtractCol (kernels/CUDA/ExtractCol.h:26-45); positions as DenseMatrix<int64_t> -------
+template <class DTRes, class DTArg, class DTSel> struct ExtractCol {
+    static void apply(DTRes *&res, const DTArg *arg, const DTSel *sel, DCTX(ctx)) {
+        using VT = typename DTRes::VT;
+        static_assert(std::is_same<typename DTSel::VT, int64_t>::value, "column positions are int64_t");
+        if (res == nullptr)
+            res = DataObjectFactory::create<DTRes>(arg->getNumRows(), sel->getNumRows(), false, ctx);
+        check(dh_extract_col(VT(), detail::raw(ctx), res->getValues(), res->getRowSkip(), arg->getValues(),
+                             arg->getNumRows(), arg->getNumCols(), arg->getRowSkip(), sel->getValues(), sel->getNumRows(),
+                             sel->getNumCols(), sel->getRowSkip()));
+    }
+};
+template <class DTRes, class DTArg, class DTSel> void extractCol(DTRes *&res, const DTArg *arg, const DTSel *sel, DCTX(ctx)) {
+    ExtractCol<DTRes, DTArg, DTSel>::apply(res, arg, sel, ctx);
+}
+
+// --- Transpose (kernels/CUDA/Transpose.h:33-47) ----------------------------------------------
+template <class DTRes, class DTArg> struct Transpose {
+    static void apply(DTRes *&res, const DTArg *arg, DCTX(ctx)) {
+        using VT = typename DTRes::VT;
+        if (res == nullptr)
+            res = DataObjectFactory::create<DTRes>(arg->getNumCols(), arg->getNumRows(), false, ctx);
+        check(dh_transpose(VT(), detail::raw(ctx), res->getValues(), res->getRowSkip(), arg->getValues(),
+                           arg->getNumRows(), arg->getNumCols(), arg->getRowSkip()));
+    }
+};
+template <class DTRes, class DTArg> void transpose(DTRes *&res, const DTArg *arg, DCTX(ctx)) {
+    Transpose<DTRes, DTArg>::apply(res, arg, ctx);
+}
+
+// --- Gemv (kernels/CUDA/Gemv.h:34-48): res = t(mat) * vec ------------------------------------
+template <class DTRes, class DTMat, class DTVec> struct Gemv {
+    static void apply(DTRes *&res, const DTMat *mat, const DTVec *vec, DCTX(ctx)) {
+        using VT = typename DTRes::VT;
+        if (res == nullptr)
+            res = DataObjectFactory::create<DTRes>(mat->getNumCols(), 1, false, ctx);
+        check(dh_gemv(VT(), detail::raw(ctx), res->getValues(), res->getRowSkip(), mat->getValues(), mat->getNumRows(),
+                      mat->getNumCols(), mat->getRowSkip(), vec->getValues(), vec->getNumRows(), vec->getRowSkip()));
+    }
+};
+template <class DTRes, class DTMat, class DTVec> void gemv(DTRes *&res, const DTMat *mat, const DTVec *vec, DCTX(ctx)) {
+    Gemv<DTRes, DTMat, DTVec>::apply(res, mat, vec, ctx);
+}
 
 } // namespace HIP

@@ -34,3 +34,10 @@ extern "C" dh_status dh_softmax_f64(dh_ctx *ctx, double *res, size_t ld_res, con
                                    size_t ld) {
     return dh_dnn::softmax<double>(ctx, res, ld_res, arg, rows, cols, ld);
 }
+
+extern "C" dh_status dh_avgpool_forward_f64(dh_ctx *ctx, double *res, size_t *res_h, size_t *res_w, const double *data,
+                                             size_t batch, size_t channels, size_t img_h, size_t img_w, size_t pool_h,
+                                             size_t pool_w, size_t stride_h, size_t stride_w, size_t pad_h, size_t pad_w) {
+    return dh_dnn::avgpool_forward<double>(ctx, res, res_h, res_w, data, batch, channels, img_h, img_w, pool_h, pool_w, stride_h,
+                                       stride_w, pad_h, pad_w);
+}

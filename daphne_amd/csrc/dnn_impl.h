@@ -492,6 +492,89 @@ dh_status maxpool_forward(dh_ctx *ctx, T *res, size_t *res_h, size_t *res_w, con
 }
 
 // ---------------------------------------------------------------------------------------
+// AvgPool forward with the CPU kernel's arithmetic (Pooling.cpp:28-107, Pooling.h:33-44): per window
+// row the values are summed left to right, the row sum is scaled by 1 / (pool_h * pool_w) - the full
+// window, padding included - and added to the running result, rounding after each step.
+// ---------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void avgpool_kernel(T *res, const T *data, size_t total, unsigned H, unsigned W,
+                                                      unsigned P, unsigned Q, unsigned ph, unsigned pw, unsigned sh,
+                                                      unsigned sw, unsigned padh, unsigned padw, T plen, int quick) {
+#pragma clang fp contract(off)
+    const size_t idx = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (idx >= total)
+        return;
+    const unsigned PQ = P * Q, HW = H * W;
+    size_t plane;
+    unsigned pq;
+    if (total <= 0xffffffffull) {
+        plane = static_cast<unsigned>(idx) / PQ;
+        pq = static_cast<unsigned>(idx) % PQ;
+    } else {
+        plane = idx / PQ;
+        pq = static_cast<unsigned>(idx % PQ);
+    }
+    const unsigned p = pq / Q, q = pq % Q;
+    const T *in = data + plane * HW;
+    int y0, y1, x0, x1;
+    if (quick) {
+        // Pooling.cpp:57-66: one output per plane of a one-column image: the first min(pool_h, H) values
+        y0 = 0;
+        y1 = static_cast<int>(ph < H ? ph : H);
+        x0 = 0;
+        x1 = 1;
+    } else {
+        const int y_lo = static_cast<int>(p * sh) - static_cast<int>(padh);
+        const int x_lo = static_cast<int>(q * sw) - static_cast<int>(padw);
+        y0 = y_lo < 0 ? 0 : y_lo;
+        x0 = x_lo < 0 ? 0 : x_lo;
+        y1 = y_lo + static_cast<int>(ph);
+        x1 = x_lo + static_cast<int>(pw);
+        if (y1 > static_cast<int>(H))
+            y1 = H;
+        if (x1 > static_cast<int>(W))
+            x1 = W;
+    }
+    T acc = T(0);
+    for (int y = y0; y < y1; y++) {
+        T s = T(0);
+        for (int x = x0; x < x1; x++)
+            s = s + in[static_cast<unsigned>(y) * W + static_cast<unsigned>(x)];
+        const T scaled = s * plen;
+        acc = scaled + acc;
+    }
+    res[idx] = acc;
+}
+
+template <typename T>
+dh_status avgpool_forward(dh_ctx *ctx, T *res, size_t *res_h, size_t *res_w, const T *data, size_t N, size_t C,
+                          size_t H, size_t W, size_t ph, size_t pw, size_t sh, size_t sw, size_t padh, size_t padw) {
+    DH_REQUIRE_CTX(ctx);
+    if (sh == 0 || sw == 0 || ph == 0 || pw == 0 || H + 2 * padh < ph || W + 2 * padw < pw)
+        return dh_fail(DH_ERR_INVALID_ARG, "Pooling: window %zux%zu does not fit the padded image %zux%zu", ph, pw,
+                       H + 2 * padh, W + 2 * padw);
+    // Pooling.cpp:38-39: P is derived with stride_w and Q with stride_h.
+    const size_t P = (H + 2 * padh - ph) / sw + 1, Q = (W + 2 * padw - pw) / sh + 1;
+    if (res_h)
+        *res_h = P;
+    if (res_w)
+        *res_w = Q;
+    const size_t total = N * C * P * Q;
+    if (total == 0)
+        return DH_OK;
+    if (H * W >= (size_t(1) << 31) || P * Q >= (size_t(1) << 31) || dh_ceil_div(total, 256) >= (size_t(1) << 31))
+        return dh_fail(DH_ERR_RUNTIME, "Pooling: image extents exceed 2^31 elements");
+    const T plen = T(1) / static_cast<T>(pw * ph); // Pooling.cpp:50
+    hipLaunchKernelGGL((avgpool_kernel<T>), dim3(static_cast<unsigned>(dh_ceil_div(total, 256))), dim3(256), 0, ctx->stream,
+                       res, data, total, static_cast<unsigned>(H), static_cast<unsigned>(W), static_cast<unsigned>(P),
+                       static_cast<unsigned>(Q), static_cast<unsigned>(ph), static_cast<unsigned>(pw),
+                       static_cast<unsigned>(sh), static_cast<unsigned>(sw), static_cast<unsigned>(padh),
+                       static_cast<unsigned>(padw), plen, (P == 1 && Q == 1 && W == 1) ? 1 : 0);
+    DH_CHECK_LAUNCH();
+    return DH_OK;
+}
+
+// ---------------------------------------------------------------------------------------
 // Per-channel streaming ops: BiasAdd and BatchNorm inference. The matrix is viewed as
 // (rows * C) x HW: every view row has one channel, so the statistics are fetched once per row.
 // ---------------------------------------------------------------------------------------

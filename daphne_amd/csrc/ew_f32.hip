@@ -17,3 +17,10 @@ extern "C" dh_status dh_ew_unary_f32(dh_ctx *ctx, int op, float *res, size_t ld_
                                     size_t cols, size_t ld_arg) {
     return dh_ew::ew_unary<float>(ctx, op, res, ld_res, arg, rows, cols, ld_arg);
 }
+
+// CUDA::NN::Activation::Forward<ReLU,...>::apply (kernels/CUDA/Activation.cpp:21-47): max(0, x) with NaN
+// passed through, which is std::max(x, 0) of the elementwise MAX.
+extern "C" dh_status dh_relu_forward_f32(dh_ctx *ctx, float *res, size_t ld_res, const float *data, size_t rows, size_t cols,
+                                          size_t ld_data) {
+    return dh_ew::ew_binary_sca<float>(ctx, DH_BIN_MAX, res, ld_res, data, rows, cols, ld_data, float(0));
+}

@@ -17,3 +17,10 @@ extern "C" dh_status dh_ew_unary_f64(dh_ctx *ctx, int op, double *res, size_t ld
                                     size_t cols, size_t ld_arg) {
     return dh_ew::ew_unary<double>(ctx, op, res, ld_res, arg, rows, cols, ld_arg);
 }
+
+// CUDA::NN::Activation::Forward<ReLU,...>::apply (kernels/CUDA/Activation.cpp:21-47): max(0, x) with NaN
+// passed through, which is std::max(x, 0) of the elementwise MAX.
+extern "C" dh_status dh_relu_forward_f64(dh_ctx *ctx, double *res, size_t ld_res, const double *data, size_t rows, size_t cols,
+                                          size_t ld_data) {
+    return dh_ew::ew_binary_sca<double>(ctx, DH_BIN_MAX, res, ld_res, data, rows, cols, ld_data, double(0));
+}

@@ -19,3 +19,15 @@ extern "C" dh_status dh_affine_forward_f64(dh_ctx *ctx, double *res, const doubl
     return dh_gemm::affine<double>(ctx, res, data, data_rows, data_cols, weights, w_rows, w_cols, bias, bias_rows,
                                bias_cols);
 }
+
+// Gemv<DenseMatrix<T>,...>::apply (kernels/Gemv.h:51-77, kernels/CUDA/Gemv.cpp:42-68): res = t(mat) vec.
+extern "C" dh_status dh_gemv_f64(dh_ctx *ctx, double *res, size_t ld_res, const double *mat, size_t rows, size_t cols, size_t ld_mat,
+                                  const double *vec, size_t vec_rows, size_t ld_vec) {
+    DH_REQUIRE_CTX(ctx);
+    if (vec_rows != rows)
+        return dh_fail(DH_ERR_RUNTIME, "Gemv - #rows of mat and #rows of vec must be the same, but got %zu and %zu", rows,
+                       vec_rows);
+    if (ld_mat < cols || ld_res < 1 || ld_vec < 1)
+        return dh_fail(DH_ERR_RUNTIME, "Gemv - a leading dimension is smaller than its column count");
+    return dh_gemm::gemv<double>(ctx, true, rows, cols, mat, ld_mat, vec, ld_vec, res, ld_res);
+}

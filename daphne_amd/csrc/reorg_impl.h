@@ -1,0 +1,230 @@
+// Data reorganisation kernels for DenseMatrix<float|double>: Fill, ColBind, ExtractCol, Transpose.
+// They stand in for kernels/CUDA/{Fill.cu,ColBind.cu,ExtractCol.cu,Transpose.cpp} of the reference
+// (paths relative to src/runtime/local/) with the argument checks of the CPU kernels
+// (kernels/ColBind.h:58-91, kernels/ExtractCol.h:57-114, kernels/Transpose.h:51-76), and all take
+// leading dimensions so that views work. Instantiated per value type by reorg_f32.hip / reorg_f64.hip.
+//
+// All four are pure HBM traffic; each thread moves one 16-byte vector where pointers and leading
+// dimensions allow it, a scalar otherwise, in one-shot grids (no grid-stride loops).
+#pragma once
+
+#include "common.h"
+
+namespace dh_reorg {
+
+// dst[r][c] = src ? src[r][c] : value, for a cols-wide block (cols counted in vectors of VEC)
+template <typename T, int VEC, bool FILL>
+__global__ __launch_bounds__(256) void block2d_kernel(T *dst, size_t ld_dst, const T *src, size_t ld_src, size_t rows,
+                                                      size_t cvecs, T value) {
+    const size_t cv = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    const size_t r = static_cast<size_t>(blockIdx.y) * blockDim.y + threadIdx.y;
+    if (cv >= cvecs || r >= rows)
+        return;
+    T v[VEC];
+    if constexpr (FILL) {
+#pragma unroll
+        for (int i = 0; i < VEC; i++)
+            v[i] = value;
+    } else {
+        dh_load_vec_stream<T, VEC>(src + r * ld_src + cv * VEC, v);
+    }
+    dh_store_vec<T, VEC>(dst + r * ld_dst + cv * VEC, v);
+}
+
+template <typename T, bool FILL>
+static inline dh_status block2d(dh_ctx *ctx, T *dst, size_t ld_dst, const T *src, size_t ld_src, size_t rows, size_t cols,
+                                T value) {
+    if (rows == 0 || cols == 0)
+        return DH_OK;
+    constexpr int V = 16 / sizeof(T);
+    // a contiguous block is one long row: keeps narrow matrices on full-width vectors
+    if (ld_dst == cols && (FILL || ld_src == cols)) {
+        const size_t total = rows * cols;
+        size_t w = 256 * V;
+        while (w > 1 && total % w)
+            w >>= 1;
+        if (w >= static_cast<size_t>(V)) {
+            cols = w;
+            rows = total / w;
+            ld_dst = w;
+            ld_src = w;
+        }
+    }
+    const bool vec = cols % V == 0 && ld_dst % V == 0 && dh_aligned(dst, 16) && (FILL || (ld_src % V == 0 && dh_aligned(src, 16)));
+    const size_t cvecs = vec ? cols / V : cols;
+    unsigned tx = 1;
+    while (tx < 256 && tx < cvecs)
+        tx <<= 1;
+    const unsigned ty = 256 / tx;
+    const size_t gx = dh_ceil_div(cvecs, tx), gy = dh_ceil_div(rows, ty);
+    if (gx >= (size_t(1) << 31) || gy >= 65536) {
+        // very tall blocks: rows go to grid.x in slices of 65535 * ty rows
+        const size_t slice = static_cast<size_t>(65535) * ty;
+        for (size_t r0 = 0; r0 < rows; r0 += slice) {
+            const size_t nr = rows - r0 < slice ? rows - r0 : slice;
+            dh_status st = block2d<T, FILL>(ctx, dst + r0 * ld_dst, ld_dst, FILL ? nullptr : src + r0 * ld_src, ld_src, nr,
+                                            cols, value);
+            if (st != DH_OK)
+                return st;
+        }
+        return DH_OK;
+    }
+    const dim3 grid(static_cast<unsigned>(gx), static_cast<unsigned>(gy)), block(tx, ty);
+    if (vec)
+        hipLaunchKernelGGL((block2d_kernel<T, V, FILL>), grid, block, 0, ctx->stream, dst, ld_dst, src, ld_src, rows, cvecs,
+                           value);
+    else
+        hipLaunchKernelGGL((block2d_kernel<T, 1, FILL>), grid, block, 0, ctx->stream, dst, ld_dst, src, ld_src, rows, cvecs,
+                           value);
+    DH_CHECK_LAUNCH();
+    return DH_OK;
+}
+
+// Fill<DenseMatrix<VT>,VT>::apply (kernels/CUDA/Fill.cu:27-49)
+template <typename T> dh_status fill(dh_ctx *ctx, T *res, size_t ld_res, T value, size_t rows, size_t cols) {
+    DH_REQUIRE_CTX(ctx);
+    if (ld_res < cols)
+        return dh_fail(DH_ERR_RUNTIME, "Fill - leading dimension smaller than the column count");
+    return block2d<T, true>(ctx, res, ld_res, nullptr, 0, rows, cols, value);
+}
+
+// ColBind<DenseMatrix<VT>,...>::apply (kernels/ColBind.h:58-91, kernels/CUDA/ColBind.cu:47-70)
+template <typename T>
+dh_status col_bind(dh_ctx *ctx, T *res, size_t ld_res, const T *lhs, size_t lr, size_t lc, size_t ld_lhs, const T *rhs,
+                   size_t rr, size_t rc, size_t ld_rhs) {
+    DH_REQUIRE_CTX(ctx);
+    if (lr != rr)
+        return dh_fail(DH_ERR_RUNTIME,
+                       "ColBind - the two operands must have the same number of rows, but lhs has %zu and rhs has %zu rows",
+                       lr, rr);
+    if (ld_res < lc + rc || ld_lhs < lc || ld_rhs < rc)
+        return dh_fail(DH_ERR_RUNTIME, "ColBind - a leading dimension is smaller than its column count");
+    dh_status st = block2d<T, false>(ctx, res, ld_res, lhs, ld_lhs, lr, lc, T(0));
+    if (st != DH_OK)
+        return st;
+    return block2d<T, false>(ctx, res + lc, ld_res, rhs, ld_rhs, lr, rc, T(0));
+}
+
+// Column positions: negative ones count from the end (kernels/ExtractCol.h:98-101); the first position
+// that is still out of range is reported through the flag as index + 1.
+static __global__ void check_sel_kernel(const long long *sel, size_t nsel, size_t ld_sel, size_t cols, int *flag) {
+    for (size_t k = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; k < nsel;
+         k += static_cast<size_t>(gridDim.x) * blockDim.x) {
+        long long v = sel[k * ld_sel];
+        if (v < 0)
+            v += static_cast<long long>(cols);
+        if (v < 0 || static_cast<unsigned long long>(v) >= cols)
+            atomicMin(flag, static_cast<int>(k < 0x7ffffffe ? k + 1 : 0x7fffffff));
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void extract_col_kernel(T *res, size_t ld_res, const T *arg, size_t ld, size_t rows,
+                                                          size_t cols, const long long *sel, size_t nsel, size_t ld_sel) {
+    const size_t k = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    const size_t r = static_cast<size_t>(blockIdx.y) * blockDim.y + threadIdx.y;
+    if (k >= nsel || r >= rows)
+        return;
+    long long c = sel[k * ld_sel];
+    if (c < 0)
+        c += static_cast<long long>(cols);
+    res[r * ld_res + k] = arg[r * ld + static_cast<size_t>(c)];
+}
+
+// ExtractCol<DenseMatrix<VT>,DenseMatrix<VT>,DenseMatrix<int64_t>>::apply
+// (kernels/ExtractCol.h:74-114, kernels/CUDA/ExtractCol.cu:21-56)
+template <typename T>
+dh_status extract_col(dh_ctx *ctx, T *res, size_t ld_res, const T *arg, size_t rows, size_t cols, size_t ld,
+                      const long long *sel, size_t sel_rows, size_t sel_cols, size_t ld_sel) {
+    DH_REQUIRE_CTX(ctx);
+    if (sel_cols != 1)
+        return dh_fail(DH_ERR_RUNTIME,
+                       "invalid argument passed to ExtractCol: column selection must be given as column matrix but has "
+                       "'%zu' columns instead of one",
+                       sel_cols);
+    if (ld < cols || ld_res < sel_rows || ld_sel < 1)
+        return dh_fail(DH_ERR_RUNTIME, "ExtractCol - a leading dimension is smaller than its column count");
+    if (sel_rows == 0 || rows == 0)
+        return DH_OK;
+    // validate the positions first: the CPU kernel throws before anything is usable
+    *ctx->flag_host = 0x7fffffff;
+    DH_CHECK_HIP(hipMemcpyAsync(ctx->flag_dev, ctx->flag_host, sizeof(int), hipMemcpyHostToDevice, ctx->stream));
+    size_t cg = dh_ceil_div(sel_rows, 256);
+    if (cg > 1024)
+        cg = 1024;
+    hipLaunchKernelGGL(check_sel_kernel, dim3(static_cast<unsigned>(cg)), dim3(256), 0, ctx->stream, sel, sel_rows, ld_sel,
+                       cols, ctx->flag_dev);
+    DH_CHECK_LAUNCH();
+    DH_CHECK_HIP(hipMemcpyAsync(ctx->flag_host, ctx->flag_dev, sizeof(int), hipMemcpyDeviceToHost, ctx->stream));
+    DH_CHECK_HIP(hipStreamSynchronize(ctx->stream));
+    if (*ctx->flag_host != 0x7fffffff) {
+        const size_t bad = static_cast<size_t>(*ctx->flag_host) - 1;
+        long long v = 0;
+        DH_CHECK_HIP(hipMemcpy(&v, sel + bad * ld_sel, sizeof(v), hipMemcpyDeviceToHost));
+        return dh_fail(DH_ERR_OUT_OF_RANGE,
+                       "invalid argument '%lld' passed to ExtractCol: out of bounds for dense matrix with column "
+                       "boundaries '[0, %zu)'",
+                       v, cols);
+    }
+    unsigned tx = 1;
+    while (tx < 256 && tx < sel_rows)
+        tx <<= 1;
+    const unsigned ty = 256 / tx;
+    const size_t gx = dh_ceil_div(sel_rows, tx);
+    const size_t slice = static_cast<size_t>(65535) * ty;
+    for (size_t r0 = 0; r0 < rows; r0 += slice) {
+        const size_t nr = rows - r0 < slice ? rows - r0 : slice;
+        hipLaunchKernelGGL((extract_col_kernel<T>), dim3(static_cast<unsigned>(gx), static_cast<unsigned>(dh_ceil_div(nr, ty))),
+                           dim3(tx, ty), 0, ctx->stream, res + r0 * ld_res, ld_res, arg + r0 * ld, ld, nr, cols, sel, sel_rows,
+                           ld_sel);
+        DH_CHECK_LAUNCH();
+    }
+    return DH_OK;
+}
+
+// 64 x 64 tile through LDS: rows are read along columns of the source and written along columns of the
+// result, both as contiguous 256-byte runs per wavefront; the odd LDS stride keeps the transposed read
+// free of bank conflicts.
+template <typename T>
+__global__ __launch_bounds__(256) void transpose_kernel(T *res, size_t ld_res, const T *arg, size_t ld, size_t rows,
+                                                        size_t cols) {
+    constexpr int TS = 64;
+    __shared__ T tile[TS][TS + 1];
+    const int tx = threadIdx.x % TS, ty = threadIdx.x / TS; // 64 x 4
+    const size_t r0 = static_cast<size_t>(blockIdx.y) * TS, c0 = static_cast<size_t>(blockIdx.x) * TS;
+#pragma unroll
+    for (int i = 0; i < TS; i += 4) {
+        const size_t r = r0 + ty + i, c = c0 + tx;
+        if (r < rows && c < cols)
+            tile[ty + i][tx] = arg[r * ld + c];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < TS; i += 4) {
+        const size_t orow = c0 + ty + i, ocol = r0 + tx; // result is cols x rows
+        if (orow < cols && ocol < rows)
+            res[orow * ld_res + ocol] = tile[tx][ty + i];
+    }
+}
+
+// Transpose<DenseMatrix<VT>,DenseMatrix<VT>>::apply (kernels/Transpose.h:51-76, kernels/CUDA/Transpose.cpp)
+template <typename T> dh_status transpose(dh_ctx *ctx, T *res, size_t ld_res, const T *arg, size_t rows, size_t cols, size_t ld) {
+    DH_REQUIRE_CTX(ctx);
+    if (ld < cols || ld_res < rows)
+        return dh_fail(DH_ERR_RUNTIME, "Transpose - a leading dimension is smaller than its column count");
+    if (rows == 0 || cols == 0)
+        return DH_OK;
+    const size_t gx = dh_ceil_div(cols, 64);
+    if (gx >= (size_t(1) << 31))
+        return dh_fail(DH_ERR_RUNTIME, "Transpose - too many columns for one launch");
+    const size_t slice = static_cast<size_t>(65535) * 64;
+    for (size_t r0 = 0; r0 < rows; r0 += slice) {
+        const size_t nr = rows - r0 < slice ? rows - r0 : slice;
+        hipLaunchKernelGGL((transpose_kernel<T>), dim3(static_cast<unsigned>(gx), static_cast<unsigned>(dh_ceil_div(nr, 64))),
+                           dim3(256), 0, ctx->stream, res + r0, ld_res, arg + r0 * ld, ld, nr, cols);
+        DH_CHECK_LAUNCH();
+    }
+    return DH_OK;
+}
+
+} // namespace dh_reorg

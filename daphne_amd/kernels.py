@@ -386,3 +386,76 @@ def softmax(res, arg: DenseMatrix, ctx: HIPContext) -> DenseMatrix:
         res = DenseMatrix(ctx, arg.rows, arg.cols, arg.dtype)
     capi.check(_fn("dh_softmax", arg.dtype)(ctx._h, res.ptr, res.row_skip, arg.ptr, arg.rows, arg.cols, arg.row_skip))
     return res
+
+
+def avgPoolForward(res, data: DenseMatrix, batch_size, num_channels, img_h, img_w, pool_h, pool_w, stride_h,
+                   stride_w, pad_h, pad_w, ctx: HIPContext):
+    """CUDA::NN::Pooling::Forward<AVG>::apply (kernels/CUDA/Pooling.h:31-35; CPU kernels/AvgPoolForward.h,
+    Pooling.cpp:28-107). Returns (res, res_h, res_w)."""
+    dt = data.dtype
+    P = (img_h + 2 * pad_h - pool_h) // stride_w + 1 if img_h + 2 * pad_h >= pool_h else 0
+    Q = (img_w + 2 * pad_w - pool_w) // stride_h + 1 if img_w + 2 * pad_w >= pool_w else 0
+    if res is None:
+        res = DenseMatrix(ctx, batch_size, num_channels * P * Q, dt)
+    rh, rw = C.c_size_t(), C.c_size_t()
+    capi.check(_fn("dh_avgpool_forward", dt)(ctx._h, res.ptr, C.byref(rh), C.byref(rw), data.ptr, batch_size,
+                                             num_channels, img_h, img_w, pool_h, pool_w, stride_h, stride_w, pad_h,
+                                             pad_w))
+    return res, rh.value, rw.value
+
+
+def reluForward(res, data: DenseMatrix, ctx: HIPContext) -> DenseMatrix:
+    """CUDA::NN::Activation::Forward<ReLU>::apply (kernels/CUDA/Activation.h:24-33)."""
+    if res is None:
+        res = DenseMatrix(ctx, data.rows, data.cols, data.dtype)
+    capi.check(_fn("dh_relu_forward", data.dtype)(ctx._h, res.ptr, res.row_skip, data.ptr, data.rows, data.cols,
+                                                  data.row_skip))
+    return res
+
+
+def fill(res, arg, numRows: int, numCols: int, ctx: HIPContext, dtype=np.float64) -> DenseMatrix:
+    """CUDA::Fill::apply (kernels/CUDA/Fill.h:30-47)."""
+    if res is None:
+        res = DenseMatrix(ctx, numRows, numCols, dtype)
+    capi.check(_fn("dh_fill", res.dtype)(ctx._h, res.ptr, res.row_skip, arg, numRows, numCols))
+    return res
+
+
+def colBind(res, lhs: DenseMatrix, rhs: DenseMatrix, ctx: HIPContext) -> DenseMatrix:
+    """CUDA::ColBind::apply (kernels/CUDA/ColBind.h:26-34; CPU kernels/ColBind.h:58-91)."""
+    dt = _same_dtype(lhs, rhs, res)
+    if res is None:
+        res = DenseMatrix(ctx, lhs.rows, lhs.cols + rhs.cols, dt)
+    capi.check(_fn("dh_col_bind", dt)(ctx._h, res.ptr, res.row_skip, lhs.ptr, lhs.rows, lhs.cols, lhs.row_skip, rhs.ptr,
+                                      rhs.rows, rhs.cols, rhs.row_skip))
+    return res
+
+
+def extractCol(res, arg: DenseMatrix, sel: DenseMatrix, ctx: HIPContext) -> DenseMatrix:
+    """CUDA::ExtractCol::apply (kernels/CUDA/ExtractCol.h:26-35; CPU kernels/ExtractCol.h:74-114). `sel` is an
+    int64 column of positions."""
+    if sel.dtype != np.dtype(np.int64):
+        raise TypeError("extractCol: positions must be int64")
+    if res is None:
+        res = DenseMatrix(ctx, arg.rows, sel.rows, arg.dtype)
+    capi.check(_fn("dh_extract_col", arg.dtype)(ctx._h, res.ptr, res.row_skip, arg.ptr, arg.rows, arg.cols, arg.row_skip,
+                                                sel.ptr, sel.rows, sel.cols, sel.row_skip))
+    return res
+
+
+def transpose(res, arg: DenseMatrix, ctx: HIPContext) -> DenseMatrix:
+    """CUDA::Transpose::apply (kernels/CUDA/Transpose.h:33-39; CPU kernels/Transpose.h:51-76)."""
+    if res is None:
+        res = DenseMatrix(ctx, arg.cols, arg.rows, arg.dtype)
+    capi.check(_fn("dh_transpose", arg.dtype)(ctx._h, res.ptr, res.row_skip, arg.ptr, arg.rows, arg.cols, arg.row_skip))
+    return res
+
+
+def gemv(res, mat: DenseMatrix, vec: DenseMatrix, ctx: HIPContext) -> DenseMatrix:
+    """CUDA::Gemv::apply (kernels/CUDA/Gemv.h:34-40; CPU kernels/Gemv.h:51-77): res = t(mat) @ vec."""
+    dt = _same_dtype(mat, vec, res)
+    if res is None:
+        res = DenseMatrix(ctx, mat.cols, 1, dt)
+    capi.check(_fn("dh_gemv", dt)(ctx._h, res.ptr, res.row_skip, mat.ptr, mat.rows, mat.cols, mat.row_skip, vec.ptr,
+                                  vec.rows, vec.row_skip))
+    return res

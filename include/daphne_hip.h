@@ -35,7 +35,8 @@ typedef enum dh_status {
     DH_ERR_INVALID_ARG = 2,  /* std::invalid_argument: e.g. conv filter larger than image    */
     DH_ERR_DOMAIN = 3,       /* std::domain_error: sqrt/ln/asin/acos outside their domain    */
     DH_ERR_HIP = 4,          /* std::runtime_error carrying the HIP error string             */
-    DH_ERR_OOM = 5           /* std::runtime_error: device allocation beyond the budget      */
+    DH_ERR_OOM = 5,          /* std::runtime_error: device allocation beyond the budget      */
+    DH_ERR_OUT_OF_RANGE = 6  /* std::out_of_range: ExtractCol position outside the matrix    */
 } dh_status;
 
 /* Thread-local text of the last failure on the calling thread ("" if none). */
@@ -303,6 +304,72 @@ dh_status dh_softmax_f32(dh_ctx *ctx, float *res, size_t ld_res, const float *ar
                          size_t cols, size_t ld);
 dh_status dh_softmax_f64(dh_ctx *ctx, double *res, size_t ld_res, const double *arg, size_t rows,
                          size_t cols, size_t ld);
+
+/* CUDA::NN::Pooling::Forward<AVG,...>::apply (kernels/CUDA/Pooling.h:31-35) with the CPU kernel's
+ * arithmetic (kernels/Pooling.cpp:28-107, Pooling.h:33-44, AvgPoolForward.h): every window row is
+ * summed left to right, scaled by 1 / (pool_h * pool_w) - the full window, zero padding included -
+ * and added to the running result. Output extents as for MAX. */
+dh_status dh_avgpool_forward_f32(dh_ctx *ctx, float *res, size_t *res_h, size_t *res_w,
+                                 const float *data, size_t batch, size_t channels, size_t img_h,
+                                 size_t img_w, size_t pool_h, size_t pool_w, size_t stride_h,
+                                 size_t stride_w, size_t pad_h, size_t pad_w);
+dh_status dh_avgpool_forward_f64(dh_ctx *ctx, double *res, size_t *res_h, size_t *res_w,
+                                 const double *data, size_t batch, size_t channels, size_t img_h,
+                                 size_t img_w, size_t pool_h, size_t pool_w, size_t stride_h,
+                                 size_t stride_w, size_t pad_h, size_t pad_w);
+
+/* CUDA::NN::Activation::Forward<ReLU,DTRes,DTArg>::apply (kernels/CUDA/Activation.h:24-33,
+ * Activation.cpp:21-47: cudnnActivationForward, RELU, NaN propagated): res = max(0, data). */
+dh_status dh_relu_forward_f32(dh_ctx *ctx, float *res, size_t ld_res, const float *data, size_t rows,
+                              size_t cols, size_t ld_data);
+dh_status dh_relu_forward_f64(dh_ctx *ctx, double *res, size_t ld_res, const double *data,
+                              size_t rows, size_t cols, size_t ld_data);
+
+/* ------------------------------------------------------------------------------------ */
+/* data reorganisation                                                                   */
+/* ------------------------------------------------------------------------------------ */
+/* CUDA::Fill<DenseMatrix<VT>,VT>::apply (kernels/CUDA/Fill.h:30-47, Fill.cu:27-49): every element
+ * of the rows x cols result becomes `value`. */
+dh_status dh_fill_f32(dh_ctx *ctx, float *res, size_t ld_res, float value, size_t rows, size_t cols);
+dh_status dh_fill_f64(dh_ctx *ctx, double *res, size_t ld_res, double value, size_t rows, size_t cols);
+
+/* CUDA::ColBind<...>::apply (kernels/CUDA/ColBind.h:26-34, ColBind.cu:47-70): res = [lhs | rhs],
+ * lhs_rows x (lhs_cols + rhs_cols). DH_ERR_RUNTIME if the row counts differ (kernels/ColBind.h:62-67). */
+dh_status dh_col_bind_f32(dh_ctx *ctx, float *res, size_t ld_res, const float *lhs, size_t lhs_rows,
+                          size_t lhs_cols, size_t ld_lhs, const float *rhs, size_t rhs_rows,
+                          size_t rhs_cols, size_t ld_rhs);
+dh_status dh_col_bind_f64(dh_ctx *ctx, double *res, size_t ld_res, const double *lhs, size_t lhs_rows,
+                          size_t lhs_cols, size_t ld_lhs, const double *rhs, size_t rhs_rows,
+                          size_t rhs_cols, size_t ld_rhs);
+
+/* CUDA::ExtractCol<DenseMatrix<VT>,DenseMatrix<VT>,DenseMatrix<int64_t>>::apply
+ * (kernels/CUDA/ExtractCol.h:26-35, ExtractCol.cu:21-56): res[r][k] = arg[r][sel[k]] with sel a
+ * sel_rows x 1 matrix of positions in device memory. As in the CPU kernel
+ * (kernels/ExtractCol.h:57-64,96-108) a negative position counts from the last column,
+ * DH_ERR_RUNTIME if sel has more than one column, DH_ERR_OUT_OF_RANGE for a position outside
+ * [0, cols). Synchronises (the positions are validated before the copy). */
+dh_status dh_extract_col_f32(dh_ctx *ctx, float *res, size_t ld_res, const float *arg, size_t rows,
+                             size_t cols, size_t ld, const int64_t *sel, size_t sel_rows,
+                             size_t sel_cols, size_t ld_sel);
+dh_status dh_extract_col_f64(dh_ctx *ctx, double *res, size_t ld_res, const double *arg, size_t rows,
+                             size_t cols, size_t ld, const int64_t *sel, size_t sel_rows,
+                             size_t sel_cols, size_t ld_sel);
+
+/* CUDA::Transpose<DenseMatrix<VT>,DenseMatrix<VT>>::apply (kernels/CUDA/Transpose.h:33-39,
+ * Transpose.cpp: cublas geam): res (cols x rows) = t(arg). */
+dh_status dh_transpose_f32(dh_ctx *ctx, float *res, size_t ld_res, const float *arg, size_t rows,
+                           size_t cols, size_t ld);
+dh_status dh_transpose_f64(dh_ctx *ctx, double *res, size_t ld_res, const double *arg, size_t rows,
+                           size_t cols, size_t ld);
+
+/* CUDA::Gemv<DenseMatrix<T>,...>::apply (kernels/CUDA/Gemv.h:34-40, Gemv.cpp:42-68; CPU
+ * kernels/Gemv.h:51-77, cblas_?gemv with CblasTrans): res (cols x 1) = t(mat) * vec, vec a
+ * rows x 1 column with row stride ld_vec. */
+dh_status dh_gemv_f32(dh_ctx *ctx, float *res, size_t ld_res, const float *mat, size_t rows, size_t cols,
+                      size_t ld_mat, const float *vec, size_t vec_rows, size_t ld_vec);
+dh_status dh_gemv_f64(dh_ctx *ctx, double *res, size_t ld_res, const double *mat, size_t rows,
+                      size_t cols, size_t ld_mat, const double *vec, size_t vec_rows, size_t ld_vec);
+
 
 
 /* ------------------------------------------------------------------------------------ */

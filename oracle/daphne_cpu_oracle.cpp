@@ -15,7 +15,7 @@
 // evaluations in tests/test_oracle_*.py.
 //
 // Status codes returned by the functions: 0 ok, 1 std::runtime_error, 2 std::invalid_argument,
-// 3 std::domain_error - the exception the reference would have thrown.
+// 3 std::domain_error, 6 std::out_of_range - the exception the reference would have thrown.
 #include <algorithm>
 #include <cmath>
 #include <cstddef>
@@ -656,6 +656,116 @@ template <typename T> int softmax(T *res, size_t ld_res, const T *arg, size_t ro
     return ST_OK;
 }
 
+// Pooling.cpp:28-107 with OP = AVG (Pooling.h:33-44), via AvgPoolForward.h. Each window row is summed
+// left to right from zero, multiplied by plen = 1 / (pool_h * pool_w) (:50, the full window even where it
+// is clipped or padded) and added to the running result. The reference's quick paths (:57-91) apply the
+// same expression to the same values as the padded general path (:92-105), which is restated here; the
+// P==1 && Q==1 && W==1 path (:57-66) sums the first min(pool_h, H) values of the plane.
+template <typename T>
+int avgpool(T *res, size_t *res_h, size_t *res_w, const T *data, size_t N, size_t C, size_t H, size_t W, size_t ph_,
+            size_t pw_, size_t sh, size_t sw, size_t padh, size_t padw) {
+    if (H + 2 * padh < ph_ || W + 2 * padw < pw_ || sh == 0 || sw == 0 || ph_ == 0 || pw_ == 0)
+        return ST_INVALID;
+    const size_t HW = H * W, CHW = C * HW;
+    const size_t P = get_pq(H, ph_, padh, sw), Q = get_pq(W, pw_, padw, sh);
+    const size_t CPQ = C * P * Q;
+    *res_h = P;
+    *res_w = Q;
+    const size_t pH = H + 2 * padh, pW = W + 2 * padw;
+    const T plen = static_cast<T>(1) / static_cast<T>(pw_ * ph_);
+    std::fill(res, res + N * CPQ, T(0));
+    auto run = [plen](T init, const T *in, size_t start, size_t len) {
+        T ret = 0;
+        for (size_t i = start; i < start + len; i++)
+            ret += in[i];
+        return ret * plen + init;
+    };
+    if (P == 1 && Q == 1 && W == 1) {
+        const size_t lenh = std::min(ph_, H);
+        for (size_t i = 0; i < N; i++)
+            for (size_t c = 0; c < C; c++)
+                res[i * C + c] = run(T(0), data, i * CHW + c * H, lenh);
+        return ST_OK;
+    }
+    std::vector<T> padded(pH * pW, T(0));
+    for (size_t i = 0; i < N; i++)
+        for (size_t c = 0; c < C; c++) {
+            const size_t off = i * CHW + c * HW;
+            for (size_t y = 0; y < H; y++)
+                for (size_t x = 0; x < W; x++)
+                    padded[(padh + y) * pW + padw + x] = data[off + y * W + x];
+            T *o = res + i * CPQ + c * P * Q;
+            for (size_t p = 0; p < P; p++)
+                for (size_t h = p * sh; h < std::min(p * sh + ph_, pH); h++)
+                    for (size_t q = 0; q < Q; q++) {
+                        const size_t len = (q * sw < pW) ? std::min(pw_, pW - q * sw) : 0;
+                        o[p * Q + q] = run(o[p * Q + q], padded.data(), h * pW + q * sw, len);
+                    }
+        }
+    return ST_OK;
+}
+
+// CUDA/Activation.cpp:21-47 (cudnnActivationForward, CUDNN_ACTIVATION_RELU, CUDNN_PROPAGATE_NAN): max(0, x),
+// a NaN stays a NaN. There is no CPU kernel; the elementwise MAX with 0 (EwBinarySca.h std::max) gives the same.
+template <typename T> int relu(T *res, size_t ld_res, const T *arg, size_t rows, size_t cols, size_t ld) {
+    for (size_t r = 0; r < rows; r++)
+        for (size_t c = 0; c < cols; c++) {
+            const T x = arg[r * ld + c];
+            res[r * ld_res + c] = (x < T(0)) ? T(0) : x;
+        }
+    return ST_OK;
+}
+
+// Fill.h (CPU) / CUDA/Fill.cu:27-49
+template <typename T> int fill(T *res, size_t ld_res, T value, size_t rows, size_t cols) {
+    for (size_t r = 0; r < rows; r++)
+        for (size_t c = 0; c < cols; c++)
+            res[r * ld_res + c] = value;
+    return ST_OK;
+}
+
+// ColBind.h:58-91
+template <typename T>
+int col_bind(T *res, size_t ld_res, const T *lhs, size_t lr, size_t lc, size_t ld_lhs, const T *rhs, size_t rr, size_t rc,
+             size_t ld_rhs) {
+    if (lr != rr)
+        return ST_RUNTIME;
+    for (size_t r = 0; r < lr; r++) {
+        if (lc)
+            std::memcpy(res + r * ld_res, lhs + r * ld_lhs, lc * sizeof(T));
+        if (rc)
+            std::memcpy(res + r * ld_res + lc, rhs + r * ld_rhs, rc * sizeof(T));
+    }
+    return ST_OK;
+}
+
+// ExtractCol.h:57-114: positions as int64, a negative one counts from the end, anything still outside
+// [0, cols) is std::out_of_range (status 6); more than one selection column is a runtime error.
+template <typename T>
+int extract_col(T *res, size_t ld_res, const T *arg, size_t rows, size_t cols, size_t ld, const int64_t *sel,
+                size_t sel_rows, size_t sel_cols) {
+    if (sel_cols != 1)
+        return ST_RUNTIME;
+    for (size_t r = 0; r < rows; r++)
+        for (size_t c = 0; c < sel_rows; c++) {
+            int64_t idx = sel[c];
+            if (idx < 0)
+                idx += static_cast<int64_t>(cols);
+            if (idx < 0 || cols <= static_cast<size_t>(idx))
+                return 6;
+            res[r * ld_res + c] = arg[r * ld + static_cast<size_t>(idx)];
+        }
+    return ST_OK;
+}
+
+// Transpose.h:51-76
+template <typename T> int transpose(T *res, size_t ld_res, const T *arg, size_t rows, size_t cols, size_t ld) {
+    for (size_t r = 0; r < rows; r++)
+        for (size_t c = 0; c < cols; c++)
+            res[c * ld_res + r] = arg[r * ld + c];
+    return ST_OK;
+}
+
 } // namespace
 
 // ---------------------------------------------------------------------------------------
@@ -721,6 +831,29 @@ template <typename T> int softmax(T *res, size_t ld_res, const T *arg, size_t ro
     }                                                                                                                   \
     extern "C" int oracle_softmax_##SUF(T *res, size_t ld_res, const T *arg, size_t rows, size_t cols, size_t ld) {     \
         return softmax<T>(res, ld_res, arg, rows, cols, ld);                                                            \
+    }                                                                                                                   \
+    extern "C" int oracle_avgpool_forward_##SUF(T *res, size_t *res_h, size_t *res_w, const T *data, size_t N,          \
+                                                size_t C, size_t H, size_t W, size_t ph, size_t pw, size_t sh,          \
+                                                size_t sw, size_t padh, size_t padw) {                                  \
+        return avgpool<T>(res, res_h, res_w, data, N, C, H, W, ph, pw, sh, sw, padh, padw);                             \
+    }                                                                                                                   \
+    extern "C" int oracle_relu_forward_##SUF(T *res, size_t ld_res, const T *arg, size_t rows, size_t cols,             \
+                                             size_t ld) {                                                               \
+        return relu<T>(res, ld_res, arg, rows, cols, ld);                                                               \
+    }                                                                                                                   \
+    extern "C" int oracle_fill_##SUF(T *res, size_t ld_res, T value, size_t rows, size_t cols) {                        \
+        return fill<T>(res, ld_res, value, rows, cols);                                                                 \
+    }                                                                                                                   \
+    extern "C" int oracle_col_bind_##SUF(T *res, size_t ld_res, const T *lhs, size_t lr, size_t lc, size_t ld_lhs,      \
+                                         const T *rhs, size_t rr, size_t rc, size_t ld_rhs) {                           \
+        return col_bind<T>(res, ld_res, lhs, lr, lc, ld_lhs, rhs, rr, rc, ld_rhs);                                      \
+    }                                                                                                                   \
+    extern "C" int oracle_extract_col_##SUF(T *res, size_t ld_res, const T *arg, size_t rows, size_t cols, size_t ld,   \
+                                            const int64_t *sel, size_t sel_rows, size_t sel_cols) {                     \
+        return extract_col<T>(res, ld_res, arg, rows, cols, ld, sel, sel_rows, sel_cols);                               \
+    }                                                                                                                   \
+    extern "C" int oracle_transpose_##SUF(T *res, size_t ld_res, const T *arg, size_t rows, size_t cols, size_t ld) {   \
+        return transpose<T>(res, ld_res, arg, rows, cols, ld);                                                          \
     }
 
 ORACLE_EXPORTS(f32, float)

@@ -2,12 +2,14 @@
 import numpy as np
 
 import oracle_binding as orc
-from golden_cases import DomainError, KernelError
+from golden_cases import DomainError, KernelError, OutOfRange
 
 
 def _st(st):
     if st == orc.ST_DOMAIN:
         raise DomainError()
+    if st == 6:
+        raise OutOfRange(st)
     if st != 0:
         raise KernelError(st)
 
@@ -57,6 +59,21 @@ class OracleBackend:
     def softmax(self, x):
         st, r = orc.softmax(x); _st(st); return r
 
+    def avgpool(self, x, N, C, H, W, ph, pw, sh, sw, padh, padw):
+        st, r, oh, ow = orc.avgpool(x, N, C, H, W, ph, pw, sh, sw, padh, padw); _st(st); return r, oh, ow
+
+    def relu(self, x):
+        st, r = orc.relu(x); _st(st); return r
+
+    def transpose(self, x):
+        st, r = orc.transpose(x); _st(st); return r
+
+    def col_bind(self, a, b):
+        st, r = orc.col_bind(a, b); _st(st); return r
+
+    def extract_col(self, a, sel):
+        st, r = orc.extract_col(a, sel); _st(st); return r
+
     def affine(self, x, w, b):
         st, mm = orc.matmul(x, w); _st(st)
         if b is None:
@@ -79,6 +96,8 @@ class HipBackend:
             return fn(*a)
         except self.capi.DaphneHipDomainError:
             raise DomainError()
+        except self.capi.DaphneHipOutOfRange as e:
+            raise OutOfRange(str(e))
         except self.capi.DaphneHipError as e:
             raise KernelError(str(e))
 
@@ -117,6 +136,23 @@ class HipBackend:
     def maxpool(self, x, N, C, H, W, ph, pw, sh, sw, padh, padw):
         r, oh, ow = self._call(self.k.maxPoolForward, None, self._d(x), N, C, H, W, ph, pw, sh, sw, padh, padw, self.ctx)
         return r.to_numpy(), oh, ow
+
+    def avgpool(self, x, N, C, H, W, ph, pw, sh, sw, padh, padw):
+        r, oh, ow = self._call(self.k.avgPoolForward, None, self._d(x), N, C, H, W, ph, pw, sh, sw, padh, padw, self.ctx)
+        return r.to_numpy(), oh, ow
+
+    def relu(self, x):
+        return self._call(self.k.reluForward, None, self._d(x), self.ctx).to_numpy()
+
+    def transpose(self, x):
+        return self._call(self.k.transpose, None, self._d(x), self.ctx).to_numpy()
+
+    def col_bind(self, a, b):
+        return self._call(self.k.colBind, None, self._d(a), self._d(b), self.ctx).to_numpy()
+
+    def extract_col(self, a, sel):
+        return self._call(self.k.extractCol, None, self._d(a), self._d(np.ascontiguousarray(sel, dtype=np.int64)),
+                          self.ctx).to_numpy()
 
     def bias_add(self, x, b):
         return self._call(self.k.biasAdd, None, self._d(x), self._d(b), self.ctx).to_numpy()

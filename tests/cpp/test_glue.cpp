@@ -200,6 +200,72 @@ template <typename VT> void run_all(DaphneContext *dctx) {
         for (auto *m : {x, b, res, s, sm, in, w, b0, aff, one, zero, bn})
             DataObjectFactory::destroy(m);
     }
+    // TransposeTest.cpp (3x4), ColBindTest.cpp, ExtractColTest.cpp:159-197, CUDA/DNNActivationTest.cpp:34-40,
+    // DNNPoolingTestForward.cpp AVG (first plane of the 2x2 / stride 2 / pad 1 result), FillTest.cpp
+    {
+        auto m = G(3, {1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12});
+        DT *mt = nullptr;
+        HIP::transpose(mt, m, dctx);
+        CHECK(mt->getNumRows() == 4 && mt->getNumCols() == 3);
+        CHECK(equals(mt, {1, 5, 9, 2, 6, 10, 3, 7, 11, 4, 8, 12}));
+        auto m0 = G(3, {1, 2, 3, 4, 5, 6}), m1 = G(3, {10, 20, 30, 40, 50, 60, 70, 80, 90});
+        DT *cb = nullptr;
+        HIP::colBind(cb, m0, m1, dctx);
+        CHECK(equals(cb, {1, 2, 10, 20, 30, 3, 4, 40, 50, 60, 5, 6, 70, 80, 90}));
+        bool threw = false;
+        try {
+            DT *bad = nullptr;
+            HIP::colBind(bad, m0, mt, dctx);
+        } catch (const std::runtime_error &) {
+            threw = true;
+        }
+        CHECK(threw);
+        auto arg = G(3, {1, 2, 3, 4, 5, 6, 7, 8, 9});
+        using DTSel = DenseMatrix<int64_t>;
+        auto sel = genGivenVals<DTSel>(8, {1, 2, 2, 0, 1, 0, 1, 2}, dctx);
+        DT *ex = nullptr;
+        HIP::extractCol(ex, arg, sel, dctx);
+        CHECK(equals(ex, {2, 3, 3, 1, 2, 1, 2, 3, 5, 6, 6, 4, 5, 4, 5, 6, 8, 9, 9, 7, 8, 7, 8, 9}));
+        auto selbad = genGivenVals<DTSel>(2, {1, 3}, dctx);
+        threw = false;
+        try {
+            DT *bad = nullptr;
+            HIP::extractCol(bad, arg, selbad, dctx);
+        } catch (const std::out_of_range &) {
+            threw = true;
+        }
+        CHECK(threw);
+        auto in = G(1, {-3, -2, -1, 0, 1, 2, 3, 4, 5});
+        DT *rl = nullptr;
+        HIP::NN::Activation::Forward<HIP::NN::Activation::ReLU, DT, DT>::apply(rl, in, dctx);
+        CHECK(equals(rl, {0, 0, 0, 0, 1, 2, 3, 4, 5}));
+        DT *f = nullptr;
+        HIP::fill(f, VT(2.5), 3, 4, dctx);
+        CHECK(equals(f, std::vector<VT>(12, VT(2.5))));
+        std::vector<VT> img(150);
+        for (int i = 0; i < 150; i++)
+            img[i] = VT(i + 1);
+        auto pin = G(2, img);
+        DT *avg = nullptr;
+        size_t oh = 0, ow = 0;
+        HIP::NN::Pooling::Forward<HIP::NN::Pooling::AVG, DT, DT>::apply(avg, oh, ow, pin, 2, 3, 5, 5, 2, 2, 2, 2, 1, 1, dctx);
+        CHECK(oh == 3 && ow == 3);
+        auto av = avg->toHost();
+        const VT first[9] = {0.25, 1.25, 2.25, 4.25, 10, 12, 9.25, 20, 22};
+        bool ok = av.size() == 54;
+        for (int i = 0; ok && i < 9; i++)
+            ok = av[i] == first[i];
+        CHECK(ok);
+        auto X = G(7, {1, 4, 5, 3, 7, 1, 2, 3, 5, 9, 8, 1, 1, 2, 3, 5, 1, 9, 2, 3, 1}), yv = G(7, {1, 2, 3, 4, 5, 6, 7});
+        DT *gv = nullptr, *gm = nullptr;
+        HIP::gemv(gv, X, yv, dctx);
+        HIP::matMul(gm, X, yv, true, false, dctx);
+        CHECK(equals(gv, gm->toHost()));
+        for (auto *q : {m, mt, m0, m1, cb, arg, ex, in, rl, f, pin, avg, X, yv, gv, gm})
+            DataObjectFactory::destroy(q);
+        DataObjectFactory::destroy(sel);
+        DataObjectFactory::destroy(selbad);
+    }
     // SyrkTest.cpp:32-58 (syrk == t(X) X) and SolveTest.cpp:42-68 (normal equations)
     {
         auto X = G(7, {1, 4, 5, 3, 7, 1, 2, 3, 5, 9, 8, 1, 1, 2, 3, 5, 1, 9, 2, 3, 1}), w = G(3, {1, 2, 3});

@@ -25,7 +25,8 @@ FILES = [
     "DNNConv2DForwardTest.cpp", "DNNPoolingTestForward.cpp", "DNNBiasAddForwardTest.cpp",
     "DNNBatchNorm2DForwardTest.cpp", "CUDA/MatMulTest.cpp", "CUDA/DNNAffineTest.cpp", "CUDA/BiasAddTest.cpp",
     "CUDA/DNNBatchNormTest.cpp", "CUDA/DNNConvolutionTest.cpp", "CUDA/DNNSoftmaxTest.cpp",
-    "CUDA/DNNActivationTest.cpp", "CUDA/DNNPoolingTest.cpp",
+    "CUDA/DNNActivationTest.cpp", "CUDA/DNNPoolingTest.cpp", "TransposeTest.cpp", "ColBindTest.cpp",
+    "ExtractColTest.cpp",
 ]
 
 NUM = re.compile(r"^[-+]?(\d+\.?\d*|\.\d+)([eE][-+]?\d+)?[fFlL]?$")

@@ -33,6 +33,10 @@ class KernelError(Exception):
     pass
 
 
+class OutOfRange(KernelError):
+    pass
+
+
 def load():
     return json.loads(GOLDEN.read_text())
 
@@ -197,14 +201,15 @@ def run(backend, f, c, k, dt):
         res, oh, ow = backend.conv2d(inp, flt, None, inp.shape[0], *p)
         _eq(res, M("result"))
     elif "Pooling" in file and fn == "checkPoolingForward":
-        if "AVG" in c["name"]:
-            raise Skip("average pooling is outside the kernel set")
         if file.startswith("CUDA/"):
             raise Skip("CUDA/DNNPoolingTest.cpp is not part of the reference's test build and its expectation "
                        "belongs to other parameters than its call")
         p = _ints(f["helper_calls"][0]["args"])  # C H W ph pw sh sw padh padw
         inp = M(args[0])
-        res, oh, ow = backend.maxpool(inp, inp.shape[0], *p)
+        if "AVG" in c["name"]:
+            res, oh, ow = backend.avgpool(inp, inp.shape[0], *p)
+        else:
+            res, oh, ow = backend.maxpool(inp, inp.shape[0], *p)
         _eq(res, M(args[1]))
     elif fn in ("checkBiasAddForward", "checkBiasAdd"):
         _eq(backend.bias_add(M(args[0]), M(args[1])), M(args[2]))
@@ -218,7 +223,29 @@ def run(backend, f, c, k, dt):
     elif file.endswith("CUDA/DNNAffineTest.cpp") and fn == "direct":
         _eq(backend.affine(M("input"), M("weights"), M("bias")), M("result"))
     elif file.endswith("CUDA/DNNActivationTest.cpp") and fn == "direct":
+        _eq(backend.relu(M("input")), M("result"))
         # ReLU == ewBinaryObjSca(MAX, x, 0): the reference has no CPU activation kernel
         _eq(backend.ew_binary_sca(BIN["MAX"], M("input"), 0.0), M("result"))
+    elif fn == "checkTranspose":
+        _eq(backend.transpose(M(args[0])), M(args[1]))
+    elif file.endswith("ColBindTest.cpp") and fn == "direct" and "Frame" not in c["name"]:
+        _eq(backend.col_bind(M("m0"), M("m1")), M("exp"))
+    elif file.endswith("ExtractColTest.cpp") and fn in ("checkExtractCol", "checkExtractColThrow"):
+        if "DenseMatrix" not in c["name"] and "arg" not in mats:
+            raise Skip("frames are outside the dense float/double kernel set")
+        arg = M(args[1])
+        if not any(d["pos"] < pos for d in c["matrices"].get(args[2].strip(), [])):
+            raise Skip("empty selection built without a literal")
+        sel = matrix(mats[args[2].strip()], np.float64).astype(np.int64)
+        if fn == "checkExtractColThrow":
+            try:
+                backend.extract_col(arg, sel)
+            except OutOfRange:
+                return
+            raise AssertionError("expected std::out_of_range")
+        exp = matrix(mats[args[3].strip()], dt)
+        if exp.size == 0:
+            exp = exp.reshape(arg.shape[0], 0)
+        _eq(backend.extract_col(arg, sel), exp)
     else:
         raise Skip(f"{fn} is outside the dense float/double kernel set")

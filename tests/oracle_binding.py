@@ -41,6 +41,8 @@ def _sc(dt, v):
 
 def _ld(a):
     """Leading dimension (elements) of a 2-D row-major array or view."""
+    if a.size == 0:
+        return max(a.shape[1], 1)
     assert a.ndim == 2 and (a.shape[1] <= 1 or a.strides[1] == a.itemsize)
     return a.strides[0] // a.itemsize if a.shape[0] > 1 else max(a.shape[1], 1)
 
@@ -160,6 +162,53 @@ def softmax(arg):
     res = np.empty(arg.shape, arg.dtype)
     st = _f("softmax", arg.dtype)(_p(res), sz(_ld(res)), _p(arg), sz(arg.shape[0]), sz(arg.shape[1]), sz(_ld(arg)))
     return st, res
+
+def avgpool(data, N, Cc, H, W, ph, pw, sh, sw, padh, padw):
+    P = (H + 2 * padh - ph) // sw + 1
+    Q = (W + 2 * padw - pw) // sh + 1
+    res = np.empty((N, Cc * P * Q), data.dtype)
+    rh, rw = sz(), sz()
+    st = _f("avgpool_forward", data.dtype)(_p(res), C.byref(rh), C.byref(rw), _p(data), sz(N), sz(Cc), sz(H), sz(W),
+                                           sz(ph), sz(pw), sz(sh), sz(sw), sz(padh), sz(padw))
+    return st, res, rh.value, rw.value
+
+
+def relu(arg):
+    res = np.empty(arg.shape, arg.dtype)
+    st = _f("relu_forward", arg.dtype)(_p(res), sz(_ld(res)), _p(arg), sz(arg.shape[0]), sz(arg.shape[1]), sz(_ld(arg)))
+    return st, res
+
+
+def fill(value, rows, cols, dt):
+    res = np.empty((rows, cols), dt)
+    st = _f("fill", dt)(_p(res), sz(max(cols, 1)), _sc(dt, value), sz(rows), sz(cols))
+    return st, res
+
+
+def col_bind(lhs, rhs):
+    res = np.empty((lhs.shape[0], lhs.shape[1] + rhs.shape[1]), lhs.dtype)
+    st = _f("col_bind", lhs.dtype)(_p(res), sz(_ld(res)), _p(lhs), sz(lhs.shape[0]), sz(lhs.shape[1]), sz(_ld(lhs)),
+                                   _p(rhs), sz(rhs.shape[0]), sz(rhs.shape[1]), sz(_ld(rhs)))
+    return st, res
+
+
+def extract_col(arg, sel):
+    sel = np.ascontiguousarray(sel, dtype=np.int64)
+    res = np.empty((arg.shape[0], sel.shape[0]), arg.dtype)
+    st = _f("extract_col", arg.dtype)(_p(res), sz(_ld(res)), _p(arg), sz(arg.shape[0]), sz(arg.shape[1]), sz(_ld(arg)),
+                                      _p(sel), sz(sel.shape[0]), sz(sel.shape[1] if sel.ndim == 2 else 1))
+    return st, res
+
+
+def transpose(arg):
+    res = np.empty((arg.shape[1], arg.shape[0]), arg.dtype)
+    st = _f("transpose", arg.dtype)(_p(res), sz(_ld(res)), _p(arg), sz(arg.shape[0]), sz(arg.shape[1]), sz(_ld(arg)))
+    return st, res
+
+
+def gemv(mat, vec):
+    """Gemv.h:51-77: t(mat) @ vec, through the same restatement as MatMul with transa."""
+    return matmul(mat, vec, True, False)
 
 
 def zscore_pipeline(X, threads=4, thr=64.0):

@@ -187,3 +187,51 @@ def test_vectorized_engine_equals_plain_kernels():
     assert s == float((r1 > 64.0).sum())
     for threads in (1, 2, 7):
         assert np.array_equal(orc.zscore_pipeline(x, threads=threads, thr=64.0)[3], r1)
+
+
+# ---------------------------------------------------------------------------------------------------
+# data reorganisation, ReLU and average pooling: numpy definitions and brute force
+# ---------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+def test_reorg_kernels_against_numpy(dt):
+    rng = np.random.default_rng(11)
+    a, b = rng.standard_normal((13, 7)).astype(dt), rng.standard_normal((13, 4)).astype(dt)
+    assert np.array_equal(orc.transpose(a)[1], a.T)
+    assert np.array_equal(orc.col_bind(a, b)[1], np.hstack([a, b]))
+    assert orc.col_bind(a, b[:5])[0] == orc.ST_RUNTIME
+    sel = np.array([[6], [-7], [0], [3], [3]], dtype=np.int64)
+    assert np.array_equal(orc.extract_col(a, sel)[1], a[:, [6, 0, 0, 3, 3]])
+    assert orc.extract_col(a, np.array([[7]], dtype=np.int64))[0] == 6
+    assert orc.extract_col(a, np.array([[-8]], dtype=np.int64))[0] == 6
+    assert orc.extract_col(a, np.zeros((2, 2), np.int64))[0] == orc.ST_RUNTIME
+    assert np.array_equal(orc.fill(2.5, 4, 3, dt)[1], np.full((4, 3), 2.5, dt))
+    assert orc.fill(1.0, 0, 3, dt)[1].shape == (0, 3)
+    x = a.copy()
+    x[0, :3] = [np.nan, -0.0, -np.inf]
+    r = orc.relu(x)[1]
+    assert np.isnan(r[0, 0]) and r[0, 2] == 0 and np.array_equal(r[1:], np.maximum(x[1:], 0))
+    v = rng.standard_normal((13, 1)).astype(dt)
+    np.testing.assert_allclose(orc.gemv(a, v)[1], a.T.astype(np.float64) @ v.astype(np.float64), rtol=1e-5 if dt == np.float32 else 1e-12,
+                               atol=1e-5 if dt == np.float32 else 1e-12)
+
+
+@pytest.mark.parametrize("p", [(2, 3, 5, 5, 2, 2, 2, 2, 1, 1), (1, 2, 6, 7, 3, 2, 1, 1, 0, 0), (2, 1, 9, 8, 2, 3, 3, 2, 1, 2),
+                               (2, 2, 4, 1, 3, 1, 1, 1, 0, 0)])
+def test_avgpool_brute_force(p):
+    """Mean over the window of the zero-padded image with the FULL window as divisor (Pooling.cpp:50); output extents
+    with the swapped strides of Pooling.cpp:38-39; the one-column quick path sums the first min(pool_h, H) values."""
+    N, C_, H, W, ph, pw, sh, sw, padh, padw = p
+    rng = np.random.default_rng(sum(p))
+    x = rng.standard_normal((N, C_ * H * W))
+    st, got, oh, ow = orc.avgpool(x, *p)
+    P, Q = (H + 2 * padh - ph) // sw + 1, (W + 2 * padw - pw) // sh + 1
+    assert st == 0 and (oh, ow) == (P, Q)
+    img = np.pad(x.reshape(N, C_, H, W), ((0, 0), (0, 0), (padh, padh), (padw, padw)))
+    exp = np.zeros((N, C_, P, Q))
+    if P == 1 and Q == 1 and W == 1:
+        exp[:, :, 0, 0] = x.reshape(N, C_, H)[:, :, :min(ph, H)].sum(axis=2) / (ph * pw)
+    else:
+        for i in range(P):
+            for j in range(Q):
+                exp[:, :, i, j] = img[:, :, i * sh:i * sh + ph, j * sw:j * sw + pw].sum(axis=(2, 3)) / (ph * pw)
+    np.testing.assert_allclose(got, exp.reshape(N, -1), rtol=1e-12, atol=1e-12)
