@@ -386,9 +386,10 @@ __global__ __launch_bounds__(256) void maxpool_kernel(T *res, const T *data, siz
 // Non-overlapping 2x2 windows (stride 2, no padding, even H and W): the tensor is a flat list of row
 // pairs [R][2][W] -> [R][W/2]. Each thread loads VI consecutive values of both rows of a pair and
 // writes VI/2 outputs, all as single vector accesses.
-template <typename T, int VI>
+template <typename T, int VI, bool AVG = false>
 __global__ __launch_bounds__(256) void maxpool2x2_kernel(T *res, const T *data, size_t items, unsigned W,
                                                          unsigned wvecs) {
+#pragma clang fp contract(off)
     const size_t item = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
     if (item >= items)
         return;
@@ -416,12 +417,20 @@ __global__ __launch_bounds__(256) void maxpool2x2_kernel(T *res, const T *data, 
 #pragma unroll
     for (int i = 0; i < VI / 2; i++) {
         // window order of Pooling.cpp:77-105 with the accumulator starting at zero
-        T m = T(0);
-        m = (m < a[2 * i]) ? a[2 * i] : m;
-        m = (m < a[2 * i + 1]) ? a[2 * i + 1] : m;
-        m = (m < b[2 * i]) ? b[2 * i] : m;
-        m = (m < b[2 * i + 1]) ? b[2 * i + 1] : m;
-        o[i] = m;
+        if constexpr (AVG) {
+            // per window row: sum from zero, scale by 1/4, add to the running result (Pooling.h:34-40)
+            const T s0 = (T(0) + a[2 * i]) + a[2 * i + 1];
+            const T s1 = (T(0) + b[2 * i]) + b[2 * i + 1];
+            const T r0 = s0 * T(0.25) + T(0);
+            o[i] = s1 * T(0.25) + r0;
+        } else {
+            T m = T(0);
+            m = (m < a[2 * i]) ? a[2 * i] : m;
+            m = (m < a[2 * i + 1]) ? a[2 * i + 1] : m;
+            m = (m < b[2 * i]) ? b[2 * i] : m;
+            m = (m < b[2 * i + 1]) ? b[2 * i + 1] : m;
+            o[i] = m;
+        }
     }
     T *out = res + r * (W / 2) + static_cast<size_t>(j) * (VI / 2);
     if constexpr (VI / 2 == 1) {
@@ -564,6 +573,15 @@ dh_status avgpool_forward(dh_ctx *ctx, T *res, size_t *res_h, size_t *res_w, con
         return DH_OK;
     if (H * W >= (size_t(1) << 31) || P * Q >= (size_t(1) << 31) || dh_ceil_div(total, 256) >= (size_t(1) << 31))
         return dh_fail(DH_ERR_RUNTIME, "Pooling: image extents exceed 2^31 elements");
+    constexpr int VI = 16 / sizeof(T);
+    if (ph == 2 && pw == 2 && sh == 2 && sw == 2 && padh == 0 && padw == 0 && H % 2 == 0 && W % VI == 0 &&
+        total < (size_t(1) << 39) && dh_aligned(data, 16) && dh_aligned(res, 8)) {
+        const size_t items = N * C * P * (W / VI);
+        hipLaunchKernelGGL((maxpool2x2_kernel<T, VI, true>), dim3(static_cast<unsigned>(dh_ceil_div(items, 256))), dim3(256),
+                           0, ctx->stream, res, data, items, static_cast<unsigned>(W), static_cast<unsigned>(W / VI));
+        DH_CHECK_LAUNCH();
+        return DH_OK;
+    }
     const T plen = T(1) / static_cast<T>(pw * ph); // Pooling.cpp:50
     hipLaunchKernelGGL((avgpool_kernel<T>), dim3(static_cast<unsigned>(dh_ceil_div(total, 256))), dim3(256), 0, ctx->stream,
                        res, data, total, static_cast<unsigned>(H), static_cast<unsigned>(W), static_cast<unsigned>(P),

@@ -88,6 +88,22 @@ template <typename T> dh_status fill(dh_ctx *ctx, T *res, size_t ld_res, T value
     return block2d<T, true>(ctx, res, ld_res, nullptr, 0, rows, cols, value);
 }
 
+// One thread per 16-byte vector of the result row: whole result rows leave as contiguous runs.
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void col_bind_kernel(T *res, size_t ld_res, const T *lhs, size_t ld_lhs, size_t lvecs,
+                                                       const T *rhs, size_t ld_rhs, size_t rvecs, size_t rows) {
+    const size_t cv = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    const size_t r = static_cast<size_t>(blockIdx.y) * blockDim.y + threadIdx.y;
+    if (cv >= lvecs + rvecs || r >= rows)
+        return;
+    T v[VEC];
+    if (cv < lvecs)
+        dh_load_vec_stream<T, VEC>(lhs + r * ld_lhs + cv * VEC, v);
+    else
+        dh_load_vec_stream<T, VEC>(rhs + r * ld_rhs + (cv - lvecs) * VEC, v);
+    dh_store_vec<T, VEC>(res + r * ld_res + cv * VEC, v);
+}
+
 // ColBind<DenseMatrix<VT>,...>::apply (kernels/ColBind.h:58-91, kernels/CUDA/ColBind.cu:47-70)
 template <typename T>
 dh_status col_bind(dh_ctx *ctx, T *res, size_t ld_res, const T *lhs, size_t lr, size_t lc, size_t ld_lhs, const T *rhs,
@@ -99,6 +115,28 @@ dh_status col_bind(dh_ctx *ctx, T *res, size_t ld_res, const T *lhs, size_t lr, 
                        lr, rr);
     if (ld_res < lc + rc || ld_lhs < lc || ld_rhs < rc)
         return dh_fail(DH_ERR_RUNTIME, "ColBind - a leading dimension is smaller than its column count");
+    constexpr int V = 16 / sizeof(T);
+    const bool vec = lc % V == 0 && rc % V == 0 && ld_res % V == 0 && ld_lhs % V == 0 && ld_rhs % V == 0 &&
+                     dh_aligned(res, 16) && dh_aligned(lhs, 16) && dh_aligned(rhs, 16);
+    if (vec && lr > 0 && lc + rc > 0) {
+        const size_t cvecs = (lc + rc) / V;
+        unsigned tx = 1;
+        while (tx < 256 && tx < cvecs)
+            tx <<= 1;
+        const unsigned ty = 256 / tx;
+        const size_t gx = dh_ceil_div(cvecs, tx);
+        const size_t slice = static_cast<size_t>(65535) * ty;
+        if (gx < (size_t(1) << 31)) {
+            for (size_t r0 = 0; r0 < lr; r0 += slice) {
+                const size_t nr = lr - r0 < slice ? lr - r0 : slice;
+                hipLaunchKernelGGL((col_bind_kernel<T, V>), dim3(static_cast<unsigned>(gx), static_cast<unsigned>(dh_ceil_div(nr, ty))),
+                                   dim3(tx, ty), 0, ctx->stream, res + r0 * ld_res, ld_res, lhs + r0 * ld_lhs, ld_lhs, lc / V,
+                                   rhs + r0 * ld_rhs, ld_rhs, rc / V, nr);
+                DH_CHECK_LAUNCH();
+            }
+            return DH_OK;
+        }
+    }
     dh_status st = block2d<T, false>(ctx, res, ld_res, lhs, ld_lhs, lr, lc, T(0));
     if (st != DH_OK)
         return st;
@@ -207,6 +245,45 @@ __global__ __launch_bounds__(256) void transpose_kernel(T *res, size_t ld_res, c
     }
 }
 
+// The same tile with 16-byte global accesses on both sides: a lane loads VEC consecutive source columns and
+// later stores VEC consecutive result columns (= source rows). LDS is written and read with scalars (the odd
+// stride that makes both directions conflict free rules out vector LDS accesses). Needs rows, cols and both
+// leading dimensions to be multiples of VEC and 16-byte aligned pointers.
+template <typename T>
+__global__ __launch_bounds__(256) void transpose_vec_kernel(T *res, size_t ld_res, const T *arg, size_t ld, size_t rows,
+                                                            size_t cols) {
+    constexpr int TS = 64, VEC = 16 / sizeof(T);
+    constexpr int LPR = TS / VEC;        // lanes per tile row
+    constexpr int RPS = 256 / LPR;       // tile rows per step of the workgroup
+    __shared__ T tile[TS][TS + 1];
+    const int m = threadIdx.x % LPR, q = threadIdx.x / LPR;
+    const size_t r0 = static_cast<size_t>(blockIdx.y) * TS, c0 = static_cast<size_t>(blockIdx.x) * TS;
+    T v[TS / RPS][VEC];
+#pragma unroll
+    for (int s_ = 0; s_ < TS / RPS; s_++) {
+        const size_t r = r0 + q + s_ * RPS, c = c0 + m * VEC;
+        if (r < rows && c < cols)
+            dh_load_vec_stream<T, VEC>(arg + r * ld + c, v[s_]);
+    }
+#pragma unroll
+    for (int s_ = 0; s_ < TS / RPS; s_++)
+#pragma unroll
+        for (int e = 0; e < VEC; e++)
+            tile[q + s_ * RPS][m * VEC + e] = v[s_][e];
+    __syncthreads();
+#pragma unroll
+    for (int s_ = 0; s_ < TS / RPS; s_++) {
+        const int cq = q + s_ * RPS; // source column inside the tile = result row
+        const size_t orow = c0 + cq, ocol = r0 + m * VEC;
+        T o[VEC];
+#pragma unroll
+        for (int e = 0; e < VEC; e++)
+            o[e] = tile[m * VEC + e][cq];
+        if (orow < cols && ocol < rows)
+            dh_store_vec<T, VEC>(res + orow * ld_res + ocol, o);
+    }
+}
+
 // Transpose<DenseMatrix<VT>,DenseMatrix<VT>>::apply (kernels/Transpose.h:51-76, kernels/CUDA/Transpose.cpp)
 template <typename T> dh_status transpose(dh_ctx *ctx, T *res, size_t ld_res, const T *arg, size_t rows, size_t cols, size_t ld) {
     DH_REQUIRE_CTX(ctx);
@@ -217,11 +294,19 @@ template <typename T> dh_status transpose(dh_ctx *ctx, T *res, size_t ld_res, co
     const size_t gx = dh_ceil_div(cols, 64);
     if (gx >= (size_t(1) << 31))
         return dh_fail(DH_ERR_RUNTIME, "Transpose - too many columns for one launch");
+    constexpr int V = 16 / sizeof(T);
+    const bool vec = rows % V == 0 && cols % V == 0 && ld % V == 0 && ld_res % V == 0 && dh_aligned(arg, 16) &&
+                     dh_aligned(res, 16);
     const size_t slice = static_cast<size_t>(65535) * 64;
     for (size_t r0 = 0; r0 < rows; r0 += slice) {
         const size_t nr = rows - r0 < slice ? rows - r0 : slice;
-        hipLaunchKernelGGL((transpose_kernel<T>), dim3(static_cast<unsigned>(gx), static_cast<unsigned>(dh_ceil_div(nr, 64))),
-                           dim3(256), 0, ctx->stream, res + r0, ld_res, arg + r0 * ld, ld, nr, cols);
+        const dim3 grid(static_cast<unsigned>(gx), static_cast<unsigned>(dh_ceil_div(nr, 64)));
+        if (vec)
+            hipLaunchKernelGGL((transpose_vec_kernel<T>), grid, dim3(256), 0, ctx->stream, res + r0, ld_res, arg + r0 * ld, ld,
+                               nr, cols);
+        else
+            hipLaunchKernelGGL((transpose_kernel<T>), grid, dim3(256), 0, ctx->stream, res + r0, ld_res, arg + r0 * ld, ld, nr,
+                               cols);
         DH_CHECK_LAUNCH();
     }
     return DH_OK;

@@ -69,9 +69,12 @@ struct TsTnArgs {
 
 // Wave tile: TM = 16*VA*RA rows by TN = 16*VB*RB columns of C; WM x WN wave tiles per workgroup,
 // the remaining 4/(WM*WN) waves split K.
-template <typename T, int VA, int RA, int VB, int RB, int WM, int WN>
+// SYM: A and B are the same matrix (t(X) X). Only MFMA tiles on or above the diagonal are computed and the
+// slab is filled by mirroring; waves whose tile lies below the diagonal have nothing to do.
+template <typename T, int VA, int RA, int VB, int RB, int WM, int WN, bool SYM = false>
 __global__ __launch_bounds__(256) void ts_tn_kernel(TsTnArgs g) {
     using M = Mfma16<T>;
+    static_assert(!SYM || (VA == VB && RA == RB && WM == WN), "the symmetric form needs the same tiling on both sides");
     constexpr int KW = 4 / (WM * WN);
     constexpr int TM = 16 * VA * RA, TN = 16 * VB * RB;
     constexpr int NACC = RA * VA * RB * VB;         // MFMA tiles per wave
@@ -82,6 +85,10 @@ __global__ __launch_bounds__(256) void ts_tn_kernel(TsTnArgs g) {
     const T *A = static_cast<const T *>(g.A);
     const T *B = static_cast<const T *>(g.B);
     const bool stream = g.stream != 0;
+    // diagonal wave tile of a symmetric product: B fragments are the A fragments, lower MFMA tiles are skipped
+    const bool diag = SYM && wm == wn;
+    if (SYM && wm > wn)
+        return; // only with WM = WN = 2, where no wave splits K and there is no barrier below
 
     // first column of each vector this lane loads; vectors that start beyond the matrix are skipped
     unsigned ca[RA], cb[RB];
@@ -128,6 +135,16 @@ __global__ __launch_bounds__(256) void ts_tn_kernel(TsTnArgs g) {
                     fr.a[u][a][e] = T(0);
             }
         }
+        if (diag) {
+            if constexpr (SYM) {
+#pragma unroll
+                for (int b = 0; b < RB; b++)
+#pragma unroll
+                    for (int f = 0; f < VB; f++)
+                        fr.b[u][b][f] = fr.a[u][b][f];
+            }
+            return;
+        }
 #pragma unroll
         for (int b = 0; b < RB; b++) {
             if (okb[b] && row_ok) {
@@ -140,6 +157,19 @@ __global__ __launch_bounds__(256) void ts_tn_kernel(TsTnArgs g) {
         }
     };
     auto mma_quad = [&](const Frag &fr, int u) {
+        if (diag) {
+#pragma unroll
+            for (int a = 0; a < RA; a++)
+#pragma unroll
+                for (int e = 0; e < VA; e++)
+#pragma unroll
+                    for (int b = 0; b < RB; b++)
+#pragma unroll
+                        for (int f = 0; f < VB; f++)
+                            if (a * VA + e <= b * VB + f)
+                                acc[a][e][b][f] = M::mma(fr.a[u][a][e], fr.b[u][b][f], acc[a][e][b][f]);
+            return;
+        }
 #pragma unroll
         for (int a = 0; a < RA; a++)
 #pragma unroll
@@ -245,9 +275,16 @@ __global__ __launch_bounds__(256) void ts_tn_kernel(TsTnArgs g) {
 #pragma unroll
                     for (int b = 0; b < RB; b++)
 #pragma unroll
-                        for (int f = 0; f < VB; f++)
-                            if (cb[b] + f < g.n)
-                                slab[static_cast<size_t>(row) * g.n + cb[b] + f] = acc[a][e][b][f][v];
+                        for (int f = 0; f < VB; f++) {
+                            if (diag && a * VA + e > b * VB + f)
+                                continue; // not computed: arrives as the mirror image of its transpose
+                            const unsigned col = cb[b] + f;
+                            if (col < g.n) {
+                                slab[static_cast<size_t>(row) * g.n + col] = acc[a][e][b][f][v];
+                                if (SYM && (!diag || a * VA + e < b * VB + f))
+                                    slab[static_cast<size_t>(col) * g.n + row] = acc[a][e][b][f][v];
+                            }
+                        }
                 }
             }
 }
@@ -404,6 +441,9 @@ template <typename T, int VA, int RA, int WM, int VB, int RB, int WN>
 static inline void ts_tn_launch(dh_ctx *ctx, const TsTnArgs &g, unsigned blocks) {
     hipLaunchKernelGGL((ts_tn_kernel<T, VA, RA, VB, RB, WM, WN>), dim3(blocks), dim3(256), 0, ctx->stream, g);
 }
+template <typename T, int V_, int R_, int W_> static inline void ts_tn_launch_sym(dh_ctx *ctx, const TsTnArgs &g, unsigned blocks) {
+    hipLaunchKernelGGL((ts_tn_kernel<T, V_, R_, V_, R_, W_, W_, true>), dim3(blocks), dim3(256), 0, ctx->stream, g);
+}
 
 // Returns false when the shape or the alignment does not fit (the caller then takes the tiled GEMM).
 template <typename T>
@@ -423,10 +463,15 @@ bool ts_tn(dh_ctx *ctx, size_t m, size_t n, size_t K, const T *A, size_t lda, co
     const int nacc = (cls_a == 0 ? 1 : V * R64) * (cls_b == 0 ? 1 : V * R64);
     const int unroll = nacc >= 16 ? 2 : 4;
     const size_t gran = static_cast<size_t>(4) * kw * unroll;
-    // one or two workgroups per CU (more only add slab traffic), each with at least four load groups per wave
-    size_t blocks = static_cast<size_t>(ctx->num_cus) * (nacc >= 16 ? 1 : 2);
+    // Workgroups: two per CU keep enough loads in flight (more were slower in every shape measured), and
+    // each must stream at least eight times the bytes of the slab it writes at the end.
+    const size_t slabf = 8;
+    size_t blocks = static_cast<size_t>(ctx->num_cus) * 2;
     size_t k_chunk = dh_ceil_div(dh_ceil_div(K, blocks), gran) * gran;
-    const size_t min_chunk = gran * 4;
+    size_t min_chunk = dh_ceil_div(slabf * m * n, m + n);
+    if (min_chunk < gran * 4)
+        min_chunk = gran * 4;
+    min_chunk = dh_ceil_div(min_chunk, gran) * gran;
     if (k_chunk < min_chunk)
         k_chunk = min_chunk;
     blocks = dh_ceil_div(K, k_chunk);
@@ -446,6 +491,16 @@ bool ts_tn(dh_ctx *ctx, size_t m, size_t n, size_t K, const T *A, size_t lda, co
     g.n = static_cast<unsigned>(n);
     g.stream = (wm * wn == 1 && static_cast<const void *>(A) != static_cast<const void *>(B)) ? 1 : 0;
     const unsigned nb = static_cast<unsigned>(blocks);
+    const size_t elems = m * n;
+    if (static_cast<const void *>(A) == static_cast<const void *>(B) && m == n && lda == ldb && cls_a == 1) {
+        // t(X) X with up to 64 columns: upper MFMA tiles only (10 of 16 per step). With 65..128 columns the four
+        // waves own one 64 x 64 quadrant each and the slowest of them still has a full one, so nothing is gained.
+        ts_tn_launch_sym<T, V, R64, 1>(ctx, g, nb);
+        hipLaunchKernelGGL((ts_slab_reduce_kernel<T>), dim3(static_cast<unsigned>(dh_ceil_div(elems, 32))), dim3(256), 0,
+                           ctx->stream, C, ldc, static_cast<const T *>(wsv), nb, g.m, g.n);
+        *status = DH_OK;
+        return true;
+    }
 #define DH_TS_B(VA_, RA_, WM_)                                                                     \
     do {                                                                                           \
         if (cls_b == 0)                                                                            \
@@ -462,7 +517,6 @@ bool ts_tn(dh_ctx *ctx, size_t m, size_t n, size_t K, const T *A, size_t lda, co
     else
         DH_TS_B(V, R64, 2);
 #undef DH_TS_B
-    const size_t elems = m * n;
     hipLaunchKernelGGL((ts_slab_reduce_kernel<T>), dim3(static_cast<unsigned>(dh_ceil_div(elems, 32))), dim3(256), 0,
                        ctx->stream, C, ldc, static_cast<const T *>(wsv), nb, g.m, g.n);
     *status = DH_OK;
