@@ -22,6 +22,15 @@ CONV_CASES = [  # N, C, H, W, F, Hf, Wf, sh, sw, ph, pw
     (2, 8, 9, 9, 130, 3, 3, 1, 2, 0, 1),
     (130, 2, 5, 6, 5, 1, 1, 1, 1, 0, 0),
     (1, 4, 7, 7, 3, 7, 7, 1, 1, 0, 0),
+    # images of at least 127 output pixels (the tile of 128 pixels spans at most two images): channel stages with a
+    # partial last stage, strides, wide rows, 1x1 filters, K tails
+    (3, 20, 16, 16, 24, 3, 3, 1, 1, 1, 1),
+    (2, 4, 33, 31, 10, 3, 3, 2, 2, 1, 1),
+    (2, 2, 12, 200, 6, 3, 5, 1, 1, 1, 2),
+    (3, 16, 12, 12, 64, 1, 1, 1, 1, 0, 0),
+    (2, 7, 20, 9, 33, 4, 2, 1, 1, 0, 0),
+    (1, 40, 15, 15, 16, 3, 3, 1, 1, 1, 1),
+    (7, 3, 13, 11, 5, 3, 3, 1, 1, 1, 1),
 ]
 
 
@@ -56,6 +65,26 @@ def test_conv2d_integer_valued_exact(ctx, dt):
     got, _, _ = conv2dForward(None, DenseMatrix.from_numpy(ctx, x), DenseMatrix.from_numpy(ctx, w),
                               DenseMatrix.from_numpy(ctx, b), N, C, H, W, Hf, Wf, 1, 1, 1, 1, ctx)
     assert_exact(got.to_numpy(), exp)
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+def test_conv2d_non_finite_inputs_stay_local(ctx, dt):
+    """An infinity or NaN in the image reaches exactly the outputs whose window covers it - in particular the zero
+    padding of the K dimension (45 taps in tiles of 16 / 8) must not multiply it into anything."""
+    rng = np.random.default_rng(9)
+    N, C, H, W, F, Hf, Wf = 2, 5, 12, 12, 9, 3, 3
+    x = rng.random((N, C * H * W)).astype(dt)
+    x[0, 0] = np.inf          # image 0, channel 0, (0, 0)
+    x[1, 3 * H * W + 5 * W + 7] = np.nan
+    w = (rng.random((F, C * Hf * Wf)) + 0.5).astype(dt)
+    st, exp, _, _ = orc.conv2d(x, w, None, N, C, H, W, Hf, Wf, 1, 1, 1, 1)
+    got, _, _ = conv2dForward(None, DenseMatrix.from_numpy(ctx, x), DenseMatrix.from_numpy(ctx, w), None, N, C, H, W, Hf, Wf,
+                              1, 1, 1, 1, ctx)
+    got = got.to_numpy()
+    assert np.array_equal(np.isfinite(got), np.isfinite(exp))
+    assert np.array_equal(np.isnan(got), np.isnan(exp))
+    fin = np.isfinite(exp)
+    assert_close(got[fin], exp[fin], elementwise=False)
 
 
 def test_conv2d_filter_mismatch(ctx):
