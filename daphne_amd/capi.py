@@ -93,6 +93,7 @@ _LATE_SIGNATURES: dict[str, list] = {
     "dh_bias_add": [vp, vp, vp, sz, sz, vp, sz],
     "dh_batchnorm_inference": [vp, vp, vp, sz, sz, vp, vp, vp, vp, sz, "T", i32],
     "dh_softmax": [vp, vp, sz, vp, sz, sz, sz],
+    "dh_agg_col_moments": [vp, vp, vp, i32, vp, sz, sz, sz],
     "dh_avgpool_forward": [vp, vp, C.POINTER(sz), C.POINTER(sz), vp, sz, sz, sz, sz, sz, sz, sz, sz, sz, sz],
     "dh_relu_forward": [vp, vp, sz, vp, sz, sz, sz],
     "dh_fill": [vp, vp, sz, "T", sz, sz],

@@ -25,3 +25,8 @@ extern "C" dh_status dh_agg_col_idx_f32(dh_ctx *ctx, int op, uint64_t *res, cons
                                        size_t cols, size_t ld) {
     return dh_agg::agg_col_idx<float>(ctx, op, res, arg, rows, cols, ld);
 }
+
+extern "C" dh_status dh_agg_col_moments_f32(dh_ctx *ctx, float *res_mean, float *res_var, int stddev, const float *arg, size_t rows,
+                                             size_t cols, size_t ld) {
+    return dh_agg::agg_col_moments<float>(ctx, res_mean, res_var, stddev, arg, rows, cols, ld);
+}

@@ -800,7 +800,8 @@ __global__ __launch_bounds__(THREADS) void col_var_stage1(const T *arg, size_t r
 // OUT: 0 variance, 1 stddev, 2 mean (unused by the public API but kept for pipelines).
 template <typename T, int OUT>
 __global__ __launch_bounds__(THREADS) void col_var_stage2(const T *part_mean, const T *part_m2, size_t nparts,
-                                                          size_t cols, size_t rows, size_t slab, T *res) {
+                                                          size_t cols, size_t rows, size_t slab, T *res,
+                                                          T *res_mean = nullptr) {
     // (S2_TX columns, S2_TY partial lanes): every lane merges its share of the per-block
     // (count, mean, M2) triples with Chan's formula in double, lane 0 then merges the lanes.
     __shared__ double lds_n[S2_TY][S2_TX], lds_mean[S2_TY][S2_TX], lds_m2[S2_TY][S2_TX];
@@ -844,6 +845,8 @@ __global__ __launch_bounds__(THREADS) void col_var_stage2(const T *part_mean, co
     if constexpr (OUT == 2)
         v = cmean;
     res[c] = static_cast<T>(v);
+    if (res_mean)
+        res_mean[c] = static_cast<T>(cmean);
 }
 
 // IDXMIN / IDXMAX per column.
@@ -1033,6 +1036,44 @@ template <typename T> dh_status agg_col(dh_ctx *ctx, int op, T *res, const T *ar
     }
     if (st != DH_OK)
         return st;
+    DH_CHECK_LAUNCH();
+    return DH_OK;
+}
+
+// Column means and variances (or standard deviations) from ONE pass over the matrix: the per-block
+// (count, mean, M2) triples that the variance needs carry the mean anyway. Same results as agg_col with
+// MEAN and VAR / STDDEV within rounding (the mean comes out of the Chan merge in double instead of sum / rows).
+template <typename T>
+dh_status agg_col_moments(dh_ctx *ctx, T *res_mean, T *res_var, int stddev, const T *arg, size_t rows, size_t cols, size_t ld) {
+    DH_REQUIRE_CTX(ctx);
+    if (ld < cols)
+        return dh_fail(DH_ERR_RUNTIME, "AggCol - leading dimension smaller than the column count");
+    if (res_mean == nullptr || res_var == nullptr)
+        return dh_fail(DH_ERR_RUNTIME, "AggCol - result pointer is null");
+    if (cols == 0)
+        return DH_OK;
+    if (rows == 0)
+        return dh_fail(DH_ERR_RUNTIME, "AggCol - the argument has no rows");
+    constexpr int V = dh_vec<T>::N;
+    ColPlan p = col_plan<T>(ctx, arg, rows, cols, ld);
+    void *wsv = nullptr;
+    dh_status st = dh_workspace(ctx, 2 * p.nparts * cols * sizeof(T), &wsv);
+    if (st != DH_OK)
+        return st;
+    T *pm = static_cast<T *>(wsv);
+    T *pq = pm + p.nparts * cols;
+    const size_t lds = 2 * static_cast<size_t>(THREADS) * p.vec * sizeof(T);
+    if (p.vec == V)
+        hipLaunchKernelGGL((col_var_stage1<T, V>), p.grid, p.block, lds, ctx->stream, arg, rows, p.cvecs, ld, p.slab, pm, pq);
+    else
+        hipLaunchKernelGGL((col_var_stage1<T, 1>), p.grid, p.block, lds, ctx->stream, arg, rows, p.cvecs, ld, p.slab, pm, pq);
+    const dim3 g2(static_cast<unsigned>(dh_ceil_div(cols, S2_TX)));
+    if (stddev)
+        hipLaunchKernelGGL((col_var_stage2<T, 1>), g2, dim3(S2_TX, S2_TY), 0, ctx->stream, pm, pq, p.nparts, cols, rows, p.slab,
+                           res_var, res_mean);
+    else
+        hipLaunchKernelGGL((col_var_stage2<T, 0>), g2, dim3(S2_TX, S2_TY), 0, ctx->stream, pm, pq, p.nparts, cols, rows, p.slab,
+                           res_var, res_mean);
     DH_CHECK_LAUNCH();
     return DH_OK;
 }

@@ -269,6 +269,17 @@ def aggCol(opCode, res, arg: DenseMatrix, ctx: HIPContext) -> DenseMatrix:
     return res
 
 
+def aggColMoments(arg: DenseMatrix, ctx: HIPContext, stddev: bool = False, res_mean=None, res_var=None):
+    """aggCol(MEAN) and aggCol(VAR | STDDEV) of the same matrix from one pass over it. Returns (mean, var)."""
+    if res_mean is None:
+        res_mean = DenseMatrix(ctx, 1, arg.cols, arg.dtype)
+    if res_var is None:
+        res_var = DenseMatrix(ctx, 1, arg.cols, arg.dtype)
+    capi.check(_fn("dh_agg_col_moments", arg.dtype)(ctx._h, res_mean.ptr, res_var.ptr, int(stddev), arg.ptr, arg.rows,
+                                                    arg.cols, arg.row_skip))
+    return res_mean, res_var
+
+
 # ------------------------------------------------------------------------------------------
 # contractions
 # ------------------------------------------------------------------------------------------

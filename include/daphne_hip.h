@@ -189,6 +189,14 @@ dh_status dh_agg_col_f32(dh_ctx *ctx, int op, float *res, const float *arg, size
                          size_t cols, size_t ld);
 dh_status dh_agg_col_f64(dh_ctx *ctx, int op, double *res, const double *arg, size_t rows,
                          size_t cols, size_t ld);
+/* colMeans and colVars (or colStddevs when `stddev` != 0) of the same matrix in ONE pass: what
+ * dh_agg_col with DH_AGG_MEAN and DH_AGG_VAR / DH_AGG_STDDEV (kernels/AggCol.h:143-170) return, for a
+ * caller - a fused pipeline, or a rewrite of mean(X,1) + var(X,1) on one input - that needs both. The
+ * reference has two separate kernel calls here; results agree with them within rounding. */
+dh_status dh_agg_col_moments_f32(dh_ctx *ctx, float *res_mean, float *res_var, int stddev,
+                                 const float *arg, size_t rows, size_t cols, size_t ld);
+dh_status dh_agg_col_moments_f64(dh_ctx *ctx, double *res_mean, double *res_var, int stddev,
+                                 const double *arg, size_t rows, size_t cols, size_t ld);
 /* AggCol with IDXMIN / IDXMAX (kernels/AggCol.h:70-122): first row of the strict extremum
  * per column. */
 dh_status dh_agg_col_idx_f32(dh_ctx *ctx, int op, uint64_t *res, const float *arg, size_t rows,

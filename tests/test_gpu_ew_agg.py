@@ -241,3 +241,31 @@ def test_agg_on_views(ctx, dt):
             cmp(aggCol(op, None, V, ctx).to_numpy(), orc.agg_col(op, v)[1], **kw)
             cmp(np.array([aggAll(op, V, ctx)]), np.array([orc.agg_all(op, v)[1]]))
         assert_exact(aggRow(AggOpCode.IDXMIN, None, V, ctx).to_numpy(), orc.agg_row(AggOpCode.IDXMIN, v)[1])
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("shape", AGG_SHAPES + [(200000, 64)])
+def test_agg_col_moments_one_pass(ctx, dt, shape):
+    """Column means and variances from one pass equal the two separate aggregations (oracle: AggCol MEAN / VAR / STDDEV)."""
+    from daphne_amd.kernels import aggColMoments
+    rng = np.random.default_rng(shape[0] + 3 * shape[1])
+    a = (rng.standard_normal(shape) * 2 + 5).astype(dt)
+    A = DenseMatrix.from_numpy(ctx, a)
+    mean, var = aggColMoments(A, ctx)
+    _, sd = aggColMoments(A, ctx, stddev=True)
+    truth_mean, truth_var = a.astype(np.float64).mean(axis=0, keepdims=True), a.astype(np.float64).var(axis=0, keepdims=True)
+    assert_close(mean.to_numpy(), truth_mean.astype(dt))
+    assert_close(var.to_numpy(), truth_var.astype(dt), elementwise=False)
+    assert_close(sd.to_numpy(), np.sqrt(truth_var).astype(dt), elementwise=False)
+    if shape[0] <= 50000:
+        assert_close(mean.to_numpy(), orc.agg_col(AggOpCode.MEAN, a)[1])
+        assert_close(var.to_numpy(), orc.agg_col(AggOpCode.VAR, a)[1], elementwise=False)
+    # the same numbers as the separate device kernels
+    assert_close(mean.to_numpy(), aggCol(AggOpCode.MEAN, None, A, ctx).to_numpy())
+    assert_exact(var.to_numpy(), aggCol(AggOpCode.VAR, None, A, ctx).to_numpy())
+    # a view
+    if shape[0] > 10 and shape[1] > 4:
+        v, V = a[3:-2, 1:-1], A.slice(3, shape[0] - 2, 1, shape[1] - 1)
+        m2, v2 = aggColMoments(V, ctx)
+        assert_close(m2.to_numpy(), v.astype(np.float64).mean(axis=0, keepdims=True).astype(dt))
+        assert_close(v2.to_numpy(), v.astype(np.float64).var(axis=0, keepdims=True).astype(dt), elementwise=False)
