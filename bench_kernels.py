@@ -1,0 +1,215 @@
+#!/usr/bin/env python3
+"""Per-kernel throughput survey on one MI355X: every device kernel of the library at a large shape, float and double,
+against the roofline that bounds it (HBM 8 TB/s for the streaming kernels, the dtype's MFMA peak for contractions).
+
+    python bench_kernels.py [--reps 20] [--dtype f32|f64|both] [--only group|substring]
+
+One JSON line per measurement: {"kernel", "dtype", "shape", "us", "achieved", "unit", "peak", "frac"}. Bytes are the
+algorithmic ones (distinct inputs and outputs once each), flops 2mnk / n(n+1)k / 2 N F P Q C Hf Wf. Timing: device
+events around `reps` back-to-back launches on the context's stream after one warm-up launch; inputs are generated on
+the device. bench.py carries the headline pipeline; this file is the evidence for the single kernels.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM = 8000.0
+MFMA = {"f32": 157.3, "f64": 78.6}
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--reps", type=int, default=20)
+    ap.add_argument("--dtype", default="both", choices=["f32", "f64", "both"])
+    ap.add_argument("--only", default="")
+    args = ap.parse_args()
+
+    import numpy as np
+    import torch
+
+    from daphne_amd import kernels as K
+    from daphne_amd.kernels import AggOpCode as A, BinaryOpCode as B, DenseMatrix as DM, UnaryOpCode as U
+    from daphne_amd.pipeline import SELF, VectorizedPipeline
+
+    if not torch.cuda.is_available():
+        print("bench_kernels.py: no GPU visible", file=sys.stderr)
+        return 1
+    ctx = K.HIPContext(0)
+    gen = torch.Generator(device="cuda").manual_seed(7)
+
+    def timed(fn):
+        fn()
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(args.reps):
+            fn()
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) / args.reps * 1e3  # microseconds
+
+    def emit(kernel, dt, shape, us, nbytes=None, flops=None):
+        if args.only and args.only not in groups and args.only not in kernel:
+            return
+        if flops is None:
+            ach, unit, peak = nbytes / us / 1e3, "GB/s", HBM
+        else:
+            ach, unit, peak = flops / us / 1e6, "TFLOP/s", MFMA[dt]
+        print(json.dumps({"kernel": kernel, "dtype": dt, "shape": shape, "us": round(us, 1), "achieved": round(ach, 1),
+                          "unit": unit, "peak": peak, "frac": round(ach / peak, 3)}), flush=True)
+
+    groups = ("ew", "agg", "pipeline", "reorg", "tall", "gemm", "dnn", "solve")
+
+    def want(group):
+        # --only takes a group name (runs that group) or a substring of a kernel name (runs all, prints the matches)
+        return not args.only or args.only == group or args.only not in groups
+
+    for dt in (["f32", "f64"] if args.dtype == "both" else [args.dtype]):
+        tdt, ndt, sz = (torch.float32, np.float32, 4) if dt == "f32" else (torch.float64, np.float64, 8)
+        rows, cols = (20_000_000, 64) if dt == "f32" else (10_000_000, 64)
+        nb = rows * cols * sz
+        shape = f"{rows}x{cols}"
+        X = DM.from_torch(ctx, torch.randn(rows, cols, device="cuda", dtype=tdt, generator=gen) * 2 + 5)
+        R = DM(ctx, rows, cols, ndt)
+        rowv = DM.from_torch(ctx, torch.rand(1, cols, device="cuda", dtype=tdt, generator=gen) + 1)
+        colv = DM.from_torch(ctx, torch.rand(rows, 1, device="cuda", dtype=tdt, generator=gen) + 1)
+        r1 = DM(ctx, rows, 1, ndt)
+        ri = DM(ctx, rows, 1, np.uint64)
+        c1 = DM(ctx, 1, cols, ndt)
+
+        # --- elementwise ---------------------------------------------------------------------------------------
+        if want("ew"):
+            emit("ewBinaryMat SUB row-vector", dt, shape, timed(lambda: K.ewBinaryMat(B.SUB, R, X, rowv, ctx)), 2 * nb)
+            emit("ewBinaryMat DIV column-vector", dt, shape, timed(lambda: K.ewBinaryMat(B.DIV, R, X, colv, ctx)), 2 * nb + rows * sz)
+            emit("ewBinaryMat MUL same shape", dt, shape, timed(lambda: K.ewBinaryMat(B.MUL, R, X, X, ctx)), 2 * nb)
+            emit("ewBinaryMat ADD two inputs", dt, shape, timed(lambda: K.ewBinaryMat(B.ADD, R, X, R, ctx)), 3 * nb)
+            emit("ewBinaryObjSca GT", dt, shape, timed(lambda: K.ewBinaryObjSca(B.GT, R, X, 5.0, ctx)), 2 * nb)
+            K.ewUnaryMat(U.ABS, R, X, ctx)
+            emit("ewUnaryMat SQRT in place (domain-checked)", dt, shape, timed(lambda: K.ewUnaryMat(U.SQRT, R, R, ctx)), 2 * nb)
+            emit("ewUnaryMat EXP on a column", dt, f"{rows}x1", timed(lambda: K.ewUnaryMat(U.EXP, r1, colv, ctx)), 2 * rows * sz)
+            emit("reluForward in place", dt, shape, timed(lambda: K.reluForward(R, R, ctx)), 2 * nb)
+        # --- aggregations --------------------------------------------------------------------------------------
+        if want("agg"):
+            emit("aggAll SUM", dt, shape, timed(lambda: K.aggAll(A.SUM, X, ctx)), nb)
+            emit("aggAll VAR (two passes)", dt, shape, timed(lambda: K.aggAll(A.VAR, X, ctx)), 2 * nb)
+            emit("aggRow SUM", dt, shape, timed(lambda: K.aggRow(A.SUM, r1, X, ctx)), nb + rows * sz)
+            emit("aggRow MAX", dt, shape, timed(lambda: K.aggRow(A.MAX, r1, X, ctx)), nb + rows * sz)
+            emit("aggRow VAR (two passes over the row)", dt, shape, timed(lambda: K.aggRow(A.VAR, r1, X, ctx)), nb + rows * sz)
+            emit("aggRow IDXMIN", dt, shape, timed(lambda: K.aggRow(A.IDXMIN, ri, X, ctx)), nb + rows * 8)
+            emit("aggCol SUM", dt, shape, timed(lambda: K.aggCol(A.SUM, c1, X, ctx)), nb)
+            emit("aggCol MAX", dt, shape, timed(lambda: K.aggCol(A.MAX, c1, X, ctx)), nb)
+            emit("aggCol VAR (one pass)", dt, shape, timed(lambda: K.aggCol(A.VAR, c1, X, ctx)), nb)
+            emit("aggColMoments mean+var (one pass)", dt, shape, timed(lambda: K.aggColMoments(X, ctx, res_mean=c1, res_var=rowv)), nb)
+            ci = DM(ctx, 1, cols, np.uint64)
+            emit("aggCol IDXMAX", dt, shape, timed(lambda: K.aggCol(A.IDXMAX, ci, X, ctx)), nb)
+            rowv = DM.from_torch(ctx, torch.rand(1, cols, device="cuda", dtype=tdt, generator=gen) + 1)
+        # --- fused pipeline ------------------------------------------------------------------------------------
+        if want("pipeline"):
+            p = VectorizedPipeline(ctx, X)
+            p.ewBinary(B.SUB, c1).ewBinary(B.DIV, rowv).ewBinary(B.MUL, SELF).rowAgg(A.SUM)
+            p.storeRow(r1)
+            p.ewBinary(B.GT, float(cols))
+            p.reduceAll(A.SUM)
+            emit("VectorizedPipeline z-score/rowSums/count", dt, shape, timed(p.run), nb + rows * sz)
+        # --- data reorganisation -------------------------------------------------------------------------------
+        if want("reorg"):
+            emit("fill", dt, shape, timed(lambda: K.fill(R, 2.5, rows, cols, ctx)), nb)
+            T = DM(ctx, cols, rows, ndt)
+            emit("transpose", dt, shape, timed(lambda: K.transpose(T, X, ctx)), 2 * nb)
+            T.destroy()
+            L = DM.from_torch(ctx, torch.randn(rows, 16, device="cuda", dtype=tdt, generator=gen))
+            CB = DM(ctx, rows, cols + 16, ndt)
+            emit("colBind 64|16 columns", dt, shape, timed(lambda: K.colBind(CB, X, L, ctx)), 2 * (nb + rows * 16 * sz))
+            CB.destroy()
+            sel = DM.from_numpy(ctx, np.array([63, 0, 17, 5, 9, 33, 2, 41], dtype=np.int64).reshape(-1, 1))
+            E = DM(ctx, rows, 8, ndt)
+            emit("extractCol 8 of 64 columns (sector traffic: whole rows)", dt, shape, timed(lambda: K.extractCol(E, X, sel, ctx)),
+                 nb + rows * 8 * sz)
+            E.destroy()
+            L.destroy()
+        # --- tall-and-skinny contractions ----------------------------------------------------------------------
+        if want("tall"):
+            y = colv
+            gv = DM(ctx, cols, 1, ndt)
+            emit("tall gemv t(X) y", dt, shape, timed(lambda: K.gemv(gv, X, y, ctx)), nb + rows * sz)
+            S = DM(ctx, cols, cols, ndt)
+            emit("tall syrk t(X) X", dt, shape, timed(lambda: K.syrk(S, X, True, ctx)), nb)
+            Cc = DM.from_torch(ctx, torch.randn(16, cols, device="cuda", dtype=tdt, generator=gen))
+            XC = DM(ctx, rows, 16, ndt)
+            emit("tall matMul X t(C), C 16x64", dt, shape, timed(lambda: K.matMul(XC, X, Cc, False, True, ctx)), nb + rows * 16 * sz)
+            PtX = DM(ctx, 16, cols, ndt)
+            emit("tall matMul t(P) X, P rows x 16", dt, shape, timed(lambda: K.matMul(PtX, XC, X, True, False, ctx)), nb + rows * 16 * sz)
+            XC.destroy()
+        for m in (X, R, colv, r1, ri):
+            m.destroy()
+        ctx.releaseCached()
+        torch.cuda.empty_cache()
+
+        # --- square contractions (shorter than the headline shapes of bench.py --config 4) -------------------------
+        if want("gemm"):
+            n = 8192 if dt == "f32" else 4096
+            Am = DM.from_torch(ctx, torch.rand(n, n, device="cuda", dtype=tdt, generator=gen) - 0.5)
+            Bm = DM.from_torch(ctx, torch.rand(n, n, device="cuda", dtype=tdt, generator=gen) - 0.5)
+            Cm = DM(ctx, n, n, ndt)
+            for ta, tb in ((False, False), (False, True), (True, False), (True, True)):
+                emit(f"matMul {'T' if ta else 'N'}{'T' if tb else 'N'}", dt, f"{n}^3", timed(lambda: K.matMul(Cm, Am, Bm, ta, tb, ctx)),
+                     flops=2.0 * n ** 3)
+            emit("syrk t(X) X", dt, f"{n}x{n}", timed(lambda: K.syrk(Cm, Am, True, ctx)), flops=float(n) * (n + 1) * n)
+            emit("syrk X t(X)", dt, f"{n}x{n}", timed(lambda: K.syrk(Cm, Am, False, ctx)), flops=float(n) * (n + 1) * n)
+            for m in (Am, Bm, Cm):
+                m.destroy()
+        # --- DNN ---------------------------------------------------------------------------------------------
+        if want("dnn"):
+            N = 4096 if dt == "f32" else 2048
+            x2 = DM.from_torch(ctx, torch.rand(N, 32 * 14 * 14, device="cuda", dtype=tdt, generator=gen))
+            w2 = DM.from_torch(ctx, torch.randn(64, 800, device="cuda", dtype=tdt, generator=gen) * 0.05)
+            b2 = DM.from_torch(ctx, torch.randn(64, 1, device="cuda", dtype=tdt, generator=gen) * 0.1)
+            o2 = DM(ctx, N, 64 * 196, ndt)
+            emit("conv2dForward 32->64 ch, 14x14, 5x5 pad 2 (incl. border copy)", dt, f"batch {N}",
+                 timed(lambda: K.conv2dForward(o2, x2, w2, b2, N, 32, 14, 14, 5, 5, 1, 1, 2, 2, ctx)), flops=2.0 * N * 64 * 196 * 800)
+            emit("biasAdd 64 channels", dt, f"{N}x{64 * 196}", timed(lambda: K.biasAdd(o2, o2, b2, ctx)), 2 * N * 64 * 196 * sz)
+            one = DM.from_torch(ctx, torch.ones(64, 1, device="cuda", dtype=tdt))
+            emit("batchNormInferenceForward 64 channels", dt, f"{N}x{64 * 196}",
+                 timed(lambda: K.batchNormInferenceForward(o2, o2, one, b2, b2, one, 1e-5, ctx)), 2 * N * 64 * 196 * sz)
+            pl = DM(ctx, N, 64 * 49, ndt)
+            emit("maxPoolForward 2x2/2 on 14x14", dt, f"{N}x{64 * 196}",
+                 timed(lambda: K.maxPoolForward(pl, o2, N, 64, 14, 14, 2, 2, 2, 2, 0, 0, ctx)), 1.25 * N * 64 * 196 * sz)
+            emit("avgPoolForward 2x2/2 on 14x14", dt, f"{N}x{64 * 196}",
+                 timed(lambda: K.avgPoolForward(pl, o2, N, 64, 14, 14, 2, 2, 2, 2, 0, 0, ctx)), 1.25 * N * 64 * 196 * sz)
+            emit("maxPoolForward 3x3/2 pad 1 on 14x14 (generic kernel)", dt, f"{N}x{64 * 196}",
+                 timed(lambda: K.maxPoolForward(None, o2, N, 64, 14, 14, 3, 3, 2, 2, 1, 1, ctx)),
+                 (1 + 49.0 / 196) * N * 64 * 196 * sz)
+            w3 = DM.from_torch(ctx, torch.randn(3136, 512, device="cuda", dtype=tdt, generator=gen) * 0.02)
+            b3 = DM.from_torch(ctx, torch.randn(1, 512, device="cuda", dtype=tdt, generator=gen) * 0.1)
+            h3 = DM(ctx, N, 512, ndt)
+            emit("affineForward 3136 -> 512", dt, f"batch {N}", timed(lambda: K.affineForward(h3, pl, w3, b3, ctx)),
+                 flops=2.0 * N * 3136 * 512)
+            big = DM.from_torch(ctx, torch.randn(1_000_000, 10, device="cuda", dtype=tdt, generator=gen))
+            sm = DM(ctx, 1_000_000, 10, ndt)
+            emit("softmax 10 classes", dt, "1000000x10", timed(lambda: K.softmax(sm, big, ctx)), 2 * 10_000_000 * sz)
+            for m in (x2, w2, b2, o2, one, pl, w3, b3, h3, big, sm):
+                m.destroy()
+        # --- solve -------------------------------------------------------------------------------------------
+        if want("solve"):
+            n = 100
+            As = DM.from_torch(ctx, torch.rand(n, n, device="cuda", dtype=tdt, generator=gen) + n * torch.eye(n, device="cuda", dtype=tdt))
+            bs = DM.from_torch(ctx, torch.rand(n, 1, device="cuda", dtype=tdt, generator=gen))
+            xs = DM(ctx, n, 1, ndt)
+            us = timed(lambda: K.solve(xs, As, bs, ctx))
+            if want("solve"):
+                print(json.dumps({"kernel": "solve 100x100 (latency bound, incl. the singularity flag read-back)", "dtype": dt,
+                                  "shape": "100x100", "us": round(us, 1)}), flush=True)
+        ctx.releaseCached()
+        torch.cuda.empty_cache()
+    ctx.destroy()
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -331,19 +331,32 @@ __global__ __launch_bounds__(THREADS) void row_kernel(T *res, size_t ld_res, con
             row[u] = arg + (r < rows ? r : rows - 1) * ld;
         }
         T acc[UR];
+        T first[UR];      // element 0 of the row, known to the lane that loads it (NANFIRST)
+        T xk[UR][VEC];    // the lane's values when the row fits one vector per lane (second pass of VAR / STDDEV)
+        const bool in_regs = cvecs <= static_cast<size_t>(G);
 #pragma unroll
-        for (int u = 0; u < UR; u++)
+        for (int u = 0; u < UR; u++) {
             acc[u] = R::id();
+            first[u] = T(0);
+        }
         for (size_t cv = lane; cv < cvecs; cv += G) {
             T x[UR][VEC];
 #pragma unroll
             for (int u = 0; u < UR; u++)
                 dh_load_vec_stream<T, VEC>(row[u] + cv * VEC, x[u]);
 #pragma unroll
-            for (int u = 0; u < UR; u++)
+            for (int u = 0; u < UR; u++) {
+                if constexpr (NANFIRST) {
+                    if (cv == 0)
+                        first[u] = x[u][0];
+                }
 #pragma unroll
-                for (int i = 0; i < VEC; i++)
+                for (int i = 0; i < VEC; i++) {
                     acc[u] = R::comb(acc[u], x[u][i]);
+                    if constexpr (FINAL >= 2)
+                        xk[u][i] = x[u][i];
+                }
+            }
         }
 #pragma unroll
         for (int u = 0; u < UR; u++) {
@@ -357,18 +370,30 @@ __global__ __launch_bounds__(THREADS) void row_kernel(T *res, size_t ld_res, con
 #pragma unroll
             for (int u = 0; u < UR; u++)
                 s[u] = T(0);
-            for (size_t cv = lane; cv < cvecs; cv += G) {
-                T x[UR][VEC];
+            if (in_regs) {
+                if (static_cast<size_t>(lane) < cvecs) {
 #pragma unroll
-                for (int u = 0; u < UR; u++)
-                    load_vec<T, VEC>(row[u] + cv * VEC, x[u]);
+                    for (int u = 0; u < UR; u++)
 #pragma unroll
-                for (int u = 0; u < UR; u++)
+                        for (int i = 0; i < VEC; i++) {
+                            const T d = xk[u][i] - acc[u];
+                            s[u] = s[u] + d * d;
+                        }
+                }
+            } else {
+                for (size_t cv = lane; cv < cvecs; cv += G) {
+                    T x[UR][VEC];
 #pragma unroll
-                    for (int i = 0; i < VEC; i++) {
-                        const T d = x[u][i] - acc[u];
-                        s[u] = s[u] + d * d;
-                    }
+                    for (int u = 0; u < UR; u++)
+                        load_vec<T, VEC>(row[u] + cv * VEC, x[u]);
+#pragma unroll
+                    for (int u = 0; u < UR; u++)
+#pragma unroll
+                        for (int i = 0; i < VEC; i++) {
+                            const T d = x[u][i] - acc[u];
+                            s[u] = s[u] + d * d;
+                        }
+                }
             }
 #pragma unroll
             for (int u = 0; u < UR; u++) {
@@ -381,9 +406,9 @@ __global__ __launch_bounds__(THREADS) void row_kernel(T *res, size_t ld_res, con
 #pragma unroll
         for (int u = 0; u < UR; u++) {
             if constexpr (NANFIRST) {
-                const T first = row[u][0];
-                if (dev_isnan(first))
-                    acc[u] = first;
+                // only the group's lane 0 holds the row's element 0; the results are taken from that lane below
+                if (dev_isnan(first[u]))
+                    acc[u] = first[u];
             }
         }
         if (GPW * UR <= DH_WAVE) {

@@ -574,11 +574,19 @@ dh_status avgpool_forward(dh_ctx *ctx, T *res, size_t *res_h, size_t *res_w, con
     if (H * W >= (size_t(1) << 31) || P * Q >= (size_t(1) << 31) || dh_ceil_div(total, 256) >= (size_t(1) << 31))
         return dh_fail(DH_ERR_RUNTIME, "Pooling: image extents exceed 2^31 elements");
     constexpr int VI = 16 / sizeof(T);
-    if (ph == 2 && pw == 2 && sh == 2 && sw == 2 && padh == 0 && padw == 0 && H % 2 == 0 && W % VI == 0 &&
-        total < (size_t(1) << 39) && dh_aligned(data, 16) && dh_aligned(res, 8)) {
+    const bool pairs = ph == 2 && pw == 2 && sh == 2 && sw == 2 && padh == 0 && padw == 0 && H % 2 == 0 && W % 2 == 0 &&
+                       total < (size_t(1) << 39);
+    if (pairs && W % VI == 0 && dh_aligned(data, 16) && dh_aligned(res, 8)) {
         const size_t items = N * C * P * (W / VI);
         hipLaunchKernelGGL((maxpool2x2_kernel<T, VI, true>), dim3(static_cast<unsigned>(dh_ceil_div(items, 256))), dim3(256),
                            0, ctx->stream, res, data, items, static_cast<unsigned>(W), static_cast<unsigned>(W / VI));
+        DH_CHECK_LAUNCH();
+        return DH_OK;
+    }
+    if (pairs && VI > 2 && dh_aligned(data, 8)) {
+        const size_t items = N * C * P * (W / 2);
+        hipLaunchKernelGGL((maxpool2x2_kernel<T, 2, true>), dim3(static_cast<unsigned>(dh_ceil_div(items, 256))), dim3(256), 0,
+                           ctx->stream, res, data, items, static_cast<unsigned>(W), static_cast<unsigned>(W / 2));
         DH_CHECK_LAUNCH();
         return DH_OK;
     }
@@ -731,6 +739,62 @@ __global__ __launch_bounds__(256) void softmax_kernel(T *res, size_t ld_res, con
     }
 }
 
+// Rows of up to KEEP * G values stay in registers: one read and one write of the row, one-shot grid. Same
+// per-lane order and shuffle trees as softmax_kernel, so both give the same bits.
+template <typename T, int KEEP>
+__global__ __launch_bounds__(256) void softmax_reg_kernel(T *res, size_t ld_res, const T *arg, size_t rows, size_t cols,
+                                                          size_t ld, int G) {
+    constexpr int RPG = 4; // rows per lane group, all loaded before any arithmetic
+    const int lane = threadIdx.x % G;
+    const size_t rpb = 256 / G;
+    const size_t r0 = static_cast<size_t>(blockIdx.x) * rpb * RPG + threadIdx.x / G;
+    T x[RPG][KEEP];
+#pragma unroll
+    for (int j = 0; j < RPG; j++) {
+        const size_t r = r0 + j * rpb;
+#pragma unroll
+        for (int k = 0; k < KEEP; k++) {
+            const size_t c = lane + static_cast<size_t>(k) * G;
+            x[j][k] = (r < rows && c < cols) ? arg[r * ld + c] : -std::numeric_limits<T>::infinity();
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < RPG; j++) {
+        const size_t r = r0 + j * rpb; // uniform over the lane group
+        T mx = -std::numeric_limits<T>::infinity();
+#pragma unroll
+        for (int k = 0; k < KEEP; k++)
+            mx = (mx < x[j][k]) ? x[j][k] : mx; // columns past the end hold -inf
+        for (int off = G / 2; off >= 1; off >>= 1) {
+            const T o = dh_shfl_xor(mx, off);
+            mx = (mx < o) ? o : mx;
+        }
+        const T first = __shfl(x[j][0], (threadIdx.x % DH_WAVE) - lane, DH_WAVE); // lane 0 of the group holds column 0
+        if (first != first)
+            mx = first;
+        T sum = T(0);
+#pragma unroll
+        for (int k = 0; k < KEEP; k++) {
+            const size_t c = lane + static_cast<size_t>(k) * G;
+            if (c < cols) {
+                x[j][k] = dev_exp<T>(x[j][k] - mx);
+                sum += x[j][k];
+            }
+        }
+        for (int off = G / 2; off >= 1; off >>= 1)
+            sum += dh_shfl_xor(sum, off);
+        const T inv = T(1) / sum;
+        if (r < rows) {
+#pragma unroll
+            for (int k = 0; k < KEEP; k++) {
+                const size_t c = lane + static_cast<size_t>(k) * G;
+                if (c < cols)
+                    res[r * ld_res + c] = x[j][k] * inv;
+            }
+        }
+    }
+}
+
 template <typename T>
 dh_status softmax(dh_ctx *ctx, T *res, size_t ld_res, const T *arg, size_t rows, size_t cols, size_t ld) {
     DH_REQUIRE_CTX(ctx);
@@ -741,7 +805,17 @@ dh_status softmax(dh_ctx *ctx, T *res, size_t ld_res, const T *arg, size_t rows,
     int G = 1;
     while (G < 64 && static_cast<size_t>(G) < cols)
         G <<= 1;
-    size_t grid = dh_ceil_div(rows, 256 / G);
+    const size_t oneshot = dh_ceil_div(rows, 256 / G);
+    if (cols <= static_cast<size_t>(G) * 4 && oneshot < (size_t(1) << 31)) {
+        const dim3 grid(static_cast<unsigned>(dh_ceil_div(oneshot, 4))); // four rows per lane group
+        if (cols <= static_cast<size_t>(G))
+            hipLaunchKernelGGL((softmax_reg_kernel<T, 1>), grid, dim3(256), 0, ctx->stream, res, ld_res, arg, rows, cols, ld, G);
+        else
+            hipLaunchKernelGGL((softmax_reg_kernel<T, 4>), grid, dim3(256), 0, ctx->stream, res, ld_res, arg, rows, cols, ld, G);
+        DH_CHECK_LAUNCH();
+        return DH_OK;
+    }
+    size_t grid = oneshot;
     const size_t cap = static_cast<size_t>(ctx->num_cus) * 16;
     if (grid > cap)
         grid = cap;
