@@ -357,10 +357,18 @@ __global__ __launch_bounds__(256) void maxpool_kernel(T *res, const T *data, siz
                                                       unsigned pw, unsigned sh, unsigned sw, unsigned padh,
                                                       unsigned padw) {
     const unsigned PQ = P * Q, HW = H * W;
+    const bool small = total <= 0xffffffffull; // 32-bit divisions suffice (uniform)
     for (size_t idx = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x; idx < total;
          idx += static_cast<size_t>(gridDim.x) * 256) {
-        const size_t plane = idx / PQ;
-        const unsigned pq = static_cast<unsigned>(idx % PQ);
+        size_t plane;
+        unsigned pq;
+        if (small) {
+            plane = static_cast<unsigned>(idx) / PQ;
+            pq = static_cast<unsigned>(idx) % PQ;
+        } else {
+            plane = idx / PQ;
+            pq = static_cast<unsigned>(idx % PQ);
+        }
         const unsigned p = pq / Q, q = pq % Q;
         const T *in = data + plane * HW;
         // window in image coordinates, clipped at the border (Pooling.cpp:77,89,102); the padding
@@ -469,7 +477,7 @@ dh_status maxpool_forward(dh_ctx *ctx, T *res, size_t *res_h, size_t *res_w, con
     if (H * W >= (size_t(1) << 31) || P * Q >= (size_t(1) << 31))
         return dh_fail(DH_ERR_RUNTIME, "Pooling: image extents exceed 2^31 elements");
     size_t grid = dh_ceil_div(total, 256);
-    const size_t cap = static_cast<size_t>(ctx->num_cus) * 32;
+    const size_t cap = size_t(1) << 30; // one output per thread; the loop only matters beyond 2^38 outputs
     if (grid > cap)
         grid = cap;
     constexpr int VI = 16 / sizeof(T);

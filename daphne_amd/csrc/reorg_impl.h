@@ -16,8 +16,8 @@ namespace dh_reorg {
 template <typename T, int VEC, bool FILL>
 __global__ __launch_bounds__(256) void block2d_kernel(T *dst, size_t ld_dst, const T *src, size_t ld_src, size_t rows,
                                                       size_t cvecs, T value) {
-    const size_t cv = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-    const size_t r = static_cast<size_t>(blockIdx.y) * blockDim.y + threadIdx.y;
+    const size_t cv = static_cast<size_t>(blockIdx.y) * blockDim.x + threadIdx.x;
+    const size_t r = static_cast<size_t>(blockIdx.x) * blockDim.y + threadIdx.y; // rows on grid.x: no 65535 limit
     if (cv >= cvecs || r >= rows)
         return;
     T v[VEC];
@@ -56,20 +56,10 @@ static inline dh_status block2d(dh_ctx *ctx, T *dst, size_t ld_dst, const T *src
     while (tx < 256 && tx < cvecs)
         tx <<= 1;
     const unsigned ty = 256 / tx;
-    const size_t gx = dh_ceil_div(cvecs, tx), gy = dh_ceil_div(rows, ty);
-    if (gx >= (size_t(1) << 31) || gy >= 65536) {
-        // very tall blocks: rows go to grid.x in slices of 65535 * ty rows
-        const size_t slice = static_cast<size_t>(65535) * ty;
-        for (size_t r0 = 0; r0 < rows; r0 += slice) {
-            const size_t nr = rows - r0 < slice ? rows - r0 : slice;
-            dh_status st = block2d<T, FILL>(ctx, dst + r0 * ld_dst, ld_dst, FILL ? nullptr : src + r0 * ld_src, ld_src, nr,
-                                            cols, value);
-            if (st != DH_OK)
-                return st;
-        }
-        return DH_OK;
-    }
-    const dim3 grid(static_cast<unsigned>(gx), static_cast<unsigned>(gy)), block(tx, ty);
+    const size_t gcols = dh_ceil_div(cvecs, tx), grows = dh_ceil_div(rows, ty);
+    if (gcols >= 65536 || grows >= (size_t(1) << 31))
+        return dh_fail(DH_ERR_RUNTIME, "matrix extents exceed one launch (%zu x %zu)", rows, cols);
+    const dim3 grid(static_cast<unsigned>(grows), static_cast<unsigned>(gcols)), block(tx, ty);
     if (vec)
         hipLaunchKernelGGL((block2d_kernel<T, V, FILL>), grid, block, 0, ctx->stream, dst, ld_dst, src, ld_src, rows, cvecs,
                            value);
@@ -92,8 +82,8 @@ template <typename T> dh_status fill(dh_ctx *ctx, T *res, size_t ld_res, T value
 template <typename T, int VEC>
 __global__ __launch_bounds__(256) void col_bind_kernel(T *res, size_t ld_res, const T *lhs, size_t ld_lhs, size_t lvecs,
                                                        const T *rhs, size_t ld_rhs, size_t rvecs, size_t rows) {
-    const size_t cv = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-    const size_t r = static_cast<size_t>(blockIdx.y) * blockDim.y + threadIdx.y;
+    const size_t cv = static_cast<size_t>(blockIdx.y) * blockDim.x + threadIdx.x;
+    const size_t r = static_cast<size_t>(blockIdx.x) * blockDim.y + threadIdx.y; // rows on grid.x: no 65535 limit
     if (cv >= lvecs + rvecs || r >= rows)
         return;
     T v[VEC];
@@ -124,16 +114,11 @@ dh_status col_bind(dh_ctx *ctx, T *res, size_t ld_res, const T *lhs, size_t lr, 
         while (tx < 256 && tx < cvecs)
             tx <<= 1;
         const unsigned ty = 256 / tx;
-        const size_t gx = dh_ceil_div(cvecs, tx);
-        const size_t slice = static_cast<size_t>(65535) * ty;
-        if (gx < (size_t(1) << 31)) {
-            for (size_t r0 = 0; r0 < lr; r0 += slice) {
-                const size_t nr = lr - r0 < slice ? lr - r0 : slice;
-                hipLaunchKernelGGL((col_bind_kernel<T, V>), dim3(static_cast<unsigned>(gx), static_cast<unsigned>(dh_ceil_div(nr, ty))),
-                                   dim3(tx, ty), 0, ctx->stream, res + r0 * ld_res, ld_res, lhs + r0 * ld_lhs, ld_lhs, lc / V,
-                                   rhs + r0 * ld_rhs, ld_rhs, rc / V, nr);
-                DH_CHECK_LAUNCH();
-            }
+        const size_t gcols = dh_ceil_div(cvecs, tx), grows = dh_ceil_div(lr, ty);
+        if (gcols < 65536 && grows < (size_t(1) << 31)) {
+            hipLaunchKernelGGL((col_bind_kernel<T, V>), dim3(static_cast<unsigned>(grows), static_cast<unsigned>(gcols)),
+                               dim3(tx, ty), 0, ctx->stream, res, ld_res, lhs, ld_lhs, lc / V, rhs, ld_rhs, rc / V, lr);
+            DH_CHECK_LAUNCH();
             return DH_OK;
         }
     }
@@ -159,8 +144,8 @@ static __global__ void check_sel_kernel(const long long *sel, size_t nsel, size_
 template <typename T>
 __global__ __launch_bounds__(256) void extract_col_kernel(T *res, size_t ld_res, const T *arg, size_t ld, size_t rows,
                                                           size_t cols, const long long *sel, size_t nsel, size_t ld_sel) {
-    const size_t k = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-    const size_t r = static_cast<size_t>(blockIdx.y) * blockDim.y + threadIdx.y;
+    const size_t k = static_cast<size_t>(blockIdx.y) * blockDim.x + threadIdx.x;
+    const size_t r = static_cast<size_t>(blockIdx.x) * blockDim.y + threadIdx.y;
     if (k >= nsel || r >= rows)
         return;
     long long c = sel[k * ld_sel];
@@ -208,15 +193,12 @@ dh_status extract_col(dh_ctx *ctx, T *res, size_t ld_res, const T *arg, size_t r
     while (tx < 256 && tx < sel_rows)
         tx <<= 1;
     const unsigned ty = 256 / tx;
-    const size_t gx = dh_ceil_div(sel_rows, tx);
-    const size_t slice = static_cast<size_t>(65535) * ty;
-    for (size_t r0 = 0; r0 < rows; r0 += slice) {
-        const size_t nr = rows - r0 < slice ? rows - r0 : slice;
-        hipLaunchKernelGGL((extract_col_kernel<T>), dim3(static_cast<unsigned>(gx), static_cast<unsigned>(dh_ceil_div(nr, ty))),
-                           dim3(tx, ty), 0, ctx->stream, res + r0 * ld_res, ld_res, arg + r0 * ld, ld, nr, cols, sel, sel_rows,
-                           ld_sel);
-        DH_CHECK_LAUNCH();
-    }
+    const size_t gcols = dh_ceil_div(sel_rows, tx), grows = dh_ceil_div(rows, ty);
+    if (gcols >= 65536 || grows >= (size_t(1) << 31))
+        return dh_fail(DH_ERR_RUNTIME, "ExtractCol - extents exceed one launch");
+    hipLaunchKernelGGL((extract_col_kernel<T>), dim3(static_cast<unsigned>(grows), static_cast<unsigned>(gcols)), dim3(tx, ty),
+                       0, ctx->stream, res, ld_res, arg, ld, rows, cols, sel, sel_rows, ld_sel);
+    DH_CHECK_LAUNCH();
     return DH_OK;
 }
 
@@ -229,7 +211,7 @@ __global__ __launch_bounds__(256) void transpose_kernel(T *res, size_t ld_res, c
     constexpr int TS = 64;
     __shared__ T tile[TS][TS + 1];
     const int tx = threadIdx.x % TS, ty = threadIdx.x / TS; // 64 x 4
-    const size_t r0 = static_cast<size_t>(blockIdx.y) * TS, c0 = static_cast<size_t>(blockIdx.x) * TS;
+    const size_t r0 = static_cast<size_t>(blockIdx.x) * TS, c0 = static_cast<size_t>(blockIdx.y) * TS;
 #pragma unroll
     for (int i = 0; i < TS; i += 4) {
         const size_t r = r0 + ty + i, c = c0 + tx;
@@ -257,7 +239,7 @@ __global__ __launch_bounds__(256) void transpose_vec_kernel(T *res, size_t ld_re
     constexpr int RPS = 256 / LPR;       // tile rows per step of the workgroup
     __shared__ T tile[TS][TS + 1];
     const int m = threadIdx.x % LPR, q = threadIdx.x / LPR;
-    const size_t r0 = static_cast<size_t>(blockIdx.y) * TS, c0 = static_cast<size_t>(blockIdx.x) * TS;
+    const size_t r0 = static_cast<size_t>(blockIdx.x) * TS, c0 = static_cast<size_t>(blockIdx.y) * TS;
     T v[TS / RPS][VEC];
 #pragma unroll
     for (int s_ = 0; s_ < TS / RPS; s_++) {
@@ -291,24 +273,18 @@ template <typename T> dh_status transpose(dh_ctx *ctx, T *res, size_t ld_res, co
         return dh_fail(DH_ERR_RUNTIME, "Transpose - a leading dimension is smaller than its column count");
     if (rows == 0 || cols == 0)
         return DH_OK;
-    const size_t gx = dh_ceil_div(cols, 64);
-    if (gx >= (size_t(1) << 31))
-        return dh_fail(DH_ERR_RUNTIME, "Transpose - too many columns for one launch");
+    const size_t gcols = dh_ceil_div(cols, 64), grows = dh_ceil_div(rows, 64);
+    if (gcols >= 65536 || grows >= (size_t(1) << 31))
+        return dh_fail(DH_ERR_RUNTIME, "Transpose - extents exceed one launch (%zu x %zu)", rows, cols);
     constexpr int V = 16 / sizeof(T);
     const bool vec = rows % V == 0 && cols % V == 0 && ld % V == 0 && ld_res % V == 0 && dh_aligned(arg, 16) &&
                      dh_aligned(res, 16);
-    const size_t slice = static_cast<size_t>(65535) * 64;
-    for (size_t r0 = 0; r0 < rows; r0 += slice) {
-        const size_t nr = rows - r0 < slice ? rows - r0 : slice;
-        const dim3 grid(static_cast<unsigned>(gx), static_cast<unsigned>(dh_ceil_div(nr, 64)));
-        if (vec)
-            hipLaunchKernelGGL((transpose_vec_kernel<T>), grid, dim3(256), 0, ctx->stream, res + r0, ld_res, arg + r0 * ld, ld,
-                               nr, cols);
-        else
-            hipLaunchKernelGGL((transpose_kernel<T>), grid, dim3(256), 0, ctx->stream, res + r0, ld_res, arg + r0 * ld, ld, nr,
-                               cols);
-        DH_CHECK_LAUNCH();
-    }
+    const dim3 grid(static_cast<unsigned>(grows), static_cast<unsigned>(gcols));
+    if (vec)
+        hipLaunchKernelGGL((transpose_vec_kernel<T>), grid, dim3(256), 0, ctx->stream, res, ld_res, arg, ld, rows, cols);
+    else
+        hipLaunchKernelGGL((transpose_kernel<T>), grid, dim3(256), 0, ctx->stream, res, ld_res, arg, ld, rows, cols);
+    DH_CHECK_LAUNCH();
     return DH_OK;
 }
 
