@@ -827,43 +827,46 @@ template <typename T, int OUT>
 __global__ __launch_bounds__(THREADS) void col_var_stage2(const T *part_mean, const T *part_m2, size_t nparts,
                                                           size_t cols, size_t rows, size_t slab, T *res,
                                                           T *res_mean = nullptr) {
-    // (S2_TX columns, S2_TY partial lanes): every lane merges its share of the per-block
-    // (count, mean, M2) triples with Chan's formula in double, lane 0 then merges the lanes.
-    __shared__ double lds_n[S2_TY][S2_TX], lds_mean[S2_TY][S2_TX], lds_m2[S2_TY][S2_TX];
+    // (S2_TX columns, S2_TY partial lanes). Pooled moments of the per-block (count, mean, M2) triples in double:
+    //     mean = sum n_p mean_p / N,   M2 = sum M2_p + sum n_p (mean_p - mean)^2
+    // - the closed form of merging them pairwise with Chan's formula, without a division per partial.
+    __shared__ double lds_a[S2_TY][S2_TX], lds_b[S2_TY][S2_TX];
     const size_t c = static_cast<size_t>(blockIdx.x) * S2_TX + threadIdx.x;
-    double cn = 0.0, cmean = 0.0, cm2 = 0.0;
-    if (c < cols) {
+    auto count = [&](size_t p) {
+        const size_t r_begin = p * slab;
+        if (r_begin >= rows)
+            return 0.0;
+        return static_cast<double>(((r_begin + slab < rows) ? r_begin + slab : rows) - r_begin);
+    };
+    double s1 = 0.0, s2 = 0.0;
+    if (c < cols)
         for (size_t p = threadIdx.y; p < nparts; p += S2_TY) {
-            const size_t r_begin = p * slab;
-            if (r_begin >= rows)
-                break;
-            const size_t r_end = (r_begin + slab < rows) ? r_begin + slab : rows;
-            const double np_ = static_cast<double>(r_end - r_begin);
-            const double mp = static_cast<double>(part_mean[p * cols + c]);
-            const double qp = static_cast<double>(part_m2[p * cols + c]);
-            const double delta = mp - cmean;
-            const double nt = cn + np_;
-            cmean += delta * np_ / nt;
-            cm2 += qp + delta * delta * cn * np_ / nt;
-            cn = nt;
+            s1 += count(p) * static_cast<double>(part_mean[p * cols + c]);
+            s2 += static_cast<double>(part_m2[p * cols + c]);
         }
+    lds_a[threadIdx.y][threadIdx.x] = s1;
+    lds_b[threadIdx.y][threadIdx.x] = s2;
+    __syncthreads();
+    double tot1 = 0.0, tot2 = 0.0;
+    for (int y = 0; y < S2_TY; y++) {
+        tot1 += lds_a[y][threadIdx.x];
+        tot2 += lds_b[y][threadIdx.x];
     }
-    lds_n[threadIdx.y][threadIdx.x] = cn;
-    lds_mean[threadIdx.y][threadIdx.x] = cmean;
-    lds_m2[threadIdx.y][threadIdx.x] = cm2;
+    const double cmean = tot1 / static_cast<double>(rows);
+    __syncthreads();
+    double s3 = 0.0;
+    if (c < cols)
+        for (size_t p = threadIdx.y; p < nparts; p += S2_TY) {
+            const double d = static_cast<double>(part_mean[p * cols + c]) - cmean;
+            s3 += count(p) * d * d;
+        }
+    lds_a[threadIdx.y][threadIdx.x] = s3;
     __syncthreads();
     if (threadIdx.y != 0 || c >= cols)
         return;
-    for (int y = 1; y < S2_TY; y++) {
-        const double np_ = lds_n[y][threadIdx.x];
-        if (np_ == 0.0)
-            continue;
-        const double delta = lds_mean[y][threadIdx.x] - cmean;
-        const double nt = cn + np_;
-        cmean += delta * np_ / nt;
-        cm2 += lds_m2[y][threadIdx.x] + delta * delta * cn * np_ / nt;
-        cn = nt;
-    }
+    double cm2 = tot2;
+    for (int y = 0; y < S2_TY; y++)
+        cm2 += lds_a[y][threadIdx.x];
     double v = cm2 / static_cast<double>(rows);
     if constexpr (OUT == 1)
         v = sqrt(v);

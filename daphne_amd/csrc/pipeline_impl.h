@@ -17,27 +17,37 @@ bool jit_lookup(int device, const char *tname, int vec, int kv, const dh_pipe_in
                 std::string *err, bool compile_only);
 void jit_set_last_mode(int m);
 
+// Folds the per-workgroup partials of a full reduction. One workgroup of 1024 threads, four independent
+// accumulators per thread so that the loads overlap; the association is fixed by the partial count alone.
+constexpr int STAGE2_THREADS = 1024;
 template <typename T>
-__global__ __launch_bounds__(THREADS) void pipeline_all_stage2(const T *partials, size_t np, int op, T *out) {
-    __shared__ T lds[THREADS / DH_WAVE];
-    T a = (op == DH_AGG_SUM) ? T(0)
-                             : (op == DH_AGG_MIN) ? dh_inf<T>() : -dh_inf<T>();
-    for (size_t i = threadIdx.x; i < np; i += THREADS) {
-        const T v = partials[i];
-        a = (op == DH_AGG_SUM) ? a + v : (op == DH_AGG_MIN) ? ((v < a) ? v : a) : ((a < v) ? v : a);
+__global__ __launch_bounds__(STAGE2_THREADS) void pipeline_all_stage2(const T *partials, size_t np, int op, T *out) {
+    __shared__ T lds[STAGE2_THREADS / DH_WAVE];
+    const T id = (op == DH_AGG_SUM) ? T(0) : (op == DH_AGG_MIN) ? dh_inf<T>() : -dh_inf<T>();
+    auto comb = [op](T a, T v) {
+        return (op == DH_AGG_SUM) ? a + v : (op == DH_AGG_MIN) ? ((v < a) ? v : a) : ((a < v) ? v : a);
+    };
+    T a0 = id, a1 = id, a2 = id, a3 = id;
+    size_t i = threadIdx.x;
+    for (; i + 3 * STAGE2_THREADS < np; i += 4 * STAGE2_THREADS) {
+        const T v0 = partials[i], v1 = partials[i + STAGE2_THREADS], v2 = partials[i + 2 * STAGE2_THREADS],
+                v3 = partials[i + 3 * STAGE2_THREADS];
+        a0 = comb(a0, v0);
+        a1 = comb(a1, v1);
+        a2 = comb(a2, v2);
+        a3 = comb(a3, v3);
     }
-    for (int off = DH_WAVE / 2; off >= 1; off >>= 1) {
-        const T ov = dh_shfl_xor(a, off);
-        a = (op == DH_AGG_SUM) ? a + ov : (op == DH_AGG_MIN) ? ((ov < a) ? ov : a) : ((a < ov) ? ov : a);
-    }
+    for (; i < np; i += STAGE2_THREADS)
+        a0 = comb(a0, partials[i]);
+    T a = comb(comb(a0, a1), comb(a2, a3));
+    for (int off = DH_WAVE / 2; off >= 1; off >>= 1)
+        a = comb(a, dh_shfl_xor(a, off));
     if ((threadIdx.x % DH_WAVE) == 0)
         lds[threadIdx.x / DH_WAVE] = a;
     __syncthreads();
     if (threadIdx.x == 0) {
-        for (int w = 1; w < THREADS / DH_WAVE; w++) {
-            const T ov = lds[w];
-            a = (op == DH_AGG_SUM) ? a + ov : (op == DH_AGG_MIN) ? ((ov < a) ? ov : a) : ((a < ov) ? ov : a);
-        }
+        for (int w = 1; w < STAGE2_THREADS / DH_WAVE; w++)
+            a = comb(a, lds[w]);
         out[0] = a;
     }
 }
@@ -210,7 +220,7 @@ dh_status run(dh_ctx *ctx, const dh_pipe_instr *prog, int n, const IO_C *cio, si
     DH_CHECK_LAUNCH();
     for (int s = 0; s < 2; s++)
         if (reduce_ops[s] != -1) {
-            hipLaunchKernelGGL((pipeline_all_stage2<T>), dim3(1), dim3(THREADS), 0, ctx->stream, partials + s * grid, grid,
+            hipLaunchKernelGGL((pipeline_all_stage2<T>), dim3(1), dim3(STAGE2_THREADS), 0, ctx->stream, partials + s * grid, grid,
                                reduce_ops[s], reduce_out[s]);
             DH_CHECK_LAUNCH();
         }
