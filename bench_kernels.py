@@ -1,5 +1,5 @@
 #!/usr/bin/env python3
-"""Per-kernel throughput survey on one MI355X: every device kernel of the library at a large shape, float and double,
+"""Per-kernel throughput table on one MI355X: every device kernel of the library at a large shape, float and double,
 against the roofline that bounds it (HBM 8 TB/s for the streaming kernels, the dtype's MFMA peak for contractions).
 
     python bench_kernels.py [--reps 20] [--dtype f32|f64|both] [--only group|substring]
