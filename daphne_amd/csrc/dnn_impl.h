@@ -229,6 +229,16 @@ __global__ __launch_bounds__(64 * WN) void conv2d_kernel(ConvArgs g) {
     // out[img][f][pq]: lanes along pixels -> contiguous stores
     T *out = static_cast<T *>(g.res);
     const T *bias = static_cast<const T *>(g.bias);
+    // this lane's bias values first: loaded inside the store loop, every one of them would wait behind the
+    // previous store (the compiler cannot rule out that res and bias overlap)
+    T bv[FM][M::ACC];
+#pragma unroll
+    for (int i = 0; i < FM; i++)
+#pragma unroll
+        for (int v = 0; v < M::ACC; v++) {
+            const size_t f = f0 + i * M::MT + M::row(lane, v);
+            bv[i][v] = (bias && f < g.F) ? bias[f] : T(0);
+        }
 #pragma unroll
     for (int j = 0; j < FN; j++) {
         const size_t pix = pix0 + wave * TN + j * M::NT + M::col(lane);
@@ -248,7 +258,7 @@ __global__ __launch_bounds__(64 * WN) void conv2d_kernel(ConvArgs g) {
                 for (int v = 0; v < M::ACC; v++) {
                     const size_t f = f0 + i * M::MT + M::row(lane, v);
                     if (f < g.F)
-                        obase[f * PQ] = acc[i][j][v] + (bias ? bias[f] : T(0));
+                        obase[f * PQ] = acc[i][j][v] + bv[i][v];
                 }
         }
     }
