@@ -89,4 +89,13 @@ dh_status dh_workspace(dh_ctx *ctx, size_t bytes, void **out);
 static inline size_t dh_ceil_div(size_t a, size_t b) { return (a + b - 1) / b; }
 static inline bool dh_aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
 
+// Lane mapping of a fused pipeline for rows of a given width (pipeline_jit.hip): vec values per load,
+// G lanes per row, KV vectors per lane, U = 4 / KV rows in flight per lane group, S steps per run.
+namespace dh_pipe {
+struct PipeShape {
+    int vec, G, KV, U, S;
+};
+bool pipe_shape(size_t cols, int vec, PipeShape *sh);
+} // namespace dh_pipe
+
 #include "dev_common.h"

@@ -35,7 +35,48 @@ template <typename T> __device__ __forceinline__ T dh_nan();
 template <> __device__ __forceinline__ float dh_nan<float>() { return __builtin_nanf(""); }
 template <> __device__ __forceinline__ double dh_nan<double>() { return __builtin_nan(""); }
 
+// One data-parallel-primitive move of a 32-bit or 64-bit value (CTRL: quad_perm 0x00-0xff,
+// row_half_mirror 0x141, row_mirror 0x140); source lanes that are inactive read as zero.
+template <int CTRL, typename T> __device__ __forceinline__ T dh_dpp(T v) {
+    static_assert(sizeof(T) == 4 || sizeof(T) == 8, "32-bit or 64-bit values only");
+    if constexpr (sizeof(T) == 4) {
+        return __builtin_bit_cast(T, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+    } else {
+        const unsigned long long b = __builtin_bit_cast(unsigned long long, v);
+        const unsigned lo = static_cast<unsigned>(__builtin_amdgcn_update_dpp(0, static_cast<int>(b), CTRL, 0xf, 0xf, true));
+        const unsigned hi = static_cast<unsigned>(__builtin_amdgcn_update_dpp(0, static_cast<int>(b >> 32), CTRL, 0xf, 0xf, true));
+        return __builtin_bit_cast(T, (static_cast<unsigned long long>(hi) << 32) | lo);
+    }
+}
 template <typename T> __device__ __forceinline__ T dh_shfl_xor(T v, int mask) { return __shfl_xor(v, mask, DH_WAVE); }
+
+// Butterfly all-reduce over aligned groups of G lanes (G a power of two <= 64): step(peer) is called
+// once per level, and peer(v) returns the value v of this lane's partner at that level. Below 16
+// lanes the partner is the lane's image under a quad swap or a mirror of the 8 / 16 lanes around it
+// (one register move), above it is lane ^ 16 / lane ^ 32 (through the LDS crossbar). Each level pairs
+// the two halves of a block that the previous levels have made uniform, so after the last one every
+// lane of a group holds the combination of the whole group - provided the combine is commutative.
+// Partners are always in the same group: a group must be wholly active or wholly inactive.
+template <int CTRL> struct dh_peer_dpp {
+    template <typename T> __device__ __forceinline__ T operator()(T v) const { return dh_dpp<CTRL>(v); }
+};
+template <int OFF> struct dh_peer_xor {
+    template <typename T> __device__ __forceinline__ T operator()(T v) const { return __shfl_xor(v, OFF, DH_WAVE); }
+};
+template <class Step> __device__ __forceinline__ void dh_butterfly(int G, Step &&step) {
+    if (G >= 2)
+        step(dh_peer_dpp<0xB1>{}); // quad_perm [1,0,3,2]
+    if (G >= 4)
+        step(dh_peer_dpp<0x4E>{}); // quad_perm [2,3,0,1]
+    if (G >= 8)
+        step(dh_peer_dpp<0x141>{}); // row_half_mirror: lane i of 8 <-> 7 - i
+    if (G >= 16)
+        step(dh_peer_dpp<0x140>{}); // row_mirror: lane i of 16 <-> 15 - i
+    if (G >= 32)
+        step(dh_peer_xor<16>{});
+    if (G >= 64)
+        step(dh_peer_xor<32>{});
+}
 template <typename T> __device__ __forceinline__ T dh_shfl_down(T v, int d) { return __shfl_down(v, d, DH_WAVE); }
 
 // 16-byte (VEC = 16 / sizeof(T)) or scalar (VEC = 1) global load / store into a register array.
@@ -75,3 +116,5 @@ template <typename T, int VEC> __device__ __forceinline__ void dh_load_vec_strea
             v[i] = t[i];
     }
 }
+// Streaming store of one value that this kernel does not read again (results of a pass over a large input).
+template <typename T> __device__ __forceinline__ void dh_store_stream(T *p, T v) { __builtin_nontemporal_store(v, p); }

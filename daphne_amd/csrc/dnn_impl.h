@@ -736,10 +736,10 @@ __global__ __launch_bounds__(256) void softmax_kernel(T *res, size_t ld_res, con
             const T v = in[c];
             mx = (mx < v) ? v : mx;
         }
-        for (int off = G / 2; off >= 1; off >>= 1) {
-            const T o = dh_shfl_xor(mx, off);
+        dh_butterfly(G, [&](auto peer) {
+            const T o = peer(mx);
             mx = (mx < o) ? o : mx;
-        }
+        });
         const T first = in[0];
         if (first != first)
             mx = first;
@@ -749,8 +749,7 @@ __global__ __launch_bounds__(256) void softmax_kernel(T *res, size_t ld_res, con
             out[c] = e;
             sum += e;
         }
-        for (int off = G / 2; off >= 1; off >>= 1)
-            sum += dh_shfl_xor(sum, off);
+        dh_butterfly(G, [&](auto peer) { sum += peer(sum); });
         const T inv = T(1) / sum;
         for (size_t c = lane; c < cols; c += G)
             out[c] *= inv;
@@ -783,10 +782,10 @@ __global__ __launch_bounds__(256) void softmax_reg_kernel(T *res, size_t ld_res,
 #pragma unroll
         for (int k = 0; k < KEEP; k++)
             mx = (mx < x[j][k]) ? x[j][k] : mx; // columns past the end hold -inf
-        for (int off = G / 2; off >= 1; off >>= 1) {
-            const T o = dh_shfl_xor(mx, off);
+        dh_butterfly(G, [&](auto peer) {
+            const T o = peer(mx);
             mx = (mx < o) ? o : mx;
-        }
+        });
         const T first = __shfl(x[j][0], (threadIdx.x % DH_WAVE) - lane, DH_WAVE); // lane 0 of the group holds column 0
         if (first != first)
             mx = first;
@@ -799,8 +798,7 @@ __global__ __launch_bounds__(256) void softmax_reg_kernel(T *res, size_t ld_res,
                 sum += x[j][k];
             }
         }
-        for (int off = G / 2; off >= 1; off >>= 1)
-            sum += dh_shfl_xor(sum, off);
+        dh_butterfly(G, [&](auto peer) { sum += peer(sum); });
         const T inv = T(1) / sum;
         if (r < rows) {
 #pragma unroll

@@ -346,8 +346,7 @@ __global__ __launch_bounds__(256) void gemv_n_kernel(T *y, size_t incy, const T 
         T s = T(0);
         for (size_t c = lane; c < k; c += G)
             s += A[r * lda + c] * x[c * incx];
-        for (int off = G / 2; off >= 1; off >>= 1)
-            s += dh_shfl_xor(s, off);
+        dh_butterfly(G, [&](auto peer) { s += peer(s); });
         if (lane == 0)
             y[r * incy] = s;
     }

@@ -13,35 +13,44 @@ namespace dh_pipe {
 
 // pipeline_jit.hip
 bool jit_enabled();
-bool jit_lookup(int device, const char *tname, int vec, int kv, const dh_pipe_instr *prog, int n, hipFunction_t *fn,
-                std::string *err, bool compile_only);
+bool jit_lookup(int device, const char *tname, int vec, int kv, size_t cols, int G, int S, const dh_pipe_instr *prog, int n,
+                hipFunction_t *fn, std::string *err, bool compile_only);
 void jit_set_last_mode(int m);
 
-// Folds the per-workgroup partials of a full reduction. One workgroup of 1024 threads, four independent
-// accumulators per thread so that the loads overlap; the association is fixed by the partial count alone.
+// Folds the per-workgroup partials of a full reduction. One workgroup of 1024 threads; every thread keeps 16
+// loads in flight (indices past the end are clamped for the load and replaced by the identity afterwards) and
+// four independent accumulators; the association is fixed by the partial count alone.
 constexpr int STAGE2_THREADS = 1024;
 template <typename T>
 __global__ __launch_bounds__(STAGE2_THREADS) void pipeline_all_stage2(const T *partials, size_t np, int op, T *out) {
     __shared__ T lds[STAGE2_THREADS / DH_WAVE];
+    constexpr int UN = 16;
     const T id = (op == DH_AGG_SUM) ? T(0) : (op == DH_AGG_MIN) ? dh_inf<T>() : -dh_inf<T>();
     auto comb = [op](T a, T v) {
         return (op == DH_AGG_SUM) ? a + v : (op == DH_AGG_MIN) ? ((v < a) ? v : a) : ((a < v) ? v : a);
     };
     T a0 = id, a1 = id, a2 = id, a3 = id;
-    size_t i = threadIdx.x;
-    for (; i + 3 * STAGE2_THREADS < np; i += 4 * STAGE2_THREADS) {
-        const T v0 = partials[i], v1 = partials[i + STAGE2_THREADS], v2 = partials[i + 2 * STAGE2_THREADS],
-                v3 = partials[i + 3 * STAGE2_THREADS];
-        a0 = comb(a0, v0);
-        a1 = comb(a1, v1);
-        a2 = comb(a2, v2);
-        a3 = comb(a3, v3);
+    for (size_t i = threadIdx.x; i < np; i += static_cast<size_t>(UN) * STAGE2_THREADS) {
+        T v[UN];
+#pragma unroll
+        for (int k = 0; k < UN; k++) {
+            const size_t j = i + static_cast<size_t>(k) * STAGE2_THREADS;
+            v[k] = partials[j < np ? j : np - 1];
+        }
+#pragma unroll
+        for (int k = 0; k < UN; k++)
+            if (i + static_cast<size_t>(k) * STAGE2_THREADS >= np)
+                v[k] = id;
+#pragma unroll
+        for (int k = 0; k < UN; k += 4) {
+            a0 = comb(a0, v[k]);
+            a1 = comb(a1, v[k + 1]);
+            a2 = comb(a2, v[k + 2]);
+            a3 = comb(a3, v[k + 3]);
+        }
     }
-    for (; i < np; i += STAGE2_THREADS)
-        a0 = comb(a0, partials[i]);
     T a = comb(comb(a0, a1), comb(a2, a3));
-    for (int off = DH_WAVE / 2; off >= 1; off >>= 1)
-        a = comb(a, dh_shfl_xor(a, off));
+    dh_butterfly(DH_WAVE, [&](auto peer) { a = comb(a, peer(a)); });
     if ((threadIdx.x % DH_WAVE) == 0)
         lds[threadIdx.x / DH_WAVE] = a;
     __syncthreads();
@@ -155,23 +164,19 @@ dh_status run(dh_ctx *ctx, const dh_pipe_instr *prog, int n, const IO_C *cio, si
             return dh_fail(DH_ERR_RUNTIME, "vectorizedPipeline: instruction %d: unknown kind %d", i, in.kind);
         }
     }
-    const int vec = vec_ok ? V : 1;
-    const size_t cvecs = cols / vec;
-    int G = 1;
-    while (G < DH_WAVE && static_cast<size_t>(G) < cvecs)
-        G <<= 1;
-    const size_t per_lane = dh_ceil_div(cvecs, G);
-    if (per_lane > 4)
+    PipeShape sh;
+    if (!pipe_shape(cols, vec_ok ? V : 1, &sh))
         return dh_fail(DH_ERR_RUNTIME,
                        "vectorizedPipeline: rows of %zu values do not fit the register tile (at most %d per row here); "
                        "run the operators one by one instead",
-                       cols, 64 * vec * 4);
-    const int KV = per_lane <= 1 ? 1 : (per_lane <= 2 ? 2 : 4);
-    const int U = 4 / KV;
+                       cols, 64 * (vec_ok ? V : 1) * 4);
+    const int vec = sh.vec, G = sh.G, KV = sh.KV, U = sh.U, S = sh.S;
     const size_t groups_per_block = THREADS / G;
-    size_t grid = dh_ceil_div(rows, groups_per_block * U);
-    // measured on the 20M x 64 z-score body: 16 blocks per CU 5.28 TB/s, 64 -> 5.71, 512 -> 4.87
-    const size_t cap = static_cast<size_t>(ctx->num_cus) * 64;
+    // One run of S = 4 steps per wavefront wherever the grid can express it. Measured on the 20M x 64 z-score
+    // body (kernel alone): S = 1 1.05-1.25 ms (set-up and the workgroup fold per 16 rows of a wavefront), S = 2 0.89,
+    // S = 4 0.83-0.86, S = 8 0.85-0.86, S = 16 0.94; S = 4 on a grid capped at 64 workgroups per CU 0.89.
+    size_t grid = dh_ceil_div(rows, groups_per_block * U * S);
+    const size_t cap = 0x7fffffffull;
     if (grid > cap)
         grid = cap;
     void *wsv = nullptr;
@@ -186,7 +191,8 @@ dh_status run(dh_ctx *ctx, const dh_pipe_instr *prog, int n, const IO_C *cio, si
     hipFunction_t jit_fn = nullptr;
     std::string jit_err;
     const bool use_jit = n >= 1 && jit_enabled() &&
-                         jit_lookup(ctx->device, sizeof(T) == 4 ? "float" : "double", vec, KV, P.ins, n, &jit_fn, &jit_err, false);
+                         jit_lookup(ctx->device, sizeof(T) == 4 ? "float" : "double", vec, KV, cols, G, S, P.ins, n, &jit_fn, &jit_err,
+                                    false);
     const dim3 g(static_cast<unsigned>(grid)), b(THREADS);
     if (use_jit) {
         size_t a_rows = rows, a_cols = cols;
@@ -198,7 +204,7 @@ dh_status run(dh_ctx *ctx, const dh_pipe_instr *prog, int n, const IO_C *cio, si
     } else {
         jit_set_last_mode(0);
 #define DH_LAUNCH(VEC_, KV_)                                                                       \
-    hipLaunchKernelGGL((pipeline_kernel<T, VEC_, KV_>), g, b, 0, ctx->stream, P, io, rows, cols, G, partials,        \
+    hipLaunchKernelGGL((pipeline_kernel<T, VEC_, KV_>), g, b, 0, ctx->stream, P, io, rows, cols, G, S, partials,        \
                        ctx->flag_dev)
         if (vec_ok) {
             if (KV == 1)

@@ -123,6 +123,55 @@ template <typename T, int N> __device__ __forceinline__ bool apply_unary(int op,
     return bad;
 }
 
+// t[i] / d[i] for divisors that do not change from step to step (a row-vector operand): the correctly
+// rounded quotient from the same operation sequence as the general division (reciprocal, one / two
+// Newton steps on it, quotient, two / one residual corrections - the sequence the compiler emits for
+// a / b), minus its scaling and special-case handling. That is valid while no operand needs scaling:
+// every |t[i]| and |d[i]| within [2^-40, 2^40] (float) or [2^-300, 2^300] (double). The reciprocal part
+// depends on d alone and moves out of the row loop, which leaves 5 (float) / 3 (double) operations per
+// item instead of 11 / 13. Returns false, having changed nothing, when a value of this wavefront is
+// outside that range (zeros, infinities, subnormals); the caller then divides the ordinary way.
+__device__ __forceinline__ float pipe_abs(float v) { return __builtin_fabsf(v); }
+__device__ __forceinline__ double pipe_abs(double v) { return __builtin_fabs(v); }
+__device__ __forceinline__ float pipe_max(float a, float b) { return __builtin_fmaxf(a, b); }
+__device__ __forceinline__ double pipe_max(double a, double b) { return __builtin_fmax(a, b); }
+__device__ __forceinline__ float pipe_min(float a, float b) { return __builtin_fminf(a, b); }
+__device__ __forceinline__ double pipe_min(double a, double b) { return __builtin_fmin(a, b); }
+template <typename T, int N> __device__ __forceinline__ bool div_by_invariant(T (&t)[N], const T (&d)[N]) {
+    const T hi = sizeof(T) == 4 ? T(0x1p40) : T(0x1p300), lo = sizeof(T) == 4 ? T(0x1p-40) : T(0x1p-300);
+    T tmax = T(0), tmin = hi, dmax = T(0), dmin = hi;
+#pragma unroll
+    for (int i = 0; i < N; i++) {
+        const T at = pipe_abs(t[i]), ad = pipe_abs(d[i]);
+        tmax = pipe_max(tmax, at);
+        tmin = pipe_min(tmin, at);
+        dmax = pipe_max(dmax, ad);
+        dmin = pipe_min(dmin, ad);
+    }
+    const bool ok = tmax <= hi && tmin >= lo && dmax <= hi && dmin >= lo;
+    if (__builtin_amdgcn_ballot_w64(!ok) != 0)
+        return false;
+#pragma unroll
+    for (int i = 0; i < N; i++) {
+        const T n = t[i], b = d[i];
+        if constexpr (sizeof(T) == 4) {
+            const T r0 = __builtin_amdgcn_rcpf(b);
+            const T r = __builtin_fmaf(__builtin_fmaf(-b, r0, 1.0f), r0, r0);
+            const T q0 = n * r;
+            const T q1 = __builtin_fmaf(__builtin_fmaf(-b, q0, n), r, q0);
+            t[i] = __builtin_fmaf(__builtin_fmaf(-b, q1, n), r, q1);
+        } else {
+            const T r0 = __builtin_amdgcn_rcp(b);
+            const T r1 = __builtin_fma(r0, __builtin_fma(-b, r0, 1.0), r0);
+            const T r = __builtin_fma(r1, __builtin_fma(-b, r1, 1.0), r1);
+            const T q0 = n * r;
+            t[i] = __builtin_fma(__builtin_fma(-b, q0, n), r, q0);
+        }
+    }
+    return true;
+}
+
+
 // The instruction source. RuntimeProgram reads the list from the kernel argument (generic
 // interpreter, compiled ahead of time). A program type with is_const = true and a constexpr
 // table makes the same body a straight-line kernel: the instruction loop is fully unrolled and
@@ -136,8 +185,10 @@ struct RuntimeProgram {
 
 // One instantiation per (value type, vector width, vectors per lane, program source). U rows are
 // in flight per lane group so that a lane always holds U*KV*VEC = 16 bytes * 4 of data.
+// G lanes share a row; a wavefront works through runs of S consecutive steps. The run-time
+// specialisation passes cols, G and S as literals, so that everything derived from them folds.
 template <typename T, int VEC, int KV, class PG>
-__device__ __forceinline__ void pipeline_body(const Program &P, const PipeIO<T> &io, size_t rows, size_t cols, int G,
+__device__ __forceinline__ void pipeline_body(const Program &P, const PipeIO<T> &io, size_t rows, size_t cols, int G, int S,
                                                            T *all_partials /* [2][gridDim.x] */, int *flag) {
     constexpr int U = 4 / KV;
     constexpr int N = U * KV * VEC;
@@ -154,8 +205,12 @@ __device__ __forceinline__ void pipeline_body(const Program &P, const PipeIO<T> 
     const int GPW = DH_WAVE / G;            // lane groups (rows) per wavefront and load
     const int g_in_wave = wlane / G;
     const size_t rows_per_step = static_cast<size_t>(GPW) * (4 / KV);
-    const size_t wave_id = static_cast<size_t>(blockIdx.x) * (THREADS / DH_WAVE) + tid / DH_WAVE;
-    const size_t wave_stride = static_cast<size_t>(gridDim.x) * (THREADS / DH_WAVE) * rows_per_step;
+    // wave-uniform values are kept in scalar registers (the index of the wavefront in its workgroup is
+    // uniform, which the compiler cannot see from threadIdx alone)
+    const size_t wave_id = static_cast<size_t>(blockIdx.x) * (THREADS / DH_WAVE) +
+                           static_cast<size_t>(__builtin_amdgcn_readfirstlane(tid / DH_WAVE));
+    const size_t n_waves = static_cast<size_t>(gridDim.x) * (THREADS / DH_WAVE);
+    const size_t rows_per_run = rows_per_step * static_cast<size_t>(S);
     // vmask: does this lane's j-th vector exist in the row? coff: its element offset, clamped
     // into the row so that every load is in bounds without a guard (masked values are never
     // stored, reduced or domain-checked).
@@ -166,6 +221,13 @@ __device__ __forceinline__ void pipeline_body(const Program &P, const PipeIO<T> 
         vmask[j] = static_cast<size_t>(lane + j * G) < cvecs;
         coff[j] = (vmask[j] ? static_cast<size_t>(lane + j * G) : 0) * VEC;
     }
+    // element offset of this lane's (u, j) vector of X from the first row of a step
+    size_t xoff[U][KV];
+#pragma unroll
+    for (int u = 0; u < U; u++)
+#pragma unroll
+        for (int j = 0; j < KV; j++)
+            xoff[u][j] = static_cast<size_t>(u * GPW + g_in_wave) * io.ld_x + coff[j];
     // this lane's share of every bound row-vector operand lives in registers for the whole kernel
     T rv0[KV * VEC], rv1[KV * VEC], rv2[KV * VEC], rv3[KV * VEC];
 #pragma unroll
@@ -189,7 +251,12 @@ __device__ __forceinline__ void pipeline_body(const Program &P, const PipeIO<T> 
         a = (op == DH_AGG_SUM) ? a + v : (op == DH_AGG_MIN) ? ((v < a) ? v : a) : ((a < v) ? v : a);
     };
 
-    for (size_t base = wave_id * rows_per_step; base < rows; base += wave_stride) {
+    for (size_t run = wave_id; run * rows_per_run < rows; run += n_waves)
+#pragma unroll 1
+    for (int sstep = 0; sstep < S; sstep++) {
+        const size_t base = run * rows_per_run + static_cast<size_t>(sstep) * rows_per_step;
+        if (base >= rows)
+            break;
         T t[N], o[N], r[U];
         size_t row[U], lrow[U]; // lrow: row index for loads, clamped to the last row
         bool live[U];
@@ -200,12 +267,13 @@ __device__ __forceinline__ void pipeline_body(const Program &P, const PipeIO<T> 
             lrow[u] = live[u] ? row[u] : rows - 1;
             r[u] = T(0);
         }
+        const T *xbase = io.x + base * io.ld_x; // the step's first row, which always exists
 #pragma unroll
         for (int u = 0; u < U; u++)
 #pragma unroll
             for (int j = 0; j < KV; j++) {
                 T x[VEC];
-                dh_load_vec_stream<T, VEC>(io.x + lrow[u] * io.ld_x + coff[j], x);
+                dh_load_vec_stream<T, VEC>(xbase + (live[u] ? xoff[u][j] : coff[j]), x);
 #pragma unroll
                 for (int e = 0; e < VEC; e++)
                     t[(u * KV + j) * VEC + e] = x[e];
@@ -272,7 +340,10 @@ __device__ __forceinline__ void pipeline_body(const Program &P, const PipeIO<T> 
                                 o[u * KV * VEC + i] = r[u];
                         break;
                     }
-                    apply_binary<T, N>(ins.op, t, o, ins.swap != 0);
+                    // the specialised kernel divides by a row vector with the loop-invariant part hoisted
+                    if (!(PG::is_const && ins.op == DH_BIN_DIV && ins.operand == DH_OPD_ROWVEC && ins.swap == 0 &&
+                          div_by_invariant<T, N>(t, o)))
+                        apply_binary<T, N>(ins.op, t, o, ins.swap != 0);
                 } else {
                     T ov[U];
 #pragma unroll
@@ -327,15 +398,15 @@ __device__ __forceinline__ void pipeline_body(const Program &P, const PipeIO<T> 
                                     bi = idx;
                                 }
                             }
-                        for (int off = G / 2; off >= 1; off >>= 1) {
-                            const T ov = dh_shfl_xor(best, off);
-                            const unsigned oi = dh_shfl_xor(bi, off);
+                        dh_butterfly(G, [&](auto peer) {
+                            const T ov = peer(best);
+                            const unsigned oi = peer(bi);
                             const bool better = is_min ? (ov < best) : (ov > best);
                             if (better || (ov == best && oi < bi)) {
                                 best = ov;
                                 bi = oi;
                             }
-                        }
+                        });
                         if ((first != first) || bi == ~0u)
                             bi = 0;
                         r[u] = static_cast<T>(bi);
@@ -350,10 +421,10 @@ __device__ __forceinline__ void pipeline_body(const Program &P, const PipeIO<T> 
                                 if (vmask[j])
                                     a = is_min ? ((x < a) ? x : a) : ((a < x) ? x : a);
                             }
-                        for (int off = G / 2; off >= 1; off >>= 1) {
-                            const T ov = dh_shfl_xor(a, off);
+                        dh_butterfly(G, [&](auto peer) {
+                            const T ov = peer(a);
                             a = is_min ? ((ov < a) ? ov : a) : ((a < ov) ? ov : a);
-                        }
+                        });
                         r[u] = (first != first) ? first : a;
                     } else if (op == DH_AGG_PROD) {
                         T a = T(1);
@@ -363,8 +434,7 @@ __device__ __forceinline__ void pipeline_body(const Program &P, const PipeIO<T> 
                             for (int e = 0; e < VEC; e++)
                                 if (vmask[j])
                                     a = a * t[(u * KV + j) * VEC + e];
-                        for (int off = G / 2; off >= 1; off >>= 1)
-                            a = a * dh_shfl_xor(a, off);
+                        dh_butterfly(G, [&](auto peer) { a = a * peer(a); });
                         r[u] = a;
                     } else { // SUM MEAN VAR STDDEV
                         T a = T(0);
@@ -374,8 +444,7 @@ __device__ __forceinline__ void pipeline_body(const Program &P, const PipeIO<T> 
                             for (int e = 0; e < VEC; e++)
                                 if (vmask[j])
                                     a = a + t[(u * KV + j) * VEC + e];
-                        for (int off = G / 2; off >= 1; off >>= 1)
-                            a = a + dh_shfl_xor(a, off);
+                        dh_butterfly(G, [&](auto peer) { a = a + peer(a); });
                         if (op != DH_AGG_SUM)
                             a = a / static_cast<T>(cols);
                         if (op == DH_AGG_VAR || op == DH_AGG_STDDEV) {
@@ -389,8 +458,7 @@ __device__ __forceinline__ void pipeline_body(const Program &P, const PipeIO<T> 
                                         const T d = t[(u * KV + j) * VEC + e] - mean;
                                         s = s + d * d;
                                     }
-                            for (int off = G / 2; off >= 1; off >>= 1)
-                                s = s + dh_shfl_xor(s, off);
+                            dh_butterfly(G, [&](auto peer) { s = s + peer(s); });
                             s = s / static_cast<T>(cols);
                             a = (op == DH_AGG_STDDEV) ? dh_ew::dh_sqrt<T>(s) : s;
                         }
@@ -429,10 +497,10 @@ __device__ __forceinline__ void pipeline_body(const Program &P, const PipeIO<T> 
                     const size_t orow = base + static_cast<size_t>(wlane);
                     if (wlane < GPW * U && orow < rows) {
                         if (ins.kind == DH_PIPE_STORE_ROW)
-                            static_cast<T *>(io.out_row[ins.index])[orow * io.ld_out_row[ins.index]] = mine;
+                            dh_store_stream(static_cast<T *>(io.out_row[ins.index]) + orow * io.ld_out_row[ins.index], mine);
                         else
-                            static_cast<uint64_t *>(io.out_row[ins.index])[orow * io.ld_out_row[ins.index]] =
-                                static_cast<uint64_t>(mine);
+                            dh_store_stream(static_cast<uint64_t *>(io.out_row[ins.index]) + orow * io.ld_out_row[ins.index],
+                                            static_cast<uint64_t>(mine));
                     }
                 } else {
                     // fewer than 4 lanes per row: every lane group stores its own results
@@ -491,10 +559,10 @@ __device__ __forceinline__ void pipeline_body(const Program &P, const PipeIO<T> 
         if (!(slot == 0 ? all_init0 : all_init1))
             a = (op == DH_AGG_SUM) ? T(0)
                                    : (op == DH_AGG_MIN) ? dh_inf<T>() : -dh_inf<T>();
-        for (int off = DH_WAVE / 2; off >= 1; off >>= 1) {
-            const T ov = dh_shfl_xor(a, off);
+        dh_butterfly(DH_WAVE, [&](auto peer) {
+            const T ov = peer(a);
             a = (op == DH_AGG_SUM) ? a + ov : (op == DH_AGG_MIN) ? ((ov < a) ? ov : a) : ((a < ov) ? ov : a);
-        }
+        });
         if ((tid % DH_WAVE) == 0)
             lds_red[slot][tid / DH_WAVE] = a;
         __syncthreads();
@@ -513,8 +581,8 @@ __device__ __forceinline__ void pipeline_body(const Program &P, const PipeIO<T> 
 
 template <typename T, int VEC, int KV>
 __global__ __launch_bounds__(THREADS) void pipeline_kernel(Program P, PipeIO<T> io, size_t rows, size_t cols, int G,
-                                                           T *all_partials, int *flag) {
-    pipeline_body<T, VEC, KV, RuntimeProgram>(P, io, rows, cols, G, all_partials, flag);
+                                                           int S, T *all_partials, int *flag) {
+    pipeline_body<T, VEC, KV, RuntimeProgram>(P, io, rows, cols, G, S, all_partials, flag);
 }
 
 } // namespace dh_pipe

@@ -460,9 +460,10 @@ dh_status dh_vectorized_pipeline_f64(dh_ctx *ctx, const dh_pipe_instr *program, 
  * switched off (environment DH_PIPELINE_JIT=0) or fails, a generic kernel interprets the list.
  * Returns how the calling thread's last pipeline ran: 1 specialised, 0 interpreted. */
 int dh_vectorized_pipeline_last_mode(void);
-/* Compiles the specialised kernel of a body without loading or running it (no device needed).
- * value_type 0 = float, 1 = double; vec = items per 16-byte vector or 1; kv = 1, 2 or 4. */
-dh_status dh_vectorized_pipeline_compile_check(int value_type, int vec, int kv,
+/* Compiles the specialised kernel of a body for rows of `cols` values without loading or running
+ * it (no device needed). value_type 0 = float, 1 = double; vectorised != 0: rows are read as
+ * 16-byte vectors (cols a multiple of 4 / 2), as the launch does for aligned operands. */
+dh_status dh_vectorized_pipeline_compile_check(int value_type, size_t cols, int vectorised,
                                                const dh_pipe_instr *program, int num_instr);
 
 #ifdef __cplusplus

@@ -74,7 +74,7 @@ def test_pipeline_body_specialisation_compiles():
                                      OPD_ROWVEC, OPD_SCALAR, OPD_SELF, PipeInstr)
 
     lib = capi.lib()
-    lib.dh_vectorized_pipeline_compile_check.argtypes = [C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_int]
+    lib.dh_vectorized_pipeline_compile_check.argtypes = [C.c_int, C.c_size_t, C.c_int, C.c_void_p, C.c_int]
     zscore = [PipeInstr(kind=KIND_EW_BINARY, op=1, operand=OPD_ROWVEC, index=0),
               PipeInstr(kind=KIND_EW_BINARY, op=3, operand=OPD_ROWVEC, index=1),
               PipeInstr(kind=KIND_EW_BINARY, op=2, operand=OPD_SELF),
@@ -87,7 +87,7 @@ def test_pipeline_body_specialisation_compiles():
                   PipeInstr(kind=KIND_ROW_AGG, op=4), PipeInstr(kind=KIND_STORE_ROW_IDX, index=0),
                   PipeInstr(kind=KIND_ROW_AGG, op=8), PipeInstr(kind=KIND_EW_BINARY, op=3, operand=OPD_ROWREG),
                   PipeInstr(kind=KIND_REDUCE_ALL, op=3, domain=0, index=1)]
-    for prog, vt, vec, kv in ((zscore, 0, 4, 1), (every_kind, 1, 2, 2)):
+    for prog, vt, cols, vectorised in ((zscore, 0, 64, 1), (every_kind, 1, 100, 1), (every_kind, 0, 7, 0)):
         arr = (PipeInstr * len(prog))(*prog)
-        st = lib.dh_vectorized_pipeline_compile_check(vt, vec, kv, C.cast(arr, C.c_void_p), len(prog))
+        st = lib.dh_vectorized_pipeline_compile_check(vt, cols, vectorised, C.cast(arr, C.c_void_p), len(prog))
         assert st == capi.DH_OK, lib.dh_last_error().decode()

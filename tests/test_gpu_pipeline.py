@@ -169,3 +169,41 @@ def test_pipeline_errors(ctx):
         p.run()
     with pytest.raises(capi.DaphneHipError, match="row/column vector"):
         VectorizedPipeline(ctx, x).ewBinary(BinaryOpCode.ADD, DenseMatrix.from_numpy(ctx, np.ones((3, 3), np.float32)))
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("rows,cols", [(4096, 64), (1000, 16), (257, 40), (33, 7), (100, 512)])
+def test_pipeline_division_by_row_vector_is_ieee_division(ctx, dt, rows, cols):
+    """t / rowvec inside a specialised body takes a short division sequence when every operand is well inside the
+    exponent range and the general one otherwise; either way the quotient is the correctly rounded one, bit for bit
+    (numpy divides in IEEE arithmetic, as the reference's CPU and CUDA kernels do)."""
+    rng = np.random.default_rng(rows + cols)
+    # (a) everything in the comfortable range, spread over many binades
+    x = (rng.standard_normal((rows, cols)) * np.exp2(rng.integers(-30, 30, (rows, cols)))).astype(dt)
+    x[x == 0] = 1
+    d = ((rng.random((1, cols)) + 0.5) * np.exp2(rng.integers(-30, 30, (1, cols))) * rng.choice([-1, 1], (1, cols))).astype(dt)
+    # (b) the same with rows that leave the range: zeros of both signs, infinities, NaN, subnormals, huge and tiny values
+    x2 = x.copy()
+    fi = np.finfo(dt)
+    specials = np.array([0.0, -0.0, np.inf, -np.inf, np.nan, fi.tiny / 8, -fi.tiny / 4, fi.max, -fi.max / 3, fi.tiny,
+                         fi.eps, 1 / fi.eps], dtype=dt)
+    idx = rng.integers(0, rows * cols, 200)
+    x2.reshape(-1)[idx] = specials[rng.integers(0, specials.size, idx.size)]
+    # (c) a divisor outside the range
+    d2 = d.copy()
+    d2[0, 0] = fi.tiny / 2
+    d2[0, cols // 2] = fi.max / 2
+    for xa, da in ((x, d), (x2, d), (x, d2), (x2, d2)):
+        X, D = DenseMatrix.from_numpy(ctx, xa), DenseMatrix.from_numpy(ctx, da)
+        p = VectorizedPipeline(ctx, X)
+        p.ewBinary(BinaryOpCode.DIV, D)
+        out = p.storeTile()
+        p.run()
+        assert capi.lib().dh_vectorized_pipeline_last_mode() == 1
+        with np.errstate(all="ignore"):
+            want = xa / da
+        got = out.to_numpy()
+        nan = np.isnan(want)
+        assert np.array_equal(np.isnan(got), nan)
+        assert np.array_equal(got[~nan].view(np.uint32 if dt == np.float32 else np.uint64),
+                              want[~nan].view(np.uint32 if dt == np.float32 else np.uint64))
