@@ -920,28 +920,58 @@ __global__ __launch_bounds__(THREADS) void col_idx_stage1(const T *arg, size_t r
     const size_t cv = static_cast<size_t>(blockIdx.y) * blockDim.x + threadIdx.x;
     const size_t r_begin = static_cast<size_t>(blockIdx.x) * slab;
     const size_t r_end = (r_begin + slab < rows) ? r_begin + slab : rows;
+    // the running index is kept relative to the slab, in 32 bits (the launch checks that a slab is shorter than 2^32 rows)
+    constexpr unsigned NONE = ~0u;
     T best[VEC];
-    unsigned long long bi[VEC];
+    unsigned bk[VEC];
 #pragma unroll
     for (int i = 0; i < VEC; i++) {
         best[i] = worst;
-        bi[i] = ~0ull;
+        bk[i] = NONE;
     }
     if (cv < cvecs) {
-        for (size_t r = r_begin + threadIdx.y; r < r_end; r += blockDim.y) {
+        const size_t step = blockDim.y;
+        const T *col = arg + cv * VEC;
+        size_t r0 = r_begin + threadIdx.y;
+        // rows are visited in ascending order by every thread, so that on equal values the first one stays
+        for (; r0 + (UNROLL - 1) * step < r_end; r0 += step * UNROLL) {
+            T x[UNROLL][VEC];
+#pragma unroll
+            for (int u = 0; u < UNROLL; u++)
+                dh_load_vec_stream<T, VEC>(col + (r0 + u * step) * ld, x[u]);
+#pragma unroll
+            for (int u = 0; u < UNROLL; u++) {
+                const unsigned k = static_cast<unsigned>(r0 - r_begin) + static_cast<unsigned>(u * step);
+#pragma unroll
+                for (int i = 0; i < VEC; i++) {
+                    const bool better = IS_MIN ? (x[u][i] < best[i]) : (x[u][i] > best[i]);
+                    const bool first_seen = (bk[i] == NONE) && !dev_isnan(x[u][i]);
+                    if (better || first_seen) {
+                        best[i] = x[u][i];
+                        bk[i] = k;
+                    }
+                }
+            }
+        }
+        for (; r0 < r_end; r0 += step) {
             T x[VEC];
-            load_vec<T, VEC>(arg + r * ld + cv * VEC, x);
+            dh_load_vec_stream<T, VEC>(col + r0 * ld, x);
+            const unsigned k = static_cast<unsigned>(r0 - r_begin);
 #pragma unroll
             for (int i = 0; i < VEC; i++) {
                 const bool better = IS_MIN ? (x[i] < best[i]) : (x[i] > best[i]);
-                const bool first_seen = (bi[i] == ~0ull) && !dev_isnan(x[i]);
+                const bool first_seen = (bk[i] == NONE) && !dev_isnan(x[i]);
                 if (better || first_seen) {
                     best[i] = x[i];
-                    bi[i] = r;
+                    bk[i] = k;
                 }
             }
         }
     }
+    unsigned long long bi[VEC];
+#pragma unroll
+    for (int i = 0; i < VEC; i++)
+        bi[i] = bk[i] == NONE ? ~0ull : static_cast<unsigned long long>(r_begin) + bk[i];
     const int w = blockDim.x * VEC;
 #pragma unroll
     for (int i = 0; i < VEC; i++) {
@@ -972,20 +1002,45 @@ __global__ __launch_bounds__(THREADS) void col_idx_stage1(const T *arg, size_t r
 template <typename T, bool IS_MIN>
 __global__ __launch_bounds__(THREADS) void col_idx_stage2(const T *part_val, const unsigned long long *part_idx,
                                                           size_t nparts, size_t cols, const T *arg, uint64_t *res) {
-    const size_t c = static_cast<size_t>(blockIdx.x) * THREADS + threadIdx.x;
-    if (c >= cols)
-        return;
-    T b = part_val[c];
-    unsigned long long k = part_idx[c];
-    for (size_t p = 1; p < nparts; p++) {
-        const T ov = part_val[p * cols + c];
-        const unsigned long long oi = part_idx[p * cols + c];
+    // block = (S2_TX columns, S2_TY partial lanes) like col_stage2: each lane merges every S2_TY-th partial with four
+    // loads in flight, the lanes are merged through LDS. The merge (better value, or equal value and lower index) is
+    // associative and commutative, so the result does not depend on the split.
+    __shared__ T lds_v[S2_TY][S2_TX];
+    __shared__ unsigned long long lds_k[S2_TY][S2_TX];
+    const size_t c = static_cast<size_t>(blockIdx.x) * S2_TX + threadIdx.x;
+    T b = IS_MIN ? std::numeric_limits<T>::infinity() : -std::numeric_limits<T>::infinity();
+    unsigned long long k = ~0ull;
+    auto merge = [&](T ov, unsigned long long oi) {
         const bool better = IS_MIN ? (ov < b) : (ov > b);
         if (better || (ov == b && oi < k)) {
             b = ov;
             k = oi;
         }
+    };
+    if (c < cols) {
+        size_t p = threadIdx.y;
+        for (; p + 3 * S2_TY < nparts; p += 4 * S2_TY) {
+            T v[4];
+            unsigned long long id[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                v[u] = part_val[(p + u * S2_TY) * cols + c];
+                id[u] = part_idx[(p + u * S2_TY) * cols + c];
+            }
+#pragma unroll
+            for (int u = 0; u < 4; u++)
+                merge(v[u], id[u]);
+        }
+        for (; p < nparts; p += S2_TY)
+            merge(part_val[p * cols + c], part_idx[p * cols + c]);
     }
+    lds_v[threadIdx.y][threadIdx.x] = b;
+    lds_k[threadIdx.y][threadIdx.x] = k;
+    __syncthreads();
+    if (threadIdx.y != 0 || c >= cols)
+        return;
+    for (int y = 1; y < S2_TY; y++)
+        merge(lds_v[y][threadIdx.x], lds_k[y][threadIdx.x]);
     // AggCol.h:75-91: row 0 seeds the running extremum; a NaN there is never displaced.
     if (dev_isnan(arg[c]) || k == ~0ull)
         k = 0;
@@ -1157,19 +1212,21 @@ template <typename T> dh_status agg_col_idx(dh_ctx *ctx, int op, uint64_t *res, 
     unsigned long long *pidx = static_cast<unsigned long long *>(wsv);
     T *pval = reinterpret_cast<T *>(pidx + p.nparts * cols);
     const size_t lds = static_cast<size_t>(THREADS) * p.vec * (sizeof(T) + sizeof(unsigned long long));
-    const dim3 g2(static_cast<unsigned>(dh_ceil_div(cols, THREADS)));
+    if (p.slab >= 0xffffffffull)
+        return dh_fail(DH_ERR_RUNTIME, "AggCol - more than 2^32 rows per workgroup are not supported");
+    const dim3 g2(static_cast<unsigned>(dh_ceil_div(cols, S2_TX)));
     if (op == DH_AGG_IDXMIN) {
         if (p.vec == V)
             hipLaunchKernelGGL((col_idx_stage1<T, V, true>), p.grid, p.block, lds, ctx->stream, arg, rows, p.cvecs, ld, p.slab, pval, pidx);
         else
             hipLaunchKernelGGL((col_idx_stage1<T, 1, true>), p.grid, p.block, lds, ctx->stream, arg, rows, p.cvecs, ld, p.slab, pval, pidx);
-        hipLaunchKernelGGL((col_idx_stage2<T, true>), g2, dim3(THREADS), 0, ctx->stream, pval, pidx, p.nparts, cols, arg, res);
+        hipLaunchKernelGGL((col_idx_stage2<T, true>), g2, dim3(S2_TX, S2_TY), 0, ctx->stream, pval, pidx, p.nparts, cols, arg, res);
     } else {
         if (p.vec == V)
             hipLaunchKernelGGL((col_idx_stage1<T, V, false>), p.grid, p.block, lds, ctx->stream, arg, rows, p.cvecs, ld, p.slab, pval, pidx);
         else
             hipLaunchKernelGGL((col_idx_stage1<T, 1, false>), p.grid, p.block, lds, ctx->stream, arg, rows, p.cvecs, ld, p.slab, pval, pidx);
-        hipLaunchKernelGGL((col_idx_stage2<T, false>), g2, dim3(THREADS), 0, ctx->stream, pval, pidx, p.nparts, cols, arg, res);
+        hipLaunchKernelGGL((col_idx_stage2<T, false>), g2, dim3(S2_TX, S2_TY), 0, ctx->stream, pval, pidx, p.nparts, cols, arg, res);
     }
     DH_CHECK_LAUNCH();
     return DH_OK;

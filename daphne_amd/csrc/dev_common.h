@@ -116,5 +116,18 @@ template <typename T, int VEC> __device__ __forceinline__ void dh_load_vec_strea
             v[i] = t[i];
     }
 }
+// Streaming counterpart of dh_store_vec for results that this kernel does not read again.
+template <typename T, int VEC> __device__ __forceinline__ void dh_store_vec_stream(T *p, const T (&v)[VEC]) {
+    if constexpr (VEC == 1) {
+        __builtin_nontemporal_store(v[0], p);
+    } else {
+        using V = typename dh_native_vec<T>::type;
+        V t;
+#pragma unroll
+        for (int i = 0; i < VEC; i++)
+            t[i] = v[i];
+        __builtin_nontemporal_store(t, reinterpret_cast<V *>(p));
+    }
+}
 // Streaming store of one value that this kernel does not read again (results of a pass over a large input).
 template <typename T> __device__ __forceinline__ void dh_store_stream(T *p, T v) { __builtin_nontemporal_store(v, p); }

@@ -650,7 +650,7 @@ __global__ __launch_bounds__(256) void channel_kernel(T *res, const T *data, siz
                 for (int i = 0; i < VEC; i++)
                     o[i] = x[i] + b;
             }
-            dh_store_vec<T, VEC>(res + r * HW + cv * VEC, o);
+            dh_store_vec_stream<T, VEC>(res + r * HW + cv * VEC, o);
         }
     }
 }

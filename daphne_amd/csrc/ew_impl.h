@@ -103,7 +103,7 @@ __global__ __launch_bounds__(EW_THREADS) void ew_kernel(T *res, size_t ld_res, c
                     any_bad |= F<T>::bad(a[i]);
             }
         }
-        dh_store_vec<T, VEC>(res + r * ld_res + c, o);
+        dh_store_vec_stream<T, VEC>(res + r * ld_res + c, o);
     }
     if constexpr (MODE == UNARY) {
         if constexpr (F<T>::checks) {

@@ -262,7 +262,7 @@ __global__ __launch_bounds__(256) void transpose_vec_kernel(T *res, size_t ld_re
         for (int e = 0; e < VEC; e++)
             o[e] = tile[m * VEC + e][cq];
         if (orow < cols && ocol < rows)
-            dh_store_vec<T, VEC>(res + orow * ld_res + ocol, o);
+            dh_store_vec_stream<T, VEC>(res + orow * ld_res + ocol, o);
     }
 }
 
