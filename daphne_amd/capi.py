@@ -80,6 +80,20 @@ def _signatures(lib: C.CDLL) -> None:
             fn = getattr(lib, f"{name}_{suf}", None)
             if fn is not None:
                 fn.argtypes = [ct if a == "T" else a for a in at]
+    # integer value types: elementwise for all four, aggregations and data reorganisation for 64-bit ones
+    for suf, ct in (("si64", C.c_int64), ("ui64", C.c_uint64), ("si32", C.c_int32), ("ui32", C.c_uint32)):
+        getattr(lib, f"dh_ew_binary_{suf}").argtypes = [ctxp, i32, vp, sz, vp, sz, sz, sz, vp, sz, sz, sz]
+        getattr(lib, f"dh_ew_binary_sca_{suf}").argtypes = [ctxp, i32, vp, sz, vp, sz, sz, sz, ct]
+    lib.dh_agg_all_si64.argtypes = [ctxp, i32, vp, sz, sz, sz, C.POINTER(C.c_int64)]
+    lib.dh_agg_row_si64.argtypes = [ctxp, i32, vp, sz, vp, sz, sz, sz]
+    lib.dh_agg_row_idx_si64.argtypes = [ctxp, i32, vp, sz, vp, sz, sz, sz]
+    lib.dh_agg_col_si64.argtypes = [ctxp, i32, vp, vp, sz, sz, sz]
+    lib.dh_agg_col_idx_si64.argtypes = [ctxp, i32, vp, vp, sz, sz, sz]
+    lib.dh_fill_si64.argtypes = [ctxp, vp, sz, C.c_int64, sz, sz]
+    lib.dh_fill_ui64.argtypes = [ctxp, vp, sz, C.c_uint64, sz, sz]
+    lib.dh_col_bind_si64.argtypes = _LATE_SIGNATURES["dh_col_bind"]
+    lib.dh_extract_col_si64.argtypes = _LATE_SIGNATURES["dh_extract_col"]
+    lib.dh_transpose_si64.argtypes = _LATE_SIGNATURES["dh_transpose"]
 
 
 # Entry points added after the first kernels; bound when the library exports them.

@@ -201,6 +201,31 @@ DH_OVERLOAD2(dh_extract_col)
 DH_OVERLOAD2(dh_transpose)
 DH_OVERLOAD2(dh_gemv)
 #undef DH_OVERLOAD2
+// integer value types, as far as the reference instantiates its device kernels for them
+// (kernels/CUDA/EwBinaryMat.cu:267-270, EwBinaryObjSca.cu:91-94, AggAll.cu:155, AggRow.cu:146, AggCol.cu:89,
+// Fill.cu:47,49, ColBind.cu:75, ExtractCol.cu:58); any other combination fails to compile, like a missing
+// instantiation fails to link there
+#define DH_OVERLOAD_INT(NAME, SUF, T)                                                                                   \
+    template <typename... A> inline dh_status NAME(T, A... a) { return NAME##_##SUF(a...); }
+DH_OVERLOAD_INT(dh_ew_binary, si64, int64_t)
+DH_OVERLOAD_INT(dh_ew_binary, ui64, uint64_t)
+DH_OVERLOAD_INT(dh_ew_binary, si32, int32_t)
+DH_OVERLOAD_INT(dh_ew_binary, ui32, uint32_t)
+DH_OVERLOAD_INT(dh_ew_binary_sca, si64, int64_t)
+DH_OVERLOAD_INT(dh_ew_binary_sca, ui64, uint64_t)
+DH_OVERLOAD_INT(dh_ew_binary_sca, si32, int32_t)
+DH_OVERLOAD_INT(dh_ew_binary_sca, ui32, uint32_t)
+DH_OVERLOAD_INT(dh_agg_all, si64, int64_t)
+DH_OVERLOAD_INT(dh_agg_row, si64, int64_t)
+DH_OVERLOAD_INT(dh_agg_row_idx, si64, int64_t)
+DH_OVERLOAD_INT(dh_agg_col, si64, int64_t)
+DH_OVERLOAD_INT(dh_agg_col_idx, si64, int64_t)
+DH_OVERLOAD_INT(dh_fill, si64, int64_t)
+DH_OVERLOAD_INT(dh_fill, ui64, uint64_t)
+DH_OVERLOAD_INT(dh_col_bind, si64, int64_t)
+DH_OVERLOAD_INT(dh_extract_col, si64, int64_t)
+DH_OVERLOAD_INT(dh_transpose, si64, int64_t)
+#undef DH_OVERLOAD_INT
 
 // --- EwBinaryMat (kernels/CUDA/EwBinaryMat.h:31-47) ---------------------------------------
 template <class DTRes, class DTLhs, class DTRhs> struct EwBinaryMat {

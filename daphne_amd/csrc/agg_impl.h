@@ -40,18 +40,27 @@ template <typename T> struct RProd {
     static __device__ __forceinline__ T id() { return T(1); }
     static __device__ __forceinline__ T comb(T a, T b) { return a * b; }
 };
+// identity of MIN (largest) / MAX (smallest): the infinities, or the extreme values of an integer type
+template <typename T> __device__ __forceinline__ constexpr T agg_largest() {
+    return std::numeric_limits<T>::is_integer ? std::numeric_limits<T>::max() : std::numeric_limits<T>::infinity();
+}
+template <typename T> __device__ __forceinline__ constexpr T agg_smallest() {
+    return std::numeric_limits<T>::is_integer ? std::numeric_limits<T>::lowest() : -std::numeric_limits<T>::infinity();
+}
+template <typename T> constexpr bool agg_is_int = std::numeric_limits<T>::is_integer;
 template <typename T> struct RMin {
-    static __device__ __forceinline__ T id() { return std::numeric_limits<T>::infinity(); }
+    static __device__ __forceinline__ T id() { return agg_largest<T>(); }
     static __device__ __forceinline__ T comb(T a, T b) { return (b < a) ? b : a; }
 };
 template <typename T> struct RMax {
-    static __device__ __forceinline__ T id() { return -std::numeric_limits<T>::infinity(); }
+    static __device__ __forceinline__ T id() { return agg_smallest<T>(); }
     static __device__ __forceinline__ T comb(T a, T b) { return (a < b) ? b : a; }
 };
 
 template <typename T> __device__ __forceinline__ T dev_sqrt(T a);
 template <> __device__ __forceinline__ float dev_sqrt<float>(float a) { return sqrtf(a); }
 template <> __device__ __forceinline__ double dev_sqrt<double>(double a) { return sqrt(a); }
+template <> __device__ __forceinline__ long dev_sqrt<long>(long a) { return static_cast<long>(sqrt(static_cast<double>(a))); }
 template <typename T> __device__ __forceinline__ bool dev_isnan(T a) { return a != a; }
 
 template <typename T, int VEC> __device__ __forceinline__ void load_vec(const T *p, T (&v)[VEC]) {
@@ -235,6 +244,12 @@ template <typename T> dh_status agg_all_dev(dh_ctx *ctx, int op, const T *arg, s
         return dh_fail(DH_ERR_RUNTIME, "AggAll - leading dimension smaller than the column count");
     if (op == DH_AGG_IDXMIN || op == DH_AGG_IDXMAX || op < 0 || op > DH_AGG_VAR)
         return dh_fail(DH_ERR_RUNTIME, "unsupported AggOpCode"); // AggAll.h:147,161
+    if constexpr (agg_is_int<T>) {
+        // The reference's integer MEAN / VAR / STDDEV divide and subtract in integer arithmetic (AggAll.h:163-191);
+        // its device library has SUM / MIN / MAX for si64 only (CUDA/AggAll.cu:155, AggRow.cu:146, AggCol.cu:89).
+        if (op == DH_AGG_MEAN || op == DH_AGG_VAR || op == DH_AGG_STDDEV)
+            return dh_fail(DH_ERR_RUNTIME, "%s: MEAN, VAR and STDDEV of integer value types are not supported on the device", __func__);
+    }
     void *wsv = nullptr;
     const size_t max_partials = static_cast<size_t>(ctx->num_cus) * 8 * 2 + 1024 + 16;
     dh_status st = dh_workspace(ctx, (max_partials + 64) * sizeof(T), &wsv);
@@ -457,7 +472,7 @@ __global__ __launch_bounds__(THREADS) void row_idx_kernel(uint64_t *res, size_t 
     const size_t rows_per_step = static_cast<size_t>(GPW) * UR;
     const size_t wave_id = static_cast<size_t>(blockIdx.x) * (THREADS / DH_WAVE) + tid / DH_WAVE;
     const size_t wave_stride = static_cast<size_t>(gridDim.x) * (THREADS / DH_WAVE) * rows_per_step;
-    const T worst = IS_MIN ? std::numeric_limits<T>::infinity() : -std::numeric_limits<T>::infinity();
+    const T worst = IS_MIN ? agg_largest<T>() : agg_smallest<T>();
     for (size_t base = wave_id * rows_per_step; base < rows; base += wave_stride) {
         const T *row[UR];
         T best[UR];
@@ -580,6 +595,12 @@ template <typename T> dh_status agg_row(dh_ctx *ctx, int op, T *res, size_t ld_r
         return DH_OK;
     if (cols == 0)
         return dh_fail(DH_ERR_RUNTIME, "AggRow - the argument has no columns");
+    if constexpr (agg_is_int<T>) {
+        // The reference's integer MEAN / VAR / STDDEV divide and subtract in integer arithmetic (AggAll.h:163-191);
+        // its device library has SUM / MIN / MAX for si64 only (CUDA/AggAll.cu:155, AggRow.cu:146, AggCol.cu:89).
+        if (op == DH_AGG_MEAN || op == DH_AGG_VAR || op == DH_AGG_STDDEV)
+            return dh_fail(DH_ERR_RUNTIME, "%s: MEAN, VAR and STDDEV of integer value types are not supported on the device", __func__);
+    }
     switch (op) {
     case DH_AGG_SUM:
         row_launch<T, RSum<T>, 0, false>(ctx, res, ld_res, arg, rows, cols, ld);
@@ -916,7 +937,7 @@ __global__ __launch_bounds__(THREADS) void col_idx_stage1(const T *arg, size_t r
     extern __shared__ unsigned char lds_raw[];
     unsigned long long *lds_idx = reinterpret_cast<unsigned long long *>(lds_raw);        // [TY][TX*VEC]
     T *lds_val = reinterpret_cast<T *>(lds_idx + blockDim.y * blockDim.x * VEC);          // [TY][TX*VEC]
-    const T worst = IS_MIN ? std::numeric_limits<T>::infinity() : -std::numeric_limits<T>::infinity();
+    const T worst = IS_MIN ? agg_largest<T>() : agg_smallest<T>();
     const size_t cv = static_cast<size_t>(blockIdx.y) * blockDim.x + threadIdx.x;
     const size_t r_begin = static_cast<size_t>(blockIdx.x) * slab;
     const size_t r_end = (r_begin + slab < rows) ? r_begin + slab : rows;
@@ -1008,7 +1029,7 @@ __global__ __launch_bounds__(THREADS) void col_idx_stage2(const T *part_val, con
     __shared__ T lds_v[S2_TY][S2_TX];
     __shared__ unsigned long long lds_k[S2_TY][S2_TX];
     const size_t c = static_cast<size_t>(blockIdx.x) * S2_TX + threadIdx.x;
-    T b = IS_MIN ? std::numeric_limits<T>::infinity() : -std::numeric_limits<T>::infinity();
+    T b = IS_MIN ? agg_largest<T>() : agg_smallest<T>();
     unsigned long long k = ~0ull;
     auto merge = [&](T ov, unsigned long long oi) {
         const bool better = IS_MIN ? (ov < b) : (ov > b);
@@ -1107,6 +1128,12 @@ template <typename T> dh_status agg_col(dh_ctx *ctx, int op, T *res, const T *ar
         return DH_OK;
     if (rows == 0)
         return dh_fail(DH_ERR_RUNTIME, "AggCol - the argument has no rows");
+    if constexpr (agg_is_int<T>) {
+        // The reference's integer MEAN / VAR / STDDEV divide and subtract in integer arithmetic (AggAll.h:163-191);
+        // its device library has SUM / MIN / MAX for si64 only (CUDA/AggAll.cu:155, AggRow.cu:146, AggCol.cu:89).
+        if (op == DH_AGG_MEAN || op == DH_AGG_VAR || op == DH_AGG_STDDEV)
+            return dh_fail(DH_ERR_RUNTIME, "%s: MEAN, VAR and STDDEV of integer value types are not supported on the device", __func__);
+    }
     dh_status st = DH_OK;
     switch (op) {
     case DH_AGG_SUM:

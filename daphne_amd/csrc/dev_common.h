@@ -18,14 +18,49 @@ template <> struct dh_vec<double> {
     static constexpr int N = 2;
 };
 
+// integer value types (the reference instantiates its elementwise kernels for si64 / ui64 / si32 / ui32 and its
+// aggregations for si64, kernels/CUDA/EwBinaryMat.cu:265-270, AggAll.cu:153-155)
+template <> struct dh_vec<int> {
+    using type = int4;
+    static constexpr int N = 4;
+};
+template <> struct dh_vec<unsigned> {
+    using type = uint4;
+    static constexpr int N = 4;
+};
+template <> struct dh_vec<long> {
+    using type = longlong2;
+    static constexpr int N = 2;
+};
+template <> struct dh_vec<unsigned long> {
+    using type = ulonglong2;
+    static constexpr int N = 2;
+};
+
 typedef float dh_f32x4_native __attribute__((ext_vector_type(4)));
 typedef double dh_f64x2_native __attribute__((ext_vector_type(2)));
+typedef int dh_i32x4_native __attribute__((ext_vector_type(4)));
+typedef unsigned dh_u32x4_native __attribute__((ext_vector_type(4)));
+typedef long dh_i64x2_native __attribute__((ext_vector_type(2)));
+typedef unsigned long dh_u64x2_native __attribute__((ext_vector_type(2)));
 template <typename T> struct dh_native_vec;
 template <> struct dh_native_vec<float> {
     using type = dh_f32x4_native;
 };
 template <> struct dh_native_vec<double> {
     using type = dh_f64x2_native;
+};
+template <> struct dh_native_vec<int> {
+    using type = dh_i32x4_native;
+};
+template <> struct dh_native_vec<unsigned> {
+    using type = dh_u32x4_native;
+};
+template <> struct dh_native_vec<long> {
+    using type = dh_i64x2_native;
+};
+template <> struct dh_native_vec<unsigned long> {
+    using type = dh_u64x2_native;
 };
 
 template <typename T> __device__ __forceinline__ T dh_inf();

@@ -98,22 +98,31 @@ __global__ __launch_bounds__(EW_THREADS) void ew_kernel(T *res, size_t ld_res, c
 #pragma unroll
         for (int i = 0; i < VEC; i++) {
             o[i] = F<T>::apply(a[i], b[i]);
-            if constexpr (MODE == UNARY) {
-                if constexpr (F<T>::checks)
+            if constexpr (F<T>::checks) {
+                if constexpr (MODE == UNARY)
                     any_bad |= F<T>::bad(a[i]);
+                else
+                    any_bad |= F<T>::bad(a[i], b[i]);
             }
         }
         dh_store_vec_stream<T, VEC>(res + r * ld_res + c, o);
     }
-    if constexpr (MODE == UNARY) {
-        if constexpr (F<T>::checks) {
-            if (any_bad)
-                *flag = 1;
-        }
+    if constexpr (F<T>::checks) {
+        if (any_bad)
+            *flag = 1;
     }
 }
 
 static __global__ void set_flag_kernel(int *flag, int v) { *flag = v; }
+
+// C++ names of the value types as the reference prints them (ValueTypeUtils::cppNameFor)
+template <typename T> static inline const char *type_name();
+template <> inline const char *type_name<float>() { return "float"; }
+template <> inline const char *type_name<double>() { return "double"; }
+template <> inline const char *type_name<int>() { return "int32_t"; }
+template <> inline const char *type_name<unsigned>() { return "uint32_t"; }
+template <> inline const char *type_name<long>() { return "int64_t"; }
+template <> inline const char *type_name<unsigned long>() { return "uint64_t"; }
 
 // ---------------------------------------------------------------------------------------
 // host-side launch
@@ -191,9 +200,13 @@ static inline void launch(dh_ctx *ctx, T *res, size_t ld_res, const T *lhs, size
 template <typename T, int MODE>
 static inline dh_status dispatch_binary(dh_ctx *ctx, int op, T *res, size_t ld_res, const T *lhs, size_t ld_lhs,
                                         const T *rhs, size_t ld_rhs, T sca, size_t rows, size_t cols) {
+    // integer DIV and MOD report operands that have no integer result (see ew_ops.h) through the context's flag
+    const bool checks = dh_is_int<T>::value && (op == DH_BIN_DIV || op == DH_BIN_MOD);
+    if (checks)
+        hipLaunchKernelGGL(set_flag_kernel, dim3(1), dim3(1), 0, ctx->stream, ctx->flag_dev, 0);
 #define DH_CASE(CODE, FUN)                                                                         \
     case CODE:                                                                                     \
-        launch<T, FUN, MODE>(ctx, res, ld_res, lhs, ld_lhs, rhs, ld_rhs, sca, rows, cols, nullptr); \
+        launch<T, FUN, MODE>(ctx, res, ld_res, lhs, ld_lhs, rhs, ld_rhs, sca, rows, cols, ctx->flag_dev); \
         break;
     switch (op) {
         DH_CASE(DH_BIN_ADD, BAdd)
@@ -217,14 +230,20 @@ static inline dh_status dispatch_binary(dh_ctx *ctx, int op, T *res, size_t ld_r
     case DH_BIN_CONCAT:
         // EwBinarySca.h:75-77: the op exists but is not supported on these value types.
         return dh_fail(DH_ERR_RUNTIME, "the binary operation %s is not supported on the value types %s (res), %s (lhs), and %s (rhs)",
-                       op == DH_BIN_CONCAT ? "CONCAT" : "BITWISE_AND", sizeof(T) == 4 ? "float" : "double",
-                       sizeof(T) == 4 ? "float" : "double", sizeof(T) == 4 ? "float" : "double");
+                       op == DH_BIN_CONCAT ? "CONCAT" : "BITWISE_AND", type_name<T>(), type_name<T>(), type_name<T>());
     default:
         // EwBinarySca.h:73
         return dh_fail(DH_ERR_RUNTIME, "unknown BinaryOpCode: %d", op);
     }
 #undef DH_CASE
     DH_CHECK_LAUNCH();
+    if (checks) {
+        DH_CHECK_HIP(hipMemcpyAsync(ctx->flag_host, ctx->flag_dev, sizeof(int), hipMemcpyDeviceToHost, ctx->stream));
+        DH_CHECK_HIP(hipStreamSynchronize(ctx->stream));
+        if (*ctx->flag_host != 0)
+            return dh_fail(DH_ERR_DOMAIN, "integer %s: a divisor is zero%s", op == DH_BIN_DIV ? "division" : "remainder",
+                           op == DH_BIN_DIV ? " or the quotient does not fit the value type" : "");
+    }
     return DH_OK;
 }
 
@@ -295,8 +314,7 @@ dh_status ew_unary(dh_ctx *ctx, int op, T *res, size_t ld_res, const T *arg, siz
     case DH_UN_LOWER:
         // EwUnarySca.h:104-107
         return dh_fail(DH_ERR_RUNTIME, "the unary operation %s is not supported on the value types %s (res) and %s(arg)",
-                       op == DH_UN_UPPER ? "UPPER" : "LOWER", sizeof(T) == 4 ? "float" : "double",
-                       sizeof(T) == 4 ? "float" : "double");
+                       op == DH_UN_UPPER ? "UPPER" : "LOWER", type_name<T>(), type_name<T>());
     default:
         // EwUnarySca.h:102
         return dh_fail(DH_ERR_RUNTIME, "unknown UnaryOpCode: %d", op);

@@ -38,17 +38,78 @@ template <typename T> __device__ __forceinline__ T dh_fmod(T a, T b);
 template <> __device__ __forceinline__ float dh_fmod<float>(float a, float b) { return fmodf(a, b); }
 template <> __device__ __forceinline__ double dh_fmod<double>(double a, double b) { return fmod(a, b); }
 
-#define DH_BIN_FUNCTOR(NAME, EXPR)                                                                 \
+// Floating-point value types evaluate the expressions of EwBinarySca.h:143-167 directly. Integer value types go
+// the way C++ takes for the same expressions: pow / fmod / log promote both operands to double and the result is
+// converted back (truncated); comparisons and logic give 0 / 1. An integer division or remainder by zero, and the
+// signed overflow INT_MIN / -1, stop the reference's process with a hardware trap; here bad() reports them and the
+// call fails with a domain error. Conversions of out-of-range or NaN doubles back to an integer are undefined in
+// C++ and unspecified here.
+template <typename T> struct dh_is_int {
+    static constexpr bool value = false;
+};
+template <> struct dh_is_int<int> {
+    static constexpr bool value = true;
+};
+template <> struct dh_is_int<unsigned> {
+    static constexpr bool value = true;
+};
+template <> struct dh_is_int<long> {
+    static constexpr bool value = true;
+};
+template <> struct dh_is_int<unsigned long> {
+    static constexpr bool value = true;
+};
+template <typename T> __device__ __forceinline__ bool dh_int_div_traps(T a, T b) {
+    if constexpr (!dh_is_int<T>::value) {
+        return false;
+    } else {
+        if (b == T(0))
+            return true;
+        if constexpr (T(-1) < T(0)) // signed: the most negative value divided by -1 does not fit
+            return b == T(-1) && a == static_cast<T>(T(1) << (sizeof(T) * 8 - 1));
+        return false;
+    }
+}
+template <typename T> __device__ __forceinline__ T dh_pow_any(T a, T b) {
+    if constexpr (!dh_is_int<T>::value) {
+        return dh_pow<T>(a, b);
+    } else {
+        // The exact power of two integers is an integer; where it fits the 53 bits of a double, a correctly rounded
+        // pow() returns exactly that. Rounding to the nearest integer removes the last-bit error a device pow() may
+        // have there (negative exponents give |result| <= 1, which truncates as it stands).
+        const double r = pow(static_cast<double>(a), static_cast<double>(b));
+        return static_cast<T>((b >= T(0)) ? rint(r) : r);
+    }
+}
+template <typename T> __device__ __forceinline__ T dh_mod_any(T a, T b) {
+    if constexpr (!dh_is_int<T>::value)
+        return dh_fmod<T>(a, b);
+    else
+        return static_cast<T>(fmod(static_cast<double>(a), static_cast<double>(b))); // exact in double, as on the host
+}
+template <typename T> __device__ __forceinline__ T dh_log_any(T a, T b) {
+    if constexpr (!dh_is_int<T>::value)
+        return dh_log<T>(a) / dh_log<T>(b);
+    else
+        return static_cast<T>(log(static_cast<double>(a)) / log(static_cast<double>(b)));
+}
+
+#define DH_BIN_FUNCTOR_C(NAME, EXPR, CHK, BAD)                                                     \
     template <typename T> struct NAME {                                                            \
+        static constexpr bool checks = dh_is_int<T>::value && (CHK);                               \
         static __device__ __forceinline__ T apply(T a, T b) { return EXPR; }                       \
+        static __device__ __forceinline__ bool bad(T a, T b) { return (BAD); }                     \
     };
+#define DH_BIN_FUNCTOR(NAME, EXPR) DH_BIN_FUNCTOR_C(NAME, EXPR, false, false)
 DH_BIN_FUNCTOR(BAdd, a + b)
 DH_BIN_FUNCTOR(BSub, a - b)
 DH_BIN_FUNCTOR(BMul, a *b)
-DH_BIN_FUNCTOR(BDiv, a / b) // IEEE division, as the CPU kernel; the CUDA kernel multiplies by 1/b
-DH_BIN_FUNCTOR(BPow, dh_pow<T>(a, b))
-DH_BIN_FUNCTOR(BMod, dh_fmod<T>(a, b))
-DH_BIN_FUNCTOR(BLog, dh_log<T>(a) / dh_log<T>(b))
+// IEEE division, as the CPU kernel (the CUDA kernel multiplies by 1/b); a trapping integer division yields 0 and is reported
+DH_BIN_FUNCTOR_C(BDiv, (dh_int_div_traps<T>(a, b) ? T(0) : a / b), true, dh_int_div_traps<T>(a, b))
+DH_BIN_FUNCTOR(BPow, dh_pow_any<T>(a, b))
+// fmod(a, 0) is NaN, which no integer can hold: reported like the division
+DH_BIN_FUNCTOR_C(BMod, ((dh_is_int<T>::value && b == T(0)) ? T(0) : dh_mod_any<T>(a, b)), true, (b == T(0)))
+DH_BIN_FUNCTOR(BLog, dh_log_any<T>(a, b))
 DH_BIN_FUNCTOR(BEq, static_cast<T>(a == b))
 DH_BIN_FUNCTOR(BNeq, static_cast<T>(a != b))
 DH_BIN_FUNCTOR(BLt, static_cast<T>(a < b))
@@ -60,6 +121,7 @@ DH_BIN_FUNCTOR(BMax, (a < b) ? b : a) // std::max(a, b)
 DH_BIN_FUNCTOR(BAnd, static_cast<T>((a != T(0)) && (b != T(0))))
 DH_BIN_FUNCTOR(BOr, static_cast<T>((a != T(0)) || (b != T(0))))
 #undef DH_BIN_FUNCTOR
+#undef DH_BIN_FUNCTOR_C
 
 template <typename T> __device__ __forceinline__ T dh_sign(T a) {
     return (a == T(0)) ? T(0) : ((a < T(0)) ? T(-1) : ((a > T(0)) ? T(1) : dh_nan<T>()));

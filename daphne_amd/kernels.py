@@ -35,7 +35,10 @@ class AggOpCode(enum.IntEnum):  # runtime/local/kernels/AggOpCode.h:25-35
     SUM = 0; PROD = 1; MIN = 2; MAX = 3; IDXMIN = 4; IDXMAX = 5; MEAN = 6; STDDEV = 7; VAR = 8
 
 
-_SUFFIX = {np.dtype(np.float32): "f32", np.dtype(np.float64): "f64"}
+_SUFFIX = {np.dtype(np.float32): "f32", np.dtype(np.float64): "f64", np.dtype(np.int64): "si64",
+           np.dtype(np.uint64): "ui64", np.dtype(np.int32): "si32", np.dtype(np.uint32): "ui32"}
+_CTYPE = {np.dtype(np.float32): C.c_float, np.dtype(np.float64): C.c_double, np.dtype(np.int64): C.c_int64,
+          np.dtype(np.uint64): C.c_uint64, np.dtype(np.int32): C.c_int32, np.dtype(np.uint32): C.c_uint32}
 
 
 class HIPContext:
@@ -134,7 +137,7 @@ class DenseMatrix:
 
         assert t.is_cuda and t.dim() == 2 and t.stride(1) == 1
         dt = {torch.float32: np.float32, torch.float64: np.float64, torch.int64: np.int64,
-              torch.uint64: np.uint64}[t.dtype]
+              torch.uint64: np.uint64, torch.int32: np.int32, torch.uint32: np.uint32}[t.dtype]
         return DenseMatrix(ctx, t.shape[0], t.shape[1], dt, ptr=t.data_ptr(), row_skip=t.stride(0) if t.shape[0] > 1 else t.shape[1],
                            keepalive=t)
 
@@ -183,7 +186,10 @@ def _fn(name: str, dtype):
         suf = _SUFFIX[np.dtype(dtype)]
     except KeyError:
         raise capi.DaphneHipError(capi.DH_ERR_RUNTIME, f"{name}: unsupported value type {dtype}")
-    return getattr(capi.lib(), f"{name}_{suf}")
+    fn = getattr(capi.lib(), f"{name}_{suf}", None)
+    if fn is None:  # e.g. MatMul or the unary operators on integers: not instantiated, as in the reference
+        raise capi.DaphneHipError(capi.DH_ERR_RUNTIME, f"{name}: not instantiated for the value type {np.dtype(dtype)}")
+    return fn
 
 
 def _same_dtype(*ms):
@@ -213,7 +219,7 @@ def ewBinaryObjSca(opCode, res, lhs: DenseMatrix, rhs: float, ctx: HIPContext) -
     if res is None:
         res = DenseMatrix(ctx, lhs.rows, lhs.cols, dt)
     capi.check(_fn("dh_ew_binary_sca", dt)(ctx._h, int(opCode), res.ptr, res.row_skip, lhs.ptr, lhs.rows, lhs.cols,
-                                           lhs.row_skip, float(rhs)))
+                                           lhs.row_skip, rhs if dt.kind in "iu" else float(rhs)))
     return res
 
 
@@ -232,8 +238,7 @@ def ewUnaryMat(opCode, res, arg: DenseMatrix, ctx: HIPContext) -> DenseMatrix:
 # ------------------------------------------------------------------------------------------
 def aggAll(opCode, arg: DenseMatrix, ctx: HIPContext) -> float:
     """CUDA::aggAll (kernels/CUDA/AggAll.h:44-50): returns the scalar."""
-    ct = C.c_float if arg.dtype == np.float32 else C.c_double
-    out = ct()
+    out = _CTYPE[arg.dtype]()
     capi.check(_fn("dh_agg_all", arg.dtype)(ctx._h, int(opCode), arg.ptr, arg.rows, arg.cols, arg.row_skip,
                                             C.byref(out)))
     return arg.dtype.type(out.value)

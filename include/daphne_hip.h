@@ -379,6 +379,70 @@ dh_status dh_gemv_f64(dh_ctx *ctx, double *res, size_t ld_res, const double *mat
                       size_t cols, size_t ld_mat, const double *vec, size_t vec_rows, size_t ld_vec);
 
 
+/* ------------------------------------------------------------------------------------ */
+/* integer value types                                                                   */
+/* ------------------------------------------------------------------------------------ */
+/* The reference instantiates its device kernels for integers as well:
+ * EwBinaryMat for si64 / si32 / ui32 / ui64 (kernels/CUDA/EwBinaryMat.cu:267-270), EwBinaryObjSca for
+ * the same four (EwBinaryObjSca.cu:91-94), AggAll / AggRow / AggCol for si64 (AggAll.cu:155,
+ * AggRow.cu:146, AggCol.cu:89), Fill for si64 / ui64 (Fill.cu:47,49), ColBind and ExtractCol for si64
+ * (ColBind.cu:75, ExtractCol.cu:58). Arguments as for the floating-point entry points above.
+ *
+ * Elementwise semantics are those of the CPU kernel's expressions evaluated on integers
+ * (kernels/EwBinarySca.h:143-167): + - * / wrap and truncate as C++ integer arithmetic does,
+ * POW / MOD / LOG go through double (pow, fmod, log(l)/log(r)) and are truncated back, comparisons and
+ * AND / OR give 0 or 1. Where the host process would trap - division or remainder by zero, and the most
+ * negative value divided by -1 - the call returns DH_ERR_DOMAIN (res then holds 0 at those items);
+ * only DIV and MOD synchronise the stream for that check.
+ *
+ * Aggregations: SUM PROD MIN MAX and (dh_agg_row_idx / dh_agg_col_idx) IDXMIN IDXMAX; sums wrap.
+ * MEAN VAR STDDEV return DH_ERR_RUNTIME for integers (the reference's device library has none
+ * either; its CPU kernel divides in integer arithmetic, kernels/AggAll.h:163-191). */
+dh_status dh_ew_binary_si64(dh_ctx *ctx, int op, int64_t *res, size_t ld_res, const int64_t *lhs,
+                            size_t lhs_rows, size_t lhs_cols, size_t ld_lhs, const int64_t *rhs,
+                            size_t rhs_rows, size_t rhs_cols, size_t ld_rhs);
+dh_status dh_ew_binary_sca_si64(dh_ctx *ctx, int op, int64_t *res, size_t ld_res, const int64_t *lhs,
+                                size_t rows, size_t cols, size_t ld_lhs, int64_t rhs);
+dh_status dh_ew_binary_ui64(dh_ctx *ctx, int op, uint64_t *res, size_t ld_res, const uint64_t *lhs,
+                            size_t lhs_rows, size_t lhs_cols, size_t ld_lhs, const uint64_t *rhs,
+                            size_t rhs_rows, size_t rhs_cols, size_t ld_rhs);
+dh_status dh_ew_binary_sca_ui64(dh_ctx *ctx, int op, uint64_t *res, size_t ld_res, const uint64_t *lhs,
+                                size_t rows, size_t cols, size_t ld_lhs, uint64_t rhs);
+dh_status dh_ew_binary_si32(dh_ctx *ctx, int op, int32_t *res, size_t ld_res, const int32_t *lhs,
+                            size_t lhs_rows, size_t lhs_cols, size_t ld_lhs, const int32_t *rhs,
+                            size_t rhs_rows, size_t rhs_cols, size_t ld_rhs);
+dh_status dh_ew_binary_sca_si32(dh_ctx *ctx, int op, int32_t *res, size_t ld_res, const int32_t *lhs,
+                                size_t rows, size_t cols, size_t ld_lhs, int32_t rhs);
+dh_status dh_ew_binary_ui32(dh_ctx *ctx, int op, uint32_t *res, size_t ld_res, const uint32_t *lhs,
+                            size_t lhs_rows, size_t lhs_cols, size_t ld_lhs, const uint32_t *rhs,
+                            size_t rhs_rows, size_t rhs_cols, size_t ld_rhs);
+dh_status dh_ew_binary_sca_ui32(dh_ctx *ctx, int op, uint32_t *res, size_t ld_res, const uint32_t *lhs,
+                                size_t rows, size_t cols, size_t ld_lhs, uint32_t rhs);
+
+dh_status dh_agg_all_si64(dh_ctx *ctx, int op, const int64_t *arg, size_t rows, size_t cols, size_t ld,
+                          int64_t *result_host);
+dh_status dh_agg_row_si64(dh_ctx *ctx, int op, int64_t *res, size_t ld_res, const int64_t *arg,
+                          size_t rows, size_t cols, size_t ld);
+dh_status dh_agg_row_idx_si64(dh_ctx *ctx, int op, uint64_t *res, size_t ld_res, const int64_t *arg,
+                              size_t rows, size_t cols, size_t ld);
+dh_status dh_agg_col_si64(dh_ctx *ctx, int op, int64_t *res, const int64_t *arg, size_t rows,
+                          size_t cols, size_t ld);
+dh_status dh_agg_col_idx_si64(dh_ctx *ctx, int op, uint64_t *res, const int64_t *arg, size_t rows,
+                              size_t cols, size_t ld);
+
+dh_status dh_fill_si64(dh_ctx *ctx, int64_t *res, size_t ld_res, int64_t value, size_t rows, size_t cols);
+dh_status dh_fill_ui64(dh_ctx *ctx, uint64_t *res, size_t ld_res, uint64_t value, size_t rows, size_t cols);
+dh_status dh_col_bind_si64(dh_ctx *ctx, int64_t *res, size_t ld_res, const int64_t *lhs, size_t lhs_rows,
+                           size_t lhs_cols, size_t ld_lhs, const int64_t *rhs, size_t rhs_rows,
+                           size_t rhs_cols, size_t ld_rhs);
+dh_status dh_extract_col_si64(dh_ctx *ctx, int64_t *res, size_t ld_res, const int64_t *arg, size_t rows,
+                              size_t cols, size_t ld, const int64_t *sel, size_t sel_rows,
+                              size_t sel_cols, size_t ld_sel);
+/* Transpose has no integer instantiation in the reference (cublas geam); provided for completeness. */
+dh_status dh_transpose_si64(dh_ctx *ctx, int64_t *res, size_t ld_res, const int64_t *arg, size_t rows,
+                            size_t cols, size_t ld);
+
+
 
 /* ------------------------------------------------------------------------------------ */
 /* fused vectorized pipeline                                                             */

@@ -81,14 +81,34 @@ template <typename T> BinFn<T> bin_fn(int op, bool *unknown) {
     }
 }
 
+// Integer DIV by zero (and INT_MIN / -1) is a hardware trap in the reference's process, and MOD by zero converts
+// a NaN to an integer (undefined): both are reported as a domain error here, with 0 stored, instead of being executed.
+template <typename T> struct SafeBin {
+    BinFn<T> f;
+    int op;
+    bool bad = false;
+    T operator()(T l, T r) {
+        if constexpr (std::numeric_limits<T>::is_integer) {
+            const bool div_traps = r == T(0) || (std::numeric_limits<T>::is_signed && r == T(-1) &&
+                                                 l == std::numeric_limits<T>::min());
+            if ((op == 3 && div_traps) || (op == 5 && r == T(0))) {
+                bad = true;
+                return T(0);
+            }
+        }
+        return f(l, r);
+    }
+};
+
 // EwBinaryMat.h:54-108
 template <typename T>
 int ew_binary(int op, T *res, size_t ld_res, const T *lhs, size_t lr, size_t lc, size_t ld_lhs, const T *rhs,
               size_t rr, size_t rc, size_t ld_rhs) {
     bool unknown;
-    BinFn<T> f = bin_fn<T>(op, &unknown);
-    if (!f)
+    BinFn<T> fp = bin_fn<T>(op, &unknown);
+    if (!fp)
         return ST_RUNTIME;
+    SafeBin<T> f{fp, op};
     if (lr == rr && lc == rc) {
         for (size_t r = 0; r < lr; r++) {
             for (size_t c = 0; c < lc; c++)
@@ -114,23 +134,24 @@ int ew_binary(int op, T *res, size_t ld_res, const T *lhs, size_t lr, size_t lc,
         }
     } else
         return ST_RUNTIME;
-    return ST_OK;
+    return f.bad ? ST_DOMAIN : ST_OK;
 }
 
 // EwBinaryObjSca.h:57-79
 template <typename T>
 int ew_binary_sca(int op, T *res, size_t ld_res, const T *lhs, size_t rows, size_t cols, size_t ld_lhs, T rhs) {
     bool unknown;
-    BinFn<T> f = bin_fn<T>(op, &unknown);
-    if (!f)
+    BinFn<T> fp = bin_fn<T>(op, &unknown);
+    if (!fp)
         return ST_RUNTIME;
+    SafeBin<T> f{fp, op};
     for (size_t r = 0; r < rows; r++) {
         for (size_t c = 0; c < cols; c++)
             res[c] = f(lhs[c], rhs);
         lhs += ld_lhs;
         res += ld_res;
     }
-    return ST_OK;
+    return f.bad ? ST_DOMAIN : ST_OK;
 }
 
 // EwUnarySca.h:182-206 (+ domain checks :129-157); UnaryOpCode.h:28-55 order.
@@ -218,8 +239,8 @@ template <typename T> T agg_neutral(int op) {
     switch (op) {
     case A_SUM: return T(0);
     case A_PROD: return T(1);
-    case A_MIN: return std::numeric_limits<T>::infinity();
-    case A_MAX: return -std::numeric_limits<T>::infinity();
+    case A_MIN: return std::numeric_limits<T>::has_infinity ? std::numeric_limits<T>::infinity() : std::numeric_limits<T>::max();
+    case A_MAX: return std::numeric_limits<T>::has_infinity ? -std::numeric_limits<T>::infinity() : std::numeric_limits<T>::min();
     default: return T(0);
     }
 }
@@ -858,3 +879,54 @@ template <typename T> int transpose(T *res, size_t ld_res, const T *arg, size_t 
 
 ORACLE_EXPORTS(f32, float)
 ORACLE_EXPORTS(f64, double)
+
+// Integer value types (the reference instantiates these device kernels for them: kernels/CUDA/EwBinaryMat.cu:267-270,
+// EwBinaryObjSca.cu:91-94, AggAll.cu:155, AggRow.cu:146, AggCol.cu:89, Fill.cu:47,49, ColBind.cu:75, ExtractCol.cu:58):
+// the same templates as above, i.e. the reference's expressions evaluated in C++ integer arithmetic.
+#define ORACLE_EW_INT_EXPORTS(SUF, T)                                                                                   \
+    extern "C" int oracle_ew_binary_##SUF(int op, T *res, size_t ld_res, const T *lhs, size_t lr, size_t lc,            \
+                                          size_t ld_lhs, const T *rhs, size_t rr, size_t rc, size_t ld_rhs) {           \
+        return ew_binary<T>(op, res, ld_res, lhs, lr, lc, ld_lhs, rhs, rr, rc, ld_rhs);                                 \
+    }                                                                                                                   \
+    extern "C" int oracle_ew_binary_sca_##SUF(int op, T *res, size_t ld_res, const T *lhs, size_t rows, size_t cols,    \
+                                              size_t ld_lhs, T rhs) {                                                   \
+        return ew_binary_sca<T>(op, res, ld_res, lhs, rows, cols, ld_lhs, rhs);                                         \
+    }
+ORACLE_EW_INT_EXPORTS(si64, int64_t)
+ORACLE_EW_INT_EXPORTS(ui64, uint64_t)
+ORACLE_EW_INT_EXPORTS(si32, int32_t)
+ORACLE_EW_INT_EXPORTS(ui32, uint32_t)
+
+extern "C" int oracle_agg_all_si64(int op, const int64_t *arg, size_t rows, size_t cols, size_t ld, int64_t *out) {
+    return agg_all<int64_t>(op, arg, rows, cols, ld, out);
+}
+extern "C" int oracle_agg_row_si64(int op, int64_t *res, size_t ld_res, const int64_t *arg, size_t rows, size_t cols, size_t ld) {
+    return agg_row<int64_t>(op, res, ld_res, arg, rows, cols, ld);
+}
+extern "C" int oracle_agg_row_idx_si64(int op, uint64_t *res, size_t ld_res, const int64_t *arg, size_t rows, size_t cols,
+                                       size_t ld) {
+    return agg_row_idx<int64_t>(op, res, ld_res, arg, rows, cols, ld);
+}
+extern "C" int oracle_agg_col_si64(int op, int64_t *res, const int64_t *arg, size_t rows, size_t cols, size_t ld) {
+    return agg_col<int64_t>(op, res, arg, rows, cols, ld);
+}
+extern "C" int oracle_agg_col_idx_si64(int op, uint64_t *res, const int64_t *arg, size_t rows, size_t cols, size_t ld) {
+    return agg_col_idx<int64_t>(op, res, arg, rows, cols, ld);
+}
+extern "C" int oracle_fill_si64(int64_t *res, size_t ld_res, int64_t value, size_t rows, size_t cols) {
+    return fill<int64_t>(res, ld_res, value, rows, cols);
+}
+extern "C" int oracle_fill_ui64(uint64_t *res, size_t ld_res, uint64_t value, size_t rows, size_t cols) {
+    return fill<uint64_t>(res, ld_res, value, rows, cols);
+}
+extern "C" int oracle_col_bind_si64(int64_t *res, size_t ld_res, const int64_t *lhs, size_t lr, size_t lc, size_t ld_lhs,
+                                    const int64_t *rhs, size_t rr, size_t rc, size_t ld_rhs) {
+    return col_bind<int64_t>(res, ld_res, lhs, lr, lc, ld_lhs, rhs, rr, rc, ld_rhs);
+}
+extern "C" int oracle_extract_col_si64(int64_t *res, size_t ld_res, const int64_t *arg, size_t rows, size_t cols, size_t ld,
+                                       const int64_t *sel, size_t sel_rows, size_t sel_cols) {
+    return extract_col<int64_t>(res, ld_res, arg, rows, cols, ld, sel, sel_rows, sel_cols);
+}
+extern "C" int oracle_transpose_si64(int64_t *res, size_t ld_res, const int64_t *arg, size_t rows, size_t cols, size_t ld) {
+    return transpose<int64_t>(res, ld_res, arg, rows, cols, ld);
+}

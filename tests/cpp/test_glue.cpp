@@ -282,6 +282,64 @@ template <typename VT> void run_all(DaphneContext *dctx) {
     }
 }
 
+// Integer instantiations (EwBinaryMatTest.cpp:34, EwBinaryObjScaTest.cpp:36 run with uint32_t; AggAllTest.cpp:32 with
+// int64_t among others): the reference's literals where they are integers, plus integer-only behaviour.
+template <typename VT> void run_integer_elementwise(DaphneContext *dctx) {
+    using DT = DenseMatrix<VT>;
+    auto G = [&](size_t rows, std::vector<VT> v) { return genGivenVals<DT>(rows, v, dctx); };
+    // EwBinaryMatTest.cpp:69-102 (add), :104-125 (mul), :178-222 (div), :523-557 (max)
+    auto m1 = G(2, {1, 2, 0, 0, 1, 3}), m2 = G(2, {0, 9, 0, 0, 3, 4}), m3 = G(2, {1, 11, 0, 0, 4, 7});
+    DT *res = nullptr;
+    HIP::ewBinaryMat(BinaryOpCode::ADD, res, m1, m2, dctx);
+    CHECK(equals(res, m3->toHost()));
+    HIP::ewBinaryMat(BinaryOpCode::MUL, res, m1, m2, dctx);
+    CHECK(equals(res, {0, 18, 0, 0, 3, 12}));
+    HIP::ewBinaryMat(BinaryOpCode::MAX, res, m1, m2, dctx);
+    CHECK(equals(res, {1, 9, 0, 0, 3, 4}));
+    auto d1 = G(2, {7, 9, 20, 0, 1, 100}), d2 = G(2, {2, 3, 6, 5, 1, 7});
+    HIP::ewBinaryMat(BinaryOpCode::DIV, res, d1, d2, dctx);
+    CHECK(equals(res, {3, 3, 3, 0, 1, 14})); // truncating division
+    HIP::ewBinaryMat(BinaryOpCode::MOD, res, d1, d2, dctx);
+    CHECK(equals(res, {1, 0, 2, 0, 0, 2}));
+    HIP::ewBinaryObjSca(BinaryOpCode::POW, res, d2, VT(3), dctx);
+    CHECK(equals(res, {8, 27, 216, 125, 1, 343}));
+    HIP::ewBinaryObjSca(BinaryOpCode::GE, res, d1, VT(9), dctx);
+    CHECK(equals(res, {0, 1, 1, 0, 0, 1}));
+    // a zero divisor is reported instead of trapping the process
+    CHECK_THROWS_AS(HIP::ewBinaryMat(BinaryOpCode::DIV, res, d1, m1, dctx), std::domain_error);
+    CHECK_THROWS_AS(HIP::ewBinaryObjSca(BinaryOpCode::MOD, res, d1, VT(0), dctx), std::domain_error);
+    for (auto *m : {m1, m2, m3, d1, d2, res})
+        DataObjectFactory::destroy(m);
+}
+
+static void run_si64(DaphneContext *dctx) {
+    using DT = DenseMatrix<int64_t>;
+    auto G = [&](size_t rows, std::vector<int64_t> v) { return genGivenVals<DT>(rows, v, dctx); };
+    // AggRowTest.cpp / AggColTest.cpp literal, AggAllTest.cpp:62-75
+    auto m = G(3, {3, 0, 2, 0, 0, 0, 1, 0, 0, 1, 0, 3});
+    CHECK(HIP::aggAll<int64_t>(AggOpCode::SUM, m, dctx) == 10);
+    CHECK(HIP::aggAll<int64_t>(AggOpCode::MAX, m, dctx) == 3);
+    CHECK(HIP::aggAll<int64_t>(AggOpCode::MIN, m, dctx) == 0);
+    DT *r = nullptr, *c = nullptr, *t = nullptr, *b = nullptr, *f = nullptr;
+    HIP::aggRow(AggOpCode::SUM, r, m, dctx);
+    CHECK(equals(r, {5, 1, 4}));
+    HIP::aggCol(AggOpCode::MAX, c, m, dctx);
+    CHECK(equals(c, {3, 1, 2, 3}));
+    DenseMatrix<size_t> *idx = nullptr;
+    HIP::aggRow(AggOpCode::IDXMAX, idx, m, dctx);
+    CHECK(equals(idx, {0, 2, 3}));
+    CHECK_THROWS_AS(HIP::aggAll<int64_t>(AggOpCode::MEAN, m, dctx), std::runtime_error);
+    HIP::transpose(t, m, dctx);
+    CHECK(equals(t, {3, 0, 0, 0, 0, 1, 2, 1, 0, 0, 0, 3}));
+    HIP::colBind(b, m, r, dctx);
+    CHECK(equals(b, {3, 0, 2, 0, 5, 0, 0, 1, 0, 1, 0, 1, 0, 3, 4}));
+    HIP::fill(f, int64_t(-7), 2, 3, dctx);
+    CHECK(equals(f, {-7, -7, -7, -7, -7, -7}));
+    for (auto *x : {m, r, c, t, b, f})
+        DataObjectFactory::destroy(x);
+    DataObjectFactory::destroy(idx);
+}
+
 int main() {
     // test/runtime/local/kernels/CUDA_ContextTest.cpp:25-30
     auto dctx = std::make_unique<DaphneContext>();
@@ -295,6 +353,11 @@ int main() {
     CHECK(HIPContext::get(dctx.get(), 0)->getMemBudget() > 0);
     run_all<float>(dctx.get());
     run_all<double>(dctx.get());
+    run_integer_elementwise<int64_t>(dctx.get());
+    run_integer_elementwise<uint64_t>(dctx.get());
+    run_integer_elementwise<int32_t>(dctx.get());
+    run_integer_elementwise<uint32_t>(dctx.get());
+    run_si64(dctx.get());
     std::printf("%s: %d checks, %d failed\n", g_fail ? "FAILED" : "PASSED", g_checks, g_fail);
     return g_fail ? 1 : 0;
 }

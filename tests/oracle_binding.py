@@ -14,7 +14,10 @@ ORACLE_DIR = Path(__file__).resolve().parent.parent / "oracle"
 LIB = ORACLE_DIR / "liboracle.so"
 
 ST_OK, ST_RUNTIME, ST_INVALID, ST_DOMAIN = 0, 1, 2, 3
-_SUF = {np.dtype(np.float32): "f32", np.dtype(np.float64): "f64"}
+_SUF = {np.dtype(np.float32): "f32", np.dtype(np.float64): "f64", np.dtype(np.int64): "si64", np.dtype(np.uint64): "ui64",
+        np.dtype(np.int32): "si32", np.dtype(np.uint32): "ui32"}
+_CT = {np.dtype(np.float32): C.c_float, np.dtype(np.float64): C.c_double, np.dtype(np.int64): C.c_int64,
+       np.dtype(np.uint64): C.c_uint64, np.dtype(np.int32): C.c_int32, np.dtype(np.uint32): C.c_uint32}
 _lib = None
 
 
@@ -36,7 +39,8 @@ def _f(name, dt):
 
 
 def _sc(dt, v):
-    return C.c_float(v) if np.dtype(dt) == np.float32 else C.c_double(v)
+    dt = np.dtype(dt)
+    return _CT[dt](int(v) if dt.kind in "iu" else v)
 
 
 def _ld(a):

@@ -16,3 +16,14 @@ def test_hip_matches_reference_vectors(ctx, cid, f, c, k, dt):
         gc.run(HipBackend(ctx), f, c, k, dt)
     except gc.Skip as e:
         pytest.skip(str(e))
+
+
+@pytest.mark.parametrize("dt", [np.int64, np.uint64, np.int32, np.uint32], ids=["si64", "ui64", "si32", "ui32"])
+@pytest.mark.parametrize("cid,f,c,k", CHECKS, ids=[c[0] for c in CHECKS])
+def test_hip_matches_reference_vectors_for_integers(ctx, cid, f, c, k, dt):
+    """The reference runs these tests with integer value types too (VALUE_TYPES in EwBinaryMatTest.cpp:34,
+    AggAllTest.cpp:32, AggRowTest.cpp:33 ...): literals that are integers of the type are replayed with it."""
+    try:
+        gc.run(HipBackend(ctx), f, c, k, dt)
+    except gc.Skip as e:
+        pytest.skip(str(e))

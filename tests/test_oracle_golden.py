@@ -33,3 +33,14 @@ def test_golden_file_covers_the_kernel_set():
                  "CUDA/DNNSoftmaxTest.cpp", "CUDA/DNNActivationTest.cpp", "TransposeTest.cpp", "ColBindTest.cpp",
                  "ExtractColTest.cpp"):
         assert ran.get(must, 0) > 0, f"no vector of {must} was replayed"
+
+
+@pytest.mark.parametrize("dt", [np.int64, np.uint64, np.int32, np.uint32], ids=["si64", "ui64", "si32", "ui32"])
+@pytest.mark.parametrize("cid,f,c,k", CHECKS, ids=[c[0] for c in CHECKS])
+def test_oracle_matches_reference_vectors_for_integers(cid, f, c, k, dt):
+    """The reference runs these tests with integer value types too (VALUE_TYPES in EwBinaryMatTest.cpp:34,
+    AggAllTest.cpp:32, AggRowTest.cpp:33 ...): literals that are integers of the type are replayed with it."""
+    try:
+        gc.run(OracleBackend(), f, c, k, dt)
+    except gc.Skip as e:
+        pytest.skip(str(e))

@@ -235,3 +235,95 @@ def test_avgpool_brute_force(p):
             for j in range(Q):
                 exp[:, :, i, j] = img[:, :, i * sh:i * sh + ph, j * sw:j * sw + pw].sum(axis=(2, 3)) / (ph * pw)
     np.testing.assert_allclose(got, exp.reshape(N, -1), rtol=1e-12, atol=1e-12)
+
+
+INT_TYPES = [np.int64, np.uint64, np.int32, np.uint32]
+
+
+@pytest.mark.parametrize("dt", INT_TYPES, ids=["si64", "ui64", "si32", "ui32"])
+def test_integer_elementwise_against_exact_python_arithmetic(dt):
+    """The integer instantiations are pinned by Python's exact integers: + - * wrap modulo 2^bits, / truncates toward
+    zero, MOD keeps the sign of the dividend (fmod), POW is the exact power where it fits, comparisons give 0 / 1."""
+    rng = np.random.default_rng(5)
+    info = np.iinfo(dt)
+    signed = info.min < 0
+    bits = info.bits
+    lo = -50 if signed else 0
+    a = rng.integers(lo, 50, (7, 9)).astype(dt)
+    b = rng.integers(lo, 50, (7, 9)).astype(dt)
+    b[b == 0] = 3
+    big = rng.integers(info.max // 2, info.max, (7, 9), dtype=np.uint64 if not signed else np.int64).astype(dt)
+
+    def wrap(v):
+        v &= (1 << bits) - 1
+        return v - (1 << bits) if signed and v >= 1 << (bits - 1) else v
+
+    def table(f, x, y):
+        return np.array([[f(int(p), int(q)) for p, q in zip(r, s)] for r, s in zip(x, y)], dtype=object)
+
+    def tdiv(p, q):
+        return abs(p) // abs(q) * (1 if (p < 0) == (q < 0) else -1)
+
+    cases = {0: lambda p, q: wrap(p + q), 1: lambda p, q: wrap(p - q), 2: lambda p, q: wrap(p * q), 3: tdiv,
+             5: lambda p, q: p - q * tdiv(p, q), 7: lambda p, q: int(p == q), 8: lambda p, q: int(p != q),
+             9: lambda p, q: int(p < q), 10: lambda p, q: int(p <= q), 11: lambda p, q: int(p > q),
+             12: lambda p, q: int(p >= q), 13: min, 14: max, 15: lambda p, q: int(bool(p) and bool(q)),
+             16: lambda p, q: int(bool(p) or bool(q))}
+    for op, f in cases.items():
+        for x, y in ((a, b), (big, b)) if op in (0, 1, 2, 13, 14) else ((a, b),):
+            st, got = orc.ew_binary(op, x, y)
+            assert st == orc.ST_OK
+            want = table(f, x, y)
+            assert np.array_equal(got.astype(object), want), (op, dt)
+        s = 7
+        st, got = orc.ew_binary_sca(op, a, s)
+        assert st == orc.ST_OK and np.array_equal(got.astype(object), table(f, a, np.full(a.shape, s, dtype=dt)))
+    # POW: exact where it fits 53 bits; a negative exponent truncates to 0 (or +-1 for bases +-1)
+    base = rng.integers(lo // 10, 6, (5, 5)).astype(dt)
+    ex = rng.integers(0, 9, (5, 5)).astype(dt)
+    st, got = orc.ew_binary(4, base, ex)
+    assert st == orc.ST_OK and np.array_equal(got.astype(object), table(lambda p, q: wrap(p ** q), base, ex))
+    # row- and column-vector broadcasts take the same scalar path
+    st, got = orc.ew_binary(0, a, b[:1])
+    assert np.array_equal(got, a + b[:1])
+    st, got = orc.ew_binary(2, a, b[:, :1])
+    assert np.array_equal(got, a * b[:, :1])
+    # what would trap in the reference's process is a domain error here: x / 0, x mod 0, and INT_MIN / -1
+    z = b.copy()
+    z[2, 3] = 0
+    assert orc.ew_binary(3, a, z)[0] == orc.ST_DOMAIN and orc.ew_binary(5, a, z)[0] == orc.ST_DOMAIN
+    assert orc.ew_binary_sca(3, a, 0)[0] == orc.ST_DOMAIN
+    if signed:
+        m = a.copy()
+        m[0, 0] = info.min
+        assert orc.ew_binary_sca(3, m, -1)[0] == orc.ST_DOMAIN
+        assert orc.ew_binary_sca(5, m, -1)[0] == orc.ST_OK  # fmod is defined there
+
+
+def test_si64_aggregations_against_numpy():
+    rng = np.random.default_rng(6)
+    x = rng.integers(-1000, 1000, (37, 23)).astype(np.int64)
+    x[5, 7] = np.iinfo(np.int64).max
+    x[9, 2] = np.iinfo(np.int64).min
+    for op, f in ((0, np.sum), (2, np.min), (3, np.max)):
+        with np.errstate(over="ignore"):
+            assert orc.agg_all(op, x) == (orc.ST_OK, f(x))
+            st, r = orc.agg_row(op, x)
+            assert st == orc.ST_OK and np.array_equal(r[:, 0], f(x, axis=1))
+            st, c = orc.agg_col(op, x)
+            assert st == orc.ST_OK and np.array_equal(c[0], f(x, axis=0))
+    small = rng.integers(-3, 4, (6, 5)).astype(np.int64)
+    assert orc.agg_all(1, small)[1] == np.prod(small)
+    ties = rng.integers(0, 4, (50, 12)).astype(np.int64)  # many ties: the first one wins
+    assert np.array_equal(orc.agg_row(4, ties)[1][:, 0], np.argmin(ties, axis=1))
+    assert np.array_equal(orc.agg_row(5, ties)[1][:, 0], np.argmax(ties, axis=1))
+    assert np.array_equal(orc.agg_col(4, ties)[1][0], np.argmin(ties, axis=0))
+    assert np.array_equal(orc.agg_col(5, ties)[1][0], np.argmax(ties, axis=0))
+    v = x[3:30, 4:20]  # a view: row stride larger than the width
+    assert orc.agg_all(0, v)[1] == v.sum() and np.array_equal(orc.agg_col(3, v)[1][0], v.max(axis=0))
+    # data reorganisation of 64-bit integers
+    assert np.array_equal(orc.transpose(x)[1], x.T)
+    assert np.array_equal(orc.col_bind(x, ties[:37])[1], np.hstack([x, ties[:37]]))
+    assert np.array_equal(orc.extract_col(x, np.array([[3], [0], [-1]]))[1], x[:, [3, 0, -1]])
+    assert np.array_equal(orc.fill(-5, 3, 4, np.int64)[1], np.full((3, 4), -5, np.int64))
+    assert np.array_equal(orc.fill(2 ** 63 + 1, 2, 2, np.uint64)[1], np.full((2, 2), 2 ** 63 + 1, np.uint64))
