@@ -23,6 +23,9 @@
 #include "common.h"
 
 namespace dh_gemm {
+#ifndef TS_SYM_U
+#define TS_SYM_U 4 // quads per register set of the symmetric one-wave form (measured: 2 1.00 ms, 4 0.90, 8 0.92, 12 0.95)
+#endif
 
 typedef float ts_f32x4 __attribute__((ext_vector_type(4)));
 typedef double ts_f64x4 __attribute__((ext_vector_type(4)));
@@ -78,7 +81,9 @@ __global__ __launch_bounds__(256) void ts_tn_kernel(TsTnArgs g) {
     constexpr int KW = 4 / (WM * WN);
     constexpr int TM = 16 * VA * RA, TN = 16 * VB * RB;
     constexpr int NACC = RA * VA * RB * VB;         // MFMA tiles per wave
-    constexpr int U = NACC >= 16 ? 2 : 4;           // quads (4 rows of K) in flight per wave
+    // quads (4 rows of K) per register set: with 16 accumulator tiles only two fit beside them, except in the symmetric
+    // one-wave form, where the B fragments are the A fragments and 10 of the 16 tiles exist
+    constexpr int U = NACC >= 16 ? ((SYM && WM == 1) ? TS_SYM_U : 2) : 4;
     const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
     const int wm = wave % WM, wn = (wave / WM) % WN, wk = wave / (WM * WN);
     const int i = lane % 16, h = lane / 16;
@@ -123,16 +128,28 @@ __global__ __launch_bounds__(256) void ts_tn_kernel(TsTnArgs g) {
     struct Frag {
         T a[U][RA][VA], b[U][RB][VB];
     };
+    // Every load is issued unconditionally, and nothing touches the loaded registers before the matrix instructions
+    // do: a branch around a load (or a fix-up right after it) makes the compiler wait for ALL outstanding loads at
+    // that point, which would serialise the two register sets. Vectors that start beyond the matrix read column 0
+    // instead - they only feed rows / columns of C beyond m / n, which are never stored. Rows beyond the chunk
+    // (possible in the tail loop only) read its last row and are zeroed, since a row of K reaches every output.
+    unsigned ca_ld[RA], cb_ld[RB];
+#pragma unroll
+    for (int a = 0; a < RA; a++)
+        ca_ld[a] = oka[a] ? ca[a] : 0;
+#pragma unroll
+    for (int b = 0; b < RB; b++)
+        cb_ld[b] = okb[b] ? cb[b] : 0;
     auto load_quad = [&](Frag &fr, int u, size_t k, bool guard) {
         const bool row_ok = !guard || k < ke;
+        const size_t kl = row_ok ? k : ke - 1;
 #pragma unroll
         for (int a = 0; a < RA; a++) {
-            if (oka[a] && row_ok) {
-                ts_load<T, VA>(A + k * g.lda + ca[a], fr.a[u][a], stream);
-            } else {
+            ts_load<T, VA>(A + kl * g.lda + ca_ld[a], fr.a[u][a], stream);
+            if (guard) {
 #pragma unroll
                 for (int e = 0; e < VA; e++)
-                    fr.a[u][a][e] = T(0);
+                    fr.a[u][a][e] = row_ok ? fr.a[u][a][e] : T(0);
             }
         }
         if (diag) {
@@ -147,12 +164,11 @@ __global__ __launch_bounds__(256) void ts_tn_kernel(TsTnArgs g) {
         }
 #pragma unroll
         for (int b = 0; b < RB; b++) {
-            if (okb[b] && row_ok) {
-                ts_load<T, VB>(B + k * g.ldb + cb[b], fr.b[u][b], stream);
-            } else {
+            ts_load<T, VB>(B + kl * g.ldb + cb_ld[b], fr.b[u][b], stream);
+            if (guard) {
 #pragma unroll
                 for (int f = 0; f < VB; f++)
-                    fr.b[u][b][f] = T(0);
+                    fr.b[u][b][f] = row_ok ? fr.b[u][b][f] : T(0);
             }
         }
     };
@@ -184,8 +200,6 @@ __global__ __launch_bounds__(256) void ts_tn_kernel(TsTnArgs g) {
     // quad q of this wave covers rows kb + (q*KW + wk)*4 .. +3; lane group h takes row +h
     size_t k = kb + static_cast<size_t>(wk) * 4 + h;
     constexpr size_t STEP = static_cast<size_t>(KW) * 4;
-    // a full group: every row of its last quad is inside the chunk
-    auto full = [&]() { return k - h + (U - 1) * STEP + 4 <= ke; };
     auto load_group = [&](Frag &fr) {
 #pragma unroll
         for (int u = 0; u < U; u++)
@@ -198,21 +212,35 @@ __global__ __launch_bounds__(256) void ts_tn_kernel(TsTnArgs g) {
             mma_quad(fr, u);
     };
     Frag f0, f1;
-    if (full()) {
+    // The number of full groups of this wavefront is known up front, so the steady state is a counted loop whose
+    // body is one basic block: loads into one register set, matrix instructions on the other, twice. That lets the
+    // compiler's wait counts leave the new loads in flight (a load inside a conditional would make the wait at
+    // the join cover it). The odd group left over is finished after the loop.
+    const size_t k0 = kb + static_cast<size_t>(wk) * 4; // first row of this wavefront's first quad
+    const size_t need = (U - 1) * STEP + 4;             // rows from the start of a group to the end of its last quad
+    const unsigned n_full = ke >= k0 + need ? static_cast<unsigned>((ke - k0 - need) / (U * STEP)) + 1 : 0;
+    if (n_full > 0) {
         load_group(f0);
-        while (true) {
-            bool more = full();
-            if (more)
-                load_group(f1);
+        const unsigned pairs = (n_full - 1) / 2;
+        // (the scheduling barriers keep the compiler from sinking the loads below the matrix instructions that
+        // they are meant to overlap with)
+        for (unsigned p = 0; p < pairs; p++) {
+            load_group(f1);
+            __builtin_amdgcn_sched_barrier(0);
             mma_group(f0);
-            if (!more)
-                break;
-            more = full();
-            if (more)
-                load_group(f0);
+            __builtin_amdgcn_sched_barrier(0);
+            load_group(f0);
+            __builtin_amdgcn_sched_barrier(0);
             mma_group(f1);
-            if (!more)
-                break;
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if ((n_full - 1) % 2) {
+            load_group(f1);
+            __builtin_amdgcn_sched_barrier(0);
+            mma_group(f0);
+            mma_group(f1);
+        } else {
+            mma_group(f0);
         }
     }
     while (k - h < ke) {
@@ -331,6 +359,7 @@ struct TsNtArgs {
     size_t lda, ldb, ldc, M;
     unsigned n, K;
     unsigned kpad;   // K rounded up to whole chunks
+    int vec_store;   // C rows are 16-byte aligned
 };
 
 // NB column blocks of 16; each wave walks over row blocks of 16, two at a time.
@@ -339,6 +368,10 @@ template <typename T, int NB> __global__ __launch_bounds__(256) void ts_nt_kerne
     constexpr int V = 16 / sizeof(T);
     constexpr int KC = 4 * V;     // k values per chunk
     constexpr int RBW = 8;        // row blocks per wave
+    // float: the operands of the matrix instruction are exchanged, which transposes the result tile in the
+    // registers (row = 4 * (lane / 16) + v becomes the column) and turns four 4-byte stores per lane into one of
+    // 16 bytes; the double layout (row = 4 * v + lane / 16) already stores whole 128-byte rows
+    constexpr bool SWAP = sizeof(T) == 4;
     extern __shared__ __attribute__((aligned(16))) unsigned char ts_nt_lds[];
     T *lb = reinterpret_cast<T *>(ts_nt_lds); // [NB*16][kpad + V], zero padded
     const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
@@ -347,6 +380,120 @@ template <typename T, int NB> __global__ __launch_bounds__(256) void ts_nt_kerne
     const T *B = static_cast<const T *>(g.B);
     T *C = static_cast<T *>(g.C);
     const unsigned ldl = g.kpad + V;
+
+    // The work of a wavefront is a sequence of steps (pair of 16-row blocks, group of four k chunks), walked with two
+    // register sets: the eight vector loads of step s + 1 are in flight while the matrix cores work on step s, and
+    // the first step's loads are issued before B is staged into LDS, so that they overlap the staging and its barrier.
+    // All loads are unconditional (a branch around a load makes the compiler wait for every outstanding load at
+    // its first use): rows beyond M read the last row - they only produce rows of C that are not stored -, k
+    // beyond K reads k = 0 and is zeroed when it is used (the padded part of B is zero, but 0 * NaN would still
+    // be NaN), and steps beyond the last repeat the last one.
+    const size_t row0 = (static_cast<size_t>(blockIdx.x) * 4 + wave) * (16 * RBW);
+    const unsigned chunks = g.kpad / KC;
+    const unsigned cg = (chunks + 3) / 4;            // chunk groups per row-block pair
+    const unsigned nsteps = (RBW / 2) * cg;          // even
+    struct Frag {
+        T a[2][4][V];
+    };
+    auto load_step = [&](Frag &fr, unsigned pair, unsigned grp) {
+        const size_t r0 = row0 + static_cast<size_t>(pair) * 32 + i, r1 = r0 + 16;
+        const T *a0 = A + (r0 < g.M ? r0 : g.M - 1) * g.lda, *a1 = A + (r1 < g.M ? r1 : g.M - 1) * g.lda;
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            const unsigned kv = (grp * 4 + c) * KC + h * V;
+            const unsigned kl = kv < g.K ? kv : 0;
+            ts_load<T, V>(a0 + kl, fr.a[0][c], true);
+            ts_load<T, V>(a1 + kl, fr.a[1][c], true);
+        }
+    };
+    typename M::acc_t acc[2][NB];
+    auto compute_step = [&](const Frag &fr, unsigned pair, unsigned grp) {
+        if (grp == 0) {
+#pragma unroll
+            for (int b = 0; b < NB; b++) {
+                acc[0][b] = typename M::acc_t{0, 0, 0, 0};
+                acc[1][b] = typename M::acc_t{0, 0, 0, 0};
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            const unsigned ch = grp * 4 + c;
+            if (ch < chunks) {
+                const bool kok = ch * KC + h * V < g.K;
+#pragma unroll
+                for (int b = 0; b < NB; b++) {
+                    T fb[V];
+                    dh_load_vec<T, V>(lb + (b * 16 + i) * ldl + ch * KC + h * V, fb);
+#pragma unroll
+                    for (int e = 0; e < V; e++) {
+                        const T x0 = kok ? fr.a[0][c][e] : T(0), x1 = kok ? fr.a[1][c][e] : T(0);
+                        if constexpr (SWAP) {
+                            acc[0][b] = M::mma(fb[e], x0, acc[0][b]);
+                            acc[1][b] = M::mma(fb[e], x1, acc[1][b]);
+                        } else {
+                            acc[0][b] = M::mma(x0, fb[e], acc[0][b]);
+                            acc[1][b] = M::mma(x1, fb[e], acc[1][b]);
+                        }
+                    }
+                }
+            }
+        }
+        if (grp + 1 != cg)
+            return;
+        const size_t rbase = row0 + static_cast<size_t>(pair) * 32;
+        if constexpr (SWAP) {
+            // the tile was computed transposed: register v of lane (i, h) is C[row i][column 4h + v], so a lane
+            // stores four neighbouring columns at once and a wavefront 16 whole rows
+#pragma unroll
+            for (int t = 0; t < 2; t++) {
+                const size_t row = rbase + static_cast<size_t>(t) * 16 + i;
+                if (row < g.M) {
+#pragma unroll
+                    for (int b = 0; b < NB; b++) {
+                        const int col = b * 16 + 4 * h;
+                        T *dst = C + row * g.ldc + col;
+                        if (g.vec_store && col + 3 < static_cast<int>(g.n)) {
+                            T o[4] = {acc[t][b][0], acc[t][b][1], acc[t][b][2], acc[t][b][3]};
+                            dh_store_vec_stream<T, 4>(dst, o);
+                        } else {
+#pragma unroll
+                            for (int v = 0; v < 4; v++)
+                                if (col + v < static_cast<int>(g.n))
+                                    dst[v] = acc[t][b][v];
+                        }
+                    }
+                }
+            }
+        } else {
+#pragma unroll
+            for (int t = 0; t < 2; t++)
+#pragma unroll
+                for (int v = 0; v < 4; v++) {
+                    const size_t row = rbase + static_cast<size_t>(t) * 16 + M::row(lane, v);
+                    if (row < g.M) {
+#pragma unroll
+                        for (int b = 0; b < NB; b++)
+                            if (b * 16 + i < static_cast<int>(g.n))
+                                dh_store_stream(C + row * g.ldc + b * 16 + i, acc[t][b][v]);
+                    }
+                }
+        }
+    };
+    // (pair, grp) of a step and of the one after it, stepped without divisions
+    auto advance = [&](unsigned &pair, unsigned &grp) {
+        if (++grp == cg) {
+            grp = 0;
+            if (pair + 1 < RBW / 2)
+                pair++;
+            else
+                grp = cg - 1; // beyond the last step: stay on it
+        }
+    };
+    Frag f0, f1;
+    unsigned lp = 0, lg = 0; // step being loaded
+    unsigned cp = 0, cgp = 0; // step being computed
+    load_step(f0, lp, lg);
+    __builtin_amdgcn_sched_barrier(0);
 
     for (unsigned idx = tid; idx < NB * 16 * (g.kpad / V); idx += 256) {
         const unsigned j = idx / (g.kpad / V), kv = (idx % (g.kpad / V)) * V;
@@ -362,69 +509,20 @@ template <typename T, int NB> __global__ __launch_bounds__(256) void ts_nt_kerne
     }
     __syncthreads();
 
-    const size_t row0 = (static_cast<size_t>(blockIdx.x) * 4 + wave) * (16 * RBW);
-    const unsigned chunks = g.kpad / KC;
-    for (int rb = 0; rb < RBW; rb += 2) {
-        const size_t r0 = row0 + static_cast<size_t>(rb) * 16 + i, r1 = r0 + 16;
-        if (r0 - i >= g.M)
-            break;
-        const bool ok0 = r0 < g.M, ok1 = r1 < g.M;
-        typename M::acc_t acc[2][NB];
-#pragma unroll
-        for (int b = 0; b < NB; b++) {
-            acc[0][b] = typename M::acc_t{0, 0, 0, 0};
-            acc[1][b] = typename M::acc_t{0, 0, 0, 0};
-        }
-        // chunks in groups of 4: eight vector loads in flight per lane
-        for (unsigned c0 = 0; c0 < chunks; c0 += 4) {
-            T fa[2][4][V];
-#pragma unroll
-            for (int c = 0; c < 4; c++) {
-                const unsigned kv = (c0 + c) * KC + h * V;
-                const bool kok = kv < g.K;
-                if (ok0 && kok) {
-                    ts_load<T, V>(A + r0 * g.lda + kv, fa[0][c], true);
-                } else {
-#pragma unroll
-                    for (int e = 0; e < V; e++)
-                        fa[0][c][e] = T(0);
-                }
-                if (ok1 && kok) {
-                    ts_load<T, V>(A + r1 * g.lda + kv, fa[1][c], true);
-                } else {
-#pragma unroll
-                    for (int e = 0; e < V; e++)
-                        fa[1][c][e] = T(0);
-                }
-            }
-#pragma unroll
-            for (int c = 0; c < 4; c++) {
-                if (c0 + c < chunks) {
-#pragma unroll
-                    for (int b = 0; b < NB; b++) {
-                        T fb[V];
-                        dh_load_vec<T, V>(lb + (b * 16 + i) * ldl + (c0 + c) * KC + h * V, fb);
-#pragma unroll
-                        for (int e = 0; e < V; e++) {
-                            acc[0][b] = M::mma(fa[0][c][e], fb[e], acc[0][b]);
-                            acc[1][b] = M::mma(fa[1][c][e], fb[e], acc[1][b]);
-                        }
-                    }
-                }
-            }
-        }
-#pragma unroll
-        for (int t = 0; t < 2; t++)
-#pragma unroll
-            for (int v = 0; v < 4; v++) {
-                const size_t row = row0 + static_cast<size_t>(rb + t) * 16 + M::row(lane, v);
-                if (row < g.M) {
-#pragma unroll
-                    for (int b = 0; b < NB; b++)
-                        if (b * 16 + i < static_cast<int>(g.n))
-                            C[row * g.ldc + b * 16 + i] = acc[t][b][v];
-                }
-            }
+
+    for (unsigned s2 = 0; s2 < nsteps; s2 += 2) {
+        advance(lp, lg);
+        load_step(f1, lp, lg);
+        __builtin_amdgcn_sched_barrier(0);
+        compute_step(f0, cp, cgp);
+        __builtin_amdgcn_sched_barrier(0);
+        advance(cp, cgp);
+        advance(lp, lg);
+        load_step(f0, lp, lg);
+        __builtin_amdgcn_sched_barrier(0);
+        compute_step(f1, cp, cgp);
+        __builtin_amdgcn_sched_barrier(0);
+        advance(cp, cgp);
     }
 }
 
@@ -461,12 +559,15 @@ bool ts_tn(dh_ctx *ctx, size_t m, size_t n, size_t K, const T *A, size_t lda, co
         return false;
     const int wm = cls_a == 2 ? 2 : 1, wn = cls_b == 2 ? 2 : 1, kw = 4 / (wm * wn);
     const int nacc = (cls_a == 0 ? 1 : V * R64) * (cls_b == 0 ? 1 : V * R64);
-    const int unroll = nacc >= 16 ? 2 : 4;
+    const bool sym = static_cast<const void *>(A) == static_cast<const void *>(B) && m == n && lda == ldb && cls_a == 1;
+    const int unroll = nacc >= 16 ? (sym ? TS_SYM_U : 2) : 4; // quads per register set, as in the kernel
     const size_t gran = static_cast<size_t>(4) * kw * unroll;
     // Workgroups: two per CU keep enough loads in flight (more were slower in every shape measured), and
     // each must stream at least eight times the bytes of the slab it writes at the end.
     const size_t slabf = 8;
-    size_t blocks = static_cast<size_t>(ctx->num_cus) * 2;
+    // The symmetric form is bound by the matrix cores as much as by memory; a second workgroup per CU only gets in
+    // the way there (20M x 64 floats: 0.90 ms with one, 1.36 ms with two).
+    size_t blocks = static_cast<size_t>(ctx->num_cus) * (sym ? 1 : 2);
     size_t k_chunk = dh_ceil_div(dh_ceil_div(K, blocks), gran) * gran;
     size_t min_chunk = dh_ceil_div(slabf * m * n, m + n);
     if (min_chunk < gran * 4)
@@ -492,7 +593,7 @@ bool ts_tn(dh_ctx *ctx, size_t m, size_t n, size_t K, const T *A, size_t lda, co
     g.stream = (wm * wn == 1 && static_cast<const void *>(A) != static_cast<const void *>(B)) ? 1 : 0;
     const unsigned nb = static_cast<unsigned>(blocks);
     const size_t elems = m * n;
-    if (static_cast<const void *>(A) == static_cast<const void *>(B) && m == n && lda == ldb && cls_a == 1) {
+    if (sym) {
         // t(X) X with up to 64 columns: upper MFMA tiles only (10 of 16 per step). With 65..128 columns the four
         // waves own one 64 x 64 quadrant each and the slowest of them still has a full one, so nothing is gained.
         ts_tn_launch_sym<T, V, R64, 1>(ctx, g, nb);
@@ -543,6 +644,7 @@ bool ts_nt(dh_ctx *ctx, size_t M, size_t n, size_t K, const T *A, size_t lda, co
     g.n = static_cast<unsigned>(n);
     g.K = static_cast<unsigned>(K);
     g.kpad = static_cast<unsigned>(dh_ceil_div(K, KC) * KC);
+    g.vec_store = dh_aligned(C, 16) && (ldc * sizeof(T)) % 16 == 0;
     const size_t lds = static_cast<size_t>(nb) * 16 * (g.kpad + V) * sizeof(T);
     const size_t blocks = dh_ceil_div(M, 4 * 16 * 8);
     if (blocks >= (size_t(1) << 31) || lds > (size_t(48) << 10))
