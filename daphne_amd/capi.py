@@ -115,6 +115,12 @@ _LATE_SIGNATURES: dict[str, list] = {
     "dh_extract_col": [vp, vp, sz, vp, sz, sz, sz, vp, sz, sz, sz],
     "dh_transpose": [vp, vp, sz, vp, sz, sz, sz],
     "dh_gemv": [vp, vp, sz, vp, sz, sz, sz, vp, sz, sz],
+    "dh_batchnorm_train_forward": [vp, vp, vp, vp, vp, vp, vp, sz, sz, vp, vp, vp, vp, sz, "T", "T"],
+    "dh_batchnorm_backward": [vp, vp, vp, vp, vp, vp, vp, vp, sz, sz, vp, sz, "T"],
+    "dh_maxpool_backward": [vp, vp, vp, vp, sz, sz, sz, sz, sz, sz, sz, sz, sz, sz],
+    "dh_avgpool_backward": [vp, vp, vp, vp, sz, sz, sz, sz, sz, sz, sz, sz, sz, sz],
+    "dh_conv2d_backward_data": [vp, vp, vp, vp, sz, sz, sz, sz, sz, sz, sz, sz, sz, sz, sz],
+    "dh_conv2d_backward_filter": [vp, vp, vp, vp, sz, sz, sz, sz, sz, sz, sz, sz, sz, sz, sz],
 }
 
 

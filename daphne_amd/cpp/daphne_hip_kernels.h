@@ -200,6 +200,12 @@ DH_OVERLOAD2(dh_col_bind)
 DH_OVERLOAD2(dh_extract_col)
 DH_OVERLOAD2(dh_transpose)
 DH_OVERLOAD2(dh_gemv)
+DH_OVERLOAD2(dh_batchnorm_train_forward)
+DH_OVERLOAD2(dh_batchnorm_backward)
+DH_OVERLOAD2(dh_maxpool_backward)
+DH_OVERLOAD2(dh_avgpool_backward)
+DH_OVERLOAD2(dh_conv2d_backward_data)
+DH_OVERLOAD2(dh_conv2d_backward_filter)
 #undef DH_OVERLOAD2
 // integer value types, as far as the reference instantiates its device kernels for them
 // (kernels/CUDA/EwBinaryMat.cu:267-270, EwBinaryObjSca.cu:91-94, AggAll.cu:155, AggRow.cu:146, AggCol.cu:89,
@@ -601,5 +607,89 @@ template <class DTRes, class DTMat, class DTVec> struct Gemv {
 template <class DTRes, class DTMat, class DTVec> void gemv(DTRes *&res, const DTMat *mat, const DTVec *vec, DCTX(ctx)) {
     Gemv<DTRes, DTMat, DTVec>::apply(res, mat, vec, ctx);
 }
+
+// --- DNN training kernels: the reference has them on the CPU only; same template parameters and argument order ---
+// BatchNorm2DTrainForward (kernels/BatchNorm2DTrainForward.h:38-57). The four statistics results are C x 1 here
+// (the reference allocates C x C and fills the first C values).
+template <class DTRes, class DTArg> struct BatchNorm2DTrainForward {
+    static void apply(DTRes *&res, DTRes *&new_emaMean, DTRes *&new_emaVar, DTRes *&mean, DTRes *&invVar, const DTArg *in,
+                      const DTArg *gamma, const DTArg *beta, const DTArg *emaMean, const DTArg *emaVar,
+                      const typename DTArg::VT eps, const typename DTArg::VT mu, DCTX(ctx)) {
+        using VT = typename DTArg::VT;
+        const size_t C = gamma->getNumRows() * gamma->getNumCols();
+        if (res == nullptr)
+            res = DataObjectFactory::create<DTRes>(in->getNumRows(), in->getNumCols(), false, ctx);
+        for (DTRes **m : {&new_emaMean, &new_emaVar, &mean, &invVar})
+            if (*m == nullptr)
+                *m = DataObjectFactory::create<DTRes>(C, 1, false, ctx);
+        check(dh_batchnorm_train_forward(VT(), detail::raw(ctx), res->getValues(), new_emaMean->getValues(),
+                                         new_emaVar->getValues(), mean->getValues(), invVar->getValues(), in->getValues(),
+                                         in->getNumRows(), in->getNumCols(), gamma->getValues(), beta->getValues(),
+                                         emaMean->getValues(), emaVar->getValues(), C, eps, mu));
+    }
+};
+// BatchNorm2DBackward (kernels/BatchNorm2DBackward.h:38-53)
+template <class DTRes, class DTArg> struct BatchNorm2DBackward {
+    static void apply(DTRes *&dX, DTRes *&dGamma, DTRes *&dBeta, const DTArg *mean, const DTArg *invVar, const DTArg *in,
+                      const DTArg *dout, const DTArg *gamma, const typename DTArg::VT eps, DCTX(ctx)) {
+        using VT = typename DTArg::VT;
+        const size_t C = gamma->getNumRows() * gamma->getNumCols();
+        if (dX == nullptr)
+            dX = DataObjectFactory::create<DTRes>(in->getNumRows(), in->getNumCols(), false, ctx);
+        if (dGamma == nullptr)
+            dGamma = DataObjectFactory::create<DTRes>(C, 1, false, ctx);
+        if (dBeta == nullptr)
+            dBeta = DataObjectFactory::create<DTRes>(C, 1, false, ctx);
+        check(dh_batchnorm_backward(VT(), detail::raw(ctx), dX->getValues(), dGamma->getValues(), dBeta->getValues(),
+                                    mean->getValues(), invVar->getValues(), in->getValues(), dout->getValues(), in->getNumRows(),
+                                    in->getNumCols(), gamma->getValues(), C, eps));
+    }
+};
+// MaxPoolBackward / AvgPoolBackward (kernels/MaxPoolBackward.h:35-40, AvgPoolBackward.h:35-40)
+#define DH_POOL_BACKWARD(NAME, FN)                                                                                      \
+    template <class DTRes, class DTArg> struct NAME {                                                                   \
+        static void apply(DTRes *&res, const DTArg *input, const DTArg *dOut, const size_t batch_size,                  \
+                          const size_t num_channels, const size_t img_h, const size_t img_w, const size_t pool_h,       \
+                          const size_t pool_w, const size_t stride_h, const size_t stride_w, const size_t pad_h,        \
+                          const size_t pad_w, DCTX(ctx)) {                                                              \
+            using VT = typename DTArg::VT;                                                                              \
+            if (res == nullptr)                                                                                         \
+                res = DataObjectFactory::create<DTRes>(batch_size, num_channels * img_h * img_w, false, ctx);           \
+            check(FN(VT(), detail::raw(ctx), res->getValues(), input->getValues(), dOut->getValues(), batch_size,       \
+                     num_channels, img_h, img_w, pool_h, pool_w, stride_h, stride_w, pad_h, pad_w));                    \
+        }                                                                                                               \
+    };
+DH_POOL_BACKWARD(MaxPoolBackward, dh_maxpool_backward)
+DH_POOL_BACKWARD(AvgPoolBackward, dh_avgpool_backward)
+#undef DH_POOL_BACKWARD
+// Conv2DBackwardData (kernels/Conv2DBackwardData.h:35-46): `output` is the gradient w.r.t. the convolution's result
+template <class DTRes, class DTArg> struct Conv2DBackwardData {
+    static void apply(const DTArg *filter, const DTArg *output, const size_t stride_h, const size_t stride_w, const size_t pad_h,
+                      const size_t pad_w, const size_t input_batch_size, const size_t input_num_channels, const size_t input_h,
+                      const size_t input_w, const size_t filter_num_filters, const size_t filter_num_channels,
+                      const size_t filter_h, const size_t filter_w, DTRes *&data, DCTX(ctx)) {
+        using VT = typename DTArg::VT;
+        (void)filter_num_channels;
+        if (data == nullptr)
+            data = DataObjectFactory::create<DTRes>(input_batch_size, input_num_channels * input_h * input_w, false, ctx);
+        check(dh_conv2d_backward_data(VT(), detail::raw(ctx), data->getValues(), filter->getValues(), output->getValues(),
+                                      input_batch_size, input_num_channels, input_h, input_w, filter_num_filters, filter_h,
+                                      filter_w, stride_h, stride_w, pad_h, pad_w));
+    }
+};
+// Conv2DBackwardFilter (kernels/Conv2DBackwardFilter.h:35-46)
+template <class DTRes, class DTArg> struct Conv2DBackwardFilter {
+    static void apply(DTRes *&dFilter, const DTArg *input, const DTArg *output, const size_t stride_h, const size_t stride_w,
+                      const size_t pad_h, const size_t pad_w, const size_t input_batch_size, const size_t input_num_channels,
+                      const size_t input_h, const size_t input_w, const size_t filter_num_filters,
+                      const size_t filter_num_channels, const size_t filter_h, const size_t filter_w, DCTX(ctx)) {
+        using VT = typename DTArg::VT;
+        if (dFilter == nullptr)
+            dFilter = DataObjectFactory::create<DTRes>(filter_num_filters, filter_num_channels * filter_h * filter_w, false, ctx);
+        check(dh_conv2d_backward_filter(VT(), detail::raw(ctx), dFilter->getValues(), input->getValues(), output->getValues(),
+                                        input_batch_size, input_num_channels, input_h, input_w, filter_num_filters, filter_h,
+                                        filter_w, stride_h, stride_w, pad_h, pad_w));
+    }
+};
 
 } // namespace HIP

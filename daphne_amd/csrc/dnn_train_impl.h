@@ -1,0 +1,472 @@
+// DNN training kernels for DenseMatrix<float|double>: batch normalisation in training mode (forward) and the backward
+// passes of batch normalisation, max / average pooling and 2-D convolution. The reference has these as CPU kernels
+// only (src/runtime/local/kernels/BatchNorm2DTrainForward.h:66-118, BatchNorm2DBackward.h:63-120,
+// MaxPoolBackward.h:35-82, AvgPoolBackward.h:35-77, Conv2DBackwardData.h:88-158, Conv2DBackwardFilter.h:68-152);
+// these are their device counterparts, data NCHW as rows of images like the forward kernels.
+//
+// Per-channel statistics are deterministic two-stage reductions with double accumulators (every workgroup owns a
+// channel and a slice of the images; a small second kernel folds the slices in order and derives the per-channel
+// coefficients); the elementwise passes use one 16-byte vector per thread where the layout allows. The pooling and
+// convolution gradients are written as gathers - one thread per gradient element, visiting its contributions in the
+// reference's order - so that no atomics are needed and results do not depend on timing.
+//
+// Pooling keeps the forward kernels' quirk of taking the output height from stride_w and the width from stride_h
+// (MaxPoolBackward.h:45-46). Conv2DBackwardData of the reference is only consistent where the output extent equals
+// the filter extent; here it is the adjoint of the forward convolution for every shape, which coincides with the
+// reference there (its test vector is reproduced).
+#pragma once
+
+#include "common.h"
+
+#include <cmath>
+
+namespace dh_train {
+
+constexpr int THREADS = 256;
+
+// ---------------------------------------------------------------------------------------
+// per-channel reductions
+// ---------------------------------------------------------------------------------------
+// MODE 0: sum x          MODE 1: sum (x - mean[c])^2          MODE 2: sum dy, sum dy*(x - mean[c]), sum (x - mean[c])
+template <typename T, int MODE>
+__global__ __launch_bounds__(THREADS) void chan_stage1(const T *x, const T *dy, const T *mean, size_t N, size_t C, size_t HW,
+                                                       size_t imgs_per_slice, double *partials /* [C][S][3] */) {
+    constexpr int K = MODE == 2 ? 3 : 1;
+    __shared__ double lds[K][THREADS / DH_WAVE];
+    const size_t c = blockIdx.x, s = blockIdx.y;
+    const size_t n0 = s * imgs_per_slice, n1 = (n0 + imgs_per_slice < N) ? n0 + imgs_per_slice : N;
+    const size_t CHW = C * HW;
+    const double mu = MODE >= 1 ? static_cast<double>(mean[c]) : 0.0;
+    double a0 = 0.0, a1 = 0.0, a2 = 0.0;
+    const size_t items = (n1 > n0 ? n1 - n0 : 0) * HW;
+    for (size_t i = threadIdx.x; i < items; i += THREADS) {
+        const size_t n = n0 + i / HW, j = i % HW;
+        const size_t off = n * CHW + c * HW + j;
+        const double v = static_cast<double>(x[off]);
+        if constexpr (MODE == 0) {
+            a0 += v;
+        } else if constexpr (MODE == 1) {
+            a0 += (v - mu) * (v - mu);
+        } else {
+            const double g = static_cast<double>(dy[off]);
+            a0 += g;
+            a1 += g * (v - mu);
+            a2 += v - mu;
+        }
+    }
+    double a[3] = {a0, a1, a2};
+#pragma unroll
+    for (int k = 0; k < K; k++) {
+        double v = a[k];
+        dh_butterfly(DH_WAVE, [&](auto peer) { v += peer(v); });
+        if (threadIdx.x % DH_WAVE == 0)
+            lds[k][threadIdx.x / DH_WAVE] = v;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+#pragma unroll
+        for (int k = 0; k < K; k++) {
+            double v = 0.0;
+            for (int w = 0; w < THREADS / DH_WAVE; w++)
+                v += lds[k][w];
+            partials[(c * gridDim.y + s) * 3 + k] = v;
+        }
+    }
+}
+
+// Folds the slices of every channel (one thread per channel, slices in order) and derives what the next pass needs.
+// STEP 0: mean[c] = sum / m.
+// STEP 1: var = sum / m; inv_var, moving averages; coef[c] = sqrt(var + eps) for the normalisation pass.
+// STEP 2: dBeta, dGamma and coef[c][0..1] = dVar * 2/m, dMean / m for the gradient pass.
+template <typename T, int STEP>
+__global__ void chan_stage2(const double *partials, size_t C, size_t S, double m, T *mean, T *inv_var, T *new_ema_mean,
+                            T *new_ema_var, const T *ema_mean, const T *ema_var, T eps, T mu_, const T *gamma, T *dGamma,
+                            T *dBeta, T *coef) {
+    const size_t c = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (c >= C)
+        return;
+    double s0 = 0.0, s1 = 0.0, s2 = 0.0;
+    for (size_t s = 0; s < S; s++) {
+        s0 += partials[(c * S + s) * 3 + 0];
+        if (STEP == 2) {
+            s1 += partials[(c * S + s) * 3 + 1];
+            s2 += partials[(c * S + s) * 3 + 2];
+        }
+    }
+    if constexpr (STEP == 0) {
+        mean[c] = static_cast<T>(s0 / m);
+    } else if constexpr (STEP == 1) {
+        const T var = static_cast<T>(s0 / m), mn = mean[c];
+        const T sd = sizeof(T) == 4 ? static_cast<T>(sqrtf(static_cast<float>(var + eps))) : static_cast<T>(sqrt(static_cast<double>(var + eps)));
+        inv_var[c] = T(1) / sd;
+        new_ema_mean[c] = (T(1) - mu_) * ema_mean[c] + mu_ * mn;
+        new_ema_var[c] = (T(1) - mu_) * ema_var[c] + mu_ * var;
+        coef[c] = sd;
+    } else {
+        // BatchNorm2DBackward.h:88-118 with the sums taken out of the loops
+        const double iv = static_cast<double>(inv_var[c]), g = static_cast<double>(gamma[c]);
+        dBeta[c] = static_cast<T>(s0);
+        dGamma[c] = static_cast<T>(s1 * iv);
+        const double dVar = -(g * s1) * 0.5 * iv * iv * iv;
+        const double c2m = 2.0 / m;
+        const double dMean = -(g * s0) * iv + dVar * (-c2m) * s2;
+        coef[2 * c] = static_cast<T>(dVar * c2m);
+        coef[2 * c + 1] = static_cast<T>(dMean / m);
+    }
+}
+
+// Elementwise passes over the (N*C) x HW view. FWD: res = gamma * ((x - mean) / sd) + beta
+// (BatchNorm2DTrainForward.h:108-115). Else: dX = (dy * gamma) * inv_var + coef0 * (x - mean) + coef1
+// (BatchNorm2DBackward.h:110-118).
+template <typename T, int VEC, bool FWD>
+__global__ __launch_bounds__(THREADS) void chan_apply(T *res, const T *x, const T *dy, size_t rows, size_t C, size_t HW,
+                                                      const T *mean, const T *gamma, const T *beta, const T *inv_var,
+                                                      const T *coef) {
+    const size_t cvecs = HW / VEC;
+    const size_t r = static_cast<size_t>(blockIdx.x) * blockDim.y + threadIdx.y;
+    if (r >= rows)
+        return;
+    const size_t c = r % C;
+    const T mn = mean[c], g = gamma[c];
+    const T p0 = FWD ? coef[c] : inv_var[c], p1 = FWD ? beta[c] : coef[2 * c], p2 = FWD ? T(0) : coef[2 * c + 1];
+    for (size_t cv = static_cast<size_t>(blockIdx.y) * blockDim.x + threadIdx.x; cv < cvecs;
+         cv += static_cast<size_t>(gridDim.y) * blockDim.x) {
+        T a[VEC], b[VEC], o[VEC];
+        dh_load_vec_stream<T, VEC>(x + r * HW + cv * VEC, a);
+        if constexpr (!FWD)
+            dh_load_vec_stream<T, VEC>(dy + r * HW + cv * VEC, b);
+#pragma unroll
+        for (int i = 0; i < VEC; i++) {
+            if constexpr (FWD)
+                o[i] = g * ((a[i] - mn) / p0) + p1;
+            else
+                o[i] = (b[i] * g) * p0 + p1 * (a[i] - mn) + p2;
+        }
+        dh_store_vec_stream<T, VEC>(res + r * HW + cv * VEC, o);
+    }
+}
+
+struct ChanPlan {
+    size_t S, imgs_per_slice;
+};
+static inline ChanPlan chan_plan(const dh_ctx *ctx, size_t N, size_t C) {
+    // about eight workgroups per CU over all channels, every slice at least one image
+    size_t S = dh_ceil_div(static_cast<size_t>(ctx->num_cus) * 8, C);
+    if (S > N)
+        S = N;
+    if (S < 1)
+        S = 1;
+    if (S > 65535)
+        S = 65535;
+    ChanPlan p;
+    p.imgs_per_slice = dh_ceil_div(N, S);
+    p.S = dh_ceil_div(N, p.imgs_per_slice);
+    return p;
+}
+
+template <typename T, bool FWD>
+static inline void launch_apply(dh_ctx *ctx, T *res, const T *x, const T *dy, size_t rows, size_t C, size_t HW, const T *mean,
+                                const T *gamma, const T *beta, const T *inv_var, const T *coef) {
+    constexpr int V = dh_vec<T>::N;
+    const bool vec_ok = HW % V == 0 && dh_aligned(res, 16) && dh_aligned(x, 16) && (FWD || dh_aligned(dy, 16));
+    const size_t cvecs = vec_ok ? HW / V : HW;
+    unsigned tx = 1;
+    while (tx < THREADS && tx < cvecs)
+        tx <<= 1;
+    const unsigned ty = THREADS / tx;
+    size_t gy = dh_ceil_div(cvecs, tx);
+    if (gy > 65535)
+        gy = 65535;
+    const dim3 grid(static_cast<unsigned>(dh_ceil_div(rows, static_cast<size_t>(ty))), static_cast<unsigned>(gy)), block(tx, ty);
+    if (vec_ok)
+        hipLaunchKernelGGL((chan_apply<T, V, FWD>), grid, block, 0, ctx->stream, res, x, dy, rows, C, HW, mean, gamma, beta,
+                           inv_var, coef);
+    else
+        hipLaunchKernelGGL((chan_apply<T, 1, FWD>), grid, block, 0, ctx->stream, res, x, dy, rows, C, HW, mean, gamma, beta,
+                           inv_var, coef);
+}
+
+template <typename T>
+dh_status batchnorm_train_forward(dh_ctx *ctx, T *res, T *new_ema_mean, T *new_ema_var, T *mean, T *inv_var, const T *in,
+                                  size_t rows, size_t cols, const T *gamma, const T *beta, const T *ema_mean, const T *ema_var,
+                                  size_t C, T eps, T mu) {
+    DH_REQUIRE_CTX(ctx);
+    if (C == 0 || cols % C != 0)
+        return dh_fail(DH_ERR_INVALID_ARG, "BatchNorm2DTrainForward - the number of columns (%zu) is not a multiple of the channel count (%zu)", cols, C);
+    if (rows == 0 || cols == 0)
+        return DH_OK;
+    if (rows * (cols / C) >= (size_t(1) << 31) * C && rows >= (size_t(1) << 31))
+        return dh_fail(DH_ERR_RUNTIME, "BatchNorm2DTrainForward - too many images");
+    const size_t HW = cols / C;
+    const ChanPlan p = chan_plan(ctx, rows, C);
+    void *wsv = nullptr;
+    dh_status st = dh_workspace(ctx, C * p.S * 3 * sizeof(double) + 2 * C * sizeof(T) + 256, &wsv);
+    if (st != DH_OK)
+        return st;
+    double *partials = static_cast<double *>(wsv);
+    T *coef = reinterpret_cast<T *>(partials + C * p.S * 3);
+    const double m = static_cast<double>(rows) * static_cast<double>(HW);
+    const dim3 g1(static_cast<unsigned>(C), static_cast<unsigned>(p.S)), g2(static_cast<unsigned>(dh_ceil_div(C, 64)));
+    hipLaunchKernelGGL((chan_stage1<T, 0>), g1, dim3(THREADS), 0, ctx->stream, in, nullptr, nullptr, rows, C, HW,
+                       p.imgs_per_slice, partials);
+    hipLaunchKernelGGL((chan_stage2<T, 0>), g2, dim3(64), 0, ctx->stream, partials, C, p.S, m, mean, inv_var, new_ema_mean,
+                       new_ema_var, ema_mean, ema_var, eps, mu, gamma, nullptr, nullptr, coef);
+    hipLaunchKernelGGL((chan_stage1<T, 1>), g1, dim3(THREADS), 0, ctx->stream, in, nullptr, mean, rows, C, HW, p.imgs_per_slice,
+                       partials);
+    hipLaunchKernelGGL((chan_stage2<T, 1>), g2, dim3(64), 0, ctx->stream, partials, C, p.S, m, mean, inv_var, new_ema_mean,
+                       new_ema_var, ema_mean, ema_var, eps, mu, gamma, nullptr, nullptr, coef);
+    launch_apply<T, true>(ctx, res, in, nullptr, rows * C, C, HW, mean, gamma, beta, inv_var, coef);
+    DH_CHECK_LAUNCH();
+    return DH_OK;
+}
+
+template <typename T>
+dh_status batchnorm_backward(dh_ctx *ctx, T *dX, T *dGamma, T *dBeta, const T *mean, const T *inv_var, const T *in, const T *dout,
+                             size_t rows, size_t cols, const T *gamma, size_t C) {
+    DH_REQUIRE_CTX(ctx);
+    if (C == 0 || cols % C != 0)
+        return dh_fail(DH_ERR_INVALID_ARG, "BatchNorm2DBackward - the number of columns (%zu) is not a multiple of the channel count (%zu)", cols, C);
+    if (rows == 0 || cols == 0)
+        return DH_OK;
+    const size_t HW = cols / C;
+    const ChanPlan p = chan_plan(ctx, rows, C);
+    void *wsv = nullptr;
+    dh_status st = dh_workspace(ctx, C * p.S * 3 * sizeof(double) + 2 * C * sizeof(T) + 256, &wsv);
+    if (st != DH_OK)
+        return st;
+    double *partials = static_cast<double *>(wsv);
+    T *coef = reinterpret_cast<T *>(partials + C * p.S * 3);
+    const double m = static_cast<double>(rows) * static_cast<double>(HW);
+    const dim3 g1(static_cast<unsigned>(C), static_cast<unsigned>(p.S)), g2(static_cast<unsigned>(dh_ceil_div(C, 64)));
+    hipLaunchKernelGGL((chan_stage1<T, 2>), g1, dim3(THREADS), 0, ctx->stream, in, dout, mean, rows, C, HW, p.imgs_per_slice,
+                       partials);
+    hipLaunchKernelGGL((chan_stage2<T, 2>), g2, dim3(64), 0, ctx->stream, partials, C, p.S, m, const_cast<T *>(mean),
+                       const_cast<T *>(inv_var), nullptr, nullptr, nullptr, nullptr, T(0), T(0), gamma, dGamma, dBeta, coef);
+    launch_apply<T, false>(ctx, dX, in, dout, rows * C, C, HW, mean, gamma, nullptr, inv_var, coef);
+    DH_CHECK_LAUNCH();
+    return DH_OK;
+}
+
+// ---------------------------------------------------------------------------------------
+// pooling backward (gather form)
+// ---------------------------------------------------------------------------------------
+struct PoolBwdArgs {
+    unsigned C, H, W, P, Q, ph, pw, sh, sw, padh, padw;
+    size_t total; // N*C*H*W
+};
+
+template <typename T, bool AVG>
+__global__ __launch_bounds__(THREADS) void pool_backward_kernel(T *res, const T *input, const T *dOut, PoolBwdArgs g) {
+#pragma clang fp contract(off) // plen * g is rounded before it is added, as on the host
+    const size_t idx = static_cast<size_t>(blockIdx.x) * THREADS + threadIdx.x;
+    if (idx >= g.total)
+        return;
+    const unsigned HW = g.H * g.W;
+    const size_t img = idx / HW; // (n, c) plane
+    const unsigned hw = static_cast<unsigned>(idx % HW), h = hw / g.W, w = hw % g.W;
+    const unsigned hp = h + g.padh, wp = w + g.padw; // position in the zero-padded plane
+    const unsigned pH = g.H + 2 * g.padh, pW = g.W + 2 * g.padw;
+    const T *plane = input + img * HW;
+    const T *dplane = dOut + img * (static_cast<size_t>(g.P) * g.Q);
+    const T plen = T(1) / static_cast<T>(g.pw * g.ph);
+    // windows (p, q) that contain (hp, wp): p*sh <= hp < p*sh + ph
+    const unsigned p_lo = hp + 1 > g.ph ? (hp + 1 - g.ph + g.sh - 1) / g.sh : 0, q_lo = wp + 1 > g.pw ? (wp + 1 - g.pw + g.sw - 1) / g.sw : 0;
+    unsigned p_hi = hp / g.sh, q_hi = wp / g.sw;
+    if (p_hi >= g.P)
+        p_hi = g.P - 1;
+    if (q_hi >= g.Q)
+        q_hi = g.Q - 1;
+    auto val = [&](unsigned a, unsigned b) -> T { // padded plane
+        return (a >= g.padh && b >= g.padw && a - g.padh < g.H && b - g.padw < g.W) ? plane[(a - g.padh) * g.W + (b - g.padw)] : T(0);
+    };
+    T acc = T(0);
+    for (unsigned p = p_lo; p <= p_hi && p < g.P; p++)
+        for (unsigned q = q_lo; q <= q_hi && q < g.Q; q++) {
+            if (p * g.sh + g.ph > pH || q * g.sw + g.pw > pW)
+                continue; // window would leave the padded plane
+            const T gr = dplane[p * g.Q + q];
+            if constexpr (AVG) {
+                acc = acc + plen * gr;
+            } else {
+                // first maximum in row-major order, found with a strict comparison starting from the window origin
+                unsigned ma = p * g.sh, mb = q * g.sw;
+                T mv = val(ma, mb);
+                for (unsigned a = 0; a < g.ph; a++)
+                    for (unsigned b = 0; b < g.pw; b++) {
+                        const T v = val(p * g.sh + a, q * g.sw + b);
+                        if (v > mv) {
+                            mv = v;
+                            ma = p * g.sh + a;
+                            mb = q * g.sw + b;
+                        }
+                    }
+                if (ma == hp && mb == wp)
+                    acc = acc + gr;
+            }
+        }
+    res[idx] = acc;
+}
+
+template <typename T, bool AVG>
+dh_status pool_backward(dh_ctx *ctx, T *res, const T *input, const T *dOut, size_t N, size_t C, size_t H, size_t W, size_t ph,
+                        size_t pw, size_t sh, size_t sw, size_t padh, size_t padw) {
+    DH_REQUIRE_CTX(ctx);
+    if (H + 2 * padh < ph || W + 2 * padw < pw || sh == 0 || sw == 0 || ph == 0 || pw == 0)
+        return dh_fail(DH_ERR_INVALID_ARG, "Pooling backward - window, stride and padding do not fit the image");
+    if ((H | W | C | ph | pw | sh | sw | padh | padw) >> 30)
+        return dh_fail(DH_ERR_RUNTIME, "Pooling backward - extents beyond 2^30 are not supported");
+    PoolBwdArgs g;
+    g.C = C, g.H = H, g.W = W, g.ph = ph, g.pw = pw, g.sh = sh, g.sw = sw, g.padh = padh, g.padw = padw;
+    g.P = static_cast<unsigned>((H + 2 * padh - ph) / sw + 1); // stride_w for the height, as in the reference
+    g.Q = static_cast<unsigned>((W + 2 * padw - pw) / sh + 1);
+    g.total = N * C * H * W;
+    if (g.total == 0)
+        return DH_OK;
+    const size_t blocks = dh_ceil_div(g.total, THREADS);
+    if (blocks >= (size_t(1) << 31))
+        return dh_fail(DH_ERR_RUNTIME, "Pooling backward - too many elements for one launch");
+    hipLaunchKernelGGL((pool_backward_kernel<T, AVG>), dim3(static_cast<unsigned>(blocks)), dim3(THREADS), 0, ctx->stream, res,
+                       input, dOut, g);
+    DH_CHECK_LAUNCH();
+    return DH_OK;
+}
+
+// ---------------------------------------------------------------------------------------
+// convolution backward
+// ---------------------------------------------------------------------------------------
+struct ConvBwdArgs {
+    unsigned N, C, H, W, F, Hf, Wf, P, Q, sh, sw, padh, padw;
+};
+
+// dX[n][c][h][w] = sum_f sum_r sum_s dY[n][f][p][q] * Wt[f][c][r][s], p*sh + r = h + padh, q*sw + s = w + padw;
+// one thread per element, filters ascending and filter rows / columns descending like the reference's rotated filter.
+template <typename T> __global__ __launch_bounds__(THREADS) void conv_backward_data_kernel(T *dX, const T *filter, const T *dY, ConvBwdArgs g) {
+    const size_t total = static_cast<size_t>(g.N) * g.C * g.H * g.W;
+    const size_t idx = static_cast<size_t>(blockIdx.x) * THREADS + threadIdx.x;
+    if (idx >= total)
+        return;
+    const unsigned HW = g.H * g.W, PQ = g.P * g.Q;
+    const size_t nc = idx / HW;
+    const unsigned n = static_cast<unsigned>(nc / g.C), c = static_cast<unsigned>(nc % g.C);
+    const unsigned hw = static_cast<unsigned>(idx % HW), hh = hw / g.W + g.padh, ww = hw % g.W + g.padw;
+    const T *dyn = dY + static_cast<size_t>(n) * g.F * PQ;
+    T acc = T(0);
+    for (unsigned f = 0; f < g.F; f++) {
+        const T *wf = filter + (static_cast<size_t>(f) * g.C + c) * g.Hf * g.Wf;
+        const T *dyf = dyn + static_cast<size_t>(f) * PQ;
+        for (unsigned r = g.Hf; r-- > 0;) {
+            if (hh < r || (hh - r) % g.sh)
+                continue;
+            const unsigned p = (hh - r) / g.sh;
+            if (p >= g.P)
+                continue;
+            for (unsigned s = g.Wf; s-- > 0;) {
+                if (ww < s || (ww - s) % g.sw)
+                    continue;
+                const unsigned q = (ww - s) / g.sw;
+                if (q >= g.Q)
+                    continue;
+                acc = acc + dyf[p * g.Q + q] * wf[r * g.Wf + s];
+            }
+        }
+    }
+    dX[idx] = acc;
+}
+
+// dW[f][c][r][s] = sum_n sum_p sum_q Xpad[n][c][p*sh + r][q*sw + s] * dY[n][f][p][q]. One workgroup per (f, c): its
+// threads walk over (n, p, q), each keeping the partial sums of up to TAPS filter taps in registers (larger filters
+// take several rounds); the partial sums are folded through LDS in a fixed order, in double.
+template <typename T, int TAPS>
+__global__ __launch_bounds__(THREADS) void conv_backward_filter_kernel(T *dW, const T *input, const T *dY, ConvBwdArgs g) {
+    __shared__ double lds[THREADS / DH_WAVE][TAPS];
+    const unsigned f = blockIdx.x / g.C, c = blockIdx.x % g.C;
+    const unsigned HW = g.H * g.W, PQ = g.P * g.Q, taps = g.Hf * g.Wf;
+    const size_t items = static_cast<size_t>(g.N) * PQ;
+    for (unsigned t0 = 0; t0 < taps; t0 += TAPS) {
+        double acc[TAPS];
+#pragma unroll
+        for (int t = 0; t < TAPS; t++)
+            acc[t] = 0.0;
+        for (size_t i = threadIdx.x; i < items; i += THREADS) {
+            const unsigned n = static_cast<unsigned>(i / PQ), pq = static_cast<unsigned>(i % PQ), p = pq / g.Q, q = pq % g.Q;
+            const double gr = static_cast<double>(dY[(static_cast<size_t>(n) * g.F + f) * PQ + pq]);
+            const T *plane = input + (static_cast<size_t>(n) * g.C + c) * HW;
+#pragma unroll
+            for (int t = 0; t < TAPS; t++) {
+                const unsigned tap = t0 + t;
+                if (tap < taps) {
+                    const unsigned hh = p * g.sh + tap / g.Wf, ww = q * g.sw + tap % g.Wf;
+                    if (hh >= g.padh && ww >= g.padw && hh - g.padh < g.H && ww - g.padw < g.W)
+                        acc[t] += static_cast<double>(plane[(hh - g.padh) * g.W + (ww - g.padw)]) * gr;
+                }
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < TAPS; t++) {
+            double v = acc[t];
+            dh_butterfly(DH_WAVE, [&](auto peer) { v += peer(v); });
+            if (threadIdx.x % DH_WAVE == 0)
+                lds[threadIdx.x / DH_WAVE][t] = v;
+        }
+        __syncthreads();
+        if (threadIdx.x < TAPS && t0 + threadIdx.x < taps) {
+            double v = 0.0;
+            for (int w = 0; w < THREADS / DH_WAVE; w++)
+                v += lds[w][threadIdx.x];
+            dW[(static_cast<size_t>(f) * g.C + c) * taps + t0 + threadIdx.x] = static_cast<T>(v);
+        }
+        __syncthreads();
+    }
+}
+
+static inline dh_status conv_bwd_args(ConvBwdArgs *g, size_t N, size_t C, size_t H, size_t W, size_t F, size_t Hf, size_t Wf,
+                                      size_t sh, size_t sw, size_t padh, size_t padw) {
+    if (H + 2 * padh < Hf || W + 2 * padw < Wf || sh == 0 || sw == 0 || Hf == 0 || Wf == 0)
+        return dh_fail(DH_ERR_INVALID_ARG, "Conv2D backward - filter, stride and padding do not fit the image");
+    if ((N | C | H | W | F | Hf | Wf | sh | sw | padh | padw) >> 30)
+        return dh_fail(DH_ERR_RUNTIME, "Conv2D backward - extents beyond 2^30 are not supported");
+    g->N = N, g->C = C, g->H = H, g->W = W, g->F = F, g->Hf = Hf, g->Wf = Wf, g->sh = sh, g->sw = sw, g->padh = padh, g->padw = padw;
+    g->P = static_cast<unsigned>((H + 2 * padh - Hf) / sh + 1);
+    g->Q = static_cast<unsigned>((W + 2 * padw - Wf) / sw + 1);
+    return DH_OK;
+}
+
+template <typename T>
+dh_status conv2d_backward_data(dh_ctx *ctx, T *dX, const T *filter, const T *dY, size_t N, size_t C, size_t H, size_t W, size_t F,
+                               size_t Hf, size_t Wf, size_t sh, size_t sw, size_t padh, size_t padw) {
+    DH_REQUIRE_CTX(ctx);
+    ConvBwdArgs g;
+    dh_status st = conv_bwd_args(&g, N, C, H, W, F, Hf, Wf, sh, sw, padh, padw);
+    if (st != DH_OK)
+        return st;
+    const size_t total = N * C * H * W;
+    if (total == 0)
+        return DH_OK;
+    const size_t blocks = dh_ceil_div(total, THREADS);
+    if (blocks >= (size_t(1) << 31))
+        return dh_fail(DH_ERR_RUNTIME, "Conv2D backward - too many elements for one launch");
+    hipLaunchKernelGGL((conv_backward_data_kernel<T>), dim3(static_cast<unsigned>(blocks)), dim3(THREADS), 0, ctx->stream, dX, filter,
+                       dY, g);
+    DH_CHECK_LAUNCH();
+    return DH_OK;
+}
+
+template <typename T>
+dh_status conv2d_backward_filter(dh_ctx *ctx, T *dW, const T *input, const T *dY, size_t N, size_t C, size_t H, size_t W, size_t F,
+                                 size_t Hf, size_t Wf, size_t sh, size_t sw, size_t padh, size_t padw) {
+    DH_REQUIRE_CTX(ctx);
+    ConvBwdArgs g;
+    dh_status st = conv_bwd_args(&g, N, C, H, W, F, Hf, Wf, sh, sw, padh, padw);
+    if (st != DH_OK)
+        return st;
+    if (F * C == 0)
+        return DH_OK;
+    if (F * C >= (size_t(1) << 31))
+        return dh_fail(DH_ERR_RUNTIME, "Conv2D backward - too many filter planes for one launch");
+    hipLaunchKernelGGL((conv_backward_filter_kernel<T, 16>), dim3(static_cast<unsigned>(F * C)), dim3(THREADS), 0, ctx->stream, dW,
+                       input, dY, g);
+    DH_CHECK_LAUNCH();
+    return DH_OK;
+}
+
+} // namespace dh_train

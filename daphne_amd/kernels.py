@@ -475,3 +475,79 @@ def gemv(res, mat: DenseMatrix, vec: DenseMatrix, ctx: HIPContext) -> DenseMatri
     capi.check(_fn("dh_gemv", dt)(ctx._h, res.ptr, res.row_skip, mat.ptr, mat.rows, mat.cols, mat.row_skip, vec.ptr,
                                   vec.rows, vec.row_skip))
     return res
+
+
+# ------------------------------------------------------------------------------------------
+# DNN training kernels
+# ------------------------------------------------------------------------------------------
+def batchNorm2DTrainForward(in_: DenseMatrix, gamma: DenseMatrix, beta: DenseMatrix, emaMean: DenseMatrix, emaVar: DenseMatrix,
+                            eps: float, mu: float, ctx: HIPContext):
+    """BatchNorm2DTrainForward::apply (kernels/BatchNorm2DTrainForward.h:66-118). Returns (res, new_emaMean, new_emaVar,
+    mean, invVar); the four statistics are C x 1 (the reference returns C x C matrices with the first C values set)."""
+    dt = _same_dtype(in_, gamma, beta, emaMean, emaVar)
+    C = gamma.rows * gamma.cols
+    res = DenseMatrix(ctx, in_.rows, in_.cols, dt)
+    outs = [DenseMatrix(ctx, C, 1, dt) for _ in range(4)]
+    capi.check(_fn("dh_batchnorm_train_forward", dt)(ctx._h, res.ptr, outs[0].ptr, outs[1].ptr, outs[2].ptr, outs[3].ptr, in_.ptr,
+                                                     in_.rows, in_.cols, gamma.ptr, beta.ptr, emaMean.ptr, emaVar.ptr, C, eps, mu))
+    return (res, *outs)
+
+
+def batchNorm2DBackward(mean: DenseMatrix, invVar: DenseMatrix, in_: DenseMatrix, dout: DenseMatrix, gamma: DenseMatrix,
+                        eps: float, ctx: HIPContext):
+    """BatchNorm2DBackward::apply (kernels/BatchNorm2DBackward.h:63-120). Returns (dX, dGamma, dBeta)."""
+    dt = _same_dtype(in_, dout, gamma, mean, invVar)
+    C = gamma.rows * gamma.cols
+    dX, dG, dB = DenseMatrix(ctx, in_.rows, in_.cols, dt), DenseMatrix(ctx, C, 1, dt), DenseMatrix(ctx, C, 1, dt)
+    capi.check(_fn("dh_batchnorm_backward", dt)(ctx._h, dX.ptr, dG.ptr, dB.ptr, mean.ptr, invVar.ptr, in_.ptr, dout.ptr, in_.rows,
+                                                in_.cols, gamma.ptr, C, eps))
+    return dX, dG, dB
+
+
+def _poolBackward(name, res, input_, dOut, N, C, H, W, ph, pw, sh, sw, padh, padw, ctx):
+    dt = _same_dtype(input_, dOut, res)
+    if res is None:
+        res = DenseMatrix(ctx, N, C * H * W, dt)
+    capi.check(_fn(name, dt)(ctx._h, res.ptr, input_.ptr, dOut.ptr, N, C, H, W, ph, pw, sh, sw, padh, padw))
+    return res
+
+
+def maxPoolBackward(res, input_: DenseMatrix, dOut: DenseMatrix, batch_size, num_channels, img_h, img_w, pool_h, pool_w,
+                    stride_h, stride_w, pad_h, pad_w, ctx: HIPContext) -> DenseMatrix:
+    """MaxPoolBackward::apply (kernels/MaxPoolBackward.h:35-82), same argument order."""
+    return _poolBackward("dh_maxpool_backward", res, input_, dOut, batch_size, num_channels, img_h, img_w, pool_h, pool_w,
+                         stride_h, stride_w, pad_h, pad_w, ctx)
+
+
+def avgPoolBackward(res, input_: DenseMatrix, dOut: DenseMatrix, batch_size, num_channels, img_h, img_w, pool_h, pool_w,
+                    stride_h, stride_w, pad_h, pad_w, ctx: HIPContext) -> DenseMatrix:
+    """AvgPoolBackward::apply (kernels/AvgPoolBackward.h:35-77), same argument order."""
+    return _poolBackward("dh_avgpool_backward", res, input_, dOut, batch_size, num_channels, img_h, img_w, pool_h, pool_w,
+                         stride_h, stride_w, pad_h, pad_w, ctx)
+
+
+def conv2DBackwardData(filter_: DenseMatrix, output: DenseMatrix, stride_h, stride_w, pad_h, pad_w, input_batch_size,
+                       input_num_channels, input_h, input_w, filter_num_filters, filter_num_channels, filter_h, filter_w,
+                       data, ctx: HIPContext) -> DenseMatrix:
+    """Conv2DBackwardData::apply (kernels/Conv2DBackwardData.h:88-100), same argument order (`output` is the gradient
+    w.r.t. the convolution's output, `data` the result)."""
+    dt = _same_dtype(filter_, output, data)
+    if data is None:
+        data = DenseMatrix(ctx, input_batch_size, input_num_channels * input_h * input_w, dt)
+    capi.check(_fn("dh_conv2d_backward_data", dt)(ctx._h, data.ptr, filter_.ptr, output.ptr, input_batch_size, input_num_channels,
+                                                  input_h, input_w, filter_num_filters, filter_h, filter_w, stride_h, stride_w,
+                                                  pad_h, pad_w))
+    return data
+
+
+def conv2DBackwardFilter(dFilter, input_: DenseMatrix, output: DenseMatrix, stride_h, stride_w, pad_h, pad_w, input_batch_size,
+                         input_num_channels, input_h, input_w, filter_num_filters, filter_num_channels, filter_h, filter_w,
+                         ctx: HIPContext) -> DenseMatrix:
+    """Conv2DBackwardFilter::apply (kernels/Conv2DBackwardFilter.h:68-76), same argument order."""
+    dt = _same_dtype(input_, output, dFilter)
+    if dFilter is None:
+        dFilter = DenseMatrix(ctx, filter_num_filters, filter_num_channels * filter_h * filter_w, dt)
+    capi.check(_fn("dh_conv2d_backward_filter", dt)(ctx._h, dFilter.ptr, input_.ptr, output.ptr, input_batch_size,
+                                                    input_num_channels, input_h, input_w, filter_num_filters, filter_h, filter_w,
+                                                    stride_h, stride_w, pad_h, pad_w))
+    return dFilter

@@ -443,6 +443,74 @@ dh_status dh_transpose_si64(dh_ctx *ctx, int64_t *res, size_t ld_res, const int6
                             size_t cols, size_t ld);
 
 
+/* ------------------------------------------------------------------------------------ */
+/* DNN training kernels                                                                  */
+/* ------------------------------------------------------------------------------------ */
+/* Device counterparts of kernels the reference has on the CPU only. Images are rows: data is
+ * N x (C*H*W), per-channel parameters are vectors of `channels` values in device memory.
+ *
+ * BatchNorm2DTrainForward<DenseMatrix<VT>,DenseMatrix<VT>>::apply (kernels/BatchNorm2DTrainForward.h:66-118):
+ * per channel mean and (population) variance over all images and pixels; mean[c], inv_var[c] =
+ * 1 / sqrt(var + eps), new_ema_x[c] = (1 - mu) * ema_x[c] + mu * x, res = gamma * (in - mean) /
+ * sqrt(var + eps) + beta. (The reference allocates its four statistics results as C x C matrices and fills
+ * the first C values; here they are C values.) */
+dh_status dh_batchnorm_train_forward_f32(dh_ctx *ctx, float *res, float *new_ema_mean, float *new_ema_var,
+                                         float *mean, float *inv_var, const float *in, size_t rows, size_t cols,
+                                         const float *gamma, const float *beta, const float *ema_mean,
+                                         const float *ema_var, size_t channels, float eps, float mu);
+dh_status dh_batchnorm_train_forward_f64(dh_ctx *ctx, double *res, double *new_ema_mean, double *new_ema_var,
+                                         double *mean, double *inv_var, const double *in, size_t rows, size_t cols,
+                                         const double *gamma, const double *beta, const double *ema_mean,
+                                         const double *ema_var, size_t channels, double eps, double mu);
+
+/* BatchNorm2DBackward<...>::apply (kernels/BatchNorm2DBackward.h:63-120): dBeta = sum dout, dGamma =
+ * sum dout * (in - mean) * inv_var, dX as derived there; `mean` and `inv_var` are the results of the
+ * training forward pass. eps is accepted and unused, as in the reference. */
+dh_status dh_batchnorm_backward_f32(dh_ctx *ctx, float *dX, float *dGamma, float *dBeta, const float *mean,
+                                    const float *inv_var, const float *in, const float *dout, size_t rows,
+                                    size_t cols, const float *gamma, size_t channels, float eps);
+dh_status dh_batchnorm_backward_f64(dh_ctx *ctx, double *dX, double *dGamma, double *dBeta, const double *mean,
+                                    const double *inv_var, const double *in, const double *dout, size_t rows,
+                                    size_t cols, const double *gamma, size_t channels, double eps);
+
+/* MaxPoolBackward / AvgPoolBackward<...>::apply (kernels/MaxPoolBackward.h:35-82, AvgPoolBackward.h:35-77):
+ * res (N x C*H*W) = gradient w.r.t. the pooling input, dOut is N x (C*P*Q) with P and Q as in the forward
+ * kernels (P from stride_w, Q from stride_h). MAX sends a window's gradient to its first maximum in
+ * row-major order over the zero-padded image (what lands on the padding is dropped); AVG spreads
+ * dOut / (pool_h * pool_w) over the window. */
+dh_status dh_maxpool_backward_f32(dh_ctx *ctx, float *res, const float *input, const float *dOut, size_t N,
+                                  size_t C, size_t H, size_t W, size_t pool_h, size_t pool_w, size_t stride_h,
+                                  size_t stride_w, size_t pad_h, size_t pad_w);
+dh_status dh_maxpool_backward_f64(dh_ctx *ctx, double *res, const double *input, const double *dOut, size_t N,
+                                  size_t C, size_t H, size_t W, size_t pool_h, size_t pool_w, size_t stride_h,
+                                  size_t stride_w, size_t pad_h, size_t pad_w);
+dh_status dh_avgpool_backward_f32(dh_ctx *ctx, float *res, const float *input, const float *dOut, size_t N,
+                                  size_t C, size_t H, size_t W, size_t pool_h, size_t pool_w, size_t stride_h,
+                                  size_t stride_w, size_t pad_h, size_t pad_w);
+dh_status dh_avgpool_backward_f64(dh_ctx *ctx, double *res, const double *input, const double *dOut, size_t N,
+                                  size_t C, size_t H, size_t W, size_t pool_h, size_t pool_w, size_t stride_h,
+                                  size_t stride_w, size_t pad_h, size_t pad_w);
+
+/* Conv2DBackwardData<...>::apply (kernels/Conv2DBackwardData.h:88-158): dX (N x C*H*W) from the filter
+ * (F x C*Hf*Wf) and the output gradient dY (N x F*P*Q) - the adjoint of dh_conv2d_forward in its data
+ * argument. The reference's kernel is consistent only where the output extent equals the filter extent
+ * and pad_h == pad_w (its loops use the filter's extent for dY, :72-82,142); results coincide there.
+ * Conv2DBackwardFilter<...>::apply (kernels/Conv2DBackwardFilter.h:68-152): dW (F x C*Hf*Wf) from the
+ * input and dY - the adjoint in the filter argument. */
+dh_status dh_conv2d_backward_data_f32(dh_ctx *ctx, float *dX, const float *filter, const float *dY, size_t N,
+                                         size_t C, size_t H, size_t W, size_t F, size_t Hf, size_t Wf,
+                                         size_t stride_h, size_t stride_w, size_t pad_h, size_t pad_w);
+dh_status dh_conv2d_backward_data_f64(dh_ctx *ctx, double *dX, const double *filter, const double *dY, size_t N,
+                                         size_t C, size_t H, size_t W, size_t F, size_t Hf, size_t Wf,
+                                         size_t stride_h, size_t stride_w, size_t pad_h, size_t pad_w);
+dh_status dh_conv2d_backward_filter_f32(dh_ctx *ctx, float *dW, const float *input, const float *dY, size_t N,
+                                         size_t C, size_t H, size_t W, size_t F, size_t Hf, size_t Wf,
+                                         size_t stride_h, size_t stride_w, size_t pad_h, size_t pad_w);
+dh_status dh_conv2d_backward_filter_f64(dh_ctx *ctx, double *dW, const double *input, const double *dY, size_t N,
+                                         size_t C, size_t H, size_t W, size_t F, size_t Hf, size_t Wf,
+                                         size_t stride_h, size_t stride_w, size_t pad_h, size_t pad_w);
+
+
 
 /* ------------------------------------------------------------------------------------ */
 /* fused vectorized pipeline                                                             */

@@ -81,6 +81,38 @@ class OracleBackend:
         return mm + b  # 1 x N (or 1 x 1) bias broadcast over rows
 
 
+    # DNN training kernels
+    def batchnorm_train_forward(self, x, g, b, m, v, eps, mu):
+        st, *outs = orc.batchnorm_train_forward(x, g, b, m, v, eps, mu)
+        _st(st)
+        return outs
+
+    def batchnorm_backward(self, mean, inv_var, x, dout, gamma, eps):
+        st, *outs = orc.batchnorm_backward(mean, inv_var, x, dout, gamma)
+        _st(st)
+        return outs
+
+    def maxpool_backward(self, x, dout, *a):
+        st, r = orc.maxpool_backward(x, dout, *a)
+        _st(st)
+        return r
+
+    def avgpool_backward(self, x, dout, *a):
+        st, r = orc.avgpool_backward(x, dout, *a)
+        _st(st)
+        return r
+
+    def conv2d_backward_data(self, filt, dy, N, C, H, W, F, Hf, Wf, sh, sw, ph, pw):
+        st, r = orc.conv2d_backward_data(filt, dy, N, C, H, W, F, Hf, Wf, sh, sw, ph, pw)
+        _st(st)
+        return r
+
+    def conv2d_backward_filter(self, x, dy, N, C, H, W, F, Hf, Wf, sh, sw, ph, pw):
+        st, r = orc.conv2d_backward_filter(x, dy, N, C, H, W, F, Hf, Wf, sh, sw, ph, pw)
+        _st(st)
+        return r
+
+
 class HipBackend:
     name = "hip"
 
@@ -166,4 +198,28 @@ class HipBackend:
 
     def affine(self, x, w, b):
         return self._call(self.k.affineForward, None, self._d(x), self._d(w), self._d(b) if b is not None else None,
+                          self.ctx).to_numpy()
+
+    # DNN training kernels
+    def batchnorm_train_forward(self, x, g, b, m, v, eps, mu):
+        outs = self._call(self.k.batchNorm2DTrainForward, self._d(x), self._d(g), self._d(b), self._d(m), self._d(v), eps, mu, self.ctx)
+        return [o.to_numpy() for o in outs]
+
+    def batchnorm_backward(self, mean, inv_var, x, dout, gamma, eps):
+        outs = self._call(self.k.batchNorm2DBackward, self._d(mean), self._d(inv_var), self._d(x), self._d(dout), self._d(gamma), eps,
+                          self.ctx)
+        return [o.to_numpy() for o in outs]
+
+    def maxpool_backward(self, x, dout, *a):
+        return self._call(self.k.maxPoolBackward, None, self._d(x), self._d(dout), *a, self.ctx).to_numpy()
+
+    def avgpool_backward(self, x, dout, *a):
+        return self._call(self.k.avgPoolBackward, None, self._d(x), self._d(dout), *a, self.ctx).to_numpy()
+
+    def conv2d_backward_data(self, filt, dy, N, C, H, W, F, Hf, Wf, sh, sw, ph, pw):
+        return self._call(self.k.conv2DBackwardData, self._d(filt), self._d(dy), sh, sw, ph, pw, N, C, H, W, F, C, Hf, Wf, None,
+                          self.ctx).to_numpy()
+
+    def conv2d_backward_filter(self, x, dy, N, C, H, W, F, Hf, Wf, sh, sw, ph, pw):
+        return self._call(self.k.conv2DBackwardFilter, None, self._d(x), self._d(dy), sh, sw, ph, pw, N, C, H, W, F, C, Hf, Wf,
                           self.ctx).to_numpy()

@@ -282,6 +282,72 @@ template <typename VT> void run_all(DaphneContext *dctx) {
     }
 }
 
+// DNN training kernels with the reference's own vectors (DNNConv2DBackwardTest.cpp:23-95, DNNPoolingBackwardTest.cpp:25-110,
+// DNNBatchNorm2DBackwardTest.cpp:22-70, DNNBatchNorm2DForwardTest.cpp:51-90)
+template <typename VT> void run_training(DaphneContext *dctx) {
+    using DT = DenseMatrix<VT>;
+    auto G = [&](size_t rows, std::vector<VT> v) { return genGivenVals<DT>(rows, v, dctx); };
+    {
+        auto dy = G(1, {1, 2, 3, 4, 5, 6, 7, 8});
+        auto filter = G(2, {1, 0, 0, 2, 2, 0, 0, 3, 3, 0, 0, 4, 5, 0, 0, 6, 6, 0, 0, 7, 7, 0, 0, 8});
+        DT *dx = nullptr, *dw = nullptr;
+        HIP::Conv2DBackwardData<DT, DT>::apply(filter, dy, 2, 2, 1, 1, 1, 3, 3, 3, 2, 3, 2, 2, dx, dctx);
+        CHECK(equals(dx, {32, 0, 40, 0, 44, 0, 48, 0, 56, 38, 0, 48, 0, 56, 0, 58, 0, 68, 44, 0, 56, 0, 68, 0, 68, 0, 80}));
+        auto in = G(1, {1, 2, 3, 4, 5, 6, 7, 8, 9, 1, 2, 3, 4, 5, 6, 7, 8, 9, 1, 2, 3, 4, 5, 6, 7, 8, 9});
+        HIP::Conv2DBackwardFilter<DT, DT>::apply(dw, in, dy, 2, 2, 1, 1, 1, 3, 3, 3, 2, 3, 2, 2, dctx);
+        CHECK(equals(dw, {20, 36, 36, 64, 20, 36, 36, 64, 20, 36, 36, 64, 40, 76, 76, 144, 40, 76, 76, 144, 40, 76, 76, 144}));
+        for (auto *m : {dy, filter, dx, dw, in})
+            DataObjectFactory::destroy(m);
+    }
+    {
+        std::vector<VT> iv(54), dv;
+        for (int i = 0; i < 54; i++)
+            iv[i] = VT(i + 1);
+        for (int r = 0; r < 2; r++)
+            for (int i = 1; i <= 12; i++)
+                dv.push_back(VT(i));
+        auto in = G(2, iv), dout = G(2, dv);
+        DT *rmax = nullptr, *ravg = nullptr;
+        HIP::MaxPoolBackward<DT, DT>::apply(rmax, in, dout, 2, 3, 3, 3, 2, 2, 2, 2, 1, 1, dctx);
+        std::vector<VT> emax, eavg, one = {1, 0, 2, 0, 0, 0, 3, 0, 4, 5, 0, 6, 0, 0, 0, 7, 0, 8, 9, 0, 10, 0, 0, 0, 11, 0, 12};
+        std::vector<VT> onea = {0.25, 0.50, 0.50, 0.75, 1.00, 1.00, 0.75, 1.00, 1.00, 1.25, 1.50, 1.50, 1.75, 2.00,
+                                2.00, 1.75, 2.00, 2.00, 2.25, 2.50, 2.50, 2.75, 3.00, 3.00, 2.75, 3.00, 3.00};
+        for (int r = 0; r < 2; r++) {
+            emax.insert(emax.end(), one.begin(), one.end());
+            eavg.insert(eavg.end(), onea.begin(), onea.end());
+        }
+        CHECK(equals(rmax, emax));
+        HIP::AvgPoolBackward<DT, DT>::apply(ravg, in, dout, 2, 3, 3, 3, 2, 2, 2, 2, 1, 1, dctx);
+        CHECK(equals(ravg, eavg));
+        for (auto *m : {in, dout, rmax, ravg})
+            DataObjectFactory::destroy(m);
+    }
+    {
+        std::vector<VT> v;
+        for (int r = 0; r < 2; r++)
+            for (int i = 1; i <= 12; i++)
+                v.push_back(VT(i));
+        auto in = G(2, v), dout = G(2, v), gamma = G(3, {1, 1, 1}), mean = G(3, {2.5, 6.5, 10.5});
+        const VT ivv = VT(1 / std::sqrt(1.25f + 1e-5f));
+        auto invVar = G(3, {ivv, ivv, ivv});
+        DT *dX = nullptr, *dG = nullptr, *dB = nullptr;
+        HIP::BatchNorm2DBackward<DT, DT>::apply(dX, dG, dB, mean, invVar, in, dout, gamma, VT(1e-5), dctx);
+        CHECK(approx(dG, {8.9442, 8.9442, 8.9442}, 1e-3));
+        CHECK(approx(dB, {20, 52, 84}, 1e-4));
+        CHECK(std::fabs(double(dX->toHost()[0]) + 1.0733e-05) < 1e-5);
+        // training forward: statistics of the batch, output normalised per channel
+        DT *res = nullptr, *nm = nullptr, *nv = nullptr, *mn = nullptr, *iv2 = nullptr;
+        auto zeros = G(3, {0, 0, 0}), ones = G(3, {1, 1, 1});
+        HIP::BatchNorm2DTrainForward<DT, DT>::apply(res, nm, nv, mn, iv2, in, gamma, zeros, zeros, ones, VT(1e-5), VT(1), dctx);
+        CHECK(approx(mn, {2.5, 6.5, 10.5}, 1e-5));
+        CHECK(approx(nv, {1.25, 1.25, 1.25}, 1e-5));
+        CHECK(approx(iv2, {ivv, ivv, ivv}, 1e-5));
+        CHECK(std::fabs(double(res->toHost()[0]) - (1 - 2.5) * double(ivv)) < 1e-5);
+        for (auto *m : {in, dout, gamma, mean, invVar, dX, dG, dB, res, nm, nv, mn, iv2, zeros, ones})
+            DataObjectFactory::destroy(m);
+    }
+}
+
 // Integer instantiations (EwBinaryMatTest.cpp:34, EwBinaryObjScaTest.cpp:36 run with uint32_t; AggAllTest.cpp:32 with
 // int64_t among others): the reference's literals where they are integers, plus integer-only behaviour.
 template <typename VT> void run_integer_elementwise(DaphneContext *dctx) {
@@ -353,6 +419,8 @@ int main() {
     CHECK(HIPContext::get(dctx.get(), 0)->getMemBudget() > 0);
     run_all<float>(dctx.get());
     run_all<double>(dctx.get());
+    run_training<float>(dctx.get());
+    run_training<double>(dctx.get());
     run_integer_elementwise<int64_t>(dctx.get());
     run_integer_elementwise<uint64_t>(dctx.get());
     run_integer_elementwise<int32_t>(dctx.get());

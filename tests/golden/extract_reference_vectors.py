@@ -26,7 +26,7 @@ FILES = [
     "DNNBatchNorm2DForwardTest.cpp", "CUDA/MatMulTest.cpp", "CUDA/DNNAffineTest.cpp", "CUDA/BiasAddTest.cpp",
     "CUDA/DNNBatchNormTest.cpp", "CUDA/DNNConvolutionTest.cpp", "CUDA/DNNSoftmaxTest.cpp",
     "CUDA/DNNActivationTest.cpp", "CUDA/DNNPoolingTest.cpp", "TransposeTest.cpp", "ColBindTest.cpp",
-    "ExtractColTest.cpp",
+    "ExtractColTest.cpp", "DNNConv2DBackwardTest.cpp", "DNNPoolingBackwardTest.cpp", "DNNBatchNorm2DBackwardTest.cpp",
 ]
 
 NUM = re.compile(r"^[-+]?(\d+\.?\d*|\.\d+)([eE][-+]?\d+)?[fFlL]?$")

@@ -271,5 +271,34 @@ def run(backend, f, c, k, dt):
         if exp.size == 0:
             exp = exp.reshape(arg.shape[0], 0)
         _eq(backend.extract_col(arg, sel), exp)
+    elif fn == "checkConv2DBackwardData":
+        # DNNConv2DBackwardTest.cpp:23-27: apply(filter, in, 2, 2, 1, 1, 1, 3, 3, 3, 2, 3, 2, 2, res)
+        _eq(backend.conv2d_backward_data(M(args[1]), M(args[0]), 1, 3, 3, 3, 2, 2, 2, 2, 2, 1, 1), M(args[2]))
+    elif fn == "checkConv2DBackwardFilter":
+        # :53-57: apply(res, input, dOutput, 2, 2, 1, 1, 1, 3, 3, 3, 2, 3, 2, 2)
+        _eq(backend.conv2d_backward_filter(M(args[0]), M(args[1]), 1, 3, 3, 3, 2, 2, 2, 2, 2, 1, 1), M(args[2]))
+    elif fn in ("check_avg", "check_max") and file.endswith("DNNPoolingBackwardTest.cpp"):
+        # DNNPoolingBackwardTest.cpp:41-51: apply(res, in, dOut, 2, 3, 3, 3, 2, 2, 2, 2, 1, 1)
+        x, dout = matrix(mats["genInput"], dt), matrix(mats["genDOut"], dt)
+        f = backend.avgpool_backward if fn == "check_avg" else backend.maxpool_backward
+        _eq(f(x, dout, 2, 3, 3, 3, 2, 2, 2, 2, 1, 1), M(args[2]))
+    elif fn == "checkBatchNorm2DBackward":
+        # DNNBatchNorm2DBackwardTest.cpp:22-36; invVar is written there as 1 / sqrt(1.25f + 1e-5f)
+        x, dout, gamma, mean = M(args[0]), M(args[1]), M(args[2]), M(args[3])
+        inv_var = np.full(mean.shape, 1 / np.sqrt(np.float32(1.25) + np.float32(1e-5)), dtype=dt)
+        dX, dG, dB = backend.batchnorm_backward(mean, inv_var, x, dout, gamma, 1e-5)
+        _approx(dX, M(args[5]), 1e-5)
+        _approx(dG.reshape(-1, 1), M(args[6]).reshape(-1, 1), 1e-4)
+        _approx(dB.reshape(-1, 1), M(args[7]).reshape(-1, 1), 1e-5)
+    elif fn == "checkBatchNorm2DTrainForward":
+        # DNNBatchNorm2DForwardTest.cpp:51-64: epsilon 1e-5, mu 1
+        x = M(args[0])
+        res, nm, nv, mean, inv_var = backend.batchnorm_train_forward(x, M(args[1]), M(args[2]), M(args[3]), M(args[4]), 1e-5, 1.0)
+        _approx(res, M(args[5]), 1e-4)
+        # with mu = 1 the new moving averages are the batch statistics themselves
+        C = mean.size
+        per_c = x.reshape(x.shape[0], C, -1).transpose(1, 0, 2).reshape(C, -1).astype(np.float64)
+        _approx(nm.reshape(-1, 1), per_c.mean(axis=1).reshape(-1, 1).astype(dt), 1e-5)
+        _approx(nv.reshape(-1, 1), per_c.var(axis=1).reshape(-1, 1).astype(dt), 1e-4)
     else:
         raise Skip(f"{fn} is outside the dense float/double kernel set")

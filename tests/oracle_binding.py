@@ -226,3 +226,53 @@ def zscore_pipeline(X, threads=4, thr=64.0):
     st = lib().oracle_zscore_pipeline_f32(_p(X), sz(rows), sz(cols), C.c_int(threads), C.c_float(thr), _p(mu), _p(sd),
                                           _p(r), _p(s), _p(secs))
     return st, mu, sd, r, s[0], secs
+
+
+# -- DNN training kernels (oracle/dnn_training_cpu.cpp) ---------------------------------------
+def batchnorm_train_forward(x, gamma, beta, ema_mean, ema_var, eps, mu):
+    dt = x.dtype
+    C = gamma.size
+    res = np.empty_like(x)
+    outs = [np.empty((C, 1), dt) for _ in range(4)]  # new_ema_mean, new_ema_var, mean, inv_var
+    st = _f("batchnorm_train_forward", dt)(_p(res), _p(outs[0]), _p(outs[1]), _p(outs[2]), _p(outs[3]), _p(x), sz(x.shape[0]),
+                                           sz(x.shape[1]), _p(gamma), _p(beta), _p(ema_mean), _p(ema_var), sz(C),
+                                           _sc(dt, eps), _sc(dt, mu))
+    return st, res, outs[0], outs[1], outs[2], outs[3]
+
+
+def batchnorm_backward(mean, inv_var, x, dout, gamma):
+    dt = x.dtype
+    C = gamma.size
+    dX, dG, dB = np.empty_like(x), np.empty((C, 1), dt), np.empty((C, 1), dt)
+    st = _f("batchnorm_backward", dt)(_p(dX), _p(dG), _p(dB), _p(mean), _p(inv_var), _p(x), _p(dout), sz(x.shape[0]),
+                                      sz(x.shape[1]), _p(gamma), sz(C))
+    return st, dX, dG, dB
+
+
+def _pool_backward(name, x, dout, N, C, H, W, ph, pw, sh, sw, padh, padw):
+    res = np.empty((N, C * H * W), x.dtype)
+    st = _f(name, x.dtype)(_p(res), _p(x), _p(dout), sz(N), sz(C), sz(H), sz(W), sz(ph), sz(pw), sz(sh), sz(sw), sz(padh),
+                           sz(padw))
+    return st, res
+
+
+def maxpool_backward(x, dout, N, C, H, W, ph, pw, sh, sw, padh, padw):
+    return _pool_backward("maxpool_backward", x, dout, N, C, H, W, ph, pw, sh, sw, padh, padw)
+
+
+def avgpool_backward(x, dout, N, C, H, W, ph, pw, sh, sw, padh, padw):
+    return _pool_backward("avgpool_backward", x, dout, N, C, H, W, ph, pw, sh, sw, padh, padw)
+
+
+def conv2d_backward_data(filt, dy, N, C, H, W, F, Hf, Wf, sh, sw, padh, padw):
+    dX = np.empty((N, C * H * W), filt.dtype)
+    st = _f("conv2d_backward_data", filt.dtype)(_p(dX), _p(filt), _p(dy), sz(N), sz(C), sz(H), sz(W), sz(F), sz(Hf), sz(Wf),
+                                                sz(sh), sz(sw), sz(padh), sz(padw))
+    return st, dX
+
+
+def conv2d_backward_filter(x, dy, N, C, H, W, F, Hf, Wf, sh, sw, padh, padw):
+    dW = np.empty((F, C * Hf * Wf), x.dtype)
+    st = _f("conv2d_backward_filter", x.dtype)(_p(dW), _p(x), _p(dy), sz(N), sz(C), sz(H), sz(W), sz(F), sz(Hf), sz(Wf),
+                                               sz(sh), sz(sw), sz(padh), sz(padw))
+    return st, dW

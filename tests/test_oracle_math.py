@@ -327,3 +327,110 @@ def test_si64_aggregations_against_numpy():
     assert np.array_equal(orc.extract_col(x, np.array([[3], [0], [-1]]))[1], x[:, [3, 0, -1]])
     assert np.array_equal(orc.fill(-5, 3, 4, np.int64)[1], np.full((3, 4), -5, np.int64))
     assert np.array_equal(orc.fill(2 ** 63 + 1, 2, 2, np.uint64)[1], np.full((2, 2), 2 ** 63 + 1, np.uint64))
+
+
+# -- DNN training kernels: pinned by calculus and linear algebra, independent of the restated loops ----------
+def _conv_fwd(x, w, N, C, H, W, F, Hf, Wf, sh, sw, ph, pw):
+    st, out, P, Q = orc.conv2d(x, w, np.zeros((F, 1), x.dtype), N, C, H, W, Hf, Wf, sh, sw, ph, pw)
+    assert st == orc.ST_OK
+    return out, P, Q
+
+
+@pytest.mark.parametrize("case", [(2, 3, 7, 6, 4, 3, 3, 1, 1, 1, 1), (1, 2, 9, 8, 3, 2, 3, 2, 1, 0, 1), (3, 1, 5, 5, 2, 5, 5, 1, 1, 2, 2),
+                                  (2, 2, 8, 8, 2, 3, 2, 2, 3, 1, 0), (1, 3, 3, 3, 2, 2, 2, 2, 2, 1, 1)])
+def test_conv_backward_is_the_adjoint_of_the_forward_convolution(case):
+    """<conv(x, w), dy> = <x, backward_data(w, dy)> = <w, backward_filter(x, dy)>: the convolution is bilinear, so both
+    gradients are fixed by the forward kernel (itself pinned by the reference's vectors and brute force)."""
+    N, C, H, W, F, Hf, Wf, sh, sw, ph, pw = case
+    rng = np.random.default_rng(sum(case))
+    x = rng.standard_normal((N, C * H * W))
+    w = rng.standard_normal((F, C * Hf * Wf))
+    y, P, Q = _conv_fwd(x, w, *case)
+    dy = rng.standard_normal(y.shape)
+    st, dx = orc.conv2d_backward_data(w, dy, *case)
+    assert st == orc.ST_OK
+    st, dw = orc.conv2d_backward_filter(x, dy, *case)
+    assert st == orc.ST_OK
+    lhs = float((y * dy).sum())
+    assert abs(lhs - float((x * dx).sum())) <= 1e-10 * max(1.0, abs(lhs))
+    assert abs(lhs - float((w * dw).sum())) <= 1e-10 * max(1.0, abs(lhs))
+    # and each single gradient entry is the forward result of a unit impulse
+    e = np.zeros_like(x)
+    e[0, 5] = 1.0
+    ye, _, _ = _conv_fwd(e, w, *case)
+    assert abs(float((ye * dy).sum()) - dx[0, 5]) <= 1e-12 * max(1.0, abs(dx[0, 5]))
+
+
+@pytest.mark.parametrize("p", [(2, 3, 6, 6, 2, 2, 2, 2, 0, 0), (1, 2, 7, 5, 3, 3, 1, 1, 1, 1), (2, 1, 8, 8, 3, 2, 2, 2, 1, 0),
+                               (1, 1, 5, 5, 2, 2, 1, 1, 0, 0)])
+def test_pooling_backward_against_adjoint_and_brute_force(p):
+    N, C, H, W, ph, pw, sh, sw, padh, padw = p
+    rng = np.random.default_rng(sum(p))
+    x = rng.permutation(N * C * H * W).astype(np.float64).reshape(N, C * H * W) + 1.0  # distinct, positive: unique maxima
+    st, y, P, Q = orc.avgpool(x, *p)
+    assert st == orc.ST_OK
+    dy = rng.standard_normal(y.shape)
+    # average pooling is linear: its backward pass is the adjoint
+    st, dx = orc.avgpool_backward(x, dy, *p)
+    assert st == orc.ST_OK
+    assert abs(float((y * dy).sum()) - float((x * dx).sum())) <= 1e-10 * max(1.0, abs(float((y * dy).sum())))
+    # max pooling: every window sends its gradient to the position of its maximum (brute force on the padded image)
+    st, dxm = orc.maxpool_backward(x, dy, *p)
+    assert st == orc.ST_OK
+    want = np.zeros((N, C, H + 2 * padh, W + 2 * padw))
+    xp = np.zeros_like(want)
+    xp[:, :, padh:padh + H, padw:padw + W] = x.reshape(N, C, H, W)
+    d4 = dy.reshape(N, C, P, Q)
+    for n in range(N):
+        for c in range(C):
+            for a in range(P):
+                for b in range(Q):
+                    win = xp[n, c, a * sh:a * sh + ph, b * sw:b * sw + pw]
+                    if win.shape != (ph, pw):
+                        continue
+                    i, j = np.unravel_index(np.argmax(win), win.shape)  # first maximum in row-major order
+                    want[n, c, a * sh + i, b * sw + j] += d4[n, c, a, b]
+    np.testing.assert_allclose(dxm.reshape(N, C, H, W), want[:, :, padh:padh + H, padw:padw + W], rtol=0, atol=1e-12)
+
+
+def test_batchnorm_training_against_numpy_and_finite_differences():
+    rng = np.random.default_rng(8)
+    N, C, HW = 5, 3, 7
+    x = rng.standard_normal((N, C * HW)) * 2 + 1
+    gamma, beta = rng.random((C, 1)) + 0.5, rng.standard_normal((C, 1))
+    em, ev = rng.standard_normal((C, 1)), rng.random((C, 1)) + 0.5
+    eps, mu = 1e-5, 0.3
+    st, res, nm, nv, mean, iv = orc.batchnorm_train_forward(x, gamma, beta, em, ev, eps, mu)
+    assert st == orc.ST_OK
+    xc = x.reshape(N, C, HW).transpose(1, 0, 2).reshape(C, -1)
+    m, v = xc.mean(axis=1, keepdims=True), xc.var(axis=1, keepdims=True)
+    np.testing.assert_allclose(mean, m, rtol=1e-12)
+    np.testing.assert_allclose(iv, 1 / np.sqrt(v + eps), rtol=1e-12)
+    np.testing.assert_allclose(nm, (1 - mu) * em + mu * m, rtol=1e-12)
+    np.testing.assert_allclose(nv, (1 - mu) * ev + mu * v, rtol=1e-12)
+    want = (gamma * (xc - m) / np.sqrt(v + eps) + beta).reshape(C, N, HW).transpose(1, 0, 2).reshape(N, C * HW)
+    np.testing.assert_allclose(res, want, rtol=1e-11, atol=1e-12)
+
+    # backward: gradient of L = <dout, BN(x)> by central differences, through the forward kernel itself
+    dout = rng.standard_normal(x.shape)
+    st, dX, dG, dB = orc.batchnorm_backward(mean, iv, x, dout, gamma)
+    assert st == orc.ST_OK
+
+    def loss(xx, gg, bb):
+        return float((orc.batchnorm_train_forward(xx, gg, bb, em, ev, eps, mu)[1] * dout).sum())
+
+    h = 1e-6
+    for (i, j) in ((0, 0), (2, 9), (4, 20), (1, 13)):
+        xp, xm = x.copy(), x.copy()
+        xp[i, j] += h
+        xm[i, j] -= h
+        assert abs((loss(xp, gamma, beta) - loss(xm, gamma, beta)) / (2 * h) - dX[i, j]) <= 1e-6 * max(1.0, abs(dX[i, j]))
+    for c in range(C):
+        gp, gm = gamma.copy(), gamma.copy()
+        gp[c] += h
+        gm[c] -= h
+        assert abs((loss(x, gp, beta) - loss(x, gm, beta)) / (2 * h) - dG[c, 0]) <= 1e-6 * max(1.0, abs(dG[c, 0]))
+        bp, bm = beta.copy(), beta.copy()
+        bp[c] += h
+        bm[c] -= h
+        assert abs((loss(x, gamma, bp) - loss(x, gamma, bm)) / (2 * h) - dB[c, 0]) <= 1e-6 * max(1.0, abs(dB[c, 0]))
