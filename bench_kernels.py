@@ -195,7 +195,7 @@ def main() -> int:
             emit("softmax 10 classes", dt, "1000000x10", timed(lambda: K.softmax(sm, big, ctx)), 2 * 10_000_000 * sz)
             for m in (x2, w2, b2, o2, one, pl, w3, b3, h3, big, sm):
                 m.destroy()
-        # --- DNN training kernels (first versions: gathers and plain per-channel reductions, no matrix cores) ------
+        # --- DNN training kernels ---------------------------------------------------------------------------------
         if want("train"):
             N = 4096 if dt == "f32" else 2048
             el = N * 64 * 196
@@ -204,9 +204,9 @@ def main() -> int:
             gam = DM.from_torch(ctx, torch.rand(64, 1, device="cuda", dtype=tdt, generator=gen) + 0.5)
             zer = DM.from_torch(ctx, torch.zeros(64, 1, device="cuda", dtype=tdt))
             res_bn = K.batchNorm2DTrainForward(x, gam, zer, zer, gam, 1e-5, 0.1, ctx)
-            emit("batchNorm2DTrainForward 64 channels (three passes over the input)", dt, f"{N}x{64 * 196}",
+            emit("batchNorm2DTrainForward 64 channels (statistics pass + normalisation pass)", dt, f"{N}x{64 * 196}",
                  timed(lambda: K.batchNorm2DTrainForward(x, gam, zer, zer, gam, 1e-5, 0.1, ctx)), 2 * el * sz)
-            emit("batchNorm2DBackward 64 channels (two passes over input and gradient)", dt, f"{N}x{64 * 196}",
+            emit("batchNorm2DBackward 64 channels (sums pass + gradient pass)", dt, f"{N}x{64 * 196}",
                  timed(lambda: K.batchNorm2DBackward(res_bn[3], res_bn[4], x, dy, gam, 1e-5, ctx)), 3 * el * sz)
             dpool = DM.from_torch(ctx, torch.randn(N, 64 * 49, device="cuda", dtype=tdt, generator=gen))
             dxp = DM(ctx, N, 64 * 196, ndt)
@@ -214,15 +214,15 @@ def main() -> int:
                  timed(lambda: K.maxPoolBackward(dxp, x, dpool, N, 64, 14, 14, 2, 2, 2, 2, 0, 0, ctx)), 2.25 * el * sz)
             emit("avgPoolBackward 2x2/2 on 14x14", dt, f"{N}x{64 * 196}",
                  timed(lambda: K.avgPoolBackward(dxp, x, dpool, N, 64, 14, 14, 2, 2, 2, 2, 0, 0, ctx)), 1.25 * el * sz)
-            Nc = N // 8  # the convolution gradients are plain-ALU kernels: a smaller batch keeps the run short
+            Nc = N
             xc = DM.from_torch(ctx, torch.rand(Nc, 32 * 196, device="cuda", dtype=tdt, generator=gen))
             wc = DM.from_torch(ctx, torch.randn(64, 800, device="cuda", dtype=tdt, generator=gen) * 0.05)
             dyc = DM.from_torch(ctx, torch.randn(Nc, 64 * 196, device="cuda", dtype=tdt, generator=gen))
             dxc, dwc = DM(ctx, Nc, 32 * 196, ndt), DM(ctx, 64, 800, ndt)
             fl = 2.0 * Nc * 64 * 196 * 800
-            emit("conv2DBackwardData 64->32 ch, 14x14, 5x5 pad 2 (gather, no matrix cores)", dt, f"batch {Nc}",
+            emit("conv2DBackwardData 64->32 ch, 14x14, 5x5 pad 2 (frame + rotated filters + forward convolution)", dt, f"batch {Nc}",
                  timed(lambda: K.conv2DBackwardData(wc, dyc, 1, 1, 2, 2, Nc, 32, 14, 14, 64, 32, 5, 5, dxc, ctx)), flops=fl)
-            emit("conv2DBackwardFilter 32->64 ch, 14x14, 5x5 pad 2 (per-filter-plane reduction, no matrix cores)", dt, f"batch {Nc}",
+            emit("conv2DBackwardFilter 32->64 ch, 14x14, 5x5 pad 2 (patch matrix + split-K GEMM)", dt, f"batch {Nc}",
                  timed(lambda: K.conv2DBackwardFilter(dwc, xc, dyc, 1, 1, 2, 2, Nc, 32, 14, 14, 64, 32, 5, 5, ctx)), flops=fl)
             for m in (x, dy, gam, zer, dpool, dxp, xc, wc, dyc, dxc, dwc, *res_bn):
                 m.destroy()

@@ -28,15 +28,16 @@ constexpr int THREADS = 256;
 // per-channel reductions
 // ---------------------------------------------------------------------------------------
 // MODE 0: sum x          MODE 1: sum (x - mean[c])^2          MODE 2: sum dy, sum dy*(x - mean[c]), sum (x - mean[c])
+// MODE 3: sum (x - s), sum (x - s)^2 with s = the channel's first value: mean and variance from one pass
 template <typename T, int MODE>
 __global__ __launch_bounds__(THREADS) void chan_stage1(const T *x, const T *dy, const T *mean, size_t N, size_t C, size_t HW,
                                                        size_t imgs_per_slice, double *partials /* [C][S][3] */) {
-    constexpr int K = MODE == 2 ? 3 : 1;
+    constexpr int K = MODE == 2 ? 3 : (MODE == 3 ? 2 : 1);
     __shared__ double lds[K][THREADS / DH_WAVE];
     const size_t c = blockIdx.x, s = blockIdx.y;
     const size_t n0 = s * imgs_per_slice, n1 = (n0 + imgs_per_slice < N) ? n0 + imgs_per_slice : N;
     const size_t CHW = C * HW;
-    const double mu = MODE >= 1 ? static_cast<double>(mean[c]) : 0.0;
+    const double mu = MODE == 3 ? static_cast<double>(x[c * HW]) : (MODE >= 1 ? static_cast<double>(mean[c]) : 0.0);
     double a0 = 0.0, a1 = 0.0, a2 = 0.0;
     const size_t items = (n1 > n0 ? n1 - n0 : 0) * HW;
     for (size_t i = threadIdx.x; i < items; i += THREADS) {
@@ -47,6 +48,9 @@ __global__ __launch_bounds__(THREADS) void chan_stage1(const T *x, const T *dy, 
             a0 += v;
         } else if constexpr (MODE == 1) {
             a0 += (v - mu) * (v - mu);
+        } else if constexpr (MODE == 3) {
+            a0 += v - mu;
+            a1 += (v - mu) * (v - mu);
         } else {
             const double g = static_cast<double>(dy[off]);
             a0 += g;
@@ -78,16 +82,19 @@ __global__ __launch_bounds__(THREADS) void chan_stage1(const T *x, const T *dy, 
 // STEP 0: mean[c] = sum / m.
 // STEP 1: var = sum / m; inv_var, moving averages; coef[c] = sqrt(var + eps) for the normalisation pass.
 // STEP 2: dBeta, dGamma and coef[c][0..1] = dVar * 2/m, dMean / m for the gradient pass.
+// STEP 3: STEP 0 and STEP 1 from the shifted sums of MODE 3 (x0 = the input, whose first value per channel is the shift).
 template <typename T, int STEP>
 __global__ void chan_stage2(const double *partials, size_t C, size_t S, double m, T *mean, T *inv_var, T *new_ema_mean,
                             T *new_ema_var, const T *ema_mean, const T *ema_var, T eps, T mu_, const T *gamma, T *dGamma,
-                            T *dBeta, T *coef) {
+                            T *dBeta, T *coef, const T *x0 = nullptr, size_t HW = 0) {
     const size_t c = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (c >= C)
         return;
     double s0 = 0.0, s1 = 0.0, s2 = 0.0;
     for (size_t s = 0; s < S; s++) {
         s0 += partials[(c * S + s) * 3 + 0];
+        if (STEP == 3)
+            s1 += partials[(c * S + s) * 3 + 1];
         if (STEP == 2) {
             s1 += partials[(c * S + s) * 3 + 1];
             s2 += partials[(c * S + s) * 3 + 2];
@@ -95,8 +102,18 @@ __global__ void chan_stage2(const double *partials, size_t C, size_t S, double m
     }
     if constexpr (STEP == 0) {
         mean[c] = static_cast<T>(s0 / m);
-    } else if constexpr (STEP == 1) {
-        const T var = static_cast<T>(s0 / m), mn = mean[c];
+    } else if constexpr (STEP == 1 || STEP == 3) {
+        T var, mn;
+        if constexpr (STEP == 3) {
+            const double d = s0 / m; // mean - shift
+            mn = static_cast<T>(static_cast<double>(x0[c * HW]) + d);
+            const double v = s1 / m - d * d;
+            var = static_cast<T>(v > 0.0 ? v : 0.0);
+            mean[c] = mn;
+        } else {
+            var = static_cast<T>(s0 / m);
+            mn = mean[c];
+        }
         const T sd = sizeof(T) == 4 ? static_cast<T>(sqrtf(static_cast<float>(var + eps))) : static_cast<T>(sqrt(static_cast<double>(var + eps)));
         inv_var[c] = T(1) / sd;
         new_ema_mean[c] = (T(1) - mu_) * ema_mean[c] + mu_ * mn;
@@ -207,14 +224,11 @@ dh_status batchnorm_train_forward(dh_ctx *ctx, T *res, T *new_ema_mean, T *new_e
     T *coef = reinterpret_cast<T *>(partials + C * p.S * 3);
     const double m = static_cast<double>(rows) * static_cast<double>(HW);
     const dim3 g1(static_cast<unsigned>(C), static_cast<unsigned>(p.S)), g2(static_cast<unsigned>(dh_ceil_div(C, 64)));
-    hipLaunchKernelGGL((chan_stage1<T, 0>), g1, dim3(THREADS), 0, ctx->stream, in, nullptr, nullptr, rows, C, HW,
-                       p.imgs_per_slice, partials);
-    hipLaunchKernelGGL((chan_stage2<T, 0>), g2, dim3(64), 0, ctx->stream, partials, C, p.S, m, mean, inv_var, new_ema_mean,
-                       new_ema_var, ema_mean, ema_var, eps, mu, gamma, nullptr, nullptr, coef);
-    hipLaunchKernelGGL((chan_stage1<T, 1>), g1, dim3(THREADS), 0, ctx->stream, in, nullptr, mean, rows, C, HW, p.imgs_per_slice,
+    // mean and variance from ONE pass: sums of (x - s) and (x - s)^2 around the channel's first value, in double
+    hipLaunchKernelGGL((chan_stage1<T, 3>), g1, dim3(THREADS), 0, ctx->stream, in, nullptr, nullptr, rows, C, HW, p.imgs_per_slice,
                        partials);
-    hipLaunchKernelGGL((chan_stage2<T, 1>), g2, dim3(64), 0, ctx->stream, partials, C, p.S, m, mean, inv_var, new_ema_mean,
-                       new_ema_var, ema_mean, ema_var, eps, mu, gamma, nullptr, nullptr, coef);
+    hipLaunchKernelGGL((chan_stage2<T, 3>), g2, dim3(64), 0, ctx->stream, partials, C, p.S, m, mean, inv_var, new_ema_mean,
+                       new_ema_var, ema_mean, ema_var, eps, mu, gamma, nullptr, nullptr, coef, in, HW);
     launch_apply<T, true>(ctx, res, in, nullptr, rows * C, C, HW, mean, gamma, beta, inv_var, coef);
     DH_CHECK_LAUNCH();
     return DH_OK;
@@ -307,6 +321,71 @@ __global__ __launch_bounds__(THREADS) void pool_backward_kernel(T *res, const T 
     res[idx] = acc;
 }
 
+// 2x2 windows, stride 2, no padding, even image height, width a multiple of the vector: every pixel belongs to
+// exactly one window. A thread takes VI columns of an image-row pair: two vector loads of the input (MAX only), VI/2
+// gradients, two vector stores. VI is the 16-byte vector, or half of it for floats when the width is only even.
+template <typename T, int VI, bool AVG>
+__global__ __launch_bounds__(THREADS) void pool2x2_backward_kernel(T *res, const T *input, const T *dOut, unsigned H, unsigned W, size_t total) {
+#pragma clang fp contract(off)
+    typedef T vec_t __attribute__((ext_vector_type(VI)));
+    const size_t idx = static_cast<size_t>(blockIdx.x) * THREADS + threadIdx.x;
+    if (idx >= total)
+        return;
+    const unsigned wv = W / VI, P = H / 2, Q = W / 2;
+    const unsigned j = static_cast<unsigned>(idx % wv);
+    const size_t pr = idx / wv; // (plane, p)
+    const size_t plane = pr / P;
+    const unsigned p = static_cast<unsigned>(pr % P);
+    const size_t in0 = (plane * H + 2 * p) * W + static_cast<size_t>(j) * VI;
+    const T *dy = dOut + (plane * P + p) * Q + static_cast<size_t>(j) * (VI / 2);
+    T o0[VI], o1[VI];
+    if constexpr (AVG) {
+#pragma unroll
+        for (int k = 0; k < VI / 2; k++) {
+            const T v = (T(1) / T(4)) * dy[k];
+            o0[2 * k] = o0[2 * k + 1] = o1[2 * k] = o1[2 * k + 1] = v;
+        }
+    } else {
+        const vec_t v0 = __builtin_nontemporal_load(reinterpret_cast<const vec_t *>(input + in0));
+        const vec_t v1 = __builtin_nontemporal_load(reinterpret_cast<const vec_t *>(input + in0 + W));
+        T x0[VI], x1[VI];
+#pragma unroll
+        for (int e = 0; e < VI; e++) {
+            x0[e] = v0[e];
+            x1[e] = v1[e];
+        }
+#pragma unroll
+        for (int k = 0; k < VI / 2; k++) {
+            // first maximum in row-major order with a strict comparison (MaxPoolBackward.h:62-69)
+            int best = 0;
+            T m = x0[2 * k];
+            if (x0[2 * k + 1] > m) {
+                m = x0[2 * k + 1];
+                best = 1;
+            }
+            if (x1[2 * k] > m) {
+                m = x1[2 * k];
+                best = 2;
+            }
+            if (x1[2 * k + 1] > m)
+                best = 3;
+            const T gv = dy[k];
+            o0[2 * k] = best == 0 ? gv : T(0);
+            o0[2 * k + 1] = best == 1 ? gv : T(0);
+            o1[2 * k] = best == 2 ? gv : T(0);
+            o1[2 * k + 1] = best == 3 ? gv : T(0);
+        }
+    }
+    vec_t w0, w1;
+#pragma unroll
+    for (int e = 0; e < VI; e++) {
+        w0[e] = o0[e];
+        w1[e] = o1[e];
+    }
+    __builtin_nontemporal_store(w0, reinterpret_cast<vec_t *>(res + in0));
+    __builtin_nontemporal_store(w1, reinterpret_cast<vec_t *>(res + in0 + W));
+}
+
 template <typename T, bool AVG>
 dh_status pool_backward(dh_ctx *ctx, T *res, const T *input, const T *dOut, size_t N, size_t C, size_t H, size_t W, size_t ph,
                         size_t pw, size_t sh, size_t sw, size_t padh, size_t padw) {
@@ -322,6 +401,23 @@ dh_status pool_backward(dh_ctx *ctx, T *res, const T *input, const T *dOut, size
     g.total = N * C * H * W;
     if (g.total == 0)
         return DH_OK;
+    constexpr int VFULL = dh_vec<T>::N;
+    if (ph == 2 && pw == 2 && sh == 2 && sw == 2 && padh == 0 && padw == 0 && H % 2 == 0 && W % 2 == 0 && dh_aligned(res, 16) &&
+        dh_aligned(input, 16)) {
+        const int vi = W % VFULL == 0 ? VFULL : 2;
+        const size_t total = N * C * (H / 2) * (W / vi);
+        if (dh_ceil_div(total, THREADS) < (size_t(1) << 31)) {
+            const dim3 grid(static_cast<unsigned>(dh_ceil_div(total, THREADS)));
+            if (vi == VFULL)
+                hipLaunchKernelGGL((pool2x2_backward_kernel<T, VFULL, AVG>), grid, dim3(THREADS), 0, ctx->stream, res, input, dOut,
+                                   static_cast<unsigned>(H), static_cast<unsigned>(W), total);
+            else
+                hipLaunchKernelGGL((pool2x2_backward_kernel<T, 2, AVG>), grid, dim3(THREADS), 0, ctx->stream, res, input, dOut,
+                                   static_cast<unsigned>(H), static_cast<unsigned>(W), total);
+            DH_CHECK_LAUNCH();
+            return DH_OK;
+        }
+    }
     const size_t blocks = dh_ceil_div(g.total, THREADS);
     if (blocks >= (size_t(1) << 31))
         return dh_fail(DH_ERR_RUNTIME, "Pooling backward - too many elements for one launch");
@@ -431,9 +527,169 @@ static inline dh_status conv_bwd_args(ConvBwdArgs *g, size_t N, size_t C, size_t
     return DH_OK;
 }
 
+// ---------------------------------------------------------------------------------------
+// convolution gradients on the matrix cores
+// ---------------------------------------------------------------------------------------
+// Both gradients are contractions, so they are handed to the kernels that already run them on the matrix cores:
+//  * data:   dX = forward convolution (stride 1, no padding) of the output gradient - dilated by the stride and
+//            placed in a zero frame of (H + Hf - 1) x (W + Wf - 1) - with the filters rotated by 180 degrees and
+//            their filter / channel axes exchanged;
+//  * filter: dW (F x C*Hf*Wf) = dY as an F x (N*P*Q) matrix times the patch matrix (N*P*Q) x (C*Hf*Wf) of the input.
+// The sums then run in the order of those kernels (results agree with the gather kernels above to rounding). The
+// temporaries come from the context's block cache; shapes whose temporaries would be very large, or padding beyond
+// the filter extent, take the gather kernels.
+static inline dh_status conv_fwd(dh_ctx *ctx, float *res, size_t *rh, size_t *rw, const float *data, const float *filter, size_t fr,
+                                 size_t fc, size_t N, size_t C, size_t H, size_t W, size_t Hf, size_t Wf) {
+    return dh_conv2d_forward_f32(ctx, res, rh, rw, data, filter, fr, fc, nullptr, N, C, H, W, Hf, Wf, 1, 1, 0, 0);
+}
+static inline dh_status conv_fwd(dh_ctx *ctx, double *res, size_t *rh, size_t *rw, const double *data, const double *filter, size_t fr,
+                                 size_t fc, size_t N, size_t C, size_t H, size_t W, size_t Hf, size_t Wf) {
+    return dh_conv2d_forward_f64(ctx, res, rh, rw, data, filter, fr, fc, nullptr, N, C, H, W, Hf, Wf, 1, 1, 0, 0);
+}
+static inline dh_status mat_mul(dh_ctx *ctx, float *res, size_t ldr, const float *a, size_t ar, size_t ac, size_t lda, const float *b,
+                                size_t br, size_t bc, size_t ldb) {
+    return dh_matmul_f32(ctx, res, ldr, a, ar, ac, lda, b, br, bc, ldb, 0, 0);
+}
+static inline dh_status mat_mul(dh_ctx *ctx, double *res, size_t ldr, const double *a, size_t ar, size_t ac, size_t lda, const double *b,
+                                size_t br, size_t bc, size_t ldb) {
+    return dh_matmul_f64(ctx, res, ldr, a, ar, ac, lda, b, br, bc, ldb, 0, 0);
+}
+
+// frame[n][f][a][b], a < H + Hf - 1, b < W + Wf - 1: dY[n][f][p][q] at (p*sh + Hf-1-padh, q*sw + Wf-1-padw), else 0
+template <typename T> __global__ __launch_bounds__(THREADS) void dilate_frame_kernel(T *frame, const T *dY, ConvBwdArgs g, size_t total) {
+    const size_t idx = static_cast<size_t>(blockIdx.x) * THREADS + threadIdx.x;
+    if (idx >= total)
+        return;
+    const unsigned FH = g.H + g.Hf - 1, FW = g.W + g.Wf - 1;
+    const size_t plane = idx / (static_cast<size_t>(FH) * FW); // (n, f)
+    const unsigned ab = static_cast<unsigned>(idx % (static_cast<size_t>(FH) * FW)), a = ab / FW, b = ab % FW;
+    const unsigned oh = g.Hf - 1 - g.padh, ow = g.Wf - 1 - g.padw;
+    T v = T(0);
+    if (a >= oh && b >= ow && (a - oh) % g.sh == 0 && (b - ow) % g.sw == 0) {
+        const unsigned p = (a - oh) / g.sh, q = (b - ow) / g.sw;
+        if (p < g.P && q < g.Q)
+            v = dY[plane * (static_cast<size_t>(g.P) * g.Q) + p * g.Q + q];
+    }
+    frame[idx] = v;
+}
+// wr[c][(f, r, s)] = w[f][(c, Hf-1-r, Wf-1-s)]
+template <typename T> __global__ __launch_bounds__(THREADS) void rotate_filter_kernel(T *wr, const T *w, ConvBwdArgs g) {
+    const unsigned taps = g.Hf * g.Wf;
+    const size_t total = static_cast<size_t>(g.C) * g.F * taps;
+    const size_t idx = static_cast<size_t>(blockIdx.x) * THREADS + threadIdx.x;
+    if (idx >= total)
+        return;
+    const unsigned t = static_cast<unsigned>(idx % taps), f = static_cast<unsigned>((idx / taps) % g.F), c = static_cast<unsigned>(idx / (static_cast<size_t>(taps) * g.F));
+    wr[idx] = w[(static_cast<size_t>(f) * g.C + c) * taps + (taps - 1 - t)];
+}
+// patch[(n, p, q)][(c, r, s)] = Xpad[n][c][p*sh + r][q*sw + s]; a thread writes VEC consecutive (c, r, s) of one row
+template <typename T, int VEC> __global__ __launch_bounds__(THREADS) void im2col_kernel(T *patch, const T *input, ConvBwdArgs g, size_t total_vecs) {
+    const size_t idx = static_cast<size_t>(blockIdx.x) * THREADS + threadIdx.x;
+    if (idx >= total_vecs)
+        return;
+    const unsigned taps = g.Hf * g.Wf, Kp = g.C * taps, PQ = g.P * g.Q, kvecs = Kp / VEC;
+    const size_t row = idx / kvecs;
+    const unsigned k0 = static_cast<unsigned>(idx % kvecs) * VEC;
+    const unsigned n = static_cast<unsigned>(row / PQ), pq = static_cast<unsigned>(row % PQ), p = pq / g.Q, q = pq % g.Q;
+    const T *img = input + static_cast<size_t>(n) * g.C * g.H * g.W;
+    unsigned c = k0 / taps, t = k0 % taps, r = t / g.Wf, s_ = t % g.Wf;
+    T v[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; e++) {
+        const unsigned hh = p * g.sh + r, ww = q * g.sw + s_;
+        v[e] = (hh >= g.padh && ww >= g.padw && hh - g.padh < g.H && ww - g.padw < g.W)
+                   ? img[(static_cast<size_t>(c) * g.H + (hh - g.padh)) * g.W + (ww - g.padw)]
+                   : T(0);
+        if (++s_ == g.Wf) { // next (c, r, s) without divisions
+            s_ = 0;
+            if (++r == g.Hf) {
+                r = 0;
+                c++;
+            }
+        }
+    }
+    dh_store_vec<T, VEC>(patch + row * Kp + k0, v);
+}
+// a[f][(n, pq)] = dY[n][f][pq]
+template <typename T> __global__ __launch_bounds__(THREADS) void dy_rows_kernel(T *a, const T *dY, ConvBwdArgs g, size_t total) {
+    const size_t idx = static_cast<size_t>(blockIdx.x) * THREADS + threadIdx.x;
+    if (idx >= total)
+        return;
+    const unsigned PQ = g.P * g.Q;
+    const size_t L = static_cast<size_t>(g.N) * PQ;
+    const unsigned f = static_cast<unsigned>(idx / L);
+    const size_t l = idx % L;
+    const unsigned n = static_cast<unsigned>(l / PQ), pq = static_cast<unsigned>(l % PQ);
+    a[idx] = dY[(static_cast<size_t>(n) * g.F + f) * PQ + pq];
+}
+
+constexpr size_t TRAIN_TEMP_LIMIT = size_t(24) << 30; // bytes of temporaries beyond which the gather kernels are used
+
+static inline unsigned blocks_for(size_t total) { return static_cast<unsigned>(dh_ceil_div(total, static_cast<size_t>(THREADS))); }
+
+template <typename T> static bool conv_backward_data_mfma(dh_ctx *ctx, T *dX, const T *filter, const T *dY, const ConvBwdArgs &g, dh_status *st) {
+    if (g.padh > g.Hf - 1 || g.padw > g.Wf - 1)
+        return false;
+    const size_t FH = g.H + g.Hf - 1, FW = g.W + g.Wf - 1;
+    const size_t frame_elems = static_cast<size_t>(g.N) * g.F * FH * FW, wr_elems = static_cast<size_t>(g.C) * g.F * g.Hf * g.Wf;
+    // too little work to pay for the extra passes, or too large temporaries
+    if (static_cast<size_t>(g.N) * g.C * g.H * g.W < (size_t(1) << 16) || frame_elems * sizeof(T) > TRAIN_TEMP_LIMIT ||
+        dh_ceil_div(frame_elems, static_cast<size_t>(THREADS)) >= (size_t(1) << 31))
+        return false;
+    void *frame = nullptr, *wr = nullptr;
+    *st = dh_malloc(ctx, frame_elems * sizeof(T), 0, &frame);
+    if (*st != DH_OK)
+        return true;
+    *st = dh_malloc(ctx, wr_elems * sizeof(T), 0, &wr);
+    if (*st != DH_OK) {
+        dh_free(ctx, frame);
+        return true;
+    }
+    hipLaunchKernelGGL((dilate_frame_kernel<T>), dim3(blocks_for(frame_elems)), dim3(THREADS), 0, ctx->stream, static_cast<T *>(frame), dY, g,
+                       frame_elems);
+    hipLaunchKernelGGL((rotate_filter_kernel<T>), dim3(blocks_for(wr_elems)), dim3(THREADS), 0, ctx->stream, static_cast<T *>(wr), filter, g);
+    size_t rh = 0, rw = 0;
+    *st = conv_fwd(ctx, dX, &rh, &rw, static_cast<const T *>(frame), static_cast<const T *>(wr), g.C, static_cast<size_t>(g.F) * g.Hf * g.Wf,
+                   g.N, g.F, FH, FW, g.Hf, g.Wf);
+    // blocks go back to the cache; reuse is ordered by the context's stream
+    dh_free(ctx, frame);
+    dh_free(ctx, wr);
+    if (*st == DH_OK && (rh != g.H || rw != g.W))
+        *st = dh_fail(DH_ERR_RUNTIME, "Conv2D backward - internal extent mismatch (%zu x %zu for %u x %u)", rh, rw, g.H, g.W);
+    return true;
+}
+
+template <typename T> static bool conv_backward_filter_mfma(dh_ctx *ctx, T *dW, const T *input, const T *dY, const ConvBwdArgs &g, dh_status *st) {
+    const size_t L = static_cast<size_t>(g.N) * g.P * g.Q, Kp = static_cast<size_t>(g.C) * g.Hf * g.Wf;
+    const size_t patch_elems = L * Kp, a_elems = static_cast<size_t>(g.F) * L;
+    if (L < 4096 || (patch_elems + a_elems) * sizeof(T) > TRAIN_TEMP_LIMIT || dh_ceil_div(patch_elems, static_cast<size_t>(THREADS)) >= (size_t(1) << 31))
+        return false;
+    void *patch = nullptr, *a = nullptr;
+    *st = dh_malloc(ctx, patch_elems * sizeof(T), 0, &patch);
+    if (*st != DH_OK)
+        return true;
+    *st = dh_malloc(ctx, a_elems * sizeof(T), 0, &a);
+    if (*st != DH_OK) {
+        dh_free(ctx, patch);
+        return true;
+    }
+    constexpr int V = dh_vec<T>::N;
+    if (Kp % V == 0)
+        hipLaunchKernelGGL((im2col_kernel<T, V>), dim3(blocks_for(patch_elems / V)), dim3(THREADS), 0, ctx->stream, static_cast<T *>(patch),
+                           input, g, patch_elems / V);
+    else
+        hipLaunchKernelGGL((im2col_kernel<T, 1>), dim3(blocks_for(patch_elems)), dim3(THREADS), 0, ctx->stream, static_cast<T *>(patch), input,
+                           g, patch_elems);
+    hipLaunchKernelGGL((dy_rows_kernel<T>), dim3(blocks_for(a_elems)), dim3(THREADS), 0, ctx->stream, static_cast<T *>(a), dY, g, a_elems);
+    *st = mat_mul(ctx, dW, Kp, static_cast<const T *>(a), g.F, L, L, static_cast<const T *>(patch), L, Kp, Kp);
+    dh_free(ctx, patch);
+    dh_free(ctx, a);
+    return true;
+}
+
 template <typename T>
 dh_status conv2d_backward_data(dh_ctx *ctx, T *dX, const T *filter, const T *dY, size_t N, size_t C, size_t H, size_t W, size_t F,
-                               size_t Hf, size_t Wf, size_t sh, size_t sw, size_t padh, size_t padw) {
+                               size_t Hf, size_t Wf, size_t sh, size_t sw, size_t padh, size_t padw, bool use_mfma = true) {
     DH_REQUIRE_CTX(ctx);
     ConvBwdArgs g;
     dh_status st = conv_bwd_args(&g, N, C, H, W, F, Hf, Wf, sh, sw, padh, padw);
@@ -442,6 +698,8 @@ dh_status conv2d_backward_data(dh_ctx *ctx, T *dX, const T *filter, const T *dY,
     const size_t total = N * C * H * W;
     if (total == 0)
         return DH_OK;
+    if (use_mfma && conv_backward_data_mfma<T>(ctx, dX, filter, dY, g, &st))
+        return st;
     const size_t blocks = dh_ceil_div(total, THREADS);
     if (blocks >= (size_t(1) << 31))
         return dh_fail(DH_ERR_RUNTIME, "Conv2D backward - too many elements for one launch");
@@ -453,7 +711,7 @@ dh_status conv2d_backward_data(dh_ctx *ctx, T *dX, const T *filter, const T *dY,
 
 template <typename T>
 dh_status conv2d_backward_filter(dh_ctx *ctx, T *dW, const T *input, const T *dY, size_t N, size_t C, size_t H, size_t W, size_t F,
-                                 size_t Hf, size_t Wf, size_t sh, size_t sw, size_t padh, size_t padw) {
+                                 size_t Hf, size_t Wf, size_t sh, size_t sw, size_t padh, size_t padw, bool use_mfma = true) {
     DH_REQUIRE_CTX(ctx);
     ConvBwdArgs g;
     dh_status st = conv_bwd_args(&g, N, C, H, W, F, Hf, Wf, sh, sw, padh, padw);
@@ -463,6 +721,8 @@ dh_status conv2d_backward_filter(dh_ctx *ctx, T *dW, const T *input, const T *dY
         return DH_OK;
     if (F * C >= (size_t(1) << 31))
         return dh_fail(DH_ERR_RUNTIME, "Conv2D backward - too many filter planes for one launch");
+    if (use_mfma && conv_backward_filter_mfma<T>(ctx, dW, input, dY, g, &st))
+        return st;
     hipLaunchKernelGGL((conv_backward_filter_kernel<T, 16>), dim3(static_cast<unsigned>(F * C)), dim3(THREADS), 0, ctx->stream, dW,
                        input, dY, g);
     DH_CHECK_LAUNCH();

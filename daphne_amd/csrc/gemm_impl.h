@@ -473,6 +473,12 @@ dh_status gemm(dh_ctx *ctx, bool ta, bool tb, size_t m, size_t n, size_t k, cons
         } else if (m <= 32 && n <= 64) {
             bm = 32;
             bn = 64;
+        } else if (m <= 64 && n >= 512) {
+            bm = 64;
+            bn = 256;
+        } else if (n <= 64 && m >= 512) {
+            bm = 256;
+            bn = 64;
         }
     }
     g.tiles_m = static_cast<int>(dh_ceil_div(m, bm));
@@ -528,6 +534,10 @@ dh_status gemm(dh_ctx *ctx, bool ta, bool tb, size_t m, size_t n, size_t k, cons
         launch_cfg<T, 128, 128, GEMM_BK, 2, 2, EPI_STORE, true>(ctx, g, ta, tb, grid);
     else if (bm == 128 && bn == 128)
         DH_LAUNCH(128, 128, 2, 2);
+    else if (bm == 256 && bn == 64)
+        DH_LAUNCH(256, 64, 4, 1);
+    else if (bm == 64 && bn == 256)
+        DH_LAUNCH(64, 256, 1, 4);
     else if (bm == 256)
         DH_LAUNCH(256, 32, 4, 1);
     else if (bn == 256)

@@ -59,7 +59,8 @@ def test_batchnorm_train_forward_and_backward(ctx, dt, N, C, H, W):
 @pytest.mark.parametrize("dt", DTYPES)
 @pytest.mark.parametrize("p", [(2, 3, 3, 3, 2, 2, 2, 2, 1, 1), (4, 6, 28, 28, 2, 2, 2, 2, 0, 0), (3, 2, 14, 14, 3, 3, 2, 2, 1, 1),
                                (2, 2, 9, 7, 3, 2, 1, 1, 1, 0), (1, 1, 5, 5, 5, 5, 1, 1, 0, 0), (2, 3, 8, 8, 2, 2, 1, 1, 0, 0),
-                               (5, 4, 12, 12, 4, 4, 3, 3, 2, 2)])
+                               (5, 4, 12, 12, 4, 4, 3, 3, 2, 2), (3, 5, 14, 14, 2, 2, 2, 2, 0, 0), (2, 2, 7, 8, 2, 2, 2, 2, 0, 0),
+                               (64, 16, 14, 16, 2, 2, 2, 2, 0, 0)])
 def test_pooling_backward(ctx, dt, p):
     N, C, H, W, ph, pw, sh, sw, padh, padw = p
     rng = np.random.default_rng(sum(p))
@@ -88,7 +89,11 @@ def test_pooling_backward_all_negative_window_goes_to_the_padding(ctx):
 @pytest.mark.parametrize("dt", DTYPES)
 @pytest.mark.parametrize("case", [(1, 3, 3, 3, 2, 2, 2, 2, 2, 1, 1), (4, 3, 12, 12, 5, 3, 3, 1, 1, 1, 1), (2, 2, 9, 8, 3, 2, 3, 2, 1, 0, 1),
                                   (3, 1, 5, 5, 2, 5, 5, 1, 1, 2, 2), (2, 4, 14, 14, 6, 5, 5, 1, 1, 2, 2), (2, 2, 8, 8, 2, 3, 2, 2, 3, 1, 0),
-                                  (16, 8, 7, 7, 4, 7, 7, 1, 1, 3, 3)])
+                                  (16, 8, 7, 7, 4, 7, 7, 1, 1, 3, 3),
+                                  # large enough for the matrix-core paths (frame + forward convolution, patch matrix + GEMM)
+                                  (64, 8, 12, 12, 6, 3, 3, 1, 1, 1, 1), (64, 4, 16, 16, 8, 5, 5, 2, 2, 2, 2),
+                                  (48, 6, 15, 13, 5, 3, 2, 1, 2, 0, 1), (40, 3, 28, 28, 7, 5, 5, 1, 1, 2, 2),
+                                  (96, 5, 12, 12, 3, 2, 2, 3, 3, 1, 1)])
 def test_conv_backward(ctx, dt, case):
     N, C, H, W, F, Hf, Wf, sh, sw, ph, pw = case
     rng = np.random.default_rng(sum(case))

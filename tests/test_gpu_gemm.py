@@ -21,6 +21,7 @@ DTYPES = [np.float32, np.float64]
 SHAPES = [  # (m, n, k)
     (1, 1, 1), (3, 5, 7), (16, 16, 16), (33, 17, 65), (128, 128, 128), (129, 127, 130), (200, 300, 50),
     (256, 32, 64), (1000, 16, 64), (16, 64, 3000), (20, 300, 40), (5, 5, 20000), (260, 7, 9), (384, 512, 640),
+    (64, 800, 5000), (40, 513, 300), (800, 64, 5000), (513, 33, 100),  # 64 x 256 and 256 x 64 tiles, with and without split-K
 ]
 
 
