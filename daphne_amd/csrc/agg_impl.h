@@ -101,9 +101,10 @@ template <typename T, class R> __device__ __forceinline__ T block_reduce(T v) {
 // =======================================================================================
 // AggAll
 // =======================================================================================
-// Stage 1: (TX, TY) walk over rows x cvecs vectors; one partial per block.
+// Stage 1: block b owns the contiguous rows [b*slab, (b+1)*slab) and walks them with (TX, TY) threads over
+// rows x cvecs vectors; one partial per block.
 template <typename T, int VEC, class R, bool SQDEV>
-__global__ __launch_bounds__(THREADS) void all_stage1(const T *arg, size_t rows, size_t cvecs, size_t ld,
+__global__ __launch_bounds__(THREADS) void all_stage1(const T *arg, size_t rows, size_t cvecs, size_t ld, size_t slab,
                                                       const T *mean_dev, T *partials) {
     T m = T(0);
     if constexpr (SQDEV)
@@ -112,12 +113,14 @@ __global__ __launch_bounds__(THREADS) void all_stage1(const T *arg, size_t rows,
 #pragma unroll
     for (int i = 0; i < VEC; i++)
         acc[i] = R::id();
-    const size_t row_step = static_cast<size_t>(gridDim.x) * blockDim.y;
+    const size_t row_step = blockDim.y;
+    const size_t r_begin = static_cast<size_t>(blockIdx.x) * slab;
+    const size_t r_end = (r_begin + slab < rows) ? r_begin + slab : rows;
     for (size_t cv = static_cast<size_t>(blockIdx.y) * blockDim.x + threadIdx.x; cv < cvecs;
          cv += static_cast<size_t>(gridDim.y) * blockDim.x) {
         // main loop: UNROLL independent, unguarded loads in flight; then a guarded tail
-        size_t r0 = static_cast<size_t>(blockIdx.x) * blockDim.y + threadIdx.y;
-        for (; r0 + (UNROLL - 1) * row_step < rows; r0 += row_step * UNROLL) {
+        size_t r0 = r_begin + threadIdx.y;
+        for (; r0 + (UNROLL - 1) * row_step < r_end; r0 += row_step * UNROLL) {
             T x[UNROLL][VEC];
 #pragma unroll
             for (int u = 0; u < UNROLL; u++)
@@ -133,7 +136,7 @@ __global__ __launch_bounds__(THREADS) void all_stage1(const T *arg, size_t rows,
                 }
             }
         }
-        for (; r0 < rows; r0 += row_step) {
+        for (; r0 < r_end; r0 += row_step) {
             T x[VEC];
             dh_load_vec_stream<T, VEC>(arg + r0 * ld + cv * VEC, x);
 #pragma unroll
@@ -172,7 +175,7 @@ __global__ __launch_bounds__(THREADS) void all_stage2(const T *partials, size_t 
 
 struct Plan2D {
     dim3 grid, block;
-    size_t nblocks;
+    size_t nblocks, slab;
 };
 static inline Plan2D plan2d(const dh_ctx *ctx, size_t rows, size_t cvecs) {
     unsigned tx = 1;
@@ -183,7 +186,8 @@ static inline Plan2D plan2d(const dh_ctx *ctx, size_t rows, size_t cvecs) {
     if (gy > 512)
         gy = 512;
     const size_t max_blocks = static_cast<size_t>(ctx->num_cus) * 8;
-    size_t gx = dh_ceil_div(rows, static_cast<size_t>(ty) * UNROLL);
+    const size_t min_slab = static_cast<size_t>(ty) * UNROLL;
+    size_t gx = dh_ceil_div(rows, min_slab);
     size_t cap = max_blocks / gy;
     if (cap < 1)
         cap = 1;
@@ -191,7 +195,12 @@ static inline Plan2D plan2d(const dh_ctx *ctx, size_t rows, size_t cvecs) {
         gx = cap;
     if (gx < 1)
         gx = 1;
+    size_t slab = dh_ceil_div(dh_ceil_div(rows, gx), min_slab) * min_slab;
+    gx = dh_ceil_div(rows, slab);
+    if (gx < 1)
+        gx = 1;
     Plan2D p;
+    p.slab = slab;
     p.grid = dim3(static_cast<unsigned>(gx), static_cast<unsigned>(gy), 1);
     p.block = dim3(tx, ty, 1);
     p.nblocks = gx * gy;
@@ -211,14 +220,14 @@ static inline size_t all_stage1_launch(dh_ctx *ctx, const T *arg, size_t rows, s
         if (body_rows) {
             Plan2D p = plan2d(ctx, body_rows, THREADS);
             hipLaunchKernelGGL((all_stage1<T, V, R, SQDEV>), p.grid, p.block, 0, ctx->stream, arg, body_rows,
-                               size_t(THREADS), width, mean_dev, partials);
+                               size_t(THREADS), width, p.slab, mean_dev, partials);
             np += p.nblocks;
         }
         const size_t done = body_rows * width;
         if (done < n) {
             Plan2D p = plan2d(ctx, 1, n - done);
             hipLaunchKernelGGL((all_stage1<T, 1, R, SQDEV>), p.grid, p.block, 0, ctx->stream, arg + done, size_t(1),
-                               n - done, n - done, mean_dev, partials + np);
+                               n - done, n - done, p.slab, mean_dev, partials + np);
             np += p.nblocks;
         }
         return np;
@@ -227,12 +236,12 @@ static inline size_t all_stage1_launch(dh_ctx *ctx, const T *arg, size_t rows, s
     if (vec_ok) {
         Plan2D p = plan2d(ctx, rows, cols / V);
         hipLaunchKernelGGL((all_stage1<T, V, R, SQDEV>), p.grid, p.block, 0, ctx->stream, arg, rows, cols / V, ld,
-                           mean_dev, partials);
+                           p.slab, mean_dev, partials);
         np = p.nblocks;
     } else {
         Plan2D p = plan2d(ctx, rows, cols);
         hipLaunchKernelGGL((all_stage1<T, 1, R, SQDEV>), p.grid, p.block, 0, ctx->stream, arg, rows, cols, ld,
-                           mean_dev, partials);
+                           p.slab, mean_dev, partials);
         np = p.nblocks;
     }
     return np;
