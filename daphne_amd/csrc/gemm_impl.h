@@ -151,27 +151,49 @@ struct GemmArgs {
     int tiles_m, tiles_n;
     int triangular;     // 1: only tiles with tile_n >= tile_m exist (Syrk)
     int aligned_a, aligned_b;
+    int tile_offset;    // added to the workgroup's tile id (the launch that finishes the tiles a first launch left)
+    int compact;        // 1: C holds one dense BM x BN block per (K slice, workgroup) instead of the result matrix
 };
 
-// Maps the linear workgroup id to a tile. See file comment for the XCD regrouping.
-__device__ __forceinline__ void tile_of_block(const GemmArgs &g, int &tm, int &tn) {
-    const int nb = gridDim.x;
-    int id = blockIdx.x;
+// Consecutive workgroup ids are dealt round-robin to the 8 XCDs: regroup them so that each XCD walks a
+// contiguous range of tile ids.
+__device__ __forceinline__ int regroup_for_xcds(int id, int nb) {
     constexpr int XCDS = 8;
-    if (nb % XCDS == 0)
-        id = (id % XCDS) * (nb / XCDS) + id / XCDS;
+    return (nb % XCDS == 0) ? (id % XCDS) * (nb / XCDS) + id / XCDS : id;
+}
+
+// Maps a tile id to a tile. Rectangular results: panels of 8 tile rows, walked down the rows first, so that
+// 64 consecutive ids share 8 row panels of A and 8 column panels of B. Triangular results: the same 8 x 8
+// groups over the tiles on and above the diagonal (the groups on the diagonal hold their upper triangle).
+__device__ __forceinline__ void tile_of_id(const GemmArgs &g, int id, int &tm, int &tn) {
+    constexpr int PANEL = 8;
     if (g.triangular) {
-        // row-wise enumeration of the upper triangle: row i holds tiles_n - i tiles
-        int i = 0, rem = id;
-        while (rem >= g.tiles_n - i) {
-            rem -= g.tiles_n - i;
-            i++;
+        const int nt = g.tiles_n;
+        int first = 0, rem = id, h = 0, diag = 0;
+        for (;; first += PANEL) {
+            h = (nt - first < PANEL) ? nt - first : PANEL; // tile rows in this panel
+            diag = h * (h + 1) / 2;
+            const int right = (nt - first - PANEL > 0) ? nt - first - PANEL : 0; // tile columns right of the diagonal group
+            const int here = diag + h * right;
+            if (rem < here || first + PANEL >= nt)
+                break;
+            rem -= here;
         }
-        tm = i;
-        tn = i + rem;
+        if (rem < diag) {
+            int i = 0;
+            while (rem >= h - i) {
+                rem -= h - i;
+                i++;
+            }
+            tm = first + i;
+            tn = first + i + rem;
+        } else {
+            rem -= diag;
+            tm = first + rem % h;
+            tn = first + PANEL + rem / h;
+        }
         return;
     }
-    constexpr int PANEL = 8;
     const int per_panel = PANEL * g.tiles_n;
     const int panel = id / per_panel;
     const int first_m = panel * PANEL;
@@ -200,7 +222,7 @@ __global__ __launch_bounds__(64 * WM * WN, FULL ? 2 : 1) void gemm_kernel(GemmAr
     __shared__ __attribute__((aligned(16))) T lds_b[2][LB::ELEMS];
 
     int tile_m, tile_n;
-    tile_of_block(g, tile_m, tile_n);
+    tile_of_id(g, regroup_for_xcds(blockIdx.x, gridDim.x) + g.tile_offset, tile_m, tile_n);
     const size_t m0 = static_cast<size_t>(tile_m) * BM, n0 = static_cast<size_t>(tile_n) * BN;
     const size_t k_begin = static_cast<size_t>(blockIdx.z) * g.k_chunk;
     const size_t k_end = (k_begin + g.k_chunk < g.k) ? k_begin + g.k_chunk : g.k;
@@ -283,6 +305,13 @@ __global__ __launch_bounds__(64 * WM * WN, FULL ? 2 : 1) void gemm_kernel(GemmAr
 
     // epilogue
     T *C = static_cast<T *>(g.C) + static_cast<size_t>(blockIdx.z) * g.slab_stride;
+    size_t ldc = g.ldc, row_off = 0, col_off = 0;
+    if (g.compact) {
+        C = static_cast<T *>(g.C) + (static_cast<size_t>(blockIdx.z) * gridDim.x + blockIdx.x) * (BM * BN);
+        ldc = BN;
+        row_off = m0;
+        col_off = n0;
+    }
 #pragma unroll
     for (int i = 0; i < FM; i++)
 #pragma unroll
@@ -296,7 +325,7 @@ __global__ __launch_bounds__(64 * WM * WN, FULL ? 2 : 1) void gemm_kernel(GemmAr
                 for (int v = 0; v < M::ACC; v++) {
                     const size_t r = m0 + wave_m * TM + i * M::MT + M::row(lane, v);
                     if (FULL || r < g.m)
-                        C[r * g.ldc + c] = acc[i][j][v] + b;
+                        C[(r - row_off) * ldc + (c - col_off)] = acc[i][j][v] + b;
                 }
             }
         }
@@ -324,12 +353,54 @@ __global__ __launch_bounds__(256) void slab_reduce_kernel(T *C, size_t ldc, cons
         C[c * ldc + r] = s;
 }
 
-// Upper -> lower mirror for a Syrk that ran without split-K.
+// Folds the dense BM x BN blocks that a compact launch of `ntail` workgroups and `nslabs` K slices left
+// (block of slice z, workgroup b at slabs[(z * ntail + b) * BM * BN]) into the result, in slice order.
+template <typename T, int BM, int BN>
+__global__ __launch_bounds__(256) void tail_reduce_kernel(GemmArgs g, const T *slabs, int nslabs, int ntail) {
+    int tm, tn;
+    tile_of_id(g, regroup_for_xcds(blockIdx.x, ntail) + g.tile_offset, tm, tn);
+    T *C = static_cast<T *>(g.C);
+    const T *bias = static_cast<const T *>(g.bias);
+    const int e = blockIdx.y * 256 + threadIdx.x; // grid.y = BM * BN / 256: one element of the tile per thread
+    const size_t r = static_cast<size_t>(tm) * BM + e / BN, c = static_cast<size_t>(tn) * BN + e % BN;
+    if (r >= g.m || c >= g.n)
+        return;
+    const T *p = slabs + static_cast<size_t>(blockIdx.x) * (BM * BN) + e;
+    const size_t step = static_cast<size_t>(ntail) * (BM * BN);
+    T sum = T(0);
+    int z = 0;
+    for (; z + 4 <= nslabs; z += 4) {
+        const T a0 = p[z * step], a1 = p[(z + 1) * step], a2 = p[(z + 2) * step], a3 = p[(z + 3) * step];
+        sum = (((sum + a0) + a1) + a2) + a3;
+    }
+    for (; z < nslabs; z++)
+        sum += p[z * step];
+    if (bias)
+        sum += bias[c * g.bias_stride];
+    C[r * g.ldc + c] = sum;
+}
+
+// Upper -> lower mirror for a Syrk that ran without split-K: workgroup (bx, by), by >= bx, copies the 64 x 64
+// tile (bx, by) above the diagonal through LDS into tile (by, bx) below it, both sides along rows.
 template <typename T> __global__ __launch_bounds__(256) void mirror_kernel(T *C, size_t ldc, size_t n) {
-    const size_t c = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-    const size_t r = static_cast<size_t>(blockIdx.y) * blockDim.y + threadIdx.y;
-    if (r < n && c < n && c > r)
-        C[c * ldc + r] = C[r * ldc + c];
+    __shared__ T tile[64][65];
+    if (blockIdx.y < blockIdx.x)
+        return;
+    const int tx = threadIdx.x % 64, ty = threadIdx.x / 64;
+    const size_t up = static_cast<size_t>(blockIdx.x) * 64, low = static_cast<size_t>(blockIdx.y) * 64;
+#pragma unroll 4
+    for (int i = ty; i < 64; i += 4) {
+        const size_t r = up + i, c = low + tx;
+        if (r < n && c < n)
+            tile[i][tx] = C[r * ldc + c];
+    }
+    __syncthreads();
+#pragma unroll 4
+    for (int i = ty; i < 64; i += 4) {
+        const size_t r = low + i, c = up + tx;
+        if (r < n && c < r)
+            C[r * ldc + c] = tile[tx][i];
+    }
 }
 
 // ---------------------------------------------------------------------------------------
@@ -519,7 +590,28 @@ dh_status gemm(dh_ctx *ctx, bool ta, bool tb, size_t m, size_t n, size_t k, cons
         g.ldc = n;
         g.slab_stride = m * n;
     }
-    const dim3 grid(static_cast<unsigned>(tiles), 1, static_cast<unsigned>(ksplit));
+    // A tile count a little above a multiple of the resident workgroups would leave most of the device idle while
+    // the last few tiles run: those tiles go to a second launch that also splits K, into dense per-tile blocks
+    // that a small kernel folds into the result in slice order.
+    size_t tail = 0, tail_split = 1;
+    if (direct && bm == 128 && bn == 128 && tiles > slots && k_tiles >= 32) {
+        const size_t excess = tiles % slots;
+        if (excess > 0 && excess * 4 <= slots) {
+            tail = excess;
+            tail_split = slots / excess;
+            if (tail_split > k_tiles / 8)
+                tail_split = k_tiles / 8;
+        }
+    }
+    T *tail_slabs = nullptr;
+    if (tail) {
+        void *wsv = nullptr;
+        dh_status st = dh_workspace(ctx, tail_split * tail * bm * bn * sizeof(T), &wsv);
+        if (st != DH_OK)
+            return st;
+        tail_slabs = static_cast<T *>(wsv);
+    }
+    const dim3 grid(static_cast<unsigned>(tiles - tail), 1, static_cast<unsigned>(ksplit));
     const bool fuse_bias = direct && bias != nullptr;
 #define DH_LAUNCH(BM_, BN_, WM_, WN_)                                                              \
     do {                                                                                           \
@@ -528,8 +620,9 @@ dh_status gemm(dh_ctx *ctx, bool ta, bool tb, size_t m, size_t n, size_t k, cons
         else                                                                                       \
             launch_cfg<T, BM_, BN_, GEMM_BK, WM_, WN_, EPI_STORE>(ctx, g, ta, tb, grid);           \
     } while (0)
-    const bool full = bm == 128 && bn == 128 && !fuse_bias && m % 128 == 0 && n % 128 == 0 && k % GEMM_BK == 0 &&
-                      g.aligned_a && g.aligned_b && k > 0;
+    const bool interior = bm == 128 && bn == 128 && m % 128 == 0 && n % 128 == 0 && k % GEMM_BK == 0 &&
+                          g.aligned_a && g.aligned_b && k > 0;
+    const bool full = interior && !fuse_bias;
     if (full)
         launch_cfg<T, 128, 128, GEMM_BK, 2, 2, EPI_STORE, true>(ctx, g, ta, tb, grid);
     else if (bm == 128 && bn == 128)
@@ -546,6 +639,26 @@ dh_status gemm(dh_ctx *ctx, bool ta, bool tb, size_t m, size_t n, size_t k, cons
         DH_LAUNCH(32, 64, 1, 2);
 #undef DH_LAUNCH
     DH_CHECK_LAUNCH();
+    if (tail) {
+        GemmArgs t = g;
+        t.C = tail_slabs;
+        t.bias = nullptr;
+        t.tile_offset = static_cast<int>(tiles - tail);
+        t.compact = 1;
+        t.k_chunk = dh_ceil_div(k_tiles, tail_split) * GEMM_BK;
+        const size_t slices = dh_ceil_div(k, t.k_chunk);
+        const dim3 tgrid(static_cast<unsigned>(tail), 1, static_cast<unsigned>(slices));
+        if (interior)
+            launch_cfg<T, 128, 128, GEMM_BK, 2, 2, EPI_STORE, true>(ctx, t, ta, tb, tgrid);
+        else
+            launch_cfg<T, 128, 128, GEMM_BK, 2, 2, EPI_STORE>(ctx, t, ta, tb, tgrid);
+        DH_CHECK_LAUNCH();
+        GemmArgs r = g;
+        r.tile_offset = t.tile_offset;
+        hipLaunchKernelGGL((tail_reduce_kernel<T, 128, 128>), dim3(static_cast<unsigned>(tail), 128 * 128 / 256), dim3(256), 0, ctx->stream, r,
+                           tail_slabs, static_cast<int>(slices), static_cast<int>(tail));
+        DH_CHECK_LAUNCH();
+    }
     const dim3 eb(64, 4), eg(static_cast<unsigned>(dh_ceil_div(n, 64)), static_cast<unsigned>(dh_ceil_div(m, 4)));
     if (!direct) {
         if (triangular)
@@ -556,7 +669,8 @@ dh_status gemm(dh_ctx *ctx, bool ta, bool tb, size_t m, size_t n, size_t k, cons
                                static_cast<int>(ksplit), m, n, bias, bias_stride);
         DH_CHECK_LAUNCH();
     } else if (triangular) {
-        hipLaunchKernelGGL((mirror_kernel<T>), eg, eb, 0, ctx->stream, C, ldc, n);
+        const unsigned mt = static_cast<unsigned>(dh_ceil_div(n, 64));
+        hipLaunchKernelGGL((mirror_kernel<T>), dim3(mt, mt), dim3(256), 0, ctx->stream, C, ldc, n);
         DH_CHECK_LAUNCH();
     }
     return DH_OK;

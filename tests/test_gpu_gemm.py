@@ -132,6 +132,44 @@ def test_syrk(ctx, dt, trans_left, rows, cols):
 
 
 @pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("trans_left", [True, False])
+@pytest.mark.parametrize("n,k", [(1300, 300), (2100, 70), (4100, 520)])
+def test_syrk_many_tiles(ctx, dt, trans_left, n, k):
+    """Results of 11, 17 and 33 tiles a side: the triangular tile order walks several groups of 8 x 8 tiles, and at
+    33 a side (561 tiles, more than the device holds at once) the last tiles run as a launch of their own that
+    splits K. Integer-valued inputs: every order of summation gives the same bits; the expectation is numpy's."""
+    rng = np.random.default_rng(n + k)
+    x = rng.integers(-3, 4, (k, n) if trans_left else (n, k)).astype(dt)
+    xi = x.astype(np.int64)
+    exp = ((xi.T @ xi) if trans_left else (xi @ xi.T)).astype(dt)
+    got = syrk(None, DenseMatrix.from_numpy(ctx, x), trans_left, ctx).to_numpy()
+    assert_exact(got, exp)
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("ta,tb", [(False, False), (True, True)])
+@pytest.mark.parametrize("m,n,k", [(4224, 2048, 512), (4200, 2040, 520)])
+def test_matmul_leftover_tiles(ctx, dt, ta, tb, m, n, k):
+    """33 x 16 = 528 tiles of 128 x 128: 512 run as one launch, the other 16 as a second launch that splits K
+    (with and without partial tiles). Integer-valued inputs, exact; then a random case with a bias row through
+    Affine, norm-wise against numpy in double."""
+    rng = np.random.default_rng(m + n + k)
+    a = rng.integers(-3, 4, (k, m) if ta else (m, k)).astype(dt)
+    b = rng.integers(-3, 4, (n, k) if tb else (k, n)).astype(dt)
+    exp = ((a.T if ta else a).astype(np.int64) @ (b.T if tb else b).astype(np.int64)).astype(dt)
+    got = matMul(None, DenseMatrix.from_numpy(ctx, a), DenseMatrix.from_numpy(ctx, b), ta, tb, ctx).to_numpy()
+    assert_exact(got, exp)
+    if not ta and not tb:
+        x = (rng.random((m, k)) - 0.5).astype(dt)
+        w = (rng.standard_normal((k, n)) * np.sqrt(2.0 / k)).astype(dt)
+        bias = (rng.standard_normal((1, n)) * 0.1).astype(dt)
+        truth = (x.astype(np.float64) @ w.astype(np.float64) + bias.astype(np.float64)).astype(dt)
+        got = affineForward(None, DenseMatrix.from_numpy(ctx, x), DenseMatrix.from_numpy(ctx, w),
+                            DenseMatrix.from_numpy(ctx, bias), ctx).to_numpy()
+        assert_close(got, truth, elementwise=False)
+
+
+@pytest.mark.parametrize("dt", DTYPES)
 def test_syrk_integer_valued_exact(ctx, dt):
     rng = np.random.default_rng(9)
     x = rng.integers(-3, 4, (3000, 150)).astype(dt)
