@@ -21,6 +21,7 @@
 #include "gemm_impl.h"
 
 #include <limits>
+#include <type_traits>
 
 namespace dh_dnn {
 
@@ -264,6 +265,216 @@ __global__ __launch_bounds__(64 * WN) void conv2d_kernel(ConvArgs g) {
     }
 }
 
+// ---------------------------------------------------------------------------------------
+// Convolution with the image resident in LDS. One workgroup of 8 waves takes one image (all of its channels,
+// with the zero border written out while it is copied in), 16 * MFW filters and up to `chunk` output pixels, and
+// runs the whole K = C * Hf * Wf contraction without a barrier: every wave owns one block of 16 filters and NF
+// blocks of 16 pixels as accumulators of the 16x16x4 matrix instruction, reads its filter fragment from the
+// padded filter matrix in global memory (a 16-byte vector per lane, one block of K ahead) and gathers the
+// patch fragment straight from the LDS image at "pixel offset + table[k]".
+// ---------------------------------------------------------------------------------------
+struct ConvResidentArgs {
+    const void *x;     // N x C x H x W
+    const void *wpack; // filter matrix padded with zeros to Fpad x Kpad
+    const int *ktab;   // k -> c*Hp*Wp + hy*Wp + hx (0 beyond K)
+    const void *bias;
+    void *res;
+    unsigned C, H, W, Hp, Wp, ph, pw, Q, sh, sw, F, Kpad, HpWp, PQ, chunk;
+    unsigned CG, KG;   // channels per stage of the LDS image and their share of K (a multiple of the K block)
+};
+
+// Copies one image (C x H x W at x) into LDS as C x Hp x Wp with the zero border of Padding.h:11-22 written out,
+// by the nt threads of a workgroup. A thread keeps its position(s) inside the padded plane and walks the
+// channels, so the divisions are done once; planes of fewer than nt elements are taken by several groups of
+// threads side by side.
+template <typename T>
+__device__ __forceinline__ void conv_stage_frame(T *frame, const T *x, unsigned C, unsigned H, unsigned W, unsigned Wp,
+                                                 unsigned ph, unsigned pw, unsigned HpWp, unsigned frame_elems, int tid,
+                                                 unsigned nt) {
+    constexpr int VEC = 16 / sizeof(T);
+    const unsigned HW = H * W;
+    if (ph == 0 && pw == 0 && frame_elems % VEC == 0 && reinterpret_cast<size_t>(x) % 16 == 0) {
+        // no border: the frame is the image, copied with 16-byte vectors, four loads of a thread in flight at once
+        constexpr int UN = 4;
+        const unsigned nvec = frame_elems / VEC;
+        for (unsigned v0 = tid; v0 < nvec; v0 += nt * UN) {
+            T t[UN][VEC];
+#pragma unroll
+            for (int u = 0; u < UN; u++) {
+                const unsigned v = v0 + u * nt;
+                dh_load_vec_stream<T, VEC>(x + static_cast<size_t>(v < nvec ? v : v0) * VEC, t[u]);
+            }
+#pragma unroll
+            for (int u = 0; u < UN; u++)
+                if (v0 + u * nt < nvec)
+                    dh_store_vec<T, VEC>(frame + static_cast<size_t>(v0 + u * nt) * VEC, t[u]);
+        }
+        return;
+    }
+    const bool narrow = HpWp < nt;
+    const unsigned groups = narrow ? nt / HpWp : 1;
+    const unsigned grp = narrow ? tid / HpWp : 0;
+    if (grp >= groups)
+        return;
+    for (unsigned r = narrow ? tid % HpWp : tid; r < HpWp; r += nt) {
+        const unsigned y = r / Wp - ph, xx = r % Wp - pw; // wraps to a huge value inside the border
+        const bool in = y < H && xx < W;
+        const T *src = x + (in ? y * W + xx : 0);
+        T *dst = frame + r;
+        // batches of UN channels: all loads of a batch are issued (unconditionally, from clamped addresses) before
+        // the first value is stored; lanes on the border load the image's first element and store zeros
+        constexpr int UN = 16;
+        for (unsigned c0 = grp; c0 < C; c0 += groups * UN) {
+            T v[UN];
+#pragma unroll
+            for (int u = 0; u < UN; u++) {
+                const unsigned c = c0 + u * groups;
+                v[u] = __builtin_nontemporal_load(src + static_cast<size_t>(c < C ? c : c0) * HW);
+            }
+#pragma unroll
+            for (int u = 0; u < UN; u++) {
+                const unsigned c = c0 + u * groups;
+                if (c < C)
+                    dst[c * HpWp] = in ? v[u] : T(0);
+            }
+        }
+    }
+}
+
+template <typename T, int MFW, int NF>
+__global__ __launch_bounds__(512) void conv2d_resident_kernel(ConvResidentArgs g) {
+    using M = dh_gemm::Mfma16<T>;
+    constexpr int VEC = 16 / sizeof(T), NPARTS = 8 / MFW;
+    extern __shared__ __attribute__((aligned(16))) unsigned char conv_lds[];
+    int *ktab = reinterpret_cast<int *>(conv_lds);               // Kpad entries: a multiple of 16 bytes
+    T *frame = reinterpret_cast<T *>(conv_lds + g.Kpad * sizeof(int));
+    const int tid = threadIdx.x, lane = tid % 64, wave = __builtin_amdgcn_readfirstlane(tid / 64);
+    const unsigned img = blockIdx.x, f0 = blockIdx.y * (16 * MFW), px0 = blockIdx.z * g.chunk;
+
+    for (unsigned k = tid; k < g.Kpad; k += 512)
+        ktab[k] = g.ktab[k];
+
+    const int mf = wave % MFW, part = wave / MFW;
+    const int li = lane % 16, lk = lane / 16;
+    // this lane's pixel in each of the wave's pixel blocks; blocks past the image end are skipped (uniform)
+    int pixoff[NF], outoff[NF];
+    int nfv = 0;
+#pragma unroll
+    for (int j = 0; j < NF; j++) {
+        const unsigned first = px0 + (j * NPARTS + part) * 16; // blocks dealt round-robin: the waves' counts differ by at most one
+        const unsigned px = first + li;
+        const bool ok = px < g.PQ;
+        const unsigned pp = ok ? px / g.Q : 0, qq = ok ? px % g.Q : 0;
+        pixoff[j] = static_cast<int>(pp * g.sh * g.Wp + qq * g.sw);
+        outoff[j] = ok ? static_cast<int>(px) : -1;
+        if (first < g.PQ)
+            nfv = j + 1;
+    }
+    typename M::acc_t acc[NF];
+#pragma unroll
+    for (int j = 0; j < NF; j++)
+        acc[j] = typename M::acc_t{0, 0, 0, 0};
+
+    const T *wrow = static_cast<const T *>(g.wpack) + static_cast<size_t>(f0 + mf * 16 + li) * g.Kpad + lk * VEC;
+    const int *ktl = ktab + lk * VEC;
+    // The contraction, for a number of pixel blocks fixed at compile time: no branch inside the loop body, so that
+    // LDS reads and matrix instructions of neighbouring blocks interleave. A wave with fewer blocks than NF - 1
+    // computes all NF (the spare ones gather pixel 0 and are never stored).
+    // k_begin .. k_end: this stage's share of K; sub: the table offset of the stage's first channel
+    auto contract = [&](auto nv_tag, unsigned k_begin, unsigned k_end, int sub) {
+        constexpr int NV = decltype(nv_tag)::value;
+        T a_cur[VEC], b_cur[NV];
+        int kt[VEC];
+        dh_load_vec<T, VEC>(wrow + k_begin, a_cur);
+#pragma unroll
+        for (int s_ = 0; s_ < VEC; s_++)
+            kt[s_] = max(ktl[k_begin + s_] - sub, 0); // the zero entries beyond K stay inside the stage
+#pragma unroll
+        for (int j = 0; j < NV; j++)
+            b_cur[j] = frame[pixoff[j] + kt[0]];
+        for (unsigned k0 = k_begin; k0 < k_end; k0 += 4 * VEC) {
+            // the next block's filter values and table entries, loaded unconditionally (the last block loads itself again)
+            const unsigned kn = (k0 + 4 * VEC < k_end) ? k0 + 4 * VEC : k0;
+            T a_nxt[VEC];
+            int kt_nxt[VEC];
+            dh_load_vec<T, VEC>(wrow + kn, a_nxt);
+#pragma unroll
+            for (int s_ = 0; s_ < VEC; s_++)
+                kt_nxt[s_] = max(ktl[kn + s_] - sub, 0);
+#pragma unroll
+            for (int s_ = 0; s_ < VEC; s_++) {
+                // the patch values of the following step are on their way while this step's matrix instructions run
+                const int kt_after = (s_ + 1 < VEC) ? kt[s_ + 1] : kt_nxt[0];
+                T b_nxt[NV];
+#pragma unroll
+                for (int j = 0; j < NV; j++)
+                    b_nxt[j] = frame[pixoff[j] + kt_after];
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int j = 0; j < NV; j++)
+                    acc[j] = M::mma(a_cur[s_], b_cur[j], acc[j]);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int j = 0; j < NV; j++)
+                    b_cur[j] = b_nxt[j];
+            }
+#pragma unroll
+            for (int s_ = 0; s_ < VEC; s_++) {
+                a_cur[s_] = a_nxt[s_];
+                kt[s_] = kt_nxt[s_];
+            }
+        }
+    };
+    // The image goes through LDS in stages of CG channels (all of them when they fit); the accumulators stay.
+    const T *ximg = static_cast<const T *>(g.x) + static_cast<size_t>(img) * g.C * g.H * g.W;
+    for (unsigned c0 = 0, k_begin = 0; c0 < g.C; c0 += g.CG, k_begin += g.KG) {
+        const unsigned cg = (g.C - c0 < g.CG) ? g.C - c0 : g.CG;
+        const unsigned k_end = (c0 + g.CG < g.C) ? k_begin + g.KG : g.Kpad;
+        if (c0)
+            __syncthreads(); // every wave is done with the previous stage
+        conv_stage_frame<T>(frame, ximg + static_cast<size_t>(c0) * g.H * g.W, cg, g.H, g.W, g.Wp, g.ph, g.pw, g.HpWp,
+                            cg * g.HpWp, tid, 512);
+        __syncthreads();
+        const int sub = static_cast<int>(c0 * g.HpWp);
+        if (nfv == NF - 1)
+            contract(std::integral_constant<int, NF - 1>{}, k_begin, k_end, sub);
+        else if (nfv > 0)
+            contract(std::integral_constant<int, NF>{}, k_begin, k_end, sub);
+    }
+
+    T *out = static_cast<T *>(g.res) + static_cast<size_t>(img) * g.F * g.PQ;
+    const T *bias = static_cast<const T *>(g.bias);
+    T bv[4];
+#pragma unroll
+    for (int v = 0; v < 4; v++) {
+        const unsigned f = f0 + mf * 16 + M::row(lane, v);
+        bv[v] = (bias && f < g.F) ? bias[f] : T(0);
+    }
+#pragma unroll
+    for (int j = 0; j < NF; j++) {
+        if (j < nfv && outoff[j] >= 0) {
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                const unsigned f = f0 + mf * 16 + M::row(lane, v);
+                if (f < g.F)
+                    out[static_cast<size_t>(f) * g.PQ + outoff[j]] = acc[j][v] + bv[v];
+            }
+        }
+    }
+}
+
+template <typename T, int MFW, int NF> static inline dh_status conv2d_resident_launch(dh_ctx *ctx, const ConvResidentArgs &g, dim3 grid, size_t lds) {
+    static size_t allowed = 0; // dynamic LDS beyond 64 KiB has to be asked for once per kernel
+    if (lds > 65536 && lds > allowed) {
+        DH_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&conv2d_resident_kernel<T, MFW, NF>),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
+        allowed = lds;
+    }
+    hipLaunchKernelGGL((conv2d_resident_kernel<T, MFW, NF>), grid, dim3(512), lds, ctx->stream, g);
+    DH_CHECK_LAUNCH();
+    return DH_OK;
+}
+
 template <typename T>
 dh_status conv2d_forward(dh_ctx *ctx, T *res, size_t *res_h, size_t *res_w, const T *data, const T *filter,
                          size_t filter_rows, size_t filter_cols, const T *bias, size_t N, size_t C, size_t H,
@@ -294,6 +505,80 @@ dh_status conv2d_forward(dh_ctx *ctx, T *res, size_t *res_h, size_t *res_w, cons
     if (C * Hp * Wp * images_per_tile * sizeof(T) >= (size_t(1) << 32) || K >= (size_t(1) << 31) ||
         P * Q >= (size_t(1) << 31) || N >= (size_t(1) << 31) || F >= (size_t(1) << 31))
         return dh_fail(DH_ERR_RUNTIME, "Convolution: image or filter extents exceed the 32-bit addressing of a tile");
+    {
+        // Image resident in LDS: the padded image and the offset table must fit, and every wave should own at
+        // least three blocks of 16 pixels (smaller images leave the waves idle; they take the tiled kernel below).
+        const int mfw = F <= 16 ? 1 : (F <= 32 ? 2 : 4);
+        const size_t parts = 8 / mfw;
+        const size_t blocks16 = dh_ceil_div(P * Q, 16);
+        const size_t kpad = dh_ceil_div(K, BK) * BK;
+        // channels per stage: the whole image if it takes no more than 48 KiB (three workgroups per CU), else the
+        // fewest equal stages that do, provided a stage's share of K is a whole number of K blocks
+        size_t cg = C;
+        if (C * Hp * Wp * sizeof(T) > 48 * 1024) {
+            const size_t stages = dh_ceil_div(C * Hp * Wp * sizeof(T), static_cast<size_t>(44 * 1024));
+            const size_t per = dh_ceil_div(C, stages);
+            if (per >= 1 && (per * Hf * Wf) % BK == 0)
+                cg = per;
+        }
+        const size_t lds = kpad * sizeof(int) + cg * Hp * Wp * sizeof(T);
+        const size_t fgroups = dh_ceil_div(F, static_cast<size_t>(16 * mfw));
+        const size_t chunks = dh_ceil_div(blocks16, parts * 13);            // at most 13 blocks per wave
+        const size_t nf = dh_ceil_div(blocks16, parts * chunks);            // spread evenly over the chunks
+        const size_t chunk = parts * nf * 16;
+        // One workgroup per CU (more than 80 KiB of LDS) has nothing to cover its loading phase and its LDS
+        // latencies with: taken only when a wave has at least six blocks of matrix instructions per step.
+        if (lds <= 150 * 1024 && (lds <= 80 * 1024 || nf >= 6) && blocks16 >= 3 * parts && K >= 32 && fgroups < 65536 &&
+            chunks < 65536) {
+            const size_t fpad = fgroups * 16 * mfw;
+            const size_t tab_bytes = dh_ceil_div(kpad * sizeof(int), 256) * 256;
+            void *wsv = nullptr;
+            dh_status st = dh_workspace(ctx, tab_bytes + fpad * kpad * sizeof(T), &wsv);
+            if (st != DH_OK)
+                return st;
+            int *tab = static_cast<int *>(wsv);
+            T *wpack = reinterpret_cast<T *>(static_cast<char *>(wsv) + tab_bytes);
+            size_t pg = dh_ceil_div(fpad * kpad, 256);
+            if (pg > 1024)
+                pg = 1024;
+            hipLaunchKernelGGL((conv_prep_kernel<T>), dim3(static_cast<unsigned>(pg)), dim3(256), 0, ctx->stream, tab, wpack,
+                               filter, static_cast<unsigned>(F), static_cast<unsigned>(fpad), static_cast<unsigned>(K),
+                               static_cast<unsigned>(kpad), static_cast<unsigned>(Hp * Wp), static_cast<unsigned>(Wp),
+                               static_cast<unsigned>(Hf), static_cast<unsigned>(Wf));
+            DH_CHECK_LAUNCH();
+            ConvResidentArgs r{};
+            r.x = data;
+            r.wpack = wpack;
+            r.ktab = tab;
+            r.bias = bias;
+            r.res = res;
+            r.C = static_cast<unsigned>(C);
+            r.H = static_cast<unsigned>(H);
+            r.W = static_cast<unsigned>(W);
+            r.Hp = static_cast<unsigned>(Hp);
+            r.Wp = static_cast<unsigned>(Wp);
+            r.ph = static_cast<unsigned>(ph);
+            r.pw = static_cast<unsigned>(pw);
+            r.Q = static_cast<unsigned>(Q);
+            r.sh = static_cast<unsigned>(sh);
+            r.sw = static_cast<unsigned>(sw);
+            r.F = static_cast<unsigned>(F);
+            r.Kpad = static_cast<unsigned>(kpad);
+            r.HpWp = static_cast<unsigned>(Hp * Wp);
+            r.CG = static_cast<unsigned>(cg);
+            r.KG = static_cast<unsigned>(cg * Hf * Wf);
+            r.PQ = static_cast<unsigned>(P * Q);
+            r.chunk = static_cast<unsigned>(chunk);
+            const dim3 grid(static_cast<unsigned>(N), static_cast<unsigned>(fgroups), static_cast<unsigned>(chunks));
+#define DH_CONV_RES(MFW_)                                                                          \
+    (nf <= 4 ? conv2d_resident_launch<T, MFW_, 4>(ctx, r, grid, lds)                               \
+             : (nf <= 7 ? conv2d_resident_launch<T, MFW_, 7>(ctx, r, grid, lds)                    \
+                        : (nf <= 10 ? conv2d_resident_launch<T, MFW_, 10>(ctx, r, grid, lds)       \
+                                    : conv2d_resident_launch<T, MFW_, 13>(ctx, r, grid, lds))))
+            return mfw == 1 ? DH_CONV_RES(1) : (mfw == 2 ? DH_CONV_RES(2) : DH_CONV_RES(4));
+#undef DH_CONV_RES
+        }
+    }
     const size_t gx = dh_ceil_div(pixels, BN);
     if (gx >= (size_t(1) << 31))
         return dh_fail(DH_ERR_RUNTIME, "Convolution: too many output pixels for one launch");

@@ -16,9 +16,10 @@
 // reference there (its test vector is reproduced).
 #pragma once
 
-#include "common.h"
+#include "dnn_impl.h"
 
 #include <cmath>
+#include <type_traits>
 
 namespace dh_train {
 
@@ -659,6 +660,267 @@ template <typename T> static bool conv_backward_data_mfma(dh_ctx *ctx, T *dX, co
     return true;
 }
 
+// ---------------------------------------------------------------------------------------
+// Filter gradient with the image resident in LDS (the forward convolution's layout with the roles swapped):
+//     dW[f][k] = sum over images n and pixels pq of dY[n][f][pq] * patch_n[k][pq],   k = (c, hy, hx)
+// A workgroup of 8 waves keeps 16 * MFW filters x `chunk` filter columns as accumulators of the 16x16x4 matrix
+// instruction for its whole run over the images n = blockIdx.x, blockIdx.x + gridDim.x, ...: per image it copies
+// the padded image into LDS, reads dY rows from global memory (a 16-byte vector of consecutive pixels per lane)
+// and gathers the patch values from LDS at "column offset + pixel offset". Every workgroup leaves one partial
+// F x K slab; a second kernel adds the slabs in order.
+// ---------------------------------------------------------------------------------------
+struct ConvFilterResidentArgs {
+    const void *x;     // N x C x H x W
+    const void *dy;    // N x F x P x Q
+    const int *koff;   // column k -> c*Hp*Wp + hy*Wp + hx, padded with zeros to the columns all chunks cover
+    const int *pixtab; // pixel pq -> p*sh*Wp + q*sw, padded with zeros to PQpad
+    void *slabs;       // [gridDim.x][F][K]
+    unsigned N, C, H, W, Wp, ph, pw, F, K, PQ, PQpad, HpWp, frame, chunk;
+};
+
+static __global__ __launch_bounds__(256) void conv_filter_tables_kernel(int *koff, int *pixtab, unsigned K, unsigned Kcols, unsigned PQ,
+                                                                        unsigned PQpad, unsigned HpWp, unsigned Wp, unsigned Hf,
+                                                                        unsigned Wf, unsigned Q, unsigned sh, unsigned sw) {
+    const unsigned t = blockIdx.x * 256 + threadIdx.x, nt = gridDim.x * 256;
+    for (unsigned k = t; k < Kcols; k += nt) {
+        int off = 0;
+        if (k < K) {
+            const unsigned c = k / (Hf * Wf), hw = k % (Hf * Wf);
+            off = static_cast<int>(c * HpWp + (hw / Wf) * Wp + hw % Wf);
+        }
+        koff[k] = off;
+    }
+    for (unsigned i = t; i < PQpad; i += nt)
+        pixtab[i] = i < PQ ? static_cast<int>((i / Q) * sh * Wp + (i % Q) * sw) : 0;
+}
+
+template <typename T, int MFW, int WAVES, int NF>
+__global__ __launch_bounds__(64 * WAVES) void conv_filter_resident_kernel(ConvFilterResidentArgs g) {
+    using M = dh_gemm::Mfma16<T>;
+    constexpr int VEC = 16 / sizeof(T), NPARTS = WAVES / MFW, NT = 64 * WAVES;
+    static_assert(WAVES % MFW == 0, "waves per filter block");
+    extern __shared__ __attribute__((aligned(16))) unsigned char conv_lds[];
+    int *pixtab = reinterpret_cast<int *>(conv_lds); // PQpad entries: a multiple of 16 bytes
+    T *frame = reinterpret_cast<T *>(conv_lds + g.PQpad * sizeof(int));
+    const int tid = threadIdx.x, lane = tid % 64, wave = __builtin_amdgcn_readfirstlane(tid / 64);
+    const unsigned f0 = blockIdx.y * (16 * MFW), col0 = blockIdx.z * g.chunk;
+    for (unsigned i = tid; i < g.PQpad; i += NT)
+        pixtab[i] = g.pixtab[i];
+
+    const int mf = wave % MFW, part = wave / MFW;
+    const int li = lane % 16, lk = lane / 16;
+    // this lane's filter column in each of the wave's column blocks (dealt round-robin over the waves)
+    int koffs[NF];
+    int nfv = 0;
+#pragma unroll
+    for (int j = 0; j < NF; j++) {
+        const unsigned first = col0 + (j * NPARTS + part) * 16;
+        koffs[j] = g.koff[first + li];
+        if (first < g.K)
+            nfv = j + 1;
+    }
+    typename M::acc_t acc[NF];
+#pragma unroll
+    for (int j = 0; j < NF; j++)
+        acc[j] = typename M::acc_t{0, 0, 0, 0};
+
+    const unsigned frow = f0 + mf * 16 + li;
+    const bool rowok = frow < g.F;
+    const T *dy = static_cast<const T *>(g.dy);
+    const int *pixl = pixtab + lk * VEC;
+
+    for (unsigned img = blockIdx.x; img < g.N; img += gridDim.x) {
+        __syncthreads(); // every wave is done with the previous image
+        dh_dnn::conv_stage_frame<T>(frame, static_cast<const T *>(g.x) + static_cast<size_t>(img) * g.C * g.H * g.W, g.C, g.H, g.W,
+                                    g.Wp, g.ph, g.pw, g.HpWp, g.frame, tid, NT);
+        __syncthreads();
+        const T *arow = dy + (static_cast<size_t>(img) * g.F + (rowok ? frow : 0)) * g.PQ + lk * VEC;
+        // dY values of pixel block q0 for this lane; lanes past the row end (or past F) read the tensor's first
+        // vector instead and are zeroed when the values are taken into use
+        auto a_ok = [&](unsigned q0) { return rowok && q0 + lk * VEC < g.PQ; };
+        auto contract = [&](auto nv_tag) {
+            constexpr int NV = decltype(nv_tag)::value;
+            // dY comes from HBM: its vectors are asked for two pixel blocks ahead
+            T a_cur[VEC], a_nxt[VEC], b_cur[NV];
+            int pt[VEC];
+            const unsigned q1 = (4 * VEC < g.PQpad) ? 4 * VEC : 0;
+            bool ok_nxt = a_ok(q1);
+            {
+                const bool ok = a_ok(0);
+                dh_load_vec<T, VEC>(ok ? arow : dy, a_cur);
+                dh_load_vec<T, VEC>(ok_nxt ? arow + q1 : dy, a_nxt);
+#pragma unroll
+                for (int s_ = 0; s_ < VEC; s_++)
+                    a_cur[s_] = ok ? a_cur[s_] : T(0);
+            }
+#pragma unroll
+            for (int s_ = 0; s_ < VEC; s_++)
+                pt[s_] = pixl[s_];
+#pragma unroll
+            for (int j = 0; j < NV; j++)
+                b_cur[j] = frame[koffs[j] + pt[0]];
+            for (unsigned q0 = 0; q0 < g.PQpad; q0 += 4 * VEC) {
+                const unsigned qn = (q0 + 4 * VEC < g.PQpad) ? q0 + 4 * VEC : q0;
+                const unsigned qnn = (q0 + 8 * VEC < g.PQpad) ? q0 + 8 * VEC : q0;
+                const bool ok_nn = a_ok(qnn);
+                T a_nn[VEC];
+                int pt_nxt[VEC];
+                dh_load_vec<T, VEC>(ok_nn ? arow + qnn : dy, a_nn);
+#pragma unroll
+                for (int s_ = 0; s_ < VEC; s_++)
+                    pt_nxt[s_] = pixl[qn + s_];
+#pragma unroll
+                for (int s_ = 0; s_ < VEC; s_++) {
+                    const int pt_after = (s_ + 1 < VEC) ? pt[s_ + 1] : pt_nxt[0];
+                    T b_nxt[NV];
+#pragma unroll
+                    for (int j = 0; j < NV; j++)
+                        b_nxt[j] = frame[koffs[j] + pt_after];
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int j = 0; j < NV; j++)
+                        acc[j] = M::mma(a_cur[s_], b_cur[j], acc[j]);
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int j = 0; j < NV; j++)
+                        b_cur[j] = b_nxt[j];
+                }
+#pragma unroll
+                for (int s_ = 0; s_ < VEC; s_++) {
+                    a_cur[s_] = ok_nxt ? a_nxt[s_] : T(0);
+                    a_nxt[s_] = a_nn[s_];
+                    pt[s_] = pt_nxt[s_];
+                }
+                ok_nxt = ok_nn;
+            }
+        };
+        if (nfv == NF - 1)
+            contract(std::integral_constant<int, NF - 1>{});
+        else if (nfv > 0)
+            contract(std::integral_constant<int, NF>{});
+    }
+
+    T *slab = static_cast<T *>(g.slabs) + static_cast<size_t>(blockIdx.x) * g.F * g.K;
+#pragma unroll
+    for (int j = 0; j < NF; j++) {
+        const unsigned col = col0 + (j * NPARTS + part) * 16 + li;
+        if (j < nfv && col < g.K) {
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                const unsigned f = f0 + mf * 16 + M::row(lane, v);
+                if (f < g.F)
+                    slab[static_cast<size_t>(f) * g.K + col] = acc[j][v];
+            }
+        }
+    }
+}
+
+// res[i] = slabs[0][i] + slabs[1][i] + ... in slab order
+template <typename T> __global__ __launch_bounds__(THREADS) void slab_sum_kernel(T *res, const T *slabs, unsigned nslabs, size_t n) {
+    const size_t i = static_cast<size_t>(blockIdx.x) * THREADS + threadIdx.x;
+    if (i >= n)
+        return;
+    T sum = T(0);
+    unsigned z = 0;
+    for (; z + 4 <= nslabs; z += 4) {
+        const T a0 = slabs[z * n + i], a1 = slabs[(z + 1) * n + i], a2 = slabs[(z + 2) * n + i], a3 = slabs[(z + 3) * n + i];
+        sum = (((sum + a0) + a1) + a2) + a3;
+    }
+    for (; z < nslabs; z++)
+        sum += slabs[z * n + i];
+    res[i] = sum;
+}
+
+template <typename T, int MFW, int WAVES, int NF>
+static inline dh_status conv_filter_resident_launch(dh_ctx *ctx, const ConvFilterResidentArgs &g, dim3 grid, size_t lds) {
+    static size_t allowed = 0; // dynamic LDS beyond 64 KiB has to be asked for once per kernel
+    if (lds > 65536 && lds > allowed) {
+        DH_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&conv_filter_resident_kernel<T, MFW, WAVES, NF>),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
+        allowed = lds;
+    }
+    hipLaunchKernelGGL((conv_filter_resident_kernel<T, MFW, WAVES, NF>), grid, dim3(64 * WAVES), lds, ctx->stream, g);
+    DH_CHECK_LAUNCH();
+    return DH_OK;
+}
+
+template <typename T> static bool conv_backward_filter_resident(dh_ctx *ctx, T *dW, const T *input, const T *dY, const ConvBwdArgs &g, dh_status *st) {
+    constexpr int VEC = 16 / sizeof(T);
+    constexpr size_t NFMAX = 13; // column blocks per wave: 13 accumulator blocks and their operands fit 2 waves per SIMD
+    const size_t PQ = static_cast<size_t>(g.P) * g.Q, K = static_cast<size_t>(g.C) * g.Hf * g.Wf;
+    const size_t Hp = g.H + 2 * g.padh, Wp = g.W + 2 * g.padw, frame = g.C * Hp * Wp;
+    const size_t PQpad = dh_ceil_div(PQ, static_cast<size_t>(4 * VEC)) * (4 * VEC);
+    const size_t lds = PQpad * sizeof(int) + frame * sizeof(T);
+    const int mfw = g.F <= 16 ? 1 : (g.F <= 32 ? 2 : 4);
+    const size_t waves = 8;
+    const size_t parts = waves / mfw, fgroups = dh_ceil_div(static_cast<size_t>(g.F), static_cast<size_t>(16 * mfw));
+    const size_t blocks16 = dh_ceil_div(K, 16);
+    const size_t chunks = dh_ceil_div(blocks16, parts * NFMAX);
+    const size_t nf = dh_ceil_div(blocks16, parts * chunks);
+    const size_t chunk = parts * nf * 16;
+    if (PQ % VEC != 0 || !dh_aligned(dY, 16) || lds > 150 * 1024 || nf < 3 || PQ < 32 || static_cast<size_t>(g.N) * PQ < 4096 ||
+        fgroups >= 65536 || chunks >= 65536 || frame >= (size_t(1) << 31))
+        return false;
+    // up to 7 column blocks per wave take few enough registers for two workgroups per CU, LDS permitting
+    const size_t per_cu = (nf <= 7 && lds <= 80 * 1024) ? 2 : 1;
+    size_t groups = static_cast<size_t>(ctx->num_cus) * per_cu / (fgroups * chunks);
+    if (groups < 1)
+        groups = 1;
+    if (groups > g.N)
+        groups = g.N;
+    const size_t kcols = chunks * chunk;
+    void *tabs = nullptr, *slabs = nullptr;
+    *st = dh_malloc(ctx, (kcols + PQpad) * sizeof(int), 0, &tabs);
+    if (*st != DH_OK)
+        return true;
+    *st = dh_malloc(ctx, groups * g.F * K * sizeof(T), 0, &slabs);
+    if (*st != DH_OK) {
+        dh_free(ctx, tabs);
+        return true;
+    }
+    int *koff = static_cast<int *>(tabs), *pixtab = koff + kcols;
+    hipLaunchKernelGGL(conv_filter_tables_kernel, dim3(static_cast<unsigned>(dh_ceil_div(kcols + PQpad, 256))), dim3(256), 0, ctx->stream,
+                       koff, pixtab, static_cast<unsigned>(K), static_cast<unsigned>(kcols), static_cast<unsigned>(PQ),
+                       static_cast<unsigned>(PQpad), static_cast<unsigned>(Hp * Wp), static_cast<unsigned>(Wp), g.Hf, g.Wf, g.Q, g.sh, g.sw);
+    ConvFilterResidentArgs r{};
+    r.x = input;
+    r.dy = dY;
+    r.koff = koff;
+    r.pixtab = pixtab;
+    r.slabs = slabs;
+    r.N = g.N;
+    r.C = g.C;
+    r.H = g.H;
+    r.W = g.W;
+    r.Wp = static_cast<unsigned>(Wp);
+    r.ph = g.padh;
+    r.pw = g.padw;
+    r.F = g.F;
+    r.K = static_cast<unsigned>(K);
+    r.PQ = static_cast<unsigned>(PQ);
+    r.PQpad = static_cast<unsigned>(PQpad);
+    r.HpWp = static_cast<unsigned>(Hp * Wp);
+    r.frame = static_cast<unsigned>(frame);
+    r.chunk = static_cast<unsigned>(chunk);
+    const dim3 grid(static_cast<unsigned>(groups), static_cast<unsigned>(fgroups), static_cast<unsigned>(chunks));
+#define DH_CONV_FILTER_NF(MFW_, WAVES_)                                                                                   \
+    (nf <= 7 ? conv_filter_resident_launch<T, MFW_, WAVES_, 7>(ctx, r, grid, lds)                                         \
+             : (nf <= 10 ? conv_filter_resident_launch<T, MFW_, WAVES_, 10>(ctx, r, grid, lds)                            \
+                         : conv_filter_resident_launch<T, MFW_, WAVES_, 13>(ctx, r, grid, lds)))
+#define DH_CONV_FILTER_RES(MFW_) DH_CONV_FILTER_NF(MFW_, 8)
+    *st = mfw == 1 ? DH_CONV_FILTER_RES(1) : (mfw == 2 ? DH_CONV_FILTER_RES(2) : DH_CONV_FILTER_RES(4));
+#undef DH_CONV_FILTER_RES
+#undef DH_CONV_FILTER_NF
+    if (*st == DH_OK) {
+        const size_t n = static_cast<size_t>(g.F) * K;
+        hipLaunchKernelGGL((slab_sum_kernel<T>), dim3(blocks_for(n)), dim3(THREADS), 0, ctx->stream, dW, static_cast<const T *>(slabs),
+                           static_cast<unsigned>(groups), n);
+    }
+    dh_free(ctx, tabs);
+    dh_free(ctx, slabs);
+    return true;
+}
+
 template <typename T> static bool conv_backward_filter_mfma(dh_ctx *ctx, T *dW, const T *input, const T *dY, const ConvBwdArgs &g, dh_status *st) {
     const size_t L = static_cast<size_t>(g.N) * g.P * g.Q, Kp = static_cast<size_t>(g.C) * g.Hf * g.Wf;
     const size_t patch_elems = L * Kp, a_elems = static_cast<size_t>(g.F) * L;
@@ -721,6 +983,8 @@ dh_status conv2d_backward_filter(dh_ctx *ctx, T *dW, const T *input, const T *dY
         return DH_OK;
     if (F * C >= (size_t(1) << 31))
         return dh_fail(DH_ERR_RUNTIME, "Conv2D backward - too many filter planes for one launch");
+    if (use_mfma && conv_backward_filter_resident<T>(ctx, dW, input, dY, g, &st))
+        return st;
     if (use_mfma && conv_backward_filter_mfma<T>(ctx, dW, input, dY, g, &st))
         return st;
     hipLaunchKernelGGL((conv_backward_filter_kernel<T, 16>), dim3(static_cast<unsigned>(F * C)), dim3(THREADS), 0, ctx->stream, dW,
