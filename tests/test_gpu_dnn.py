@@ -31,6 +31,14 @@ CONV_CASES = [  # N, C, H, W, F, Hf, Wf, sh, sw, ph, pw
     (2, 7, 20, 9, 33, 4, 2, 1, 1, 0, 0),
     (1, 40, 15, 15, 16, 3, 3, 1, 1, 1, 1),
     (7, 3, 13, 11, 5, 3, 3, 1, 1, 1, 1),
+    # shapes for the kernel that keeps the image in LDS: pixel chunks (1600 pixels, 13 blocks a wave), three channel
+    # stages, a partial last stage (26 + 25 channels in float, 17 x 3 in double), 8 filters on a large image (one
+    # filter block per workgroup, 8 pixel parts), stride 2 with 20 filters (two filter blocks, 4 pixel parts)
+    (2, 6, 40, 40, 64, 3, 3, 1, 1, 1, 1),
+    (2, 96, 14, 14, 32, 5, 5, 1, 1, 2, 2),
+    (2, 51, 14, 14, 48, 4, 4, 1, 1, 1, 1),
+    (2, 4, 32, 32, 8, 3, 3, 1, 1, 1, 1),
+    (1, 5, 30, 30, 20, 3, 3, 2, 2, 0, 0),
 ]
 
 

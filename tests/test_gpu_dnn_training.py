@@ -93,7 +93,12 @@ def test_pooling_backward_all_negative_window_goes_to_the_padding(ctx):
                                   # large enough for the matrix-core paths (frame + forward convolution, patch matrix + GEMM)
                                   (64, 8, 12, 12, 6, 3, 3, 1, 1, 1, 1), (64, 4, 16, 16, 8, 5, 5, 2, 2, 2, 2),
                                   (48, 6, 15, 13, 5, 3, 2, 1, 2, 0, 1), (40, 3, 28, 28, 7, 5, 5, 1, 1, 2, 2),
-                                  (96, 5, 12, 12, 3, 2, 2, 3, 3, 1, 1)])
+                                  (96, 5, 12, 12, 3, 2, 2, 3, 3, 1, 1),
+                                  # filter gradient with the image resident in LDS: two column chunks of 13 blocks a wave;
+                                  # 20 filters (two filter blocks, 4 column parts); 70 filters (two groups) with stride 2;
+                                  # 8 filters (one filter block, 8 column parts)
+                                  (24, 32, 14, 14, 64, 5, 5, 1, 1, 2, 2), (32, 16, 12, 12, 20, 3, 3, 1, 1, 1, 1),
+                                  (20, 24, 31, 31, 70, 3, 3, 2, 2, 1, 1), (17, 48, 16, 16, 8, 3, 3, 1, 1, 1, 1)])
 def test_conv_backward(ctx, dt, case):
     N, C, H, W, F, Hf, Wf, sh, sw, ph, pw = case
     rng = np.random.default_rng(sum(case))
