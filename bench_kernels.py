@@ -171,7 +171,7 @@ def main() -> int:
             w2 = DM.from_torch(ctx, torch.randn(64, 800, device="cuda", dtype=tdt, generator=gen) * 0.05)
             b2 = DM.from_torch(ctx, torch.randn(64, 1, device="cuda", dtype=tdt, generator=gen) * 0.1)
             o2 = DM(ctx, N, 64 * 196, ndt)
-            emit("conv2dForward 32->64 ch, 14x14, 5x5 pad 2 (incl. border copy)", dt, f"batch {N}",
+            emit("conv2dForward 32->64 ch, 14x14, 5x5 pad 2 (image resident in LDS)", dt, f"batch {N}",
                  timed(lambda: K.conv2dForward(o2, x2, w2, b2, N, 32, 14, 14, 5, 5, 1, 1, 2, 2, ctx)), flops=2.0 * N * 64 * 196 * 800)
             emit("biasAdd 64 channels", dt, f"{N}x{64 * 196}", timed(lambda: K.biasAdd(o2, o2, b2, ctx)), 2 * N * 64 * 196 * sz)
             one = DM.from_torch(ctx, torch.ones(64, 1, device="cuda", dtype=tdt))
@@ -222,7 +222,7 @@ def main() -> int:
             fl = 2.0 * Nc * 64 * 196 * 800
             emit("conv2DBackwardData 64->32 ch, 14x14, 5x5 pad 2 (frame + rotated filters + forward convolution)", dt, f"batch {Nc}",
                  timed(lambda: K.conv2DBackwardData(wc, dyc, 1, 1, 2, 2, Nc, 32, 14, 14, 64, 32, 5, 5, dxc, ctx)), flops=fl)
-            emit("conv2DBackwardFilter 32->64 ch, 14x14, 5x5 pad 2 (patch matrix + split-K GEMM)", dt, f"batch {Nc}",
+            emit("conv2DBackwardFilter 32->64 ch, 14x14, 5x5 pad 2 (image resident in LDS, slabs per workgroup)", dt, f"batch {Nc}",
                  timed(lambda: K.conv2DBackwardFilter(dwc, xc, dyc, 1, 1, 2, 2, Nc, 32, 14, 14, 64, 32, 5, 5, ctx)), flops=fl)
             for m in (x, dy, gam, zer, dpool, dxp, xc, wc, dyc, dxc, dwc, *res_bn):
                 m.destroy()

@@ -16,6 +16,10 @@
 // written out: the gather then needs no bounds checks, and with a table k -> offset no divisions,
 // which leaves one scalar add and one load per gathered element. Pixels of all images form one long N dimension, so a
 // tile may span image boundaries and small images still fill the 128-pixel tile.
+//
+// Images of at least a few hundred output pixels take conv2d_resident_kernel instead: the padded image sits in LDS
+// (in stages of channels when it is large), the border is written while it is copied in, and the waves contract
+// over K without a barrier, gathering patch values straight from LDS.
 #pragma once
 
 #include "gemm_impl.h"

@@ -6,9 +6,16 @@
 //
 // Per-channel statistics are deterministic two-stage reductions with double accumulators (every workgroup owns a
 // channel and a slice of the images; a small second kernel folds the slices in order and derives the per-channel
-// coefficients); the elementwise passes use one 16-byte vector per thread where the layout allows. The pooling and
-// convolution gradients are written as gathers - one thread per gradient element, visiting its contributions in the
-// reference's order - so that no atomics are needed and results do not depend on timing.
+// coefficients); the elementwise passes use one 16-byte vector per thread where the layout allows. No kernel uses
+// atomics, so results do not depend on timing:
+//   - pooling gradients are gathers (one thread per gradient element, or per vector of them for 2 x 2 windows),
+//     visiting the contributions in the reference's order;
+//   - the data gradient of a convolution is a forward convolution (stride 1, no border) of the dilated, framed
+//     output gradient with the rotated, axis-swapped filters, on the matrix cores;
+//   - the filter gradient keeps the image in LDS and contracts over images and pixels on the matrix cores
+//     (conv_filter_resident_kernel; partial slabs per workgroup, added in order), or, for shapes that kernel does
+//     not take, builds the patch matrix and calls the split-K GEMM;
+//   - small problems take plain gather kernels (one thread per gradient element).
 //
 // Pooling keeps the forward kernels' quirk of taking the output height from stride_w and the width from stride_h
 // (MaxPoolBackward.h:45-46). Conv2DBackwardData of the reference is only consistent where the output extent equals

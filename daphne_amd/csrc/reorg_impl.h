@@ -94,6 +94,31 @@ __global__ __launch_bounds__(256) void col_bind_kernel(T *res, size_t ld_res, co
     dh_store_vec<T, VEC>(res + r * ld_res + cv * VEC, v);
 }
 
+// The same with the threads numbered through rows x vectors, for row widths that are not a power of two (a thread
+// tile of TX lanes per row would leave lanes idle): one division per thread, 32-bit where the count allows.
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void col_bind_flat_kernel(T *res, size_t ld_res, const T *lhs, size_t ld_lhs, size_t lvecs,
+                                                            const T *rhs, size_t ld_rhs, size_t rvecs, size_t total) {
+    const size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (i >= total)
+        return;
+    const size_t cvecs = lvecs + rvecs;
+    size_t r, cv;
+    if (total <= 0xffffffffull) {
+        r = static_cast<unsigned>(i) / static_cast<unsigned>(cvecs);
+        cv = static_cast<unsigned>(i) % static_cast<unsigned>(cvecs);
+    } else {
+        r = i / cvecs;
+        cv = i % cvecs;
+    }
+    T v[VEC];
+    if (cv < lvecs)
+        dh_load_vec_stream<T, VEC>(lhs + r * ld_lhs + cv * VEC, v);
+    else
+        dh_load_vec_stream<T, VEC>(rhs + r * ld_rhs + (cv - lvecs) * VEC, v);
+    dh_store_vec<T, VEC>(res + r * ld_res + cv * VEC, v);
+}
+
 // ColBind<DenseMatrix<VT>,...>::apply (kernels/ColBind.h:58-91, kernels/CUDA/ColBind.cu:47-70)
 template <typename T>
 dh_status col_bind(dh_ctx *ctx, T *res, size_t ld_res, const T *lhs, size_t lr, size_t lc, size_t ld_lhs, const T *rhs,
@@ -110,6 +135,13 @@ dh_status col_bind(dh_ctx *ctx, T *res, size_t ld_res, const T *lhs, size_t lr, 
                      dh_aligned(res, 16) && dh_aligned(lhs, 16) && dh_aligned(rhs, 16);
     if (vec && lr > 0 && lc + rc > 0) {
         const size_t cvecs = (lc + rc) / V;
+        if ((cvecs & (cvecs - 1)) != 0 && cvecs % 256 != 0 && dh_ceil_div(lr * cvecs, static_cast<size_t>(256)) < (size_t(1) << 31)) {
+            const size_t total = lr * cvecs;
+            hipLaunchKernelGGL((col_bind_flat_kernel<T, V>), dim3(static_cast<unsigned>(dh_ceil_div(total, static_cast<size_t>(256)))),
+                               dim3(256), 0, ctx->stream, res, ld_res, lhs, ld_lhs, lc / V, rhs, ld_rhs, rc / V, total);
+            DH_CHECK_LAUNCH();
+            return DH_OK;
+        }
         unsigned tx = 1;
         while (tx < 256 && tx < cvecs)
             tx <<= 1;
