@@ -681,6 +681,7 @@ dh_status agg_row_idx(dh_ctx *ctx, int op, uint64_t *res, size_t ld_res, const T
 }
 
 constexpr int S2_TX = 16, S2_TY = 16; // second-stage block: columns x partial lanes
+constexpr int V2_TY = 64;             // partial lanes of the variance second stage
 
 // =======================================================================================
 // AggCol
@@ -863,13 +864,13 @@ __global__ __launch_bounds__(THREADS) void col_var_stage1(const T *arg, size_t r
 
 // OUT: 0 variance, 1 stddev, 2 mean (unused by the public API but kept for pipelines).
 template <typename T, int OUT>
-__global__ __launch_bounds__(THREADS) void col_var_stage2(const T *part_mean, const T *part_m2, size_t nparts,
+__global__ __launch_bounds__(S2_TX * V2_TY) void col_var_stage2(const T *part_mean, const T *part_m2, size_t nparts,
                                                           size_t cols, size_t rows, size_t slab, T *res,
                                                           T *res_mean = nullptr) {
-    // (S2_TX columns, S2_TY partial lanes). Pooled moments of the per-block (count, mean, M2) triples in double:
+    // (S2_TX columns, V2_TY partial lanes: 1024 threads, so that a thousand partials take two rounds of loads per pass). Pooled moments of the per-block (count, mean, M2) triples in double:
     //     mean = sum n_p mean_p / N,   M2 = sum M2_p + sum n_p (mean_p - mean)^2
     // - the closed form of merging them pairwise with Chan's formula, without a division per partial.
-    __shared__ double lds_a[S2_TY][S2_TX], lds_b[S2_TY][S2_TX];
+    __shared__ double lds_a[V2_TY][S2_TX], lds_b[V2_TY][S2_TX];
     const size_t c = static_cast<size_t>(blockIdx.x) * S2_TX + threadIdx.x;
     auto count = [&](size_t p) {
         const size_t r_begin = p * slab;
@@ -881,18 +882,18 @@ __global__ __launch_bounds__(THREADS) void col_var_stage2(const T *part_mean, co
     constexpr int UN2 = 8;
     double s1 = 0.0, s2 = 0.0;
     if (c < cols)
-        for (size_t p0 = threadIdx.y; p0 < nparts; p0 += S2_TY * UN2) {
+        for (size_t p0 = threadIdx.y; p0 < nparts; p0 += V2_TY * UN2) {
             T pm[UN2], pq[UN2];
 #pragma unroll
             for (int k = 0; k < UN2; k++) {
-                const size_t p = p0 + static_cast<size_t>(k) * S2_TY;
+                const size_t p = p0 + static_cast<size_t>(k) * V2_TY;
                 const size_t pc = p < nparts ? p : nparts - 1;
                 pm[k] = part_mean[pc * cols + c];
                 pq[k] = part_m2[pc * cols + c];
             }
 #pragma unroll
             for (int k = 0; k < UN2; k++) {
-                const size_t p = p0 + static_cast<size_t>(k) * S2_TY;
+                const size_t p = p0 + static_cast<size_t>(k) * V2_TY;
                 s1 += count(p) * static_cast<double>(pm[k]);
                 s2 += p < nparts ? static_cast<double>(pq[k]) : 0.0;
             }
@@ -901,7 +902,7 @@ __global__ __launch_bounds__(THREADS) void col_var_stage2(const T *part_mean, co
     lds_b[threadIdx.y][threadIdx.x] = s2;
     __syncthreads();
     double tot1 = 0.0, tot2 = 0.0;
-    for (int y = 0; y < S2_TY; y++) {
+    for (int y = 0; y < V2_TY; y++) {
         tot1 += lds_a[y][threadIdx.x];
         tot2 += lds_b[y][threadIdx.x];
     }
@@ -909,17 +910,17 @@ __global__ __launch_bounds__(THREADS) void col_var_stage2(const T *part_mean, co
     __syncthreads();
     double s3 = 0.0;
     if (c < cols)
-        for (size_t p0 = threadIdx.y; p0 < nparts; p0 += S2_TY * UN2) {
+        for (size_t p0 = threadIdx.y; p0 < nparts; p0 += V2_TY * UN2) {
             T pm[UN2];
 #pragma unroll
             for (int k = 0; k < UN2; k++) {
-                const size_t p = p0 + static_cast<size_t>(k) * S2_TY;
+                const size_t p = p0 + static_cast<size_t>(k) * V2_TY;
                 pm[k] = part_mean[(p < nparts ? p : nparts - 1) * cols + c];
             }
 #pragma unroll
             for (int k = 0; k < UN2; k++) {
                 const double d = static_cast<double>(pm[k]) - cmean;
-                s3 += count(p0 + static_cast<size_t>(k) * S2_TY) * d * d;
+                s3 += count(p0 + static_cast<size_t>(k) * V2_TY) * d * d;
             }
         }
     lds_a[threadIdx.y][threadIdx.x] = s3;
@@ -927,7 +928,7 @@ __global__ __launch_bounds__(THREADS) void col_var_stage2(const T *part_mean, co
     if (threadIdx.y != 0 || c >= cols)
         return;
     double cm2 = tot2;
-    for (int y = 0; y < S2_TY; y++)
+    for (int y = 0; y < V2_TY; y++)
         cm2 += lds_a[y][threadIdx.x];
     double v = cm2 / static_cast<double>(rows);
     if constexpr (OUT == 1)
@@ -1177,9 +1178,9 @@ template <typename T> dh_status agg_col(dh_ctx *ctx, int op, T *res, const T *ar
             hipLaunchKernelGGL((col_var_stage1<T, 1>), p.grid, p.block, lds, ctx->stream, arg, rows, p.cvecs, ld, p.slab, pm, pq);
         const dim3 g2(static_cast<unsigned>(dh_ceil_div(cols, S2_TX)));
         if (op == DH_AGG_VAR)
-            hipLaunchKernelGGL((col_var_stage2<T, 0>), g2, dim3(S2_TX, S2_TY), 0, ctx->stream, pm, pq, p.nparts, cols, rows, p.slab, res);
+            hipLaunchKernelGGL((col_var_stage2<T, 0>), g2, dim3(S2_TX, V2_TY), 0, ctx->stream, pm, pq, p.nparts, cols, rows, p.slab, res);
         else
-            hipLaunchKernelGGL((col_var_stage2<T, 1>), g2, dim3(S2_TX, S2_TY), 0, ctx->stream, pm, pq, p.nparts, cols, rows, p.slab, res);
+            hipLaunchKernelGGL((col_var_stage2<T, 1>), g2, dim3(S2_TX, V2_TY), 0, ctx->stream, pm, pq, p.nparts, cols, rows, p.slab, res);
         break;
     }
     default:
@@ -1220,10 +1221,10 @@ dh_status agg_col_moments(dh_ctx *ctx, T *res_mean, T *res_var, int stddev, cons
         hipLaunchKernelGGL((col_var_stage1<T, 1>), p.grid, p.block, lds, ctx->stream, arg, rows, p.cvecs, ld, p.slab, pm, pq);
     const dim3 g2(static_cast<unsigned>(dh_ceil_div(cols, S2_TX)));
     if (stddev)
-        hipLaunchKernelGGL((col_var_stage2<T, 1>), g2, dim3(S2_TX, S2_TY), 0, ctx->stream, pm, pq, p.nparts, cols, rows, p.slab,
+        hipLaunchKernelGGL((col_var_stage2<T, 1>), g2, dim3(S2_TX, V2_TY), 0, ctx->stream, pm, pq, p.nparts, cols, rows, p.slab,
                            res_var, res_mean);
     else
-        hipLaunchKernelGGL((col_var_stage2<T, 0>), g2, dim3(S2_TX, S2_TY), 0, ctx->stream, pm, pq, p.nparts, cols, rows, p.slab,
+        hipLaunchKernelGGL((col_var_stage2<T, 0>), g2, dim3(S2_TX, V2_TY), 0, ctx->stream, pm, pq, p.nparts, cols, rows, p.slab,
                            res_var, res_mean);
     DH_CHECK_LAUNCH();
     return DH_OK;

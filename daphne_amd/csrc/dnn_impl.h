@@ -285,6 +285,7 @@ struct ConvResidentArgs {
     void *res;
     unsigned C, H, W, Hp, Wp, ph, pw, Q, sh, sw, F, Kpad, HpWp, PQ, chunk;
     unsigned CG, KG;   // channels per stage of the LDS image and their share of K (a multiple of the K block)
+    unsigned N, NI;    // images in all, images per workgroup (their pixels form one pixel range)
 };
 
 // Copies one image (C x H x W at x) into LDS as C x Hp x Wp with the zero border of Padding.h:11-22 written out,
@@ -353,7 +354,9 @@ __global__ __launch_bounds__(512) void conv2d_resident_kernel(ConvResidentArgs g
     int *ktab = reinterpret_cast<int *>(conv_lds);               // Kpad entries: a multiple of 16 bytes
     T *frame = reinterpret_cast<T *>(conv_lds + g.Kpad * sizeof(int));
     const int tid = threadIdx.x, lane = tid % 64, wave = __builtin_amdgcn_readfirstlane(tid / 64);
-    const unsigned img = blockIdx.x, f0 = blockIdx.y * (16 * MFW), px0 = blockIdx.z * g.chunk;
+    const unsigned img = blockIdx.x * g.NI, f0 = blockIdx.y * (16 * MFW), px0 = blockIdx.z * g.chunk;
+    const unsigned nimg = (g.N - img < g.NI) ? g.N - img : g.NI; // images of this workgroup
+    const unsigned npix = nimg * g.PQ, stage_elems = g.CG * g.HpWp;
 
     for (unsigned k = tid; k < g.Kpad; k += 512)
         ktab[k] = g.ktab[k];
@@ -367,11 +370,12 @@ __global__ __launch_bounds__(512) void conv2d_resident_kernel(ConvResidentArgs g
     for (int j = 0; j < NF; j++) {
         const unsigned first = px0 + (j * NPARTS + part) * 16; // blocks dealt round-robin: the waves' counts differ by at most one
         const unsigned px = first + li;
-        const bool ok = px < g.PQ;
-        const unsigned pp = ok ? px / g.Q : 0, qq = ok ? px % g.Q : 0;
-        pixoff[j] = static_cast<int>(pp * g.sh * g.Wp + qq * g.sw);
-        outoff[j] = ok ? static_cast<int>(px) : -1;
-        if (first < g.PQ)
+        const bool ok = px < npix;
+        const unsigned il = ok ? px / g.PQ : 0, pq = ok ? px % g.PQ : 0; // image of the workgroup, pixel in it
+        const unsigned pp = pq / g.Q, qq = pq % g.Q;
+        pixoff[j] = static_cast<int>(il * stage_elems + pp * g.sh * g.Wp + qq * g.sw);
+        outoff[j] = ok ? static_cast<int>(il * g.F * g.PQ + pq) : -1;
+        if (first < npix)
             nfv = j + 1;
     }
     typename M::acc_t acc[NF];
@@ -436,8 +440,9 @@ __global__ __launch_bounds__(512) void conv2d_resident_kernel(ConvResidentArgs g
         const unsigned k_end = (c0 + g.CG < g.C) ? k_begin + g.KG : g.Kpad;
         if (c0)
             __syncthreads(); // every wave is done with the previous stage
-        conv_stage_frame<T>(frame, ximg + static_cast<size_t>(c0) * g.H * g.W, cg, g.H, g.W, g.Wp, g.ph, g.pw, g.HpWp,
-                            cg * g.HpWp, tid, 512);
+        for (unsigned il = 0; il < nimg; il++)
+            conv_stage_frame<T>(frame + il * stage_elems, ximg + (static_cast<size_t>(il) * g.C + c0) * g.H * g.W, cg, g.H, g.W,
+                                g.Wp, g.ph, g.pw, g.HpWp, cg * g.HpWp, tid, 512);
         __syncthreads();
         const int sub = static_cast<int>(c0 * g.HpWp);
         if (nfv == NF - 1)
@@ -514,25 +519,42 @@ dh_status conv2d_forward(dh_ctx *ctx, T *res, size_t *res_h, size_t *res_w, cons
         // least three blocks of 16 pixels (smaller images leave the waves idle; they take the tiled kernel below).
         const int mfw = F <= 16 ? 1 : (F <= 32 ? 2 : 4);
         const size_t parts = 8 / mfw;
-        const size_t blocks16 = dh_ceil_div(P * Q, 16);
         const size_t kpad = dh_ceil_div(K, BK) * BK;
-        // channels per stage: the whole image if it takes no more than 48 KiB (three workgroups per CU), else the
-        // fewest equal stages that do, provided a stage's share of K is a whole number of K blocks
-        size_t cg = C;
-        if (C * Hp * Wp * sizeof(T) > 48 * 1024) {
-            const size_t stages = dh_ceil_div(C * Hp * Wp * sizeof(T), static_cast<size_t>(44 * 1024));
-            const size_t per = dh_ceil_div(C, stages);
-            if (per >= 1 && (per * Hf * Wf) % BK == 0)
-                cg = per;
-        }
-        const size_t lds = kpad * sizeof(int) + cg * Hp * Wp * sizeof(T);
+        const size_t plane_bytes = Hp * Wp * sizeof(T);
+        // LDS for the images of a stage so that three workgroups fit a CU (160 KiB) beside their offset tables
+        const size_t budget = kpad * sizeof(int) + 16 * 1024 < 52 * 1024 ? 52 * 1024 - kpad * sizeof(int) : 16 * 1024;
+        // Channels per stage for `imgs` images per workgroup: all of them if that fits the budget, else the fewest
+        // equal stages that do and whose share of K is a whole number of K blocks; failing that, all channels in
+        // one stage as long as LDS holds them at all (one workgroup per CU). 0: nothing fits.
+        auto channels_per_stage = [&](size_t imgs) -> size_t {
+            if (imgs * C * plane_bytes <= budget)
+                return C;
+            for (size_t stages = dh_ceil_div(imgs * C * plane_bytes, budget); stages <= C; stages++) {
+                const size_t per = dh_ceil_div(C, stages);
+                if ((per * Hf * Wf) % BK == 0 && imgs * per * plane_bytes <= budget)
+                    return per;
+            }
+            return imgs * C * plane_bytes + kpad * sizeof(int) <= 150 * 1024 ? C : 0;
+        };
+        // images per workgroup: one if that gives every wave six blocks of 16 pixels, else as many as do (at most 16)
+        size_t ni = dh_ceil_div(6 * parts * 16, P * Q);
+        if (ni > 16)
+            ni = 16;
+        if (ni > N)
+            ni = N;
+        size_t cg = channels_per_stage(ni);
+        while (cg == 0 && ni > 1)
+            cg = channels_per_stage(--ni);
+        const size_t blocks16 = dh_ceil_div(ni * P * Q, 16);
+        const size_t lds = kpad * sizeof(int) + ni * cg * plane_bytes;
         const size_t fgroups = dh_ceil_div(F, static_cast<size_t>(16 * mfw));
         const size_t chunks = dh_ceil_div(blocks16, parts * 13);            // at most 13 blocks per wave
         const size_t nf = dh_ceil_div(blocks16, parts * chunks);            // spread evenly over the chunks
         const size_t chunk = parts * nf * 16;
+        const size_t igroups = dh_ceil_div(N, ni);
         // One workgroup per CU (more than 80 KiB of LDS) has nothing to cover its loading phase and its LDS
         // latencies with: taken only when a wave has at least six blocks of matrix instructions per step.
-        if (lds <= 150 * 1024 && (lds <= 80 * 1024 || nf >= 6) && blocks16 >= 3 * parts && K >= 32 && fgroups < 65536 &&
+        if (cg != 0 && lds <= 150 * 1024 && (lds <= 80 * 1024 || nf >= 6) && blocks16 >= 3 * parts && K >= 32 && fgroups < 65536 &&
             chunks < 65536) {
             const size_t fpad = fgroups * 16 * mfw;
             const size_t tab_bytes = dh_ceil_div(kpad * sizeof(int), 256) * 256;
@@ -571,9 +593,11 @@ dh_status conv2d_forward(dh_ctx *ctx, T *res, size_t *res_h, size_t *res_w, cons
             r.HpWp = static_cast<unsigned>(Hp * Wp);
             r.CG = static_cast<unsigned>(cg);
             r.KG = static_cast<unsigned>(cg * Hf * Wf);
+            r.N = static_cast<unsigned>(N);
+            r.NI = static_cast<unsigned>(ni);
             r.PQ = static_cast<unsigned>(P * Q);
             r.chunk = static_cast<unsigned>(chunk);
-            const dim3 grid(static_cast<unsigned>(N), static_cast<unsigned>(fgroups), static_cast<unsigned>(chunks));
+            const dim3 grid(static_cast<unsigned>(igroups), static_cast<unsigned>(fgroups), static_cast<unsigned>(chunks));
 #define DH_CONV_RES(MFW_)                                                                          \
     (nf <= 4 ? conv2d_resident_launch<T, MFW_, 4>(ctx, r, grid, lds)                               \
              : (nf <= 7 ? conv2d_resident_launch<T, MFW_, 7>(ctx, r, grid, lds)                    \

@@ -39,6 +39,11 @@ CONV_CASES = [  # N, C, H, W, F, Hf, Wf, sh, sw, ph, pw
     (2, 51, 14, 14, 48, 4, 4, 1, 1, 1, 1),
     (2, 4, 32, 32, 8, 3, 3, 1, 1, 1, 1),
     (1, 5, 30, 30, 20, 3, 3, 2, 2, 0, 0),
+    # small feature maps: several images per workgroup (8 + 1 of 7 x 7, 12 + 8 of 4 x 4, 3 + 3 + 1 without a border and
+    # in four channel stages)
+    (9, 16, 7, 7, 32, 3, 3, 1, 1, 1, 1),
+    (20, 8, 4, 4, 64, 3, 3, 1, 1, 1, 1),
+    (7, 64, 14, 14, 32, 5, 5, 1, 1, 0, 0),
 ]
 
 
