@@ -325,6 +325,17 @@ template <typename T> dh_status agg_all(dh_ctx *ctx, int op, const T *arg, size_
 // =======================================================================================
 // AggRow
 // =======================================================================================
+// n / b for a divisor b that stays the same over many divisions, r = 1 / b computed once: the product n * r
+// corrected by its exactly computed residual (one fused multiply-add for the residual, one for the correction),
+// which yields the correctly rounded quotient of normal operands in three instructions instead of a full
+// division sequence. Infinite and NaN numerators keep the product (their residual is NaN).
+template <typename T> __device__ __forceinline__ T div_by_constant(T n, T b, T r) {
+    const T q0 = n * r;
+    const T e = __builtin_fma(-b, q0, n);
+    const T q1 = __builtin_fma(e, r, q0);
+    return (e == e) ? q1 : q0;
+}
+
 // FINAL: 0 plain reduction, 1 mean, 2 var, 3 stddev. G lanes share a row (G a power of two
 // <= 64, G divides 64). NANFIRST: MIN/MAX take a NaN in column 0 as the result (AggRow.h:108).
 template <typename T, int VEC, class R, int FINAL, bool NANFIRST>
@@ -345,6 +356,7 @@ __global__ __launch_bounds__(THREADS) void row_kernel(T *res, size_t ld_res, con
     const size_t rows_per_step = static_cast<size_t>(GPW) * UR;
     const size_t wave_id = static_cast<size_t>(blockIdx.x) * (THREADS / DH_WAVE) + tid / DH_WAVE;
     const size_t wave_stride = static_cast<size_t>(gridDim.x) * (THREADS / DH_WAVE) * rows_per_step;
+    const T ncols = static_cast<T>(cols), rcols = T(1) / ncols;
     for (size_t base = wave_id * rows_per_step; base < rows; base += wave_stride) {
         const T *row[UR];
 #pragma unroll
@@ -387,8 +399,12 @@ __global__ __launch_bounds__(THREADS) void row_kernel(T *res, size_t ld_res, con
         });
         if constexpr (FINAL >= 1) {
 #pragma unroll
-            for (int u = 0; u < UR; u++)
-                acc[u] = acc[u] / static_cast<T>(cols);
+            for (int u = 0; u < UR; u++) {
+                if constexpr (agg_is_int<T>)
+                    acc[u] = acc[u] / ncols;
+                else
+                    acc[u] = div_by_constant<T>(acc[u], ncols, rcols);
+            }
         }
         if constexpr (FINAL >= 2) {
             T s[UR];
@@ -427,7 +443,10 @@ __global__ __launch_bounds__(THREADS) void row_kernel(T *res, size_t ld_res, con
             });
 #pragma unroll
             for (int u = 0; u < UR; u++) {
-                s[u] = s[u] / static_cast<T>(cols);
+                if constexpr (agg_is_int<T>)
+                    s[u] = s[u] / ncols;
+                else
+                    s[u] = div_by_constant<T>(s[u], ncols, rcols);
                 acc[u] = (FINAL == 3) ? dev_sqrt<T>(s[u]) : s[u];
             }
         }

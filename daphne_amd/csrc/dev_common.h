@@ -88,7 +88,7 @@ template <typename T> __device__ __forceinline__ T dh_shfl_xor(T v, int mask) { 
 // Butterfly all-reduce over aligned groups of G lanes (G a power of two <= 64): step(peer) is called
 // once per level, and peer(v) returns the value v of this lane's partner at that level. Below 16
 // lanes the partner is the lane's image under a quad swap or a mirror of the 8 / 16 lanes around it
-// (one register move), above it is lane ^ 16 / lane ^ 32 (through the LDS crossbar). Each level pairs
+// (one register move), above it is lane ^ 16 / lane ^ 32 (a swap of 16-lane rows between two registers). Each level pairs
 // the two halves of a block that the previous levels have made uniform, so after the last one every
 // lane of a group holds the combination of the whole group - provided the combine is commutative.
 // Partners are always in the same group: a group must be wholly active or wholly inactive.
@@ -97,6 +97,32 @@ template <int CTRL> struct dh_peer_dpp {
 };
 template <int OFF> struct dh_peer_xor {
     template <typename T> __device__ __forceinline__ T operator()(T v) const { return __shfl_xor(v, OFF, DH_WAVE); }
+};
+// lane ^ 16 (ROWS = 16) or lane ^ 32 (ROWS = 32) by the row-swap instructions of gfx950: with both operands equal,
+// v_permlane16_swap / v_permlane32_swap leave the partner's value in the first result for lanes of the upper rows
+// and in the second for lanes of the lower rows - one ALU instruction and a select instead of a trip through LDS.
+template <int ROWS> struct dh_peer_swap {
+    static __device__ __forceinline__ unsigned word(unsigned w, bool upper) {
+        if constexpr (ROWS == 16) {
+            const auto r = __builtin_amdgcn_permlane16_swap(w, w, false, false);
+            return upper ? r[0] : r[1];
+        } else {
+            const auto r = __builtin_amdgcn_permlane32_swap(w, w, false, false);
+            return upper ? r[0] : r[1];
+        }
+    }
+    template <typename T> __device__ __forceinline__ T operator()(T v) const {
+        static_assert(sizeof(T) == 4 || sizeof(T) == 8, "32-bit or 64-bit values only");
+        const unsigned lane = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+        const bool upper = (lane & ROWS) != 0;
+        if constexpr (sizeof(T) == 4) {
+            return __builtin_bit_cast(T, word(__builtin_bit_cast(unsigned, v), upper));
+        } else {
+            const unsigned long long b = __builtin_bit_cast(unsigned long long, v);
+            const unsigned lo = word(static_cast<unsigned>(b), upper), hi = word(static_cast<unsigned>(b >> 32), upper);
+            return __builtin_bit_cast(T, (static_cast<unsigned long long>(hi) << 32) | lo);
+        }
+    }
 };
 template <class Step> __device__ __forceinline__ void dh_butterfly(int G, Step &&step) {
     if (G >= 2)
@@ -108,9 +134,9 @@ template <class Step> __device__ __forceinline__ void dh_butterfly(int G, Step &
     if (G >= 16)
         step(dh_peer_dpp<0x140>{}); // row_mirror: lane i of 16 <-> 15 - i
     if (G >= 32)
-        step(dh_peer_xor<16>{});
+        step(dh_peer_swap<16>{});
     if (G >= 64)
-        step(dh_peer_xor<32>{});
+        step(dh_peer_swap<32>{});
 }
 template <typename T> __device__ __forceinline__ T dh_shfl_down(T v, int d) { return __shfl_down(v, d, DH_WAVE); }
 
