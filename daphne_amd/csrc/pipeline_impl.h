@@ -22,7 +22,12 @@ void jit_set_last_mode(int m);
 // four independent accumulators; the association is fixed by the partial count alone.
 constexpr int STAGE2_THREADS = 1024;
 template <typename T>
-__global__ __launch_bounds__(STAGE2_THREADS) void pipeline_all_stage2(const T *partials, size_t np, int op, T *out) {
+__global__ __launch_bounds__(STAGE2_THREADS) void pipeline_all_stage2(const T *partials_all, size_t np_all, size_t chunk, int op,
+                                                                      T *out) {
+    // workgroup b folds the partials [b * chunk, (b + 1) * chunk) into out[b]
+    const size_t begin = static_cast<size_t>(blockIdx.x) * chunk;
+    const T *partials = partials_all + begin;
+    const size_t np = (begin + chunk < np_all) ? chunk : np_all - begin;
     __shared__ T lds[STAGE2_THREADS / DH_WAVE];
     constexpr int UN = 16;
     const T id = (op == DH_AGG_SUM) ? T(0) : (op == DH_AGG_MIN) ? dh_inf<T>() : -dh_inf<T>();
@@ -57,7 +62,7 @@ __global__ __launch_bounds__(STAGE2_THREADS) void pipeline_all_stage2(const T *p
     if (threadIdx.x == 0) {
         for (int w = 1; w < STAGE2_THREADS / DH_WAVE; w++)
             a = comb(a, lds[w]);
-        out[0] = a;
+        out[blockIdx.x] = a;
     }
 }
 
@@ -92,6 +97,7 @@ dh_status run(dh_ctx *ctx, const dh_pipe_instr *prog, int n, const IO_C *cio, si
     }
     constexpr int V = 16 / sizeof(T);
     bool vec_ok = (cols % V == 0) && (io.ld_x % V == 0) && dh_aligned(io.x, 16);
+    bool rowvec_used[4] = {false, false, false, false};
     bool checks = false;
     int reduce_ops[2] = {-1, -1};
     T *reduce_out[2] = {nullptr, nullptr};
@@ -115,6 +121,8 @@ dh_status run(dh_ctx *ctx, const dh_pipe_instr *prog, int n, const IO_C *cio, si
             case DH_OPD_ROWVEC:
                 if (in.domain != 0 || bad_index() || io.rowvec[idx] == nullptr)
                     return dh_fail(DH_ERR_RUNTIME, "vectorizedPipeline: instruction %d: row-vector operand %d is not bound", i, idx);
+                vec_ok = vec_ok && dh_aligned(io.rowvec[idx], 16);
+                rowvec_used[idx] = true;
                 break;
             case DH_OPD_COLVEC:
                 if (bad_index() || io.colvec[idx] == nullptr || io.ld_colvec[idx] < 1)
@@ -164,6 +172,9 @@ dh_status run(dh_ctx *ctx, const dh_pipe_instr *prog, int n, const IO_C *cio, si
             return dh_fail(DH_ERR_RUNTIME, "vectorizedPipeline: instruction %d: unknown kind %d", i, in.kind);
         }
     }
+    for (int k = 0; k < 4; k++)
+        if (!rowvec_used[k])
+            io.rowvec[k] = nullptr; // the kernel loads every bound row vector
     PipeShape sh;
     if (!pipe_shape(cols, vec_ok ? V : 1, &sh))
         return dh_fail(DH_ERR_RUNTIME,
@@ -172,15 +183,19 @@ dh_status run(dh_ctx *ctx, const dh_pipe_instr *prog, int n, const IO_C *cio, si
                        cols, 64 * (vec_ok ? V : 1) * 4);
     const int vec = sh.vec, G = sh.G, KV = sh.KV, U = sh.U, S = sh.S;
     const size_t groups_per_block = THREADS / G;
-    // One run of S = 4 steps per wavefront wherever the grid can express it. Measured on the 20M x 64 z-score
-    // body (kernel alone): S = 1 1.05-1.25 ms (set-up and the workgroup fold per 16 rows of a wavefront), S = 2 0.89,
-    // S = 4 0.83-0.86, S = 8 0.85-0.86, S = 16 0.94; S = 4 on a grid capped at 64 workgroups per CU 0.89.
+    // One run of S steps per wavefront wherever the grid can express it (S from pipe_shape: one step for float
+    // rows, four for double). A wavefront asks for its first tile before the operand vectors, so that the
+    // values it derives from them once are computed under the tile's latency; with that, the shortest
+    // wavefronts do best for float (6.4 TB/s on the 20M x 64 z-score body).
     size_t grid = dh_ceil_div(rows, groups_per_block * U * S);
     const size_t cap = 0x7fffffffull;
     if (grid > cap)
         grid = cap;
     void *wsv = nullptr;
-    dh_status st = dh_workspace(ctx, 2 * grid * sizeof(T) + 256, &wsv);
+    // one partial per wavefront and REDUCE_ALL slot, then room for the first of two folding rounds
+    const size_t np = grid * (THREADS / DH_WAVE);
+    constexpr size_t FOLD_BLOCKS = 64;
+    dh_status st = dh_workspace(ctx, (2 * np + 2 * FOLD_BLOCKS) * sizeof(T) + 256, &wsv);
     if (st != DH_OK)
         return st;
     T *partials = static_cast<T *>(wsv);
@@ -226,7 +241,20 @@ dh_status run(dh_ctx *ctx, const dh_pipe_instr *prog, int n, const IO_C *cio, si
     DH_CHECK_LAUNCH();
     for (int s = 0; s < 2; s++)
         if (reduce_ops[s] != -1) {
-            hipLaunchKernelGGL((pipeline_all_stage2<T>), dim3(1), dim3(STAGE2_THREADS), 0, ctx->stream, partials + s * grid, grid,
+            const T *src = partials + s * np;
+            size_t count = np;
+            if (np > 4 * static_cast<size_t>(STAGE2_THREADS) * 16) {
+                // many partials: 64 workgroups fold a contiguous share each, one workgroup folds their results
+                T *mid = partials + 2 * np + s * FOLD_BLOCKS;
+                const size_t chunk = dh_ceil_div(np, FOLD_BLOCKS);
+                const size_t blocks = dh_ceil_div(np, chunk);
+                hipLaunchKernelGGL((pipeline_all_stage2<T>), dim3(static_cast<unsigned>(blocks)), dim3(STAGE2_THREADS), 0, ctx->stream, src,
+                                   np, chunk, reduce_ops[s], mid);
+                DH_CHECK_LAUNCH();
+                src = mid;
+                count = blocks;
+            }
+            hipLaunchKernelGGL((pipeline_all_stage2<T>), dim3(1), dim3(STAGE2_THREADS), 0, ctx->stream, src, count, count,
                                reduce_ops[s], reduce_out[s]);
             DH_CHECK_LAUNCH();
         }

@@ -189,10 +189,9 @@ struct RuntimeProgram {
 // specialisation passes cols, G and S as literals, so that everything derived from them folds.
 template <typename T, int VEC, int KV, class PG>
 __device__ __forceinline__ void pipeline_body(const Program &P, const PipeIO<T> &io, size_t rows, size_t cols, int G, int S,
-                                                           T *all_partials /* [2][gridDim.x] */, int *flag) {
+                                                           T *all_partials /* [2][gridDim.x * waves per workgroup] */, int *flag) {
     constexpr int U = 4 / KV;
     constexpr int N = U * KV * VEC;
-    __shared__ T lds_red[2][THREADS / DH_WAVE];
 
     const int tid = threadIdx.x;
     const int lane = tid % G;
@@ -228,17 +227,48 @@ __device__ __forceinline__ void pipeline_body(const Program &P, const PipeIO<T> 
 #pragma unroll
         for (int j = 0; j < KV; j++)
             xoff[u][j] = static_cast<size_t>(u * GPW + g_in_wave) * io.ld_x + coff[j];
+    // The tile of a step: U rows x KV vectors per lane, every load unconditional (rows past the end read the
+    // step's first row; their values are never stored, reduced or domain-checked).
+    auto load_tile = [&](size_t base, T (&t)[N]) {
+        const T *xbase = io.x + base * io.ld_x; // the step's first row, which always exists
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const bool live_u = base + static_cast<size_t>(u * GPW + g_in_wave) < rows;
+#pragma unroll
+            for (int j = 0; j < KV; j++) {
+                T x[VEC];
+                dh_load_vec_stream<T, VEC>(xbase + (live_u ? xoff[u][j] : coff[j]), x);
+#pragma unroll
+                for (int e = 0; e < VEC; e++)
+                    t[(u * KV + j) * VEC + e] = x[e];
+            }
+        }
+    };
+    // The wavefront's first tile is asked for before the operand vectors: what the steps derive from those
+    // vectors once (reciprocals of a divisor, for one) is then computed while the tile is on its way, instead
+    // of holding the first loads back by a memory round trip.
+    const size_t first_base = wave_id * rows_per_run;
+    T t_first[N];
+    load_tile(first_base < rows ? first_base : 0, t_first); // unconditional: a wavefront without rows reads row 0 in vain
     // this lane's share of every bound row-vector operand lives in registers for the whole kernel
     T rv0[KV * VEC], rv1[KV * VEC], rv2[KV * VEC], rv3[KV * VEC];
+    // (loaded without a branch: an operand that is not bound reads the first row of X instead and becomes zero;
+    // bound ones are 16-byte aligned whenever VEC > 1, which the launch checks)
+    auto load_rowvec = [&](const T *p, T (&rv)[KV * VEC]) {
+        const T *q = p ? p : io.x;
 #pragma unroll
-    for (int j = 0; j < KV; j++)
+        for (int j = 0; j < KV; j++) {
+            T x[VEC];
+            dh_load_vec<T, VEC>(q + coff[j], x);
 #pragma unroll
-        for (int e = 0; e < VEC; e++) {
-            rv0[j * VEC + e] = io.rowvec[0] ? io.rowvec[0][coff[j] + e] : T(0);
-            rv1[j * VEC + e] = io.rowvec[1] ? io.rowvec[1][coff[j] + e] : T(0);
-            rv2[j * VEC + e] = io.rowvec[2] ? io.rowvec[2][coff[j] + e] : T(0);
-            rv3[j * VEC + e] = io.rowvec[3] ? io.rowvec[3][coff[j] + e] : T(0);
+            for (int e = 0; e < VEC; e++)
+                rv[j * VEC + e] = p ? x[e] : T(0);
         }
+    };
+    load_rowvec(io.rowvec[0], rv0);
+    load_rowvec(io.rowvec[1], rv1);
+    load_rowvec(io.rowvec[2], rv2);
+    load_rowvec(io.rowvec[3], rv3);
 
     // running values of the (at most two) REDUCE_ALL slots, and which combine they use
     T all_acc0 = T(0), all_acc1 = T(0);
@@ -251,13 +281,8 @@ __device__ __forceinline__ void pipeline_body(const Program &P, const PipeIO<T> 
         a = (op == DH_AGG_SUM) ? a + v : (op == DH_AGG_MIN) ? ((v < a) ? v : a) : ((a < v) ? v : a);
     };
 
-    for (size_t run = wave_id; run * rows_per_run < rows; run += n_waves)
-#pragma unroll 1
-    for (int sstep = 0; sstep < S; sstep++) {
-        const size_t base = run * rows_per_run + static_cast<size_t>(sstep) * rows_per_step;
-        if (base >= rows)
-            break;
-        T t[N], o[N], r[U];
+    auto run_step = [&](size_t base, T (&t)[N]) {
+        T o[N], r[U];
         size_t row[U], lrow[U]; // lrow: row index for loads, clamped to the last row
         bool live[U];
 #pragma unroll
@@ -267,17 +292,6 @@ __device__ __forceinline__ void pipeline_body(const Program &P, const PipeIO<T> 
             lrow[u] = live[u] ? row[u] : rows - 1;
             r[u] = T(0);
         }
-        const T *xbase = io.x + base * io.ld_x; // the step's first row, which always exists
-#pragma unroll
-        for (int u = 0; u < U; u++)
-#pragma unroll
-            for (int j = 0; j < KV; j++) {
-                T x[VEC];
-                dh_load_vec_stream<T, VEC>(xbase + (live[u] ? xoff[u][j] : coff[j]), x);
-#pragma unroll
-                for (int e = 0; e < VEC; e++)
-                    t[(u * KV + j) * VEC + e] = x[e];
-            }
         #pragma unroll(PG::is_const ? PG::N : 1)
         for (int ip = 0; ip < (PG::is_const ? PG::N : P.n); ip++) {
             const dh_pipe_instr ins = PG::get(P, ip);
@@ -545,9 +559,24 @@ __device__ __forceinline__ void pipeline_body(const Program &P, const PipeIO<T> 
             }
             }
         }
+    };
+    // The first step uses the tile asked for above; the later ones (step k of the wavefront: step k % S of its
+    // run k / S) load theirs. Bases grow with k, so the first one past the end ends the walk.
+    if (first_base < rows) {
+        run_step(first_base, t_first);
+#pragma unroll 1
+        for (unsigned k = 1;; k++) {
+            const size_t base = (wave_id + static_cast<size_t>(k / static_cast<unsigned>(S)) * n_waves) * rows_per_run +
+                                static_cast<size_t>(k % static_cast<unsigned>(S)) * rows_per_step;
+            if (base >= rows)
+                break;
+            T t[N];
+            load_tile(base, t);
+            run_step(base, t);
+        }
     }
 
-    // block-level fold of the REDUCE_ALL slots
+    // wave-level fold of the REDUCE_ALL slots
     #pragma unroll(PG::is_const ? PG::N : 1)
     for (int ip = 0; ip < (PG::is_const ? PG::N : P.n); ip++) {
         const dh_pipe_instr ins = PG::get(P, ip);
@@ -563,17 +592,10 @@ __device__ __forceinline__ void pipeline_body(const Program &P, const PipeIO<T> 
             const T ov = peer(a);
             a = (op == DH_AGG_SUM) ? a + ov : (op == DH_AGG_MIN) ? ((ov < a) ? ov : a) : ((a < ov) ? ov : a);
         });
+        // one partial per wavefront: no workgroup fold, so a wavefront retires without waiting for the others
         if ((tid % DH_WAVE) == 0)
-            lds_red[slot][tid / DH_WAVE] = a;
-        __syncthreads();
-        if (tid == 0) {
-            for (int w = 1; w < THREADS / DH_WAVE; w++) {
-                const T ov = lds_red[slot][w];
-                a = (op == DH_AGG_SUM) ? a + ov : (op == DH_AGG_MIN) ? ((ov < a) ? ov : a) : ((a < ov) ? ov : a);
-            }
-            all_partials[static_cast<size_t>(slot) * gridDim.x + blockIdx.x] = a;
-        }
-        __syncthreads();
+            all_partials[static_cast<size_t>(slot) * gridDim.x * (THREADS / DH_WAVE) +
+                         static_cast<size_t>(blockIdx.x) * (THREADS / DH_WAVE) + tid / DH_WAVE] = a;
     }
     if (any_bad)
         *flag = 1;
