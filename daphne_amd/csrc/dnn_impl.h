@@ -292,7 +292,7 @@ struct ConvResidentArgs {
 // by the nt threads of a workgroup. A thread keeps its position(s) inside the padded plane and walks the
 // channels, so the divisions are done once; planes of fewer than nt elements are taken by several groups of
 // threads side by side.
-template <typename T>
+template <typename T, int UN>
 __device__ __forceinline__ void conv_stage_frame(T *frame, const T *x, unsigned C, unsigned H, unsigned W, unsigned Wp,
                                                  unsigned ph, unsigned pw, unsigned HpWp, unsigned frame_elems, int tid,
                                                  unsigned nt) {
@@ -300,17 +300,17 @@ __device__ __forceinline__ void conv_stage_frame(T *frame, const T *x, unsigned 
     const unsigned HW = H * W;
     if (ph == 0 && pw == 0 && frame_elems % VEC == 0 && reinterpret_cast<size_t>(x) % 16 == 0) {
         // no border: the frame is the image, copied with 16-byte vectors, four loads of a thread in flight at once
-        constexpr int UN = 4;
+        constexpr int UV = 4;
         const unsigned nvec = frame_elems / VEC;
-        for (unsigned v0 = tid; v0 < nvec; v0 += nt * UN) {
-            T t[UN][VEC];
+        for (unsigned v0 = tid; v0 < nvec; v0 += nt * UV) {
+            T t[UV][VEC];
 #pragma unroll
-            for (int u = 0; u < UN; u++) {
+            for (int u = 0; u < UV; u++) {
                 const unsigned v = v0 + u * nt;
                 dh_load_vec_stream<T, VEC>(x + static_cast<size_t>(v < nvec ? v : v0) * VEC, t[u]);
             }
 #pragma unroll
-            for (int u = 0; u < UN; u++)
+            for (int u = 0; u < UV; u++)
                 if (v0 + u * nt < nvec)
                     dh_store_vec<T, VEC>(frame + static_cast<size_t>(v0 + u * nt) * VEC, t[u]);
         }
@@ -324,17 +324,16 @@ __device__ __forceinline__ void conv_stage_frame(T *frame, const T *x, unsigned 
     for (unsigned r = narrow ? tid % HpWp : tid; r < HpWp; r += nt) {
         const unsigned y = r / Wp - ph, xx = r % Wp - pw; // wraps to a huge value inside the border
         const bool in = y < H && xx < W;
-        const T *src = x + (in ? y * W + xx : 0);
+        const unsigned src = in ? y * W + xx : 0; // 32-bit offsets from the image: one register per load in flight
         T *dst = frame + r;
         // batches of UN channels: all loads of a batch are issued (unconditionally, from clamped addresses) before
         // the first value is stored; lanes on the border load the image's first element and store zeros
-        constexpr int UN = 16;
         for (unsigned c0 = grp; c0 < C; c0 += groups * UN) {
             T v[UN];
 #pragma unroll
             for (int u = 0; u < UN; u++) {
                 const unsigned c = c0 + u * groups;
-                v[u] = __builtin_nontemporal_load(src + static_cast<size_t>(c < C ? c : c0) * HW);
+                v[u] = __builtin_nontemporal_load(x + (src + (c < C ? c : c0) * HW));
             }
 #pragma unroll
             for (int u = 0; u < UN; u++) {
@@ -358,8 +357,15 @@ __global__ __launch_bounds__(512) void conv2d_resident_kernel(ConvResidentArgs g
     const unsigned nimg = (g.N - img < g.NI) ? g.N - img : g.NI; // images of this workgroup
     const unsigned npix = nimg * g.PQ, stage_elems = g.CG * g.HpWp;
 
-    for (unsigned k = tid; k < g.Kpad; k += 512)
-        ktab[k] = g.ktab[k];
+    // the offset table: its first 2048 entries are asked for now and put into LDS after the first image stage has
+    // been copied in, so that both sets of loads are on their way together
+    constexpr int KTR = 4;
+    int ktreg[KTR];
+#pragma unroll
+    for (int i = 0; i < KTR; i++) {
+        const unsigned k = tid + i * 512;
+        ktreg[i] = g.ktab[k < g.Kpad ? k : 0];
+    }
 
     const int mf = wave % MFW, part = wave / MFW;
     const int li = lane % 16, lk = lane / 16;
@@ -441,8 +447,16 @@ __global__ __launch_bounds__(512) void conv2d_resident_kernel(ConvResidentArgs g
         if (c0)
             __syncthreads(); // every wave is done with the previous stage
         for (unsigned il = 0; il < nimg; il++)
-            conv_stage_frame<T>(frame + il * stage_elems, ximg + (static_cast<size_t>(il) * g.C + c0) * g.H * g.W, cg, g.H, g.W,
+            conv_stage_frame<T, 8>(frame + il * stage_elems, ximg + (static_cast<size_t>(il) * g.C + c0) * g.H * g.W, cg, g.H, g.W,
                                 g.Wp, g.ph, g.pw, g.HpWp, cg * g.HpWp, tid, 512);
+        if (c0 == 0) {
+#pragma unroll
+            for (int i = 0; i < KTR; i++)
+                if (tid + i * 512 < g.Kpad)
+                    ktab[tid + i * 512] = ktreg[i];
+            for (unsigned k = tid + KTR * 512; k < g.Kpad; k += 512)
+                ktab[k] = g.ktab[k];
+        }
         __syncthreads();
         const int sub = static_cast<int>(c0 * g.HpWp);
         if (nfv == NF - 1)
@@ -554,6 +568,8 @@ dh_status conv2d_forward(dh_ctx *ctx, T *res, size_t *res_h, size_t *res_w, cons
         const size_t igroups = dh_ceil_div(N, ni);
         // One workgroup per CU (more than 80 KiB of LDS) has nothing to cover its loading phase and its LDS
         // latencies with: taken only when a wave has at least six blocks of matrix instructions per step.
+        // With K < 32 (one or two K blocks) the output stores dominate, and the tiled kernel below writes longer
+        // runs: 1 -> 32 channels, 5 x 5 on 28 x 28 takes 0.16 ms there and 0.28 ms here.
         if (cg != 0 && lds <= 150 * 1024 && (lds <= 80 * 1024 || nf >= 6) && blocks16 >= 3 * parts && K >= 32 && fgroups < 65536 &&
             chunks < 65536) {
             const size_t fpad = fgroups * 16 * mfw;

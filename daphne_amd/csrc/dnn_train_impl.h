@@ -738,7 +738,7 @@ __global__ __launch_bounds__(64 * WAVES) void conv_filter_resident_kernel(ConvFi
 
     for (unsigned img = blockIdx.x; img < g.N; img += gridDim.x) {
         __syncthreads(); // every wave is done with the previous image
-        dh_dnn::conv_stage_frame<T>(frame, static_cast<const T *>(g.x) + static_cast<size_t>(img) * g.C * g.H * g.W, g.C, g.H, g.W,
+        dh_dnn::conv_stage_frame<T, 32>(frame, static_cast<const T *>(g.x) + static_cast<size_t>(img) * g.C * g.H * g.W, g.C, g.H, g.W,
                                     g.Wp, g.ph, g.pw, g.HpWp, g.frame, tid, NT);
         __syncthreads();
         const T *arow = dy + (static_cast<size_t>(img) * g.F + (rowok ? frow : 0)) * g.PQ + lk * VEC;
