@@ -910,6 +910,7 @@ __global__ __launch_bounds__(S2_TX * V2_TY) void col_var_stage2(const T *part_me
                 pm[k] = part_mean[pc * cols + c];
                 pq[k] = part_m2[pc * cols + c];
             }
+            __builtin_amdgcn_sched_barrier(0); // all sixteen loads are issued before the first value is used
 #pragma unroll
             for (int k = 0; k < UN2; k++) {
                 const size_t p = p0 + static_cast<size_t>(k) * V2_TY;

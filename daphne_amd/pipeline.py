@@ -58,6 +58,7 @@ class VectorizedPipeline:
         self._keep: list = [x]
         self._scalars: list[DenseMatrix] = []
         self.domain = 0
+        self._call = None
 
     def _slot(self, what: str, limit: int = MAX_OPERANDS) -> int:
         i = self._n[what]
@@ -70,6 +71,7 @@ class VectorizedPipeline:
         if len(self.instrs) >= MAX_INSTR:
             raise capi.DaphneHipError(1, f"vectorizedPipeline: more than {MAX_INSTR} instructions")
         self.instrs.append(PipeInstr(**kw))
+        self._call = None
 
     # -- operators --------------------------------------------------------------------------
     def ewBinary(self, op, operand: Union[float, str, DenseMatrix], swap: bool = False) -> "VectorizedPipeline":
@@ -146,9 +148,13 @@ class VectorizedPipeline:
         return res
 
     def run(self) -> None:
-        arr = (PipeInstr * max(1, len(self.instrs)))(*self.instrs)
-        suf = "f32" if self.x.dtype == np.float32 else "f64"
-        fn = getattr(capi.lib(), f"dh_vectorized_pipeline_{suf}")
-        fn.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_size_t, C.c_size_t]
-        capi.check(fn(self.ctx._h, C.cast(arr, C.c_void_p), len(self.instrs), C.cast(C.pointer(self.io), C.c_void_p),
-                      self.x.rows, self.x.cols))
+        # the marshalled call is built once per recorded body (recording an operator drops it)
+        call = self._call
+        if call is None or call[0] != len(self.instrs):
+            arr = (PipeInstr * max(1, len(self.instrs)))(*self.instrs)
+            suf = "f32" if self.x.dtype == np.float32 else "f64"
+            fn = getattr(capi.lib(), f"dh_vectorized_pipeline_{suf}")
+            fn.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_size_t, C.c_size_t]
+            call = self._call = (len(self.instrs), fn, arr, C.cast(arr, C.c_void_p), C.cast(C.pointer(self.io), C.c_void_p))
+        _, fn, _, arr_p, io_p = call
+        capi.check(fn(self.ctx._h, arr_p, len(self.instrs), io_p, self.x.rows, self.x.cols))
