@@ -487,11 +487,10 @@ __global__ __launch_bounds__(512) void conv2d_resident_kernel(ConvResidentArgs g
 }
 
 template <typename T, int MFW, int NF> static inline dh_status conv2d_resident_launch(dh_ctx *ctx, const ConvResidentArgs &g, dim3 grid, size_t lds) {
-    static size_t allowed = 0; // dynamic LDS beyond 64 KiB has to be asked for once per kernel
-    if (lds > 65536 && lds > allowed) {
+    // dynamic LDS beyond 64 KiB has to be asked for, per kernel and device (the call is cheap next to the kernel)
+    if (lds > 65536) {
         DH_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&conv2d_resident_kernel<T, MFW, NF>),
                                          hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
-        allowed = lds;
     }
     hipLaunchKernelGGL((conv2d_resident_kernel<T, MFW, NF>), grid, dim3(512), lds, ctx->stream, g);
     DH_CHECK_LAUNCH();
@@ -1140,6 +1139,67 @@ __global__ __launch_bounds__(256) void softmax_reg_kernel(T *res, size_t ld_res,
     }
 }
 
+// Short rows that are no multiple of 8 values (10 classes, say) waste most lanes of a lane group and give every
+// wavefront load a few dozen scattered bytes. For contiguous matrices of such rows a workgroup copies 256 rows into
+// LDS with whole 16-byte vectors, every thread then handles one row there (sequential max, exp and sum as the
+// reference, Softmax.h:36-52), and the rows leave again as whole vectors.
+template <typename T>
+__global__ __launch_bounds__(256) void softmax_lds_kernel(T *res, const T *arg, size_t rows, unsigned cols) {
+    constexpr int VEC = 16 / sizeof(T), UN = 4;
+    extern __shared__ __attribute__((aligned(16))) unsigned char softmax_lds[];
+    T *buf = reinterpret_cast<T *>(softmax_lds); // 256 rows x cols
+    const unsigned tid = threadIdx.x;
+    const size_t r0 = static_cast<size_t>(blockIdx.x) * 256;
+    const unsigned nrows = rows - r0 < 256 ? static_cast<unsigned>(rows - r0) : 256u;
+    const unsigned n = nrows * cols, nvec = n / VEC;
+    const T *src = arg + r0 * cols; // 16-byte aligned: 256 * cols values per workgroup
+    T *dst = res + r0 * cols;
+    for (unsigned v0 = tid; v0 < nvec; v0 += 256 * UN) {
+        T t[UN][VEC];
+#pragma unroll
+        for (int u = 0; u < UN; u++) {
+            const unsigned v = v0 + u * 256;
+            dh_load_vec_stream<T, VEC>(src + static_cast<size_t>(v < nvec ? v : v0) * VEC, t[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < UN; u++)
+            if (v0 + u * 256 < nvec)
+                dh_store_vec<T, VEC>(buf + static_cast<size_t>(v0 + u * 256) * VEC, t[u]);
+    }
+    if (tid < n - nvec * VEC)
+        buf[nvec * VEC + tid] = src[nvec * VEC + tid];
+    __syncthreads();
+    if (tid < nrows) {
+        T *row = buf + tid * cols;
+        // max: NaN anywhere in the row ends up in every output through the sum, as on the CPU
+        T mx = -std::numeric_limits<T>::infinity();
+        for (unsigned c = 0; c < cols; c++) {
+            const T v = row[c];
+            mx = (mx < v) ? v : mx;
+        }
+        const T first = row[0];
+        if (first != first)
+            mx = first;
+        T sum = T(0);
+        for (unsigned c = 0; c < cols; c++) {
+            const T e = dev_exp<T>(row[c] - mx);
+            row[c] = e;
+            sum += e;
+        }
+        const T inv = T(1) / sum;
+        for (unsigned c = 0; c < cols; c++)
+            row[c] *= inv;
+    }
+    __syncthreads();
+    for (unsigned v = tid; v < nvec; v += 256) {
+        T t[VEC];
+        dh_load_vec<T, VEC>(buf + static_cast<size_t>(v) * VEC, t);
+        dh_store_vec_stream<T, VEC>(dst + static_cast<size_t>(v) * VEC, t);
+    }
+    if (tid < n - nvec * VEC)
+        dst[nvec * VEC + tid] = buf[nvec * VEC + tid];
+}
+
 template <typename T>
 dh_status softmax(dh_ctx *ctx, T *res, size_t ld_res, const T *arg, size_t rows, size_t cols, size_t ld) {
     DH_REQUIRE_CTX(ctx);
@@ -1147,6 +1207,13 @@ dh_status softmax(dh_ctx *ctx, T *res, size_t ld_res, const T *arg, size_t rows,
         return dh_fail(DH_ERR_RUNTIME, "Softmax - a leading dimension is smaller than the column count");
     if (rows == 0 || cols == 0)
         return DH_OK;
+    if (cols <= 32 && cols % 8 != 0 && ld == cols && ld_res == cols && dh_aligned(arg, 16) && dh_aligned(res, 16) &&
+        rows >= 1024 && dh_ceil_div(rows, static_cast<size_t>(256)) < (size_t(1) << 31)) {
+        hipLaunchKernelGGL((softmax_lds_kernel<T>), dim3(static_cast<unsigned>(dh_ceil_div(rows, static_cast<size_t>(256)))), dim3(256),
+                           256 * cols * sizeof(T), ctx->stream, res, arg, rows, static_cast<unsigned>(cols));
+        DH_CHECK_LAUNCH();
+        return DH_OK;
+    }
     int G = 1;
     while (G < 64 && static_cast<size_t>(G) < cols)
         G <<= 1;

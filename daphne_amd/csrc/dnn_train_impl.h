@@ -840,11 +840,10 @@ template <typename T> __global__ __launch_bounds__(THREADS) void slab_sum_kernel
 
 template <typename T, int MFW, int WAVES, int NF>
 static inline dh_status conv_filter_resident_launch(dh_ctx *ctx, const ConvFilterResidentArgs &g, dim3 grid, size_t lds) {
-    static size_t allowed = 0; // dynamic LDS beyond 64 KiB has to be asked for once per kernel
-    if (lds > 65536 && lds > allowed) {
+    // dynamic LDS beyond 64 KiB has to be asked for, per kernel and device (the call is cheap next to the kernel)
+    if (lds > 65536) {
         DH_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&conv_filter_resident_kernel<T, MFW, WAVES, NF>),
                                          hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
-        allowed = lds;
     }
     hipLaunchKernelGGL((conv_filter_resident_kernel<T, MFW, WAVES, NF>), grid, dim3(64 * WAVES), lds, ctx->stream, g);
     DH_CHECK_LAUNCH();

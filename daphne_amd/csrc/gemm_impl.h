@@ -388,11 +388,19 @@ template <typename T> __global__ __launch_bounds__(256) void mirror_kernel(T *C,
         return;
     const int tx = threadIdx.x % 64, ty = threadIdx.x / 64;
     const size_t up = static_cast<size_t>(blockIdx.x) * 64, low = static_cast<size_t>(blockIdx.y) * 64;
-#pragma unroll 4
-    for (int i = ty; i < 64; i += 4) {
-        const size_t r = up + i, c = low + tx;
-        if (r < n && c < n)
-            tile[i][tx] = C[r * ldc + c];
+    // sixteen loads per thread, all issued before the first LDS store (a guard around each load would make the
+    // compiler wait for every one in turn): positions past the matrix read its last element, which is never stored
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+        T v[8];
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            const size_t r = up + ty + 4 * (h * 8 + k), c = low + tx;
+            v[k] = C[(r < n ? r : n - 1) * ldc + (c < n ? c : n - 1)];
+        }
+#pragma unroll
+        for (int k = 0; k < 8; k++)
+            tile[ty + 4 * (h * 8 + k)][tx] = v[k];
     }
     __syncthreads();
 #pragma unroll 4

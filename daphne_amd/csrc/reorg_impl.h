@@ -244,12 +244,17 @@ __global__ __launch_bounds__(256) void transpose_kernel(T *res, size_t ld_res, c
     __shared__ T tile[TS][TS + 1];
     const int tx = threadIdx.x % TS, ty = threadIdx.x / TS; // 64 x 4
     const size_t r0 = static_cast<size_t>(blockIdx.x) * TS, c0 = static_cast<size_t>(blockIdx.y) * TS;
+    // all sixteen loads of a thread are issued before the first LDS store (a guard around each load would make the
+    // compiler wait for every one in turn): positions past the matrix read its last element, which is never stored
+    T v[TS / 4];
 #pragma unroll
-    for (int i = 0; i < TS; i += 4) {
-        const size_t r = r0 + ty + i, c = c0 + tx;
-        if (r < rows && c < cols)
-            tile[ty + i][tx] = arg[r * ld + c];
+    for (int k = 0; k < TS / 4; k++) {
+        const size_t r = r0 + ty + 4 * k, c = c0 + tx;
+        v[k] = arg[(r < rows ? r : rows - 1) * ld + (c < cols ? c : cols - 1)];
     }
+#pragma unroll
+    for (int k = 0; k < TS / 4; k++)
+        tile[ty + 4 * k][tx] = v[k];
     __syncthreads();
 #pragma unroll
     for (int i = 0; i < TS; i += 4) {
