@@ -125,8 +125,24 @@ __global__ __launch_bounds__(256) void lu_solve_lds_kernel(T *x_out, const T *A,
     T *xs = prow + n;
     const unsigned tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
     const unsigned tx = tid % 16, ty = tid / 16;
-    for (unsigned e = tid; e < n * n; e += 256)
-        a[(e / n) * ld + e % n] = A[static_cast<size_t>(e / n) * lda + e % n];
+    // copy-in: 16 x 16 threads over (row, column); a thread's loads go out in batches of eight before the first
+    // LDS store (positions past the matrix read its last element and are not stored)
+    for (unsigned r0 = ty; r0 < n; r0 += 16 * 8) {
+        for (unsigned c = tx; c < n; c += 16) {
+            T v[8];
+#pragma unroll
+            for (int k = 0; k < 8; k++) {
+                const unsigned r = r0 + 16 * k;
+                v[k] = A[static_cast<size_t>(r < n ? r : n - 1) * lda + c];
+            }
+#pragma unroll
+            for (int k = 0; k < 8; k++) {
+                const unsigned r = r0 + 16 * k;
+                if (r < n)
+                    a[r * ld + c] = v[k];
+            }
+        }
+    }
     for (unsigned i = tid; i < n; i += 256)
         xs[i] = b[i];
     if (tid == 0)
@@ -144,15 +160,15 @@ __global__ __launch_bounds__(256) void lu_solve_lds_kernel(T *x_out, const T *A,
                     bi = i;
                 }
             }
-#pragma unroll
-            for (int off = 32; off >= 1; off >>= 1) {
-                const T ov = __shfl_xor(best, off);
-                const unsigned oi = __shfl_xor(bi, off);
+            // every lane ends up with the largest value and, among equals, the lowest row
+            dh_butterfly(64, [&](auto peer) {
+                const T ov = peer(best);
+                const unsigned oi = peer(bi);
                 if (ov > best || (ov == best && oi < bi)) {
                     best = ov;
                     bi = oi;
                 }
-            }
+            });
             const unsigned p = bi;
             if (a[p * ld + j] == T(0)) {
                 if (lane == 0) {
