@@ -107,11 +107,12 @@ __global__ __launch_bounds__(SOLVE_THREADS) void lu_solve_kernel(T *lu, T *x, co
     }
 }
 
-// The whole system in LDS. Per column: wave 0 finds the pivot with shuffles, swaps the rows and
-// publishes the pivot row; after one barrier all 256 threads apply the rank-1 update (16 x 16 thread
-// grid, multipliers recomputed per row instead of stored: only U and the eliminated right-hand side
-// are needed afterwards); a second barrier closes the column. Back substitution runs in wave 0 alone,
-// right-hand side in registers, one shuffle per unknown.
+// The whole system in LDS, the right-hand side as column n of the matrix. Per column: wave 0 finds the pivot
+// (register-move reduction), swaps the rows and publishes the pivot row; after one barrier all 256 threads apply
+// the rank-1 update (16 x 16 thread grid, multipliers recomputed per row instead of stored: only U and the
+// eliminated right-hand side are needed afterwards); a second barrier closes the column. Back substitution runs
+// in wave 0 alone, right-hand side in registers, one shuffle per unknown. The kernel clears the singularity flag
+// itself.
 constexpr int LDS_SOLVE_MAX_SLOTS = 3; // rows per lane in the back substitution: n <= 192
 
 template <typename T>
@@ -119,10 +120,9 @@ __global__ __launch_bounds__(256) void lu_solve_lds_kernel(T *x_out, const T *A,
                                                            int *flag) {
     extern __shared__ __attribute__((aligned(16))) unsigned char solve_lds[];
     __shared__ int s_stop;
-    const unsigned ld = n | 1u; // odd stride: column walks spread over the banks
+    const unsigned ld = (n + 1) | 1u; // n + 1 columns; odd stride: column walks spread over the banks
     T *a = reinterpret_cast<T *>(solve_lds);
-    T *prow = a + static_cast<size_t>(n) * ld;
-    T *xs = prow + n;
+    T *prow = a + static_cast<size_t>(n) * ld; // n + 1 entries
     const unsigned tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
     const unsigned tx = tid % 16, ty = tid / 16;
     // copy-in: 16 x 16 threads over (row, column); a thread's loads go out in batches of eight before the first
@@ -144,9 +144,11 @@ __global__ __launch_bounds__(256) void lu_solve_lds_kernel(T *x_out, const T *A,
         }
     }
     for (unsigned i = tid; i < n; i += 256)
-        xs[i] = b[i];
-    if (tid == 0)
+        a[i * ld + n] = b[i];
+    if (tid == 0) {
         s_stop = 0;
+        *flag = 0;
+    }
     __syncthreads();
     for (unsigned j = 0; j < n; j++) {
         if (wave == 0) {
@@ -176,7 +178,7 @@ __global__ __launch_bounds__(256) void lu_solve_lds_kernel(T *x_out, const T *A,
                     s_stop = 1;
                 }
             } else {
-                for (unsigned c = j + lane; c < n; c += 64) {
+                for (unsigned c = j + lane; c <= n; c += 64) {
                     const T pv = a[p * ld + c];
                     prow[c] = pv;
                     if (p != j) {
@@ -184,24 +186,16 @@ __global__ __launch_bounds__(256) void lu_solve_lds_kernel(T *x_out, const T *A,
                         a[j * ld + c] = pv;
                     }
                 }
-                if (lane == 0 && p != j) {
-                    const T t = xs[j];
-                    xs[j] = xs[p];
-                    xs[p] = t;
-                }
             }
         }
         __syncthreads();
         if (s_stop)
             return;
         const T inv = T(1) / prow[j];
-        const T xj = xs[j];
         for (unsigned i = j + 1 + ty; i < n; i += 16) {
             const T l = a[i * ld + j] * inv;
-            for (unsigned c = j + 1 + tx; c < n; c += 16)
+            for (unsigned c = j + 1 + tx; c <= n; c += 16)
                 a[i * ld + c] -= l * prow[c];
-            if (tx == 0)
-                xs[i] -= l * xj;
         }
         __syncthreads();
     }
@@ -212,7 +206,7 @@ __global__ __launch_bounds__(256) void lu_solve_lds_kernel(T *x_out, const T *A,
 #pragma unroll
     for (int s_ = 0; s_ < LDS_SOLVE_MAX_SLOTS; s_++) {
         const unsigned r = lane + 64 * s_;
-        rhs[s_] = r < n ? xs[r] : T(0);
+        rhs[s_] = r < n ? a[r * ld + n] : T(0);
         res[s_] = T(0);
     }
     for (unsigned jj = n; jj-- > 0;) {
@@ -246,8 +240,7 @@ template <typename T> dh_status solve(dh_ctx *ctx, T *x, const T *A, size_t n, s
         return dh_fail(DH_ERR_RUNTIME, "#cols of lhs must match row skip");
     if (n >= (size_t(1) << 15))
         return dh_fail(DH_ERR_RUNTIME, "Solve: systems beyond 32767 unknowns are not supported by this kernel");
-    hipLaunchKernelGGL(clear_flag_kernel, dim3(1), dim3(1), 0, ctx->stream, ctx->flag_dev);
-    const size_t lds_bytes = (n * (n | 1) + 2 * n) * sizeof(T);
+    const size_t lds_bytes = (n * ((n + 1) | 1) + n + 1) * sizeof(T);
     if (n <= 64 * LDS_SOLVE_MAX_SLOTS && lds_bytes <= (size_t(150) << 10)) {
         if (lds_bytes > (size_t(64) << 10)) {
             static std::mutex attr_lock;
@@ -262,6 +255,7 @@ template <typename T> dh_status solve(dh_ctx *ctx, T *x, const T *A, size_t n, s
         hipLaunchKernelGGL((lu_solve_lds_kernel<T>), dim3(1), dim3(256), lds_bytes, ctx->stream, x, A, lda, b,
                            static_cast<unsigned>(n), ctx->flag_dev);
     } else {
+        hipLaunchKernelGGL(clear_flag_kernel, dim3(1), dim3(1), 0, ctx->stream, ctx->flag_dev);
         void *wsv = nullptr;
         dh_status st = dh_workspace(ctx, n * n * sizeof(T), &wsv);
         if (st != DH_OK)
