@@ -9,6 +9,8 @@
 // side) is factored there with two barriers per column; larger ones work in a global scratch copy.
 #include "common.h"
 
+#include <type_traits>
+
 namespace {
 
 constexpr int SOLVE_THREADS = 1024;
@@ -108,15 +110,16 @@ __global__ __launch_bounds__(SOLVE_THREADS) void lu_solve_kernel(T *lu, T *x, co
 }
 
 // The whole system in LDS, the right-hand side as column n of the matrix. Per column: wave 0 finds the pivot
-// (register-move reduction), swaps the rows and publishes the pivot row; after one barrier all 256 threads apply
-// the rank-1 update (16 x 16 thread grid, multipliers recomputed per row instead of stored: only U and the
+// (register-move reduction), swaps the rows and publishes the pivot row; after one barrier all 1024 threads apply
+// the rank-1 update (32 x 32 thread grid, multipliers recomputed per row instead of stored: only U and the
 // eliminated right-hand side are needed afterwards); a second barrier closes the column. Back substitution runs
 // in wave 0 alone, right-hand side in registers, one shuffle per unknown. The kernel clears the singularity flag
 // itself.
 constexpr int LDS_SOLVE_MAX_SLOTS = 3; // rows per lane in the back substitution: n <= 192
+constexpr unsigned LDS_SOLVE_TG = 32;  // the update runs on a TG x TG grid of threads (1024: four waves per SIMD)
 
 template <typename T>
-__global__ __launch_bounds__(256) void lu_solve_lds_kernel(T *x_out, const T *A, size_t lda, const T *b, unsigned n,
+__global__ __launch_bounds__(LDS_SOLVE_TG * LDS_SOLVE_TG) void lu_solve_lds_kernel(T *x_out, const T *A, size_t lda, const T *b, unsigned n,
                                                            int *flag) {
     extern __shared__ __attribute__((aligned(16))) unsigned char solve_lds[];
     __shared__ int s_stop;
@@ -124,26 +127,27 @@ __global__ __launch_bounds__(256) void lu_solve_lds_kernel(T *x_out, const T *A,
     T *a = reinterpret_cast<T *>(solve_lds);
     T *prow = a + static_cast<size_t>(n) * ld; // n + 1 entries
     const unsigned tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
-    const unsigned tx = tid % 16, ty = tid / 16;
-    // copy-in: 16 x 16 threads over (row, column); a thread's loads go out in batches of eight before the first
+    constexpr unsigned TG = LDS_SOLVE_TG;
+    const unsigned tx = tid % TG, ty = tid / TG;
+    // copy-in: TG x TG threads over (row, column); a thread's loads go out in batches of eight before the first
     // LDS store (positions past the matrix read its last element and are not stored)
-    for (unsigned r0 = ty; r0 < n; r0 += 16 * 8) {
-        for (unsigned c = tx; c < n; c += 16) {
+    for (unsigned r0 = ty; r0 < n; r0 += TG * 8) {
+        for (unsigned c = tx; c < n; c += TG) {
             T v[8];
 #pragma unroll
             for (int k = 0; k < 8; k++) {
-                const unsigned r = r0 + 16 * k;
+                const unsigned r = r0 + TG * k;
                 v[k] = A[static_cast<size_t>(r < n ? r : n - 1) * lda + c];
             }
 #pragma unroll
             for (int k = 0; k < 8; k++) {
-                const unsigned r = r0 + 16 * k;
+                const unsigned r = r0 + TG * k;
                 if (r < n)
                     a[r * ld + c] = v[k];
             }
         }
     }
-    for (unsigned i = tid; i < n; i += 256)
+    for (unsigned i = tid; i < n; i += TG * TG)
         a[i * ld + n] = b[i];
     if (tid == 0) {
         s_stop = 0;
@@ -162,14 +166,17 @@ __global__ __launch_bounds__(256) void lu_solve_lds_kernel(T *x_out, const T *A,
                     bi = i;
                 }
             }
-            // every lane ends up with the largest value and, among equals, the lowest row
+            // the largest value first (one instruction per level), then the lowest row among the lanes that hold it
+            T top = best;
             dh_butterfly(64, [&](auto peer) {
-                const T ov = peer(best);
+                const T ov = peer(top);
+                top = ov > top ? ov : top;
+            });
+            if (best != top)
+                bi = 0xffffffffu;
+            dh_butterfly(64, [&](auto peer) {
                 const unsigned oi = peer(bi);
-                if (ov > best || (ov == best && oi < bi)) {
-                    best = ov;
-                    bi = oi;
-                }
+                bi = oi < bi ? oi : bi;
             });
             const unsigned p = bi;
             if (a[p * ld + j] == T(0)) {
@@ -192,10 +199,68 @@ __global__ __launch_bounds__(256) void lu_solve_lds_kernel(T *x_out, const T *A,
         if (s_stop)
             return;
         const T inv = T(1) / prow[j];
-        for (unsigned i = j + 1 + ty; i < n; i += 16) {
-            const T l = a[i * ld + j] * inv;
-            for (unsigned c = j + 1 + tx; c <= n; c += 16)
-                a[i * ld + c] -= l * prow[c];
+        // Rank-1 update of the rows and columns past j, KM rows x (KM + 1) columns per thread. All operands are read
+        // before the first result is written (the compiler must assume that the stores alias the loads, which
+        // would make every element wait for its predecessor): positions past the end read element (n - 1, n).
+        auto update = [&](auto km_tag) {
+            constexpr int KM = decltype(km_tag)::value;
+            T l[KM], pc[KM + 1], v[KM][KM + 1];
+#pragma unroll
+            for (int k = 0; k < KM; k++) {
+                const unsigned i = j + 1 + ty + TG * k;
+                l[k] = a[(i < n ? i : n - 1) * ld + j];
+            }
+#pragma unroll
+            for (int m = 0; m <= KM; m++) {
+                const unsigned c = j + 1 + tx + TG * m;
+                pc[m] = prow[c <= n ? c : n];
+            }
+#pragma unroll
+            for (int k = 0; k < KM; k++)
+#pragma unroll
+                for (int m = 0; m <= KM; m++) {
+                    const unsigned i = j + 1 + ty + TG * k, c = j + 1 + tx + TG * m;
+                    v[k][m] = a[(i < n ? i : n - 1) * ld + (c <= n ? c : n)];
+                }
+#pragma unroll
+            for (int k = 0; k < KM; k++) {
+                const unsigned i = j + 1 + ty + TG * k;
+                const T lk = l[k] * inv;
+#pragma unroll
+                for (int m = 0; m <= KM; m++) {
+                    const unsigned c = j + 1 + tx + TG * m;
+                    if (i < n && c <= n)
+                        a[i * ld + c] = v[k][m] - lk * pc[m];
+                }
+            }
+        };
+        switch ((n - j - 1 + TG - 1) / TG) { // blocks of TG rows left; the columns (one more: the right-hand side) need at most one block more
+        case 0:
+            break;
+        case 1:
+            update(std::integral_constant<int, 1>{});
+            break;
+        case 2:
+            update(std::integral_constant<int, 2>{});
+            break;
+        case 3:
+            update(std::integral_constant<int, 3>{});
+            break;
+        case 4:
+            update(std::integral_constant<int, 4>{});
+            break;
+        case 5:
+            update(std::integral_constant<int, 5>{});
+            break;
+        case 6:
+            update(std::integral_constant<int, 6>{});
+            break;
+        default:
+            for (unsigned i = j + 1 + ty; i < n; i += TG) {
+                const T l = a[i * ld + j] * inv;
+                for (unsigned c = j + 1 + tx; c <= n; c += TG)
+                    a[i * ld + c] -= l * prow[c];
+            }
         }
         __syncthreads();
     }
@@ -252,7 +317,7 @@ template <typename T> dh_status solve(dh_ctx *ctx, T *x, const T *A, size_t n, s
                 attr_set[ctx->device] = true;
             }
         }
-        hipLaunchKernelGGL((lu_solve_lds_kernel<T>), dim3(1), dim3(256), lds_bytes, ctx->stream, x, A, lda, b,
+        hipLaunchKernelGGL((lu_solve_lds_kernel<T>), dim3(1), dim3(LDS_SOLVE_TG * LDS_SOLVE_TG), lds_bytes, ctx->stream, x, A, lda, b,
                            static_cast<unsigned>(n), ctx->flag_dev);
     } else {
         hipLaunchKernelGGL(clear_flag_kernel, dim3(1), dim3(1), 0, ctx->stream, ctx->flag_dev);
