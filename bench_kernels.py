@@ -182,7 +182,7 @@ def main() -> int:
                  timed(lambda: K.maxPoolForward(pl, o2, N, 64, 14, 14, 2, 2, 2, 2, 0, 0, ctx)), 1.25 * N * 64 * 196 * sz)
             emit("avgPoolForward 2x2/2 on 14x14", dt, f"{N}x{64 * 196}",
                  timed(lambda: K.avgPoolForward(pl, o2, N, 64, 14, 14, 2, 2, 2, 2, 0, 0, ctx)), 1.25 * N * 64 * 196 * sz)
-            emit("maxPoolForward 3x3/2 pad 1 on 14x14 (generic kernel)", dt, f"{N}x{64 * 196}",
+            emit("maxPoolForward 3x3/2 pad 1 on 14x14 (planes staged in LDS)", dt, f"{N}x{64 * 196}",
                  timed(lambda: K.maxPoolForward(None, o2, N, 64, 14, 14, 3, 3, 2, 2, 1, 1, ctx)),
                  (1 + 49.0 / 196) * N * 64 * 196 * sz)
             w3 = DM.from_torch(ctx, torch.randn(3136, 512, device="cuda", dtype=tdt, generator=gen) * 0.02)

@@ -729,6 +729,98 @@ __global__ __launch_bounds__(256) void maxpool_kernel(T *res, const T *data, siz
     }
 }
 
+// Pooling over small planes, `ppb` whole planes per workgroup: the planes are contiguous in memory, so
+// the workgroup copies them into LDS with 16-byte loads (batches of four per thread, all issued before
+// the first LDS store) and then gathers every window from LDS; the outputs of the planes are contiguous
+// as well and go out coalesced. Window clipping and arithmetic are those of maxpool_kernel /
+// avgpool_kernel. The host picks ppb so that a workgroup's first element is 16-byte aligned.
+template <typename T, bool AVG>
+__global__ __launch_bounds__(256) void pool_planes_kernel(T *res, const T *data, size_t planes, unsigned ppb, unsigned H,
+                                                          unsigned W, unsigned P, unsigned Q, unsigned ph, unsigned pw,
+                                                          unsigned sh, unsigned sw, unsigned padh, unsigned padw, T plen) {
+#pragma clang fp contract(off)
+    extern __shared__ __attribute__((aligned(16))) unsigned char pool_lds[];
+    T *tile = reinterpret_cast<T *>(pool_lds);
+    constexpr int VEC = 16 / sizeof(T);
+    const unsigned tid = threadIdx.x;
+    const size_t first = static_cast<size_t>(blockIdx.x) * ppb;
+    const size_t left = planes - first;
+    const unsigned here = left < ppb ? static_cast<unsigned>(left) : ppb;
+    const unsigned HW = H * W, PQ = P * Q;
+    const unsigned n_in = here * HW, nvec = n_in / VEC;
+    const T *src = data + first * HW;
+    for (unsigned v0 = 0; v0 < nvec; v0 += 256 * 4) {
+        T r[4][VEC];
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const unsigned i = v0 + tid + 256 * k;
+            dh_load_vec_stream<T, VEC>(src + static_cast<size_t>(i < nvec ? i : nvec - 1) * VEC, r[k]);
+        }
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const unsigned i = v0 + tid + 256 * k;
+            if (i < nvec)
+                dh_store_vec<T, VEC>(tile + static_cast<size_t>(i) * VEC, r[k]);
+        }
+    }
+    for (unsigned i = nvec * VEC + tid; i < n_in; i += 256)
+        tile[i] = src[i];
+    __syncthreads();
+    const unsigned n_out = here * PQ;
+    T *dst = res + first * PQ;
+    for (unsigned o = tid; o < n_out; o += 256) {
+        const unsigned plane = o / PQ, pq = o % PQ;
+        const unsigned p = pq / Q, q = pq % Q;
+        const T *in = tile + plane * HW;
+        const int y_lo = static_cast<int>(p * sh) - static_cast<int>(padh);
+        const int x_lo = static_cast<int>(q * sw) - static_cast<int>(padw);
+        const int y0 = y_lo < 0 ? 0 : y_lo, x0 = x_lo < 0 ? 0 : x_lo;
+        int y1 = y_lo + static_cast<int>(ph), x1 = x_lo + static_cast<int>(pw);
+        if (y1 > static_cast<int>(H))
+            y1 = H;
+        if (x1 > static_cast<int>(W))
+            x1 = W;
+        T acc = T(0);
+        for (int y = y0; y < y1; y++) {
+            if constexpr (AVG) {
+                T s = T(0);
+                for (int x = x0; x < x1; x++)
+                    s = s + in[static_cast<unsigned>(y) * W + static_cast<unsigned>(x)];
+                const T scaled = s * plen;
+                acc = scaled + acc;
+            } else {
+                for (int x = x0; x < x1; x++) {
+                    const T v = in[static_cast<unsigned>(y) * W + static_cast<unsigned>(x)];
+                    acc = (acc < v) ? v : acc; // std::max(acc, v)
+                }
+            }
+        }
+        dst[o] = acc;
+    }
+}
+
+// Planes per workgroup for pool_planes_kernel: about 16 KB of input and a plane count whose elements
+// fill whole 16-byte vectors, so that every workgroup starts on a vector boundary. 0: the planes are
+// too large for this kernel or the input is not aligned.
+template <typename T> inline unsigned pool_planes_per_block(const T *data, size_t HW, size_t planes) {
+    constexpr size_t VEC = 16 / sizeof(T);
+    const size_t target = (16 * 1024) / sizeof(T);
+    if (HW == 0 || HW > target || !dh_aligned(data, 16))
+        return 0;
+    size_t unit = VEC; // smallest plane count with unit * HW % VEC == 0
+    while (unit > 1 && ((unit / 2) * HW) % VEC == 0)
+        unit /= 2;
+    size_t ppb = target / HW;
+    if (ppb >= unit)
+        ppb -= ppb % unit;
+    else if (planes > ppb)
+        return 0;
+    // small inputs: more workgroups before more planes per workgroup
+    while (ppb >= 2 * unit && (ppb / 2) % unit == 0 && dh_ceil_div(planes, ppb) < 2048)
+        ppb /= 2;
+    return static_cast<unsigned>(ppb);
+}
+
 // Non-overlapping 2x2 windows (stride 2, no padding, even H and W): the tensor is a flat list of row
 // pairs [R][2][W] -> [R][W/2]. Each thread loads VI consecutive values of both rows of a pair and
 // writes VI/2 outputs, all as single vector accesses.
@@ -835,6 +927,12 @@ dh_status maxpool_forward(dh_ctx *ctx, T *res, size_t *res_h, size_t *res_w, con
         // value is what the CPU kernel returns for every output.
         hipLaunchKernelGGL((fill_kernel<T>), dim3(static_cast<unsigned>(grid)), dim3(256), 0, ctx->stream, res, total,
                            std::numeric_limits<T>::max());
+    } else if (const unsigned ppb = pool_planes_per_block(data, H * W, N * C); ppb != 0 && dh_ceil_div(N * C, ppb) < (size_t(1) << 31)) {
+        hipLaunchKernelGGL((pool_planes_kernel<T, false>), dim3(static_cast<unsigned>(dh_ceil_div(N * C, ppb))), dim3(256),
+                           ppb * H * W * sizeof(T), ctx->stream, res, data, N * C, ppb, static_cast<unsigned>(H),
+                           static_cast<unsigned>(W), static_cast<unsigned>(P), static_cast<unsigned>(Q),
+                           static_cast<unsigned>(ph), static_cast<unsigned>(pw), static_cast<unsigned>(sh),
+                           static_cast<unsigned>(sw), static_cast<unsigned>(padh), static_cast<unsigned>(padw), T(0));
     } else {
         hipLaunchKernelGGL((maxpool_kernel<T>), dim3(static_cast<unsigned>(grid)), dim3(256), 0, ctx->stream, res, data,
                            total, 0u, static_cast<unsigned>(H), static_cast<unsigned>(W), static_cast<unsigned>(P),
@@ -937,11 +1035,22 @@ dh_status avgpool_forward(dh_ctx *ctx, T *res, size_t *res_h, size_t *res_w, con
         return DH_OK;
     }
     const T plen = T(1) / static_cast<T>(pw * ph); // Pooling.cpp:50
+    const bool quick = P == 1 && Q == 1 && W == 1;
+    if (const unsigned ppb = quick ? 0 : pool_planes_per_block(data, H * W, N * C);
+        ppb != 0 && dh_ceil_div(N * C, ppb) < (size_t(1) << 31)) {
+        hipLaunchKernelGGL((pool_planes_kernel<T, true>), dim3(static_cast<unsigned>(dh_ceil_div(N * C, ppb))), dim3(256),
+                           ppb * H * W * sizeof(T), ctx->stream, res, data, N * C, ppb, static_cast<unsigned>(H),
+                           static_cast<unsigned>(W), static_cast<unsigned>(P), static_cast<unsigned>(Q),
+                           static_cast<unsigned>(ph), static_cast<unsigned>(pw), static_cast<unsigned>(sh),
+                           static_cast<unsigned>(sw), static_cast<unsigned>(padh), static_cast<unsigned>(padw), plen);
+        DH_CHECK_LAUNCH();
+        return DH_OK;
+    }
     hipLaunchKernelGGL((avgpool_kernel<T>), dim3(static_cast<unsigned>(dh_ceil_div(total, 256))), dim3(256), 0, ctx->stream,
                        res, data, total, static_cast<unsigned>(H), static_cast<unsigned>(W), static_cast<unsigned>(P),
                        static_cast<unsigned>(Q), static_cast<unsigned>(ph), static_cast<unsigned>(pw),
                        static_cast<unsigned>(sh), static_cast<unsigned>(sw), static_cast<unsigned>(padh),
-                       static_cast<unsigned>(padw), plen, (P == 1 && Q == 1 && W == 1) ? 1 : 0);
+                       static_cast<unsigned>(padw), plen, quick ? 1 : 0);
     DH_CHECK_LAUNCH();
     return DH_OK;
 }

@@ -116,6 +116,12 @@ POOL_CASES = [  # N, C, H, W, ph, pw, sh, sw, padh, padw
     (2, 2, 9, 7, 3, 2, 3, 3, 0, 0),
     (4, 5, 6, 1, 6, 1, 1, 1, 0, 0),   # P == Q == 1 and W == 1: the reference's quick path
     (1, 1, 4, 4, 4, 4, 1, 1, 0, 0),
+    (333, 64, 14, 14, 3, 3, 2, 2, 1, 1),  # several planes per workgroup staged in LDS, short last workgroup
+    (301, 33, 7, 7, 3, 3, 1, 1, 1, 1),    # planes of 49 values: workgroups of a multiple of four planes, scalar tail
+    (5, 7, 5, 5, 3, 3, 2, 2, 0, 0),
+    (1, 3, 7, 9, 2, 3, 1, 2, 1, 0),       # fewer planes than fill a vector-aligned workgroup
+    (2, 2, 80, 80, 3, 3, 2, 2, 1, 1),     # planes too large for the LDS kernel
+    (2, 3, 64, 64, 5, 5, 3, 3, 2, 2),     # one 16 KB plane per workgroup (float)
 ]
 
 

@@ -170,6 +170,9 @@ POOL = [  # N, C, H, W, ph, pw, sh, sw, padh, padw
     (2, 3, 5, 5, 2, 2, 1, 1, 0, 0), (3, 2, 8, 8, 2, 2, 2, 2, 0, 0), (2, 2, 9, 7, 3, 2, 2, 3, 1, 0), (1, 1, 6, 6, 3, 3, 3, 3, 0, 0),
     (2, 4, 7, 1, 7, 1, 1, 1, 0, 0),    # one output per plane of a one-column image (the quick path)
     (2, 2, 5, 1, 3, 1, 1, 1, 0, 0), (4, 3, 12, 10, 4, 5, 1, 1, 2, 2), (64, 8, 28, 28, 2, 2, 2, 2, 0, 0),
+    (333, 64, 14, 14, 3, 3, 2, 2, 1, 1),   # several planes per workgroup staged in LDS, short last workgroup
+    (301, 33, 7, 7, 3, 3, 1, 1, 1, 1),     # planes of 49 values: a multiple of four planes per workgroup
+    (2, 2, 80, 80, 4, 4, 2, 2, 1, 1),      # planes too large for the LDS kernel
 ]
 
 
