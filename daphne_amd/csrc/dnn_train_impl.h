@@ -35,35 +35,61 @@ constexpr int THREADS = 256;
 // ---------------------------------------------------------------------------------------
 // per-channel reductions
 // ---------------------------------------------------------------------------------------
-// MODE 0: sum x          MODE 1: sum (x - mean[c])^2          MODE 2: sum dy, sum dy*(x - mean[c]), sum (x - mean[c])
+// MODE 2: sum dy, sum dy*(x - mean[c]), sum (x - mean[c])
 // MODE 3: sum (x - s), sum (x - s)^2 with s = the channel's first value: mean and variance from one pass
-template <typename T, int MODE>
+// A workgroup takes one channel of a slice of images. Its threads walk the (image, vector) positions of that channel
+// with a stride of THREADS positions, kept as an (image, vector) pair that is advanced without divisions; four
+// positions are loaded before the first is used, positions past the slice read its last image and count as zero.
+template <typename T, int MODE, int VEC>
 __global__ __launch_bounds__(THREADS) void chan_stage1(const T *x, const T *dy, const T *mean, size_t N, size_t C, size_t HW,
                                                        size_t imgs_per_slice, double *partials /* [C][S][3] */) {
-    constexpr int K = MODE == 2 ? 3 : (MODE == 3 ? 2 : 1);
+    static_assert(MODE == 2 || MODE == 3, "unknown reduction");
+    constexpr int K = MODE == 2 ? 3 : 2;
+    constexpr int UN = 4;
     __shared__ double lds[K][THREADS / DH_WAVE];
     const size_t c = blockIdx.x, s = blockIdx.y;
     const size_t n0 = s * imgs_per_slice, n1 = (n0 + imgs_per_slice < N) ? n0 + imgs_per_slice : N;
     const size_t CHW = C * HW;
-    const double mu = MODE == 3 ? static_cast<double>(x[c * HW]) : (MODE >= 1 ? static_cast<double>(mean[c]) : 0.0);
+    const double mu = MODE == 3 ? static_cast<double>(x[c * HW]) : static_cast<double>(mean[c]);
     double a0 = 0.0, a1 = 0.0, a2 = 0.0;
-    const size_t items = (n1 > n0 ? n1 - n0 : 0) * HW;
-    for (size_t i = threadIdx.x; i < items; i += THREADS) {
-        const size_t n = n0 + i / HW, j = i % HW;
-        const size_t off = n * CHW + c * HW + j;
-        const double v = static_cast<double>(x[off]);
-        if constexpr (MODE == 0) {
-            a0 += v;
-        } else if constexpr (MODE == 1) {
-            a0 += (v - mu) * (v - mu);
-        } else if constexpr (MODE == 3) {
-            a0 += v - mu;
-            a1 += (v - mu) * (v - mu);
-        } else {
-            const double g = static_cast<double>(dy[off]);
-            a0 += g;
-            a1 += g * (v - mu);
-            a2 += v - mu;
+    const size_t imgs = n1 > n0 ? n1 - n0 : 0;
+    if (imgs > 0) {
+        const size_t cvecs = HW / VEC;
+        const size_t dn = THREADS / cvecs, dj = THREADS % cvecs; // one stride, as images and vectors
+        size_t n = threadIdx.x / cvecs, j = threadIdx.x % cvecs;
+        const T *xc = x + n0 * CHW + c * HW;
+        const T *gc = MODE == 2 ? dy + n0 * CHW + c * HW : nullptr;
+        while (n < imgs) {
+            T v[UN][VEC], g[UN][VEC];
+            bool valid[UN];
+#pragma unroll
+            for (int u = 0; u < UN; u++) {
+                valid[u] = n < imgs;
+                const size_t off = (valid[u] ? n : imgs - 1) * CHW + j * VEC;
+                dh_load_vec_stream<T, VEC>(xc + off, v[u]);
+                if constexpr (MODE == 2)
+                    dh_load_vec_stream<T, VEC>(gc + off, g[u]);
+                n += dn;
+                j += dj;
+                const bool wrap = j >= cvecs;
+                j -= wrap ? cvecs : 0;
+                n += wrap ? 1 : 0;
+            }
+#pragma unroll
+            for (int u = 0; u < UN; u++)
+#pragma unroll
+                for (int e = 0; e < VEC; e++) {
+                    const double d = valid[u] ? static_cast<double>(v[u][e]) - mu : 0.0;
+                    if constexpr (MODE == 3) {
+                        a0 += d;
+                        a1 += d * d;
+                    } else {
+                        const double gr = valid[u] ? static_cast<double>(g[u][e]) : 0.0;
+                        a0 += gr;
+                        a1 += gr * d;
+                        a2 += d;
+                    }
+                }
         }
     }
     double a[3] = {a0, a1, a2};
@@ -84,6 +110,18 @@ __global__ __launch_bounds__(THREADS) void chan_stage1(const T *x, const T *dy, 
             partials[(c * gridDim.y + s) * 3 + k] = v;
         }
     }
+}
+
+template <typename T, int MODE>
+static inline void launch_stage1(dh_ctx *ctx, dim3 grid, const T *x, const T *dy, const T *mean, size_t N, size_t C, size_t HW,
+                                 size_t imgs_per_slice, double *partials) {
+    constexpr int V = dh_vec<T>::N;
+    if (HW % V == 0 && dh_aligned(x, 16) && (MODE != 2 || dh_aligned(dy, 16)))
+        hipLaunchKernelGGL((chan_stage1<T, MODE, V>), grid, dim3(THREADS), 0, ctx->stream, x, dy, mean, N, C, HW, imgs_per_slice,
+                           partials);
+    else
+        hipLaunchKernelGGL((chan_stage1<T, MODE, 1>), grid, dim3(THREADS), 0, ctx->stream, x, dy, mean, N, C, HW, imgs_per_slice,
+                           partials);
 }
 
 // Folds the slices of every channel (one thread per channel, slices in order) and derives what the next pass needs.
@@ -233,8 +271,7 @@ dh_status batchnorm_train_forward(dh_ctx *ctx, T *res, T *new_ema_mean, T *new_e
     const double m = static_cast<double>(rows) * static_cast<double>(HW);
     const dim3 g1(static_cast<unsigned>(C), static_cast<unsigned>(p.S)), g2(static_cast<unsigned>(dh_ceil_div(C, 64)));
     // mean and variance from ONE pass: sums of (x - s) and (x - s)^2 around the channel's first value, in double
-    hipLaunchKernelGGL((chan_stage1<T, 3>), g1, dim3(THREADS), 0, ctx->stream, in, nullptr, nullptr, rows, C, HW, p.imgs_per_slice,
-                       partials);
+    launch_stage1<T, 3>(ctx, g1, in, nullptr, nullptr, rows, C, HW, p.imgs_per_slice, partials);
     hipLaunchKernelGGL((chan_stage2<T, 3>), g2, dim3(64), 0, ctx->stream, partials, C, p.S, m, mean, inv_var, new_ema_mean,
                        new_ema_var, ema_mean, ema_var, eps, mu, gamma, nullptr, nullptr, coef, in, HW);
     launch_apply<T, true>(ctx, res, in, nullptr, rows * C, C, HW, mean, gamma, beta, inv_var, coef);
@@ -260,8 +297,7 @@ dh_status batchnorm_backward(dh_ctx *ctx, T *dX, T *dGamma, T *dBeta, const T *m
     T *coef = reinterpret_cast<T *>(partials + C * p.S * 3);
     const double m = static_cast<double>(rows) * static_cast<double>(HW);
     const dim3 g1(static_cast<unsigned>(C), static_cast<unsigned>(p.S)), g2(static_cast<unsigned>(dh_ceil_div(C, 64)));
-    hipLaunchKernelGGL((chan_stage1<T, 2>), g1, dim3(THREADS), 0, ctx->stream, in, dout, mean, rows, C, HW, p.imgs_per_slice,
-                       partials);
+    launch_stage1<T, 2>(ctx, g1, in, dout, mean, rows, C, HW, p.imgs_per_slice, partials);
     hipLaunchKernelGGL((chan_stage2<T, 2>), g2, dim3(64), 0, ctx->stream, partials, C, p.S, m, const_cast<T *>(mean),
                        const_cast<T *>(inv_var), nullptr, nullptr, nullptr, nullptr, T(0), T(0), gamma, dGamma, dBeta, coef);
     launch_apply<T, false>(ctx, dX, in, dout, rows * C, C, HW, mean, gamma, nullptr, inv_var, coef);
@@ -339,13 +375,21 @@ __global__ __launch_bounds__(THREADS) void pool2x2_backward_kernel(T *res, const
     const size_t idx = static_cast<size_t>(blockIdx.x) * THREADS + threadIdx.x;
     if (idx >= total)
         return;
-    const unsigned wv = W / VI, P = H / 2, Q = W / 2;
-    const unsigned j = static_cast<unsigned>(idx % wv);
-    const size_t pr = idx / wv; // (plane, p)
-    const size_t plane = pr / P;
-    const unsigned p = static_cast<unsigned>(pr % P);
-    const size_t in0 = (plane * H + 2 * p) * W + static_cast<size_t>(j) * VI;
-    const T *dy = dOut + (plane * P + p) * Q + static_cast<size_t>(j) * (VI / 2);
+    // Planes are contiguous and H is even, so the tensor is a flat list of row pairs: pair pr starts at element
+    // pr * 2 * W of the input and at pr * Q of the gradient. One division, 32 bits wide where the count allows.
+    const unsigned wv = W / VI, Q = W / 2;
+    unsigned j;
+    size_t pr;
+    if (total <= 0xffffffffull) {
+        const unsigned i32 = static_cast<unsigned>(idx);
+        pr = i32 / wv;
+        j = i32 % wv;
+    } else {
+        pr = idx / wv;
+        j = static_cast<unsigned>(idx % wv);
+    }
+    const size_t in0 = pr * 2 * W + static_cast<size_t>(j) * VI;
+    const T *dy = dOut + pr * Q + static_cast<size_t>(j) * (VI / 2);
     T o0[VI], o1[VI];
     if constexpr (AVG) {
 #pragma unroll
@@ -394,6 +438,40 @@ __global__ __launch_bounds__(THREADS) void pool2x2_backward_kernel(T *res, const
     __builtin_nontemporal_store(w1, reinterpret_cast<vec_t *>(res + in0 + W));
 }
 
+// AvgPool gradient of 2x2 windows with stride 2 (no padding, even H and W). Planes are contiguous, so the result is
+// a flat list of value pairs, Q = W / 2 to an image row, and pair (row, q) is twice a quarter of gradient
+// (row / 2, q). A thread writes ONE vector of VI / 2 pairs and consecutive threads write consecutive vectors; both
+// image rows of a window row read the same Q gradients.
+template <typename T, int VI>
+__global__ __launch_bounds__(THREADS) void avgpool2x2_backward_kernel(T *res, const T *dOut, unsigned Q, size_t total) {
+#pragma clang fp contract(off)
+    const size_t idx = static_cast<size_t>(blockIdx.x) * THREADS + threadIdx.x;
+    if (idx >= total)
+        return;
+    const bool small = total * (VI / 2) <= 0xffffffffull; // 32-bit divisions suffice (uniform)
+    T g[VI / 2];
+#pragma unroll
+    for (int k = 0; k < VI / 2; k++) {
+        const size_t pair = idx * (VI / 2) + k;
+        size_t row; // image row over all planes
+        unsigned q;
+        if (small) {
+            row = static_cast<unsigned>(pair) / Q;
+            q = static_cast<unsigned>(pair) % Q;
+        } else {
+            row = pair / Q;
+            q = static_cast<unsigned>(pair % Q);
+        }
+        g[k] = dOut[(row >> 1) * Q + q];
+    }
+    typedef T vec_t __attribute__((ext_vector_type(VI)));
+    vec_t w;
+#pragma unroll
+    for (int k = 0; k < VI / 2; k++)
+        w[2 * k] = w[2 * k + 1] = (T(1) / T(4)) * g[k];
+    __builtin_nontemporal_store(w, reinterpret_cast<vec_t *>(res + idx * VI));
+}
+
 template <typename T, bool AVG>
 dh_status pool_backward(dh_ctx *ctx, T *res, const T *input, const T *dOut, size_t N, size_t C, size_t H, size_t W, size_t ph,
                         size_t pw, size_t sh, size_t sw, size_t padh, size_t padw) {
@@ -410,6 +488,17 @@ dh_status pool_backward(dh_ctx *ctx, T *res, const T *input, const T *dOut, size
     if (g.total == 0)
         return DH_OK;
     constexpr int VFULL = dh_vec<T>::N;
+    if (AVG && ph == 2 && pw == 2 && sh == 2 && sw == 2 && padh == 0 && padw == 0 && H % 2 == 0 && W % 2 == 0 &&
+        dh_aligned(res, 16)) {
+        const size_t total = g.total / VFULL; // H and W are even: H * W is a multiple of four
+        if (dh_ceil_div(total, THREADS) < (size_t(1) << 31)) {
+            const dim3 grid(static_cast<unsigned>(dh_ceil_div(total, THREADS)));
+            hipLaunchKernelGGL((avgpool2x2_backward_kernel<T, VFULL>), grid, dim3(THREADS), 0, ctx->stream, res, dOut,
+                               static_cast<unsigned>(W / 2), total);
+            DH_CHECK_LAUNCH();
+            return DH_OK;
+        }
+    }
     if (ph == 2 && pw == 2 && sh == 2 && sw == 2 && padh == 0 && padw == 0 && H % 2 == 0 && W % 2 == 0 && dh_aligned(res, 16) &&
         dh_aligned(input, 16)) {
         const int vi = W % VFULL == 0 ? VFULL : 2;

@@ -60,7 +60,8 @@ def test_batchnorm_train_forward_and_backward(ctx, dt, N, C, H, W):
 @pytest.mark.parametrize("p", [(2, 3, 3, 3, 2, 2, 2, 2, 1, 1), (4, 6, 28, 28, 2, 2, 2, 2, 0, 0), (3, 2, 14, 14, 3, 3, 2, 2, 1, 1),
                                (2, 2, 9, 7, 3, 2, 1, 1, 1, 0), (1, 1, 5, 5, 5, 5, 1, 1, 0, 0), (2, 3, 8, 8, 2, 2, 1, 1, 0, 0),
                                (5, 4, 12, 12, 4, 4, 3, 3, 2, 2), (3, 5, 14, 14, 2, 2, 2, 2, 0, 0), (2, 2, 7, 8, 2, 2, 2, 2, 0, 0),
-                               (64, 16, 14, 16, 2, 2, 2, 2, 0, 0)])
+                               (64, 16, 14, 16, 2, 2, 2, 2, 0, 0), (2, 3, 2, 2, 2, 2, 2, 2, 0, 0), (1, 1, 2, 6, 2, 2, 2, 2, 0, 0),
+                               (3, 2, 6, 10, 2, 2, 2, 2, 0, 0), (130, 64, 14, 14, 2, 2, 2, 2, 0, 0)])
 def test_pooling_backward(ctx, dt, p):
     N, C, H, W, ph, pw, sh, sw, padh, padw = p
     rng = np.random.default_rng(sum(p))
