@@ -122,6 +122,7 @@ POOL_CASES = [  # N, C, H, W, ph, pw, sh, sw, padh, padw
     (1, 3, 7, 9, 2, 3, 1, 2, 1, 0),       # fewer planes than fill a vector-aligned workgroup
     (2, 2, 80, 80, 3, 3, 2, 2, 1, 1),     # planes too large for the LDS kernel
     (2, 3, 64, 64, 5, 5, 3, 3, 2, 2),     # one 16 KB plane per workgroup (float)
+    (7, 11887, 14, 14, 3, 3, 2, 2, 1, 1), # thousands of workgroups, short last one
 ]
 
 

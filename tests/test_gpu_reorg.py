@@ -173,6 +173,7 @@ POOL = [  # N, C, H, W, ph, pw, sh, sw, padh, padw
     (333, 64, 14, 14, 3, 3, 2, 2, 1, 1),   # several planes per workgroup staged in LDS, short last workgroup
     (301, 33, 7, 7, 3, 3, 1, 1, 1, 1),     # planes of 49 values: a multiple of four planes per workgroup
     (2, 2, 80, 80, 4, 4, 2, 2, 1, 1),      # planes too large for the LDS kernel
+    (7, 11887, 14, 14, 3, 2, 2, 2, 1, 0),  # thousands of workgroups, short last one
 ]
 
 
