@@ -336,17 +336,21 @@ template <typename T> __device__ __forceinline__ T div_by_constant(T n, T b, T r
     return (e == e) ? q1 : q0;
 }
 
+constexpr int ROW_UR = 4; // rows per lane group and step of the row kernels
+
 // FINAL: 0 plain reduction, 1 mean, 2 var, 3 stddev. G lanes share a row (G a power of two
 // <= 64, G divides 64). NANFIRST: MIN/MAX take a NaN in column 0 as the result (AggRow.h:108).
-template <typename T, int VEC, class R, int FINAL, bool NANFIRST>
+template <typename T, int VEC, class R, int FINAL, bool NANFIRST, int KV>
 __global__ __launch_bounds__(THREADS) void row_kernel(T *res, size_t ld_res, const T *arg, size_t rows,
                                                       size_t cols, size_t ld, int G) {
     // UR rows per lane group are processed together so that UR independent loads are in flight;
     // rows past the end are clamped to the last row for loading and dropped at the store.
     // Per step a wavefront owns GPW * UR consecutive rows (row (u, g) = base + u * GPW + g for
     // lane group g): load u covers GPW whole rows back to back, and the step's results are one
-    // contiguous run stored by the first GPW * UR lanes.
-    constexpr int UR = 4;
+    // contiguous run stored by the first GPW * UR lanes. A lane takes KV vectors of a row per pass, G lanes
+    // apart: fewer lanes per row mean fewer exchange levels, which is what 8-byte values (two moves per level
+    // and value) are short of.
+    constexpr int UR = ROW_UR;
     const int tid = threadIdx.x;
     const int lane = tid % G;
     const int wlane = tid % DH_WAVE;
@@ -357,6 +361,7 @@ __global__ __launch_bounds__(THREADS) void row_kernel(T *res, size_t ld_res, con
     const size_t wave_id = static_cast<size_t>(blockIdx.x) * (THREADS / DH_WAVE) + tid / DH_WAVE;
     const size_t wave_stride = static_cast<size_t>(gridDim.x) * (THREADS / DH_WAVE) * rows_per_step;
     const T ncols = static_cast<T>(cols), rcols = T(1) / ncols;
+    const size_t pass = static_cast<size_t>(G) * KV; // vectors of a row per pass of its lane group
     for (size_t base = wave_id * rows_per_step; base < rows; base += wave_stride) {
         const T *row[UR];
 #pragma unroll
@@ -366,29 +371,39 @@ __global__ __launch_bounds__(THREADS) void row_kernel(T *res, size_t ld_res, con
         }
         T acc[UR];
         T first[UR];      // element 0 of the row, known to the lane that loads it (NANFIRST)
-        T xk[UR][VEC];    // the lane's values when the row fits one vector per lane (second pass of VAR / STDDEV)
-        const bool in_regs = cvecs <= static_cast<size_t>(G);
+        T xk[UR][KV][VEC]; // the lane's values when the row fits one pass (second pass of VAR / STDDEV)
+        const bool in_regs = cvecs <= pass;
 #pragma unroll
         for (int u = 0; u < UR; u++) {
             acc[u] = R::id();
             first[u] = T(0);
         }
-        for (size_t cv = lane; cv < cvecs; cv += G) {
-            T x[UR][VEC];
+        for (size_t cv = lane; cv < cvecs; cv += pass) {
+            T x[UR][KV][VEC];
+            // vectors past the row's end re-read the lane's first one and are left out below
 #pragma unroll
-            for (int u = 0; u < UR; u++)
-                dh_load_vec_stream<T, VEC>(row[u] + cv * VEC, x[u]);
+            for (int k = 0; k < KV; k++)
 #pragma unroll
-            for (int u = 0; u < UR; u++) {
-                if constexpr (NANFIRST) {
-                    if (cv == 0)
-                        first[u] = x[u][0];
+                for (int u = 0; u < UR; u++) {
+                    const size_t c = cv + static_cast<size_t>(k) * G;
+                    dh_load_vec_stream<T, VEC>(row[u] + (c < cvecs ? c : cv) * VEC, x[u][k]);
                 }
 #pragma unroll
-                for (int i = 0; i < VEC; i++) {
-                    acc[u] = R::comb(acc[u], x[u][i]);
-                    if constexpr (FINAL >= 2)
-                        xk[u][i] = x[u][i];
+            for (int k = 0; k < KV; k++) {
+                const bool valid = k == 0 || cv + static_cast<size_t>(k) * G < cvecs;
+#pragma unroll
+                for (int u = 0; u < UR; u++) {
+                    if constexpr (NANFIRST) {
+                        if (k == 0 && cv == 0)
+                            first[u] = x[u][0][0];
+                    }
+#pragma unroll
+                    for (int i = 0; i < VEC; i++) {
+                        const T next = R::comb(acc[u], x[u][k][i]);
+                        acc[u] = valid ? next : acc[u];
+                        if constexpr (FINAL >= 2)
+                            xk[u][k][i] = x[u][k][i];
+                    }
                 }
             }
         }
@@ -412,28 +427,40 @@ __global__ __launch_bounds__(THREADS) void row_kernel(T *res, size_t ld_res, con
             for (int u = 0; u < UR; u++)
                 s[u] = T(0);
             if (in_regs) {
-                if (static_cast<size_t>(lane) < cvecs) {
+#pragma unroll
+                for (int k = 0; k < KV; k++) {
+                    const bool valid = static_cast<size_t>(lane) + static_cast<size_t>(k) * G < cvecs;
 #pragma unroll
                     for (int u = 0; u < UR; u++)
 #pragma unroll
                         for (int i = 0; i < VEC; i++) {
-                            const T d = xk[u][i] - acc[u];
-                            s[u] = s[u] + d * d;
+                            const T d = xk[u][k][i] - acc[u];
+                            const T next = s[u] + d * d;
+                            s[u] = valid ? next : s[u];
                         }
                 }
             } else {
-                for (size_t cv = lane; cv < cvecs; cv += G) {
-                    T x[UR][VEC];
+                for (size_t cv = lane; cv < cvecs; cv += pass) {
+                    T x[UR][KV][VEC];
 #pragma unroll
-                    for (int u = 0; u < UR; u++)
-                        load_vec<T, VEC>(row[u] + cv * VEC, x[u]);
+                    for (int k = 0; k < KV; k++)
 #pragma unroll
-                    for (int u = 0; u < UR; u++)
-#pragma unroll
-                        for (int i = 0; i < VEC; i++) {
-                            const T d = x[u][i] - acc[u];
-                            s[u] = s[u] + d * d;
+                        for (int u = 0; u < UR; u++) {
+                            const size_t c = cv + static_cast<size_t>(k) * G;
+                            load_vec<T, VEC>(row[u] + (c < cvecs ? c : cv) * VEC, x[u][k]);
                         }
+#pragma unroll
+                    for (int k = 0; k < KV; k++) {
+                        const bool valid = k == 0 || cv + static_cast<size_t>(k) * G < cvecs;
+#pragma unroll
+                        for (int u = 0; u < UR; u++)
+#pragma unroll
+                            for (int i = 0; i < VEC; i++) {
+                                const T d = x[u][k][i] - acc[u];
+                                const T next = s[u] + d * d;
+                                s[u] = valid ? next : s[u];
+                            }
+                    }
                 }
             }
             dh_butterfly(G, [&](auto peer) {
@@ -486,10 +513,10 @@ __global__ __launch_bounds__(THREADS) void row_kernel(T *res, size_t ld_res, con
 // mapping as row_kernel (a wavefront owns GPW * UR consecutive rows per step, results stored as one
 // contiguous run). I is the index type carried through the reduction: 32 bits unless a row has 2^32
 // or more columns.
-template <typename T, int VEC, bool IS_MIN, typename I>
+template <typename T, int VEC, bool IS_MIN, typename I, int KV>
 __global__ __launch_bounds__(THREADS) void row_idx_kernel(uint64_t *res, size_t ld_res, const T *arg, size_t rows,
                                                           size_t cols, size_t ld, int G) {
-    constexpr int UR = 4;
+    constexpr int UR = ROW_UR;
     constexpr I NONE = ~static_cast<I>(0);
     const int tid = threadIdx.x;
     const int lane = tid % G;
@@ -514,25 +541,36 @@ __global__ __launch_bounds__(THREADS) void row_idx_kernel(uint64_t *res, size_t 
             bi[u] = NONE;
             nan0[u] = false;
         }
-        for (size_t cv = lane; cv < cvecs; cv += G) {
-            T x[UR][VEC];
+        const size_t pass = static_cast<size_t>(G) * KV; // vectors of a row per pass: KV per lane, G lanes apart
+        for (size_t cv = lane; cv < cvecs; cv += pass) {
+            T x[UR][KV][VEC];
+            // vectors past the row's end re-read the lane's first one and are left out below
 #pragma unroll
-            for (int u = 0; u < UR; u++)
-                dh_load_vec_stream<T, VEC>(row[u] + cv * VEC, x[u]);
+            for (int k = 0; k < KV; k++)
 #pragma unroll
-            for (int u = 0; u < UR; u++) {
-                if (cv == 0)
-                    nan0[u] = dev_isnan(x[u][0]);
+                for (int u = 0; u < UR; u++) {
+                    const size_t c = cv + static_cast<size_t>(k) * G;
+                    dh_load_vec_stream<T, VEC>(row[u] + (c < cvecs ? c : cv) * VEC, x[u][k]);
+                }
 #pragma unroll
-                for (int i = 0; i < VEC; i++) {
-                    const I idx = static_cast<I>(cv * VEC + i);
-                    const bool better = IS_MIN ? (x[u][i] < best[u]) : (x[u][i] > best[u]);
-                    // within a lane indices only grow, so a tie keeps the earlier one, except
-                    // against the sentinel (an actual +-inf value must beat "nothing seen yet")
-                    const bool first_seen = (bi[u] == NONE) && (x[u][i] == best[u]);
-                    if (better || first_seen) {
-                        best[u] = x[u][i];
-                        bi[u] = idx;
+            for (int k = 0; k < KV; k++) {
+                const size_t c = cv + static_cast<size_t>(k) * G;
+                const bool valid = k == 0 || c < cvecs;
+#pragma unroll
+                for (int u = 0; u < UR; u++) {
+                    if (k == 0 && cv == 0)
+                        nan0[u] = dev_isnan(x[u][0][0]);
+#pragma unroll
+                    for (int i = 0; i < VEC; i++) {
+                        const I idx = static_cast<I>(c * VEC + i);
+                        const bool better = IS_MIN ? (x[u][k][i] < best[u]) : (x[u][k][i] > best[u]);
+                        // within a lane indices only grow, so a tie keeps the earlier one, except
+                        // against the sentinel (an actual +-inf value must beat "nothing seen yet")
+                        const bool first_seen = (bi[u] == NONE) && (x[u][k][i] == best[u]);
+                        if (valid && (better || first_seen)) {
+                            best[u] = x[u][k][i];
+                            bi[u] = idx;
+                        }
                     }
                 }
             }
@@ -580,12 +618,16 @@ __global__ __launch_bounds__(THREADS) void row_idx_kernel(uint64_t *res, size_t 
     }
 }
 
-static inline int pick_group(size_t cvecs) {
+static inline int pick_group(size_t cvecs, int kv = 1) {
     int g = 1;
-    while (g < DH_WAVE && static_cast<size_t>(g) < cvecs)
+    while (g < DH_WAVE && static_cast<size_t>(g) * kv < cvecs)
         g <<= 1;
     return g;
 }
+// Vectors per lane and pass of the row kernels. Two where the exchanges dominate: 8-byte values in the two-butterfly
+// reductions and in the (value, index) reductions. Measured on 10M x 64 doubles: VAR 963 -> 842 us, IDXMIN 943 -> 793 us;
+// the one-butterfly reductions and all 4-byte cases lose 3-5 % with two.
+template <typename T> constexpr int row_kv(bool two_exchanges_or_index) { return sizeof(T) == 8 && two_exchanges_or_index ? 2 : 1; }
 
 static inline unsigned row_grid(const dh_ctx *ctx, size_t rows, int G) {
     const size_t rpb = static_cast<size_t>(THREADS / G) * 4; // rows per block and step (4 per lane group)
@@ -605,12 +647,13 @@ static inline void row_launch(dh_ctx *ctx, T *res, size_t ld_res, const T *arg, 
     constexpr int V = dh_vec<T>::N;
     const bool vec_ok = (cols % V == 0) && (ld % V == 0) && dh_aligned(arg, 16);
     if (vec_ok) {
-        const int G = pick_group(cols / V);
-        hipLaunchKernelGGL((row_kernel<T, V, R, FINAL, NANFIRST>), dim3(row_grid(ctx, rows, G)), dim3(THREADS), 0,
+        constexpr int KV = row_kv<T>(FINAL >= 2);
+        const int G = pick_group(cols / V, KV);
+        hipLaunchKernelGGL((row_kernel<T, V, R, FINAL, NANFIRST, KV>), dim3(row_grid(ctx, rows, G)), dim3(THREADS), 0,
                            ctx->stream, res, ld_res, arg, rows, cols, ld, G);
     } else {
         const int G = pick_group(cols);
-        hipLaunchKernelGGL((row_kernel<T, 1, R, FINAL, NANFIRST>), dim3(row_grid(ctx, rows, G)), dim3(THREADS), 0,
+        hipLaunchKernelGGL((row_kernel<T, 1, R, FINAL, NANFIRST, 1>), dim3(row_grid(ctx, rows, G)), dim3(THREADS), 0,
                            ctx->stream, res, ld_res, arg, rows, cols, ld, G);
     }
 }
@@ -671,17 +714,18 @@ dh_status agg_row_idx(dh_ctx *ctx, int op, uint64_t *res, size_t ld_res, const T
         return dh_fail(DH_ERR_RUNTIME, "AggRow - the argument has no columns");
     constexpr int V = dh_vec<T>::N;
     const bool vec_ok = (cols % V == 0) && (ld % V == 0) && dh_aligned(arg, 16);
-    const int G = pick_group(vec_ok ? cols / V : cols);
+    constexpr int KV = row_kv<T>(true);
+    const int G = vec_ok ? pick_group(cols / V, KV) : pick_group(cols);
     const dim3 grid(row_grid(ctx, rows, G)), block(THREADS);
     const bool wide = cols >= 0xffffffffull; // index does not fit 32 bits next to the sentinel
 #define DH_ROW_IDX(VEC_, MIN_)                                                                                          \
     do {                                                                                                                \
         if (wide)                                                                                                       \
-            hipLaunchKernelGGL((row_idx_kernel<T, VEC_, MIN_, unsigned long long>), grid, block, 0, ctx->stream, res,   \
-                               ld_res, arg, rows, cols, ld, G);                                                         \
+            hipLaunchKernelGGL((row_idx_kernel<T, VEC_, MIN_, unsigned long long, 1>), grid, block, 0, ctx->stream,     \
+                               res, ld_res, arg, rows, cols, ld, G);                                                    \
         else                                                                                                            \
-            hipLaunchKernelGGL((row_idx_kernel<T, VEC_, MIN_, unsigned>), grid, block, 0, ctx->stream, res, ld_res,     \
-                               arg, rows, cols, ld, G);                                                                 \
+            hipLaunchKernelGGL((row_idx_kernel<T, VEC_, MIN_, unsigned, (VEC_) == 1 ? 1 : KV>), grid, block, 0,         \
+                               ctx->stream, res, ld_res, arg, rows, cols, ld, G);                                       \
     } while (0)
     if (vec_ok) {
         if (op == DH_AGG_IDXMIN)
