@@ -211,7 +211,7 @@ def run(args) -> int:
             cpu = {"value": round(nb / dt, 2), "unit": "images/s", "cores": 1, "kind": "port",
                    "sample": f"batch {nb} of {N}, raw-pointer restatement of the reference loops, single thread ({dt:.2f} s)"}
         c2 = layer_tflops["conv2+bias"]
-        roof = {"bound": "mfma", "kernel": "conv2d_kernel<float,64,128,16,4> (conv2: 4096x32x14x14, 64 filters 5x5)",
+        roof = {"bound": "mfma", "kernel": "conv2d_resident_kernel<float,4,7> (conv2: 4096x32x14x14, 64 filters 5x5, images resident in LDS)",
                 "achieved": c2, "peak": MFMA_PEAK["f32"], "unit": "TFLOP/s", "frac": round(c2 / MFMA_PEAK["f32"], 4), "traffic": None}
         out = _line(N / ms * 1e3, "images/s", ms, args, "f32",
                     "LeNet-style CNN inference, batch 4096, 1x28x28 input, conv-pool-conv-pool-affine-affine-softmax",

@@ -365,79 +365,6 @@ __global__ __launch_bounds__(THREADS) void pool_backward_kernel(T *res, const T 
     res[idx] = acc;
 }
 
-// 2x2 windows, stride 2, no padding, even image height, width a multiple of the vector: every pixel belongs to
-// exactly one window. A thread takes VI columns of an image-row pair: two vector loads of the input (MAX only), VI/2
-// gradients, two vector stores. VI is the 16-byte vector, or half of it for floats when the width is only even.
-template <typename T, int VI, bool AVG>
-__global__ __launch_bounds__(THREADS) void pool2x2_backward_kernel(T *res, const T *input, const T *dOut, unsigned H, unsigned W, size_t total) {
-#pragma clang fp contract(off)
-    typedef T vec_t __attribute__((ext_vector_type(VI)));
-    const size_t idx = static_cast<size_t>(blockIdx.x) * THREADS + threadIdx.x;
-    if (idx >= total)
-        return;
-    // Planes are contiguous and H is even, so the tensor is a flat list of row pairs: pair pr starts at element
-    // pr * 2 * W of the input and at pr * Q of the gradient. One division, 32 bits wide where the count allows.
-    const unsigned wv = W / VI, Q = W / 2;
-    unsigned j;
-    size_t pr;
-    if (total <= 0xffffffffull) {
-        const unsigned i32 = static_cast<unsigned>(idx);
-        pr = i32 / wv;
-        j = i32 % wv;
-    } else {
-        pr = idx / wv;
-        j = static_cast<unsigned>(idx % wv);
-    }
-    const size_t in0 = pr * 2 * W + static_cast<size_t>(j) * VI;
-    const T *dy = dOut + pr * Q + static_cast<size_t>(j) * (VI / 2);
-    T o0[VI], o1[VI];
-    if constexpr (AVG) {
-#pragma unroll
-        for (int k = 0; k < VI / 2; k++) {
-            const T v = (T(1) / T(4)) * dy[k];
-            o0[2 * k] = o0[2 * k + 1] = o1[2 * k] = o1[2 * k + 1] = v;
-        }
-    } else {
-        const vec_t v0 = __builtin_nontemporal_load(reinterpret_cast<const vec_t *>(input + in0));
-        const vec_t v1 = __builtin_nontemporal_load(reinterpret_cast<const vec_t *>(input + in0 + W));
-        T x0[VI], x1[VI];
-#pragma unroll
-        for (int e = 0; e < VI; e++) {
-            x0[e] = v0[e];
-            x1[e] = v1[e];
-        }
-#pragma unroll
-        for (int k = 0; k < VI / 2; k++) {
-            // first maximum in row-major order with a strict comparison (MaxPoolBackward.h:62-69)
-            int best = 0;
-            T m = x0[2 * k];
-            if (x0[2 * k + 1] > m) {
-                m = x0[2 * k + 1];
-                best = 1;
-            }
-            if (x1[2 * k] > m) {
-                m = x1[2 * k];
-                best = 2;
-            }
-            if (x1[2 * k + 1] > m)
-                best = 3;
-            const T gv = dy[k];
-            o0[2 * k] = best == 0 ? gv : T(0);
-            o0[2 * k + 1] = best == 1 ? gv : T(0);
-            o1[2 * k] = best == 2 ? gv : T(0);
-            o1[2 * k + 1] = best == 3 ? gv : T(0);
-        }
-    }
-    vec_t w0, w1;
-#pragma unroll
-    for (int e = 0; e < VI; e++) {
-        w0[e] = o0[e];
-        w1[e] = o1[e];
-    }
-    __builtin_nontemporal_store(w0, reinterpret_cast<vec_t *>(res + in0));
-    __builtin_nontemporal_store(w1, reinterpret_cast<vec_t *>(res + in0 + W));
-}
-
 // AvgPool gradient of 2x2 windows with stride 2 (no padding, even H and W). Planes are contiguous, so the result is
 // a flat list of value pairs, Q = W / 2 to an image row, and pair (row, q) is twice a quarter of gradient
 // (row / 2, q). A thread writes ONE vector of VI / 2 pairs and consecutive threads write consecutive vectors; both
@@ -472,6 +399,64 @@ __global__ __launch_bounds__(THREADS) void avgpool2x2_backward_kernel(T *res, co
     __builtin_nontemporal_store(w, reinterpret_cast<vec_t *>(res + idx * VI));
 }
 
+// MaxPool gradient of 2x2 windows with stride 2 (no padding, even H and W), flat like the average above: a thread
+// writes one vector of VI / 2 value pairs of the result. For each pair it reads both rows of the pair's window (the
+// other image row of the window asks for the same values; they come from the cache) and the window's gradient, and
+// keeps the gradient where the first maximum of the window (row-major order, strict comparison,
+// MaxPoolBackward.h:62-69) lies in its own row.
+template <typename T, int VI>
+__global__ __launch_bounds__(THREADS) void maxpool2x2_backward_kernel(T *res, const T *input, const T *dOut, unsigned Q,
+                                                                           size_t total) {
+    typedef T pair_t __attribute__((ext_vector_type(2)));
+    typedef T vec_t __attribute__((ext_vector_type(VI)));
+    const size_t idx = static_cast<size_t>(blockIdx.x) * THREADS + threadIdx.x;
+    if (idx >= total)
+        return;
+    const bool small = total * (VI / 2) <= 0xffffffffull; // 32-bit divisions suffice (uniform)
+    pair_t top[VI / 2], bot[VI / 2];
+    T g[VI / 2];
+    bool lower[VI / 2]; // this pair lies in the window's second row
+#pragma unroll
+    for (int k = 0; k < VI / 2; k++) {
+        const size_t pair = idx * (VI / 2) + k;
+        size_t row; // image row over all planes
+        unsigned q;
+        if (small) {
+            row = static_cast<unsigned>(pair) / Q;
+            q = static_cast<unsigned>(pair) % Q;
+        } else {
+            row = pair / Q;
+            q = static_cast<unsigned>(pair % Q);
+        }
+        const size_t wrow = row >> 1;
+        const T *x0 = input + wrow * 4 * Q + 2 * q; // an image row holds 2 * Q values
+        top[k] = *reinterpret_cast<const pair_t *>(x0);
+        bot[k] = *reinterpret_cast<const pair_t *>(x0 + 2 * Q);
+        g[k] = dOut[wrow * Q + q];
+        lower[k] = (row & 1) != 0;
+    }
+    vec_t w;
+#pragma unroll
+    for (int k = 0; k < VI / 2; k++) {
+        int best = 0;
+        T m = top[k][0];
+        if (top[k][1] > m) {
+            m = top[k][1];
+            best = 1;
+        }
+        if (bot[k][0] > m) {
+            m = bot[k][0];
+            best = 2;
+        }
+        if (bot[k][1] > m)
+            best = 3;
+        const int first = lower[k] ? 2 : 0;
+        w[2 * k] = best == first ? g[k] : T(0);
+        w[2 * k + 1] = best == first + 1 ? g[k] : T(0);
+    }
+    __builtin_nontemporal_store(w, reinterpret_cast<vec_t *>(res + idx * VI));
+}
+
 template <typename T, bool AVG>
 dh_status pool_backward(dh_ctx *ctx, T *res, const T *input, const T *dOut, size_t N, size_t C, size_t H, size_t W, size_t ph,
                         size_t pw, size_t sh, size_t sw, size_t padh, size_t padw) {
@@ -488,29 +473,17 @@ dh_status pool_backward(dh_ctx *ctx, T *res, const T *input, const T *dOut, size
     if (g.total == 0)
         return DH_OK;
     constexpr int VFULL = dh_vec<T>::N;
-    if (AVG && ph == 2 && pw == 2 && sh == 2 && sw == 2 && padh == 0 && padw == 0 && H % 2 == 0 && W % 2 == 0 &&
-        dh_aligned(res, 16)) {
+    if (ph == 2 && pw == 2 && sh == 2 && sw == 2 && padh == 0 && padw == 0 && H % 2 == 0 && W % 2 == 0 &&
+        dh_aligned(res, 16) && (AVG || dh_aligned(input, 2 * sizeof(T)))) {
         const size_t total = g.total / VFULL; // H and W are even: H * W is a multiple of four
         if (dh_ceil_div(total, THREADS) < (size_t(1) << 31)) {
             const dim3 grid(static_cast<unsigned>(dh_ceil_div(total, THREADS)));
-            hipLaunchKernelGGL((avgpool2x2_backward_kernel<T, VFULL>), grid, dim3(THREADS), 0, ctx->stream, res, dOut,
-                               static_cast<unsigned>(W / 2), total);
-            DH_CHECK_LAUNCH();
-            return DH_OK;
-        }
-    }
-    if (ph == 2 && pw == 2 && sh == 2 && sw == 2 && padh == 0 && padw == 0 && H % 2 == 0 && W % 2 == 0 && dh_aligned(res, 16) &&
-        dh_aligned(input, 16)) {
-        const int vi = W % VFULL == 0 ? VFULL : 2;
-        const size_t total = N * C * (H / 2) * (W / vi);
-        if (dh_ceil_div(total, THREADS) < (size_t(1) << 31)) {
-            const dim3 grid(static_cast<unsigned>(dh_ceil_div(total, THREADS)));
-            if (vi == VFULL)
-                hipLaunchKernelGGL((pool2x2_backward_kernel<T, VFULL, AVG>), grid, dim3(THREADS), 0, ctx->stream, res, input, dOut,
-                                   static_cast<unsigned>(H), static_cast<unsigned>(W), total);
+            if constexpr (AVG)
+                hipLaunchKernelGGL((avgpool2x2_backward_kernel<T, VFULL>), grid, dim3(THREADS), 0, ctx->stream, res, dOut,
+                                   static_cast<unsigned>(W / 2), total);
             else
-                hipLaunchKernelGGL((pool2x2_backward_kernel<T, 2, AVG>), grid, dim3(THREADS), 0, ctx->stream, res, input, dOut,
-                                   static_cast<unsigned>(H), static_cast<unsigned>(W), total);
+                hipLaunchKernelGGL((maxpool2x2_backward_kernel<T, VFULL>), grid, dim3(THREADS), 0, ctx->stream, res, input,
+                                   dOut, static_cast<unsigned>(W / 2), total);
             DH_CHECK_LAUNCH();
             return DH_OK;
         }
