@@ -220,7 +220,7 @@ def main() -> int:
             dyc = DM.from_torch(ctx, torch.randn(Nc, 64 * 196, device="cuda", dtype=tdt, generator=gen))
             dxc, dwc = DM(ctx, Nc, 32 * 196, ndt), DM(ctx, 64, 800, ndt)
             fl = 2.0 * Nc * 64 * 196 * 800
-            emit("conv2DBackwardData 64->32 ch, 14x14, 5x5 pad 2 (frame + rotated filters + forward convolution)", dt, f"batch {Nc}",
+            emit("conv2DBackwardData 64->32 ch, 14x14, 5x5 pad 2 (rotated filters + forward convolution of the padded output gradient)", dt, f"batch {Nc}",
                  timed(lambda: K.conv2DBackwardData(wc, dyc, 1, 1, 2, 2, Nc, 32, 14, 14, 64, 32, 5, 5, dxc, ctx)), flops=fl)
             emit("conv2DBackwardFilter 32->64 ch, 14x14, 5x5 pad 2 (image resident in LDS, slabs per workgroup)", dt, f"batch {Nc}",
                  timed(lambda: K.conv2DBackwardFilter(dwc, xc, dyc, 1, 1, 2, 2, Nc, 32, 14, 14, 64, 32, 5, 5, ctx)), flops=fl)

@@ -609,12 +609,14 @@ static inline dh_status conv_bwd_args(ConvBwdArgs *g, size_t N, size_t C, size_t
 // temporaries come from the context's block cache; shapes whose temporaries would be very large, or padding beyond
 // the filter extent, take the gather kernels.
 static inline dh_status conv_fwd(dh_ctx *ctx, float *res, size_t *rh, size_t *rw, const float *data, const float *filter, size_t fr,
-                                 size_t fc, size_t N, size_t C, size_t H, size_t W, size_t Hf, size_t Wf) {
-    return dh_conv2d_forward_f32(ctx, res, rh, rw, data, filter, fr, fc, nullptr, N, C, H, W, Hf, Wf, 1, 1, 0, 0);
+                                 size_t fc, size_t N, size_t C, size_t H, size_t W, size_t Hf, size_t Wf, size_t padh = 0,
+                                 size_t padw = 0) {
+    return dh_conv2d_forward_f32(ctx, res, rh, rw, data, filter, fr, fc, nullptr, N, C, H, W, Hf, Wf, 1, 1, padh, padw);
 }
 static inline dh_status conv_fwd(dh_ctx *ctx, double *res, size_t *rh, size_t *rw, const double *data, const double *filter, size_t fr,
-                                 size_t fc, size_t N, size_t C, size_t H, size_t W, size_t Hf, size_t Wf) {
-    return dh_conv2d_forward_f64(ctx, res, rh, rw, data, filter, fr, fc, nullptr, N, C, H, W, Hf, Wf, 1, 1, 0, 0);
+                                 size_t fc, size_t N, size_t C, size_t H, size_t W, size_t Hf, size_t Wf, size_t padh = 0,
+                                 size_t padw = 0) {
+    return dh_conv2d_forward_f64(ctx, res, rh, rw, data, filter, fr, fc, nullptr, N, C, H, W, Hf, Wf, 1, 1, padh, padw);
 }
 static inline dh_status mat_mul(dh_ctx *ctx, float *res, size_t ldr, const float *a, size_t ar, size_t ac, size_t lda, const float *b,
                                 size_t br, size_t bc, size_t ldb) {
@@ -631,8 +633,16 @@ template <typename T> __global__ __launch_bounds__(THREADS) void dilate_frame_ke
     if (idx >= total)
         return;
     const unsigned FH = g.H + g.Hf - 1, FW = g.W + g.Wf - 1;
-    const size_t plane = idx / (static_cast<size_t>(FH) * FW); // (n, f)
-    const unsigned ab = static_cast<unsigned>(idx % (static_cast<size_t>(FH) * FW)), a = ab / FW, b = ab % FW;
+    size_t plane; // (n, f)
+    unsigned ab;
+    if (total <= 0xffffffffull) { // 32-bit divisions suffice (uniform)
+        plane = static_cast<unsigned>(idx) / (FH * FW);
+        ab = static_cast<unsigned>(idx) % (FH * FW);
+    } else {
+        plane = idx / (static_cast<size_t>(FH) * FW);
+        ab = static_cast<unsigned>(idx % (static_cast<size_t>(FH) * FW));
+    }
+    const unsigned a = ab / FW, b = ab % FW;
     const unsigned oh = g.Hf - 1 - g.padh, ow = g.Wf - 1 - g.padw;
     T v = T(0);
     if (a >= oh && b >= ow && (a - oh) % g.sh == 0 && (b - ow) % g.sw == 0) {
@@ -707,6 +717,21 @@ template <typename T> static bool conv_backward_data_mfma(dh_ctx *ctx, T *dX, co
         dh_ceil_div(frame_elems, static_cast<size_t>(THREADS)) >= (size_t(1) << 31))
         return false;
     void *frame = nullptr, *wr = nullptr;
+    if (g.sh == 1 && g.sw == 1 && g.P + g.Hf - 1 == g.H + 2 * g.padh && g.Q + g.Wf - 1 == g.W + 2 * g.padw) {
+        // nothing to dilate: the frame is dY with Hf - 1 - padh rows and Wf - 1 - padw columns of zeros on every side,
+        // which is the forward convolution's own padding
+        *st = dh_malloc(ctx, wr_elems * sizeof(T), 0, &wr);
+        if (*st != DH_OK)
+            return true;
+        hipLaunchKernelGGL((rotate_filter_kernel<T>), dim3(blocks_for(wr_elems)), dim3(THREADS), 0, ctx->stream, static_cast<T *>(wr), filter, g);
+        size_t rh = 0, rw = 0;
+        *st = conv_fwd(ctx, dX, &rh, &rw, dY, static_cast<const T *>(wr), g.C, static_cast<size_t>(g.F) * g.Hf * g.Wf, g.N, g.F, g.P, g.Q,
+                       g.Hf, g.Wf, g.Hf - 1 - g.padh, g.Wf - 1 - g.padw);
+        dh_free(ctx, wr);
+        if (*st == DH_OK && (rh != g.H || rw != g.W))
+            *st = dh_fail(DH_ERR_RUNTIME, "Conv2D backward - internal extent mismatch (%zu x %zu for %u x %u)", rh, rw, g.H, g.W);
+        return true;
+    }
     *st = dh_malloc(ctx, frame_elems * sizeof(T), 0, &frame);
     if (*st != DH_OK)
         return true;

@@ -95,6 +95,9 @@ def test_pooling_backward_all_negative_window_goes_to_the_padding(ctx):
                                   (64, 8, 12, 12, 6, 3, 3, 1, 1, 1, 1), (64, 4, 16, 16, 8, 5, 5, 2, 2, 2, 2),
                                   (48, 6, 15, 13, 5, 3, 2, 1, 2, 0, 1), (40, 3, 28, 28, 7, 5, 5, 1, 1, 2, 2),
                                   (96, 5, 12, 12, 3, 2, 2, 3, 3, 1, 1),
+                                  # stride 1 (data gradient = forward convolution of dY with its own padding): no padding in the
+                                  # forward direction is the widest one here; uneven filter and padding
+                                  (30, 4, 24, 24, 5, 5, 5, 1, 1, 0, 0), (64, 8, 12, 13, 6, 3, 2, 1, 1, 0, 1), (33, 8, 10, 10, 16, 4, 4, 1, 1, 3, 3),
                                   # filter gradient with the image resident in LDS: two column chunks of 13 blocks a wave;
                                   # 20 filters (two filter blocks, 4 column parts); 70 filters (two groups) with stride 2;
                                   # 8 filters (one filter block, 8 column parts)
