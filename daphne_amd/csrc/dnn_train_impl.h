@@ -189,7 +189,8 @@ __global__ __launch_bounds__(THREADS) void chan_apply(T *res, const T *x, const 
     const size_t r = static_cast<size_t>(blockIdx.x) * blockDim.y + threadIdx.y;
     if (r >= rows)
         return;
-    const size_t c = r % C;
+    // 32-bit remainder where the row count allows (uniform)
+    const size_t c = rows <= 0xffffffffull ? static_cast<unsigned>(r) % static_cast<unsigned>(C) : r % C;
     const T mn = mean[c], g = gamma[c];
     const T p0 = FWD ? coef[c] : inv_var[c], p1 = FWD ? beta[c] : coef[2 * c], p2 = FWD ? T(0) : coef[2 * c + 1];
     for (size_t cv = static_cast<size_t>(blockIdx.y) * blockDim.x + threadIdx.x; cv < cvecs;
@@ -320,8 +321,16 @@ __global__ __launch_bounds__(THREADS) void pool_backward_kernel(T *res, const T 
     if (idx >= g.total)
         return;
     const unsigned HW = g.H * g.W;
-    const size_t img = idx / HW; // (n, c) plane
-    const unsigned hw = static_cast<unsigned>(idx % HW), h = hw / g.W, w = hw % g.W;
+    size_t img; // (n, c) plane
+    unsigned hw;
+    if (g.total <= 0xffffffffull) { // 32-bit divisions suffice (uniform)
+        img = static_cast<unsigned>(idx) / HW;
+        hw = static_cast<unsigned>(idx) % HW;
+    } else {
+        img = idx / HW;
+        hw = static_cast<unsigned>(idx % HW);
+    }
+    const unsigned h = hw / g.W, w = hw % g.W;
     const unsigned hp = h + g.padh, wp = w + g.padw; // position in the zero-padded plane
     const unsigned pH = g.H + 2 * g.padh, pW = g.W + 2 * g.padw;
     const T *plane = input + img * HW;
