@@ -569,6 +569,8 @@ dh_status conv2d_forward(dh_ctx *ctx, T *res, size_t *res_h, size_t *res_w, cons
         // latencies with: taken only when a wave has at least six blocks of matrix instructions per step.
         // With K < 32 (one or two K blocks) the output stores dominate, and the tiled kernel below writes longer
         // runs: 1 -> 32 channels, 5 x 5 on 28 x 28 takes 0.16 ms there and 0.28 ms here.
+        // (One thread per pixel on the ordinary ALUs, weights broadcast from LDS, was tried for that layer as well:
+        // 0.15 ms, bound by the LDS reads of the weights; four pixels per thread to share them: 0.20 ms.)
         if (cg != 0 && lds <= 150 * 1024 && (lds <= 80 * 1024 || nf >= 6) && blocks16 >= 3 * parts && K >= 32 && fgroups < 65536 &&
             chunks < 65536) {
             const size_t fpad = fgroups * 16 * mfw;
@@ -927,7 +929,8 @@ dh_status maxpool_forward(dh_ctx *ctx, T *res, size_t *res_h, size_t *res_w, con
         // value is what the CPU kernel returns for every output.
         hipLaunchKernelGGL((fill_kernel<T>), dim3(static_cast<unsigned>(grid)), dim3(256), 0, ctx->stream, res, total,
                            std::numeric_limits<T>::max());
-    } else if (const unsigned ppb = pool_planes_per_block(data, H * W, N * C); ppb != 0 && dh_ceil_div(N * C, ppb) < (size_t(1) << 31)) {
+    } else if (const unsigned ppb = pool_planes_per_block(data, H * W, N * C);
+               ppb != 0 && dh_ceil_div(N * C, ppb) < (size_t(1) << 31) && ppb * P * Q < (size_t(1) << 31)) {
         hipLaunchKernelGGL((pool_planes_kernel<T, false>), dim3(static_cast<unsigned>(dh_ceil_div(N * C, ppb))), dim3(256),
                            ppb * H * W * sizeof(T), ctx->stream, res, data, N * C, ppb, static_cast<unsigned>(H),
                            static_cast<unsigned>(W), static_cast<unsigned>(P), static_cast<unsigned>(Q),
@@ -1037,7 +1040,7 @@ dh_status avgpool_forward(dh_ctx *ctx, T *res, size_t *res_h, size_t *res_w, con
     const T plen = T(1) / static_cast<T>(pw * ph); // Pooling.cpp:50
     const bool quick = P == 1 && Q == 1 && W == 1;
     if (const unsigned ppb = quick ? 0 : pool_planes_per_block(data, H * W, N * C);
-        ppb != 0 && dh_ceil_div(N * C, ppb) < (size_t(1) << 31)) {
+        ppb != 0 && dh_ceil_div(N * C, ppb) < (size_t(1) << 31) && ppb * P * Q < (size_t(1) << 31)) {
         hipLaunchKernelGGL((pool_planes_kernel<T, true>), dim3(static_cast<unsigned>(dh_ceil_div(N * C, ppb))), dim3(256),
                            ppb * H * W * sizeof(T), ctx->stream, res, data, N * C, ppb, static_cast<unsigned>(H),
                            static_cast<unsigned>(W), static_cast<unsigned>(P), static_cast<unsigned>(Q),

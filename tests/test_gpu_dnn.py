@@ -44,6 +44,12 @@ CONV_CASES = [  # N, C, H, W, F, Hf, Wf, sh, sw, ph, pw
     (9, 16, 7, 7, 32, 3, 3, 1, 1, 1, 1),
     (20, 8, 4, 4, 64, 3, 3, 1, 1, 1, 1),
     (7, 64, 14, 14, 32, 5, 5, 1, 1, 0, 0),
+    # fewer than 32 filter taps: 33 filters (a partial filter block) and
+    # uneven strides, 17 filters with wide padding, 31 taps in a column, more than 256 pixels per image
+    (3, 1, 19, 23, 33, 3, 5, 2, 3, 1, 2),
+    (2, 3, 9, 9, 17, 3, 3, 1, 1, 2, 2),
+    (2, 1, 40, 40, 9, 31, 1, 1, 1, 15, 0),
+    (70, 1, 28, 28, 6, 5, 5, 1, 1, 0, 0),
 ]
 
 
