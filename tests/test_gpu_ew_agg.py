@@ -159,7 +159,7 @@ def test_ew_unary_domain_error(ctx, dt, op, bad):
 
 AGG_VALUE_OPS = [AggOpCode.SUM, AggOpCode.PROD, AggOpCode.MIN, AggOpCode.MAX, AggOpCode.MEAN, AggOpCode.STDDEV,
                  AggOpCode.VAR]
-AGG_SHAPES = [(1000, 64), (7, 5), (1, 300), (300, 1), (4100, 16), (3, 1030), (50000, 4)]
+AGG_SHAPES = [(1000, 64), (7, 5), (1, 300), (300, 1), (4100, 16), (3, 1030), (50000, 4), (33, 6), (100, 12), (64, 22), (257, 66)]
 
 
 def _agg_input(rng, shape, dt, op):
@@ -190,7 +190,8 @@ def test_agg_row_col_all(ctx, dt, op, shape):
 
 @pytest.mark.parametrize("dt", DTYPES)
 @pytest.mark.parametrize("op", [AggOpCode.IDXMIN, AggOpCode.IDXMAX])
-@pytest.mark.parametrize("shape", [(2000, 16), (7, 5), (1, 300), (300, 1), (513, 64), (3, 1030), (9, 130)])
+@pytest.mark.parametrize("shape", [(2000, 16), (7, 5), (1, 300), (300, 1), (513, 64), (3, 1030), (9, 130), (33, 6), (100, 12),
+                                   (64, 22), (257, 66)])
 def test_agg_idx_bit_exact(ctx, dt, op, shape):
     rng = np.random.default_rng(shape[0] + 7 * shape[1])
     # few distinct values -> many ties; plus NaN / inf rows
