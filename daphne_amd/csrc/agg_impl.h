@@ -744,7 +744,9 @@ dh_status agg_row_idx(dh_ctx *ctx, int op, uint64_t *res, size_t ld_res, const T
 }
 
 constexpr int S2_TX = 16, S2_TY = 16; // second-stage block: columns x partial lanes
-constexpr int V2_TY = 64;             // partial lanes of the variance second stage
+constexpr int V2_TX = 4, V2_TY = 64;   // variance second stage: small blocks, few columns each. It is a chain of two
+                                       // passes over ~1000 partials and three barriers, i.e. latency: 16 x 64 threads in
+                                       // 4 blocks took 32 us on 64 columns, 4 x 256 in 16 blocks 24 us, 4 x 64 9 us
 
 // =======================================================================================
 // AggCol
@@ -927,14 +929,14 @@ __global__ __launch_bounds__(THREADS) void col_var_stage1(const T *arg, size_t r
 
 // OUT: 0 variance, 1 stddev, 2 mean (unused by the public API but kept for pipelines).
 template <typename T, int OUT>
-__global__ __launch_bounds__(S2_TX * V2_TY) void col_var_stage2(const T *part_mean, const T *part_m2, size_t nparts,
+__global__ __launch_bounds__(V2_TX * V2_TY) void col_var_stage2(const T *part_mean, const T *part_m2, size_t nparts,
                                                           size_t cols, size_t rows, size_t slab, T *res,
                                                           T *res_mean = nullptr) {
-    // (S2_TX columns, V2_TY partial lanes: 1024 threads, so that a thousand partials take two rounds of loads per pass). Pooled moments of the per-block (count, mean, M2) triples in double:
+    // (V2_TX columns, V2_TY partial lanes: 1024 threads). Pooled moments of the per-block (count, mean, M2) triples in double:
     //     mean = sum n_p mean_p / N,   M2 = sum M2_p + sum n_p (mean_p - mean)^2
     // - the closed form of merging them pairwise with Chan's formula, without a division per partial.
-    __shared__ double lds_a[V2_TY][S2_TX], lds_b[V2_TY][S2_TX];
-    const size_t c = static_cast<size_t>(blockIdx.x) * S2_TX + threadIdx.x;
+    __shared__ double lds_a[V2_TY][V2_TX], lds_b[V2_TY][V2_TX];
+    const size_t c = static_cast<size_t>(blockIdx.x) * V2_TX + threadIdx.x;
     auto count = [&](size_t p) {
         const size_t r_begin = p * slab;
         if (r_begin >= rows)
@@ -1240,11 +1242,11 @@ template <typename T> dh_status agg_col(dh_ctx *ctx, int op, T *res, const T *ar
             hipLaunchKernelGGL((col_var_stage1<T, V>), p.grid, p.block, lds, ctx->stream, arg, rows, p.cvecs, ld, p.slab, pm, pq);
         else
             hipLaunchKernelGGL((col_var_stage1<T, 1>), p.grid, p.block, lds, ctx->stream, arg, rows, p.cvecs, ld, p.slab, pm, pq);
-        const dim3 g2(static_cast<unsigned>(dh_ceil_div(cols, S2_TX)));
+        const dim3 g2(static_cast<unsigned>(dh_ceil_div(cols, V2_TX)));
         if (op == DH_AGG_VAR)
-            hipLaunchKernelGGL((col_var_stage2<T, 0>), g2, dim3(S2_TX, V2_TY), 0, ctx->stream, pm, pq, p.nparts, cols, rows, p.slab, res);
+            hipLaunchKernelGGL((col_var_stage2<T, 0>), g2, dim3(V2_TX, V2_TY), 0, ctx->stream, pm, pq, p.nparts, cols, rows, p.slab, res);
         else
-            hipLaunchKernelGGL((col_var_stage2<T, 1>), g2, dim3(S2_TX, V2_TY), 0, ctx->stream, pm, pq, p.nparts, cols, rows, p.slab, res);
+            hipLaunchKernelGGL((col_var_stage2<T, 1>), g2, dim3(V2_TX, V2_TY), 0, ctx->stream, pm, pq, p.nparts, cols, rows, p.slab, res);
         break;
     }
     default:
@@ -1283,12 +1285,12 @@ dh_status agg_col_moments(dh_ctx *ctx, T *res_mean, T *res_var, int stddev, cons
         hipLaunchKernelGGL((col_var_stage1<T, V>), p.grid, p.block, lds, ctx->stream, arg, rows, p.cvecs, ld, p.slab, pm, pq);
     else
         hipLaunchKernelGGL((col_var_stage1<T, 1>), p.grid, p.block, lds, ctx->stream, arg, rows, p.cvecs, ld, p.slab, pm, pq);
-    const dim3 g2(static_cast<unsigned>(dh_ceil_div(cols, S2_TX)));
+    const dim3 g2(static_cast<unsigned>(dh_ceil_div(cols, V2_TX)));
     if (stddev)
-        hipLaunchKernelGGL((col_var_stage2<T, 1>), g2, dim3(S2_TX, V2_TY), 0, ctx->stream, pm, pq, p.nparts, cols, rows, p.slab,
+        hipLaunchKernelGGL((col_var_stage2<T, 1>), g2, dim3(V2_TX, V2_TY), 0, ctx->stream, pm, pq, p.nparts, cols, rows, p.slab,
                            res_var, res_mean);
     else
-        hipLaunchKernelGGL((col_var_stage2<T, 0>), g2, dim3(S2_TX, V2_TY), 0, ctx->stream, pm, pq, p.nparts, cols, rows, p.slab,
+        hipLaunchKernelGGL((col_var_stage2<T, 0>), g2, dim3(V2_TX, V2_TY), 0, ctx->stream, pm, pq, p.nparts, cols, rows, p.slab,
                            res_var, res_mean);
     DH_CHECK_LAUNCH();
     return DH_OK;
