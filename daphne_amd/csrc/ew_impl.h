@@ -115,6 +115,25 @@ __global__ __launch_bounds__(EW_THREADS) void ew_kernel(T *res, size_t ld_res, c
 
 static __global__ void set_flag_kernel(int *flag, int v) { *flag = v; }
 
+// Checked unary operator on a small matrix (a vector of column statistics, say): one workgroup computes the results
+// and sets the flag to whether any argument lay outside the domain - no separate launch to clear the flag first.
+constexpr size_t EW_SMALL_CHECKED = 4096; // elements
+template <typename T, template <typename> class F>
+__global__ __launch_bounds__(EW_THREADS) void ew_unary_small_checked_kernel(T *res, size_t ld_res, const T *arg, size_t ld_arg,
+                                                                            unsigned rows, unsigned cols, int *flag) {
+    static_assert(F<T>::checks, "only for operators with a domain");
+    int any_bad = 0;
+    for (unsigned i = threadIdx.x; i < rows * cols; i += EW_THREADS) {
+        const unsigned r = i / cols, c = i % cols;
+        const T a = arg[static_cast<size_t>(r) * ld_arg + c];
+        any_bad |= F<T>::bad(a) ? 1 : 0;
+        res[static_cast<size_t>(r) * ld_res + c] = F<T>::apply(a, T(0));
+    }
+    const int any = __syncthreads_or(any_bad);
+    if (threadIdx.x == 0)
+        *flag = any ? 1 : 0;
+}
+
 // C++ names of the value types as the reference prints them (ValueTypeUtils::cppNameFor)
 template <typename T> static inline const char *type_name();
 template <> inline const char *type_name<float>() { return "float"; }
@@ -283,14 +302,30 @@ dh_status ew_unary(dh_ctx *ctx, int op, T *res, size_t ld_res, const T *arg, siz
     if (ld_res < cols || ld_arg < cols)
         return dh_fail(DH_ERR_RUNTIME, "EwUnaryMat - a leading dimension is smaller than the column count");
     const bool checks = (op == DH_UN_SQRT || op == DH_UN_LN || op == DH_UN_ASIN || op == DH_UN_ACOS);
-    if (checks) {
+    const bool small_checked = checks && rows * cols <= EW_SMALL_CHECKED && rows * cols > 0;
+    if (small_checked) {
+#define DH_SMALL(FUN)                                                                                                   \
+    hipLaunchKernelGGL((ew_unary_small_checked_kernel<T, FUN>), dim3(1), dim3(EW_THREADS), 0, ctx->stream, res, ld_res, arg, ld_arg, \
+                       static_cast<unsigned>(rows), static_cast<unsigned>(cols), ctx->flag_dev)
+        if (op == DH_UN_SQRT)
+            DH_SMALL(USqrt);
+        else if (op == DH_UN_LN)
+            DH_SMALL(ULn);
+        else if (op == DH_UN_ASIN)
+            DH_SMALL(UAsin);
+        else
+            DH_SMALL(UAcos);
+#undef DH_SMALL
+    } else if (checks) {
         hipLaunchKernelGGL(set_flag_kernel, dim3(1), dim3(1), 0, ctx->stream, ctx->flag_dev, 0);
     }
 #define DH_CASE(CODE, FUN)                                                                         \
     case CODE:                                                                                     \
         launch<T, FUN, UNARY>(ctx, res, ld_res, arg, ld_arg, nullptr, 0, T(0), rows, cols, ctx->flag_dev); \
         break;
-    switch (op) {
+    switch (small_checked ? -1 : op) {
+    case -1: // done above
+        break;
         DH_CASE(DH_UN_MINUS, UMinus)
         DH_CASE(DH_UN_ABS, UAbs)
         DH_CASE(DH_UN_SIGN, USign)

@@ -145,16 +145,18 @@ def test_ew_unary(ctx, dt, op):
 @pytest.mark.parametrize("dt", DTYPES)
 @pytest.mark.parametrize("op,bad", [(UnaryOpCode.SQRT, -1.0), (UnaryOpCode.LN, -1e-30), (UnaryOpCode.ASIN, 1.5),
                                     (UnaryOpCode.ACOS, -1.0001)])
-def test_ew_unary_domain_error(ctx, dt, op, bad):
-    a = np.full((100, 33), 0.5, dt)
-    a[77, 20] = bad
+@pytest.mark.parametrize("shape", [(100, 33), (300, 40), (1, 64)])  # one workgroup that also sets the flag; the large kernel
+def test_ew_unary_domain_error(ctx, dt, op, bad, shape):
+    a = np.full(shape, 0.5, dt)
+    a[shape[0] * 3 // 4, 20] = bad
     st, _ = orc.ew_unary(op, a)
     assert st == orc.ST_DOMAIN
     with pytest.raises(capi.DaphneHipDomainError, match="invalid argument"):
         ewUnaryMat(op, None, DenseMatrix.from_numpy(ctx, a), ctx)
     # the flag is cleared again for the next call
-    a[77, 20] = 0.25
-    ewUnaryMat(op, None, DenseMatrix.from_numpy(ctx, a), ctx)
+    a[shape[0] * 3 // 4, 20] = 0.25
+    d = DenseMatrix.from_numpy(ctx, a)
+    assert_close(ewUnaryMat(op, d, d, ctx).to_numpy(), orc.ew_unary(op, a)[1])  # in place
 
 
 AGG_VALUE_OPS = [AggOpCode.SUM, AggOpCode.PROD, AggOpCode.MIN, AggOpCode.MAX, AggOpCode.MEAN, AggOpCode.STDDEV,
