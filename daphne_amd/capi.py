@@ -64,6 +64,11 @@ def _signatures(lib: C.CDLL) -> None:
     lib.dh_d2h.argtypes = [ctxp, vp, vp, sz]
     lib.dh_d2d.argtypes = [ctxp, vp, vp, sz]
     lib.dh_timer_start.argtypes = [ctxp]
+    lib.dh_ctx_set_pipeline_mode.argtypes = [ctxp, i32]
+    lib.dh_ctx_get_pipeline_mode.argtypes = [ctxp]
+    lib.dh_vectorized_pipeline_last_mode.argtypes = []
+    lib.dh_vectorized_pipeline_cache_size.argtypes = []
+    lib.dh_vectorized_pipeline_cache_size.restype = sz
     lib.dh_timer_stop_ms.argtypes = [ctxp, C.POINTER(C.c_float)]
     for suf, ct in (("f32", C.c_float), ("f64", C.c_double)):
         f = lambda name: getattr(lib, f"{name}_{suf}")

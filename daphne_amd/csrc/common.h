@@ -24,6 +24,12 @@ struct dh_ctx {
     size_t mem_budget = 0;
     size_t mem_in_use = 0;
     std::mutex lock;                  // guards allocations / mem_in_use / the block cache
+    // Held by every entry point from its first line to its return (DH_REQUIRE_CTX). The workspace, the domain
+    // flag and the AggAll result slot below exist once per context, and a call that reads one of them back
+    // synchronises the stream before it returns: with the whole call under this lock, host threads that share
+    // a context take turns, their kernels run in the order of the context's stream, and none sees another's
+    // flag, scalar or partials. Recursive because entry points call each other (Affine -> MatMul, ...).
+    std::recursive_mutex call_lock;
     struct Block {
         size_t requested, capacity;
     };
@@ -35,9 +41,8 @@ struct dh_ctx {
     size_t reserved_bytes = 0; // capacities of live + cached blocks
 
     // Reduction workspace (partials of the two-stage aggregations, split-K slabs). Grown on
-    // demand under ws_lock; kernels using it are serialised by that lock only for the
-    // duration of the enqueue, so concurrent host threads must not share one context for
-    // overlapping workspace kernels on different streams.
+    // demand under ws_lock (after a stream synchronise); its users are ordered by call_lock and
+    // the context's stream.
     std::mutex ws_lock;
     void *ws = nullptr;
     size_t ws_bytes = 0;
@@ -48,6 +53,9 @@ struct dh_ctx {
 
     hipEvent_t ev_start = nullptr, ev_stop = nullptr;
     int num_cus = 0;
+    // How fused pipeline bodies run on this context: -1 as the environment says (DH_PIPELINE_JIT, default:
+    // specialised at run time), 0 interpreted, 1 specialised.
+    int pipeline_mode = -1;
 };
 
 // ---------------------------------------------------------------------------------------
@@ -72,10 +80,15 @@ dh_status dh_fail(dh_status st, const char *fmt, ...) __attribute__((format(prin
                            hipGetErrorString(e__));                                                \
     } while (0)
 
+// First statement of every entry point: rejects a null context, takes the context's call lock until the
+// enclosing function returns, and makes the context's device current for the calling thread.
+#define DH_CAT2(a, b) a##b
+#define DH_CAT(a, b) DH_CAT2(a, b)
 #define DH_REQUIRE_CTX(ctx)                                                                        \
+    if ((ctx) == nullptr)                                                                          \
+        return dh_fail(DH_ERR_RUNTIME, "%s: context is null", __func__);                           \
+    std::lock_guard<std::recursive_mutex> DH_CAT(dh_call_guard_, __LINE__)((ctx)->call_lock);      \
     do {                                                                                           \
-        if ((ctx) == nullptr)                                                                      \
-            return dh_fail(DH_ERR_RUNTIME, "%s: context is null", __func__);                       \
         hipError_t e__ = hipSetDevice((ctx)->device);                                              \
         if (e__ != hipSuccess)                                                                     \
             return dh_fail(DH_ERR_HIP, "hipSetDevice(%d): %s", (ctx)->device,                      \

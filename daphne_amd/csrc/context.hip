@@ -122,11 +122,9 @@ extern "C" dh_status dh_ctx_props(const dh_ctx *ctx, int *compute_units, int *cl
 }
 
 extern "C" dh_status dh_ctx_set_stream(dh_ctx *ctx, void *hip_stream) {
-    if (ctx == nullptr)
-        return dh_fail(DH_ERR_RUNTIME, "dh_ctx_set_stream: context is null");
+    DH_REQUIRE_CTX(ctx);
     if (ctx->stream != static_cast<hipStream_t>(hip_stream)) {
         // cached blocks may still be in use by work queued on the old stream
-        (void)hipSetDevice(ctx->device);
         DH_CHECK_HIP(hipStreamSynchronize(ctx->stream));
     }
     ctx->stream = static_cast<hipStream_t>(hip_stream);

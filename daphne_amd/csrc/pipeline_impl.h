@@ -16,6 +16,7 @@ bool jit_enabled();
 bool jit_lookup(int device, const char *tname, int vec, int kv, size_t cols, int G, int S, const dh_pipe_instr *prog, int n,
                 hipFunction_t *fn, std::string *err, bool compile_only);
 void jit_set_last_mode(int m);
+size_t jit_cache_size();
 
 // Folds the per-workgroup partials of a full reduction. One workgroup of 1024 threads; every thread keeps 16
 // loads in flight (indices past the end are clamped for the load and replaced by the identity afterwards) and
@@ -205,15 +206,29 @@ dh_status run(dh_ctx *ctx, const dh_pipe_instr *prog, int n, const IO_C *cio, si
     // kernel below is the fallback when specialisation is switched off or fails.
     hipFunction_t jit_fn = nullptr;
     std::string jit_err;
-    const bool use_jit = n >= 1 && jit_enabled() &&
-                         jit_lookup(ctx->device, sizeof(T) == 4 ? "float" : "double", vec, KV, cols, G, S, P.ins, n, &jit_fn, &jit_err,
-                                    false);
+    // the context's setting wins over the environment's (dh_ctx_set_pipeline_mode)
+    const bool want_jit = n >= 1 && (ctx->pipeline_mode < 0 ? jit_enabled() : ctx->pipeline_mode == 1);
+    const bool use_jit = want_jit && jit_lookup(ctx->device, sizeof(T) == 4 ? "float" : "double", vec, KV, cols, G, S, P.ins, n,
+                                                &jit_fn, &jit_err, false);
+    if (want_jit && !use_jit) {
+        // The body still runs (interpreted, at a fraction of the rate); the reason stays readable through
+        // dh_last_error() and dh_vectorized_pipeline_last_mode() says 0. Reported once per process on stderr.
+        dh_set_error("vectorizedPipeline: run-time specialisation failed, the body is interpreted instead: %s", jit_err.c_str());
+        static bool warned = false;
+        if (!warned) {
+            warned = true;
+            fprintf(stderr, "libdaphne_hip: %s\n", dh_last_error());
+        }
+    }
     const dim3 g(static_cast<unsigned>(grid)), b(THREADS);
     if (use_jit) {
         size_t a_rows = rows, a_cols = cols;
         int a_G = G;
         int *a_flag = ctx->flag_dev;
-        void *args[] = {&io, &a_rows, &a_cols, &a_G, &partials, &a_flag};
+        Immediates imm{};
+        for (int i = 0; i < n; i++)
+            imm.v[i] = prog[i].scalar;
+        void *args[] = {&io, &a_rows, &a_cols, &a_G, &partials, &a_flag, &imm};
         DH_CHECK_HIP(hipModuleLaunchKernel(jit_fn, g.x, 1, 1, b.x, 1, 1, 0, ctx->stream, args, nullptr));
         jit_set_last_mode(1);
     } else {

@@ -50,6 +50,11 @@ struct Program {
     int n;
     dh_pipe_instr ins[DH_PIPE_MAX_INSTR];
 };
+// The immediates of a body, in instruction order: an argument of the specialised kernel, so that a body
+// compiled once serves every value of its scalars.
+struct Immediates {
+    double v[DH_PIPE_MAX_INSTR];
+};
 
 template <typename T, int N> __device__ __forceinline__ void apply_binary(int op, T (&a)[N], const T (&b)[N], bool swap) {
     using namespace dh_ew;

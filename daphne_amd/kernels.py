@@ -83,6 +83,10 @@ class HIPContext:
     def sync(self) -> None:
         capi.check(capi.lib().dh_sync(self._h))
 
+    def set_pipeline_mode(self, mode: int) -> None:
+        """1: fused pipeline bodies are specialised at run time, 0: interpreted, -1: as the environment says."""
+        capi.check(capi.lib().dh_ctx_set_pipeline_mode(self._h, mode))
+
     def timer_start(self) -> None:
         capi.check(capi.lib().dh_timer_start(self._h))
 

@@ -12,9 +12,13 @@
  * available from dh_last_error(). The status selects the C++ exception type the reference
  * would have thrown (see the enum), so a C++ caller can re-throw it unchanged.
  *
- * Threading: a dh_ctx may be used from several host threads; allocation bookkeeping is
- * mutex-guarded and kernels are enqueued on the context's stream. Kernels that return a
- * value to the host (dh_agg_all_*, domain checks of dh_ew_unary_*) synchronise that stream.
+ * Threading: a dh_ctx may be used from several host threads. Every call holds the context's
+ * lock from entry to return, so calls on one context take turns and their kernels run in the
+ * order of the context's stream; the workspace, the domain flag and the scalar result slot
+ * that a context owns once are therefore never shared between two calls in flight. Kernels
+ * that return a value to the host (dh_agg_all_*, domain checks of dh_ew_unary_*) synchronise
+ * that stream while they hold the lock. Threads that should not wait for each other use one
+ * context each.
  */
 #ifndef DAPHNE_HIP_H
 #define DAPHNE_HIP_H
@@ -592,6 +596,16 @@ dh_status dh_vectorized_pipeline_f64(dh_ctx *ctx, const dh_pipe_instr *program, 
  * switched off (environment DH_PIPELINE_JIT=0) or fails, a generic kernel interprets the list.
  * Returns how the calling thread's last pipeline ran: 1 specialised, 0 interpreted. */
 int dh_vectorized_pipeline_last_mode(void);
+/* How bodies run on this context: 1 specialised at run time, 0 interpreted by the generic kernel, -1 (the
+ * initial setting) as the environment says. A specialisation that fails does not fail the call: the body is
+ * interpreted, dh_vectorized_pipeline_last_mode() returns 0 and dh_last_error() holds the compiler's output. */
+dh_status dh_ctx_set_pipeline_mode(dh_ctx *ctx, int mode);
+int dh_ctx_get_pipeline_mode(const dh_ctx *ctx);
+/* Number of specialised bodies this process holds. A body is keyed by its instruction kinds, op codes,
+ * operand slots, value type and row width; its immediates are kernel arguments, so a scalar that changes
+ * from call to call (a threshold, a learning rate) reuses the compiled kernel. At most 128 bodies stay
+ * loaded, the least recently used one is unloaded beyond that. */
+size_t dh_vectorized_pipeline_cache_size(void);
 /* Compiles the specialised kernel of a body for rows of `cols` values without loading or running
  * it (no device needed). value_type 0 = float, 1 = double; vectorised != 0: rows are read as
  * 16-byte vectors (cols a multiple of 4 / 2), as the launch does for aligned operands. */

@@ -18,8 +18,17 @@ def assert_exact(got, exp):
         raise AssertionError(f"{(~same).sum()} mismatches, first at {bad.tolist()}: got {got[~same][:5]} exp {exp[~same][:5]}")
 
 
-def assert_close(got, exp, rtol=None, elementwise=True):
-    """Relative error check. elementwise: |g-e| <= rtol*|e| per item (plus a tiny absolute floor
+def variance_floor(x, op_is_stddev=False):
+    """Absolute floor for comparing variances (standard deviations) of the values x item by item: the rounding
+    noise of sum((x - mean)^2) / n when the true variance is (nearly) zero, 16 eps max|x|^2. It only matters for
+    such items; everywhere else the relative bound is the larger one."""
+    x = np.asarray(x)
+    f = 16 * np.finfo(x.dtype).eps * float(np.max(np.abs(x[np.isfinite(x)]), initial=0.0)) ** 2
+    return float(np.sqrt(f)) if op_is_stddev else f
+
+
+def assert_close(got, exp, rtol=None, elementwise=True, atol=0.0):
+    """Relative error check. elementwise: |g-e| <= rtol*|e| + atol per item (plus a tiny absolute floor
     for items that are exactly 0); otherwise norm-wise: max|g-e| <= rtol*max|e|."""
     got, exp = np.asarray(got), np.asarray(exp)
     assert got.shape == exp.shape, (got.shape, exp.shape)
@@ -35,7 +44,7 @@ def assert_close(got, exp, rtol=None, elementwise=True):
     err = np.abs(g - e)
     if elementwise:
         tiny = np.finfo(exp.dtype).tiny if exp.dtype.kind == "f" else 0.0
-        bound = rtol * np.abs(e) + 16 * tiny
+        bound = rtol * np.abs(e) + 16 * tiny + atol
     else:
         bound = np.full_like(e, rtol * np.abs(e).max())
     bad = err > bound

@@ -53,3 +53,50 @@ def test_reused_blocks_keep_results_intact():
         cur = nxt
     np.testing.assert_array_equal(cur.to_numpy(), x + 50.0)
     c.destroy()
+
+
+def test_two_host_threads_share_one_context():
+    """The reference calls device kernels from its main thread, its CPU workers and its device worker
+    (src/runtime/local/vectorized/MTWrapper.h:94-98). Two threads on ONE context each allocate, run a checked unary
+    operator (domain flag), a column and a full aggregation (workspace, scalar slot) of their own data and free
+    again, many times over; every result must be the thread's own, compared with the CPU oracle."""
+    import threading
+
+    import oracle_binding as orc
+    from daphne_amd.kernels import AggOpCode, UnaryOpCode, aggAll, aggCol, ewUnaryMat
+    from parity import assert_close
+
+    c = HIPContext(0)
+    errors = []
+
+    def worker(seed, rows, cols, poison):
+        try:
+            rng = np.random.default_rng(seed)
+            x = (rng.random((rows, cols)) * (seed + 1) + 0.5).astype(np.float32)
+            _, sq_e = orc.ew_unary(UnaryOpCode.SQRT, x)
+            _, col_e = orc.agg_col(AggOpCode.SUM, x)
+            _, all_e = orc.agg_all(AggOpCode.MAX, x)
+            bad = x.copy()
+            bad[rows // 2, cols // 3] = -1.0
+            for it in range(40):
+                X = DenseMatrix.from_numpy(c, x)
+                np.testing.assert_array_equal(ewUnaryMat(UnaryOpCode.SQRT, None, X, c).to_numpy(), sq_e)
+                assert_close(aggCol(AggOpCode.SUM, None, X, c).to_numpy(), col_e)
+                assert aggAll(AggOpCode.MAX, X, c) == all_e
+                if poison and it % 4 == 0:
+                    # this thread's domain error must never surface in the other thread's call
+                    with pytest.raises(capi.DaphneHipDomainError):
+                        ewUnaryMat(UnaryOpCode.SQRT, None, DenseMatrix.from_numpy(c, bad), c)
+                del X
+        except BaseException as e:  # noqa: BLE001 - reported by the main thread
+            errors.append((seed, repr(e)))
+
+    ts = [threading.Thread(target=worker, args=(1, 3000, 64, True)), threading.Thread(target=worker, args=(2, 50001, 7, False))]
+    for t in ts:
+        t.start()
+    for t in ts:
+        t.join()
+    assert not errors, errors
+    c.sync()
+    assert c.memInUse() == 0
+    c.destroy()

@@ -4,7 +4,7 @@ import numpy as np
 import pytest
 
 import oracle_binding as orc
-from parity import assert_close, assert_exact
+from parity import assert_close, assert_exact, variance_floor
 
 pytestmark = pytest.mark.gpu
 
@@ -14,6 +14,20 @@ from daphne_amd.kernels import (AggOpCode, BinaryOpCode, DenseMatrix, UnaryOpCod
 from daphne_amd.pipeline import ROWREG, SELF, VectorizedPipeline
 
 DTYPES = [np.float32, np.float64]
+
+
+@pytest.fixture(autouse=True, params=[1, 0], ids=["specialised", "interpreted"])
+def pipeline_mode(request, ctx):
+    """Every test of this module runs twice on the shared context: with bodies specialised at run time and with the
+    generic kernel interpreting them. A test that ran a body must have run it the way the context was told to."""
+    mode = request.param
+    ctx.set_pipeline_mode(mode)
+    yield mode
+    ctx.set_pipeline_mode(-1)
+
+
+def assert_ran_as(mode):
+    assert capi.lib().dh_vectorized_pipeline_last_mode() == mode
 
 
 def zscore_device(ctx, X, thr=64.0):
@@ -31,12 +45,13 @@ def zscore_device(ctx, X, thr=64.0):
 
 
 @pytest.mark.parametrize("rows,cols", [(1000, 64), (50001, 64), (777, 16), (513, 40), (300, 7), (64, 256), (5, 1000)])
-def test_zscore_pipeline_vs_oracle_engine(ctx, rows, cols):
+def test_zscore_pipeline_vs_oracle_engine(ctx, pipeline_mode, rows, cols):
     rng = np.random.default_rng(rows + cols)
     x = (rng.standard_normal((rows, cols)) * 2 + 5).astype(np.float32)
     thr = float(cols)
     st, mu_e, sd_e, r_e, s_e, _ = orc.zscore_pipeline(x, threads=3, thr=thr)
     mu, sd, r, s = zscore_device(ctx, DenseMatrix.from_numpy(ctx, x), thr)
+    assert_ran_as(pipeline_mode)
     assert_close(mu.to_numpy(), mu_e)
     assert_close(sd.to_numpy(), sd_e)
     assert_close(r.to_numpy(), r_e)
@@ -114,7 +129,8 @@ def test_pipeline_row_aggs_vs_oracle(ctx, dt, op, rows, cols):
     if is_idx or op in (AggOpCode.MIN, AggOpCode.MAX):
         assert_exact(out.to_numpy(), exp)
     else:
-        assert_close(out.to_numpy(), exp, elementwise=op not in (AggOpCode.VAR, AggOpCode.STDDEV))
+        atol = variance_floor(x, op == AggOpCode.STDDEV) if op in (AggOpCode.VAR, AggOpCode.STDDEV) else 0.0
+        assert_close(out.to_numpy(), exp, atol=atol)
 
 
 @pytest.mark.parametrize("dt", DTYPES)
@@ -173,7 +189,7 @@ def test_pipeline_errors(ctx):
 
 @pytest.mark.parametrize("dt", DTYPES)
 @pytest.mark.parametrize("rows,cols", [(4096, 64), (1000, 16), (257, 40), (33, 7), (100, 512)])
-def test_pipeline_division_by_row_vector_is_ieee_division(ctx, dt, rows, cols):
+def test_pipeline_division_by_row_vector_is_ieee_division(ctx, pipeline_mode, dt, rows, cols):
     """t / rowvec inside a specialised body takes a short division sequence when every operand is well inside the
     exponent range and the general one otherwise; either way the quotient is the correctly rounded one, bit for bit
     (numpy divides in IEEE arithmetic, as the reference's CPU and CUDA kernels do)."""
@@ -199,7 +215,7 @@ def test_pipeline_division_by_row_vector_is_ieee_division(ctx, dt, rows, cols):
         p.ewBinary(BinaryOpCode.DIV, D)
         out = p.storeTile()
         p.run()
-        assert capi.lib().dh_vectorized_pipeline_last_mode() == 1
+        assert_ran_as(pipeline_mode)
         with np.errstate(all="ignore"):
             want = xa / da
         got = out.to_numpy()
@@ -207,3 +223,50 @@ def test_pipeline_division_by_row_vector_is_ieee_division(ctx, dt, rows, cols):
         assert np.array_equal(np.isnan(got), nan)
         assert np.array_equal(got[~nan].view(np.uint32 if dt == np.float32 else np.uint64),
                               want[~nan].view(np.uint32 if dt == np.float32 else np.uint64))
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("rows,cols", [(3000, 64), (257, 40), (33, 7)])
+def test_interpreted_body_equals_specialised_body(ctx, dt, rows, cols):
+    """The generic kernel and the run-time specialised one instantiate the same body: same results, bit for bit."""
+    rng = np.random.default_rng(rows + cols)
+    x = (rng.standard_normal((rows, cols)) * 2 + 5).astype(dt)
+    rv = (rng.random((1, cols)) + 0.5).astype(dt)
+    X, RV = DenseMatrix.from_numpy(ctx, x), DenseMatrix.from_numpy(ctx, rv)
+    outs = {}
+    for mode in (1, 0):
+        ctx.set_pipeline_mode(mode)
+        p = VectorizedPipeline(ctx, X)
+        p.ewBinary(BinaryOpCode.SUB, 5.0).ewBinary(BinaryOpCode.DIV, RV).ewBinary(BinaryOpCode.MUL, SELF)
+        tile = p.storeTile()
+        p.rowAgg(AggOpCode.SUM)
+        r = p.storeRow()
+        p.ewBinary(BinaryOpCode.GT, float(cols))
+        s = p.reduceAll(AggOpCode.SUM)
+        p.run()
+        assert_ran_as(mode)
+        outs[mode] = (tile.to_numpy(), r.to_numpy(), s.to_numpy())
+    for a, b in zip(outs[1], outs[0]):
+        assert_exact(a, b)
+
+
+def test_changing_immediates_reuse_the_compiled_body(ctx, pipeline_mode):
+    """A body is compiled per structure, not per value of its scalars: thresholds that change from call to call (and
+    NaN / infinite ones, which have no literal form) run the same kernel."""
+    if pipeline_mode != 1:
+        pytest.skip("only the specialised path compiles anything")
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal((2000, 24)).astype(np.float32)
+    X = DenseMatrix.from_numpy(ctx, x)
+    sizes = []
+    for k, thr in enumerate([0.5, -0.25, 3.0, float("inf"), float("nan"), 1e-30, 7.75]):
+        p = VectorizedPipeline(ctx, X)
+        p.ewBinary(BinaryOpCode.MUL, 1.0 + k).ewBinary(BinaryOpCode.GT, thr)
+        out = p.storeTile()
+        p.run()
+        assert_ran_as(1)
+        sizes.append(capi.lib().dh_vectorized_pipeline_cache_size())
+        with np.errstate(invalid="ignore"):
+            want = ((x * np.float32(1.0 + k)) > np.float32(thr)).astype(np.float32)
+        assert_exact(out.to_numpy(), want)
+    assert len(set(sizes)) == 1, sizes
