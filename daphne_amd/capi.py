@@ -69,6 +69,9 @@ def _signatures(lib: C.CDLL) -> None:
     lib.dh_vectorized_pipeline_last_mode.argtypes = []
     lib.dh_vectorized_pipeline_cache_size.argtypes = []
     lib.dh_vectorized_pipeline_cache_size.restype = sz
+    lib.dh_agg_col_noalloc_f32.argtypes = [ctxp, i32, vp, vp, sz, sz, sz]
+    lib.dh_agg_col_noalloc_scratch_bytes.argtypes = []
+    lib.dh_agg_col_noalloc_scratch_bytes.restype = sz
     lib.dh_timer_stop_ms.argtypes = [ctxp, C.POINTER(C.c_float)]
     for suf, ct in (("f32", C.c_float), ("f64", C.c_double)):
         f = lambda name: getattr(lib, f"{name}_{suf}")

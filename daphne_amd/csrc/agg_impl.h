@@ -1177,12 +1177,28 @@ template <typename T> static inline ColPlan col_plan(const dh_ctx *ctx, const T 
     return p;
 }
 
+// Where the per-block partials of a column aggregation live: the context's workspace (grown on demand), or a
+// buffer the caller of agg_col brings along, which is then never grown - a request beyond it is an error.
+struct ColScratch {
+    void *buf = nullptr;
+    size_t bytes = 0;
+};
+static inline dh_status col_partials(dh_ctx *ctx, const ColScratch &sc, size_t need, void **out) {
+    if (sc.buf == nullptr)
+        return dh_workspace(ctx, need, out);
+    if (need > sc.bytes)
+        return dh_fail(DH_ERR_RUNTIME, "AggCol - %zu bytes of partial results do not fit the fixed scratch buffer of %zu bytes",
+                       need, sc.bytes);
+    *out = sc.buf;
+    return DH_OK;
+}
+
 template <typename T, class R, int FINAL, bool NANFIRST>
-static inline dh_status col_launch(dh_ctx *ctx, T *res, const T *arg, size_t rows, size_t cols, size_t ld) {
+static inline dh_status col_launch(dh_ctx *ctx, T *res, const T *arg, size_t rows, size_t cols, size_t ld, const ColScratch &sc) {
     constexpr int V = dh_vec<T>::N;
     ColPlan p = col_plan<T>(ctx, arg, rows, cols, ld);
     void *wsv = nullptr;
-    dh_status st = dh_workspace(ctx, p.nparts * cols * sizeof(T), &wsv);
+    dh_status st = col_partials(ctx, sc, p.nparts * cols * sizeof(T), &wsv);
     if (st != DH_OK)
         return st;
     T *partials = static_cast<T *>(wsv);
@@ -1196,7 +1212,8 @@ static inline dh_status col_launch(dh_ctx *ctx, T *res, const T *arg, size_t row
     return DH_OK;
 }
 
-template <typename T> dh_status agg_col(dh_ctx *ctx, int op, T *res, const T *arg, size_t rows, size_t cols, size_t ld) {
+template <typename T>
+dh_status agg_col(dh_ctx *ctx, int op, T *res, const T *arg, size_t rows, size_t cols, size_t ld, const ColScratch &sc = ColScratch()) {
     DH_REQUIRE_CTX(ctx);
     if (ld < cols)
         return dh_fail(DH_ERR_RUNTIME, "AggCol - leading dimension smaller than the column count");
@@ -1213,26 +1230,26 @@ template <typename T> dh_status agg_col(dh_ctx *ctx, int op, T *res, const T *ar
     dh_status st = DH_OK;
     switch (op) {
     case DH_AGG_SUM:
-        st = col_launch<T, RSum<T>, 0, false>(ctx, res, arg, rows, cols, ld);
+        st = col_launch<T, RSum<T>, 0, false>(ctx, res, arg, rows, cols, ld, sc);
         break;
     case DH_AGG_PROD:
-        st = col_launch<T, RProd<T>, 0, false>(ctx, res, arg, rows, cols, ld);
+        st = col_launch<T, RProd<T>, 0, false>(ctx, res, arg, rows, cols, ld, sc);
         break;
     case DH_AGG_MIN:
-        st = col_launch<T, RMin<T>, 0, true>(ctx, res, arg, rows, cols, ld);
+        st = col_launch<T, RMin<T>, 0, true>(ctx, res, arg, rows, cols, ld, sc);
         break;
     case DH_AGG_MAX:
-        st = col_launch<T, RMax<T>, 0, true>(ctx, res, arg, rows, cols, ld);
+        st = col_launch<T, RMax<T>, 0, true>(ctx, res, arg, rows, cols, ld, sc);
         break;
     case DH_AGG_MEAN:
-        st = col_launch<T, RSum<T>, 1, false>(ctx, res, arg, rows, cols, ld);
+        st = col_launch<T, RSum<T>, 1, false>(ctx, res, arg, rows, cols, ld, sc);
         break;
     case DH_AGG_VAR:
     case DH_AGG_STDDEV: {
         constexpr int V = dh_vec<T>::N;
         ColPlan p = col_plan<T>(ctx, arg, rows, cols, ld);
         void *wsv = nullptr;
-        st = dh_workspace(ctx, 2 * p.nparts * cols * sizeof(T), &wsv);
+        st = col_partials(ctx, sc, 2 * p.nparts * cols * sizeof(T), &wsv);
         if (st != DH_OK)
             return st;
         T *pm = static_cast<T *>(wsv);

@@ -99,6 +99,9 @@ dh_status dh_fail(dh_status st, const char *fmt, ...) __attribute__((format(prin
 // buffer after a stream synchronise.
 dh_status dh_workspace(dh_ctx *ctx, size_t bytes, void **out);
 
+// agg_noalloc.hip: looks up the address of the current device's fixed scratch array (once per device).
+dh_status dh_noalloc_bind_device(int device);
+
 static inline size_t dh_ceil_div(size_t a, size_t b) { return (a + b - 1) / b; }
 static inline bool dh_aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
 

@@ -72,6 +72,11 @@ extern "C" dh_status dh_ctx_create(int device, dh_ctx **out) {
         dh_ctx_destroy(ctx);
         return dh_fail(DH_ERR_HIP, "dh_ctx_create: could not allocate the context's flag words / events");
     }
+    // the fixed scratch array of the entry point that allocates nothing: bound here, with the device current
+    if (dh_status st = dh_noalloc_bind_device(device); st != DH_OK) {
+        dh_ctx_destroy(ctx);
+        return st;
+    }
     *out = ctx;
     return DH_OK;
 }

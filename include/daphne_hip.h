@@ -193,6 +193,18 @@ dh_status dh_agg_col_f32(dh_ctx *ctx, int op, float *res, const float *arg, size
                          size_t cols, size_t ld);
 dh_status dh_agg_col_f64(dh_ctx *ctx, int op, double *res, const double *arg, size_t rows,
                          size_t cols, size_t ld);
+/* dh_agg_col_f32 for callers that cannot allocate (code under HIP stream capture, tight serving loops,
+ * harnesses that forbid hipMalloc). It has no counterpart in the reference. Same arguments, op codes and
+ * results as dh_agg_col_f32, bit for bit; the partial results of its two kernels go to a fixed 8 MiB array
+ * in device memory that the library holds per GPU, so the call reaches no hipMalloc / hipFree. An input whose
+ * partials (4 B x columns x row slabs; twice that for VAR / STDDEV) exceed the array fails with DH_ERR_RUNTIME
+ * and leaves res untouched; the slab count shrinks as the matrix gets wider, so on a 256-CU device that only
+ * happens beyond 2 Mi columns (1 Mi for VAR / STDDEV). All calls on one GPU share the array: calls that overlap on one GPU race, calls in stream order
+ * do not. */
+dh_status dh_agg_col_noalloc_f32(dh_ctx *ctx, int op, float *res, const float *arg, size_t rows,
+                                 size_t cols, size_t ld);
+/* Size of that array in bytes. */
+size_t dh_agg_col_noalloc_scratch_bytes(void);
 /* colMeans and colVars (or colStddevs when `stddev` != 0) of the same matrix in ONE pass: what
  * dh_agg_col with DH_AGG_MEAN and DH_AGG_VAR / DH_AGG_STDDEV (kernels/AggCol.h:143-170) return, for a
  * caller - a fused pipeline, or a rewrite of mean(X,1) + var(X,1) on one input - that needs both. The
