@@ -1,8 +1,10 @@
-"""Builds libdaphne_hip.so (gfx950 only) with hipcc. No GPU is needed to build.
+"""Builds libdaphne_hip.so (gfx950 only) with hipcc, and on top of it libHIPKernels.so, the generated
+`HIP_<mnemonic>__<types>` entry points that DAPHNE's compiled programs call, with its catalog. No GPU is needed to build.
 
-    python -m daphne_amd.build          # compile every .hip under csrc/ and link
+    python -m daphne_amd.build          # compile every .hip under csrc/ and link, then the kernel library
 
-The library is placed next to this file so that it is found without installation.
+libdaphne_hip.so is placed next to this file so that it is found without installation; libHIPKernels.so and
+HIPcatalog.json go to cpp/lib/ (the catalog names the library by a path relative to itself).
 """
 from __future__ import annotations
 
@@ -17,6 +19,16 @@ PKG_DIR = Path(__file__).resolve().parent
 CSRC = PKG_DIR / "csrc"
 OBJ_DIR = CSRC / "build"
 LIB_PATH = PKG_DIR / "libdaphne_hip.so"
+CPP_DIR = PKG_DIR / "cpp"
+KERNEL_SRC_DIR = CPP_DIR / "src" / "runtime" / "local" / "kernels" / "HIP"
+KERNEL_SPEC = KERNEL_SRC_DIR / "HIPkernels.json"
+KERNEL_GENERATOR = KERNEL_SRC_DIR / "genHIPKernelInst.py"
+KERNEL_LIB_DIR = CPP_DIR / "lib"
+KERNEL_LIB_PATH = KERNEL_LIB_DIR / "libHIPKernels.so"
+KERNEL_CATALOG_PATH = KERNEL_LIB_DIR / "HIPcatalog.json"
+# host-side C++ of the kernel layer: DAPHNE's include paths, served here by the stand-in headers
+HOST_CXX_FLAGS = ["-std=c++17", "-O1", "-Wall", f"-I{CPP_DIR / 'src'}", f"-I{CPP_DIR / 'standalone'}",
+                  f"-I{PKG_DIR.parent / 'include'}"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",
@@ -36,9 +48,13 @@ def _hipcc() -> str:
     return exe
 
 
+# The interpreting pipeline kernel rounds every operator of a body by itself, like the run-time specialised one.
+EXTRA_FLAGS = {"pipeline_f32.hip": ["-ffp-contract=off"], "pipeline_f64.hip": ["-ffp-contract=off"]}
+
+
 def _compile(src: Path) -> Path:
     obj = OBJ_DIR / (src.stem + ".o")
-    cmd = [_hipcc(), *HIPCC_FLAGS, "-c", str(src), "-o", str(obj)]
+    cmd = [_hipcc(), *HIPCC_FLAGS, *EXTRA_FLAGS.get(src.name, []), "-c", str(src), "-o", str(obj)]
     proc = subprocess.run(cmd, capture_output=True, text=True)
     if proc.returncode != 0:
         raise RuntimeError(f"hipcc failed for {src.name}:\n{proc.stderr}")
@@ -99,6 +115,33 @@ def build_all(jobs: int | None = None, verbose: bool = True) -> Path:
     return LIB_PATH
 
 
+def generate_kernel_sources() -> Path:
+    """Runs the generator: cpp/build/HIPkernels.cpp and cpp/lib/HIPcatalog.json from HIPkernels.json."""
+    out_cpp = CPP_DIR / "build" / "HIPkernels.cpp"
+    proc = subprocess.run([sys.executable, str(KERNEL_GENERATOR), str(KERNEL_SPEC), str(out_cpp), str(KERNEL_CATALOG_PATH), "HIP"],
+                          capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"kernel generator failed:\n{proc.stdout}{proc.stderr}")
+    return out_cpp
+
+
+def build_kernel_library(verbose: bool = True) -> Path:
+    """libHIPKernels.so: the generated entry points over the C++ kernel layer, compiled by the host compiler."""
+    out_cpp = generate_kernel_sources()
+    cxx = shutil.which("g++") or shutil.which("c++")
+    if cxx is None:
+        raise RuntimeError("no host C++ compiler found; libHIPKernels.so cannot be built")
+    cmd = [cxx, *HOST_CXX_FLAGS, "-fPIC", "-shared", str(out_cpp), "-o", str(KERNEL_LIB_PATH), f"-L{PKG_DIR}", "-ldaphne_hip",
+           "-Wl,-rpath,$ORIGIN/../.."]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"compiling the kernel library failed:\n{proc.stderr}")
+    if verbose:
+        print(f"[daphne_amd.build] wrote {KERNEL_LIB_PATH} and {KERNEL_CATALOG_PATH}", flush=True)
+    return KERNEL_LIB_PATH
+
+
 if __name__ == "__main__":
     build_all()
+    build_kernel_library()
     sys.exit(0)

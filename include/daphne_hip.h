@@ -118,6 +118,12 @@ dh_status dh_ctx_release_cached(dh_ctx *ctx);
 dh_status dh_h2d(dh_ctx *ctx, void *dst_dev, const void *src_host, size_t bytes);
 dh_status dh_d2h(dh_ctx *ctx, void *dst_host, const void *src_dev, size_t bytes);
 dh_status dh_d2d(dh_ctx *ctx, void *dst_dev, const void *src_dev, size_t bytes);
+/* `rows` rows of `width_bytes` bytes between two pitched device buffers, in the order of the context's stream:
+ * how a vectorized-pipeline task puts a row share's result into its place in the whole result
+ * (CompiledPipelineTaskCUDA::accumulateOutputs, runtime/local/vectorized/TasksCUDA.cpp:73-100, one cudaMemcpy
+ * per share or per row there). */
+dh_status dh_d2d_2d(dh_ctx *ctx, void *dst_dev, size_t dst_pitch, const void *src_dev, size_t src_pitch,
+                    size_t width_bytes, size_t rows);
 
 /* Stream-ordered stopwatch on the context's stream (hipEvent pair). dh_timer_stop_ms
  * synchronises on the stop event and returns the elapsed milliseconds. */

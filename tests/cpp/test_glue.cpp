@@ -4,6 +4,7 @@
 // literals are the reference's own test vectors. Built with a plain host compiler.
 #include <cmath>
 #include <cstdio>
+#include <functional>
 #include <memory>
 #include <stdexcept>
 #include <vector>
@@ -48,7 +49,7 @@ template <class DT> bool approx(const DT *m, const std::vector<typename DT::VT> 
 
 template <typename VT> void run_all(DaphneContext *dctx) {
     using DT = DenseMatrix<VT>;
-    auto G = [&](size_t rows, std::vector<VT> v) { return genGivenVals<DT>(rows, v, dctx); };
+    auto G = [&](size_t rows, std::vector<VT> v) { return genGivenVals<DT>(rows, v); };
 
     // CUDA/MatMulTest.cpp:37-123
     {
@@ -222,11 +223,11 @@ template <typename VT> void run_all(DaphneContext *dctx) {
         CHECK(threw);
         auto arg = G(3, {1, 2, 3, 4, 5, 6, 7, 8, 9});
         using DTSel = DenseMatrix<int64_t>;
-        auto sel = genGivenVals<DTSel>(8, {1, 2, 2, 0, 1, 0, 1, 2}, dctx);
+        auto sel = genGivenVals<DTSel>(8, {1, 2, 2, 0, 1, 0, 1, 2});
         DT *ex = nullptr;
         HIP::extractCol(ex, arg, sel, dctx);
         CHECK(equals(ex, {2, 3, 3, 1, 2, 1, 2, 3, 5, 6, 6, 4, 5, 4, 5, 6, 8, 9, 9, 7, 8, 7, 8, 9}));
-        auto selbad = genGivenVals<DTSel>(2, {1, 3}, dctx);
+        auto selbad = genGivenVals<DTSel>(2, {1, 3});
         threw = false;
         try {
             DT *bad = nullptr;
@@ -286,7 +287,7 @@ template <typename VT> void run_all(DaphneContext *dctx) {
 // DNNBatchNorm2DBackwardTest.cpp:22-70, DNNBatchNorm2DForwardTest.cpp:51-90)
 template <typename VT> void run_training(DaphneContext *dctx) {
     using DT = DenseMatrix<VT>;
-    auto G = [&](size_t rows, std::vector<VT> v) { return genGivenVals<DT>(rows, v, dctx); };
+    auto G = [&](size_t rows, std::vector<VT> v) { return genGivenVals<DT>(rows, v); };
     {
         auto dy = G(1, {1, 2, 3, 4, 5, 6, 7, 8});
         auto filter = G(2, {1, 0, 0, 2, 2, 0, 0, 3, 3, 0, 0, 4, 5, 0, 0, 6, 6, 0, 0, 7, 7, 0, 0, 8});
@@ -352,7 +353,7 @@ template <typename VT> void run_training(DaphneContext *dctx) {
 // int64_t among others): the reference's literals where they are integers, plus integer-only behaviour.
 template <typename VT> void run_integer_elementwise(DaphneContext *dctx) {
     using DT = DenseMatrix<VT>;
-    auto G = [&](size_t rows, std::vector<VT> v) { return genGivenVals<DT>(rows, v, dctx); };
+    auto G = [&](size_t rows, std::vector<VT> v) { return genGivenVals<DT>(rows, v); };
     // EwBinaryMatTest.cpp:69-102 (add), :104-125 (mul), :178-222 (div), :523-557 (max)
     auto m1 = G(2, {1, 2, 0, 0, 1, 3}), m2 = G(2, {0, 9, 0, 0, 3, 4}), m3 = G(2, {1, 11, 0, 0, 4, 7});
     DT *res = nullptr;
@@ -380,7 +381,7 @@ template <typename VT> void run_integer_elementwise(DaphneContext *dctx) {
 
 static void run_si64(DaphneContext *dctx) {
     using DT = DenseMatrix<int64_t>;
-    auto G = [&](size_t rows, std::vector<int64_t> v) { return genGivenVals<DT>(rows, v, dctx); };
+    auto G = [&](size_t rows, std::vector<int64_t> v) { return genGivenVals<DT>(rows, v); };
     // AggRowTest.cpp / AggColTest.cpp literal, AggAllTest.cpp:62-75
     auto m = G(3, {3, 0, 2, 0, 0, 0, 1, 0, 0, 1, 0, 3});
     CHECK(HIP::aggAll<int64_t>(AggOpCode::SUM, m, dctx) == 10);
@@ -406,7 +407,309 @@ static void run_si64(DaphneContext *dctx) {
     DataObjectFactory::destroy(idx);
 }
 
-int main() {
+// ------------------------------------------------------------------------------------------------
+// Data placement: what DenseMatrix::getValues(&alloc_desc) and AllocationDescriptorHIP do together
+// (DenseMatrix.cpp:126-234, AllocationDescriptorCUDA.h:24-75)
+// ------------------------------------------------------------------------------------------------
+template <class DT> int whereIs(const DT *m) {
+    const MetaDataObject *mdo = m->getMetaDataObject();
+    int where = 0;
+    for (size_t id : mdo->getLatest())
+        where |= mdo->getDataPlacementByID(id)->allocation->getType() == ALLOCATION_TYPE::HOST ? 1 : 2;
+    return where;
+}
+static void run_placement(DaphneContext *dctx) {
+    using DT = DenseMatrix<float>;
+    HIPContext *hc = HIPContext::get(dctx, 0);
+    const size_t allocs0 = hc->numAllocations();
+    const size_t used0 = hc->getMemInUse();
+    auto a = genGivenVals<DT>(2, {1, 2, 3, 4, 5, 6});
+    CHECK(whereIs(a) == 1 && a->getMetaDataObject()->numDataPlacements() == 1); // host only, nothing uploaded yet
+    CHECK(hc->numAllocations() == allocs0);
+    DT *r = nullptr;
+    HIP::ewBinaryObjSca(BinaryOpCode::MUL, r, a, 2.0f, dctx);
+    // the input was uploaded on first use and both copies stay valid; the result exists on the device only
+    CHECK(whereIs(a) == 3 && a->getMetaDataObject()->numDataPlacements() == 2);
+    CHECK(whereIs(r) == 2 && r->getMetaDataObject()->numDataPlacements() == 1);
+    CHECK(hc->numAllocations() == allocs0 + 2);
+    // a second use finds the device copy: no further placement, no further allocation
+    DT *r2 = nullptr;
+    HIP::ewBinaryMat(BinaryOpCode::ADD, r2, a, r, dctx);
+    CHECK(a->getMetaDataObject()->numDataPlacements() == 2 && hc->numAllocations() == allocs0 + 3);
+    // reading the result on the host downloads it once; both copies are then current
+    CHECK(equals(r2, {3, 6, 9, 12, 15, 18}));
+    CHECK(whereIs(r2) == 3);
+    // writing on the host makes the device copy stale; the next kernel uploads again and sees the new value
+    a->set(0, 0, 10.f);
+    CHECK(whereIs(a) == 1);
+    HIP::ewBinaryObjSca(BinaryOpCode::MUL, r, a, 2.0f, dctx); // in place into r
+    CHECK(whereIs(a) == 3 && whereIs(r) == 2);
+    CHECK(equals(r, {20, 4, 6, 8, 10, 12}));
+    // a kernel that writes into a matrix makes its host copy stale
+    HIP::ewBinaryObjSca(BinaryOpCode::ADD, a, a, 1.0f, dctx);
+    CHECK(whereIs(a) == 2);
+    CHECK(equals(a, {11, 3, 4, 5, 6, 7}));
+    // views share their parent's placements: a kernel on a view sees device data without another upload
+    std::unique_ptr<DT> v(a->sliceRow(1, 2));
+    DT *rv = nullptr;
+    HIP::ewBinaryObjSca(BinaryOpCode::SUB, rv, v.get(), 1.0f, dctx);
+    CHECK(equals(rv, {4, 5, 6}));
+    CHECK(a->getMetaDataObject()->numDataPlacements() == 2);
+    v.reset();
+    // destroying the matrices gives the device memory back
+    DataObjectFactory::destroy(a, r, r2, rv);
+    CHECK(hc->numAllocations() == allocs0);
+    CHECK(hc->getMemInUse() == used0);
+}
+
+// ------------------------------------------------------------------------------------------------
+// Vectorized pipeline on the device: tasks over row shares, outputs combined
+// (MultiThreadedKernelTest.cpp:30-154 bodies; TasksCUDA.cpp:21-119; MTWrapper_dense.cpp:339-373)
+// ------------------------------------------------------------------------------------------------
+// bodies as the compiler outlines them: operator by operator, results through *outputs[i], inputs given back
+template <class DT> void funAdd(DT ***outputs, Structure **inputs, DCTX(ctx)) {
+    auto *l = static_cast<DT *>(inputs[0]), *r = static_cast<DT *>(inputs[1]);
+    HIP::ewBinaryMat(BinaryOpCode::ADD, *outputs[0], l, r, ctx);
+    DataObjectFactory::destroy(l, r);
+}
+template <class DT> void funMul(DT ***outputs, Structure **inputs, DCTX(ctx)) {
+    auto *l = static_cast<DT *>(inputs[0]), *r = static_cast<DT *>(inputs[1]);
+    HIP::ewBinaryMat(BinaryOpCode::MUL, *outputs[0], l, r, ctx);
+    DataObjectFactory::destroy(l, r);
+}
+// a body that ignores the offered output and returns a matrix of its own, like the reference's compiled bodies
+template <class DT> void funAddFresh(DT ***outputs, Structure **inputs, DCTX(ctx)) {
+    auto *l = static_cast<DT *>(inputs[0]), *r = static_cast<DT *>(inputs[1]);
+    DT *fresh = nullptr;
+    HIP::ewBinaryMat(BinaryOpCode::ADD, fresh, l, r, ctx);
+    *outputs[0] = fresh;
+    DataObjectFactory::destroy(l, r);
+}
+// outputs: 0 = (x - mu) * (x - mu) by ROWS, 1 = column sums by ADD, 2 = column minima by MIN, 3 = column maxima by MAX
+template <class DT> void funStats(DT ***outputs, Structure **inputs, DCTX(ctx)) {
+    auto *x = static_cast<DT *>(inputs[0]), *mu = static_cast<DT *>(inputs[1]);
+    DT *c = nullptr;
+    HIP::ewBinaryMat(BinaryOpCode::SUB, c, x, mu, ctx);
+    HIP::ewBinaryMat(BinaryOpCode::MUL, *outputs[0], c, c, ctx);
+    HIP::aggCol(AggOpCode::SUM, *outputs[1], x, ctx);
+    HIP::aggCol(AggOpCode::MIN, *outputs[2], x, ctx);
+    HIP::aggCol(AggOpCode::MAX, *outputs[3], x, ctx);
+    DataObjectFactory::destroy(c, x, mu);
+}
+
+template <typename VT> void run_pipeline_tasks(DaphneContext *dctx) {
+    using DT = DenseMatrix<VT>;
+    using Fn = void (*)(DT ***, Structure **, DCTX(ctx));
+    const size_t rows = 1234, cols = 10;
+    std::vector<VT> a(rows * cols), b(rows * cols);
+    uint32_t s = 12345u;
+    auto rnd = [&] { // values in [0, 1), as randMatrix(..., 0.0, 1.0, ...) in the reference's test
+        s = s * 1664525u + 1013904223u;
+        return VT((s >> 8) * (1.0 / 16777216.0));
+    };
+    for (auto &v : a)
+        v = rnd();
+    for (auto &v : b)
+        v = rnd();
+    auto m1 = genGivenVals<DT>(rows, a), m2 = genGivenVals<DT>(rows, b);
+    bool isScalar[] = {false, false};
+    Structure *inputs[] = {m1, m2};
+    int64_t outRows[] = {int64_t(rows)}, outCols[] = {int64_t(cols)};
+    int64_t splits[] = {int64_t(VectorSplit::ROWS), int64_t(VectorSplit::ROWS)};
+    int64_t combines[] = {int64_t(VectorCombine::ROWS)};
+    struct Case {
+        uint64_t shares, batch;
+    };
+    const Case cases[] = {{1, 0}, {2, 0}, {7, 0}, {3, 100}, {1, 1000}};
+    for (Fn fn : {Fn(&funAdd<DT>), Fn(&funMul<DT>), Fn(&funAddFresh<DT>)}) {
+        DT *whole = nullptr; // single call on the whole matrices
+        HIP::ewBinaryMat(fn == Fn(&funMul<DT>) ? BinaryOpCode::MUL : BinaryOpCode::ADD, whole, m1, m2, dctx);
+        const auto expect = whole->toHost();
+        bool host_ok = true;
+        for (size_t i = 0; i < expect.size(); i++)
+            host_ok &= expect[i] == (fn == Fn(&funMul<DT>) ? a[i] * b[i] : a[i] + b[i]);
+        CHECK(host_ok);
+        for (const Case &c : cases) {
+            dctx->config.hip_vect_shares = c.shares;
+            dctx->config.hip_vect_batch_rows = c.batch;
+            DT *out[] = {nullptr};
+            void *fun[] = {reinterpret_cast<void *>(fn)};
+            HIP::vectorizedPipeline<DT>(out, 1, isScalar, inputs, 2, outRows, outCols, splits, combines, 1, fun, dctx);
+            CHECK(out[0] != nullptr && out[0]->getNumRows() == rows && out[0]->getNumCols() == cols);
+            CHECK(whereIs(out[0]) == 2); // combined on the device, not through the host
+            CHECK(out[0]->toHost() == expect); // ROWS: bit for bit the whole-matrix result
+            DataObjectFactory::destroy(out[0]);
+        }
+        DataObjectFactory::destroy(whole);
+    }
+    CHECK(m1->getRefCounter() == 1 && m2->getRefCounter() == 1);
+
+    // ROWS + ADD + MIN + MAX in one pipeline, a broadcast input, op-by-op body
+    {
+        DT *mu = nullptr;
+        HIP::aggCol(AggOpCode::MEAN, mu, m1, dctx);
+        DT *c = nullptr, *sq = nullptr, *sum = nullptr, *mn = nullptr, *mx = nullptr;
+        HIP::ewBinaryMat(BinaryOpCode::SUB, c, m1, mu, dctx);
+        HIP::ewBinaryMat(BinaryOpCode::MUL, sq, c, c, dctx);
+        HIP::aggCol(AggOpCode::SUM, sum, m1, dctx);
+        HIP::aggCol(AggOpCode::MIN, mn, m1, dctx);
+        HIP::aggCol(AggOpCode::MAX, mx, m1, dctx);
+        bool isScalar2[] = {false, false};
+        Structure *inputs2[] = {m1, mu};
+        int64_t outRows2[] = {int64_t(rows), 1, 1, 1}, outCols2[] = {int64_t(cols), int64_t(cols), int64_t(cols), int64_t(cols)};
+        int64_t splits2[] = {int64_t(VectorSplit::ROWS), int64_t(VectorSplit::NONE)};
+        int64_t combines2[] = {int64_t(VectorCombine::ROWS), int64_t(VectorCombine::ADD), int64_t(VectorCombine::MIN),
+                               int64_t(VectorCombine::MAX)};
+        const double tol = std::is_same<VT, float>::value ? 1e-4 : 1e-12; // sums of 1234 values in [0,1) in another order
+        for (const Case &cs : cases) {
+            dctx->config.hip_vect_shares = cs.shares;
+            dctx->config.hip_vect_batch_rows = cs.batch;
+            DT *out[] = {nullptr, nullptr, nullptr, nullptr};
+            void *fun[] = {reinterpret_cast<void *>(Fn(&funStats<DT>))};
+            HIP::vectorizedPipeline<DT>(out, 4, isScalar2, inputs2, 2, outRows2, outCols2, splits2, combines2, 1, fun, dctx);
+            CHECK(out[0]->toHost() == sq->toHost());
+            const auto got = out[1]->toHost(), want = sum->toHost();
+            bool ok = got.size() == want.size();
+            for (size_t i = 0; ok && i < got.size(); i++)
+                ok = std::fabs(double(got[i]) - double(want[i])) <= tol * std::fabs(double(want[i]));
+            CHECK(ok);
+            CHECK(out[2]->toHost() == mn->toHost()); // MIN / MAX do not depend on the order
+            CHECK(out[3]->toHost() == mx->toHost());
+            DataObjectFactory::destroy(out[0], out[1], out[2], out[3]);
+        }
+        CHECK(mu->getRefCounter() == 1);
+        DataObjectFactory::destroy(mu, c, sq, sum, mn, mx);
+    }
+
+    // the same shape of work as ONE kernel per batch: z = (x - mu) / sd by ROWS, r = rowSums(z * z) by ROWS,
+    // count of r > thr by ADD, largest r by MAX
+    {
+        DT *mu = nullptr, *var = nullptr, *sd = nullptr;
+        HIP::aggCol(AggOpCode::MEAN, mu, m1, dctx);
+        HIP::aggCol(AggOpCode::VAR, var, m1, dctx);
+        HIP::ewUnaryMat(UnaryOpCode::SQRT, sd, var, dctx);
+        const VT thr = VT(10);
+        auto I = [](int kind, int op, int domain, int operand, int index, double scalar = 0) {
+            return dh_pipe_instr{kind, op, domain, operand, index, 0, scalar};
+        };
+        HIP::FusedPipelineBody<VT> body;
+        body.program = {I(DH_PIPE_EW_BINARY, int(BinaryOpCode::SUB), 0, DH_OPD_ROWVEC, 0),
+                        I(DH_PIPE_EW_BINARY, int(BinaryOpCode::DIV), 0, DH_OPD_ROWVEC, 1),
+                        I(DH_PIPE_STORE_TILE, 0, 0, 0, 0),
+                        I(DH_PIPE_EW_BINARY, int(BinaryOpCode::MUL), 0, DH_OPD_SELF, 0),
+                        I(DH_PIPE_ROW_AGG, int(AggOpCode::SUM), 0, 0, 0),
+                        I(DH_PIPE_STORE_ROW, 0, 1, 0, 0),
+                        I(DH_PIPE_REDUCE_ALL, int(AggOpCode::MAX), 1, 0, 1),
+                        I(DH_PIPE_EW_BINARY, int(BinaryOpCode::GT), 1, DH_OPD_SCALAR, 0, double(thr)),
+                        I(DH_PIPE_REDUCE_ALL, int(AggOpCode::SUM), 1, 0, 0)};
+        body.inputs = {{HIP::PipeInput::PRIMARY, 0}, {HIP::PipeInput::ROWVEC, 0}, {HIP::PipeInput::ROWVEC, 1}};
+        body.outputs = {{HIP::PipeOutput::TILE, 0}, {HIP::PipeOutput::ROW, 0}, {HIP::PipeOutput::ALL, 0}, {HIP::PipeOutput::ALL, 1}};
+        // op by op on the whole matrix
+        DT *c = nullptr, *z = nullptr, *zz = nullptr, *r = nullptr, *gt = nullptr;
+        HIP::ewBinaryMat(BinaryOpCode::SUB, c, m1, mu, dctx);
+        HIP::ewBinaryMat(BinaryOpCode::DIV, z, c, sd, dctx);
+        HIP::ewBinaryMat(BinaryOpCode::MUL, zz, z, z, dctx);
+        HIP::aggRow(AggOpCode::SUM, r, zz, dctx);
+        HIP::ewBinaryObjSca(BinaryOpCode::GT, gt, r, thr, dctx);
+        const VT count = HIP::aggAll<VT, DT>(AggOpCode::SUM, gt, dctx), rmax = HIP::aggAll<VT, DT>(AggOpCode::MAX, r, dctx);
+        CHECK(count > VT(0) && count < VT(rows)); // the threshold splits the rows
+        bool isScalar3[] = {false, false, false};
+        Structure *inputs3[] = {m1, mu, sd};
+        int64_t outRows3[] = {int64_t(rows), int64_t(rows), 1, 1}, outCols3[] = {int64_t(cols), 1, 1, 1};
+        int64_t splits3[] = {int64_t(VectorSplit::ROWS), int64_t(VectorSplit::NONE), int64_t(VectorSplit::NONE)};
+        VectorCombine combines3[] = {VectorCombine::ROWS, VectorCombine::ROWS, VectorCombine::ADD, VectorCombine::MAX};
+        const double tol = std::is_same<VT, float>::value ? 1e-5 : 1e-13;
+        for (const Case &cs : cases) {
+            dctx->config.hip_vect_shares = cs.shares;
+            dctx->config.hip_vect_batch_rows = cs.batch;
+            DT *out[] = {nullptr, nullptr, nullptr, nullptr};
+            std::vector<std::function<void(DT ***, Structure **, DCTX(ctx))>> funcs{body};
+            HIP::VectorizedPipeline<DT>::apply(out, 4, isScalar3, inputs3, 3, outRows3, outCols3,
+                                               reinterpret_cast<const VectorSplit *>(splits3), combines3, funcs, dctx);
+            CHECK(out[0]->toHost() == z->toHost()); // same IEEE operations per element: bit for bit
+            const auto got = out[1]->toHost(), want = r->toHost();
+            bool ok = got.size() == want.size();
+            for (size_t i = 0; ok && i < got.size(); i++)
+                ok = std::fabs(double(got[i]) - double(want[i])) <= tol * std::fabs(double(want[i]));
+            CHECK(ok);
+            // rows whose r is within rounding of the threshold may fall on either side
+            size_t ambiguous = 0;
+            for (VT v : want)
+                ambiguous += std::fabs(double(v) - double(thr)) <= tol * double(thr);
+            CHECK(std::fabs(double(out[2]->toHost()[0]) - double(count)) <= double(ambiguous));
+            CHECK(std::fabs(double(out[3]->toHost()[0]) - double(rmax)) <= tol * double(rmax));
+            DataObjectFactory::destroy(out[0], out[1], out[2], out[3]);
+        }
+        DataObjectFactory::destroy(mu, var, sd, c, z);
+        DataObjectFactory::destroy(zz, r, gt);
+    }
+    dctx->config.hip_vect_shares = 1;
+    dctx->config.hip_vect_batch_rows = 0;
+    CHECK(m1->getRefCounter() == 1);
+    DataObjectFactory::destroy(m1, m2);
+}
+
+// ------------------------------------------------------------------------------------------------
+// The generated entry points of libHIPKernels.so, called the way a compiled program calls them
+// (genKernelInst.py:132-154, 236-262; ErrorHandler.cpp:80-90)
+// ------------------------------------------------------------------------------------------------
+#include <dlfcn.h>
+static void run_generated_wrappers(DaphneContext *dctx, const char *lib_path) {
+    using DT = DenseMatrix<double>;
+    void *lib = dlopen(lib_path, RTLD_NOW | RTLD_LOCAL);
+    if (!lib) {
+        std::printf("FAILED to load %s: %s\n", lib_path, dlerror());
+        g_fail++;
+        return;
+    }
+    using EwFn = void (*)(DT **, const DT *, const DT *, int, DaphneContext *);
+    using AggFn = void (*)(double *, const DT *, int, DaphneContext *);
+    using UnFn = void (*)(DT **, const DT *, int, DaphneContext *);
+    auto ewAdd = reinterpret_cast<EwFn>(dlsym(lib, "HIP_ewAdd__DenseMatrix_double__DenseMatrix_double__DenseMatrix_double"));
+    auto sumAll = reinterpret_cast<AggFn>(dlsym(lib, "HIP_sumAll__double__DenseMatrix_double"));
+    auto ewSqrt = reinterpret_cast<UnFn>(dlsym(lib, "HIP_ewSqrt__DenseMatrix_double__DenseMatrix_double"));
+    CHECK(ewAdd && sumAll && ewSqrt);
+    if (!(ewAdd && sumAll && ewSqrt))
+        return;
+    const int kAdd = dctx->dispatchMapping.registerKernel("HIP_ewAdd__DenseMatrix_double__DenseMatrix_double__DenseMatrix_double",
+                                                          "script.daphne", 3, 7);
+    const int kSum = dctx->dispatchMapping.registerKernel("HIP_sumAll__double__DenseMatrix_double", "script.daphne", 4, 1);
+    const int kSqrt = dctx->dispatchMapping.registerKernel("HIP_ewSqrt__DenseMatrix_double__DenseMatrix_double", "script.daphne", 5, 2);
+    auto a = genGivenVals<DT>(2, {1, 2, 3, 4}), b = genGivenVals<DT>(2, {10, 20, 30, 40}), bad = genGivenVals<DT>(3, {1, 2, 3});
+    dctx->config.enable_statistics = true;
+    DT *res = nullptr;
+    ewAdd(&res, a, b, kAdd, dctx);
+    CHECK(res != nullptr && equals(res, {11, 22, 33, 44}));
+    double total = 0;
+    sumAll(&total, res, kSum, dctx);
+    CHECK(total == 110);
+    CHECK(dctx->kernel_stats[kAdd].first == 1 && dctx->kernel_stats[kSum].first == 1);
+    dctx->config.enable_statistics = false;
+    // a kernel's exception comes out as the run-time error of the call site: kernel name, message, position
+    std::string what;
+    try {
+        DT *r2 = nullptr;
+        ewAdd(&r2, a, bad, kAdd, dctx);
+    } catch (const std::runtime_error &e) {
+        what = e.what();
+    }
+    CHECK(what.find("The kernel-function HIP_ewAdd__DenseMatrix_double__DenseMatrix_double__DenseMatrix_double failed during runtime") == 0);
+    CHECK(what.find("script.daphne:3:7") != std::string::npos);
+    what.clear();
+    auto neg = genGivenVals<DT>(1, {4, -1});
+    try {
+        DT *r3 = nullptr;
+        ewSqrt(&r3, neg, kSqrt, dctx);
+    } catch (const std::runtime_error &e) { // the domain error of the kernel, re-thrown as the call site's error
+        what = e.what();
+    }
+    CHECK(what.find("HIP_ewSqrt__DenseMatrix_double__DenseMatrix_double") != std::string::npos &&
+          what.find("script.daphne:5:2") != std::string::npos);
+    DataObjectFactory::destroy(a, b, bad, res, neg);
+    dlclose(lib);
+}
+
+int main(int argc, char **argv) {
     // test/runtime/local/kernels/CUDA_ContextTest.cpp:25-30
     auto dctx = std::make_unique<DaphneContext>();
     try {
@@ -426,6 +729,11 @@ int main() {
     run_integer_elementwise<int32_t>(dctx.get());
     run_integer_elementwise<uint32_t>(dctx.get());
     run_si64(dctx.get());
+    run_placement(dctx.get());
+    run_pipeline_tasks<float>(dctx.get());
+    run_pipeline_tasks<double>(dctx.get());
+    if (argc > 1) // path of libHIPKernels.so
+        run_generated_wrappers(dctx.get(), argv[1]);
     std::printf("%s: %d checks, %d failed\n", g_fail ? "FAILED" : "PASSED", g_checks, g_fail);
     return g_fail ? 1 : 0;
 }
