@@ -54,6 +54,7 @@ def _signatures(lib: C.CDLL) -> None:
     lib.dh_ctx_release_cached.argtypes = [ctxp]
     lib.dh_ctx_device.argtypes = [ctxp]
     lib.dh_ctx_props.argtypes = [ctxp, C.POINTER(i32), C.POINTER(i32), C.POINTER(sz), C.c_char_p, sz]
+    lib.dh_device_memory.argtypes = [i32, C.POINTER(sz), C.POINTER(sz)]
     lib.dh_ctx_set_stream.argtypes = [ctxp, vp]
     lib.dh_ctx_get_stream.argtypes = [ctxp]
     lib.dh_ctx_get_stream.restype = vp

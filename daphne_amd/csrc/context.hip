@@ -270,6 +270,25 @@ extern "C" dh_status dh_d2d(dh_ctx *ctx, void *dst_dev, const void *src_dev, siz
     return DH_OK;
 }
 
+extern "C" dh_status dh_device_memory(int device, size_t *free_bytes, size_t *total_bytes) {
+    int count = 0;
+    if (hipGetDeviceCount(&count) != hipSuccess || device < 0 || device >= count)
+        return dh_fail(DH_ERR_HIP, "dh_device_memory: no HIP device %d (%d visible)", device, count);
+    int prev = 0;
+    DH_CHECK_HIP(hipGetDevice(&prev));
+    DH_CHECK_HIP(hipSetDevice(device));
+    size_t f = 0, tot = 0;
+    const hipError_t e = hipMemGetInfo(&f, &tot);
+    (void)hipSetDevice(prev);
+    if (e != hipSuccess)
+        return dh_fail(DH_ERR_HIP, "dh_device_memory: hipMemGetInfo failed: %s", hipGetErrorString(e));
+    if (free_bytes)
+        *free_bytes = f;
+    if (total_bytes)
+        *total_bytes = tot;
+    return DH_OK;
+}
+
 extern "C" dh_status dh_d2d_2d(dh_ctx *ctx, void *dst_dev, size_t dst_pitch, const void *src_dev, size_t src_pitch,
                                size_t width_bytes, size_t rows) {
     DH_REQUIRE_CTX(ctx);

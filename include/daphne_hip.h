@@ -94,6 +94,10 @@ int dh_ctx_device(const dh_ctx *ctx);
 /* Number of compute units and the max engine clock in kHz (for roofline print-outs). */
 dh_status dh_ctx_props(const dh_ctx *ctx, int *compute_units, int *clock_khz, size_t *total_mem,
                        char *name, size_t name_cap);
+/* Free and total memory of a device, without a context: what the compiler's device-placement pass asks when it
+ * decides whether an operation's operands fit (compiler/lowering/MarkCUDAOpsPass.cpp:37-41 calls cudaMemGetInfo).
+ * DH_ERR_HIP when there is no such device. */
+dh_status dh_device_memory(int device, size_t *free_bytes, size_t *total_bytes);
 /* Enqueue kernels of this context on `hip_stream` (a hipStream_t; NULL = the default
  * stream, which is also the initial setting). The context never owns the stream. */
 dh_status dh_ctx_set_stream(dh_ctx *ctx, void *hip_stream);
