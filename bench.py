@@ -13,7 +13,11 @@ fused pipeline kernel alone (its bytes / its own duration, timed with events on 
 runs on). `cpu_baseline` times the reference's algorithm for the same pipeline (CPU restatement
 in oracle/, same operator-by-operator multithreaded engine) on a bounded row prefix.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--rows R] [--no-cpu]
+After the timed pipeline steps the same run measures the other half of the metric, the dense contractions at the
+sizes BASELINE.json quotes (MatMul f64 8192^3, MatMul f32 16384^3, Syrk f64 1e6 x 1024), and reports them in
+`config.contractions`; `--no-contractions` skips that.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--rows R] [--no-cpu] [--no-contractions]
 """
 from __future__ import annotations
 
@@ -28,6 +32,22 @@ sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 HBM_PEAK_GBS = 8000.0
+COUNTER_PROFILE = os.path.join("profiles", "zscore_pipeline_20Mx64_f32_hbm_counters.txt")
+
+
+def measured_traffic(kernel: str):
+    """HBM bytes per launch of `kernel` from the committed counter summary (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE,
+    scaled by a copy kernel of known size): the 'read KiB' and 'write KiB' columns of the kernel's row."""
+    try:
+        with open(os.path.join(ROOT, COUNTER_PROFILE)) as f:
+            for line in f:
+                cols = line.split()
+                if cols and cols[0] == kernel and len(cols) >= 5:
+                    return int(round((float(cols[2]) + float(cols[4])) * 1024))
+    except (OSError, ValueError):
+        pass
+    return None
+
 
 
 def main() -> int:
@@ -46,6 +66,8 @@ def main() -> int:
     ap.add_argument("--cpu-rows", type=int, default=20_000_000, help="row prefix timed on the host CPU")
     ap.add_argument("--cpu-reps", type=int, default=3, help="repetitions of the CPU baseline (median is reported)")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-contractions", action="store_true", help="skip the MatMul / Syrk measurements after the pipeline")
+    ap.add_argument("--contraction-steps", type=int, default=5)
     ap.add_argument("--calib", action="store_true",
                     help="also launch one plain elementwise copy of X (reads |X|, writes |X|): the known-size "
                          "kernel that hardware byte counters are scaled against")
@@ -152,6 +174,24 @@ def main() -> int:
 
     s_val = float(s.to_numpy()[0, 0])
     props = ctx.props()
+    # how the body ran: 1 = the kernel specialised at run time (what `roofline.kernel` names), 0 = the interpreter
+    from daphne_amd import capi
+
+    pipeline_mode = int(capi.lib().dh_vectorized_pipeline_last_mode())
+
+    xh = None
+    if not args.no_cpu:
+        xh = X_t[:min(args.cpu_rows, R)].cpu().numpy()
+
+    contractions = None
+    if not args.no_contractions:
+        import bench_other_configs
+
+        # the pipeline's matrices make room for the contraction operands (X keeps the torch tensor alive)
+        r.destroy()
+        pipe = X = X_t = None
+        torch.cuda.empty_cache()
+        contractions = bench_other_configs.measure_contractions(torch, ctx, args.contraction_steps, 1)
 
     cpu = None
     if not args.no_cpu:
@@ -159,7 +199,6 @@ def main() -> int:
 
         n_cpu = min(args.cpu_rows, R)
         threads = min(os.cpu_count() or 1, 16)
-        xh = X_t[:n_cpu].cpu().numpy()
         runs = []
         for _ in range(max(1, args.cpu_reps)):
             st, mu_c, sd_c, r_c, s_c, secs = orc.zscore_pipeline(xh, threads=threads, thr=thr)
@@ -201,6 +240,8 @@ def main() -> int:
             "stage_gbs": {"colMeans": round(bytes_s1 / t_s1 / 1e6, 1), "colVars+sqrt": round(bytes_s2 / t_s2 / 1e6, 1),
                           "fused_pipeline": round(bytes_s3 / t_s3 / 1e6, 1)},
             "count_r_gt_thr": s_val,
+            "pipeline_mode": "specialised" if pipeline_mode == 1 else "interpreted",
+            "contractions": contractions,
             "device": props["name"], "compute_units": props["compute_units"], "clock_khz": props["clock_khz"],
         },
         "roofline": {
@@ -210,15 +251,21 @@ def main() -> int:
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBS, 4),
-            # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE at the default shape
-            # (profiles/zscore_pipeline_20Mx64_f32_hbm_counters.txt): 4,999,986 KiB read + 95,583 KiB written
-            "traffic": 5217862494 if (R, Cc) == (20_000_000, 64) else None,
+            # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE at the default shape, read
+            # from the committed summary of those runs
+            "traffic": measured_traffic("dh_jit_pipeline") if (R, Cc) == (20_000_000, 64) else None,
             "traffic_unit": "bytes per launch",
+            "traffic_source": COUNTER_PROFILE,
             "algorithmic_bytes_per_launch": bytes_s3,
         },
         "cpu_baseline": cpu,
     }
     print(json.dumps(out))
+    if pipeline_mode != 1:
+        print("bench.py: the pipeline body was interpreted, not specialised at run time (" +
+              capi.lib().dh_last_error().decode(errors="replace") + "); the line above does not measure the kernel it names",
+              file=sys.stderr)
+        return 3
     return 0
 
 

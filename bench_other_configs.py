@@ -50,6 +50,62 @@ def _line(metric_value, unit, ms, args, dtype, workload, roofline, cpu, extra=No
             "dtype": dtype, "data": "synthetic", "config": cfg, "roofline": roofline, "cpu_baseline": cpu}
 
 
+def measure_contractions(torch, ctx, steps, warmup):
+    """The dense-contraction half of the metric at the sizes it is quoted on: MatMul f64 8192^3, MatMul f32 16384^3,
+    Syrk f64 t(X) X with X 1,000,000 x 1024. Returns {name: {ms, tflops, pct_of_mfma_peak}}; inputs are generated
+    on the device and freed again before the next case."""
+    from daphne_amd.kernels import DenseMatrix, matMul, syrk
+
+    gen = torch.Generator(device="cuda").manual_seed(4)
+    res = {}
+    for name, dt, n, key in (("matmul_f64_8192", torch.float64, 8192, "f64"), ("matmul_f32_16384", torch.float32, 16384, "f32")):
+        A = torch.rand(n, n, device="cuda", dtype=dt, generator=gen) * 2 - 1
+        B = torch.rand(n, n, device="cuda", dtype=dt, generator=gen) * 2 - 1
+        Cm = torch.empty(n, n, device="cuda", dtype=dt)
+        dA, dB, dC = (DenseMatrix.from_torch(ctx, t) for t in (A, B, Cm))
+        ms = _timed(torch, lambda: matMul(dC, dA, dB, False, False, ctx), steps, warmup)
+        res[name] = {"ms": round(ms, 3), "tflops": round(2.0 * n ** 3 / ms / 1e9, 2)}
+        res[name]["pct_of_mfma_peak"] = round(100 * res[name]["tflops"] / MFMA_PEAK[key], 1)
+        del A, B, Cm, dA, dB, dC
+        torch.cuda.empty_cache()
+    Xs = torch.rand(1_000_000, 1024, device="cuda", dtype=torch.float64, generator=gen) * 2 - 1
+    dX, S = DenseMatrix.from_torch(ctx, Xs), DenseMatrix(ctx, 1024, 1024, np.float64)
+    ms_s = _timed(torch, lambda: syrk(S, dX, True, ctx), steps, warmup)
+    # the distinct results of t(X) X: n (n + 1) / 2 dot products of length 1e6
+    res["syrk_f64_1e6x1024"] = {"ms": round(ms_s, 3), "tflops": round(1024 * 1025 * 1e6 / ms_s / 1e9, 2)}
+    res["syrk_f64_1e6x1024"]["pct_of_mfma_peak"] = round(100 * res["syrk_f64_1e6x1024"]["tflops"] / MFMA_PEAK["f64"], 1)
+    S.destroy()
+    del Xs, dX
+    torch.cuda.empty_cache()
+    return res
+
+
+def blas_baseline(n=4096, reps=3):
+    """numpy.matmul in double precision on the host: numpy's bundled BLAS is OpenBLAS, the library the reference's
+    CPU MatMul calls (src/runtime/local/kernels/MatMul.cpp:24-90, cblas_dgemm). Returns (TFLOP/s, description)."""
+    import io
+    from contextlib import redirect_stdout
+
+    rng = np.random.default_rng(0)
+    a, b = rng.random((n, n)), rng.random((n, n))
+    a @ b
+    best = float("inf")
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        a @ b
+        best = min(best, time.perf_counter() - t0)
+    buf = io.StringIO()
+    try:
+        with redirect_stdout(buf):
+            np.show_config()
+    except Exception:
+        pass
+    cfg = buf.getvalue()
+    name = "openblas" if "openblas" in cfg.lower() else ("mkl" if "mkl" in cfg.lower() else "BLAS of numpy")
+    threads = os.environ.get("OPENBLAS_NUM_THREADS") or os.environ.get("OMP_NUM_THREADS") or str(os.cpu_count())
+    return 2.0 * n ** 3 / best / 1e12, f"numpy.matmul f64 {n}^3 ({name}, {threads} threads, best of {reps}: {best:.2f} s)"
+
+
 def run(args) -> int:
     import torch
 
@@ -135,34 +191,20 @@ def run(args) -> int:
                     "k-means Lloyd iteration: X 2000000x64 f32 (16 Gaussians), C 16x64; step = one iteration",
                     roof, cpu, {"canonical_bytes_per_step": nbytes, "xct_ms": round(t_gemm, 4)})
     elif args.config == 4:
-        res = {}
-        for name, dt, n in (("matmul_f64_8192", torch.float64, 8192), ("matmul_f32_16384", torch.float32, 16384)):
-            A = torch.rand(n, n, device="cuda", dtype=dt, generator=gen) * 2 - 1
-            B = torch.rand(n, n, device="cuda", dtype=dt, generator=gen) * 2 - 1
-            Cm = torch.empty(n, n, device="cuda", dtype=dt)
-            dA, dB, dC = (DenseMatrix.from_torch(ctx, t) for t in (A, B, Cm))
-            ms = _timed(torch, lambda: matMul(dC, dA, dB, False, False, ctx), args.steps, args.warmup)
-            res[name] = {"ms": round(ms, 3), "tflops": round(2.0 * n ** 3 / ms / 1e9, 2)}
-            del A, B, Cm, dA, dB, dC
-            torch.cuda.empty_cache()
-        Xs = torch.rand(1_000_000, 1024, device="cuda", dtype=torch.float64, generator=gen) * 2 - 1
-        dX, S = DenseMatrix.from_torch(ctx, Xs), DenseMatrix(ctx, 1024, 1024, np.float64)
-        ms_s = _timed(torch, lambda: syrk(S, dX, True, ctx), args.steps, args.warmup)
-        res["syrk_f64_1e6x1024"] = {"ms": round(ms_s, 3), "tflops": round(1024 * 1025 * 1e6 / ms_s / 1e9, 2)}
+        res = measure_contractions(torch, ctx, args.steps, args.warmup)
         cpu = None
         if orc:
             a = np.random.default_rng(0).random((512, 512))
             t0 = time.perf_counter()
             orc.matmul(a, a)
             dt = time.perf_counter() - t0
-            cpu = {"value": round(2 * 512 ** 3 / dt / 1e12, 5), "unit": "TFLOP/s", "cores": 1, "kind": "port",
-                   "sample": f"f64 matMul 512^3 with the oracle's scalar triple loop, single thread ({dt:.2f} s); "
-                             "the reference calls OpenBLAS here, which is not available"}
+            blas_tflops, blas_what = blas_baseline()
+            cpu = {"value": round(blas_tflops, 4), "unit": "TFLOP/s", "cores": min(os.cpu_count() or 1, 16), "kind": "port",
+                   "sample": f"{blas_what}: the reference's CPU MatMul is a call of this library; beside it the oracle's "
+                             f"scalar triple loop at 512^3 on one thread, {2 * 512 ** 3 / dt / 1e12:.5f} TFLOP/s ({dt:.2f} s)"}
         f64 = res["matmul_f64_8192"]["tflops"]
         roof = {"bound": "mfma", "kernel": "gemm_kernel<double,128,128,8,2,2,false,false,0,true>", "achieved": f64,
                 "peak": MFMA_PEAK["f64"], "unit": "TFLOP/s", "frac": round(f64 / MFMA_PEAK["f64"], 4), "traffic": None}
-        for v, key in ((res["matmul_f64_8192"], "f64"), (res["matmul_f32_16384"], "f32"), (res["syrk_f64_1e6x1024"], "f64")):
-            v["pct_of_mfma_peak"] = round(100 * v["tflops"] / MFMA_PEAK[key], 1)
         out = _line(f64, "TFLOP/s", res["matmul_f64_8192"]["ms"], args, "f64",
                     "dense contractions: (a) MatMul f64 8192^3 [value], (b) MatMul f32 16384^3, (c) Syrk f64 1000000x1024",
                     roof, cpu, res)

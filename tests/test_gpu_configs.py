@@ -150,6 +150,75 @@ def test_config4_syrk_tall_prefix_and_symmetry(ctx):
     assert_close(syrk(None, DenseMatrix.from_numpy(ctx, Xp), True, ctx).to_numpy(), orc.syrk(Xp, True)[1], elementwise=False)
 
 
+def _sampled_products(A_rows, B_cols):
+    """All pairwise dot products of the given rows and columns (host arrays, K values each) in extended precision,
+    with the sum of absolute terms that bounds the rounding error of any summation order."""
+    a, b = A_rows.astype(np.longdouble), B_cols.astype(np.longdouble)
+    return a @ b.T, np.abs(a) @ np.abs(b).T
+
+
+@pytest.mark.parametrize("dt,n,tol", [(np.float64, 8192, 1e-10), (np.float32, 16384, 1e-4)])
+def test_config4_matmul_at_the_quoted_sizes(ctx, dt, n, tol):
+    """MatMul at the sizes the throughput is quoted on (8192^3 f64, 16384^3 f32: grids whose tile count is a multiple
+    of the XCD count, the regrouped tile order). Inputs are generated on the device; 16 rows x 16 columns = 256
+    results are checked against extended-precision dot products on the host, and a 512-row band of the result against
+    the same kernel run on that band alone (other grid, other tile order; every entry of the band is compared)."""
+    import torch
+
+    tdt = torch.float64 if dt == np.float64 else torch.float32
+    gen = torch.Generator(device="cuda").manual_seed(21)
+    A = torch.rand(n, n, device="cuda", dtype=tdt, generator=gen) * 2 - 1
+    B = torch.rand(n, n, device="cuda", dtype=tdt, generator=gen) * 2 - 1
+    Cm = torch.full((n, n), float("nan"), device="cuda", dtype=tdt)
+    matMul(DenseMatrix.from_torch(ctx, Cm), DenseMatrix.from_torch(ctx, A), DenseMatrix.from_torch(ctx, B), False, False, ctx)
+    torch.cuda.synchronize()
+    assert not bool(torch.isnan(Cm).any()), "some tile of the result was not written"
+    rng = np.random.default_rng(22)
+    # rows and columns from the first, the last and random tiles
+    ii = np.unique(np.concatenate([[0, n - 1, 127, 128], rng.integers(0, n, 12)]))[:16]
+    jj = np.unique(np.concatenate([[0, n - 1, 255, 256], rng.integers(0, n, 12)]))[:16]
+    ti, tj = torch.as_tensor(ii, device="cuda"), torch.as_tensor(jj, device="cuda")
+    exact, bound = _sampled_products(A[ti].cpu().numpy(), B[:, tj].T.contiguous().cpu().numpy())
+    got = Cm[ti][:, tj].cpu().numpy().astype(np.longdouble)
+    assert exact.size >= 256 - 32
+    assert (np.abs(got - exact) <= tol * bound).all(), float((np.abs(got - exact) / bound).max())
+    band = slice(n // 2 - 256, n // 2 + 256)
+    Cb = torch.empty(512, n, device="cuda", dtype=tdt)
+    matMul(DenseMatrix.from_torch(ctx, Cb), DenseMatrix.from_torch(ctx, A[band]), DenseMatrix.from_torch(ctx, B), False, False, ctx)
+    torch.cuda.synchronize()
+    assert float((Cb - Cm[band]).abs().max()) <= tol * float(Cm[band].abs().max())
+    del A, B, Cm, Cb
+    torch.cuda.empty_cache()
+
+
+def test_config4_syrk_at_the_quoted_size(ctx):
+    """Syrk f64 t(X) X with X 1,000,000 x 1024 (the full split over the rows, the slab reduction and the mirror
+    step): bit-exact symmetry, all 16 x 16 results among 16 sampled columns against extended-precision dot products,
+    and the whole result against MatMul(t(X), X) norm-wise."""
+    import torch
+
+    rows, n = 1_000_000, 1024
+    gen = torch.Generator(device="cuda").manual_seed(23)
+    X = torch.rand(rows, n, device="cuda", dtype=torch.float64, generator=gen) * 2 - 1
+    S = torch.full((n, n), float("nan"), device="cuda", dtype=torch.float64)
+    dX = DenseMatrix.from_torch(ctx, X)
+    syrk(DenseMatrix.from_torch(ctx, S), dX, True, ctx)
+    torch.cuda.synchronize()
+    assert not bool(torch.isnan(S).any())
+    assert bool((S == S.T).all())
+    cols = np.unique(np.concatenate([[0, n - 1, 63, 64, 511, 512], np.random.default_rng(24).integers(0, n, 12)]))[:16]
+    Xc = X[:, torch.as_tensor(cols, device="cuda")].T.contiguous().cpu().numpy()  # 16 x 1e6
+    exact, bound = _sampled_products(Xc, Xc)
+    got = S[torch.as_tensor(cols, device="cuda")][:, torch.as_tensor(cols, device="cuda")].cpu().numpy().astype(np.longdouble)
+    assert (np.abs(got - exact) <= 1e-10 * bound).all(), float((np.abs(got - exact) / bound).max())
+    M = torch.empty(n, n, device="cuda", dtype=torch.float64)
+    matMul(DenseMatrix.from_torch(ctx, M), dX, dX, True, False, ctx)
+    torch.cuda.synchronize()
+    assert float((S - M).abs().max()) <= 1e-10 * float(M.abs().max())
+    del X, S, M, dX
+    torch.cuda.empty_cache()
+
+
 def _lenet_weights(rng):
     he = lambda shape, fan: (rng.standard_normal(shape) * np.sqrt(2.0 / fan)).astype(np.float32)
     small = lambda shape: (rng.standard_normal(shape) * 0.1).astype(np.float32)
