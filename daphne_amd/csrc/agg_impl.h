@@ -672,6 +672,18 @@ template <typename T> dh_status agg_row(dh_ctx *ctx, int op, T *res, size_t ld_r
         if (op == DH_AGG_MEAN || op == DH_AGG_VAR || op == DH_AGG_STDDEV)
             return dh_fail(DH_ERR_RUNTIME, "%s: MEAN, VAR and STDDEV of integer value types are not supported on the device", __func__);
     }
+    // A few very wide rows (a 1 x N vector is the common case) would occupy one wavefront each in the row kernel:
+    // every such row goes through the whole-matrix reduction instead, which spreads it over the device. SUM, PROD and
+    // the moments only: they do not depend on the order of NaNs, MIN / MAX follow AggRow's own NaN rule.
+    if (rows <= 16 && cols >= (size_t(1) << 16) &&
+        (op == DH_AGG_SUM || op == DH_AGG_PROD || op == DH_AGG_MEAN || op == DH_AGG_VAR || op == DH_AGG_STDDEV)) {
+        for (size_t r = 0; r < rows; r++) {
+            const dh_status st = agg_all_dev<T>(ctx, op, arg + r * ld, 1, cols, ld, res + r * ld_res);
+            if (st != DH_OK)
+                return st;
+        }
+        return DH_OK;
+    }
     switch (op) {
     case DH_AGG_SUM:
         row_launch<T, RSum<T>, 0, false>(ctx, res, ld_res, arg, rows, cols, ld);

@@ -121,6 +121,16 @@ class HipBackend:
         self.k, self.capi, self.ctx = kernels, capi, ctx
 
     def _d(self, a):
+        if isinstance(a, np.ndarray) and a.ndim == 2 and a.size and not a.flags.c_contiguous and a.base is not None:
+            # a view with a row stride: upload the array it looks into and pass the same view of the device copy
+            root = a
+            while root.base is not None:
+                root = root.base
+            if isinstance(root, np.ndarray) and root.ndim == 2 and root.flags.c_contiguous and a.strides[1] == a.itemsize \
+                    and a.strides[0] == root.strides[0]:
+                off = (a.ctypes.data - root.ctypes.data) // a.itemsize
+                r0, c0 = divmod(off, root.shape[1])
+                return self.k.DenseMatrix.from_numpy(self.ctx, root).slice(r0, r0 + a.shape[0], c0, c0 + a.shape[1])
         return self.k.DenseMatrix.from_numpy(self.ctx, a)
 
     def _call(self, fn, *a):

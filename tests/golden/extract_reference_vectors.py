@@ -49,6 +49,8 @@ def parse_value(tok: str):
         return float("nan")
     if "infinity" in low or low == "inf":
         return sign * float("inf")
+    if "denorm_min" in low:
+        return "denorm_min" if sign > 0 else None  # the value type's smallest subnormal, resolved at replay
     if NUM.match(t):
         return sign * float(t.rstrip("fFlL"))
     return None
@@ -99,6 +101,10 @@ def extract(path: Path) -> dict:
             # a name may be defined several times (per SECTION, or per value-type branch): keep all,
             # with their position, so that a check can take the definition that precedes it
             case["matrices"].setdefault(var, []).append({"pos": m.start(), "rows": rows, "values": parsed})
+        # views made with the slicing kernels: `sliceRow(res, arg, lower, upper, ctx)` / `sliceCol(...)`
+        for m in re.finditer(r"\bslice(Row|Col)\(\s*(\w+)\s*,\s*(\w+)\s*,\s*(\d+)\s*,\s*(\d+)\s*,", body):
+            case.setdefault("slices", {})[m.group(2)] = {"of": m.group(3), "axis": m.group(1).lower(), "lo": int(m.group(4)),
+                                                         "hi": int(m.group(5)), "pos": m.start()}
         for m in re.finditer(r"\b(check\w+)\s*(?:<[^>(]*>)?\(([^;]*?)\);", body):
             case["checks"].append({"fn": m.group(1), "args": split_top(m.group(2)), "pos": m.start()})
         for m in re.finditer(r"(CHECK_THROWS|REQUIRE_THROWS_AS|CHECK_THROWS_AS|REQUIRE_THROWS)\((.*?)\);", body):

@@ -46,6 +46,11 @@ def _num(v):
 
 
 def matrix(spec, dt):
+    if "denorm_min" in spec["values"]:
+        if np.dtype(dt).kind != "f":
+            raise Skip("floating-point literal")
+        tiny = float(np.finfo(dt).smallest_subnormal)
+        spec = {**spec, "values": [tiny if v == "denorm_min" else v for v in spec["values"]]}
     vals = np.array([_num(v) for v in spec["values"]], dtype=np.float64)
     rows = spec["rows"]
     if rows == 0 or vals.size % rows:
@@ -125,8 +130,15 @@ def run(backend, f, c, k, dt):
         if not (ew or (other and np.dtype(dt) == np.int64)):
             raise Skip("kernel has no instantiation for this integer type on the device")
 
+    slices = c.get("slices", {})
+
     def M(name):
         name = name.strip()
+        if name in slices and name not in mats:
+            # a view made by sliceRow / sliceCol: stays a view (of the literal's array) down to the kernel
+            s = slices[name]
+            base = M(s["of"])
+            return base[s["lo"]:s["hi"], :] if s["axis"] == "row" else base[:, s["lo"]:s["hi"]]
         if name not in mats:
             if name in ("inputs",) and "genInput" in mats:
                 return matrix(mats["genInput"], dt)

@@ -194,6 +194,22 @@ def test_agg_row_col_all(ctx, dt, op, shape):
 
 
 @pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("op", [o for o in AGG_VALUE_OPS if o != AggOpCode.PROD])  # 300000 float factors: rounding alone exceeds 1e-4
+@pytest.mark.parametrize("shape,ld", [((1, 300_000), 300_000), ((3, 70_001), 70_016), ((16, 65_536), 65_536)])
+def test_agg_row_of_a_few_very_wide_rows(ctx, dt, op, shape, ld):
+    """A 1 x N vector and other few-row, very wide matrices: every row is spread over the device (for SUM, PROD and
+    the moments), also through a view with a row stride; the result must be the row aggregate all the same."""
+    rng = np.random.default_rng(shape[1])
+    base = np.zeros((shape[0], ld), dt)
+    base[:, :shape[1]] = _agg_input(rng, shape, dt, op)
+    a = base[:, :shape[1]]
+    A = DenseMatrix.from_numpy(ctx, base).slice(0, shape[0], 0, shape[1])
+    kw = {"atol": variance_floor(a, op == AggOpCode.STDDEV)} if op in (AggOpCode.VAR, AggOpCode.STDDEV) else {}
+    st, exp = orc.agg_row(op, np.ascontiguousarray(a))
+    (assert_exact if op in (AggOpCode.MIN, AggOpCode.MAX) else assert_close)(aggRow(op, None, A, ctx).to_numpy(), exp, **kw)
+
+
+@pytest.mark.parametrize("dt", DTYPES)
 @pytest.mark.parametrize("op", [AggOpCode.IDXMIN, AggOpCode.IDXMAX])
 @pytest.mark.parametrize("shape", [(2000, 16), (7, 5), (1, 300), (300, 1), (513, 64), (3, 1030), (9, 130), (33, 6), (100, 12),
                                    (64, 22), (257, 66)])
