@@ -130,7 +130,7 @@ def run(args) -> int:
         yt = Xt @ w + 0.1 * torch.randn(n, 1, device="cuda", dtype=torch.float64, generator=gen)
         X, y = DenseMatrix.from_torch(ctx, Xt), DenseMatrix.from_torch(ctx, yt)
         eye = DenseMatrix.from_numpy(ctx, np.eye(m))
-        ms = _timed(torch, lambda: lmds(ctx, X, y, 1e-3, eye), args.steps, args.warmup)
+        ms = _timed(torch, lambda: lmds(ctx, X, y, 1e-3), args.steps, args.warmup)
         t_syrk = _events(torch, lambda: syrk(None, X, True, ctx))
         nbytes = (n * m * 8 + m * m * 8) + (n * m * 8 + n * 8 + m * 8) + 3 * m * m * 8
         cpu = None

@@ -111,6 +111,7 @@ _LATE_SIGNATURES: dict[str, list] = {
     "dh_matmul": [vp, vp, sz, vp, sz, sz, sz, vp, sz, sz, sz, i32, i32],
     "dh_syrk": [vp, vp, sz, vp, sz, sz, sz, i32],
     "dh_solve": [vp, vp, vp, sz, sz, vp],
+    "dh_normal_equations": [vp, vp, sz, vp, sz, vp, sz, sz, sz, vp, sz, "T"],
     "dh_conv2d_forward": [vp, vp, C.POINTER(sz), C.POINTER(sz), vp, vp, sz, sz, vp, sz, sz, sz, sz, sz, sz, sz, sz, sz, sz],
     "dh_maxpool_forward": [vp, vp, C.POINTER(sz), C.POINTER(sz), vp, sz, sz, sz, sz, sz, sz, sz, sz, sz, sz],
     "dh_affine_forward": [vp, vp, vp, sz, sz, vp, sz, sz, vp, sz, sz],

@@ -757,6 +757,11 @@ dh_status matmul(dh_ctx *ctx, T *res, size_t ld_res, const T *lhs, size_t lr, si
     return gemm<T>(ctx, transa != 0, transb != 0, nr1, nc2, nc1, lhs, ld_lhs, rhs, ld_rhs, res, ld_res, nullptr, false);
 }
 
+// ts_sym_impl.h, instantiated in ts_sym_f32.hip / ts_sym_f64.hip
+template <typename T>
+bool ts_sym(dh_ctx *ctx, size_t m, size_t K, const T *X, size_t ldx, const T *y, size_t ldy, T *C, size_t ldc, T *b, size_t ldb,
+            T lambda, dh_status *status);
+
 // Syrk<DenseMatrix<T>,DenseMatrix<T>>::apply of kernels/Syrk.h:51-93.
 template <typename T>
 dh_status syrk(dh_ctx *ctx, T *res, size_t ld_res, const T *arg, size_t rows, size_t cols, size_t ld, int trans_left) {
@@ -765,6 +770,15 @@ dh_status syrk(dh_ctx *ctx, T *res, size_t ld_res, const T *arg, size_t rows, si
     const size_t k = trans_left ? rows : cols;
     if (ld < cols || ld_res < n)
         return dh_fail(DH_ERR_RUNTIME, "Syrk - a leading dimension is smaller than its column count");
+    // t(X) X of a tall matrix with 65..128 columns: the triangle only, all four waves of a workgroup splitting the rows
+    if (trans_left) {
+        dh_status st = DH_OK;
+        if (ts_sym<T>(ctx, n, k, arg, ld, nullptr, 0, res, ld_res, nullptr, 0, T(0), &st)) {
+            if (st == DH_OK)
+                DH_CHECK_LAUNCH();
+            return st;
+        }
+    }
     // transLeft: C = X^T X -> A = X transposed, B = X; else C = X X^T -> A = X, B = X transposed
     return gemm<T>(ctx, trans_left != 0, trans_left == 0, n, n, k, arg, ld, arg, ld, res, ld_res, nullptr, true);
 }

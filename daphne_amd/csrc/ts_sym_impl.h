@@ -4,28 +4,45 @@
 // The work is bound by the matrix cores, not by memory (f64: 2 m^2 flop per row of X against 8 m bytes), so the
 // point is to issue as few matrix instructions as possible: the columns are cut into NT tiles of 16 and only the
 // NT (NT + 1) / 2 tile pairs on or above the diagonal are computed (100 columns: 28 instead of the 64 of a padded
-// full product). All four waves of a workgroup hold the whole triangle in registers and split the rows of X between
-// them, as the workgroups do; a workgroup adds its four triangles through LDS and writes one partial ("slab"), and
-// a second kernel adds the slabs in a fixed order, mirrors the triangle, and adds lambda on the diagonal.
+// full product). The rows of X are cut over the workgroups; the four waves of a workgroup take a quarter of the
+// tile pairs each, over all rows of the workgroup. A workgroup writes one partial ("slab"), and a second kernel adds
+// the slabs in a fixed order, mirrors the triangle, and adds lambda on the diagonal.
 //
 // Fragments, as in ts_impl.h: the matrix instruction 16x16x4 takes A[i = lane % 16][k = lane / 16] and
 // B[k][j = lane % 16]; here both are the same row k of X, so one set of loads feeds both sides. Lane group
 // h = lane / 16 takes row k0 + h of a quad of rows. The first NV * V tiles come from NV vector loads of V values
 // (value e of vector a belongs to tile a * V + e, which therefore stands for the columns 16 V a + V i + e), the
 // last NS tiles from scalar loads of 16 consecutive columns each. That way 100 doubles are 3 vectors + 1 scalar =
-// 7 tiles, not 8. t(X) y costs no matrix instruction: every lane multiplies the values it has loaded by y[k] on
-// the ordinary ALUs, which are idle otherwise.
+// 7 tiles, not 8. t(X) y costs no matrix instruction: the wave that owns the diagonal pair of a tile multiplies the
+// values it has loaded by y[k] on the ordinary ALUs, which are idle otherwise.
 #pragma once
 
 #include "ts_impl.h"
 
 namespace dh_gemm {
+#ifndef TS_SYM_BLOCKS_PER_CU
+#define TS_SYM_BLOCKS_PER_CU 1
+#endif
+#ifndef TS_SYM_DEPTH
+#define TS_SYM_DEPTH 4
+#endif
+
+#ifdef DH_TS_SYM_PROFILE
+__device__ long long g_ts_sym_prof[2][8][4];
+#define TS_PROF(slot)                                                                                                     \
+    do {                                                                                                                   \
+        if (threadIdx.x % 64 == 0 && (blockIdx.x == 0 || blockIdx.x + 1 == gridDim.x))                                     \
+            g_ts_sym_prof[blockIdx.x == 0 ? 0 : 1][threadIdx.x / 64][slot] = __builtin_amdgcn_s_memtime();                 \
+    } while (0)
+#else
+#define TS_PROF(slot)
+#endif
 
 struct TsSymArgs {
     const void *X, *y;
     void *slabs;     // [gridDim.x][m * m + m]: the triangle in matrix layout (row <= col), then the m values of t(X) y
     size_t ldx, ldy, K;
-    size_t k_chunk;  // rows per workgroup, a multiple of 16 * U
+    size_t k_chunk;  // rows per workgroup, a multiple of 16
     unsigned m;
 };
 
@@ -33,212 +50,261 @@ template <typename T, int NV, int NS> struct TsSymShape {
     static constexpr int V = 16 / sizeof(T);
     static constexpr int NT = NV * V + NS;                  // tiles of 16 columns
     static constexpr int NP = NT * (NT + 1) / 2;            // tile pairs on or above the diagonal
-    static constexpr int U = 2;                             // quads per register set
+    static constexpr int PPW = (NP + 3) / 4;                // pairs per wave, dealt in row-major order
     // first column of tile t for lane column i
     static __device__ __forceinline__ unsigned col(int t, int i) {
         return t < NV * V ? static_cast<unsigned>(16 * V * (t / V) + V * i + (t % V))
                           : static_cast<unsigned>(NV * 16 * V + (t - NV * V) * 16 + i);
     }
-    static constexpr size_t lds_bytes() { return static_cast<size_t>(NP) * 4 * 64 * sizeof(T) + (WITH_Y_SLOTS) * sizeof(T); }
-    static constexpr int WITH_Y_SLOTS = NT * 16;
+    // pair p (row-major over ta <= tb) -> ta, tb
+    struct Pairs {
+        int a[NP], b[NP];
+    };
+    static constexpr Pairs pairs() {
+        Pairs r{};
+        int p = 0;
+        for (int ta = 0; ta < NT; ta++)
+            for (int tb = ta; tb < NT; tb++) {
+                r.a[p] = ta;
+                r.b[p] = tb;
+                p++;
+            }
+        return r;
+    }
+    // bit t: wave w needs tile t (as either side of one of its pairs) / owns the diagonal pair (t, t)
+    static constexpr unsigned need_mask(int w) {
+        const Pairs pr = pairs();
+        unsigned m = 0;
+        for (int p = w * PPW; p < (w + 1) * PPW && p < NP; p++)
+            m |= (1u << pr.a[p]) | (1u << pr.b[p]);
+        return m;
+    }
+    static constexpr unsigned diag_mask(int w) {
+        const Pairs pr = pairs();
+        unsigned m = 0;
+        for (int p = w * PPW; p < (w + 1) * PPW && p < NP; p++)
+            if (pr.a[p] == pr.b[p])
+                m |= 1u << pr.a[p];
+        return m;
+    }
 };
 
-template <typename T, int NV, int NS, bool WITH_Y>
-__global__ __launch_bounds__(256) void ts_sym_kernel(TsSymArgs g) {
+// The work of wave W: its quarter of the tile pairs over all rows of the workgroup's chunk.
+//
+// A wave issues its instructions in order, and the waves of a SIMD are served oldest first (measured: a second wave on
+// a SIMD gets the matrix core only when the first has nothing for it), so what counts is how few instructions stand
+// between one group of matrix instructions and the next: one wave per SIMD, the row address in scalar registers
+// (advanced by scalar adds), every load addressed as that scalar base plus a lane offset that never changes, and no
+// work at all on the loaded values. Then 7 matrix instructions of 64 cycles each are followed by some 40 cycles of
+// other work, not 250.
+template <typename T, int NV, int NS, bool WITH_Y, int W> __device__ __forceinline__ void ts_sym_wave(const TsSymArgs g) {
     using M = Mfma16<T>;
     using S = TsSymShape<T, NV, NS>;
-    constexpr int V = S::V, NT = S::NT, U = S::U;
-    extern __shared__ __attribute__((aligned(16))) unsigned char ts_sym_lds[];
-    const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
-    const int i = lane % 16, h = lane / 16;
-    const T *X = static_cast<const T *>(g.X);
-    const T *Y = static_cast<const T *>(g.y);
+    constexpr int V = S::V, NT = S::NT;
+    constexpr int P0 = W * S::PPW, P1 = (W + 1) * S::PPW < S::NP ? (W + 1) * S::PPW : S::NP;
+    constexpr int NPW = P1 > P0 ? P1 - P0 : 0;
+    constexpr unsigned NEED = S::need_mask(W), DIAG = S::diag_mask(W);
+    constexpr typename S::Pairs PR = S::pairs();
+    if constexpr (NPW == 0) {
+        return;
+    } else {
+        const int lane = threadIdx.x % 64;
+        const int i = lane % 16, h = lane / 16;
+        const char *X = static_cast<const char *>(g.X);
+        const char *Y = static_cast<const char *>(g.y);
+        TS_PROF(0);
 
-    // columns this lane loads; a vector or scalar that starts beyond the matrix reads column 0 instead (it only
-    // feeds rows / columns of the result beyond m, which are never stored)
-    unsigned cv[NV > 0 ? NV : 1], cs[NS > 0 ? NS : 1];
-#pragma unroll
-    for (int a = 0; a < NV; a++) {
-        const unsigned c = 16 * V * a + V * i;
-        cv[a] = c < g.m ? c : 0;
-    }
-#pragma unroll
-    for (int s = 0; s < NS; s++) {
-        const unsigned c = NV * 16 * V + s * 16 + i;
-        cs[s] = c < g.m ? c : 0;
-    }
-
-    typename M::acc_t acc[S::NP];
-#pragma unroll
-    for (int p = 0; p < S::NP; p++)
-        acc[p] = typename M::acc_t{0, 0, 0, 0};
-    T bacc[NT];
-#pragma unroll
-    for (int t = 0; t < NT; t++)
-        bacc[t] = T(0);
-
-    const size_t kb = static_cast<size_t>(blockIdx.x) * g.k_chunk;
-    const size_t ke = kb + g.k_chunk < g.K ? kb + g.k_chunk : g.K;
-
-    struct Frag {
-        T f[U][NT];
-        T y[U];
-    };
-    // Unconditional loads (a branch around a load makes the compiler wait for all outstanding loads there). Rows
-    // beyond the chunk, possible in the tail loop only, read its last row and are zeroed.
-    auto load_quad = [&](Frag &fr, int u, size_t k, bool guard) {
-        const bool row_ok = !guard || k < ke;
-        const size_t kl = row_ok ? k : ke - 1;
-        const T *row = X + kl * g.ldx;
+        // byte offsets of this lane's loads from the first row of a quad: lane group h reads row + h; a vector or
+        // scalar that starts beyond the matrix reads column 0 instead (it only feeds rows / columns of the result
+        // beyond m, which are never stored)
+        unsigned ov[NV > 0 ? NV : 1], os[NS > 0 ? NS : 1];
+        const unsigned rowoff = static_cast<unsigned>(h) * static_cast<unsigned>(g.ldx);
 #pragma unroll
         for (int a = 0; a < NV; a++) {
-            T v[V];
-            ts_load<T, V>(row + cv[a], v, true);
-#pragma unroll
-            for (int e = 0; e < V; e++)
-                fr.f[u][a * V + e] = v[e];
+            const unsigned c = 16 * V * a + V * i;
+            ov[a] = (rowoff + (c < g.m ? c : 0)) * static_cast<unsigned>(sizeof(T));
         }
 #pragma unroll
-        for (int s = 0; s < NS; s++)
-            fr.f[u][NV * V + s] = __builtin_nontemporal_load(row + cs[s]);
-        if constexpr (WITH_Y)
-            fr.y[u] = Y[kl * g.ldy];
-        if (guard) {
-#pragma unroll
-            for (int t = 0; t < NT; t++)
-                fr.f[u][t] = row_ok ? fr.f[u][t] : T(0);
+        for (int s = 0; s < NS; s++) {
+            const unsigned c = NV * 16 * V + s * 16 + i;
+            os[s] = (rowoff + (c < g.m ? c : 0)) * static_cast<unsigned>(sizeof(T));
         }
-    };
-    auto mma_quad = [&](const Frag &fr, int u) {
-        int p = 0;
-#pragma unroll
-        for (int ta = 0; ta < NT; ta++)
-#pragma unroll
-            for (int tb = ta; tb < NT; tb++)
-                acc[p] = M::mma(fr.f[u][ta], fr.f[u][tb], acc[p]), p++;
-        if constexpr (WITH_Y) {
-#pragma unroll
-            for (int t = 0; t < NT; t++)
-                bacc[t] = __builtin_fma(fr.f[u][t], fr.y[u], bacc[t]);
-        }
-    };
+        const unsigned oy = static_cast<unsigned>(h) * static_cast<unsigned>(g.ldy) * static_cast<unsigned>(sizeof(T));
 
-    // quad q of this wave covers rows kb + (4 q + wave) * 4 .. + 3; lane group h takes row + h
-    size_t k = kb + static_cast<size_t>(wave) * 4 + h;
-    constexpr size_t STEP = 16;
-    auto load_group = [&](Frag &fr) {
+        typename M::acc_t acc[NPW];
 #pragma unroll
-        for (int u = 0; u < U; u++)
-            load_quad(fr, u, k + u * STEP, false);
-        k += U * STEP;
-    };
-    auto mma_group = [&](const Frag &fr) {
+        for (int p = 0; p < NPW; p++)
+            acc[p] = typename M::acc_t{0, 0, 0, 0};
+        T bacc[NT];
 #pragma unroll
-        for (int u = 0; u < U; u++)
-            mma_quad(fr, u);
-    };
-    Frag f0, f1;
-    const size_t k0 = kb + static_cast<size_t>(wave) * 4;
-    const size_t need = (U - 1) * STEP + 4;
-    const unsigned n_full = ke >= k0 + need ? static_cast<unsigned>((ke - k0 - need) / (U * STEP)) + 1 : 0;
-    if (n_full > 0) {
-        load_group(f0);
-        const unsigned pairs = (n_full - 1) / 2;
-        for (unsigned q = 0; q < pairs; q++) {
-            load_group(f1);
-            __builtin_amdgcn_sched_barrier(0);
-            mma_group(f0);
-            __builtin_amdgcn_sched_barrier(0);
-            load_group(f0);
-            __builtin_amdgcn_sched_barrier(0);
-            mma_group(f1);
-            __builtin_amdgcn_sched_barrier(0);
-        }
-        if ((n_full - 1) % 2) {
-            load_group(f1);
-            __builtin_amdgcn_sched_barrier(0);
-            mma_group(f0);
-            mma_group(f1);
-        } else {
-            mma_group(f0);
-        }
-    }
-    while (k - h < ke) {
-        load_quad(f0, 0, k, true);
-        mma_quad(f0, 0);
-        k += STEP;
-    }
+        for (int t = 0; t < NT; t++)
+            bacc[t] = T(0);
 
-    // t(X) y: add the four rows of a quad (lane groups), leaving the sum for column col(t, i) in every lane group
-    if constexpr (WITH_Y) {
-#pragma unroll
-        for (int t = 0; t < NT; t++) {
-            bacc[t] += __shfl_xor(bacc[t], 16, 64);
-            bacc[t] += __shfl_xor(bacc[t], 32, 64);
-        }
-    }
+        const size_t kb = static_cast<size_t>(blockIdx.x) * g.k_chunk;
+        const size_t ke = kb + g.k_chunk < g.K ? kb + g.k_chunk : g.K;
 
-    // add up the four waves, one at a time into wave 0 (fixed order)
-    T *red = reinterpret_cast<T *>(ts_sym_lds);            // [NP * 4][64]
-    T *redb = red + static_cast<size_t>(S::NP) * 4 * 64;   // [NT][16]
-    for (int w = 1; w < 4; w++) {
-        if (wave == w) {
+        struct Frag {
+            T f[NT];
+            T y;
+        };
+        // the quad whose first row `row` points at into a register set, only the tiles this wave multiplies; `row`
+        // is the same in all lanes and lives in scalar registers
+        auto load_quad = [&](Frag &fr, const char *row, const char *yrow) {
+            if constexpr (WITH_Y)
+                fr.y = *reinterpret_cast<const T *>(yrow + oy);
 #pragma unroll
-            for (int p = 0; p < S::NP; p++)
+            for (int a = 0; a < NV; a++) {
+                bool all = true;
 #pragma unroll
-                for (int v = 0; v < 4; v++)
-                    red[(p * 4 + v) * 64 + lane] = acc[p][v];
-            if constexpr (WITH_Y) {
-                if (h == 0) {
+                for (int e = 0; e < V; e++)
+                    all = all && ((NEED >> (a * V + e)) & 1u);
+                if (all) {
+                    T v[V];
+                    ts_load<T, V>(reinterpret_cast<const T *>(row + ov[a]), v, false);
 #pragma unroll
-                    for (int t = 0; t < NT; t++)
-                        redb[t * 16 + i] = bacc[t];
+                    for (int e = 0; e < V; e++)
+                        fr.f[a * V + e] = v[e];
+                } else {
+                    // a vector of which this wave uses only some values: those alone (a load whose other half goes
+                    // nowhere gets its registers shared with other loads, and the waits that protects cost more)
+#pragma unroll
+                    for (int e = 0; e < V; e++)
+                        if ((NEED >> (a * V + e)) & 1u)
+                            fr.f[a * V + e] = *reinterpret_cast<const T *>(row + ov[a] + e * sizeof(T));
                 }
             }
-        }
-        __syncthreads();
-        if (wave == 0) {
 #pragma unroll
-            for (int p = 0; p < S::NP; p++)
+            for (int s = 0; s < NS; s++)
+                if ((NEED >> (NV * V + s)) & 1u)
+                    fr.f[NV * V + s] = *reinterpret_cast<const T *>(row + os[s]);
+        };
+        auto mma_quad = [&](const Frag &fr) {
+            const T(&f)[NT] = fr.f;
 #pragma unroll
-                for (int v = 0; v < 4; v++)
-                    acc[p][v] += red[(p * 4 + v) * 64 + lane];
+            for (int p = 0; p < NPW; p++)
+                acc[p] = M::mma(f[PR.a[P0 + p]], f[PR.b[P0 + p]], acc[p]);
             if constexpr (WITH_Y) {
 #pragma unroll
                 for (int t = 0; t < NT; t++)
-                    bacc[t] += redb[t * 16 + i];
+                    if ((DIAG >> t) & 1u)
+                        bacc[t] = __builtin_fma(f[t], fr.y, bacc[t]);
+            }
+        };
+
+        // D register sets: the loads of D - 1 quads are in flight while one is being multiplied. Loads that would
+        // run past the last whole quad of the chunk repeat that quad (their values are not used). The pointer of the
+        // next quad to load advances on the scalar unit.
+        constexpr int D = TS_SYM_DEPTH;
+        const unsigned nq = static_cast<unsigned>((ke - kb) / 4); // whole quads
+        Frag fr[D];
+        if (nq > 0) {
+            const unsigned last = nq - 1;
+            const size_t sx = 4 * g.ldx * sizeof(T), sy = 4 * g.ldy * sizeof(T);
+            const char *px = X + kb * g.ldx * sizeof(T), *py = WITH_Y ? Y + kb * g.ldy * sizeof(T) : nullptr;
+            unsigned nl = 0; // quad that px points at
+            auto advance = [&]() {
+                const bool more = nl < last;
+                px += more ? sx : 0;
+                py += more ? sy : 0;
+                nl += more ? 1 : 0;
+            };
+#pragma unroll
+            for (int d = 0; d < D - 1; d++) {
+                load_quad(fr[d], px, py);
+                advance();
+            }
+            for (unsigned q = 0; q < nq; q += D) {
+#pragma unroll
+                for (int d = 0; d < D; d++) {
+                    load_quad(fr[(d + D - 1) % D], px, py);
+                    advance();
+                    __builtin_amdgcn_sched_barrier(0);
+                    if (q + d < nq)
+                        mma_quad(fr[d]);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
             }
         }
-        __syncthreads();
-    }
-    if (wave != 0)
-        return;
+        // the rows after the last whole quad (fewer than four, at the very end of X): every lane addresses its own
+        // row here; lane groups without a row read the last one and contribute zeros
+        if (kb + 4 * static_cast<size_t>(nq) < ke) {
+            const size_t r = kb + 4 * static_cast<size_t>(nq) + h;
+            const bool ok = r < ke;
+            const size_t rl = ok ? r : ke - 1;
+            const char *row = X + (rl * g.ldx - rowoff) * sizeof(T); // the lane offsets include h * ldx
+            Frag ft;
+#pragma unroll
+            for (int a = 0; a < NV; a++) {
+                T v[V];
+                ts_load<T, V>(reinterpret_cast<const T *>(row + ov[a]), v, false);
+#pragma unroll
+                for (int e = 0; e < V; e++)
+                    ft.f[a * V + e] = ok ? v[e] : T(0);
+            }
+#pragma unroll
+            for (int s = 0; s < NS; s++) {
+                const T v = *reinterpret_cast<const T *>(row + os[s]);
+                ft.f[NV * V + s] = ok ? v : T(0);
+            }
+            if constexpr (WITH_Y)
+                ft.y = *reinterpret_cast<const T *>(Y + rl * g.ldy * sizeof(T));
+            mma_quad(ft);
+        }
+        TS_PROF(1);
 
-    T *slab = static_cast<T *>(g.slabs) + static_cast<size_t>(blockIdx.x) * (static_cast<size_t>(g.m) * g.m + g.m);
-    int p = 0;
+        T *slab = static_cast<T *>(g.slabs) + static_cast<size_t>(blockIdx.x) * (static_cast<size_t>(g.m) * g.m + g.m);
 #pragma unroll
-    for (int ta = 0; ta < NT; ta++)
-#pragma unroll
-        for (int tb = ta; tb < NT; tb++) {
+        for (int p = 0; p < NPW; p++) {
+            const int ta = PR.a[P0 + p], tb = PR.b[P0 + p];
             const unsigned col = S::col(tb, i);
 #pragma unroll
             for (int v = 0; v < 4; v++) {
                 const unsigned row = S::col(ta, M::row(lane, v));
-                // inside a diagonal tile both halves were computed; the lower one is dropped
-                if (row < g.m && col < g.m && row <= col)
-                    slab[static_cast<size_t>(row) * g.m + col] = acc[p][v];
+                // A tile pair (ta, tb > ta) is the only one that holds the products of its columns, and with
+                // interleaved columns some of them lie below the diagonal of the matrix: those go to their mirror
+                // position. A diagonal pair computed both halves; the lower one is dropped.
+                if (row < g.m && col < g.m && (ta != tb || row <= col)) {
+                    const unsigned lo = row < col ? row : col, hi = row < col ? col : row;
+                    slab[static_cast<size_t>(lo) * g.m + hi] = acc[p][v];
+                }
             }
-            p++;
         }
-    if constexpr (WITH_Y) {
-        if (h == 0) {
+        // t(X) y: add the four rows of a quad (lane groups); lane group 0 stores
+        if constexpr (WITH_Y) {
 #pragma unroll
             for (int t = 0; t < NT; t++) {
-                const unsigned c = S::col(t, i);
-                if (c < g.m)
-                    slab[static_cast<size_t>(g.m) * g.m + c] = bacc[t];
+                if ((DIAG >> t) & 1u) {
+                    T s = bacc[t];
+                    s += __shfl_xor(s, 16, 64);
+                    s += __shfl_xor(s, 32, 64);
+                    const unsigned c = S::col(t, i);
+                    if (h == 0 && c < g.m)
+                        slab[static_cast<size_t>(g.m) * g.m + c] = s;
+                }
             }
         }
+        TS_PROF(3);
+    }
+}
+
+// Four waves per workgroup, one per SIMD, one workgroup per CU. A workgroup takes k_chunk rows of X and each of its
+// waves a quarter of the tile pairs over all of those rows. The waves read the same rows at nearly the same time (all
+// but the first read are served by the cache), share nothing else and never wait for each other: no LDS, no barrier.
+template <typename T, int NV, int NS, bool WITH_Y>
+__global__ __launch_bounds__(256) void ts_sym_kernel(TsSymArgs g) {
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
+    switch (wave) {
+    case 0:
+        ts_sym_wave<T, NV, NS, WITH_Y, 0>(g);
+        break;
+    case 1:
+        ts_sym_wave<T, NV, NS, WITH_Y, 1>(g);
+        break;
+    case 2:
+        ts_sym_wave<T, NV, NS, WITH_Y, 2>(g);
+        break;
+    default:
+        ts_sym_wave<T, NV, NS, WITH_Y, 3>(g);
     }
 }
 
@@ -288,24 +354,10 @@ __global__ __launch_bounds__(256) void ts_sym_reduce_kernel(T *C, size_t ldc, T 
 
 template <typename T, int NV, int NS>
 static inline dh_status ts_sym_launch(dh_ctx *ctx, const TsSymArgs &g, unsigned blocks, bool with_y) {
-    using S = TsSymShape<T, NV, NS>;
-    const size_t lds = S::lds_bytes();
-    auto k0 = &ts_sym_kernel<T, NV, NS, false>;
-    auto k1 = &ts_sym_kernel<T, NV, NS, true>;
-    if (lds > (size_t(64) << 10)) {
-        static std::mutex attr_lock;
-        static bool attr_set[16][2] = {};
-        std::lock_guard<std::mutex> guard(attr_lock);
-        if (ctx->device < 16 && !attr_set[ctx->device][with_y]) {
-            DH_CHECK_HIP(hipFuncSetAttribute(with_y ? reinterpret_cast<const void *>(k1) : reinterpret_cast<const void *>(k0),
-                                             hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
-            attr_set[ctx->device][with_y] = true;
-        }
-    }
     if (with_y)
-        hipLaunchKernelGGL(k1, dim3(blocks), dim3(256), lds, ctx->stream, g);
+        hipLaunchKernelGGL((ts_sym_kernel<T, NV, NS, true>), dim3(blocks), dim3(256), 0, ctx->stream, g);
     else
-        hipLaunchKernelGGL(k0, dim3(blocks), dim3(256), lds, ctx->stream, g);
+        hipLaunchKernelGGL((ts_sym_kernel<T, NV, NS, false>), dim3(blocks), dim3(256), 0, ctx->stream, g);
     return DH_OK;
 }
 
@@ -319,8 +371,8 @@ bool ts_sym(dh_ctx *ctx, size_t m, size_t K, const T *X, size_t ldx, const T *y,
         return false;
     if (!dh_aligned(X, 16) || ldx % V != 0 || !(m % V == 0 || ldx >= (m + V - 1) / V * V))
         return false;
-    const size_t gran = 16 * 2; // rows per group of a workgroup's four waves
-    size_t blocks = static_cast<size_t>(ctx->num_cus);
+    const size_t gran = 4 * TS_SYM_DEPTH; // rows per turn of a wave's register sets
+    size_t blocks = static_cast<size_t>(ctx->num_cus) * TS_SYM_BLOCKS_PER_CU;
     size_t k_chunk = dh_ceil_div(dh_ceil_div(K, blocks), gran) * gran;
     if (k_chunk < gran * 4)
         k_chunk = gran * 4;

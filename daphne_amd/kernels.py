@@ -314,6 +314,22 @@ def syrk(res, arg: DenseMatrix, transLeft: bool, ctx: HIPContext) -> DenseMatrix
     return res
 
 
+def normalEquations(X: DenseMatrix, y: DenseMatrix, lam: float, ctx: HIPContext, A: Optional[DenseMatrix] = None,
+                    b: Optional[DenseMatrix] = None):
+    """A = t(X) X + lam I and b = t(X) y from one pass over X (dh_normal_equations_*): the operator sequence
+    syrk + ewMul + ewAdd + matMul of scripts/algorithms/lmDS_.daph:60-75. Returns (A, b)."""
+    dt = _same_dtype(X, y, A)
+    if y.rows != X.rows or y.cols != 1:
+        raise capi.DaphneHipError(1, "normalEquations: y must be a column vector with as many rows as X")
+    if A is None:
+        A = DenseMatrix(ctx, X.cols, X.cols, dt)
+    if b is None:
+        b = DenseMatrix(ctx, X.cols, 1, dt)
+    capi.check(_fn("dh_normal_equations", dt)(ctx._h, A.ptr, A.row_skip, b.ptr, b.row_skip, X.ptr, X.rows, X.cols, X.row_skip,
+                                              y.ptr, y.row_skip, lam))
+    return A, b
+
+
 def solve(res, lhs: DenseMatrix, rhs: DenseMatrix, ctx: HIPContext) -> DenseMatrix:
     """CUDA::solve (kernels/CUDA/Solve.h; CPU kernels/Solve.h:86-116): A x = b by LU."""
     dt = _same_dtype(lhs, rhs, res)

@@ -7,7 +7,7 @@ from __future__ import annotations
 import numpy as np
 
 from .kernels import (AggOpCode, BinaryOpCode, DenseMatrix, HIPContext, UnaryOpCode, affineForward, aggCol, aggRow,
-                      conv2dForward, ewBinaryMat, ewBinaryObjSca, ewUnaryMat, matMul, maxPoolForward, softmax, solve,
+                      conv2dForward, ewBinaryMat, ewBinaryObjSca, ewUnaryMat, matMul, maxPoolForward, normalEquations, softmax, solve,
                       syrk)
 from .pipeline import ROWREG, SELF, VectorizedPipeline
 
@@ -15,13 +15,17 @@ from .pipeline import ROWREG, SELF, VectorizedPipeline
 # ------------------------------------------------------------------------------------------------
 # config 1: linear regression by normal equations (lmDS)
 # ------------------------------------------------------------------------------------------------
-def lmds(ctx: HIPContext, X: DenseMatrix, y: DenseMatrix, reg: float, eye: DenseMatrix):
-    """A = t(X) @ X + reg * I ; b = t(X) @ y ; solve(A, b). `eye` is the identity (lmDS_.daph builds
-    diagMatrix(lambda)). Returns (A, b, w)."""
-    A = syrk(None, X, True, ctx)
-    lam = ewBinaryObjSca(BinaryOpCode.MUL, None, eye, reg, ctx)
-    ewBinaryMat(BinaryOpCode.ADD, A, A, lam, ctx)  # in place, res aliases lhs
-    b = matMul(None, X, y, True, False, ctx)
+def lmds(ctx: HIPContext, X: DenseMatrix, y: DenseMatrix, reg: float, eye: DenseMatrix | None = None, fused: bool = True):
+    """A = t(X) @ X + reg * I ; b = t(X) @ y ; solve(A, b). Returns (A, b, w).
+    fused: the normal equations from one pass over X (dh_normal_equations_*); otherwise operator by operator as
+    lmDS_.daph writes them, with `eye` as the identity (the script builds diagMatrix(lambda))."""
+    if fused:
+        A, b = normalEquations(X, y, reg, ctx)
+    else:
+        A = syrk(None, X, True, ctx)
+        lam = ewBinaryObjSca(BinaryOpCode.MUL, None, eye, reg, ctx)
+        ewBinaryMat(BinaryOpCode.ADD, A, A, lam, ctx)  # in place, res aliases lhs
+        b = matMul(None, X, y, True, False, ctx)
     w = solve(None, A, b, ctx)
     return A, b, w
 

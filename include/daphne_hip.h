@@ -539,6 +539,21 @@ dh_status dh_conv2d_backward_filter_f64(dh_ctx *ctx, double *dW, const double *i
 
 
 /* ------------------------------------------------------------------------------------ */
+/* normal equations                                                                      */
+/* ------------------------------------------------------------------------------------ */
+/* A (cols x cols) = t(X) X + lambda I and b (cols x 1, stride ldb) = t(X) y from ONE pass over X (rows x cols):
+ * what scripts/algorithms/lmDS_.daph:60-75 computes as `A = syrk(X) + diagMatrix(lambda)` and `b = t(X) @ y`, i.e.
+ * the operator sequence Syrk (kernels/Syrk.h:51-93) + EwBinaryObjSca MUL + EwBinaryMat ADD + MatMul with transa
+ * (kernels/MatMul.h) - two reads of X and five launches there. For 65..128 columns and at least 4096 rows only the
+ * upper triangle of the product is computed on the matrix cores and t(X) y rides along on the ordinary ALUs; other
+ * shapes run the sequence dh_syrk, a diagonal add, dh_gemv. Results equal the operator sequence's within the
+ * tolerances of the tests (sums in another order). y is rows x 1 with stride ldy. */
+dh_status dh_normal_equations_f32(dh_ctx *ctx, float *A, size_t lda, float *b, size_t ldb, const float *X, size_t rows,
+                                  size_t cols, size_t ldx, const float *y, size_t ldy, float lambda);
+dh_status dh_normal_equations_f64(dh_ctx *ctx, double *A, size_t lda, double *b, size_t ldb, const double *X, size_t rows,
+                                  size_t cols, size_t ldx, const double *y, size_t ldy, double lambda);
+
+/* ------------------------------------------------------------------------------------ */
 /* fused vectorized pipeline                                                             */
 /* ------------------------------------------------------------------------------------ */
 /* Device side of VectorizedPipeline<DenseMatrix<VT>>::apply

@@ -31,11 +31,15 @@ def test_config1_lmds_normal_equations(ctx):
     y = X @ w + 0.1 * rng.standard_normal((n, 1))
     A_e, b_e, w_e = _orc_lmds(X, y, 1e-3)
     eye = DenseMatrix.from_numpy(ctx, np.eye(m))
-    A, b, w_hat = lmds(ctx, DenseMatrix.from_numpy(ctx, X), DenseMatrix.from_numpy(ctx, y), 1e-3, eye)
-    assert_close(A.to_numpy(), A_e, elementwise=False)
-    assert_close(b.to_numpy(), b_e, elementwise=False)
-    assert_close(w_hat.to_numpy(), w_e, rtol=1e-9, elementwise=False)  # cond(A) ~ 3e2 amplifies the 1e-13 of A, b
-    assert np.abs(w_hat.to_numpy() - w).max() < 0.05  # and it recovers the generating weights
+    dX, dy = DenseMatrix.from_numpy(ctx, X), DenseMatrix.from_numpy(ctx, y)
+    # the normal equations from one pass over X, and operator by operator as the script writes them
+    for fused in (True, False):
+        A, b, w_hat = lmds(ctx, dX, dy, 1e-3, eye, fused=fused)
+        assert_close(A.to_numpy(), A_e, elementwise=False)
+        assert_close(b.to_numpy(), b_e, elementwise=False)
+        assert_close(w_hat.to_numpy(), w_e, rtol=1e-9, elementwise=False)  # cond(A) ~ 3e2 amplifies the 1e-13 of A, b
+        assert np.abs(w_hat.to_numpy() - w).max() < 0.05  # and it recovers the generating weights
+        assert_exact(A.to_numpy(), A.to_numpy().T)
 
 
 def test_config2_full_size_properties(ctx):

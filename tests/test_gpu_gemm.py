@@ -338,3 +338,48 @@ def test_matmul_tall_nt(ctx, dt, M, n, K):
     bi = rng.integers(-3, 4, (n, K)).astype(dt)
     goti = matMul(None, DenseMatrix.from_numpy(ctx, ai), DenseMatrix.from_numpy(ctx, bi), False, True, ctx).to_numpy()
     assert_exact(goti, (ai.astype(np.int64) @ bi.T.astype(np.int64)).astype(dt))
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+@pytest.mark.parametrize("cols,ld", [(65, 72), (80, 80), (81, 88), (96, 96), (100, 100), (111, 112), (112, 120), (113, 128),
+                                      (128, 128)])
+@pytest.mark.parametrize("rows", [4096, 10_007])
+def test_syrk_and_normal_equations_of_65_to_128_columns(ctx, dt, cols, ld, rows):
+    """The triangle-only kernel for 65..128 columns (every tile count and tail shape, rows that do not fill the last
+    step, a view with a row stride): syrk, and the normal equations with t(X) y from the same pass, against the
+    oracle's Syrk / MatMul and against float64 numpy."""
+    from daphne_amd.kernels import normalEquations
+
+    if (ld * np.dtype(dt).itemsize) % 16:
+        pytest.skip("rows of this stride are not 16-byte aligned for this value type: the general kernels take it")
+    rng = np.random.default_rng(rows + cols)
+    base = np.full((rows, ld), np.nan, dt)  # what lies beyond the columns must never reach a result
+    base[:, :cols] = (rng.random((rows, cols)) * 2 - 1).astype(dt)
+    x = base[:, :cols]
+    y = (rng.random((rows, 1)) * 2 - 1).astype(dt)
+    X = DenseMatrix.from_numpy(ctx, base).slice(0, rows, 0, cols)
+    Y = DenseMatrix.from_numpy(ctx, y)
+    S = syrk(None, X, True, ctx).to_numpy()
+    assert_exact(S, S.T)
+    assert_close(S, orc.syrk(np.ascontiguousarray(x), True)[1], elementwise=False)
+    lam = 0.25
+    A, b = normalEquations(X, Y, lam, ctx)
+    x64 = x.astype(np.float64)
+    assert_close(A.to_numpy(), (x64.T @ x64 + lam * np.eye(cols)).astype(dt), elementwise=False)
+    assert_close(b.to_numpy(), (x64.T @ y.astype(np.float64)).astype(dt), elementwise=False)
+    assert_exact(A.to_numpy() - np.diag(np.diag(A.to_numpy())), S - np.diag(np.diag(S)))  # the same kernel, with and without y
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+@pytest.mark.parametrize("rows,cols", [(5000, 20), (300, 100), (7000, 64), (4096, 200)])
+def test_normal_equations_of_other_shapes(ctx, dt, rows, cols):
+    """Shapes the fused kernel does not take run the operator sequence; same results."""
+    from daphne_amd.kernels import normalEquations
+
+    rng = np.random.default_rng(cols)
+    x = (rng.random((rows, cols)) * 2 - 1).astype(dt)
+    y = (rng.random((rows, 1)) * 2 - 1).astype(dt)
+    A, b = normalEquations(DenseMatrix.from_numpy(ctx, x), DenseMatrix.from_numpy(ctx, y), 1e-3, ctx)
+    x64 = x.astype(np.float64)
+    assert_close(A.to_numpy(), (x64.T @ x64 + 1e-3 * np.eye(cols)).astype(dt), elementwise=False)
+    assert_close(b.to_numpy(), (x64.T @ y.astype(np.float64)).astype(dt), elementwise=False)
