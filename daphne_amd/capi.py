@@ -113,8 +113,11 @@ _LATE_SIGNATURES: dict[str, list] = {
     "dh_solve": [vp, vp, vp, sz, sz, vp],
     "dh_normal_equations": [vp, vp, sz, vp, sz, vp, sz, sz, sz, vp, sz, "T"],
     "dh_conv2d_forward": [vp, vp, C.POINTER(sz), C.POINTER(sz), vp, vp, sz, sz, vp, sz, sz, sz, sz, sz, sz, sz, sz, sz, sz],
+    "dh_conv2d_forward_fused": [vp, vp, C.POINTER(sz), C.POINTER(sz), vp, vp, sz, sz, vp, sz, sz, sz, sz, sz, sz, sz, sz, sz, sz,
+                                C.c_uint],
     "dh_maxpool_forward": [vp, vp, C.POINTER(sz), C.POINTER(sz), vp, sz, sz, sz, sz, sz, sz, sz, sz, sz, sz],
     "dh_affine_forward": [vp, vp, vp, sz, sz, vp, sz, sz, vp, sz, sz],
+    "dh_affine_forward_fused": [vp, vp, vp, sz, sz, vp, sz, sz, vp, sz, sz, C.c_uint],
     "dh_bias_add": [vp, vp, vp, sz, sz, vp, sz],
     "dh_batchnorm_inference": [vp, vp, vp, sz, sz, vp, vp, vp, vp, sz, "T", i32],
     "dh_softmax": [vp, vp, sz, vp, sz, sz, sz],

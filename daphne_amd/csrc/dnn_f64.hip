@@ -10,6 +10,15 @@ extern "C" dh_status dh_conv2d_forward_f64(dh_ctx *ctx, double *res, size_t *res
                                       channels, img_h, img_w, filter_h, filter_w, stride_h, stride_w, pad_h, pad_w);
 }
 
+extern "C" dh_status dh_conv2d_forward_fused_f64(dh_ctx *ctx, double *res, size_t *res_h, size_t *res_w, const double *data,
+                                                const double *filter, size_t filter_rows, size_t filter_cols, const double *bias,
+                                                size_t batch, size_t channels, size_t img_h, size_t img_w, size_t filter_h,
+                                                size_t filter_w, size_t stride_h, size_t stride_w, size_t pad_h,
+                                                size_t pad_w, unsigned epilogue) {
+    return dh_dnn::conv2d_forward<double>(ctx, res, res_h, res_w, data, filter, filter_rows, filter_cols, bias, batch,
+                                      channels, img_h, img_w, filter_h, filter_w, stride_h, stride_w, pad_h, pad_w, epilogue);
+}
+
 extern "C" dh_status dh_maxpool_forward_f64(dh_ctx *ctx, double *res, size_t *res_h, size_t *res_w, const double *data,
                                            size_t batch, size_t channels, size_t img_h, size_t img_w, size_t pool_h,
                                            size_t pool_w, size_t stride_h, size_t stride_w, size_t pad_h,

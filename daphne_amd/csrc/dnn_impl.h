@@ -30,6 +30,7 @@
 namespace dh_dnn {
 
 using dh_gemm::Mfma;
+using dh_gemm::relu_of;
 using dh_gemm::TileLayout;
 using dh_gemm::TileMover;
 
@@ -41,8 +42,11 @@ struct ConvArgs {
     void *res;
     unsigned F, K, Kpad, P, Q, sh, sw, Wp;
     unsigned CHpWp;      // elements of one padded image
-    size_t pixels;       // N*P*Q
+    unsigned relu;       // 1: max(0, .) after the bias, as ewBinaryObjSca(MAX, ., 0) computes it
+    unsigned Qo, PQo;    // POOL: width and size of the pooled output plane
+    size_t pixels;       // N*P*Q; POOL: 4*N*PQo, the window positions of a pooled pixel being four consecutive "pixels"
 };
+
 
 // Table of patch offsets and the zero-padded filter matrix, so that the main loop has neither divisions
 // nor bounds checks on the filter side.
@@ -88,9 +92,13 @@ __global__ __launch_bounds__(256) void conv_pad_kernel(T *xpad, const T *x, size
     xpad[i] = (y < H && x_ < W) ? x[plane * H * W + static_cast<size_t>(y) * W + x_] : T(0);
 }
 
-template <typename T, int BM, int BN, int BK, int WN>
+// POOL: the 2 x 2 / stride 2 maximum of the (biased, optionally rectified) convolution as maxPoolForward computes it
+// (running maximum from zero over the window in row order, Pooling.cpp:77-105). The tile's pixel index then counts
+// window positions, four to a pooled pixel, so that a window's values sit in four neighbouring lanes at the end.
+template <typename T, int BM, int BN, int BK, int WN, bool POOL = false>
 __global__ __launch_bounds__(64 * WN) void conv2d_kernel(ConvArgs g) {
     using M = Mfma<T>;
+    static_assert(!POOL || (M::NT % 4 == 0 && BN % 4 == 0), "a window's four positions stay in one block of pixels");
     constexpr int THREADS = 64 * WN;
     constexpr int TN = BN / WN;
     constexpr int FM = BM / M::MT, FN = TN / M::NT;
@@ -107,7 +115,7 @@ __global__ __launch_bounds__(64 * WN) void conv2d_kernel(ConvArgs g) {
     const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
     const size_t pix0 = static_cast<size_t>(blockIdx.x) * BN;
     const unsigned f0 = blockIdx.y * BM;
-    const unsigned PQ = g.P * g.Q;
+    const unsigned PQ = POOL ? 4 * g.PQo : g.P * g.Q; // "pixels" per image
     const bool small = g.pixels <= 0xffffffffull; // 32-bit divisions suffice (uniform)
 
     // Gather mapping: thread -> one pixel of the tile and a group of KPT consecutive k. The k group is the
@@ -129,7 +137,15 @@ __global__ __launch_bounds__(64 * WN) void conv2d_kernel(ConvArgs g) {
         img = static_cast<unsigned>(gpix / PQ);
         pq = static_cast<unsigned>(gpix % PQ);
     }
-    const unsigned p = pq / g.Q, q = pq % g.Q;
+    unsigned p, q;
+    if constexpr (POOL) {
+        const unsigned po = pq / 4, wpos = pq % 4;
+        p = 2 * (po / g.Qo) + wpos / 2;
+        q = 2 * (po % g.Qo) + wpos % 2;
+    } else {
+        p = pq / g.Q;
+        q = pq % g.Q;
+    }
     const char *xblk = reinterpret_cast<const char *>(static_cast<const T *>(g.xpad) + img0 * g.CHpWp);
     // byte offset of this pixel's window origin from the block's first image (the host checks the range)
     const unsigned voff = static_cast<unsigned>(((img - static_cast<unsigned>(img0)) * g.CHpWp + p * g.sh * g.Wp + q * g.sw) *
@@ -247,23 +263,45 @@ __global__ __launch_bounds__(64 * WN) void conv2d_kernel(ConvArgs g) {
 #pragma unroll
     for (int j = 0; j < FN; j++) {
         const size_t pix = pix0 + wave * TN + j * M::NT + M::col(lane);
-        if (pix < g.pixels) {
-            size_t oimg, opq;
-            if (small) {
-                oimg = static_cast<unsigned>(pix) / PQ;
-                opq = static_cast<unsigned>(pix) % PQ;
-            } else {
-                oimg = pix / PQ;
-                opq = pix % PQ;
-            }
+        const bool live = pix < g.pixels; // POOL: the same for the four lanes of a window
+        size_t oimg, opq;
+        if (small) {
+            oimg = static_cast<unsigned>(live ? pix : 0) / PQ;
+            opq = static_cast<unsigned>(live ? pix : 0) % PQ;
+        } else {
+            oimg = (live ? pix : 0) / PQ;
+            opq = (live ? pix : 0) % PQ;
+        }
+        if constexpr (POOL) {
+            T *obase = out + oimg * g.F * g.PQo + opq / 4;
+#pragma unroll
+            for (int i = 0; i < FM; i++)
+#pragma unroll
+                for (int v = 0; v < M::ACC; v++) {
+                    const size_t f = f0 + i * M::MT + M::row(lane, v);
+                    T o = acc[i][j][v] + bv[i][v];
+                    o = g.relu ? relu_of(o) : o;
+                    // the window's values in row order, from the four lanes of the quad
+                    const T w0 = dh_dpp<0x00>(o), w1 = dh_dpp<0x55>(o), w2 = dh_dpp<0xAA>(o), w3 = dh_dpp<0xFF>(o);
+                    T m = T(0);
+                    m = (m < w0) ? w0 : m;
+                    m = (m < w1) ? w1 : m;
+                    m = (m < w2) ? w2 : m;
+                    m = (m < w3) ? w3 : m;
+                    if (live && lane % 4 == 0 && f < g.F)
+                        obase[f * g.PQo] = m;
+                }
+        } else if (live) {
             T *obase = out + oimg * g.F * PQ + opq;
 #pragma unroll
             for (int i = 0; i < FM; i++)
 #pragma unroll
                 for (int v = 0; v < M::ACC; v++) {
                     const size_t f = f0 + i * M::MT + M::row(lane, v);
-                    if (f < g.F)
-                        obase[f * PQ] = acc[i][j][v] + bv[i][v];
+                    if (f < g.F) {
+                        const T o = acc[i][j][v] + bv[i][v];
+                        obase[f * PQ] = g.relu ? relu_of(o) : o;
+                    }
                 }
         }
     }
@@ -286,6 +324,8 @@ struct ConvResidentArgs {
     unsigned C, H, W, Hp, Wp, ph, pw, Q, sh, sw, F, Kpad, HpWp, PQ, chunk;
     unsigned CG, KG;   // channels per stage of the LDS image and their share of K (a multiple of the K block)
     unsigned N, NI;    // images in all, images per workgroup (their pixels form one pixel range)
+    unsigned relu;     // 1: max(0, .) after the bias
+    unsigned Qo, PQo;  // POOL: width and size of the pooled output plane (PQ, Q stay those of the convolution)
 };
 
 // Copies one image (C x H x W at x) into LDS as C x Hp x Wp with the zero border of Padding.h:11-22 written out,
@@ -345,7 +385,11 @@ __device__ __forceinline__ void conv_stage_frame(T *frame, const T *x, unsigned 
     }
 }
 
-template <typename T, int MFW, int NF>
+// POOL: the result is the 2 x 2 / stride 2 maximum of the (biased, optionally rectified) convolution, as maxPoolForward
+// computes it (running maximum from zero over the window in row order, Pooling.cpp:77-105). The pixel index that
+// workgroups and waves divide among themselves then counts window positions, four to a pooled pixel, so that a
+// window's values end up in four neighbouring lanes.
+template <typename T, int MFW, int NF, bool POOL>
 __global__ __launch_bounds__(512) void conv2d_resident_kernel(ConvResidentArgs g) {
     using M = dh_gemm::Mfma16<T>;
     constexpr int VEC = 16 / sizeof(T), NPARTS = 8 / MFW;
@@ -355,7 +399,8 @@ __global__ __launch_bounds__(512) void conv2d_resident_kernel(ConvResidentArgs g
     const int tid = threadIdx.x, lane = tid % 64, wave = __builtin_amdgcn_readfirstlane(tid / 64);
     const unsigned img = blockIdx.x * g.NI, f0 = blockIdx.y * (16 * MFW), px0 = blockIdx.z * g.chunk;
     const unsigned nimg = (g.N - img < g.NI) ? g.N - img : g.NI; // images of this workgroup
-    const unsigned npix = nimg * g.PQ, stage_elems = g.CG * g.HpWp;
+    const unsigned PQv = POOL ? 4 * g.PQo : g.PQ, PQout = POOL ? g.PQo : g.PQ; // "pixels" and results per image
+    const unsigned npix = nimg * PQv, stage_elems = g.CG * g.HpWp;
 
     // the offset table: its first 2048 entries are asked for now and put into LDS after the first image stage has
     // been copied in, so that both sets of loads are on their way together
@@ -376,11 +421,19 @@ __global__ __launch_bounds__(512) void conv2d_resident_kernel(ConvResidentArgs g
     for (int j = 0; j < NF; j++) {
         const unsigned first = px0 + (j * NPARTS + part) * 16; // blocks dealt round-robin: the waves' counts differ by at most one
         const unsigned px = first + li;
-        const bool ok = px < npix;
-        const unsigned il = ok ? px / g.PQ : 0, pq = ok ? px % g.PQ : 0; // image of the workgroup, pixel in it
-        const unsigned pp = pq / g.Q, qq = pq % g.Q;
+        const bool ok = px < npix; // POOL: the same for the four lanes of a window
+        const unsigned il = ok ? px / PQv : 0, pq = ok ? px % PQv : 0; // image of the workgroup, pixel in it
+        unsigned pp, qq, po = pq;
+        if constexpr (POOL) {
+            po = pq / 4;
+            pp = 2 * (po / g.Qo) + (pq % 4) / 2;
+            qq = 2 * (po % g.Qo) + (pq % 4) % 2;
+        } else {
+            pp = pq / g.Q;
+            qq = pq % g.Q;
+        }
         pixoff[j] = static_cast<int>(il * stage_elems + pp * g.sh * g.Wp + qq * g.sw);
-        outoff[j] = ok ? static_cast<int>(il * g.F * g.PQ + pq) : -1;
+        outoff[j] = ok ? static_cast<int>(il * g.F * PQout + po) : -1;
         if (first < npix)
             nfv = j + 1;
     }
@@ -465,7 +518,7 @@ __global__ __launch_bounds__(512) void conv2d_resident_kernel(ConvResidentArgs g
             contract(std::integral_constant<int, NF>{}, k_begin, k_end, sub);
     }
 
-    T *out = static_cast<T *>(g.res) + static_cast<size_t>(img) * g.F * g.PQ;
+    T *out = static_cast<T *>(g.res) + static_cast<size_t>(img) * g.F * PQout;
     const T *bias = static_cast<const T *>(g.bias);
     T bv[4];
 #pragma unroll
@@ -473,35 +526,72 @@ __global__ __launch_bounds__(512) void conv2d_resident_kernel(ConvResidentArgs g
         const unsigned f = f0 + mf * 16 + M::row(lane, v);
         bv[v] = (bias && f < g.F) ? bias[f] : T(0);
     }
+    if constexpr (POOL) {
 #pragma unroll
-    for (int j = 0; j < NF; j++) {
-        if (j < nfv && outoff[j] >= 0) {
+        for (int j = 0; j < NF; j++) {
+            if (j < nfv) {
 #pragma unroll
-            for (int v = 0; v < 4; v++) {
-                const unsigned f = f0 + mf * 16 + M::row(lane, v);
-                if (f < g.F)
-                    out[static_cast<size_t>(f) * g.PQ + outoff[j]] = acc[j][v] + bv[v];
+                for (int v = 0; v < 4; v++) {
+                    const unsigned f = f0 + mf * 16 + M::row(lane, v);
+                    T o = acc[j][v] + bv[v];
+                    o = g.relu ? relu_of(o) : o;
+                    // the window's values in row order, from the four lanes of the quad
+                    const T w0 = dh_dpp<0x00>(o), w1 = dh_dpp<0x55>(o), w2 = dh_dpp<0xAA>(o), w3 = dh_dpp<0xFF>(o);
+                    T m = T(0);
+                    m = (m < w0) ? w0 : m;
+                    m = (m < w1) ? w1 : m;
+                    m = (m < w2) ? w2 : m;
+                    m = (m < w3) ? w3 : m;
+                    if (outoff[j] >= 0 && lane % 4 == 0 && f < g.F)
+                        out[static_cast<size_t>(f) * PQout + outoff[j]] = m;
+                }
+            }
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < NF; j++) {
+            if (j < nfv && outoff[j] >= 0) {
+#pragma unroll
+                for (int v = 0; v < 4; v++) {
+                    const unsigned f = f0 + mf * 16 + M::row(lane, v);
+                    if (f < g.F) {
+                        const T o = acc[j][v] + bv[v];
+                        out[static_cast<size_t>(f) * g.PQ + outoff[j]] = g.relu ? relu_of(o) : o;
+                    }
+                }
             }
         }
     }
 }
 
-template <typename T, int MFW, int NF> static inline dh_status conv2d_resident_launch(dh_ctx *ctx, const ConvResidentArgs &g, dim3 grid, size_t lds) {
+template <typename T, int MFW, int NF, bool POOL = false>
+static inline dh_status conv2d_resident_launch(dh_ctx *ctx, const ConvResidentArgs &g, dim3 grid, size_t lds) {
     // dynamic LDS beyond 64 KiB has to be asked for, per kernel and device (the call is cheap next to the kernel)
     if (lds > 65536) {
-        DH_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&conv2d_resident_kernel<T, MFW, NF>),
+        DH_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&conv2d_resident_kernel<T, MFW, NF, POOL>),
                                          hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
     }
-    hipLaunchKernelGGL((conv2d_resident_kernel<T, MFW, NF>), grid, dim3(512), lds, ctx->stream, g);
+    hipLaunchKernelGGL((conv2d_resident_kernel<T, MFW, NF, POOL>), grid, dim3(512), lds, ctx->stream, g);
     DH_CHECK_LAUNCH();
     return DH_OK;
 }
 
 template <typename T>
+dh_status maxpool_forward(dh_ctx *ctx, T *res, size_t *res_h, size_t *res_w, const T *data, size_t N, size_t C,
+                          size_t H, size_t W, size_t ph, size_t pw, size_t sh, size_t sw, size_t padh, size_t padw);
+
+// epilogue: DH_EPILOGUE_RELU and / or DH_EPILOGUE_MAXPOOL_2X2, applied to the biased convolution in that order; the
+// results are those of the separate operators (conv2dForward, ewBinaryObjSca(MAX, ., 0), maxPoolForward 2 x 2 / 2),
+// bit for bit. With pooling, res is N x F * (P / 2) * (Q / 2) and res_h / res_w are the pooled extents.
+template <typename T>
 dh_status conv2d_forward(dh_ctx *ctx, T *res, size_t *res_h, size_t *res_w, const T *data, const T *filter,
                          size_t filter_rows, size_t filter_cols, const T *bias, size_t N, size_t C, size_t H,
-                         size_t W, size_t Hf, size_t Wf, size_t sh, size_t sw, size_t ph, size_t pw) {
+                         size_t W, size_t Hf, size_t Wf, size_t sh, size_t sw, size_t ph, size_t pw,
+                         unsigned epilogue = 0) {
     DH_REQUIRE_CTX(ctx);
+    if (epilogue & ~(DH_EPILOGUE_RELU | DH_EPILOGUE_MAXPOOL_2X2))
+        return dh_fail(DH_ERR_INVALID_ARG, "Convolution: unknown epilogue flags %#x", epilogue);
+    const bool relu = (epilogue & DH_EPILOGUE_RELU) != 0, pool = (epilogue & DH_EPILOGUE_MAXPOOL_2X2) != 0;
     const size_t F = filter_rows;
     if (filter_rows * filter_cols != F * C * Hf * Wf)
         // kernels/CUDA/Convolution.cpp:32-39
@@ -512,10 +602,13 @@ dh_status conv2d_forward(dh_ctx *ctx, T *res, size_t *res_h, size_t *res_w, cons
         return dh_fail(DH_ERR_INVALID_ARG, "Convolution: filter %zux%zu does not fit the padded image %zux%zu",
                        Hf, Wf, H + 2 * ph, W + 2 * pw);
     const size_t P = (H + 2 * ph - Hf) / sh + 1, Q = (W + 2 * pw - Wf) / sw + 1; // Padding.h:6-9
+    if (pool && (P < 2 || Q < 2))
+        return dh_fail(DH_ERR_INVALID_ARG, "Pooling: window 2x2 does not fit the padded image %zux%zu", P, Q);
+    const size_t Po = pool ? (P - 2) / 2 + 1 : P, Qo = pool ? (Q - 2) / 2 + 1 : Q; // Pooling.cpp:38-39
     if (res_h)
-        *res_h = P;
+        *res_h = Po;
     if (res_w)
-        *res_w = Q;
+        *res_w = Qo;
     const size_t pixels = N * P * Q;
     if (pixels == 0 || F == 0)
         return DH_OK;
@@ -523,7 +616,8 @@ dh_status conv2d_forward(dh_ctx *ctx, T *res, size_t *res_h, size_t *res_w, cons
     constexpr int BN = 128;
     const size_t Hp = H + 2 * ph, Wp = W + 2 * pw, K = C * Hf * Wf;
     // a workgroup addresses its pixels with 32-bit byte offsets from its first image
-    const size_t images_per_tile = (BN + P * Q - 2) / (P * Q) + 1;
+    const size_t tile_px = pool ? 4 * Po * Qo : P * Q; // "pixels" per image as the tiled kernel counts them
+    const size_t images_per_tile = (BN + tile_px - 2) / tile_px + 1;
     if (C * Hp * Wp * images_per_tile * sizeof(T) >= (size_t(1) << 32) || K >= (size_t(1) << 31) ||
         P * Q >= (size_t(1) << 31) || N >= (size_t(1) << 31) || F >= (size_t(1) << 31))
         return dh_fail(DH_ERR_RUNTIME, "Convolution: image or filter extents exceed the 32-bit addressing of a tile");
@@ -571,6 +665,8 @@ dh_status conv2d_forward(dh_ctx *ctx, T *res, size_t *res_h, size_t *res_w, cons
         // runs: 1 -> 32 channels, 5 x 5 on 28 x 28 takes 0.16 ms there and 0.28 ms here.
         // (One thread per pixel on the ordinary ALUs, weights broadcast from LDS, was tried for that layer as well:
         // 0.15 ms, bound by the LDS reads of the weights; four pixels per thread to share them: 0.20 ms.)
+        // The choice does not look at the epilogue: the two kernels add up a result's terms in different orders, and
+        // a call with an epilogue has to give the bits of the plain call.
         if (cg != 0 && lds <= 150 * 1024 && (lds <= 80 * 1024 || nf >= 6) && blocks16 >= 3 * parts && K >= 32 && fgroups < 65536 &&
             chunks < 65536) {
             const size_t fpad = fgroups * 16 * mfw;
@@ -614,6 +710,24 @@ dh_status conv2d_forward(dh_ctx *ctx, T *res, size_t *res_h, size_t *res_w, cons
             r.NI = static_cast<unsigned>(ni);
             r.PQ = static_cast<unsigned>(P * Q);
             r.chunk = static_cast<unsigned>(chunk);
+            r.relu = relu;
+            r.Qo = static_cast<unsigned>(Qo);
+            r.PQo = static_cast<unsigned>(Po * Qo);
+            if (pool) {
+                // the same division of work over the window positions, four to a pooled pixel (fewer than P * Q where P or Q is odd)
+                const size_t pblocks = dh_ceil_div(ni * 4 * Po * Qo, 16);
+                const size_t pchunks = dh_ceil_div(pblocks, parts * 13);
+                const size_t np = dh_ceil_div(pblocks, parts * pchunks);
+                r.chunk = static_cast<unsigned>(parts * np * 16);
+                const dim3 pgrid(static_cast<unsigned>(igroups), static_cast<unsigned>(fgroups), static_cast<unsigned>(pchunks));
+#define DH_CONV_POOL(MFW_)                                                                         \
+    (np <= 4 ? conv2d_resident_launch<T, MFW_, 4, true>(ctx, r, pgrid, lds)                        \
+             : (np <= 7 ? conv2d_resident_launch<T, MFW_, 7, true>(ctx, r, pgrid, lds)             \
+                        : (np <= 10 ? conv2d_resident_launch<T, MFW_, 10, true>(ctx, r, pgrid, lds) \
+                                    : conv2d_resident_launch<T, MFW_, 13, true>(ctx, r, pgrid, lds))))
+                return mfw == 1 ? DH_CONV_POOL(1) : (mfw == 2 ? DH_CONV_POOL(2) : DH_CONV_POOL(4));
+#undef DH_CONV_POOL
+            }
             const dim3 grid(static_cast<unsigned>(igroups), static_cast<unsigned>(fgroups), static_cast<unsigned>(chunks));
 #define DH_CONV_RES(MFW_)                                                                          \
     (nf <= 4 ? conv2d_resident_launch<T, MFW_, 4>(ctx, r, grid, lds)                               \
@@ -624,7 +738,8 @@ dh_status conv2d_forward(dh_ctx *ctx, T *res, size_t *res_h, size_t *res_w, cons
 #undef DH_CONV_RES
         }
     }
-    const size_t gx = dh_ceil_div(pixels, BN);
+    const size_t vpixels = pool ? 4 * N * Po * Qo : pixels; // the tile's pixel index counts window positions with pooling
+    const size_t gx = dh_ceil_div(vpixels, BN);
     if (gx >= (size_t(1) << 31))
         return dh_fail(DH_ERR_RUNTIME, "Convolution: too many output pixels for one launch");
     const int BM = F <= 32 ? 32 : 64;
@@ -677,13 +792,21 @@ dh_status conv2d_forward(dh_ctx *ctx, T *res, size_t *res_h, size_t *res_w, cons
     g.sw = static_cast<unsigned>(sw);
     g.Wp = static_cast<unsigned>(Wp);
     g.CHpWp = static_cast<unsigned>(C * Hp * Wp);
-    g.pixels = pixels;
-    if (BM == 32)
-        hipLaunchKernelGGL((conv2d_kernel<T, 32, BN, BK, 4>), dim3(static_cast<unsigned>(gx), gy), dim3(256), 0,
-                           ctx->stream, g);
-    else
-        hipLaunchKernelGGL((conv2d_kernel<T, 64, BN, BK, 4>), dim3(static_cast<unsigned>(gx), gy), dim3(256), 0,
-                           ctx->stream, g);
+    g.relu = relu;
+    g.Qo = static_cast<unsigned>(Qo);
+    g.PQo = static_cast<unsigned>(Po * Qo);
+    g.pixels = vpixels;
+    const dim3 grid(static_cast<unsigned>(gx), gy);
+    if (pool) {
+        if (BM == 32)
+            hipLaunchKernelGGL((conv2d_kernel<T, 32, BN, BK, 4, true>), grid, dim3(256), 0, ctx->stream, g);
+        else
+            hipLaunchKernelGGL((conv2d_kernel<T, 64, BN, BK, 4, true>), grid, dim3(256), 0, ctx->stream, g);
+    } else if (BM == 32) {
+        hipLaunchKernelGGL((conv2d_kernel<T, 32, BN, BK, 4>), grid, dim3(256), 0, ctx->stream, g);
+    } else {
+        hipLaunchKernelGGL((conv2d_kernel<T, 64, BN, BK, 4>), grid, dim3(256), 0, ctx->stream, g);
+    }
     DH_CHECK_LAUNCH();
     return DH_OK;
 }

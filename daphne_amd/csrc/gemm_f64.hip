@@ -20,6 +20,13 @@ extern "C" dh_status dh_affine_forward_f64(dh_ctx *ctx, double *res, const doubl
                                bias_cols);
 }
 
+extern "C" dh_status dh_affine_forward_fused_f64(dh_ctx *ctx, double *res, const double *data, size_t data_rows, size_t data_cols,
+                                                const double *weights, size_t w_rows, size_t w_cols, const double *bias,
+                                                size_t bias_rows, size_t bias_cols, unsigned epilogue) {
+    return dh_gemm::affine<double>(ctx, res, data, data_rows, data_cols, weights, w_rows, w_cols, bias, bias_rows,
+                               bias_cols, epilogue);
+}
+
 // Gemv<DenseMatrix<T>,...>::apply (kernels/Gemv.h:51-77, kernels/CUDA/Gemv.cpp:42-68): res = t(mat) vec.
 extern "C" dh_status dh_gemv_f64(dh_ctx *ctx, double *res, size_t ld_res, const double *mat, size_t rows, size_t cols, size_t ld_mat,
                                   const double *vec, size_t vec_rows, size_t ld_vec) {

@@ -153,7 +153,11 @@ struct GemmArgs {
     int aligned_a, aligned_b;
     int tile_offset;    // added to the workgroup's tile id (the launch that finishes the tiles a first launch left)
     int compact;        // 1: C holds one dense BM x BN block per (K slice, workgroup) instead of the result matrix
+    int relu;           // 1: max(0, .) on the finished values (with the bias, where the bias is added)
 };
+
+// max(x, 0) with the comparison of the elementwise MAX operator ((x < 0) ? 0 : x: NaN and -0 pass through).
+template <typename T> __device__ __forceinline__ T relu_of(T x) { return (x < T(0)) ? T(0) : x; }
 
 // Consecutive workgroup ids are dealt round-robin to the 8 XCDs: regroup them so that each XCD walks a
 // contiguous range of tile ids.
@@ -324,8 +328,10 @@ __global__ __launch_bounds__(64 * WM * WN, FULL ? 2 : 1) void gemm_kernel(GemmAr
 #pragma unroll
                 for (int v = 0; v < M::ACC; v++) {
                     const size_t r = m0 + wave_m * TM + i * M::MT + M::row(lane, v);
-                    if (FULL || r < g.m)
-                        C[(r - row_off) * ldc + (c - col_off)] = acc[i][j][v] + b;
+                    if (FULL || r < g.m) {
+                        const T o = acc[i][j][v] + b;
+                        C[(r - row_off) * ldc + (c - col_off)] = (EPI == EPI_BIAS && g.relu) ? relu_of(o) : o;
+                    }
                 }
             }
         }
@@ -336,7 +342,7 @@ __global__ __launch_bounds__(64 * WM * WN, FULL ? 2 : 1) void gemm_kernel(GemmAr
 template <typename T, bool MIRROR>
 __global__ __launch_bounds__(256) void slab_reduce_kernel(T *C, size_t ldc, const T *slabs, size_t slab_stride,
                                                           size_t ld_slab, int nslabs, size_t m, size_t n,
-                                                          const T *bias, size_t bias_stride) {
+                                                          const T *bias, size_t bias_stride, int relu) {
     const size_t c = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     const size_t r = static_cast<size_t>(blockIdx.y) * blockDim.y + threadIdx.y;
     if (r >= m || c >= n)
@@ -348,6 +354,8 @@ __global__ __launch_bounds__(256) void slab_reduce_kernel(T *C, size_t ldc, cons
         s += slabs[static_cast<size_t>(z) * slab_stride + r * ld_slab + c];
     if (bias)
         s += bias[c * bias_stride];
+    if (relu)
+        s = relu_of(s);
     C[r * ldc + c] = s;
     if (MIRROR && c != r)
         C[c * ldc + r] = s;
@@ -377,6 +385,8 @@ __global__ __launch_bounds__(256) void tail_reduce_kernel(GemmArgs g, const T *s
         sum += p[z * step];
     if (bias)
         sum += bias[c * g.bias_stride];
+    if (g.relu)
+        sum = relu_of(sum);
     C[r * g.ldc + c] = sum;
 }
 
@@ -507,7 +517,8 @@ template <typename T> struct GemmBK {
 // A, B are the stored matrices; m, n, k are the GEMM dimensions after applying the transposes.
 template <typename T>
 dh_status gemm(dh_ctx *ctx, bool ta, bool tb, size_t m, size_t n, size_t k, const T *A, size_t lda, const T *B,
-               size_t ldb, T *C, size_t ldc, const T *bias, bool triangular, size_t bias_stride = 1) {
+               size_t ldb, T *C, size_t ldc, const T *bias, bool triangular, size_t bias_stride = 1, bool relu = false) {
+    // relu: only together with a bias (the stage that adds the bias applies it)
     if (m == 0 || n == 0)
         return DH_OK;
     // tall-and-skinny shapes stream straight from HBM into the matrix cores
@@ -530,6 +541,7 @@ dh_status gemm(dh_ctx *ctx, bool ta, bool tb, size_t m, size_t n, size_t k, cons
     g.B = B;
     g.bias = bias;
     g.bias_stride = bias_stride;
+    g.relu = (relu && bias != nullptr) ? 1 : 0;
     g.m = m;
     g.n = n;
     g.k = k;
@@ -671,10 +683,10 @@ dh_status gemm(dh_ctx *ctx, bool ta, bool tb, size_t m, size_t n, size_t k, cons
     if (!direct) {
         if (triangular)
             hipLaunchKernelGGL((slab_reduce_kernel<T, true>), eg, eb, 0, ctx->stream, C, ldc, slabs, m * n, n,
-                               static_cast<int>(ksplit), m, n, bias, bias_stride);
+                               static_cast<int>(ksplit), m, n, bias, bias_stride, g.relu);
         else
             hipLaunchKernelGGL((slab_reduce_kernel<T, false>), eg, eb, 0, ctx->stream, C, ldc, slabs, m * n, n,
-                               static_cast<int>(ksplit), m, n, bias, bias_stride);
+                               static_cast<int>(ksplit), m, n, bias, bias_stride, g.relu);
         DH_CHECK_LAUNCH();
     } else if (triangular) {
         const unsigned mt = static_cast<unsigned>(dh_ceil_div(n, 64));
@@ -783,11 +795,20 @@ dh_status syrk(dh_ctx *ctx, T *res, size_t ld_res, const T *arg, size_t rows, si
     return gemm<T>(ctx, trans_left != 0, trans_left == 0, n, n, k, arg, ld, arg, ld, res, ld_res, nullptr, true);
 }
 
-// CUDA::NN::Affine::Forward::apply of kernels/CUDA/Affine.cpp:42-83.
+template <typename T> __global__ __launch_bounds__(256) void relu_inplace_kernel(T *p, size_t n) {
+    for (size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x; i < n; i += static_cast<size_t>(gridDim.x) * 256)
+        p[i] = relu_of(p[i]);
+}
+
+// CUDA::NN::Affine::Forward::apply of kernels/CUDA/Affine.cpp:42-83; epilogue DH_EPILOGUE_RELU: followed by
+// CUDA::NN::Activation::Forward<ReLU> (kernels/CUDA/Activation.cpp:21-47), in the same pass where a bias is added.
 template <typename T>
 dh_status affine(dh_ctx *ctx, T *res, const T *data, size_t dr, size_t dc, const T *w, size_t wr, size_t wc,
-                 const T *bias, size_t br, size_t bc) {
+                 const T *bias, size_t br, size_t bc, unsigned epilogue = 0) {
     DH_REQUIRE_CTX(ctx);
+    if (epilogue & ~static_cast<unsigned>(DH_EPILOGUE_RELU))
+        return dh_fail(DH_ERR_INVALID_ARG, "Affine: unknown epilogue flags %#x", epilogue);
+    const bool relu = epilogue != 0;
     if (dc != wr)
         return dh_fail(DH_ERR_RUNTIME, "CUDA::NN::Affine: #cols of lhs and #rows of rhs must be the same (%zu != %zu)",
                        dc, wr);
@@ -800,7 +821,16 @@ dh_status affine(dh_ctx *ctx, T *res, const T *data, size_t dr, size_t dc, const
         if (bc != wc && bc != 1)
             return dh_fail(DH_ERR_RUNTIME, "Affine: bias has %zu columns but the weights have %zu", bc, wc);
     }
-    return gemm<T>(ctx, false, false, dr, wc, dc, data, dc, w, wc, res, wc, bias, false, (bias && bc == 1 && wc != 1) ? 0 : 1);
+    dh_status st = gemm<T>(ctx, false, false, dr, wc, dc, data, dc, w, wc, res, wc, bias, false,
+                           (bias && bc == 1 && wc != 1) ? 0 : 1, relu);
+    if (st == DH_OK && relu && !bias && dr * wc > 0) {
+        size_t grid = dh_ceil_div(dr * wc, 256);
+        if (grid > 65536)
+            grid = 65536;
+        hipLaunchKernelGGL((relu_inplace_kernel<T>), dim3(static_cast<unsigned>(grid)), dim3(256), 0, ctx->stream, res, dr * wc);
+        DH_CHECK_LAUNCH();
+    }
+    return st;
 }
 
 } // namespace dh_gemm

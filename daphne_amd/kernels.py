@@ -368,6 +368,31 @@ def conv2dForward(res, data: DenseMatrix, filter: DenseMatrix, bias, batch_size,
     return res, rh.value, rw.value
 
 
+EPILOGUE_RELU, EPILOGUE_MAXPOOL_2X2 = 1, 2  # enum dh_epilogue
+
+
+def conv2dForwardFused(res, data: DenseMatrix, filter: DenseMatrix, bias, batch_size, num_channels, img_h, img_w,
+                       filter_h, filter_w, stride_h, stride_w, pad_h, pad_w, ctx: HIPContext, relu=True, pool=False):
+    """conv2dForward with reluForward and / or maxPoolForward (2 x 2 window, stride 2, no padding) folded into the
+    store (dh_conv2d_forward_fused_*): the results of the separate kernels, bit for bit. Returns (res, res_h, res_w),
+    the extents being the pooled ones with pool=True."""
+    dt = _same_dtype(data, filter, bias, res)
+    F = filter.rows
+    P = (img_h + 2 * pad_h - filter_h) // stride_h + 1 if img_h + 2 * pad_h >= filter_h else 0
+    Q = (img_w + 2 * pad_w - filter_w) // stride_w + 1 if img_w + 2 * pad_w >= filter_w else 0
+    if pool:
+        P, Q = ((P - 2) // 2 + 1 if P >= 2 else 0), ((Q - 2) // 2 + 1 if Q >= 2 else 0)
+    if res is None:
+        res = DenseMatrix(ctx, batch_size, F * P * Q, dt)
+    rh, rw = C.c_size_t(), C.c_size_t()
+    flags = (EPILOGUE_RELU if relu else 0) | (EPILOGUE_MAXPOOL_2X2 if pool else 0)
+    capi.check(_fn("dh_conv2d_forward_fused", dt)(ctx._h, res.ptr, C.byref(rh), C.byref(rw), data.ptr, filter.ptr,
+                                                  filter.rows, filter.cols, bias.ptr if bias is not None else None,
+                                                  batch_size, num_channels, img_h, img_w, filter_h, filter_w, stride_h,
+                                                  stride_w, pad_h, pad_w, flags))
+    return res, rh.value, rw.value
+
+
 def maxPoolForward(res, data: DenseMatrix, batch_size, num_channels, img_h, img_w, pool_h, pool_w, stride_h,
                    stride_w, pad_h, pad_w, ctx: HIPContext):
     """CUDA::NN::Pooling::Forward<MAX>::apply (kernels/CUDA/Pooling.h:31-35; CPU
@@ -393,6 +418,18 @@ def affineForward(res, data: DenseMatrix, weights: DenseMatrix, bias, ctx: HIPCo
                                             weights.rows, weights.cols, bias.ptr if bias is not None else None,
                                             bias.rows if bias is not None else 0,
                                             bias.cols if bias is not None else 0))
+    return res
+
+
+def affineForwardFused(res, data: DenseMatrix, weights: DenseMatrix, bias, ctx: HIPContext, relu=True) -> DenseMatrix:
+    """affineForward followed by reluForward in one pass (dh_affine_forward_fused_*), same result bit for bit."""
+    dt = _same_dtype(data, weights, bias, res)
+    if res is None:
+        res = DenseMatrix(ctx, data.rows, weights.cols, dt)
+    capi.check(_fn("dh_affine_forward_fused", dt)(ctx._h, res.ptr, data.ptr, data.rows, data.cols, weights.ptr,
+                                                  weights.rows, weights.cols, bias.ptr if bias is not None else None,
+                                                  bias.rows if bias is not None else 0,
+                                                  bias.cols if bias is not None else 0, EPILOGUE_RELU if relu else 0))
     return res
 
 

@@ -6,8 +6,8 @@ from __future__ import annotations
 
 import numpy as np
 
-from .kernels import (AggOpCode, BinaryOpCode, DenseMatrix, HIPContext, UnaryOpCode, affineForward, aggCol, aggRow,
-                      conv2dForward, ewBinaryMat, ewBinaryObjSca, ewUnaryMat, matMul, maxPoolForward, normalEquations, softmax, solve,
+from .kernels import (AggOpCode, BinaryOpCode, DenseMatrix, HIPContext, UnaryOpCode, affineForward, affineForwardFused, aggCol,
+                      aggRow, conv2dForward, conv2dForwardFused, ewBinaryMat, ewBinaryObjSca, ewUnaryMat, matMul, maxPoolForward, normalEquations, softmax, solve,
                       syrk)
 from .pipeline import ROWREG, SELF, VectorizedPipeline
 
@@ -97,11 +97,25 @@ class KMeans:
 # ------------------------------------------------------------------------------------------------
 # config 5: LeNet-style CNN inference
 # ------------------------------------------------------------------------------------------------
-def lenet_forward(ctx: HIPContext, x: DenseMatrix, W: dict, batch: int, timer=None):
+def lenet_forward(ctx: HIPContext, x: DenseMatrix, W: dict, batch: int, timer=None, fused=True):
     """conv 5x5x32 pad 2 + bias -> ReLU -> maxpool 2x2 -> conv 5x5x64 pad 2 + bias -> ReLU -> maxpool 2x2 ->
     affine 3136->512 -> ReLU -> affine 512->10 -> softmax. W: w1 (32 x 25), b1 (32 x 1), w2 (64 x 800),
-    b2 (64 x 1), w3 (3136 x 512), b3 (1 x 512), w4 (512 x 10), b4 (1 x 10). ReLU is ewBinaryObjSca(MAX, x, 0),
-    in place. `timer(name)` is called after each layer if given."""
+    b2 (64 x 1), w3 (3136 x 512), b3 (1 x 512), w4 (512 x 10), b4 (1 x 10). fused: each layer's ReLU (and pooling)
+    in the epilogue of the kernel before it, same numbers bit for bit; else one kernel per operator, ReLU as
+    ewBinaryObjSca(MAX, x, 0) in place. `timer(name)` is called after each layer if given."""
+    t = timer or (lambda name: None)
+    if fused:
+        h, _, _ = conv2dForwardFused(None, x, W["w1"], W["b1"], batch, 1, 28, 28, 5, 5, 1, 1, 2, 2, ctx, relu=True, pool=True)
+        t("conv1+bias+relu+pool")
+        h, _, _ = conv2dForwardFused(None, h, W["w2"], W["b2"], batch, 32, 14, 14, 5, 5, 1, 1, 2, 2, ctx, relu=True, pool=True)
+        t("conv2+bias+relu+pool")
+        h = affineForwardFused(None, h, W["w3"], W["b3"], ctx)
+        t("affine1+relu")
+        h = affineForward(None, h, W["w4"], W["b4"], ctx)
+        t("affine2")
+        out = softmax(None, h, ctx)
+        t("softmax")
+        return out
     t = timer or (lambda name: None)
     h, _, _ = conv2dForward(None, x, W["w1"], W["b1"], batch, 1, 28, 28, 5, 5, 1, 1, 2, 2, ctx)
     t("conv1+bias")

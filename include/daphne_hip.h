@@ -282,6 +282,32 @@ dh_status dh_conv2d_forward_f64(dh_ctx *ctx, double *res, size_t *res_h, size_t 
                                 size_t filter_w, size_t stride_h, size_t stride_w, size_t pad_h,
                                 size_t pad_w);
 
+/* Convolution with the operators that follow it in a network folded into its epilogue, so that the
+ * activations are written once. No single kernel of the reference does this; a call replaces the
+ * kernel sequence that a script's conv2d(...), relu(...), max_pool2d(...) compile to
+ * (src/parser/daphnedsl/DaphneDSLBuiltins.cpp:883-896):
+ *   DH_EPILOGUE_RELU:         CUDA::Convolution::Forward (kernels/CUDA/Convolution.cpp:21-135), then
+ *                             CUDA::NN::Activation::Forward<ReLU> (kernels/CUDA/Activation.cpp:21-47);
+ *   DH_EPILOGUE_MAXPOOL_2X2:  then CUDA::NN::Pooling::Forward<MAX> with a 2 x 2 window, stride 2,
+ *                             no padding (kernels/CUDA/Pooling.cpp:22-65);
+ * and the result equals that of dh_conv2d_forward, dh_relu_forward and dh_maxpool_forward applied
+ * one after the other bit for bit. With pooling, res is N x (F * (P / 2) * (Q / 2)) and *res_h /
+ * *res_w receive the pooled extents; P or Q below 2 is DH_ERR_INVALID_ARG as in
+ * dh_maxpool_forward. Other arguments and errors as dh_conv2d_forward. */
+enum dh_epilogue { DH_EPILOGUE_NONE = 0, DH_EPILOGUE_RELU = 1, DH_EPILOGUE_MAXPOOL_2X2 = 2 };
+dh_status dh_conv2d_forward_fused_f32(dh_ctx *ctx, float *res, size_t *res_h, size_t *res_w,
+                                      const float *data, const float *filter, size_t filter_rows,
+                                      size_t filter_cols, const float *bias, size_t batch,
+                                      size_t channels, size_t img_h, size_t img_w, size_t filter_h,
+                                      size_t filter_w, size_t stride_h, size_t stride_w,
+                                      size_t pad_h, size_t pad_w, unsigned epilogue);
+dh_status dh_conv2d_forward_fused_f64(dh_ctx *ctx, double *res, size_t *res_h, size_t *res_w,
+                                      const double *data, const double *filter, size_t filter_rows,
+                                      size_t filter_cols, const double *bias, size_t batch,
+                                      size_t channels, size_t img_h, size_t img_w, size_t filter_h,
+                                      size_t filter_w, size_t stride_h, size_t stride_w,
+                                      size_t pad_h, size_t pad_w, unsigned epilogue);
+
 /* CUDA::NN::Pooling::Forward<MAX,...>::apply (kernels/CUDA/Pooling.h:31-35, .cpp:22-65) with
  * the CPU kernel's arithmetic (kernels/Pooling.cpp:28-107, Pooling.h:46-54,
  * MaxPoolForward.h:35-44): the result is max(0, window) because the CPU kernel folds the
@@ -307,6 +333,19 @@ dh_status dh_affine_forward_f64(dh_ctx *ctx, double *res, const double *data, si
                                 size_t data_cols, const double *weights, size_t w_rows,
                                 size_t w_cols, const double *bias, size_t bias_rows,
                                 size_t bias_cols);
+
+/* dh_affine_forward with DH_EPILOGUE_RELU folded into the store: the kernel sequence of affine(...)
+ * and relu(...) (CUDA::NN::Affine::Forward, kernels/CUDA/Affine.cpp:42-83, then
+ * CUDA::NN::Activation::Forward<ReLU>, kernels/CUDA/Activation.cpp:21-47), same result bit for bit.
+ * epilogue is DH_EPILOGUE_NONE or DH_EPILOGUE_RELU. */
+dh_status dh_affine_forward_fused_f32(dh_ctx *ctx, float *res, const float *data, size_t data_rows,
+                                      size_t data_cols, const float *weights, size_t w_rows,
+                                      size_t w_cols, const float *bias, size_t bias_rows,
+                                      size_t bias_cols, unsigned epilogue);
+dh_status dh_affine_forward_fused_f64(dh_ctx *ctx, double *res, const double *data, size_t data_rows,
+                                      size_t data_cols, const double *weights, size_t w_rows,
+                                      size_t w_cols, const double *bias, size_t bias_rows,
+                                      size_t bias_cols, unsigned epilogue);
 
 /* CUDA::BiasAdd<...>::apply (kernels/CUDA/BiasAdd.h:26-28, BiasAdd.cpp:20-55; CPU
  * kernels/BiasAdd.h:34-52): res[i, c*HW + j] = data[i, c*HW + j] + bias[c], HW = cols /

@@ -252,5 +252,8 @@ def test_config5_lenet_against_oracle_and_batch_independence(ctx):
     assert_close(got_small, exp, rtol=1e-4, elementwise=False)
     full = lenet_forward(ctx, DenseMatrix.from_numpy(ctx, x), Wd, 4096).to_numpy()
     assert full.shape == (4096, 10)
+    # one kernel per operator gives the same numbers as the layers with fused epilogues, bit for bit
+    assert_exact(lenet_forward(ctx, DenseMatrix.from_numpy(ctx, x), Wd, 4096, fused=False).to_numpy(), full)
+    assert_exact(lenet_forward(ctx, DenseMatrix.from_numpy(ctx, small), Wd, 24, fused=False).to_numpy(), got_small)
     assert_close(full[:24], got_small, rtol=1e-5, elementwise=False)  # images do not interact
     assert np.allclose(full.sum(1), 1.0, rtol=1e-5)

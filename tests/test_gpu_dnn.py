@@ -8,8 +8,8 @@ from parity import assert_close, assert_exact
 pytestmark = pytest.mark.gpu
 
 from daphne_amd import capi
-from daphne_amd.kernels import (DenseMatrix, batchNormInferenceForward, biasAdd, conv2dForward, maxPoolForward,
-                                softmax)
+from daphne_amd.kernels import (DenseMatrix, batchNormInferenceForward, biasAdd, conv2dForward, conv2dForwardFused,
+                                maxPoolForward, reluForward, softmax)
 
 DTYPES = [np.float32, np.float64]
 
@@ -71,6 +71,63 @@ def test_conv2d(ctx, dt, case):
     st, exp0, _, _ = orc.conv2d(x, w, None, N, C, H, W, Hf, Wf, sh, sw, ph, pw)
     got0, _, _ = conv2dForward(None, X, Wd, None, N, C, H, W, Hf, Wf, sh, sw, ph, pw, ctx)
     assert_close(got0.to_numpy(), exp0, elementwise=False)
+
+
+FUSED_CONV_CASES = CONV_CASES + [
+    # the layers of the LeNet configuration at a batch that leaves partial pixel blocks, odd result planes (the last
+    # row and column fall outside every 2 x 2 window), planes of a single window, many filters
+    (37, 1, 28, 28, 32, 5, 5, 1, 1, 2, 2),
+    (19, 32, 14, 14, 64, 5, 5, 1, 1, 2, 2),
+    (5, 3, 15, 13, 20, 3, 3, 1, 1, 1, 1),
+    (6, 2, 11, 11, 70, 3, 3, 1, 1, 0, 0),
+    (40, 5, 4, 4, 16, 3, 3, 1, 1, 0, 0),
+    (3, 1, 64, 64, 8, 5, 5, 1, 1, 2, 2),
+]
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("case", FUSED_CONV_CASES)
+def test_conv2d_fused_epilogues_equal_the_operator_sequence(ctx, dt, case):
+    """conv2d -> relu -> max_pool2d(2 x 2, stride 2) in one call gives the numbers of the three kernels bit for bit
+    (the fused kernel where the image fits LDS, the sequence through a temporary elsewhere), and those of the oracle."""
+    N, C, H, W, F, Hf, Wf, sh, sw, ph, pw = case
+    rng = np.random.default_rng(sum(case) + 5)
+    x = (rng.random((N, C * H * W)) - 0.3).astype(dt)
+    w = (rng.standard_normal((F, C * Hf * Wf)) * np.sqrt(2.0 / (C * Hf * Wf))).astype(dt)
+    b = (rng.standard_normal((F, 1)) * 0.1).astype(dt)
+    X, Wd, B = DenseMatrix.from_numpy(ctx, x), DenseMatrix.from_numpy(ctx, w), DenseMatrix.from_numpy(ctx, b)
+    conv, P, Q = conv2dForward(None, X, Wd, B, N, C, H, W, Hf, Wf, sh, sw, ph, pw, ctx)
+    relu = reluForward(None, conv, ctx)
+    got, gh, gw = conv2dForwardFused(None, X, Wd, B, N, C, H, W, Hf, Wf, sh, sw, ph, pw, ctx, relu=True, pool=False)
+    assert (gh, gw) == (P, Q)
+    assert_exact(got.to_numpy(), relu.to_numpy())
+    assert (relu.to_numpy() == 0).any() and (relu.to_numpy() > 0).any()
+    got0, _, _ = conv2dForwardFused(None, X, Wd, None, N, C, H, W, Hf, Wf, sh, sw, ph, pw, ctx, relu=True, pool=False)
+    conv0, _, _ = conv2dForward(None, X, Wd, None, N, C, H, W, Hf, Wf, sh, sw, ph, pw, ctx)
+    assert_exact(got0.to_numpy(), reluForward(None, conv0, ctx).to_numpy())
+    if P < 2 or Q < 2:
+        with pytest.raises(capi.DaphneHipError, match="window 2x2 does not fit"):
+            conv2dForwardFused(None, X, Wd, B, N, C, H, W, Hf, Wf, sh, sw, ph, pw, ctx, relu=True, pool=True)
+        return
+    for with_relu, before_pool in ((True, relu), (False, conv)):
+        pooled, ph_, pw_ = maxPoolForward(None, before_pool, N, F, P, Q, 2, 2, 2, 2, 0, 0, ctx)
+        got, gh, gw = conv2dForwardFused(None, X, Wd, B, N, C, H, W, Hf, Wf, sh, sw, ph, pw, ctx, relu=with_relu, pool=True)
+        assert (gh, gw) == (ph_, pw_) == (P // 2, Q // 2)
+        assert_exact(got.to_numpy(), pooled.to_numpy())
+    st, oc, _, _ = orc.conv2d(x, w, b, N, C, H, W, Hf, Wf, sh, sw, ph, pw)
+    st, orl = orc.ew_binary_sca(14, oc, 0.0)
+    st, op, _, _ = orc.maxpool(orl, N, F, P, Q, 2, 2, 2, 2, 0, 0)
+    assert_close(got.to_numpy(), op, elementwise=False)
+
+
+def test_conv2d_fused_rejects_unknown_flags(ctx):
+    x, w = DenseMatrix.from_numpy(ctx, np.ones((1, 16), np.float32)), DenseMatrix.from_numpy(ctx, np.ones((1, 4), np.float32))
+    res = DenseMatrix(ctx, 1, 9, np.float32)
+    import ctypes as C
+    rh, rw = C.c_size_t(), C.c_size_t()
+    st = capi.lib().dh_conv2d_forward_fused_f32(ctx._h, res.ptr, C.byref(rh), C.byref(rw), x.ptr, w.ptr, 1, 4, None, 1, 1, 4, 4, 2, 2,
+                                                1, 1, 0, 0, 8)
+    assert st != 0 and b"unknown epilogue" in capi.lib().dh_last_error()
 
 
 @pytest.mark.parametrize("dt", DTYPES)

@@ -14,7 +14,7 @@ from parity import assert_close, assert_exact
 pytestmark = pytest.mark.gpu
 
 from daphne_amd import capi
-from daphne_amd.kernels import DenseMatrix, affineForward, matMul, solve, syrk
+from daphne_amd.kernels import DenseMatrix, affineForward, affineForwardFused, matMul, reluForward, solve, syrk
 
 DTYPES = [np.float32, np.float64]
 
@@ -241,6 +241,23 @@ def test_affine(ctx, dt, m, k, n):
     assert_close(got, exp, elementwise=False)
     got = affineForward(None, DenseMatrix.from_numpy(ctx, x), DenseMatrix.from_numpy(ctx, w), None, ctx).to_numpy()
     assert_close(got, mm, elementwise=False)
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("m,k,n", [(1, 9, 2), (64, 100, 10), (300, 3136, 512), (257, 512, 10), (4096, 3136, 512), (700, 64, 130),
+                                   (2304, 256, 1280)])
+def test_affine_with_relu_equals_affine_then_relu(ctx, dt, m, k, n):
+    """The rectifier in the epilogue (direct store, split-K reduction, leftover tiles, no bias) against the two kernels."""
+    rng = np.random.default_rng(m + k + n + 1)
+    x = DenseMatrix.from_numpy(ctx, (rng.random((m, k)) - 0.5).astype(dt))
+    w = DenseMatrix.from_numpy(ctx, (rng.standard_normal((k, n)) * np.sqrt(2.0 / k)).astype(dt))
+    for bias in (DenseMatrix.from_numpy(ctx, (rng.standard_normal((1, n)) * 0.1).astype(dt)),
+                 DenseMatrix.from_numpy(ctx, np.full((1, 1), 0.05, dt)), None):
+        exp = reluForward(None, affineForward(None, x, w, bias, ctx), ctx).to_numpy()
+        got = affineForwardFused(None, x, w, bias, ctx).to_numpy()
+        assert_exact(got, exp)
+        assert m * n < 100 or ((exp == 0).any() and (exp > 0).any())
+        assert_exact(affineForwardFused(None, x, w, bias, ctx, relu=False).to_numpy(), affineForward(None, x, w, bias, ctx).to_numpy())
 
 
 @pytest.mark.parametrize("dt", DTYPES)
