@@ -110,7 +110,7 @@ def run(args) -> int:
     import torch
 
     sys.path.insert(0, os.path.join(os.path.dirname(os.path.abspath(__file__)), "tests"))
-    from daphne_amd.kernels import DenseMatrix, HIPContext, matMul, normalEquations, solve, syrk
+    from daphne_amd.kernels import DenseMatrix, HIPContext, kmeansAssign, kmeansUpdate, matMul, normalEquations, solve, syrk
     from daphne_amd.workloads import KMeans, lenet_forward, lmds
 
     if not torch.cuda.is_available():
@@ -162,12 +162,20 @@ def run(args) -> int:
         X = DenseMatrix.from_torch(ctx, Xt)
         km = KMeans(ctx, X, k)
         C0 = Xt[torch.arange(k, device="cuda") * 125000].contiguous()
-        state = {"C": DenseMatrix.from_torch(ctx, C0)}
+        # two centroid buffers used in turn: a fresh result matrix per iteration would put an allocation and a
+        # (synchronising) release between the kernels
+        state = {"C": DenseMatrix.from_torch(ctx, C0), "next": 0}
+        bufs = [DenseMatrix(ctx, k, f, np.float32), DenseMatrix(ctx, k, f, np.float32)]
 
-        def step():  # one Lloyd iteration
-            state["C"] = km.iterate(state["C"])
+        def step(fused=True):  # one Lloyd iteration
+            out = bufs[state["next"]]
+            state["next"] ^= 1
+            state["C"] = km.iterate(state["C"], out, fused=fused)
 
         ms = _timed(torch, step, args.steps, args.warmup)
+        ms_seq = _timed(torch, lambda: step(False), min(args.steps, 15), args.warmup)
+        t_assign = _events(torch, lambda: kmeansAssign(km.idx, X, state["C"], km.xx, km.cc, ctx))
+        t_update = _events(torch, lambda: kmeansUpdate(bufs[state["next"]], X, km.idx, k, ctx, km.counts))
         # canonical bytes per iteration: X C^T (read X, write D), D assembly 3 x |D|, idxmin (read D, write idx),
         # one-hot P, P^T X (read P and X), colSums(P)
         D = n * k * 4
@@ -190,12 +198,18 @@ def run(args) -> int:
             dt = time.perf_counter() - t0
             cpu = {"value": round(nbytes * (ns / n) / dt / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
                    "sample": f"one iteration on the first {ns} of {n} rows, single thread ({dt:.2f} s)"}
-        roof = {"bound": "hbm", "kernel": "ts_nt_kernel<float,1> (X t(C))",
-                "achieved": round((n * f * 4 + D) / t_gemm / 1e6, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round((n * f * 4 + D) / t_gemm / 1e6 / HBM_PEAK_GBS, 4), "traffic": None}
+        assign_bytes = n * f * 4 + n * 4 + n * 8  # X, xx, idx
+        fused_bytes = assign_bytes + n * f * 4 + n * 8  # and X, idx once more
+        roof = {"bound": "hbm", "kernel": "ts_nt_kernel<float,1,true,4> (assignment: X t(C), distances and row arg-min in one pass over X)",
+                "achieved": round(assign_bytes / t_assign / 1e6, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(assign_bytes / t_assign / 1e6 / HBM_PEAK_GBS, 4), "traffic": None}
         out = _line(nbytes / ms / 1e6, "GB/s", ms, args, "f32",
-                    "k-means Lloyd iteration: X 2000000x64 f32 (16 Gaussians), C 16x64; step = one iteration",
-                    roof, cpu, {"canonical_bytes_per_step": nbytes, "xct_ms": round(t_gemm, 4)})
+                    "k-means Lloyd iteration: X 2000000x64 f32 (16 Gaussians), C 16x64; step = one iteration "
+                    "(two passes over X: assignment, update)",
+                    roof, cpu, {"canonical_bytes_per_step": nbytes, "bytes_per_step_two_passes": fused_bytes,
+                                "two_pass_gbs": round(fused_bytes / ms / 1e6, 1), "assign_ms": round(t_assign, 4),
+                                "update_ms": round(t_update, 4), "xct_ms": round(t_gemm, 4),
+                                "ms_per_step_operator_sequence": round(ms_seq, 4)})
     elif args.config == 4:
         res = measure_contractions(torch, ctx, args.steps, args.warmup)
         cpu = None

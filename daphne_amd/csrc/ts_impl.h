@@ -23,6 +23,9 @@
 #include "common.h"
 
 namespace dh_gemm {
+#ifndef TS_NT_RBW
+#define TS_NT_RBW 8 // 16-row blocks per wave of ts_nt_kernel
+#endif
 #ifndef TS_SYM_U
 #define TS_SYM_U 4 // quads per register set of the symmetric one-wave form (measured: 2 1.00 ms, 4 0.90, 8 0.92, 12 0.95)
 #endif
@@ -360,14 +363,21 @@ struct TsNtArgs {
     unsigned n, K;
     unsigned kpad;   // K rounded up to whole chunks
     int vec_store;   // C rows are 16-byte aligned
+    // ASSIGN: instead of C, the first position of the row minimum of (C * -2 + row_add[row]) + col_add[col]
+    const void *row_add, *col_add;
+    unsigned long long *idx;
 };
 
-// NB column blocks of 16; each wave walks over row blocks of 16, two at a time.
-template <typename T, int NB> __global__ __launch_bounds__(256) void ts_nt_kernel(TsNtArgs g) {
+// NB column blocks of 16; each wave walks over row blocks of 16, two at a time, CPG chunks of k at a time (1, 2 or 4:
+// a count that divides the number of chunks, so that a step's body has no branch in it).
+// ASSIGN: the product is not stored; it goes on, rounded exactly as the stored one would be, into the distance
+// (C * -2 + row_add[row]) + col_add[col] (three separately rounded operations) and the row's IDXMIN over it: the first
+// position of the strict minimum, NaN never better, position 0 if the first value is NaN or all are.
+template <typename T, int NB, bool ASSIGN, int CPG> __global__ __launch_bounds__(256) void ts_nt_kernel(TsNtArgs g) {
     using M = Mfma16<T>;
     constexpr int V = 16 / sizeof(T);
     constexpr int KC = 4 * V;     // k values per chunk
-    constexpr int RBW = 8;        // row blocks per wave
+    constexpr int RBW = TS_NT_RBW; // row blocks per wave
     // float: the operands of the matrix instruction are exchanged, which transposes the result tile in the
     // registers (row = 4 * (lane / 16) + v becomes the column) and turns four 4-byte stores per lane into one of
     // 16 bytes; the double layout (row = 4 * v + lane / 16) already stores whole 128-byte rows
@@ -380,6 +390,18 @@ template <typename T, int NB> __global__ __launch_bounds__(256) void ts_nt_kerne
     const T *B = static_cast<const T *>(g.B);
     T *C = static_cast<T *>(g.C);
     const unsigned ldl = g.kpad + V;
+    // ASSIGN: this lane's columns' addends (float: columns 16 b + 4 h + v; double: column 16 b + i)
+    constexpr int CPL = SWAP ? 4 : 1;
+    T col_add[NB][CPL];
+    if constexpr (ASSIGN) {
+#pragma unroll
+        for (int b = 0; b < NB; b++)
+#pragma unroll
+            for (int v = 0; v < CPL; v++) {
+                const unsigned col = SWAP ? b * 16 + 4 * h + v : b * 16 + i;
+                col_add[b][v] = col < g.n ? static_cast<const T *>(g.col_add)[col] : dh_inf<T>(); // beyond n: never the minimum
+            }
+    }
 
     // The work of a wavefront is a sequence of steps (pair of 16-row blocks, group of four k chunks), walked with two
     // register sets: the eight vector loads of step s + 1 are in flight while the matrix cores work on step s, and
@@ -388,22 +410,49 @@ template <typename T, int NB> __global__ __launch_bounds__(256) void ts_nt_kerne
     // its first use): rows beyond M read the last row - they only produce rows of C that are not stored -, k
     // beyond K reads k = 0 and is zeroed when it is used (the padded part of B is zero, but 0 * NaN would still
     // be NaN), and steps beyond the last repeat the last one.
-    const size_t row0 = (static_cast<size_t>(blockIdx.x) * 4 + wave) * (16 * RBW);
     const unsigned chunks = g.kpad / KC;
-    const unsigned cg = (chunks + 3) / 4;            // chunk groups per row-block pair
+    const unsigned cg = chunks / CPG;                // chunk groups per row-block pair (CPG divides chunks)
     const unsigned nsteps = (RBW / 2) * cg;          // even
+    constexpr int RPL = SWAP ? 1 : 4; // ASSIGN: rows per lane and row block in the result layout
     struct Frag {
-        T a[2][4][V];
+        T a[2][CPG][V];
+        T ra[2][RPL]; // ASSIGN: the row addends, fetched with the step so that the epilogue waits for nothing new
     };
+    // A step's part of X - 32 rows by CPG chunks - is loaded the way memory likes it, whole runs of consecutive
+    // vectors (vector number 64 c + lane of load c, counted along the rows of the 16 x VPR block), and turned into
+    // the fragment layout (lane (i, h): row i, vector h of chunk c) through a piece of LDS that belongs to the wave:
+    // no barrier, the wave's own LDS instructions execute in order. Row stride SX = CPG KC + V: free of bank conflicts.
+    constexpr unsigned VPR = CPG * 4;      // vectors of a row in one step
+    constexpr unsigned SX = CPG * KC + V;
+    T *stage = lb + NB * 16 * ldl + wave * (16 * SX); // one row block at a time
+    // Addresses are a base that is the same for the whole wave plus a 32-bit byte offset per lane (the wave's rows span
+    // at most 16 RBW rows of at most 2^24 bytes): one 24-bit multiplication and an addition per load, rows beyond M
+    // cut back to the last row by a minimum on the row number.
+    const size_t row0 = (static_cast<size_t>(blockIdx.x) * 4 + wave) * (16 * RBW);
+    const size_t row0_ok = row0 < g.M ? row0 : g.M - 1;
+    const char *wave_base = reinterpret_cast<const char *>(A + row0_ok * g.lda);
+    const unsigned last_local = static_cast<unsigned>(g.M - 1 - row0_ok < 16 * RBW ? g.M - 1 - row0_ok : 16 * RBW - 1);
+    const unsigned row_bytes = static_cast<unsigned>(g.lda * sizeof(T));
     auto load_step = [&](Frag &fr, unsigned pair, unsigned grp) {
-        const size_t r0 = row0 + static_cast<size_t>(pair) * 32 + i, r1 = r0 + 16;
-        const T *a0 = A + (r0 < g.M ? r0 : g.M - 1) * g.lda, *a1 = A + (r1 < g.M ? r1 : g.M - 1) * g.lda;
 #pragma unroll
-        for (int c = 0; c < 4; c++) {
-            const unsigned kv = (grp * 4 + c) * KC + h * V;
-            const unsigned kl = kv < g.K ? kv : 0;
-            ts_load<T, V>(a0 + kl, fr.a[0][c], true);
-            ts_load<T, V>(a1 + kl, fr.a[1][c], true);
+        for (int c = 0; c < CPG; c++) {
+            const unsigned id = c * 64 + lane;
+            const unsigned kv = grp * CPG * KC + (id % VPR) * V;
+            const unsigned kb = (kv < g.K ? kv : 0) * static_cast<unsigned>(sizeof(T));
+            const unsigned r0 = pair * 32 + id / VPR, r1 = r0 + 16;
+            const unsigned l0 = r0 < last_local ? r0 : last_local, l1 = r1 < last_local ? r1 : last_local;
+            ts_load<T, V>(reinterpret_cast<const T *>(wave_base + (__umul24(l0, row_bytes) + kb)), fr.a[0][c], true);
+            ts_load<T, V>(reinterpret_cast<const T *>(wave_base + (__umul24(l1, row_bytes) + kb)), fr.a[1][c], true);
+        }
+        if constexpr (ASSIGN) {
+            const T *ra_base = static_cast<const T *>(g.row_add) + row0_ok;
+#pragma unroll
+            for (int t = 0; t < 2; t++)
+#pragma unroll
+                for (int v = 0; v < RPL; v++) {
+                    const unsigned r = pair * 32 + t * 16 + (SWAP ? i : M::row(lane, v));
+                    fr.ra[t][v] = ra_base[r < last_local ? r : last_local];
+                }
         }
     };
     typename M::acc_t acc[2][NB];
@@ -415,10 +464,22 @@ template <typename T, int NB> __global__ __launch_bounds__(256) void ts_nt_kerne
                 acc[1][b] = typename M::acc_t{0, 0, 0, 0};
             }
         }
+        T xa[2][CPG][V];
 #pragma unroll
-        for (int c = 0; c < 4; c++) {
-            const unsigned ch = grp * 4 + c;
-            if (ch < chunks) {
+        for (int t = 0; t < 2; t++) {
+#pragma unroll
+            for (int c = 0; c < CPG; c++) {
+                const unsigned id = c * 64 + lane;
+                dh_store_vec<T, V>(stage + (id / VPR) * SX + (id % VPR) * V, fr.a[t][c]);
+            }
+#pragma unroll
+            for (int c = 0; c < CPG; c++)
+                dh_load_vec<T, V>(stage + i * SX + c * KC + h * V, xa[t][c]);
+        }
+#pragma unroll
+        for (int c = 0; c < CPG; c++) {
+            const unsigned ch = grp * CPG + c;
+            {
                 const bool kok = ch * KC + h * V < g.K;
 #pragma unroll
                 for (int b = 0; b < NB; b++) {
@@ -426,7 +487,7 @@ template <typename T, int NB> __global__ __launch_bounds__(256) void ts_nt_kerne
                     dh_load_vec<T, V>(lb + (b * 16 + i) * ldl + ch * KC + h * V, fb);
 #pragma unroll
                     for (int e = 0; e < V; e++) {
-                        const T x0 = kok ? fr.a[0][c][e] : T(0), x1 = kok ? fr.a[1][c][e] : T(0);
+                        const T x0 = kok ? xa[0][c][e] : T(0), x1 = kok ? xa[1][c][e] : T(0);
                         if constexpr (SWAP) {
                             acc[0][b] = M::mma(fb[e], x0, acc[0][b]);
                             acc[1][b] = M::mma(fb[e], x1, acc[1][b]);
@@ -441,7 +502,109 @@ template <typename T, int NB> __global__ __launch_bounds__(256) void ts_nt_kerne
         if (grp + 1 != cg)
             return;
         const size_t rbase = row0 + static_cast<size_t>(pair) * 32;
-        if constexpr (SWAP) {
+        if constexpr (ASSIGN) {
+#pragma clang fp contract(off)
+            constexpr unsigned NONE = ~0u;
+            auto take = [](T &best, unsigned &bi, T ov, unsigned oi) {
+                if (ov < best || (ov == best && oi < bi)) {
+                    best = ov;
+                    bi = oi;
+                }
+            };
+            if constexpr (SWAP) {
+                // register v of lane (i, h) is C[row i][column 16 b + 4 h + v]: a row's values sit in the four lanes i + 16 h
+                T d[2][NB][4];
+#pragma unroll
+                for (int t = 0; t < 2; t++)
+#pragma unroll
+                    for (int b = 0; b < NB; b++)
+#pragma unroll
+                        for (int v = 0; v < 4; v++)
+                            d[t][b][v] = (acc[t][b][v] * T(-2) + fr.ra[t][0]) + col_add[b][v];
+                // The short way: a plain running minimum. It gives IDXMIN's answer unless a NaN is among the values or
+                // nothing lies below +inf; the sum of a lane's values tells the first (opposite infinities only send
+                // the wave the long way for nothing), the minimum itself the second.
+                T best[2], sum[2];
+                unsigned bi[2];
+                bool odd = false;
+#pragma unroll
+                for (int t = 0; t < 2; t++) {
+                    best[t] = sum[t] = d[t][0][0];
+                    bi[t] = 4 * h;
+#pragma unroll
+                    for (int b = 0; b < NB; b++)
+#pragma unroll
+                        for (int v = 0; v < 4; v++) {
+                            if (b == 0 && v == 0)
+                                continue;
+                            const bool lt = d[t][b][v] < best[t];
+                            best[t] = lt ? d[t][b][v] : best[t];
+                            bi[t] = lt ? static_cast<unsigned>(b * 16 + 4 * h + v) : bi[t];
+                            sum[t] += d[t][b][v];
+                        }
+                    take(best[t], bi[t], dh_peer_swap<16>{}(best[t]), dh_peer_swap<16>{}(bi[t]));
+                    take(best[t], bi[t], dh_peer_swap<32>{}(best[t]), dh_peer_swap<32>{}(bi[t]));
+                    odd |= (sum[t] != sum[t]) || !(best[t] < dh_inf<T>());
+                }
+                if (__ballot(odd) == 0) {
+#pragma unroll
+                    for (int t = 0; t < 2; t++) {
+                        const size_t row = rbase + static_cast<size_t>(t) * 16 + i;
+                        if (h == 0 && row < g.M)
+                            g.idx[row] = bi[t];
+                    }
+                    return;
+                }
+#pragma unroll
+                for (int t = 0; t < 2; t++) {
+                    const size_t row = rbase + static_cast<size_t>(t) * 16 + i;
+                    T best1 = dh_inf<T>(), first = T(0);
+                    unsigned bi1 = NONE;
+#pragma unroll
+                    for (int b = 0; b < NB; b++)
+#pragma unroll
+                        for (int v = 0; v < 4; v++) {
+                            const unsigned col = b * 16 + 4 * h + v;
+                            const T dv = d[t][b][v];
+                            if (b == 0 && v == 0)
+                                first = dv; // column 0 in the lanes h = 0
+                            if (col < g.n && (dv < best1 || (bi1 == NONE && !(dv != dv)))) {
+                                best1 = dv;
+                                bi1 = col;
+                            }
+                        }
+                    take(best1, bi1, dh_peer_swap<16>{}(best1), dh_peer_swap<16>{}(bi1));
+                    take(best1, bi1, dh_peer_swap<32>{}(best1), dh_peer_swap<32>{}(bi1));
+                    if (h == 0 && row < g.M)
+                        g.idx[row] = ((first != first) || bi1 == NONE) ? 0ull : static_cast<unsigned long long>(bi1);
+                }
+            } else {
+                // register v of lane (i, h) is C[row 4 v + h][column 16 b + i]: a row's values sit in the sixteen lanes of a group
+#pragma unroll
+                for (int t = 0; t < 2; t++)
+#pragma unroll
+                    for (int v = 0; v < 4; v++) {
+                        const size_t row = rbase + static_cast<size_t>(t) * 16 + M::row(lane, v);
+                        const T ra = fr.ra[t][SWAP ? 0 : v];
+                        T best = dh_inf<T>(), first = T(0);
+                        unsigned bi = NONE;
+#pragma unroll
+                        for (int b = 0; b < NB; b++) {
+                            const unsigned col = b * 16 + i;
+                            const T d = (acc[t][b][v] * T(-2) + ra) + col_add[b][0];
+                            if (b == 0)
+                                first = d; // column 0 in the lanes i = 0
+                            if (col < g.n && (d < best || (bi == NONE && !(d != d)))) {
+                                best = d;
+                                bi = col;
+                            }
+                        }
+                        dh_butterfly(16, [&](auto peer) { take(best, bi, peer(best), peer(bi)); });
+                        if (i == 0 && row < g.M)
+                            g.idx[row] = ((first != first) || bi == NONE) ? 0ull : static_cast<unsigned long long>(bi);
+                    }
+            }
+        } else if constexpr (SWAP) {
             // the tile was computed transposed: register v of lane (i, h) is C[row i][column 4h + v], so a lane
             // stores four neighbouring columns at once and a wavefront 16 whole rows
 #pragma unroll
@@ -624,11 +787,39 @@ bool ts_tn(dh_ctx *ctx, size_t m, size_t n, size_t K, const T *A, size_t lda, co
     return true;
 }
 
+// Dynamic LDS of ts_nt_kernel: B (nb blocks of 16 rows, kpad + V a row) and a staging piece per wave.
+template <typename T> inline size_t ts_nt_lds_bytes(int nb, unsigned kpad, int cpg) {
+    constexpr size_t V = 16 / sizeof(T), KC = 4 * V;
+    return (static_cast<size_t>(nb) * 16 * (kpad + V) + 4 * 16 * (cpg * KC + V)) * sizeof(T);
+}
+// chunks of k per step: the largest of 4, 2, 1 that divides their number
+template <typename T> inline int ts_nt_chunks_per_step(unsigned kpad) {
+    const unsigned chunks = kpad / (4 * (16 / sizeof(T)));
+    return chunks % 4 == 0 ? 4 : (chunks % 2 == 0 ? 2 : 1);
+}
+
+template <typename T, int NB, bool ASSIGN, int CPG>
+inline dh_status ts_nt_launch_cpg(dh_ctx *ctx, const TsNtArgs &g, size_t blocks, size_t lds) {
+    // dynamic LDS beyond 64 KiB has to be asked for, per kernel and device (the call is cheap next to the kernel)
+    if (lds > 65536)
+        DH_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&ts_nt_kernel<T, NB, ASSIGN, CPG>),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
+    hipLaunchKernelGGL((ts_nt_kernel<T, NB, ASSIGN, CPG>), dim3(static_cast<unsigned>(blocks)), dim3(256), lds, ctx->stream, g);
+    return DH_OK;
+}
+template <typename T, int NB, bool ASSIGN> inline dh_status ts_nt_launch(dh_ctx *ctx, const TsNtArgs &g, size_t blocks) {
+    const int cpg = ts_nt_chunks_per_step<T>(g.kpad);
+    const size_t lds = ts_nt_lds_bytes<T>(NB, g.kpad, cpg);
+    return cpg == 4 ? ts_nt_launch_cpg<T, NB, ASSIGN, 4>(ctx, g, blocks, lds)
+                    : (cpg == 2 ? ts_nt_launch_cpg<T, NB, ASSIGN, 2>(ctx, g, blocks, lds)
+                                : ts_nt_launch_cpg<T, NB, ASSIGN, 1>(ctx, g, blocks, lds));
+}
+
 template <typename T>
 bool ts_nt(dh_ctx *ctx, size_t M, size_t n, size_t K, const T *A, size_t lda, const T *B, size_t ldb, T *C, size_t ldc,
            dh_status *status) {
     constexpr int V = 16 / sizeof(T), KC = 4 * V;
-    if (n == 0 || n > 32 || K == 0 || K > 512 || M < 65536)
+    if (n == 0 || n > 32 || K == 0 || K > 512 || M < 65536 || lda * sizeof(T) >= (size_t(1) << 24))
         return false;
     if (!dh_aligned(A, 16) || !dh_aligned(B, 16) || lda % V || ldb % V || K % V)
         return false;
@@ -645,15 +836,10 @@ bool ts_nt(dh_ctx *ctx, size_t M, size_t n, size_t K, const T *A, size_t lda, co
     g.K = static_cast<unsigned>(K);
     g.kpad = static_cast<unsigned>(dh_ceil_div(K, KC) * KC);
     g.vec_store = dh_aligned(C, 16) && (ldc * sizeof(T)) % 16 == 0;
-    const size_t lds = static_cast<size_t>(nb) * 16 * (g.kpad + V) * sizeof(T);
-    const size_t blocks = dh_ceil_div(M, 4 * 16 * 8);
-    if (blocks >= (size_t(1) << 31) || lds > (size_t(48) << 10))
+    const size_t blocks = dh_ceil_div(M, 4 * 16 * TS_NT_RBW);
+    if (blocks >= (size_t(1) << 31) || static_cast<size_t>(nb) * 16 * (g.kpad + V) * sizeof(T) > (size_t(48) << 10))
         return false;
-    if (nb == 1)
-        hipLaunchKernelGGL((ts_nt_kernel<T, 1>), dim3(static_cast<unsigned>(blocks)), dim3(256), lds, ctx->stream, g);
-    else
-        hipLaunchKernelGGL((ts_nt_kernel<T, 2>), dim3(static_cast<unsigned>(blocks)), dim3(256), lds, ctx->stream, g);
-    *status = DH_OK;
+    *status = nb == 1 ? ts_nt_launch<T, 1, false>(ctx, g, blocks) : ts_nt_launch<T, 2, false>(ctx, g, blocks);
     return true;
 }
 

@@ -330,6 +330,34 @@ def normalEquations(X: DenseMatrix, y: DenseMatrix, lam: float, ctx: HIPContext,
     return A, b
 
 
+def kmeansAssign(idx, X: DenseMatrix, C: DenseMatrix, xx: DenseMatrix, cc: DenseMatrix, ctx: HIPContext) -> DenseMatrix:
+    """idx = idxminRow((X @ t(C)) * -2 + xx + t(cc)) in one pass over X (dh_kmeans_assign_*): the operator sequence
+    MatMul, EwBinaryObjSca MUL, EwBinaryMat ADD twice, AggRow IDXMIN of test/api/cli/algorithms/kmeans.daphne:14-16.
+    xx holds one value per row of X, cc one per row of C; idx is rows x 1, uint64."""
+    dt = _same_dtype(X, C, xx, cc)
+    if C.cols != X.cols or xx.getNumItems() != X.rows or cc.getNumItems() != C.rows:
+        raise capi.DaphneHipError(1, "kmeansAssign: C must have X's columns, xx one value per row of X, cc one per centroid")
+    if idx is None:
+        idx = DenseMatrix(ctx, X.rows, 1, np.uint64)
+    capi.check(_fn("dh_kmeans_assign", dt)(ctx._h, idx.ptr, X.ptr, X.rows, X.cols, X.row_skip, C.ptr, C.rows, C.row_skip, xx.ptr,
+                                           cc.ptr))
+    return idx
+
+
+def kmeansUpdate(C_new, X: DenseMatrix, idx: DenseMatrix, k: int, ctx: HIPContext, counts: Optional[DenseMatrix] = None):
+    """C_new = (t(P) @ X) / t(colSums(P)) for P = one-hot(idx), in one pass over X (dh_kmeans_update_*): the comparison,
+    MatMul, AggCol SUM and EwBinaryMat DIV of test/api/cli/algorithms/kmeans.daphne:17-21. Returns (C_new, counts)."""
+    dt = X.dtype
+    if idx.getNumItems() != X.rows:
+        raise capi.DaphneHipError(1, "kmeansUpdate: idx must hold one value per row of X")
+    if C_new is None:
+        C_new = DenseMatrix(ctx, k, X.cols, dt)
+    if counts is None:
+        counts = DenseMatrix(ctx, 1, k, dt)
+    capi.check(_fn("dh_kmeans_update", dt)(ctx._h, C_new.ptr, C_new.row_skip, counts.ptr, X.ptr, X.rows, X.cols, X.row_skip, idx.ptr, k))
+    return C_new, counts
+
+
 def solve(res, lhs: DenseMatrix, rhs: DenseMatrix, ctx: HIPContext) -> DenseMatrix:
     """CUDA::solve (kernels/CUDA/Solve.h; CPU kernels/Solve.h:86-116): A x = b by LU."""
     dt = _same_dtype(lhs, rhs, res)

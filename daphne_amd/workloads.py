@@ -7,7 +7,7 @@ from __future__ import annotations
 import numpy as np
 
 from .kernels import (AggOpCode, BinaryOpCode, DenseMatrix, HIPContext, UnaryOpCode, affineForward, affineForwardFused, aggCol,
-                      aggRow, conv2dForward, conv2dForwardFused, ewBinaryMat, ewBinaryObjSca, ewUnaryMat, matMul, maxPoolForward, normalEquations, softmax, solve,
+                      aggRow, conv2dForward, conv2dForwardFused, kmeansAssign, kmeansUpdate, ewBinaryMat, ewBinaryObjSca, ewUnaryMat, matMul, maxPoolForward, normalEquations, softmax, solve,
                       syrk)
 from .pipeline import ROWREG, SELF, VectorizedPipeline
 
@@ -70,13 +70,18 @@ class KMeans:
         self.PtX = DenseMatrix(ctx, k, X.cols, dt)
         self.counts = DenseMatrix(ctx, 1, k, dt)
 
-    def iterate(self, C: DenseMatrix, C_out: DenseMatrix | None = None) -> DenseMatrix:
+    def iterate(self, C: DenseMatrix, C_out: DenseMatrix | None = None, fused: bool = True) -> DenseMatrix:
+        """fused: two passes over X (kmeansAssign, kmeansUpdate); else one kernel per operator (or fused pipeline of
+        elementwise operators), with XC, the one-hot P and t(P) X in memory. self.idx holds the assignment either way."""
         ctx, X, k = self.ctx, self.X, self.k
-        matMul(self.XC, X, C, False, True, ctx)                       # X @ t(C)
         pc = VectorizedPipeline(ctx, C)
         pc.ewBinary(BinaryOpCode.MUL, SELF).rowAgg(AggOpCode.SUM)
         pc.storeRow(self.cc)
         pc.run()                                                       # rowSums(C^2), k x 1
+        if fused:
+            kmeansAssign(self.idx, X, C, self.xx, self.cc, ctx)
+            return kmeansUpdate(C_out, X, self.idx, k, ctx, self.counts)[0]
+        matMul(self.XC, X, C, False, True, ctx)                       # X @ t(C)
         cc_row = DenseMatrix(ctx, 1, k, C.dtype, ptr=self.cc.ptr, keepalive=self.cc)  # the same k values as 1 x k
         p = VectorizedPipeline(ctx, self.XC)
         p.ewBinary(BinaryOpCode.MUL, -2.0).ewBinary(BinaryOpCode.ADD, self.xx).ewBinary(BinaryOpCode.ADD, cc_row)

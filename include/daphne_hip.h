@@ -260,6 +260,34 @@ dh_status dh_syrk_f64(dh_ctx *ctx, double *res, size_t ld_res, const double *arg
 dh_status dh_solve_f32(dh_ctx *ctx, float *x, const float *A, size_t n, size_t lda, const float *b);
 dh_status dh_solve_f64(dh_ctx *ctx, double *x, const double *A, size_t n, size_t lda, const double *b);
 
+/* One Lloyd iteration of k-means in two passes over X, without the rows x k matrices (distances, one-hot
+ * membership) that the operator sequence of the script writes and reads back
+ * (test/api/cli/algorithms/kmeans.daphne:14-21 with the row arg-min as membership). No single kernel of
+ * the reference does this; the calls replace
+ *   assign:  MatMul X @ t(C) (kernels/CUDA/MatMul.cpp), EwBinaryObjSca MUL -2, EwBinaryMat ADD of the column
+ *            xx (rows x 1) and of the row cc (1 x k) (kernels/CUDA/EwBinaryMat.cpp:95-155), AggRow IDXMIN
+ *            (kernels/AggRow.h:71-94): idx[i] = first position of the minimum of
+ *            ((X t(C))[i][c] * -2 + xx[i]) + cc[c]. The distances are rounded as in that sequence, so idx
+ *            equals its result wherever dh_matmul takes its streaming kernel for X t(C) (65536 rows or
+ *            more); elsewhere the product's last bits, and with them near-ties, may differ.
+ *   update:  the one-hot comparison, MatMul t(P) @ X, AggCol SUM, EwBinaryMat DIV:
+ *            C_new[c][:] = (sum of the rows with idx = c) / (their number); counts (k values, may be
+ *            NULL) receives the numbers. An empty cluster comes out as 0 / 0.
+ * X is rows x cols with leading dimension ldx, C is k x cols (ldc), idx holds rows values. Limits
+ * (DH_ERR_INVALID_ARG beyond them): k <= 32; cols <= 512 for assign and <= 256 (float) / 128 (double)
+ * for update; rows of X and C 16-byte aligned and a whole number of 16-byte vectors long. */
+dh_status dh_kmeans_assign_f32(dh_ctx *ctx, uint64_t *idx, const float *X, size_t rows, size_t cols,
+                               size_t ldx, const float *C, size_t k, size_t ldc, const float *xx,
+                               const float *cc);
+dh_status dh_kmeans_assign_f64(dh_ctx *ctx, uint64_t *idx, const double *X, size_t rows, size_t cols,
+                               size_t ldx, const double *C, size_t k, size_t ldc, const double *xx,
+                               const double *cc);
+dh_status dh_kmeans_update_f32(dh_ctx *ctx, float *C_new, size_t ld_new, float *counts, const float *X,
+                               size_t rows, size_t cols, size_t ldx, const uint64_t *idx, size_t k);
+dh_status dh_kmeans_update_f64(dh_ctx *ctx, double *C_new, size_t ld_new, double *counts,
+                               const double *X, size_t rows, size_t cols, size_t ldx,
+                               const uint64_t *idx, size_t k);
+
 /* ------------------------------------------------------------------------------------ */
 /* DNN inference ops (NCHW images flattened to rows: one image per matrix row)           */
 /* ------------------------------------------------------------------------------------ */

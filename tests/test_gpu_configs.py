@@ -79,7 +79,8 @@ def _orc_kmeans_iter(X, C, xx):
     return orc.ew_binary(BinaryOpCode.DIV, PtX, np.ascontiguousarray(cnt.T))[1], idx, D
 
 
-def test_config3_kmeans_against_oracle(ctx):
+@pytest.mark.parametrize("fused", [True, False], ids=["two_passes", "operator_sequence"])
+def test_config3_kmeans_against_oracle(ctx, fused):
     """Mixture of 16 Gaussians, 10 Lloyd iterations at an oracle-feasible size; indices bit-exact on rows
     whose two smallest distances are not a near-tie (the GEMMs sum in different orders), centroids 1e-4."""
     rng = np.random.default_rng(3)
@@ -93,7 +94,7 @@ def test_config3_kmeans_against_oracle(ctx):
     Cd, Ce = DenseMatrix.from_numpy(ctx, C0), C0
     ties_total = 0
     for it in range(10):
-        Cd = km.iterate(Cd)
+        Cd = km.iterate(Cd, fused=fused)
         Ce, idx_e, D = _orc_kmeans_iter(X, Ce, xx)
         part = np.partition(D, 1, axis=1)
         near_tie = (part[:, 1] - part[:, 0]) <= 1e-3 * np.abs(part[:, 0])
@@ -116,8 +117,17 @@ def test_config3_full_size_properties(ctx):
     X = DenseMatrix.from_torch(ctx, Xt)
     km = KMeans(ctx, X, k)
     C = DenseMatrix.from_torch(ctx, Xt[torch.arange(k, device="cuda") * (n // k) + torch.arange(k, device="cuda")].contiguous())
-    for _ in range(3):
+    for _ in range(2):
         C = km.iterate(C)
+    # the two passes over X against the operator sequence from the same centroids: the same assignment bit for bit
+    # (the product comes from the same streaming kernel), the same sizes, centroids to rounding
+    C_seq = km.iterate(C, fused=False)
+    idx_seq, counts_seq = km.idx.to_numpy().copy(), km.counts.to_numpy().copy()
+    C = km.iterate(C)
+    assert_exact(km.idx.to_numpy(), idx_seq)
+    assert_exact(km.counts.to_numpy(), counts_seq)
+    assert float(km.counts.to_numpy().sum()) == n
+    assert_close(C.to_numpy(), C_seq.to_numpy(), rtol=1e-5, elementwise=False)
     idx = torch.from_numpy(km.idx.to_numpy()[:, 0].astype(np.int64)).cuda()
     P = torch.from_numpy(km.P.to_numpy()).cuda()
     assert bool((P.sum(1) == 1).all()) and float(P.sum()) == n

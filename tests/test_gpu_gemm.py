@@ -14,7 +14,8 @@ from parity import assert_close, assert_exact
 pytestmark = pytest.mark.gpu
 
 from daphne_amd import capi
-from daphne_amd.kernels import DenseMatrix, affineForward, affineForwardFused, matMul, reluForward, solve, syrk
+from daphne_amd.kernels import (AggOpCode, BinaryOpCode, DenseMatrix, affineForward, affineForwardFused, aggRow, ewBinaryMat,
+                                ewBinaryObjSca, kmeansAssign, kmeansUpdate, matMul, reluForward, solve, syrk)
 
 DTYPES = [np.float32, np.float64]
 
@@ -400,3 +401,90 @@ def test_normal_equations_of_other_shapes(ctx, dt, rows, cols):
     x64 = x.astype(np.float64)
     assert_close(A.to_numpy(), (x64.T @ x64 + 1e-3 * np.eye(cols)).astype(dt), elementwise=False)
     assert_close(b.to_numpy(), (x64.T @ y.astype(np.float64)).astype(dt), elementwise=False)
+
+
+KMEANS_SHAPES = [  # rows, cols, k
+    (1, 4, 1), (7, 8, 3), (100, 64, 16), (513, 64, 16), (70_000, 64, 16), (66_000, 32, 32), (65_600, 12, 17), (3000, 200, 5),
+    (2049, 128, 20), (131_072, 4, 2),
+]
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("rows,cols,k", KMEANS_SHAPES)
+def test_kmeans_assign_and_update(ctx, dt, rows, cols, k):
+    """The two passes against the operator sequence on the device (bit for bit where the product takes the streaming
+    kernel: 65536 rows or more) and against the oracle (away from near-ties)."""
+    rng = np.random.default_rng(rows + cols + k)
+    centres = rng.standard_normal((k, cols)) * 3
+    x = (centres[rng.integers(0, k, rows)] + rng.standard_normal((rows, cols))).astype(dt)
+    c = (centres + 0.3 * rng.standard_normal((k, cols))).astype(dt)
+    if k > 2:
+        c[k - 1] = c[1]  # two equal centroids: the lower position wins
+    X, C = DenseMatrix.from_numpy(ctx, x), DenseMatrix.from_numpy(ctx, c)
+    xx = aggRow(AggOpCode.SUM, None, ewBinaryMat(BinaryOpCode.MUL, None, X, X, ctx), ctx)
+    cc = aggRow(AggOpCode.SUM, None, ewBinaryMat(BinaryOpCode.MUL, None, C, C, ctx), ctx)
+    idx = kmeansAssign(None, X, C, xx, cc, ctx).to_numpy()
+    # the operator sequence
+    XC = matMul(None, X, C, False, True, ctx)
+    D = ewBinaryObjSca(BinaryOpCode.MUL, None, XC, -2.0, ctx)
+    D = ewBinaryMat(BinaryOpCode.ADD, None, D, xx, ctx)
+    cc_row = DenseMatrix.from_numpy(ctx, np.ascontiguousarray(cc.to_numpy().T))
+    D = ewBinaryMat(BinaryOpCode.ADD, None, D, cc_row, ctx)
+    idx_seq = aggRow(AggOpCode.IDXMIN, None, D, ctx).to_numpy()
+    d = D.to_numpy().astype(np.float64)
+    if rows >= 65536:
+        assert_exact(idx, idx_seq)
+    else:
+        part = np.partition(d, 1, axis=1) if k > 1 else np.concatenate([d, d + 1], axis=1)
+        clear = (part[:, 1] - part[:, 0]) > 1e-3 * np.abs(part[:, 0]) if k > 1 else np.ones(rows, bool)
+        if k > 2:
+            clear &= ~np.isin(idx_seq[:, 0], (1, k - 1))
+        assert_exact(idx[clear], idx_seq[clear])
+    assert idx.dtype == np.uint64 and (idx < k).all()
+    if k > 2:
+        assert not (idx == k - 1).any()
+    st, idx_o = orc.agg_row(AggOpCode.IDXMIN, d.astype(dt))
+    same = (idx == idx_o).mean()
+    assert same > 0.999
+    # update: per-cluster means and sizes from idx
+    if cols > (256 if dt == np.float32 else 128):
+        with pytest.raises(capi.DaphneHipError, match="features are supported"):
+            kmeansUpdate(None, X, DenseMatrix.from_numpy(ctx, idx), k, ctx)
+        return
+    Cn, counts = kmeansUpdate(None, X, DenseMatrix.from_numpy(ctx, idx), k, ctx)
+    cnt = np.bincount(idx[:, 0].astype(np.int64), minlength=k).astype(np.float64)
+    assert_exact(counts.to_numpy()[0].astype(np.float64), cnt)
+    sums = np.zeros((k, cols))
+    np.add.at(sums, idx[:, 0].astype(np.int64), x.astype(np.float64))
+    with np.errstate(invalid="ignore", divide="ignore"):
+        exp = (sums / cnt[:, None]).astype(dt)
+    assert_close(Cn.to_numpy(), exp, rtol=2e-5 if dt == np.float32 else 1e-12, elementwise=False)
+    assert np.isnan(Cn.to_numpy()[cnt == 0]).all()
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+def test_kmeans_assign_nan_semantics_and_errors(ctx, dt):
+    """IDXMIN's rules on the fused distances: NaN is never better, a row that starts with NaN or holds only NaN gives 0."""
+    rows, cols, k = 64, 8, 6
+    rng = np.random.default_rng(0)
+    x = rng.standard_normal((rows, cols)).astype(dt)
+    c = rng.standard_normal((k, cols)).astype(dt)
+    X, C = DenseMatrix.from_numpy(ctx, x), DenseMatrix.from_numpy(ctx, c)
+    xx = DenseMatrix.from_numpy(ctx, (x * x).sum(1, keepdims=True).astype(dt))
+    cc_h = (c * c).sum(1, keepdims=True).astype(dt)
+    cc_h[0] = np.nan   # distance to centroid 0 is NaN in every row: position 0 by the first-value rule
+    idx = kmeansAssign(None, X, C, xx, DenseMatrix.from_numpy(ctx, cc_h), ctx).to_numpy()
+    assert (idx == 0).all()
+    cc_h[0], cc_h[3] = (c[0] * c[0]).sum(), np.nan  # a NaN elsewhere is skipped
+    idx = kmeansAssign(None, X, C, xx, DenseMatrix.from_numpy(ctx, cc_h), ctx).to_numpy()
+    d = (x @ c.T) * -2 + (x * x).sum(1, keepdims=True) + cc_h.T
+    assert_exact(idx[:, 0], np.nanargmin(d, axis=1).astype(np.uint64))
+    with pytest.raises(capi.DaphneHipError, match="1..32 centroids"):
+        kmeansAssign(None, X, DenseMatrix.from_numpy(ctx, np.zeros((33, cols), dt)), xx, DenseMatrix.from_numpy(ctx, np.zeros((33, 1), dt)), ctx)
+    with pytest.raises(capi.DaphneHipError, match="16-byte"):
+        x3 = DenseMatrix.from_numpy(ctx, np.zeros((4, 3), dt))
+        kmeansAssign(None, x3, DenseMatrix.from_numpy(ctx, np.zeros((2, 3), dt)), DenseMatrix.from_numpy(ctx, np.zeros((4, 1), dt)),
+                     DenseMatrix.from_numpy(ctx, np.zeros((2, 1), dt)), ctx)
+    with pytest.raises(capi.DaphneHipError, match="features are supported"):
+        wide = DenseMatrix.from_numpy(ctx, np.zeros((4, 600), dt))
+        kmeansUpdate(None, wide, DenseMatrix.from_numpy(ctx, np.zeros((4, 1), np.uint64)), 2, ctx)
