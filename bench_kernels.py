@@ -146,6 +146,17 @@ def main() -> int:
             PtX = DM(ctx, 16, cols, ndt)
             emit("tall matMul t(P) X, P rows x 16", dt, shape, timed(lambda: K.matMul(PtX, XC, X, True, False, ctx)), nb + rows * 16 * sz)
             XC.destroy()
+            # the k-means passes: X once each, no rows x 16 matrix in memory
+            xxv = DM.from_torch(ctx, torch.rand(rows, 1, device="cuda", dtype=tdt, generator=gen))
+            ccv = DM.from_torch(ctx, torch.rand(16, 1, device="cuda", dtype=tdt, generator=gen))
+            idxv = DM(ctx, rows, 1, np.uint64)
+            emit("kmeansAssign (X t(C), distances, row arg-min), C 16x64", dt, shape, timed(lambda: K.kmeansAssign(idxv, X, Cc, xxv, ccv, ctx)),
+                 nb + rows * sz + rows * 8)
+            cnts = DM(ctx, 1, 16, ndt)
+            emit("kmeansUpdate (t(one-hot(idx)) X / sizes), 16 centroids", dt, shape, timed(lambda: K.kmeansUpdate(PtX, X, idxv, 16, ctx, cnts)),
+                 nb + rows * 8)
+            for m_ in (xxv, ccv, idxv, cnts):
+                m_.destroy()
         for m in (X, R, colv, r1, ri):
             m.destroy()
         ctx.releaseCached()
@@ -178,6 +189,9 @@ def main() -> int:
             emit("batchNormInferenceForward 64 channels", dt, f"{N}x{64 * 196}",
                  timed(lambda: K.batchNormInferenceForward(o2, o2, one, b2, b2, one, 1e-5, ctx)), 2 * N * 64 * 196 * sz)
             pl = DM(ctx, N, 64 * 49, ndt)
+            emit("conv2dForwardFused 32->64 ch, 14x14, 5x5 pad 2, ReLU + maxPool 2x2 in the epilogue", dt, f"batch {N}",
+                 timed(lambda: K.conv2dForwardFused(pl, x2, w2, b2, N, 32, 14, 14, 5, 5, 1, 1, 2, 2, ctx, relu=True, pool=True)),
+                 flops=2.0 * N * 64 * 196 * 800)
             emit("maxPoolForward 2x2/2 on 14x14", dt, f"{N}x{64 * 196}",
                  timed(lambda: K.maxPoolForward(pl, o2, N, 64, 14, 14, 2, 2, 2, 2, 0, 0, ctx)), 1.25 * N * 64 * 196 * sz)
             emit("avgPoolForward 2x2/2 on 14x14", dt, f"{N}x{64 * 196}",
@@ -236,6 +250,14 @@ def main() -> int:
             if not args.only or args.only in ("solve",) or args.only in "solve 100x100":
                 print(json.dumps({"kernel": "solve 100x100 (latency bound, incl. the singularity flag read-back)", "dtype": dt,
                                   "shape": "100x100", "us": round(us, 1)}), flush=True)
+            # normal equations of a 100000 x 100 regression: t(X) X + lambda I and t(X) y from one pass over X
+            Xn = DM.from_torch(ctx, torch.rand(100_000, n, device="cuda", dtype=tdt, generator=gen))
+            yn = DM.from_torch(ctx, torch.rand(100_000, 1, device="cuda", dtype=tdt, generator=gen))
+            An, bn = DM(ctx, n, n, ndt), DM(ctx, n, 1, ndt)
+            emit("normalEquations (t(X) X + lambda I, t(X) y; upper tile pairs only)", dt, "100000x100",
+                 timed(lambda: K.normalEquations(Xn, yn, 1e-3, ctx, An, bn)), 100_000 * (n + 1) * sz)
+            for m_ in (Xn, yn, An, bn):
+                m_.destroy()
         ctx.releaseCached()
         torch.cuda.empty_cache()
     ctx.destroy()

@@ -45,10 +45,7 @@ dh_status assign(dh_ctx *ctx, unsigned long long *idx, const T *X, size_t rows, 
     g.row_add = xx;
     g.col_add = cc;
     g.idx = idx;
-    const size_t blocks = dh_ceil_div(rows, 4 * 16 * TS_NT_RBW);
-    if (blocks >= (size_t(1) << 31))
-        return dh_fail(DH_ERR_RUNTIME, "kmeans assign: too many rows for one launch");
-    const dh_status st = nb == 1 ? dh_gemm::ts_nt_launch<T, 1, true>(ctx, g, blocks) : dh_gemm::ts_nt_launch<T, 2, true>(ctx, g, blocks);
+    const dh_status st = nb == 1 ? dh_gemm::ts_nt_launch<T, 1, true>(ctx, g) : dh_gemm::ts_nt_launch<T, 2, true>(ctx, g);
     if (st != DH_OK)
         return st;
     DH_CHECK_LAUNCH();

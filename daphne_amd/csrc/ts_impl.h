@@ -23,9 +23,6 @@
 #include "common.h"
 
 namespace dh_gemm {
-#ifndef TS_NT_RBW
-#define TS_NT_RBW 8 // 16-row blocks per wave of ts_nt_kernel
-#endif
 #ifndef TS_SYM_U
 #define TS_SYM_U 4 // quads per register set of the symmetric one-wave form (measured: 2 1.00 ms, 4 0.90, 8 0.92, 12 0.95)
 #endif
@@ -377,7 +374,6 @@ template <typename T, int NB, bool ASSIGN, int CPG> __global__ __launch_bounds__
     using M = Mfma16<T>;
     constexpr int V = 16 / sizeof(T);
     constexpr int KC = 4 * V;     // k values per chunk
-    constexpr int RBW = TS_NT_RBW; // row blocks per wave
     // float: the operands of the matrix instruction are exchanged, which transposes the result tile in the
     // registers (row = 4 * (lane / 16) + v becomes the column) and turns four 4-byte stores per lane into one of
     // 16 bytes; the double layout (row = 4 * v + lane / 16) already stores whole 128-byte rows
@@ -410,9 +406,15 @@ template <typename T, int NB, bool ASSIGN, int CPG> __global__ __launch_bounds__
     // its first use): rows beyond M read the last row - they only produce rows of C that are not stored -, k
     // beyond K reads k = 0 and is zeroed when it is used (the padded part of B is zero, but 0 * NaN would still
     // be NaN), and steps beyond the last repeat the last one.
+    // Pairs of row blocks are dealt to the wavefronts of the whole grid round-robin (pair number = wavefront number +
+    // j * number of wavefronts): the grid is what the device holds at once, every wavefront gets the same number of
+    // pairs to within one, and neighbouring wavefronts read neighbouring rows.
     const unsigned chunks = g.kpad / KC;
     const unsigned cg = chunks / CPG;                // chunk groups per row-block pair (CPG divides chunks)
-    const unsigned nsteps = (RBW / 2) * cg;          // even
+    const size_t total_pairs = (g.M + 31) / 32;
+    const size_t first_pair = static_cast<size_t>(blockIdx.x) * 4 + wave, pair_stride = static_cast<size_t>(gridDim.x) * 4;
+    const unsigned my_pairs = first_pair < total_pairs ? static_cast<unsigned>((total_pairs - 1 - first_pair) / pair_stride) + 1 : 0;
+    const unsigned nsteps = my_pairs * cg;
     constexpr int RPL = SWAP ? 1 : 4; // ASSIGN: rows per lane and row block in the result layout
     struct Frag {
         T a[2][CPG][V];
@@ -425,32 +427,31 @@ template <typename T, int NB, bool ASSIGN, int CPG> __global__ __launch_bounds__
     constexpr unsigned VPR = CPG * 4;      // vectors of a row in one step
     constexpr unsigned SX = CPG * KC + V;
     T *stage = lb + NB * 16 * ldl + wave * (16 * SX); // one row block at a time
-    // Addresses are a base that is the same for the whole wave plus a 32-bit byte offset per lane (the wave's rows span
-    // at most 16 RBW rows of at most 2^24 bytes): one 24-bit multiplication and an addition per load, rows beyond M
-    // cut back to the last row by a minimum on the row number.
-    const size_t row0 = (static_cast<size_t>(blockIdx.x) * 4 + wave) * (16 * RBW);
-    const size_t row0_ok = row0 < g.M ? row0 : g.M - 1;
-    const char *wave_base = reinterpret_cast<const char *>(A + row0_ok * g.lda);
-    const unsigned last_local = static_cast<unsigned>(g.M - 1 - row0_ok < 16 * RBW ? g.M - 1 - row0_ok : 16 * RBW - 1);
+    // Addresses are a base that is the same for the whole wave - the pair's first row - plus a 32-bit byte offset per
+    // lane (32 rows of at most 2^24 bytes): one 24-bit multiplication and an addition per load, rows beyond M cut
+    // back to the last row by a minimum on the row number.
     const unsigned row_bytes = static_cast<unsigned>(g.lda * sizeof(T));
     auto load_step = [&](Frag &fr, unsigned pair, unsigned grp) {
+        const size_t prow = (first_pair + static_cast<size_t>(pair) * pair_stride) * 32; // < M for every pair of this wave
+        const char *pair_base = reinterpret_cast<const char *>(A + prow * g.lda);
+        const unsigned last_local = g.M - 1 - prow < 31 ? static_cast<unsigned>(g.M - 1 - prow) : 31u;
 #pragma unroll
         for (int c = 0; c < CPG; c++) {
             const unsigned id = c * 64 + lane;
             const unsigned kv = grp * CPG * KC + (id % VPR) * V;
             const unsigned kb = (kv < g.K ? kv : 0) * static_cast<unsigned>(sizeof(T));
-            const unsigned r0 = pair * 32 + id / VPR, r1 = r0 + 16;
+            const unsigned r0 = id / VPR, r1 = r0 + 16;
             const unsigned l0 = r0 < last_local ? r0 : last_local, l1 = r1 < last_local ? r1 : last_local;
-            ts_load<T, V>(reinterpret_cast<const T *>(wave_base + (__umul24(l0, row_bytes) + kb)), fr.a[0][c], true);
-            ts_load<T, V>(reinterpret_cast<const T *>(wave_base + (__umul24(l1, row_bytes) + kb)), fr.a[1][c], true);
+            ts_load<T, V>(reinterpret_cast<const T *>(pair_base + (__umul24(l0, row_bytes) + kb)), fr.a[0][c], true);
+            ts_load<T, V>(reinterpret_cast<const T *>(pair_base + (__umul24(l1, row_bytes) + kb)), fr.a[1][c], true);
         }
         if constexpr (ASSIGN) {
-            const T *ra_base = static_cast<const T *>(g.row_add) + row0_ok;
+            const T *ra_base = static_cast<const T *>(g.row_add) + prow;
 #pragma unroll
             for (int t = 0; t < 2; t++)
 #pragma unroll
                 for (int v = 0; v < RPL; v++) {
-                    const unsigned r = pair * 32 + t * 16 + (SWAP ? i : M::row(lane, v));
+                    const unsigned r = t * 16 + (SWAP ? i : M::row(lane, v));
                     fr.ra[t][v] = ra_base[r < last_local ? r : last_local];
                 }
         }
@@ -501,7 +502,7 @@ template <typename T, int NB, bool ASSIGN, int CPG> __global__ __launch_bounds__
         }
         if (grp + 1 != cg)
             return;
-        const size_t rbase = row0 + static_cast<size_t>(pair) * 32;
+        const size_t rbase = (first_pair + static_cast<size_t>(pair) * pair_stride) * 32;
         if constexpr (ASSIGN) {
 #pragma clang fp contract(off)
             constexpr unsigned NONE = ~0u;
@@ -646,16 +647,17 @@ template <typename T, int NB, bool ASSIGN, int CPG> __global__ __launch_bounds__
     auto advance = [&](unsigned &pair, unsigned &grp) {
         if (++grp == cg) {
             grp = 0;
-            if (pair + 1 < RBW / 2)
+            if (pair + 1 < my_pairs)
                 pair++;
             else
-                grp = cg - 1; // beyond the last step: stay on it
+                grp = cg - 1; // beyond the last step: stay on it (loaded again, never computed)
         }
     };
     Frag f0, f1;
     unsigned lp = 0, lg = 0; // step being loaded
     unsigned cp = 0, cgp = 0; // step being computed
-    load_step(f0, lp, lg);
+    if (nsteps > 0)
+        load_step(f0, lp, lg);
     __builtin_amdgcn_sched_barrier(0);
 
     for (unsigned idx = tid; idx < NB * 16 * (g.kpad / V); idx += 256) {
@@ -672,7 +674,6 @@ template <typename T, int NB, bool ASSIGN, int CPG> __global__ __launch_bounds__
     }
     __syncthreads();
 
-
     for (unsigned s2 = 0; s2 < nsteps; s2 += 2) {
         advance(lp, lg);
         load_step(f1, lp, lg);
@@ -683,7 +684,8 @@ template <typename T, int NB, bool ASSIGN, int CPG> __global__ __launch_bounds__
         advance(lp, lg);
         load_step(f0, lp, lg);
         __builtin_amdgcn_sched_barrier(0);
-        compute_step(f1, cp, cgp);
+        if (s2 + 1 < nsteps)
+            compute_step(f1, cp, cgp);
         __builtin_amdgcn_sched_barrier(0);
         advance(cp, cgp);
     }
@@ -799,20 +801,28 @@ template <typename T> inline int ts_nt_chunks_per_step(unsigned kpad) {
 }
 
 template <typename T, int NB, bool ASSIGN, int CPG>
-inline dh_status ts_nt_launch_cpg(dh_ctx *ctx, const TsNtArgs &g, size_t blocks, size_t lds) {
+inline dh_status ts_nt_launch_cpg(dh_ctx *ctx, const TsNtArgs &g, size_t lds) {
+    const void *kernel = reinterpret_cast<const void *>(&ts_nt_kernel<T, NB, ASSIGN, CPG>);
     // dynamic LDS beyond 64 KiB has to be asked for, per kernel and device (the call is cheap next to the kernel)
     if (lds > 65536)
-        DH_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&ts_nt_kernel<T, NB, ASSIGN, CPG>),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
+        DH_CHECK_HIP(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
+    // as many workgroups as the device holds at once (they share out the rows among themselves), fewer for few rows
+    int per_cu = 0;
+    DH_CHECK_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, 256, lds));
+    if (per_cu < 1)
+        per_cu = 1;
+    size_t blocks = static_cast<size_t>(ctx->num_cus) * per_cu;
+    const size_t needed = dh_ceil_div(dh_ceil_div(g.M, 32), 4 * 2); // at least two pairs per wavefront
+    if (blocks > needed)
+        blocks = needed > 0 ? needed : 1;
     hipLaunchKernelGGL((ts_nt_kernel<T, NB, ASSIGN, CPG>), dim3(static_cast<unsigned>(blocks)), dim3(256), lds, ctx->stream, g);
     return DH_OK;
 }
-template <typename T, int NB, bool ASSIGN> inline dh_status ts_nt_launch(dh_ctx *ctx, const TsNtArgs &g, size_t blocks) {
+template <typename T, int NB, bool ASSIGN> inline dh_status ts_nt_launch(dh_ctx *ctx, const TsNtArgs &g) {
     const int cpg = ts_nt_chunks_per_step<T>(g.kpad);
     const size_t lds = ts_nt_lds_bytes<T>(NB, g.kpad, cpg);
-    return cpg == 4 ? ts_nt_launch_cpg<T, NB, ASSIGN, 4>(ctx, g, blocks, lds)
-                    : (cpg == 2 ? ts_nt_launch_cpg<T, NB, ASSIGN, 2>(ctx, g, blocks, lds)
-                                : ts_nt_launch_cpg<T, NB, ASSIGN, 1>(ctx, g, blocks, lds));
+    return cpg == 4 ? ts_nt_launch_cpg<T, NB, ASSIGN, 4>(ctx, g, lds)
+                    : (cpg == 2 ? ts_nt_launch_cpg<T, NB, ASSIGN, 2>(ctx, g, lds) : ts_nt_launch_cpg<T, NB, ASSIGN, 1>(ctx, g, lds));
 }
 
 template <typename T>
@@ -836,10 +846,9 @@ bool ts_nt(dh_ctx *ctx, size_t M, size_t n, size_t K, const T *A, size_t lda, co
     g.K = static_cast<unsigned>(K);
     g.kpad = static_cast<unsigned>(dh_ceil_div(K, KC) * KC);
     g.vec_store = dh_aligned(C, 16) && (ldc * sizeof(T)) % 16 == 0;
-    const size_t blocks = dh_ceil_div(M, 4 * 16 * TS_NT_RBW);
-    if (blocks >= (size_t(1) << 31) || static_cast<size_t>(nb) * 16 * (g.kpad + V) * sizeof(T) > (size_t(48) << 10))
+    if (static_cast<size_t>(nb) * 16 * (g.kpad + V) * sizeof(T) > (size_t(48) << 10))
         return false;
-    *status = nb == 1 ? ts_nt_launch<T, 1, false>(ctx, g, blocks) : ts_nt_launch<T, 2, false>(ctx, g, blocks);
+    *status = nb == 1 ? ts_nt_launch<T, 1, false>(ctx, g) : ts_nt_launch<T, 2, false>(ctx, g);
     return true;
 }
 
