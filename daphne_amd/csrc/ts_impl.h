@@ -456,8 +456,11 @@ template <typename T, int NB, bool ASSIGN, int CPG> __global__ __launch_bounds__
                 }
         }
     };
-    typename M::acc_t acc[2][NB];
-    auto compute_step = [&](const Frag &fr, unsigned pair, unsigned grp) {
+    // Two sets of accumulators: with a single step per pair of row blocks (K of at most CPG chunks) the result of one
+    // pair is finished - distances and arg-min, or the store - beside the matrix instructions of the next.
+    using AccSet = typename M::acc_t[2][NB];
+    AccSet accA, accB;
+    auto mma_step = [&](AccSet &acc, const Frag &fr, unsigned grp) {
         if (grp == 0) {
 #pragma unroll
             for (int b = 0; b < NB; b++) {
@@ -500,8 +503,8 @@ template <typename T, int NB, bool ASSIGN, int CPG> __global__ __launch_bounds__
                 }
             }
         }
-        if (grp + 1 != cg)
-            return;
+    };
+    auto finish_pair = [&](AccSet &acc, unsigned pair, const T (&radd)[2][RPL]) {
         const size_t rbase = (first_pair + static_cast<size_t>(pair) * pair_stride) * 32;
         if constexpr (ASSIGN) {
 #pragma clang fp contract(off)
@@ -521,7 +524,7 @@ template <typename T, int NB, bool ASSIGN, int CPG> __global__ __launch_bounds__
                     for (int b = 0; b < NB; b++)
 #pragma unroll
                         for (int v = 0; v < 4; v++)
-                            d[t][b][v] = (acc[t][b][v] * T(-2) + fr.ra[t][0]) + col_add[b][v];
+                            d[t][b][v] = (acc[t][b][v] * T(-2) + radd[t][0]) + col_add[b][v];
                 // The short way: a plain running minimum. It gives IDXMIN's answer unless a NaN is among the values or
                 // nothing lies below +inf; the sum of a lane's values tells the first (opposite infinities only send
                 // the wave the long way for nothing), the minimum itself the second.
@@ -586,7 +589,7 @@ template <typename T, int NB, bool ASSIGN, int CPG> __global__ __launch_bounds__
 #pragma unroll
                     for (int v = 0; v < 4; v++) {
                         const size_t row = rbase + static_cast<size_t>(t) * 16 + M::row(lane, v);
-                        const T ra = fr.ra[t][SWAP ? 0 : v];
+                        const T ra = radd[t][SWAP ? 0 : v];
                         T best = dh_inf<T>(), first = T(0);
                         unsigned bi = NONE;
 #pragma unroll
@@ -643,6 +646,11 @@ template <typename T, int NB, bool ASSIGN, int CPG> __global__ __launch_bounds__
                 }
         }
     };
+    auto compute_step = [&](const Frag &fr, unsigned pair, unsigned grp) {
+        mma_step(accA, fr, grp);
+        if (grp + 1 == cg)
+            finish_pair(accA, pair, fr.ra);
+    };
     // (pair, grp) of a step and of the one after it, stepped without divisions
     auto advance = [&](unsigned &pair, unsigned &grp) {
         if (++grp == cg) {
@@ -674,6 +682,47 @@ template <typename T, int NB, bool ASSIGN, int CPG> __global__ __launch_bounds__
     }
     __syncthreads();
 
+    if (cg == 1) {
+        // One step per pair: step s is pair s. Steady state = loads of step s + 1, matrix instructions of step s and
+        // the finish of step s - 1 in one stretch of code, so that the three overlap inside the wavefront too.
+        if (nsteps == 0)
+            return;
+        T ra0[2][RPL], ra1[2][RPL];
+        auto keep = [&](T (&dst)[2][RPL], const Frag &fr) {
+#pragma unroll
+            for (int t = 0; t < 2; t++)
+#pragma unroll
+                for (int v = 0; v < RPL; v++)
+                    dst[t][v] = fr.ra[t][v];
+        };
+        load_step(f1, nsteps > 1 ? 1 : 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        mma_step(accA, f0, 0);
+        keep(ra0, f0);
+        unsigned sdone = 1; // steps whose matrix instructions are done; the last of them is not finished yet
+        for (; sdone + 1 < nsteps; sdone += 2) {
+            load_step(f0, sdone + 1, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            mma_step(accB, f1, 0);
+            finish_pair(accA, sdone - 1, ra0);
+            keep(ra1, f1);
+            __builtin_amdgcn_sched_barrier(0);
+            load_step(f1, sdone + 2 < nsteps ? sdone + 2 : nsteps - 1, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            mma_step(accA, f0, 0);
+            finish_pair(accB, sdone, ra1);
+            keep(ra0, f0);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if (sdone < nsteps) {
+            mma_step(accB, f1, 0);
+            finish_pair(accA, sdone - 1, ra0);
+            finish_pair(accB, sdone, f1.ra);
+        } else {
+            finish_pair(accA, sdone - 1, ra0);
+        }
+        return;
+    }
     for (unsigned s2 = 0; s2 < nsteps; s2 += 2) {
         advance(lp, lg);
         load_step(f1, lp, lg);
