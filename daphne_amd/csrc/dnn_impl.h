@@ -859,7 +859,9 @@ __global__ __launch_bounds__(256) void maxpool_kernel(T *res, const T *data, siz
 // the first LDS store) and then gathers every window from LDS; the outputs of the planes are contiguous
 // as well and go out coalesced. Window clipping and arithmetic are those of maxpool_kernel /
 // avgpool_kernel. The host picks ppb so that a workgroup's first element is 16-byte aligned.
-template <typename T, bool AVG>
+// TWO: the window is 2 x 2 with stride 2, no padding, H and W even: two 2-value reads per output, arithmetic of
+// maxpool2x2_kernel.
+template <typename T, bool AVG, bool TWO = false>
 __global__ __launch_bounds__(256) void pool_planes_kernel(T *res, const T *data, size_t planes, unsigned ppb, unsigned H,
                                                           unsigned W, unsigned P, unsigned Q, unsigned ph, unsigned pw,
                                                           unsigned sh, unsigned sw, unsigned padh, unsigned padw, T plen) {
@@ -897,6 +899,25 @@ __global__ __launch_bounds__(256) void pool_planes_kernel(T *res, const T *data,
         const unsigned plane = o / PQ, pq = o % PQ;
         const unsigned p = pq / Q, q = pq % Q;
         const T *in = tile + plane * HW;
+        if constexpr (TWO) {
+            typedef T pair_t __attribute__((ext_vector_type(2)));
+            const T *w = in + 2 * p * W + 2 * q; // an even offset: the pair is aligned
+            const pair_t a = *reinterpret_cast<const pair_t *>(w), b = *reinterpret_cast<const pair_t *>(w + W);
+            if constexpr (AVG) {
+                const T s0 = (T(0) + a[0]) + a[1];
+                const T s1 = (T(0) + b[0]) + b[1];
+                const T r0 = s0 * T(0.25) + T(0);
+                dst[o] = s1 * T(0.25) + r0;
+            } else {
+                T m = T(0);
+                m = (m < a[0]) ? a[0] : m;
+                m = (m < a[1]) ? a[1] : m;
+                m = (m < b[0]) ? b[0] : m;
+                m = (m < b[1]) ? b[1] : m;
+                dst[o] = m;
+            }
+            continue;
+        }
         const int y_lo = static_cast<int>(p * sh) - static_cast<int>(padh);
         const int x_lo = static_cast<int>(q * sw) - static_cast<int>(padw);
         const int y0 = y_lo < 0 ? 0 : y_lo, x0 = x_lo < 0 ? 0 : x_lo;
@@ -1038,10 +1059,19 @@ dh_status maxpool_forward(dh_ctx *ctx, T *res, size_t *res_h, size_t *res_w, con
     constexpr int VI = 16 / sizeof(T);
     const bool pairs = ph == 2 && pw == 2 && sh == 2 && sw == 2 && padh == 0 && padw == 0 && H % 2 == 0 && W % 2 == 0 &&
                        total < (size_t(1) << 39);
-    if (pairs && W % VI == 0 && dh_aligned(data, 16) && dh_aligned(res, 8)) {
+    // rows of less than 128 bytes go through LDS even where they are whole vectors: measured 14 x 14 doubles
+    const bool short_rows = W * sizeof(T) < 128;
+    if (pairs && !short_rows && W % VI == 0 && dh_aligned(data, 16) && dh_aligned(res, 8)) {
         const size_t items = N * C * P * (W / VI);
         hipLaunchKernelGGL((maxpool2x2_kernel<T, VI>), dim3(static_cast<unsigned>(dh_ceil_div(items, 256))), dim3(256), 0,
                            ctx->stream, res, data, items, static_cast<unsigned>(W), static_cast<unsigned>(W / VI));
+    } else if (const unsigned ppb2 = pairs ? pool_planes_per_block(data, H * W, N * C) : 0;
+               ppb2 != 0 && dh_ceil_div(N * C, ppb2) < (size_t(1) << 31) && ppb2 * P * Q < (size_t(1) << 31)) {
+        // rows that are no whole number of 16-byte vectors (14 x 14 floats): the planes are contiguous, so a workgroup
+        // copies a run of them into LDS with 16-byte loads and gathers the windows there
+        hipLaunchKernelGGL((pool_planes_kernel<T, false, true>), dim3(static_cast<unsigned>(dh_ceil_div(N * C, ppb2))), dim3(256),
+                           ppb2 * H * W * sizeof(T), ctx->stream, res, data, N * C, ppb2, static_cast<unsigned>(H),
+                           static_cast<unsigned>(W), static_cast<unsigned>(P), static_cast<unsigned>(Q), 2u, 2u, 2u, 2u, 0u, 0u, T(0));
     } else if (pairs && VI > 2 && dh_aligned(data, 8)) {
         // rows of an even number of floats that is not a multiple of four: 8-byte loads, one output per thread
         const size_t items = N * C * P * (W / 2);
@@ -1146,10 +1176,19 @@ dh_status avgpool_forward(dh_ctx *ctx, T *res, size_t *res_h, size_t *res_w, con
     constexpr int VI = 16 / sizeof(T);
     const bool pairs = ph == 2 && pw == 2 && sh == 2 && sw == 2 && padh == 0 && padw == 0 && H % 2 == 0 && W % 2 == 0 &&
                        total < (size_t(1) << 39);
-    if (pairs && W % VI == 0 && dh_aligned(data, 16) && dh_aligned(res, 8)) {
+    const bool short_rows = W * sizeof(T) < 128; // as in maxpool_forward
+    if (pairs && !short_rows && W % VI == 0 && dh_aligned(data, 16) && dh_aligned(res, 8)) {
         const size_t items = N * C * P * (W / VI);
         hipLaunchKernelGGL((maxpool2x2_kernel<T, VI, true>), dim3(static_cast<unsigned>(dh_ceil_div(items, 256))), dim3(256),
                            0, ctx->stream, res, data, items, static_cast<unsigned>(W), static_cast<unsigned>(W / VI));
+        DH_CHECK_LAUNCH();
+        return DH_OK;
+    }
+    if (const unsigned ppb2 = pairs ? pool_planes_per_block(data, H * W, N * C) : 0;
+        ppb2 != 0 && dh_ceil_div(N * C, ppb2) < (size_t(1) << 31) && ppb2 * P * Q < (size_t(1) << 31)) {
+        hipLaunchKernelGGL((pool_planes_kernel<T, true, true>), dim3(static_cast<unsigned>(dh_ceil_div(N * C, ppb2))), dim3(256),
+                           ppb2 * H * W * sizeof(T), ctx->stream, res, data, N * C, ppb2, static_cast<unsigned>(H),
+                           static_cast<unsigned>(W), static_cast<unsigned>(P), static_cast<unsigned>(Q), 2u, 2u, 2u, 2u, 0u, 0u, T(0.25));
         DH_CHECK_LAUNCH();
         return DH_OK;
     }
