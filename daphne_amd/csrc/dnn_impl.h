@@ -895,6 +895,41 @@ __global__ __launch_bounds__(256) void pool_planes_kernel(T *res, const T *data,
     __syncthreads();
     const unsigned n_out = here * PQ;
     T *dst = res + first * PQ;
+    if (!TWO && PQ <= 256) {
+        // a thread keeps its place in the result plane and walks the planes: the window's extent is worked out once
+        const unsigned groups = 256 / PQ, grp = tid / PQ, pq = tid % PQ;
+        if (grp >= groups)
+            return;
+        const unsigned p = pq / Q, q = pq % Q;
+        const int y_lo = static_cast<int>(p * sh) - static_cast<int>(padh);
+        const int x_lo = static_cast<int>(q * sw) - static_cast<int>(padw);
+        const int y0 = y_lo < 0 ? 0 : y_lo, x0 = x_lo < 0 ? 0 : x_lo;
+        int y1 = y_lo + static_cast<int>(ph), x1 = x_lo + static_cast<int>(pw);
+        if (y1 > static_cast<int>(H))
+            y1 = H;
+        if (x1 > static_cast<int>(W))
+            x1 = W;
+        for (unsigned plane = grp; plane < here; plane += groups) {
+            const T *in = tile + plane * HW;
+            T acc = T(0);
+            for (int y = y0; y < y1; y++) {
+                if constexpr (AVG) {
+                    T s_ = T(0);
+                    for (int x = x0; x < x1; x++)
+                        s_ = s_ + in[static_cast<unsigned>(y) * W + static_cast<unsigned>(x)];
+                    const T scaled = s_ * plen;
+                    acc = scaled + acc;
+                } else {
+                    for (int x = x0; x < x1; x++) {
+                        const T v = in[static_cast<unsigned>(y) * W + static_cast<unsigned>(x)];
+                        acc = (acc < v) ? v : acc; // std::max(acc, v)
+                    }
+                }
+            }
+            dst[plane * PQ + pq] = acc;
+        }
+        return;
+    }
     for (unsigned o = tid; o < n_out; o += 256) {
         const unsigned plane = o / PQ, pq = o % PQ;
         const unsigned p = pq / Q, q = pq % Q;
