@@ -23,6 +23,9 @@
 #include "common.h"
 
 namespace dh_gemm {
+#ifndef TS_NT_PAIRS
+#define TS_NT_PAIRS 4 // pairs of 16-row blocks per wavefront of ts_nt_kernel
+#endif
 #ifndef TS_SYM_U
 #define TS_SYM_U 4 // quads per register set of the symmetric one-wave form (measured: 2 1.00 ms, 4 0.90, 8 0.92, 12 0.95)
 #endif
@@ -406,14 +409,16 @@ template <typename T, int NB, bool ASSIGN, int CPG> __global__ __launch_bounds__
     // its first use): rows beyond M read the last row - they only produce rows of C that are not stored -, k
     // beyond K reads k = 0 and is zeroed when it is used (the padded part of B is zero, but 0 * NaN would still
     // be NaN), and steps beyond the last repeat the last one.
-    // Pairs of row blocks are dealt to the wavefronts of the whole grid round-robin (pair number = wavefront number +
-    // j * number of wavefronts): the grid is what the device holds at once, every wavefront gets the same number of
-    // pairs to within one, and neighbouring wavefronts read neighbouring rows.
+    // A wavefront takes TS_NT_PAIRS consecutive pairs of row blocks (short-lived workgroups, thousands of them: measured
+    // against a grid of resident workgroups that deal the pairs round-robin, this is as fast at 2M rows and 7 % faster
+    // at 20M).
     const unsigned chunks = g.kpad / KC;
     const unsigned cg = chunks / CPG;                // chunk groups per row-block pair (CPG divides chunks)
     const size_t total_pairs = (g.M + 31) / 32;
-    const size_t first_pair = static_cast<size_t>(blockIdx.x) * 4 + wave, pair_stride = static_cast<size_t>(gridDim.x) * 4;
-    const unsigned my_pairs = first_pair < total_pairs ? static_cast<unsigned>((total_pairs - 1 - first_pair) / pair_stride) + 1 : 0;
+    const size_t first_pair = (static_cast<size_t>(blockIdx.x) * 4 + wave) * TS_NT_PAIRS, pair_stride = 1;
+    const unsigned my_pairs = first_pair < total_pairs
+                                  ? static_cast<unsigned>(total_pairs - first_pair < TS_NT_PAIRS ? total_pairs - first_pair : TS_NT_PAIRS)
+                                  : 0;
     const unsigned nsteps = my_pairs * cg;
     constexpr int RPL = SWAP ? 1 : 4; // ASSIGN: rows per lane and row block in the result layout
     struct Frag {
@@ -682,7 +687,9 @@ template <typename T, int NB, bool ASSIGN, int CPG> __global__ __launch_bounds__
     }
     __syncthreads();
 
-    if (cg == 1) {
+    if (cg == 1 && !ASSIGN) {
+        // (Measured: this helps the store of the product, 119 -> 113 us at 2M rows and 1163 -> 1101 us at 20M, and
+        // costs the arg-min epilogue, 103 -> 112 us and 941 -> 978 us, whose wavefronts have four steps in all.)
         // One step per pair: step s is pair s. Steady state = loads of step s + 1, matrix instructions of step s and
         // the finish of step s - 1 in one stretch of code, so that the three overlap inside the wavefront too.
         if (nsteps == 0)
@@ -855,15 +862,9 @@ inline dh_status ts_nt_launch_cpg(dh_ctx *ctx, const TsNtArgs &g, size_t lds) {
     // dynamic LDS beyond 64 KiB has to be asked for, per kernel and device (the call is cheap next to the kernel)
     if (lds > 65536)
         DH_CHECK_HIP(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
-    // as many workgroups as the device holds at once (they share out the rows among themselves), fewer for few rows
-    int per_cu = 0;
-    DH_CHECK_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, 256, lds));
-    if (per_cu < 1)
-        per_cu = 1;
-    size_t blocks = static_cast<size_t>(ctx->num_cus) * per_cu;
-    const size_t needed = dh_ceil_div(dh_ceil_div(g.M, 32), 4 * 2); // at least two pairs per wavefront
-    if (blocks > needed)
-        blocks = needed > 0 ? needed : 1;
+    const size_t blocks = dh_ceil_div(dh_ceil_div(g.M, 32), 4 * TS_NT_PAIRS);
+    if (blocks >= (size_t(1) << 31))
+        return dh_fail(DH_ERR_RUNTIME, "MatMul: too many rows for one launch of the streaming kernel");
     hipLaunchKernelGGL((ts_nt_kernel<T, NB, ASSIGN, CPG>), dim3(static_cast<unsigned>(blocks)), dim3(256), lds, ctx->stream, g);
     return DH_OK;
 }
