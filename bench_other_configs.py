@@ -130,7 +130,7 @@ def run(args) -> int:
     import torch
 
     sys.path.insert(0, os.path.join(os.path.dirname(os.path.abspath(__file__)), "tests"))
-    from daphne_amd.kernels import DenseMatrix, HIPContext, kmeansAssign, kmeansUpdate, matMul, normalEquations, solve, syrk
+    from daphne_amd.kernels import DenseMatrix, HIPContext, kmeansAssign, kmeansStep, kmeansUpdate, matMul, normalEquations, solve, syrk
     from daphne_amd.workloads import KMeans, lenet_forward, lmds
 
     if not torch.cuda.is_available():
@@ -205,7 +205,9 @@ def run(args) -> int:
 
         # (an iteration is 0.2 ms: a few dozen of them pass before the device has left its idle clocks)
         ms = _timed(torch, step, args.steps, max(args.warmup, 30))
+        ms_two = _timed(torch, lambda: step("two_passes"), args.steps, args.warmup)
         ms_seq = _timed(torch, lambda: step(False), min(args.steps, 15), args.warmup)
+        t_step = _events(torch, lambda: kmeansStep(km.idx, bufs[state["next"]], X, state["C"], km.xx, km.cc, ctx, km.counts))
         t_assign = _events(torch, lambda: kmeansAssign(km.idx, X, state["C"], km.xx, km.cc, ctx))
         t_update = _events(torch, lambda: kmeansUpdate(bufs[state["next"]], X, km.idx, k, ctx, km.counts))
         # canonical bytes per iteration: X C^T (read X, write D), D assembly 3 x |D|, idxmin (read D, write idx),
@@ -238,18 +240,20 @@ def run(args) -> int:
             cpu = {"value": round(nbytes / dt / 1e9, 4), "unit": "GB/s", "cores": threads, "kind": "port",
                    "sample": f"one iteration on all {n} rows, {threads} threads: products by numpy's {_blas_name()} sgemm, the other "
                              f"operators by the port's scalar kernels on row pieces ({dt:.2f} s)"}
-        assign_bytes = n * f * 4 + n * 4 + n * 8  # X, xx, idx
-        fused_bytes = assign_bytes + n * f * 4 + n * 8  # and X, idx once more
-        roof = {"bound": "hbm", "kernel": "ts_nt_kernel<float,1,true,4> (assignment: X t(C), distances and row arg-min in one pass over X)",
-                "achieved": round(assign_bytes / t_assign / 1e6, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(assign_bytes / t_assign / 1e6 / HBM_PEAK_GBS, 4), "traffic": None}
+        step_bytes = n * f * 4 + n * 4 + n * 8  # X, xx, idx
+        step_flops = 2 * 2.0 * n * f * k      # X t(C) and t(P) X
+        roof = {"bound": "hbm", "kernel": "ts_nt_kernel<float,1,true,4,true> + kmeans_finish_kernel (one pass over X: X t(C), distances, "
+                                          "row arg-min, t(one-hot) X and sizes)",
+                "achieved": round(step_bytes / t_step / 1e6, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(step_bytes / t_step / 1e6 / HBM_PEAK_GBS, 4), "traffic": None,
+                "mfma_tflops": round(step_flops / t_step / 1e9, 1)}
         out = _line(nbytes / ms / 1e6, "GB/s", ms, args, "f32",
                     "k-means Lloyd iteration: X 2000000x64 f32 (16 Gaussians), C 16x64; step = one iteration "
-                    "(two passes over X: assignment, update)",
-                    roof, cpu, {"canonical_bytes_per_step": nbytes, "bytes_per_step_two_passes": fused_bytes,
-                                "two_pass_gbs": round(fused_bytes / ms / 1e6, 1), "assign_ms": round(t_assign, 4),
-                                "update_ms": round(t_update, 4), "xct_ms": round(t_gemm, 4),
-                                "ms_per_step_operator_sequence": round(ms_seq, 4)})
+                    "(one pass over X: assignment and update from the same loads)",
+                    roof, cpu, {"canonical_bytes_per_step": nbytes, "bytes_per_step_one_pass": step_bytes,
+                                "one_pass_gbs": round(step_bytes / ms / 1e6, 1), "step_kernels_ms": round(t_step, 4),
+                                "assign_ms": round(t_assign, 4), "update_ms": round(t_update, 4), "xct_ms": round(t_gemm, 4),
+                                "ms_per_step_two_passes": round(ms_two, 4), "ms_per_step_operator_sequence": round(ms_seq, 4)})
     elif args.config == 4:
         res = measure_contractions(torch, ctx, args.steps, args.warmup)
         cpu = None

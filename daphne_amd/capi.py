@@ -114,6 +114,7 @@ _LATE_SIGNATURES: dict[str, list] = {
     "dh_normal_equations": [vp, vp, sz, vp, sz, vp, sz, sz, sz, vp, sz, "T"],
     "dh_kmeans_assign": [vp, vp, vp, sz, sz, sz, vp, sz, sz, vp, vp],
     "dh_kmeans_update": [vp, vp, sz, vp, vp, sz, sz, sz, vp, sz],
+    "dh_kmeans_step": [vp, vp, vp, sz, vp, vp, sz, sz, sz, vp, sz, sz, vp, vp],
     "dh_conv2d_forward": [vp, vp, C.POINTER(sz), C.POINTER(sz), vp, vp, sz, sz, vp, sz, sz, sz, sz, sz, sz, sz, sz, sz, sz],
     "dh_conv2d_forward_fused": [vp, vp, C.POINTER(sz), C.POINTER(sz), vp, vp, sz, sz, vp, sz, sz, sz, sz, sz, sz, sz, sz, sz, sz,
                                 C.c_uint],

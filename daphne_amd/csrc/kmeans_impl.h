@@ -341,4 +341,55 @@ dh_status update(dh_ctx *ctx, T *Cn, size_t ldc, T *counts, const T *X, size_t r
     return DH_OK;
 }
 
+// assign and update in one pass over X where the one-pass kernel exists (float, 49..64 features, 16-byte rows), else
+// one after the other; idx, C_new and counts as those two give them (C_new to rounding: other order of addition)
+template <typename T>
+dh_status step(dh_ctx *ctx, unsigned long long *idx, T *Cn, size_t ldcn, T *counts, const T *X, size_t rows, size_t cols, size_t ldx,
+               const T *C, size_t k, size_t ldc, const T *xx, const T *cc) {
+    DH_REQUIRE_CTX(ctx);
+    if constexpr (sizeof(T) == 4) {
+        constexpr int V = 4, KC = 16;
+        const size_t kpad = dh_ceil_div(cols, KC) * KC;
+        if (rows > 0 && k >= 1 && k <= 32 && kpad == 64 && dh_aligned(X, 16) && dh_aligned(C, 16) && ldx % V == 0 && ldc % V == 0 &&
+            cols % V == 0 && ldx >= cols && ldc >= cols && ldcn >= cols && ldx * sizeof(T) < (size_t(1) << 24)) {
+            const int nb = k <= 16 ? 1 : 2;
+            TsNtArgs g{};
+            g.A = X;
+            g.B = C;
+            g.lda = ldx;
+            g.ldb = ldc;
+            g.M = rows;
+            g.n = static_cast<unsigned>(k);
+            g.K = static_cast<unsigned>(cols);
+            g.kpad = static_cast<unsigned>(kpad);
+            g.row_add = xx;
+            g.col_add = cc;
+            g.idx = idx;
+            size_t blocks = 0;
+            dh_status st = nb == 1 ? dh_gemm::ts_nt_update_launch<T, 1>(ctx, g, &blocks) : dh_gemm::ts_nt_update_launch<T, 2>(ctx, g, &blocks);
+            if (st != DH_OK)
+                return st;
+            const size_t kp = static_cast<size_t>(nb) * 16;
+            void *wsv = nullptr;
+            st = dh_workspace(ctx, blocks * (kp * cols + kp) * sizeof(T), &wsv);
+            if (st != DH_OK)
+                return st;
+            g.slabs = wsv;
+            st = nb == 1 ? dh_gemm::ts_nt_update_launch<T, 1>(ctx, g, &blocks) : dh_gemm::ts_nt_update_launch<T, 2>(ctx, g, &blocks);
+            if (st != DH_OK)
+                return st;
+            DH_CHECK_LAUNCH();
+            hipLaunchKernelGGL((kmeans_finish_kernel<T>), dim3(static_cast<unsigned>(dh_ceil_div(k * cols, 8))), dim3(256), 0, ctx->stream, Cn,
+                               ldcn, counts, static_cast<const T *>(wsv), static_cast<unsigned>(blocks), static_cast<unsigned>(kp),
+                               static_cast<unsigned>(k), static_cast<unsigned>(cols));
+            DH_CHECK_LAUNCH();
+            return DH_OK;
+        }
+    }
+    dh_status st = assign<T>(ctx, idx, X, rows, cols, ldx, C, k, ldc, xx, cc);
+    if (st != DH_OK)
+        return st;
+    return update<T>(ctx, Cn, ldcn, counts, X, rows, cols, ldx, idx, k);
+}
+
 } // namespace dh_kmeans

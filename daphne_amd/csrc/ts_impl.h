@@ -366,6 +366,9 @@ struct TsNtArgs {
     // ASSIGN: instead of C, the first position of the row minimum of (C * -2 + row_add[row]) + col_add[col]
     const void *row_add, *col_add;
     unsigned long long *idx;
+    // UPDATE: besides, the sums of the rows of each position (the rows of t(one-hot(idx)) A) and their numbers, one
+    // partial result per workgroup: slabs[block][16 NB][K], then sizes[block][16 NB]
+    void *slabs;
 };
 
 // NB column blocks of 16; each wave walks over row blocks of 16, two at a time, CPG chunks of k at a time (1, 2 or 4:
@@ -373,7 +376,14 @@ struct TsNtArgs {
 // ASSIGN: the product is not stored; it goes on, rounded exactly as the stored one would be, into the distance
 // (C * -2 + row_add[row]) + col_add[col] (three separately rounded operations) and the row's IDXMIN over it: the first
 // position of the strict minimum, NaN never better, position 0 if the first value is NaN or all are.
-template <typename T, int NB, bool ASSIGN, int CPG> __global__ __launch_bounds__(256) void ts_nt_kernel(TsNtArgs g) {
+// UPDATE (with ASSIGN; float, one step per pair of row blocks with four chunks, i.e. 49..64 columns): the rows, still in
+// the registers they were loaded into - lane group h on row 4 c + h, lane i on vector i, the operand layout of
+// t(P) X - go through the matrix instruction once more against the one-hot of the assignment just found, so that one
+// pass over A gives the assignment, the per-position sums and the counts. The grid is then what the device holds at
+// once (one partial result per workgroup) and deals the pairs round-robin.
+template <typename T, int NB, bool ASSIGN, int CPG, bool UPDATE = false>
+__global__ __launch_bounds__(256) void ts_nt_kernel(TsNtArgs g) {
+    static_assert(!UPDATE || (ASSIGN && sizeof(T) == 4 && CPG == 4), "the one-pass form exists for float and 49..64 columns");
     using M = Mfma16<T>;
     constexpr int V = 16 / sizeof(T);
     constexpr int KC = 4 * V;     // k values per chunk
@@ -415,10 +425,15 @@ template <typename T, int NB, bool ASSIGN, int CPG> __global__ __launch_bounds__
     const unsigned chunks = g.kpad / KC;
     const unsigned cg = chunks / CPG;                // chunk groups per row-block pair (CPG divides chunks)
     const size_t total_pairs = (g.M + 31) / 32;
-    const size_t first_pair = (static_cast<size_t>(blockIdx.x) * 4 + wave) * TS_NT_PAIRS, pair_stride = 1;
-    const unsigned my_pairs = first_pair < total_pairs
-                                  ? static_cast<unsigned>(total_pairs - first_pair < TS_NT_PAIRS ? total_pairs - first_pair : TS_NT_PAIRS)
-                                  : 0;
+    const size_t first_pair = (static_cast<size_t>(blockIdx.x) * 4 + wave) * (UPDATE ? 1 : TS_NT_PAIRS);
+    const size_t pair_stride = UPDATE ? static_cast<size_t>(gridDim.x) * 4 : 1;
+    unsigned my_pairs = 0;
+    if (first_pair < total_pairs) {
+        if constexpr (UPDATE)
+            my_pairs = static_cast<unsigned>((total_pairs - 1 - first_pair) / pair_stride) + 1;
+        else
+            my_pairs = static_cast<unsigned>(total_pairs - first_pair < TS_NT_PAIRS ? total_pairs - first_pair : TS_NT_PAIRS);
+    }
     const unsigned nsteps = my_pairs * cg;
     constexpr int RPL = SWAP ? 1 : 4; // ASSIGN: rows per lane and row block in the result layout
     struct Frag {
@@ -509,7 +524,20 @@ template <typename T, int NB, bool ASSIGN, int CPG> __global__ __launch_bounds__
             }
         }
     };
-    auto finish_pair = [&](AccSet &acc, unsigned pair, const T (&radd)[2][RPL]) {
+    // UPDATE: per-position sums (register v of lane (i, h), instruction e: position 16 a + 4 h + v, column 4 i + e) and counts
+    typename M::acc_t acc_s[UPDATE ? NB : 1][V];
+    T cnt[UPDATE ? NB : 1];
+    __shared__ __attribute__((aligned(16))) unsigned ridx[UPDATE ? 4 * 32 : 4];
+    if constexpr (UPDATE) {
+#pragma unroll
+        for (int a = 0; a < NB; a++) {
+            cnt[a] = T(0);
+#pragma unroll
+            for (int e = 0; e < V; e++)
+                acc_s[a][e] = typename M::acc_t{0, 0, 0, 0};
+        }
+    }
+    auto finish_pair = [&](AccSet &acc, unsigned pair, const T (&radd)[2][RPL], const Frag &fr) {
         const size_t rbase = (first_pair + static_cast<size_t>(pair) * pair_stride) * 32;
         if constexpr (ASSIGN) {
 #pragma clang fp contract(off)
@@ -555,37 +583,62 @@ template <typename T, int NB, bool ASSIGN, int CPG> __global__ __launch_bounds__
                     take(best[t], bi[t], dh_peer_swap<32>{}(best[t]), dh_peer_swap<32>{}(bi[t]));
                     odd |= (sum[t] != sum[t]) || !(best[t] < dh_inf<T>());
                 }
-                if (__ballot(odd) == 0) {
+                if (__ballot(odd) != 0) {
+                    // the long way, with IDXMIN's rules spelled out (bi is the answer in the lanes h = 0 at least)
 #pragma unroll
                     for (int t = 0; t < 2; t++) {
-                        const size_t row = rbase + static_cast<size_t>(t) * 16 + i;
-                        if (h == 0 && row < g.M)
-                            g.idx[row] = bi[t];
+                        T best1 = dh_inf<T>(), first = T(0);
+                        unsigned bi1 = NONE;
+#pragma unroll
+                        for (int b = 0; b < NB; b++)
+#pragma unroll
+                            for (int v = 0; v < 4; v++) {
+                                const unsigned col = b * 16 + 4 * h + v;
+                                const T dv = d[t][b][v];
+                                if (b == 0 && v == 0)
+                                    first = dv; // column 0 in the lanes h = 0
+                                if (col < g.n && (dv < best1 || (bi1 == NONE && !(dv != dv)))) {
+                                    best1 = dv;
+                                    bi1 = col;
+                                }
+                            }
+                        take(best1, bi1, dh_peer_swap<16>{}(best1), dh_peer_swap<16>{}(bi1));
+                        take(best1, bi1, dh_peer_swap<32>{}(best1), dh_peer_swap<32>{}(bi1));
+                        bi[t] = ((first != first) || bi1 == NONE) ? 0u : bi1;
                     }
-                    return;
                 }
 #pragma unroll
                 for (int t = 0; t < 2; t++) {
                     const size_t row = rbase + static_cast<size_t>(t) * 16 + i;
-                    T best1 = dh_inf<T>(), first = T(0);
-                    unsigned bi1 = NONE;
-#pragma unroll
-                    for (int b = 0; b < NB; b++)
-#pragma unroll
-                        for (int v = 0; v < 4; v++) {
-                            const unsigned col = b * 16 + 4 * h + v;
-                            const T dv = d[t][b][v];
-                            if (b == 0 && v == 0)
-                                first = dv; // column 0 in the lanes h = 0
-                            if (col < g.n && (dv < best1 || (bi1 == NONE && !(dv != dv)))) {
-                                best1 = dv;
-                                bi1 = col;
-                            }
-                        }
-                    take(best1, bi1, dh_peer_swap<16>{}(best1), dh_peer_swap<16>{}(bi1));
-                    take(best1, bi1, dh_peer_swap<32>{}(best1), dh_peer_swap<32>{}(bi1));
                     if (h == 0 && row < g.M)
-                        g.idx[row] = ((first != first) || bi1 == NONE) ? 0ull : static_cast<unsigned long long>(bi1);
+                        g.idx[row] = bi[t];
+                }
+                if constexpr (UPDATE) {
+                    // the assignment goes to the lanes that hold the rows as rows: row r of the pair at entry 8 (r % 4) +
+                    // r / 4 of the wave's 32, so that lane group h finds its rows 4 c + h (c = 0 .. 7) side by side
+                    unsigned *mine = ridx + wave * 32;
+                    if (h == 0) {
+#pragma unroll
+                        for (int t = 0; t < 2; t++) {
+                            const unsigned r = t * 16 + i;
+                            mine[8 * (r % 4) + r / 4] = rbase + r < g.M ? bi[t] : NONE; // rows beyond M belong nowhere
+                        }
+                    }
+                    unsigned of_row[2][4];
+                    dh_load_vec<unsigned, 4>(mine + 8 * h, of_row[0]);
+                    dh_load_vec<unsigned, 4>(mine + 8 * h + 4, of_row[1]);
+#pragma unroll
+                    for (int t = 0; t < 2; t++)
+#pragma unroll
+                        for (int c = 0; c < 4; c++)
+#pragma unroll
+                            for (int a = 0; a < NB; a++) {
+                                const T p = of_row[t][c] == static_cast<unsigned>(a * 16 + i) ? T(1) : T(0);
+                                cnt[a] += p;
+#pragma unroll
+                                for (int e = 0; e < V; e++)
+                                    acc_s[a][e] = M::mma(p, fr.a[t][c][e], acc_s[a][e]);
+                            }
                 }
             } else {
                 // register v of lane (i, h) is C[row 4 v + h][column 16 b + i]: a row's values sit in the sixteen lanes of a group
@@ -654,7 +707,7 @@ template <typename T, int NB, bool ASSIGN, int CPG> __global__ __launch_bounds__
     auto compute_step = [&](const Frag &fr, unsigned pair, unsigned grp) {
         mma_step(accA, fr, grp);
         if (grp + 1 == cg)
-            finish_pair(accA, pair, fr.ra);
+            finish_pair(accA, pair, fr.ra, fr);
     };
     // (pair, grp) of a step and of the one after it, stepped without divisions
     auto advance = [&](unsigned &pair, unsigned &grp) {
@@ -711,22 +764,22 @@ template <typename T, int NB, bool ASSIGN, int CPG> __global__ __launch_bounds__
             load_step(f0, sdone + 1, 0);
             __builtin_amdgcn_sched_barrier(0);
             mma_step(accB, f1, 0);
-            finish_pair(accA, sdone - 1, ra0);
+            finish_pair(accA, sdone - 1, ra0, f0);
             keep(ra1, f1);
             __builtin_amdgcn_sched_barrier(0);
             load_step(f1, sdone + 2 < nsteps ? sdone + 2 : nsteps - 1, 0);
             __builtin_amdgcn_sched_barrier(0);
             mma_step(accA, f0, 0);
-            finish_pair(accB, sdone, ra1);
+            finish_pair(accB, sdone, ra1, f0);
             keep(ra0, f0);
             __builtin_amdgcn_sched_barrier(0);
         }
         if (sdone < nsteps) {
             mma_step(accB, f1, 0);
-            finish_pair(accA, sdone - 1, ra0);
-            finish_pair(accB, sdone, f1.ra);
+            finish_pair(accA, sdone - 1, ra0, f0);
+            finish_pair(accB, sdone, f1.ra, f1);
         } else {
-            finish_pair(accA, sdone - 1, ra0);
+            finish_pair(accA, sdone - 1, ra0, f0);
         }
         return;
     }
@@ -744,6 +797,61 @@ template <typename T, int NB, bool ASSIGN, int CPG> __global__ __launch_bounds__
             compute_step(f1, cp, cgp);
         __builtin_amdgcn_sched_barrier(0);
         advance(cp, cgp);
+    }
+    if constexpr (UPDATE) {
+        // counts: the four lane groups of a wave counted different rows; then the four waves, added in wave order
+#pragma unroll
+        for (int a = 0; a < NB; a++) {
+            cnt[a] += dh_peer_swap<16>{}(cnt[a]);
+            cnt[a] += dh_peer_swap<32>{}(cnt[a]);
+        }
+        constexpr int NVAL = NB * V * 4 + NB;
+        __shared__ __attribute__((aligned(16))) T red[NVAL][64];
+        for (int w = 1; w < 4; w++) {
+            if (wave == w) {
+                int q = 0;
+#pragma unroll
+                for (int a = 0; a < NB; a++) {
+#pragma unroll
+                    for (int e = 0; e < V; e++)
+#pragma unroll
+                        for (int v = 0; v < 4; v++)
+                            red[q++][lane] = acc_s[a][e][v];
+                    red[q++][lane] = cnt[a];
+                }
+            }
+            __syncthreads();
+            if (wave == 0) {
+                int q = 0;
+#pragma unroll
+                for (int a = 0; a < NB; a++) {
+#pragma unroll
+                    for (int e = 0; e < V; e++)
+#pragma unroll
+                        for (int v = 0; v < 4; v++)
+                            acc_s[a][e][v] += red[q++][lane];
+                    cnt[a] += red[q++][lane];
+                }
+            }
+            __syncthreads();
+        }
+        if (wave != 0)
+            return;
+        T *slab = static_cast<T *>(g.slabs) + static_cast<size_t>(blockIdx.x) * (NB * 16) * g.K;
+        T *sizes = static_cast<T *>(g.slabs) + static_cast<size_t>(gridDim.x) * (NB * 16) * g.K + static_cast<size_t>(blockIdx.x) * (NB * 16);
+#pragma unroll
+        for (int a = 0; a < NB; a++) {
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                const unsigned cen = a * 16 + M::row(lane, v);
+#pragma unroll
+                for (int e = 0; e < V; e++)
+                    if (static_cast<unsigned>(V * i + e) < g.K)
+                        slab[static_cast<size_t>(cen) * g.K + V * i + e] = acc_s[a][e][v];
+            }
+            if (h == 0)
+                sizes[a * 16 + i] = cnt[a];
+        }
     }
 }
 
@@ -868,6 +976,26 @@ inline dh_status ts_nt_launch_cpg(dh_ctx *ctx, const TsNtArgs &g, size_t lds) {
     hipLaunchKernelGGL((ts_nt_kernel<T, NB, ASSIGN, CPG>), dim3(static_cast<unsigned>(blocks)), dim3(256), lds, ctx->stream, g);
     return DH_OK;
 }
+// The one-pass form (UPDATE): a grid of as many workgroups as the device holds at once; *blocks_out receives their
+// number (that of the partial results in g.slabs, which must hold blocks * (16 NB K + 16 NB) values: ask with
+// g.slabs == nullptr first).
+template <typename T, int NB> inline dh_status ts_nt_update_launch(dh_ctx *ctx, const TsNtArgs &g, size_t *blocks_out) {
+    const void *kernel = reinterpret_cast<const void *>(&ts_nt_kernel<T, NB, true, 4, true>);
+    const size_t lds = ts_nt_lds_bytes<T>(NB, g.kpad, 4);
+    // three workgroups per CU (measured 2 .. 8: flat within 5 %, best at 3 .. 4; registers and LDS allow four)
+    (void)kernel;
+    constexpr int per_cu = 3;
+    size_t blocks = static_cast<size_t>(ctx->num_cus) * per_cu;
+    const size_t needed = dh_ceil_div(dh_ceil_div(g.M, 32), 4 * 2); // at least two pairs per wavefront
+    if (blocks > needed)
+        blocks = needed > 0 ? needed : 1;
+    *blocks_out = blocks;
+    if (g.slabs == nullptr)
+        return DH_OK;
+    hipLaunchKernelGGL((ts_nt_kernel<T, NB, true, 4, true>), dim3(static_cast<unsigned>(blocks)), dim3(256), lds, ctx->stream, g);
+    return DH_OK;
+}
+
 template <typename T, int NB, bool ASSIGN> inline dh_status ts_nt_launch(dh_ctx *ctx, const TsNtArgs &g) {
     const int cpg = ts_nt_chunks_per_step<T>(g.kpad);
     const size_t lds = ts_nt_lds_bytes<T>(NB, g.kpad, cpg);

@@ -358,6 +358,25 @@ def kmeansUpdate(C_new, X: DenseMatrix, idx: DenseMatrix, k: int, ctx: HIPContex
     return C_new, counts
 
 
+def kmeansStep(idx, C_new, X: DenseMatrix, C: DenseMatrix, xx: DenseMatrix, cc: DenseMatrix, ctx: HIPContext,
+               counts: Optional[DenseMatrix] = None):
+    """kmeansAssign and kmeansUpdate as one call (dh_kmeans_step_*): one pass over X where the library has a kernel for
+    it (float, 49 to 64 features), the two passes elsewhere. Returns (idx, C_new, counts)."""
+    dt = _same_dtype(X, C, xx, cc)
+    k = C.rows
+    if C.cols != X.cols or xx.getNumItems() != X.rows or cc.getNumItems() != k:
+        raise capi.DaphneHipError(1, "kmeansStep: C must have X's columns, xx one value per row of X, cc one per centroid")
+    if idx is None:
+        idx = DenseMatrix(ctx, X.rows, 1, np.uint64)
+    if C_new is None:
+        C_new = DenseMatrix(ctx, k, X.cols, dt)
+    if counts is None:
+        counts = DenseMatrix(ctx, 1, k, dt)
+    capi.check(_fn("dh_kmeans_step", dt)(ctx._h, idx.ptr, C_new.ptr, C_new.row_skip, counts.ptr, X.ptr, X.rows, X.cols, X.row_skip,
+                                         C.ptr, k, C.row_skip, xx.ptr, cc.ptr))
+    return idx, C_new, counts
+
+
 def solve(res, lhs: DenseMatrix, rhs: DenseMatrix, ctx: HIPContext) -> DenseMatrix:
     """CUDA::solve (kernels/CUDA/Solve.h; CPU kernels/Solve.h:86-116): A x = b by LU."""
     dt = _same_dtype(lhs, rhs, res)

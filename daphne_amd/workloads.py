@@ -7,7 +7,7 @@ from __future__ import annotations
 import numpy as np
 
 from .kernels import (AggOpCode, BinaryOpCode, DenseMatrix, HIPContext, UnaryOpCode, affineForward, affineForwardFused, aggCol,
-                      aggRow, conv2dForward, conv2dForwardFused, kmeansAssign, kmeansUpdate, ewBinaryMat, ewBinaryObjSca, ewUnaryMat, matMul, maxPoolForward, normalEquations, softmax, solve,
+                      aggRow, conv2dForward, conv2dForwardFused, kmeansAssign, kmeansStep, kmeansUpdate, ewBinaryMat, ewBinaryObjSca, ewUnaryMat, matMul, maxPoolForward, normalEquations, softmax, solve,
                       syrk)
 from .pipeline import ROWREG, SELF, VectorizedPipeline
 
@@ -70,17 +70,20 @@ class KMeans:
         self.PtX = DenseMatrix(ctx, k, X.cols, dt)
         self.counts = DenseMatrix(ctx, 1, k, dt)
 
-    def iterate(self, C: DenseMatrix, C_out: DenseMatrix | None = None, fused: bool = True) -> DenseMatrix:
-        """fused: two passes over X (kmeansAssign, kmeansUpdate); else one kernel per operator (or fused pipeline of
-        elementwise operators), with XC, the one-hot P and t(P) X in memory. self.idx holds the assignment either way."""
+    def iterate(self, C: DenseMatrix, C_out: DenseMatrix | None = None, fused=True) -> DenseMatrix:
+        """fused True: kmeansStep (one pass over X for 49 to 64 float features, two elsewhere); "two_passes":
+        kmeansAssign then kmeansUpdate; False: one kernel per operator (or fused pipeline of elementwise operators), with
+        XC, the one-hot P and t(P) X in memory. self.idx holds the assignment either way."""
         ctx, X, k = self.ctx, self.X, self.k
         pc = VectorizedPipeline(ctx, C)
         pc.ewBinary(BinaryOpCode.MUL, SELF).rowAgg(AggOpCode.SUM)
         pc.storeRow(self.cc)
         pc.run()                                                       # rowSums(C^2), k x 1
-        if fused:
+        if fused == "two_passes":
             kmeansAssign(self.idx, X, C, self.xx, self.cc, ctx)
             return kmeansUpdate(C_out, X, self.idx, k, ctx, self.counts)[0]
+        if fused:
+            return kmeansStep(self.idx, C_out, X, C, self.xx, self.cc, ctx, self.counts)[1]
         matMul(self.XC, X, C, False, True, ctx)                       # X @ t(C)
         cc_row = DenseMatrix(ctx, 1, k, C.dtype, ptr=self.cc.ptr, keepalive=self.cc)  # the same k values as 1 x k
         p = VectorizedPipeline(ctx, self.XC)

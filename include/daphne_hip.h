@@ -288,6 +288,18 @@ dh_status dh_kmeans_update_f64(dh_ctx *ctx, double *C_new, size_t ld_new, double
                                const double *X, size_t rows, size_t cols, size_t ldx,
                                const uint64_t *idx, size_t k);
 
+/* dh_kmeans_assign followed by dh_kmeans_update, in one pass over X where the library has a kernel for
+ * it (float, 49 to 64 features: a row, once loaded, serves the distances and then the sums), as the two
+ * calls one after the other elsewhere. idx as dh_kmeans_assign gives it; C_new and counts as
+ * dh_kmeans_update gives them (C_new to rounding: the rows are added in another order). Arguments,
+ * limits and errors of the two calls. */
+dh_status dh_kmeans_step_f32(dh_ctx *ctx, uint64_t *idx, float *C_new, size_t ld_new, float *counts,
+                             const float *X, size_t rows, size_t cols, size_t ldx, const float *C,
+                             size_t k, size_t ldc, const float *xx, const float *cc);
+dh_status dh_kmeans_step_f64(dh_ctx *ctx, uint64_t *idx, double *C_new, size_t ld_new, double *counts,
+                             const double *X, size_t rows, size_t cols, size_t ldx, const double *C,
+                             size_t k, size_t ldc, const double *xx, const double *cc);
+
 /* ------------------------------------------------------------------------------------ */
 /* DNN inference ops (NCHW images flattened to rows: one image per matrix row)           */
 /* ------------------------------------------------------------------------------------ */

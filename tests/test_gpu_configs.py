@@ -79,7 +79,7 @@ def _orc_kmeans_iter(X, C, xx):
     return orc.ew_binary(BinaryOpCode.DIV, PtX, np.ascontiguousarray(cnt.T))[1], idx, D
 
 
-@pytest.mark.parametrize("fused", [True, False], ids=["two_passes", "operator_sequence"])
+@pytest.mark.parametrize("fused", [True, "two_passes", False], ids=["one_pass", "two_passes", "operator_sequence"])
 def test_config3_kmeans_against_oracle(ctx, fused):
     """Mixture of 16 Gaussians, 10 Lloyd iterations at an oracle-feasible size; indices bit-exact on rows
     whose two smallest distances are not a near-tie (the GEMMs sum in different orders), centroids 1e-4."""
@@ -123,6 +123,10 @@ def test_config3_full_size_properties(ctx):
     # (the product comes from the same streaming kernel), the same sizes, centroids to rounding
     C_seq = km.iterate(C, fused=False)
     idx_seq, counts_seq = km.idx.to_numpy().copy(), km.counts.to_numpy().copy()
+    C2 = km.iterate(C, fused="two_passes")
+    assert_exact(km.idx.to_numpy(), idx_seq)
+    assert_exact(km.counts.to_numpy(), counts_seq)
+    assert_close(C2.to_numpy(), C_seq.to_numpy(), rtol=1e-5, elementwise=False)
     C = km.iterate(C)
     assert_exact(km.idx.to_numpy(), idx_seq)
     assert_exact(km.counts.to_numpy(), counts_seq)

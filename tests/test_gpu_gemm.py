@@ -15,7 +15,7 @@ pytestmark = pytest.mark.gpu
 
 from daphne_amd import capi
 from daphne_amd.kernels import (AggOpCode, BinaryOpCode, DenseMatrix, affineForward, affineForwardFused, aggRow, ewBinaryMat,
-                                ewBinaryObjSca, kmeansAssign, kmeansUpdate, matMul, reluForward, solve, syrk)
+                                ewBinaryObjSca, kmeansAssign, kmeansStep, kmeansUpdate, matMul, reluForward, solve, syrk)
 
 DTYPES = [np.float32, np.float64]
 
@@ -405,7 +405,7 @@ def test_normal_equations_of_other_shapes(ctx, dt, rows, cols):
 
 KMEANS_SHAPES = [  # rows, cols, k
     (1, 4, 1), (7, 8, 3), (100, 64, 16), (513, 64, 16), (70_000, 64, 16), (66_000, 32, 32), (65_600, 12, 17), (3000, 200, 5),
-    (2049, 128, 20), (131_072, 4, 2),
+    (2049, 128, 20), (131_072, 4, 2), (33, 52, 2), (300_001, 60, 30), (1_000_000, 64, 7),
 ]
 
 
@@ -452,6 +452,11 @@ def test_kmeans_assign_and_update(ctx, dt, rows, cols, k):
             kmeansUpdate(None, X, DenseMatrix.from_numpy(ctx, idx), k, ctx)
         return
     Cn, counts = kmeansUpdate(None, X, DenseMatrix.from_numpy(ctx, idx), k, ctx)
+    # both passes as one call (one pass over X for 49 to 64 float features): the same assignment and sizes bit for bit
+    idx1, Cn1, counts1 = kmeansStep(None, None, X, C, xx, cc, ctx)
+    assert_exact(idx1.to_numpy(), idx)
+    assert_exact(counts1.to_numpy(), counts.to_numpy())
+    assert_close(Cn1.to_numpy(), Cn.to_numpy(), rtol=2e-5 if dt == np.float32 else 1e-12, elementwise=False)
     cnt = np.bincount(idx[:, 0].astype(np.int64), minlength=k).astype(np.float64)
     assert_exact(counts.to_numpy()[0].astype(np.float64), cnt)
     sums = np.zeros((k, cols))
