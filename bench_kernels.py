@@ -210,6 +210,11 @@ def main() -> int:
             big = DM.from_torch(ctx, torch.randn(1_000_000, 10, device="cuda", dtype=tdt, generator=gen))
             sm = DM(ctx, 1_000_000, 10, ndt)
             emit("softmax 10 classes", dt, "1000000x10", timed(lambda: K.softmax(sm, big, ctx)), 2 * 10_000_000 * sz)
+            for m in (big, sm):
+                m.destroy()
+            big = DM.from_torch(ctx, torch.randn(16_000_000, 10, device="cuda", dtype=tdt, generator=gen))
+            sm = DM(ctx, 16_000_000, 10, ndt)
+            emit("softmax 10 classes", dt, "16000000x10", timed(lambda: K.softmax(sm, big, ctx)), 2 * 160_000_000 * sz)
             for m in (x2, w2, b2, o2, one, pl, w3, b3, h3, big, sm):
                 m.destroy()
         # --- DNN training kernels ---------------------------------------------------------------------------------

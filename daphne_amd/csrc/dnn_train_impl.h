@@ -66,7 +66,7 @@ __global__ __launch_bounds__(THREADS) void chan_stage1(const T *x, const T *dy, 
             for (int u = 0; u < UN; u++) {
                 valid[u] = n < imgs;
                 const size_t off = (valid[u] ? n : imgs - 1) * CHW + j * VEC;
-                dh_load_vec_stream<T, VEC>(xc + off, v[u]);
+                dh_load_vec<T, VEC>(xc + off, v[u]); // read again by the elementwise pass: no streaming hint
                 if constexpr (MODE == 2)
                     dh_load_vec_stream<T, VEC>(gc + off, g[u]);
                 n += dn;
@@ -181,12 +181,14 @@ __global__ void chan_stage2(const double *partials, size_t C, size_t S, double m
 // Elementwise passes over the (N*C) x HW view. FWD: res = gamma * ((x - mean) / sd) + beta
 // (BatchNorm2DTrainForward.h:108-115). Else: dX = (dy * gamma) * inv_var + coef0 * (x - mean) + coef1
 // (BatchNorm2DBackward.h:110-118).
+// The rows are taken from the last to the first: the reduction pass before it went through x from the first image to
+// the last, so the end of x is what the memory-side cache still holds (8 % of the two passes' time at 4096 x 64 x 14 x 14).
 template <typename T, int VEC, bool FWD>
 __global__ __launch_bounds__(THREADS) void chan_apply(T *res, const T *x, const T *dy, size_t rows, size_t C, size_t HW,
                                                       const T *mean, const T *gamma, const T *beta, const T *inv_var,
                                                       const T *coef) {
     const size_t cvecs = HW / VEC;
-    const size_t r = static_cast<size_t>(blockIdx.x) * blockDim.y + threadIdx.y;
+    const size_t r = static_cast<size_t>(gridDim.x - 1 - blockIdx.x) * blockDim.y + threadIdx.y;
     if (r >= rows)
         return;
     // 32-bit remainder where the row count allows (uniform)
@@ -196,7 +198,7 @@ __global__ __launch_bounds__(THREADS) void chan_apply(T *res, const T *x, const 
     for (size_t cv = static_cast<size_t>(blockIdx.y) * blockDim.x + threadIdx.x; cv < cvecs;
          cv += static_cast<size_t>(gridDim.y) * blockDim.x) {
         T a[VEC], b[VEC], o[VEC];
-        dh_load_vec_stream<T, VEC>(x + r * HW + cv * VEC, a);
+        dh_load_vec<T, VEC>(x + r * HW + cv * VEC, a);
         if constexpr (!FWD)
             dh_load_vec_stream<T, VEC>(dy + r * HW + cv * VEC, b);
 #pragma unroll
