@@ -22,6 +22,8 @@
 
 #include "common.h"
 
+#include <type_traits>
+
 namespace dh_gemm {
 #ifndef TS_NT_PAIRS
 #define TS_NT_PAIRS 4 // pairs of 16-row blocks per wavefront of ts_nt_kernel
@@ -382,7 +384,7 @@ struct TsNtArgs {
 // pass over A gives the assignment, the per-position sums and the counts. The grid is then what the device holds at
 // once (one partial result per workgroup) and deals the pairs round-robin.
 template <typename T, int NB, bool ASSIGN, int CPG, bool UPDATE = false>
-__global__ __launch_bounds__(256) void ts_nt_kernel(TsNtArgs g) {
+__global__ __launch_bounds__(256, UPDATE ? (NB == 1 ? 3 : 2) : (ASSIGN && NB == 1 ? 4 : 1)) void ts_nt_kernel(TsNtArgs g) {
     static_assert(!UPDATE || (ASSIGN && sizeof(T) == 4 && CPG == 4), "the one-pass form exists for float and 49..64 columns");
     using M = Mfma16<T>;
     constexpr int V = 16 / sizeof(T);
@@ -393,7 +395,8 @@ __global__ __launch_bounds__(256) void ts_nt_kernel(TsNtArgs g) {
     constexpr bool SWAP = sizeof(T) == 4;
     extern __shared__ __attribute__((aligned(16))) unsigned char ts_nt_lds[];
     T *lb = reinterpret_cast<T *>(ts_nt_lds); // [NB*16][kpad + V], zero padded
-    const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
+    const int tid = threadIdx.x, lane = tid % 64;
+    const int wave = __builtin_amdgcn_readfirstlane(tid / 64); // the same in all lanes: addresses built on it stay scalar
     const int i = lane % 16, h = lane / 16;
     const T *A = static_cast<const T *>(g.A);
     const T *B = static_cast<const T *>(g.B);
@@ -480,7 +483,9 @@ __global__ __launch_bounds__(256) void ts_nt_kernel(TsNtArgs g) {
     // pair is finished - distances and arg-min, or the store - beside the matrix instructions of the next.
     using AccSet = typename M::acc_t[2][NB];
     AccSet accA, accB;
-    auto mma_step = [&](AccSet &acc, const Frag &fr, unsigned grp) {
+    const bool whole_chunks = g.K == g.kpad; // no k beyond K anywhere: nothing to zero
+    auto mma_step_k = [&](AccSet &acc, const Frag &fr, unsigned grp, auto full_k) {
+        constexpr bool FULLK = decltype(full_k)::value;
         if (grp == 0) {
 #pragma unroll
             for (int b = 0; b < NB; b++) {
@@ -504,7 +509,7 @@ __global__ __launch_bounds__(256) void ts_nt_kernel(TsNtArgs g) {
         for (int c = 0; c < CPG; c++) {
             const unsigned ch = grp * CPG + c;
             {
-                const bool kok = ch * KC + h * V < g.K;
+                const bool kok = FULLK || ch * KC + h * V < g.K;
 #pragma unroll
                 for (int b = 0; b < NB; b++) {
                     T fb[V];
@@ -524,6 +529,12 @@ __global__ __launch_bounds__(256) void ts_nt_kernel(TsNtArgs g) {
             }
         }
     };
+    auto mma_step = [&](AccSet &acc, const Frag &fr, unsigned grp) {
+        if (whole_chunks)
+            mma_step_k(acc, fr, grp, std::true_type{});
+        else
+            mma_step_k(acc, fr, grp, std::false_type{});
+    };
     // UPDATE: per-position sums (register v of lane (i, h), instruction e: position 16 a + 4 h + v, column 4 i + e) and counts
     typename M::acc_t acc_s[UPDATE ? NB : 1][V];
     T cnt[UPDATE ? NB : 1];
@@ -542,11 +553,10 @@ __global__ __launch_bounds__(256) void ts_nt_kernel(TsNtArgs g) {
         if constexpr (ASSIGN) {
 #pragma clang fp contract(off)
             constexpr unsigned NONE = ~0u;
-            auto take = [](T &best, unsigned &bi, T ov, unsigned oi) {
-                if (ov < best || (ov == best && oi < bi)) {
-                    best = ov;
-                    bi = oi;
-                }
+            auto take = [](T &best, unsigned &bi, T ov, unsigned oi) { // selects, no branches
+                const bool better = (ov < best) | ((ov == best) & (oi < bi));
+                best = better ? ov : best;
+                bi = better ? oi : bi;
             };
             if constexpr (SWAP) {
                 // register v of lane (i, h) is C[row i][column 16 b + 4 h + v]: a row's values sit in the four lanes i + 16 h
