@@ -17,9 +17,20 @@ HBM_PEAK_GBS = 8000.0
 MFMA_PEAK = {"f32": 157.3, "f64": 78.6}
 
 
+CLOCK_WARMUP_S = 0.25
+
+
 def _timed(torch, fn, steps, warmup):
-    for _ in range(warmup):
+    """Wall time per step in ms over `steps` steps, after `warmup` untimed ones and as many more untimed ones as it takes
+    to fill CLOCK_WARMUP_S: the device needs tens of milliseconds of continuous work to reach its clocks, which steps of
+    0.1 ms do not give it in a few dozen repetitions (k-means: 0.26 ms per iteration over the first 50 ms, 0.115 after)."""
+    t0 = time.perf_counter()
+    done = 0
+    while done < warmup or time.perf_counter() - t0 < CLOCK_WARMUP_S:
         fn()
+        done += 1
+        if done % 16 == 0:
+            torch.cuda.synchronize()  # keeps the host no more than 16 steps ahead, so that the clock above means device work
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(steps):
@@ -204,7 +215,7 @@ def run(args) -> int:
             state["C"] = km.iterate(state["C"], out, fused=fused)
 
         # (an iteration is 0.2 ms: a few dozen of them pass before the device has left its idle clocks)
-        ms = _timed(torch, step, args.steps, max(args.warmup, 30))
+        ms = _timed(torch, step, args.steps, args.warmup)
         ms_two = _timed(torch, lambda: step("two_passes"), args.steps, args.warmup)
         ms_seq = _timed(torch, lambda: step(False), min(args.steps, 15), args.warmup)
         t_step = _events(torch, lambda: kmeansStep(km.idx, bufs[state["next"]], X, state["C"], km.xx, km.cc, ctx, km.counts))

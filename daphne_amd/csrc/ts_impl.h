@@ -426,7 +426,8 @@ __global__ __launch_bounds__(256, UPDATE ? (NB == 1 ? 3 : 2) : (ASSIGN && NB == 
     // against a grid of resident workgroups that deal the pairs round-robin, this is as fast at 2M rows and 7 % faster
     // at 20M).
     const unsigned chunks = g.kpad / KC;
-    const unsigned cg = chunks / CPG;                // chunk groups per row-block pair (CPG divides chunks)
+    // chunk groups per row-block pair (CPG divides chunks); the one-pass form only exists for a single group
+    const unsigned cg = UPDATE ? 1u : chunks / CPG;
     const size_t total_pairs = (g.M + 31) / 32;
     const size_t first_pair = (static_cast<size_t>(blockIdx.x) * 4 + wave) * (UPDATE ? 1 : TS_NT_PAIRS);
     const size_t pair_stride = UPDATE ? static_cast<size_t>(gridDim.x) * 4 : 1;
