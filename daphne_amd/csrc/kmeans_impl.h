@@ -15,6 +15,7 @@ namespace dh_kmeans {
 
 using dh_gemm::Mfma16;
 using dh_gemm::ts_load;
+using dh_gemm::ts_load_nt;
 using dh_gemm::TsNtArgs;
 
 template <typename T>
@@ -106,7 +107,7 @@ __global__ __launch_bounds__(256) void kmeans_update_kernel(UpdateArgs g) {
         fr.id[u] = g.idx[rl];
 #pragma unroll
         for (int c = 0; c < CB; c++)
-            ts_load<T, V>(X + rl * g.ldx + col_ld[c], fr.x[u][c], true);
+            ts_load_nt<T, V>(X + rl * g.ldx + col_ld[c], fr.x[u][c]);
     };
     auto mma_quad = [&](const Frag &fr, int u, bool live) {
 #pragma unroll

@@ -52,14 +52,27 @@ template <> struct Mfma16<double> {
     static __device__ __forceinline__ int row(int lane, int v) { return 4 * v + (lane / 16); }
 };
 
-// V consecutive values; `stream` marks data that no other wave will ask for again
-template <typename T, int V> __device__ __forceinline__ void ts_load(const T *p, T (&v)[V], bool stream) {
+// V consecutive values
+template <typename T, int V> __device__ __forceinline__ void ts_load(const T *p, T (&v)[V]) {
     if constexpr (V == 1) {
-        v[0] = stream ? __builtin_nontemporal_load(p) : *p;
+        v[0] = *p;
     } else {
         typedef T vec_t __attribute__((ext_vector_type(V)));
-        const vec_t t = stream ? __builtin_nontemporal_load(reinterpret_cast<const vec_t *>(p))
-                               : *reinterpret_cast<const vec_t *>(p);
+        const vec_t t = *reinterpret_cast<const vec_t *>(p);
+#pragma unroll
+        for (int e = 0; e < V; e++)
+            v[e] = t[e];
+    }
+}
+
+// The same for data that no other wave will ask for again. (A separate function: a hint chosen by a flag, even a
+// literal one, is lost when the compiler merges the hinted and the plain load of one address.)
+template <typename T, int V> __device__ __forceinline__ void ts_load_nt(const T *p, T (&v)[V]) {
+    if constexpr (V == 1) {
+        v[0] = __builtin_nontemporal_load(p);
+    } else {
+        typedef T vec_t __attribute__((ext_vector_type(V)));
+        const vec_t t = __builtin_nontemporal_load(reinterpret_cast<const vec_t *>(p));
 #pragma unroll
         for (int e = 0; e < V; e++)
             v[e] = t[e];
@@ -79,7 +92,8 @@ struct TsTnArgs {
 // the remaining 4/(WM*WN) waves split K.
 // SYM: A and B are the same matrix (t(X) X). Only MFMA tiles on or above the diagonal are computed and the
 // slab is filled by mirroring; waves whose tile lies below the diagonal have nothing to do.
-template <typename T, int VA, int RA, int VB, int RB, int WM, int WN, bool SYM = false>
+// STREAM: the operands are read once, by one wave (loads carry the streaming hint).
+template <typename T, int VA, int RA, int VB, int RB, int WM, int WN, bool SYM = false, bool STREAM = false>
 __global__ __launch_bounds__(256) void ts_tn_kernel(TsTnArgs g) {
     using M = Mfma16<T>;
     static_assert(!SYM || (VA == VB && RA == RB && WM == WN), "the symmetric form needs the same tiling on both sides");
@@ -94,7 +108,6 @@ __global__ __launch_bounds__(256) void ts_tn_kernel(TsTnArgs g) {
     const int i = lane % 16, h = lane / 16;
     const T *A = static_cast<const T *>(g.A);
     const T *B = static_cast<const T *>(g.B);
-    const bool stream = g.stream != 0;
     // diagonal wave tile of a symmetric product: B fragments are the A fragments, lower MFMA tiles are skipped
     const bool diag = SYM && wm == wn;
     if (SYM && wm > wn)
@@ -150,7 +163,10 @@ __global__ __launch_bounds__(256) void ts_tn_kernel(TsTnArgs g) {
         const size_t kl = row_ok ? k : ke - 1;
 #pragma unroll
         for (int a = 0; a < RA; a++) {
-            ts_load<T, VA>(A + kl * g.lda + ca_ld[a], fr.a[u][a], stream);
+            if constexpr (STREAM)
+                ts_load_nt<T, VA>(A + kl * g.lda + ca_ld[a], fr.a[u][a]);
+            else
+                ts_load<T, VA>(A + kl * g.lda + ca_ld[a], fr.a[u][a]);
             if (guard) {
 #pragma unroll
                 for (int e = 0; e < VA; e++)
@@ -169,7 +185,10 @@ __global__ __launch_bounds__(256) void ts_tn_kernel(TsTnArgs g) {
         }
 #pragma unroll
         for (int b = 0; b < RB; b++) {
-            ts_load<T, VB>(B + kl * g.ldb + cb_ld[b], fr.b[u][b], stream);
+            if constexpr (STREAM)
+                ts_load_nt<T, VB>(B + kl * g.ldb + cb_ld[b], fr.b[u][b]);
+            else
+                ts_load<T, VB>(B + kl * g.ldb + cb_ld[b], fr.b[u][b]);
             if (guard) {
 #pragma unroll
                 for (int f = 0; f < VB; f++)
@@ -384,7 +403,7 @@ struct TsNtArgs {
 // pass over A gives the assignment, the per-position sums and the counts. The grid is then what the device holds at
 // once (one partial result per workgroup) and deals the pairs round-robin.
 template <typename T, int NB, bool ASSIGN, int CPG, bool UPDATE = false>
-__global__ __launch_bounds__(256, UPDATE ? (NB == 1 ? 3 : 2) : (ASSIGN && NB == 1 ? 4 : 1)) void ts_nt_kernel(TsNtArgs g) {
+__global__ __launch_bounds__(256, UPDATE ? (NB == 1 ? 3 : 2) : 1) void ts_nt_kernel(TsNtArgs g) {
     static_assert(!UPDATE || (ASSIGN && sizeof(T) == 4 && CPG == 4), "the one-pass form exists for float and 49..64 columns");
     using M = Mfma16<T>;
     constexpr int V = 16 / sizeof(T);
@@ -450,7 +469,9 @@ __global__ __launch_bounds__(256, UPDATE ? (NB == 1 ? 3 : 2) : (ASSIGN && NB == 
     // no barrier, the wave's own LDS instructions execute in order. Row stride SX = CPG KC + V: free of bank conflicts.
     constexpr unsigned VPR = CPG * 4;      // vectors of a row in one step
     constexpr unsigned SX = CPG * KC + V;
-    T *stage = lb + NB * 16 * ldl + wave * (16 * SX); // one row block at a time
+    // one row block at a time; UPDATE: both row blocks of the pair, which stay there until the pair is finished
+    constexpr unsigned STAGE_BLOCKS = UPDATE ? 2 : 1;
+    T *stage = lb + NB * 16 * ldl + wave * (STAGE_BLOCKS * 16 * SX);
     // Addresses are a base that is the same for the whole wave - the pair's first row - plus a 32-bit byte offset per
     // lane (32 rows of at most 2^24 bytes): one 24-bit multiplication and an addition per load, rows beyond M cut
     // back to the last row by a minimum on the row number.
@@ -466,8 +487,15 @@ __global__ __launch_bounds__(256, UPDATE ? (NB == 1 ? 3 : 2) : (ASSIGN && NB == 
             const unsigned kb = (kv < g.K ? kv : 0) * static_cast<unsigned>(sizeof(T));
             const unsigned r0 = id / VPR, r1 = r0 + 16;
             const unsigned l0 = r0 < last_local ? r0 : last_local, l1 = r1 < last_local ? r1 : last_local;
-            ts_load<T, V>(reinterpret_cast<const T *>(pair_base + (__umul24(l0, row_bytes) + kb)), fr.a[0][c], true);
-            ts_load<T, V>(reinterpret_cast<const T *>(pair_base + (__umul24(l1, row_bytes) + kb)), fr.a[1][c], true);
+            // measured at 20M x 64 floats: the streaming hint takes the stored product from 1163 to 1047 us and the
+            // one-pass form from 115 to 109 us (2M rows), and costs the arg-min form 8 % (944 -> 1017 us)
+            if constexpr (ASSIGN && !UPDATE) {
+                ts_load<T, V>(reinterpret_cast<const T *>(pair_base + (__umul24(l0, row_bytes) + kb)), fr.a[0][c]);
+                ts_load<T, V>(reinterpret_cast<const T *>(pair_base + (__umul24(l1, row_bytes) + kb)), fr.a[1][c]);
+            } else {
+                ts_load_nt<T, V>(reinterpret_cast<const T *>(pair_base + (__umul24(l0, row_bytes) + kb)), fr.a[0][c]);
+                ts_load_nt<T, V>(reinterpret_cast<const T *>(pair_base + (__umul24(l1, row_bytes) + kb)), fr.a[1][c]);
+            }
         }
         if constexpr (ASSIGN) {
             const T *ra_base = static_cast<const T *>(g.row_add) + prow;
@@ -497,14 +525,20 @@ __global__ __launch_bounds__(256, UPDATE ? (NB == 1 ? 3 : 2) : (ASSIGN && NB == 
         T xa[2][CPG][V];
 #pragma unroll
         for (int t = 0; t < 2; t++) {
+            T *st = stage + (UPDATE ? t * 16 * SX : 0);
 #pragma unroll
             for (int c = 0; c < CPG; c++) {
+                // vector 64 c + lane of the block: row (64 c + lane) / VPR; with 16 vectors a row that is row 4 c + h,
+                // vector i, spelled out so that the four stores share one address register
                 const unsigned id = c * 64 + lane;
-                dh_store_vec<T, V>(stage + (id / VPR) * SX + (id % VPR) * V, fr.a[t][c]);
+                if constexpr (VPR == 16)
+                    dh_store_vec<T, V>(st + (4 * c + h) * SX + i * V, fr.a[t][c]);
+                else
+                    dh_store_vec<T, V>(st + (id / VPR) * SX + (id % VPR) * V, fr.a[t][c]);
             }
 #pragma unroll
             for (int c = 0; c < CPG; c++)
-                dh_load_vec<T, V>(stage + i * SX + c * KC + h * V, xa[t][c]);
+                dh_load_vec<T, V>(st + i * SX + c * KC + h * V, xa[t][c]);
         }
 #pragma unroll
         for (int c = 0; c < CPG; c++) {
@@ -632,7 +666,7 @@ __global__ __launch_bounds__(256, UPDATE ? (NB == 1 ? 3 : 2) : (ASSIGN && NB == 
 #pragma unroll
                         for (int t = 0; t < 2; t++) {
                             const unsigned r = t * 16 + i;
-                            mine[8 * (r % 4) + r / 4] = rbase + r < g.M ? bi[t] : NONE; // rows beyond M belong nowhere
+                            mine[8 * (i % 4) + i / 4 + 4 * t] = rbase + r < g.M ? bi[t] : NONE; // rows beyond M belong nowhere
                         }
                     }
                     unsigned of_row[2][4];
@@ -641,15 +675,20 @@ __global__ __launch_bounds__(256, UPDATE ? (NB == 1 ? 3 : 2) : (ASSIGN && NB == 
 #pragma unroll
                     for (int t = 0; t < 2; t++)
 #pragma unroll
-                        for (int c = 0; c < 4; c++)
+                        for (int c = 0; c < 4; c++) {
+                            // the rows as rows - row 4 c + h, vector i - come back from the staging piece (kept in
+                            // registers since they were loaded, they would cost the kernel a wave per SIMD)
+                            T xr[V];
+                            dh_load_vec<T, V>(stage + (t * 16 + 4 * c + h) * SX + i * V, xr);
 #pragma unroll
                             for (int a = 0; a < NB; a++) {
                                 const T p = of_row[t][c] == static_cast<unsigned>(a * 16 + i) ? T(1) : T(0);
                                 cnt[a] += p;
 #pragma unroll
                                 for (int e = 0; e < V; e++)
-                                    acc_s[a][e] = M::mma(p, fr.a[t][c][e], acc_s[a][e]);
+                                    acc_s[a][e] = M::mma(p, xr[e], acc_s[a][e]);
                             }
+                        }
                 }
             } else {
                 // register v of lane (i, h) is C[row 4 v + h][column 16 b + i]: a row's values sit in the sixteen lanes of a group
@@ -741,7 +780,7 @@ __global__ __launch_bounds__(256, UPDATE ? (NB == 1 ? 3 : 2) : (ASSIGN && NB == 
         const unsigned j = idx / (g.kpad / V), kv = (idx % (g.kpad / V)) * V;
         T t[V];
         if (j < g.n && kv < g.K) {
-            ts_load<T, V>(B + static_cast<size_t>(j) * g.ldb + kv, t, false);
+            ts_load<T, V>(B + static_cast<size_t>(j) * g.ldb + kv, t);
         } else {
 #pragma unroll
             for (int e = 0; e < V; e++)
@@ -817,7 +856,9 @@ __global__ __launch_bounds__(256, UPDATE ? (NB == 1 ? 3 : 2) : (ASSIGN && NB == 
             cnt[a] += dh_peer_swap<32>{}(cnt[a]);
         }
         constexpr int NVAL = NB * V * 4 + NB;
-        __shared__ __attribute__((aligned(16))) T red[NVAL][64];
+        static_assert(NVAL * 64 <= 4 * 2 * 16 * (4 * 4 * V + V), "the exchange area must fit the staging pieces");
+        __syncthreads(); // every wave is done with its staging piece: the exchange between the waves takes their place
+        T(*red)[64] = reinterpret_cast<T(*)[64]>(lb + NB * 16 * ldl);
         for (int w = 1; w < 4; w++) {
             if (wave == w) {
                 int q = 0;
@@ -877,6 +918,12 @@ template <typename T> struct TsSide {
 
 template <typename T, int VA, int RA, int WM, int VB, int RB, int WN>
 static inline void ts_tn_launch(dh_ctx *ctx, const TsTnArgs &g, unsigned blocks) {
+    if constexpr (WM * WN == 1) {
+        if (g.stream) {
+            hipLaunchKernelGGL((ts_tn_kernel<T, VA, RA, VB, RB, WM, WN, false, true>), dim3(blocks), dim3(256), 0, ctx->stream, g);
+            return;
+        }
+    }
     hipLaunchKernelGGL((ts_tn_kernel<T, VA, RA, VB, RB, WM, WN>), dim3(blocks), dim3(256), 0, ctx->stream, g);
 }
 template <typename T, int V_, int R_, int W_> static inline void ts_tn_launch_sym(dh_ctx *ctx, const TsTnArgs &g, unsigned blocks) {
@@ -969,6 +1016,11 @@ template <typename T> inline size_t ts_nt_lds_bytes(int nb, unsigned kpad, int c
     constexpr size_t V = 16 / sizeof(T), KC = 4 * V;
     return (static_cast<size_t>(nb) * 16 * (kpad + V) + 4 * 16 * (cpg * KC + V)) * sizeof(T);
 }
+// ... of the one-pass form: the staging piece holds both row blocks of a pair
+template <typename T> inline size_t ts_nt_update_lds_bytes(int nb, unsigned kpad) {
+    constexpr size_t V = 16 / sizeof(T), KC = 4 * V;
+    return (static_cast<size_t>(nb) * 16 * (kpad + V) + 4 * 2 * 16 * (4 * KC + V)) * sizeof(T);
+}
 // chunks of k per step: the largest of 4, 2, 1 that divides their number
 template <typename T> inline int ts_nt_chunks_per_step(unsigned kpad) {
     const unsigned chunks = kpad / (4 * (16 / sizeof(T)));
@@ -992,8 +1044,9 @@ inline dh_status ts_nt_launch_cpg(dh_ctx *ctx, const TsNtArgs &g, size_t lds) {
 // g.slabs == nullptr first).
 template <typename T, int NB> inline dh_status ts_nt_update_launch(dh_ctx *ctx, const TsNtArgs &g, size_t *blocks_out) {
     const void *kernel = reinterpret_cast<const void *>(&ts_nt_kernel<T, NB, true, 4, true>);
-    const size_t lds = ts_nt_lds_bytes<T>(NB, g.kpad, 4);
-    // three workgroups per CU (measured 2 .. 8: flat within 5 %, best at 3 .. 4; registers and LDS allow four)
+    const size_t lds = ts_nt_update_lds_bytes<T>(NB, g.kpad);
+    // three workgroups per CU (measured 2 .. 4 per CU: 104 .. 110 us at 2M x 64, no trend; a loop that only loads the
+    // rows this way and stores the assignment takes 86 us, 74 us without the stores)
     (void)kernel;
     constexpr int per_cu = 3;
     size_t blocks = static_cast<size_t>(ctx->num_cus) * per_cu;

@@ -160,7 +160,7 @@ template <typename T, int NV, int NS, bool WITH_Y, int W> __device__ __forceinli
                     all = all && ((NEED >> (a * V + e)) & 1u);
                 if (all) {
                     T v[V];
-                    ts_load<T, V>(reinterpret_cast<const T *>(row + ov[a]), v, false);
+                    ts_load<T, V>(reinterpret_cast<const T *>(row + ov[a]), v);
 #pragma unroll
                     for (int e = 0; e < V; e++)
                         fr.f[a * V + e] = v[e];
@@ -236,7 +236,7 @@ template <typename T, int NV, int NS, bool WITH_Y, int W> __device__ __forceinli
 #pragma unroll
             for (int a = 0; a < NV; a++) {
                 T v[V];
-                ts_load<T, V>(reinterpret_cast<const T *>(row + ov[a]), v, false);
+                ts_load<T, V>(reinterpret_cast<const T *>(row + ov[a]), v);
 #pragma unroll
                 for (int e = 0; e < V; e++)
                     ft.f[a * V + e] = ok ? v[e] : T(0);
