@@ -576,6 +576,97 @@ static inline dh_status conv2d_resident_launch(dh_ctx *ctx, const ConvResidentAr
     return DH_OK;
 }
 
+// ---------------------------------------------------------------------------------------
+// One input channel, a filter of 3 x 3 or 5 x 5, stride 1 (the first layer of a CNN on grey images): K = Hf Wf is too
+// short for the matrix cores to pay - what such a layer costs is the store of F planes per image. Here a thread takes
+// a 2 x 2 quad of output pixels: the (Hf + 1) x (Wf + 1) patch under it sits in registers, the weights are the same
+// for all lanes (scalar loads into scalar registers, the multiply-add takes them from there), and consecutive threads
+// own consecutive quads, so that each filter's results leave as whole runs of a plane - pooled (POOL: one value per
+// quad, the running maximum from zero over the window in row order, Pooling.cpp:77-105) or as the four pixels.
+// A result is bias + the chain fma(w[k], x[k], .) over k = hy Wf + hx from zero, the same for every epilogue.
+// ---------------------------------------------------------------------------------------
+__device__ __forceinline__ float dh_fma(float a, float b, float c) { return __builtin_fmaf(a, b, c); }
+__device__ __forceinline__ double dh_fma(double a, double b, double c) { return __builtin_fma(a, b, c); }
+
+struct ConvDirectArgs {
+    unsigned N, H, W, ph, pw, P2, Q2, F; // P2, Q2: quads down and across (P / 2, Q / 2)
+    unsigned relu;
+    size_t quads;                        // N * P2 * Q2
+};
+
+template <typename T, int HF, int WF, bool POOL>
+__global__ __launch_bounds__(256) void conv2d_direct_kernel(const T *__restrict__ xin, const T *__restrict__ w,
+                                                            const T *__restrict__ bias, T *__restrict__ res, ConvDirectArgs g) {
+    // (the pointers are parameters of their own and do not alias: only then do the weights take the scalar path)
+    constexpr int FB = 4; // filters at a time: 16 accumulators beside the patch
+    const size_t quad = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (quad >= g.quads)
+        return;
+    const unsigned per_img = g.P2 * g.Q2;
+    const unsigned n = static_cast<unsigned>(quad / per_img), pq = static_cast<unsigned>(quad % per_img);
+    const unsigned p2 = pq / g.Q2, q2 = pq % g.Q2;
+    const T *img = xin + static_cast<size_t>(n) * g.H * g.W;
+    T x[HF + 1][WF + 1];
+#pragma unroll
+    for (int a = 0; a < HF + 1; a++)
+#pragma unroll
+        for (int b = 0; b < WF + 1; b++) {
+            const unsigned y = 2 * p2 + a - g.ph, xx = 2 * q2 + b - g.pw; // wraps to a huge value inside the border
+            const bool in = y < g.H && xx < g.W;
+            const T v = img[in ? y * g.W + xx : 0];
+            x[a][b] = in ? v : T(0);
+        }
+    const unsigned P = 2 * g.P2, Q = 2 * g.Q2;
+    T *out = res + static_cast<size_t>(n) * g.F * (POOL ? per_img : P * Q);
+    for (unsigned f0 = 0; f0 < g.F; f0 += FB) {
+        T acc[FB][4];
+#pragma unroll
+        for (int j = 0; j < FB; j++) {
+            const T *wf = w + static_cast<size_t>(f0 + j < g.F ? f0 + j : f0) * (HF * WF); // the same address in all lanes
+            acc[j][0] = acc[j][1] = acc[j][2] = acc[j][3] = T(0);
+#pragma unroll
+            for (int hy = 0; hy < HF; hy++)
+#pragma unroll
+                for (int hx = 0; hx < WF; hx++) {
+                    const T wk = wf[hy * WF + hx];
+                    acc[j][0] = dh_fma(wk, x[hy][hx], acc[j][0]);
+                    acc[j][1] = dh_fma(wk, x[hy][hx + 1], acc[j][1]);
+                    acc[j][2] = dh_fma(wk, x[hy + 1][hx], acc[j][2]);
+                    acc[j][3] = dh_fma(wk, x[hy + 1][hx + 1], acc[j][3]);
+                }
+        }
+#pragma unroll
+        for (int j = 0; j < FB; j++) {
+            const unsigned f = f0 + j;
+            if (f < g.F) {
+                const T bv = bias ? bias[f] : T(0);
+                T o[4];
+#pragma unroll
+                for (int v = 0; v < 4; v++) {
+                    o[v] = acc[j][v] + bv;
+                    // (a running maximum that starts from zero gives the same bits with and without the rectifier
+                    // before it: negative values, zeros of either sign and NaNs never replace the maximum)
+                    if constexpr (!POOL)
+                        o[v] = g.relu ? relu_of(o[v]) : o[v];
+                }
+                if constexpr (POOL) {
+                    T m = T(0);
+#pragma unroll
+                    for (int v = 0; v < 4; v++)
+                        m = (m < o[v]) ? o[v] : m;
+                    out[static_cast<size_t>(f) * per_img + pq] = m;
+                } else {
+                    T *plane = out + static_cast<size_t>(f) * P * Q + (2 * p2) * Q + 2 * q2;
+                    plane[0] = o[0];
+                    plane[1] = o[1];
+                    plane[Q] = o[2];
+                    plane[Q + 1] = o[3];
+                }
+            }
+        }
+    }
+}
+
 template <typename T>
 dh_status maxpool_forward(dh_ctx *ctx, T *res, size_t *res_h, size_t *res_w, const T *data, size_t N, size_t C,
                           size_t H, size_t W, size_t ph, size_t pw, size_t sh, size_t sw, size_t padh, size_t padw);
@@ -612,6 +703,37 @@ dh_status conv2d_forward(dh_ctx *ctx, T *res, size_t *res_h, size_t *res_w, cons
     const size_t pixels = N * P * Q;
     if (pixels == 0 || F == 0)
         return DH_OK;
+    // One channel, 3 x 3 or 5 x 5, stride 1, even output extents: a thread per 2 x 2 quad of output pixels on the ordinary
+    // ALUs (1 -> 32 channels, 5 x 5 on 28 x 28, batch 4096, with ReLU and pooling: 0.153 ms in the tiled kernel below).
+    // As everywhere in this function the choice does not look at the epilogue.
+    if (C == 1 && sh == 1 && sw == 1 && Hf == Wf && (Hf == 3 || Hf == 5) && P % 2 == 0 && Q % 2 == 0 && N < (size_t(1) << 31) &&
+        H * W < (size_t(1) << 31) && F < (size_t(1) << 31) && N * (P / 2) * (Q / 2) < (size_t(1) << 39)) {
+        ConvDirectArgs d{};
+        d.N = static_cast<unsigned>(N);
+        d.H = static_cast<unsigned>(H);
+        d.W = static_cast<unsigned>(W);
+        d.ph = static_cast<unsigned>(ph);
+        d.pw = static_cast<unsigned>(pw);
+        d.P2 = static_cast<unsigned>(P / 2);
+        d.Q2 = static_cast<unsigned>(Q / 2);
+        d.F = static_cast<unsigned>(F);
+        d.relu = relu;
+        d.quads = N * (P / 2) * (Q / 2);
+        const dim3 dgrid(static_cast<unsigned>(dh_ceil_div(d.quads, static_cast<size_t>(256))));
+        if (Hf == 5) {
+            if (pool)
+                hipLaunchKernelGGL((conv2d_direct_kernel<T, 5, 5, true>), dgrid, dim3(256), 0, ctx->stream, data, filter, bias, res, d);
+            else
+                hipLaunchKernelGGL((conv2d_direct_kernel<T, 5, 5, false>), dgrid, dim3(256), 0, ctx->stream, data, filter, bias, res, d);
+        } else {
+            if (pool)
+                hipLaunchKernelGGL((conv2d_direct_kernel<T, 3, 3, true>), dgrid, dim3(256), 0, ctx->stream, data, filter, bias, res, d);
+            else
+                hipLaunchKernelGGL((conv2d_direct_kernel<T, 3, 3, false>), dgrid, dim3(256), 0, ctx->stream, data, filter, bias, res, d);
+        }
+        DH_CHECK_LAUNCH();
+        return DH_OK;
+    }
     constexpr int BK = dh_gemm::GemmBK<T>::value;
     constexpr int BN = 128;
     const size_t Hp = H + 2 * ph, Wp = W + 2 * pw, K = C * Hf * Wf;

@@ -82,6 +82,11 @@ FUSED_CONV_CASES = CONV_CASES + [
     (6, 2, 11, 11, 70, 3, 3, 1, 1, 0, 0),
     (40, 5, 4, 4, 16, 3, 3, 1, 1, 0, 0),
     (3, 1, 64, 64, 8, 5, 5, 1, 1, 2, 2),
+    # one channel, even result planes (a thread per 2 x 2 quad of pixels): 3 x 3 with and without padding, filter
+    # counts that are no multiple of four
+    (9, 1, 12, 10, 7, 3, 3, 1, 1, 1, 1),
+    (5, 1, 10, 8, 5, 3, 3, 1, 1, 0, 0),
+    (300, 1, 28, 28, 6, 5, 5, 1, 1, 2, 2),
 ]
 
 
@@ -118,6 +123,38 @@ def test_conv2d_fused_epilogues_equal_the_operator_sequence(ctx, dt, case):
     st, orl = orc.ew_binary_sca(14, oc, 0.0)
     st, op, _, _ = orc.maxpool(orl, N, F, P, Q, 2, 2, 2, 2, 0, 0)
     assert_close(got.to_numpy(), op, elementwise=False)
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+def test_conv2d_one_channel_special_values(ctx, dt):
+    """NaN, infinities and zeros of both signs go through the one-channel kernel's pooled store as through the three
+    separate kernels (the pooled store leaves the rectifier out: a running maximum from zero does not need it)."""
+    N, H, W, F = 6, 12, 12, 5
+    rng = np.random.default_rng(31)
+    x = (rng.random((N, H * W)) - 0.5).astype(dt)
+    x[0, 17], x[1, 40], x[2, 5], x[3, 77] = np.nan, np.inf, -np.inf, -0.0
+    x[4, :] = -0.0
+    w = rng.standard_normal((F, 25)).astype(dt)
+    w[1, :] = 0.0
+    w[2, :] = -np.abs(w[2, :])
+    b = np.array([[0.1], [-0.0], [0.0], [-0.2], [0.3]], dtype=dt)
+    X, Wd, B = DenseMatrix.from_numpy(ctx, x), DenseMatrix.from_numpy(ctx, w), DenseMatrix.from_numpy(ctx, b)
+    conv, P, Q = conv2dForward(None, X, Wd, B, N, 1, H, W, 5, 5, 1, 1, 2, 2, ctx)
+    for with_relu in (True, False):
+        before = reluForward(None, conv, ctx) if with_relu else conv
+        pooled, _, _ = maxPoolForward(None, before, N, F, P, Q, 2, 2, 2, 2, 0, 0, ctx)
+        got, _, _ = conv2dForwardFused(None, X, Wd, B, N, 1, H, W, 5, 5, 1, 1, 2, 2, ctx, relu=with_relu, pool=True)
+        g, e = got.to_numpy(), pooled.to_numpy()
+        assert_exact(g, e)
+        assert (np.signbit(g) == np.signbit(e))[~np.isnan(e)].all()
+        unp, _, _ = conv2dForwardFused(None, X, Wd, B, N, 1, H, W, 5, 5, 1, 1, 2, 2, ctx, relu=with_relu, pool=False)
+        assert_exact(unp.to_numpy(), before.to_numpy())
+        assert (np.signbit(unp.to_numpy()) == np.signbit(before.to_numpy()))[~np.isnan(before.to_numpy())].all()
+    assert np.isnan(conv.to_numpy()).any() and np.isinf(conv.to_numpy()).any()
+    st, oc, _, _ = orc.conv2d(x, w, b, N, 1, H, W, 5, 5, 1, 1, 2, 2)
+    finite = np.isfinite(oc)
+    assert (np.isfinite(conv.to_numpy()) == finite).all()
+    assert_close(conv.to_numpy()[finite], oc[finite], elementwise=False)
 
 
 def test_conv2d_fused_rejects_unknown_flags(ctx):
