@@ -195,6 +195,17 @@ def main() -> int:
             emit("conv2dForwardFused 32->64 ch, 14x14, 5x5 pad 2, ReLU + maxPool 2x2 in the epilogue", dt, f"batch {N}",
                  timed(lambda: K.conv2dForwardFused(pl, x2, w2, b2, N, 32, 14, 14, 5, 5, 1, 1, 2, 2, ctx, relu=True, pool=True)),
                  flops=2.0 * N * 64 * 196 * 800)
+            x1 = DM.from_torch(ctx, torch.rand(N, 784, device="cuda", dtype=tdt, generator=gen))
+            w1 = DM.from_torch(ctx, torch.randn(32, 25, device="cuda", dtype=tdt, generator=gen) * 0.2)
+            b1 = DM.from_torch(ctx, torch.randn(32, 1, device="cuda", dtype=tdt, generator=gen) * 0.1)
+            o1, p1 = DM(ctx, N, 32 * 784, ndt), DM(ctx, N, 32 * 196, ndt)
+            emit("conv2dForward 1->32 ch, 28x28, 5x5 pad 2 (a thread per 2x2 quad of pixels)", dt, f"batch {N}",
+                 timed(lambda: K.conv2dForward(o1, x1, w1, b1, N, 1, 28, 28, 5, 5, 1, 1, 2, 2, ctx)), flops=2.0 * N * 32 * 784 * 25)
+            emit("conv2dForwardFused 1->32 ch, 28x28, 5x5 pad 2, ReLU + maxPool 2x2 in the epilogue", dt, f"batch {N}",
+                 timed(lambda: K.conv2dForwardFused(p1, x1, w1, b1, N, 1, 28, 28, 5, 5, 1, 1, 2, 2, ctx, relu=True, pool=True)),
+                 flops=2.0 * N * 32 * 784 * 25)
+            for m_ in (x1, w1, b1, o1, p1):
+                m_.destroy()
             emit("maxPoolForward 2x2/2 on 14x14", dt, f"{N}x{64 * 196}",
                  timed(lambda: K.maxPoolForward(pl, o2, N, 64, 14, 14, 2, 2, 2, 2, 0, 0, ctx)), 1.25 * N * 64 * 196 * sz)
             emit("avgPoolForward 2x2/2 on 14x14", dt, f"{N}x{64 * 196}",
