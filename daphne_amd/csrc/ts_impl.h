@@ -603,54 +603,28 @@ __global__ __launch_bounds__(256, UPDATE ? (NB == 1 ? 3 : 2) : 1) void ts_nt_ker
 #pragma unroll
                         for (int v = 0; v < 4; v++)
                             d[t][b][v] = (acc[t][b][v] * T(-2) + radd[t][0]) + col_add[b][v];
-                // The short way: a plain running minimum. It gives IDXMIN's answer unless a NaN is among the values or
-                // nothing lies below +inf; the sum of a lane's values tells the first (opposite infinities only send
-                // the wave the long way for nothing), the minimum itself the second.
-                T best[2], sum[2];
+                // IDXMIN (AggRow.h:71-83: a running minimum from the row's first value, strict comparisons) for a row
+                // whose values lie in four lanes: the first position of the least value that is below +inf - a NaN is
+                // below nothing, so it is never taken, and columns beyond n carry +inf - and position 0 if there is
+                // none or if the row's first value is a NaN (nothing is below a NaN either). No second path for rows
+                // with NaNs: an empty cluster makes its centroid, and with it a whole column of distances, NaN.
                 unsigned bi[2];
-                bool odd = false;
 #pragma unroll
                 for (int t = 0; t < 2; t++) {
-                    best[t] = sum[t] = d[t][0][0];
-                    bi[t] = 4 * h;
+                    T best = dh_inf<T>();
+                    unsigned at = NONE;
 #pragma unroll
                     for (int b = 0; b < NB; b++)
 #pragma unroll
                         for (int v = 0; v < 4; v++) {
-                            if (b == 0 && v == 0)
-                                continue;
-                            const bool lt = d[t][b][v] < best[t];
-                            best[t] = lt ? d[t][b][v] : best[t];
-                            bi[t] = lt ? static_cast<unsigned>(b * 16 + 4 * h + v) : bi[t];
-                            sum[t] += d[t][b][v];
+                            const bool lt = d[t][b][v] < best;
+                            best = lt ? d[t][b][v] : best;
+                            at = lt ? static_cast<unsigned>(b * 16 + 4 * h + v) : at;
                         }
-                    take(best[t], bi[t], dh_peer_swap<16>{}(best[t]), dh_peer_swap<16>{}(bi[t]));
-                    take(best[t], bi[t], dh_peer_swap<32>{}(best[t]), dh_peer_swap<32>{}(bi[t]));
-                    odd |= (sum[t] != sum[t]) || !(best[t] < dh_inf<T>());
-                }
-                if (__ballot(odd) != 0) {
-                    // the long way, with IDXMIN's rules spelled out (bi is the answer in the lanes h = 0 at least)
-#pragma unroll
-                    for (int t = 0; t < 2; t++) {
-                        T best1 = dh_inf<T>(), first = T(0);
-                        unsigned bi1 = NONE;
-#pragma unroll
-                        for (int b = 0; b < NB; b++)
-#pragma unroll
-                            for (int v = 0; v < 4; v++) {
-                                const unsigned col = b * 16 + 4 * h + v;
-                                const T dv = d[t][b][v];
-                                if (b == 0 && v == 0)
-                                    first = dv; // column 0 in the lanes h = 0
-                                if (col < g.n && (dv < best1 || (bi1 == NONE && !(dv != dv)))) {
-                                    best1 = dv;
-                                    bi1 = col;
-                                }
-                            }
-                        take(best1, bi1, dh_peer_swap<16>{}(best1), dh_peer_swap<16>{}(bi1));
-                        take(best1, bi1, dh_peer_swap<32>{}(best1), dh_peer_swap<32>{}(bi1));
-                        bi[t] = ((first != first) || bi1 == NONE) ? 0u : bi1;
-                    }
+                    take(best, at, dh_peer_swap<16>{}(best), dh_peer_swap<16>{}(at));
+                    take(best, at, dh_peer_swap<32>{}(best), dh_peer_swap<32>{}(at));
+                    const T first = d[t][0][0]; // column 0 in the lanes h = 0, the ones that store
+                    bi[t] = ((first != first) || at == NONE) ? 0u : at;
                 }
 #pragma unroll
                 for (int t = 0; t < 2; t++) {
@@ -706,10 +680,9 @@ __global__ __launch_bounds__(256, UPDATE ? (NB == 1 ? 3 : 2) : 1) void ts_nt_ker
                             const T d = (acc[t][b][v] * T(-2) + ra) + col_add[b][0];
                             if (b == 0)
                                 first = d; // column 0 in the lanes i = 0
-                            if (col < g.n && (d < best || (bi == NONE && !(d != d)))) {
-                                best = d;
-                                bi = col;
-                            }
+                            const bool lt = d < best; // columns beyond n carry +inf
+                            best = lt ? d : best;
+                            bi = lt ? col : bi;
                         }
                         dh_butterfly(16, [&](auto peer) { take(best, bi, peer(best), peer(bi)); });
                         if (i == 0 && row < g.M)
