@@ -297,21 +297,22 @@ def run(args) -> int:
         xt = torch.rand(N, 784, device="cuda", generator=gen)
         x = DenseMatrix.from_torch(ctx, xt)
         ms = _timed(torch, lambda: lenet_forward(ctx, x, W, N), args.steps, args.warmup)
-        layers, last = {}, [None]
-
-        def timer(name):
-            e = torch.cuda.Event(enable_timing=True)
-            e.record()
-            if last[0] is not None:
-                layers.setdefault(name, []).append((last[0], e))
-            last[0] = e
-
-        for _ in range(9):
-            last[0] = torch.cuda.Event(enable_timing=True)
-            last[0].record()
-            lenet_forward(ctx, x, W, N, timer)
-        torch.cuda.synchronize()
-        layer_ms = {k_: round(float(np.median([a.elapsed_time(b) for a, b in v])), 4) for k_, v in layers.items()}
+        # every layer on its own, into a result matrix that is there already (a layer that allocates its result puts
+        # a synchronising release of the last one between the kernels, which the events would count)
+        from daphne_amd.kernels import affineForward, affineForwardFused, conv2dForwardFused, softmax
+        h1, _, _ = conv2dForwardFused(None, x, W["w1"], W["b1"], N, 1, 28, 28, 5, 5, 1, 1, 2, 2, ctx, relu=True, pool=True)
+        h2, _, _ = conv2dForwardFused(None, h1, W["w2"], W["b2"], N, 32, 14, 14, 5, 5, 1, 1, 2, 2, ctx, relu=True, pool=True)
+        h3 = affineForwardFused(None, h2, W["w3"], W["b3"], ctx)
+        h4 = affineForward(None, h3, W["w4"], W["b4"], ctx)
+        h5 = softmax(None, h4, ctx)
+        layer_ms = {
+            "conv1+bias+relu+pool": _events(torch, lambda: conv2dForwardFused(h1, x, W["w1"], W["b1"], N, 1, 28, 28, 5, 5, 1, 1, 2, 2, ctx, relu=True, pool=True)),
+            "conv2+bias+relu+pool": _events(torch, lambda: conv2dForwardFused(h2, h1, W["w2"], W["b2"], N, 32, 14, 14, 5, 5, 1, 1, 2, 2, ctx, relu=True, pool=True)),
+            "affine1+relu": _events(torch, lambda: affineForwardFused(h3, h2, W["w3"], W["b3"], ctx)),
+            "affine2": _events(torch, lambda: affineForward(h4, h3, W["w4"], W["b4"], ctx)),
+            "softmax": _events(torch, lambda: softmax(h5, h4, ctx)),
+        }
+        layer_ms = {k_: round(v, 4) for k_, v in layer_ms.items()}
         flops = {"conv1+bias+relu+pool": 2.0 * N * 32 * 784 * 25, "conv2+bias+relu+pool": 2.0 * N * 64 * 196 * 800,
                  "affine1+relu": 2.0 * N * 3136 * 512, "affine2": 2.0 * N * 512 * 10}
         layer_tflops = {k_: round(flops[k_] / layer_ms[k_] / 1e9, 2) for k_ in flops}
