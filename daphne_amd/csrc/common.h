@@ -50,6 +50,9 @@ struct dh_ctx {
     // One int on the device + its pinned host mirror, for domain-error flags.
     int *flag_dev = nullptr;
     int *flag_host = nullptr;
+    // The host mirror as the device sees it: a kernel that reports through it spares the copy back (the caller still
+    // waits for the stream before it reads flag_host). Plain stores only - no atomics on host memory.
+    int *flag_host_dev = nullptr;
 
     hipEvent_t ev_start = nullptr, ev_stop = nullptr;
     int num_cus = 0;

@@ -66,7 +66,8 @@ extern "C" dh_status dh_ctx_create(int device, dh_ctx **out) {
     ctx->mem_budget = static_cast<size_t>(static_cast<double>(total_b) * 0.9);
     ctx->num_cus = ctx->props.multiProcessorCount;
     bool ok = hipMalloc(reinterpret_cast<void **>(&ctx->flag_dev), 256) == hipSuccess &&
-              hipHostMalloc(reinterpret_cast<void **>(&ctx->flag_host), 256, hipHostMallocDefault) == hipSuccess &&
+              hipHostMalloc(reinterpret_cast<void **>(&ctx->flag_host), 256, hipHostMallocMapped) == hipSuccess &&
+              hipHostGetDevicePointer(reinterpret_cast<void **>(&ctx->flag_host_dev), ctx->flag_host, 0) == hipSuccess &&
               hipEventCreate(&ctx->ev_start) == hipSuccess && hipEventCreate(&ctx->ev_stop) == hipSuccess;
     if (!ok) {
         dh_ctx_destroy(ctx);

@@ -656,7 +656,7 @@ template <typename T> dh_status solve(dh_ctx *ctx, T *x, const T *A, size_t n, s
                 }
             }
             hipLaunchKernelGGL(kernel, dim3(1), dim3(LDS_SOLVE_THREADS), lds_bytes, ctx->stream, x, A, lda, b,
-                               static_cast<unsigned>(n), ctx->flag_dev);
+                               static_cast<unsigned>(n), ctx->flag_host_dev);
             return DH_OK;
         };
         dh_status lst;
@@ -669,18 +669,18 @@ template <typename T> dh_status solve(dh_ctx *ctx, T *x, const T *A, size_t n, s
         if (lst != DH_OK)
             return lst;
     } else {
-        hipLaunchKernelGGL(clear_flag_kernel, dim3(1), dim3(1), 0, ctx->stream, ctx->flag_dev);
+        hipLaunchKernelGGL(clear_flag_kernel, dim3(1), dim3(1), 0, ctx->stream, ctx->flag_host_dev);
         void *wsv = nullptr;
         dh_status st = dh_workspace(ctx, n * n * sizeof(T), &wsv);
         if (st != DH_OK)
             return st;
         hipLaunchKernelGGL((lu_solve_kernel<T>), dim3(1), dim3(SOLVE_THREADS), 0, ctx->stream, static_cast<T *>(wsv), x,
-                           A, lda, b, static_cast<unsigned>(n), ctx->flag_dev);
+                           A, lda, b, static_cast<unsigned>(n), ctx->flag_host_dev);
     }
     DH_CHECK_LAUNCH();
-    DH_CHECK_HIP(hipMemcpyAsync(ctx->flag_host, ctx->flag_dev, sizeof(int), hipMemcpyDeviceToHost, ctx->stream));
+    // the kernels write the flag into the pinned host word itself: no copy back, only the wait
     DH_CHECK_HIP(hipStreamSynchronize(ctx->stream));
-    if (*ctx->flag_host != 0)
+    if (*static_cast<volatile int *>(ctx->flag_host) != 0)
         // Solve.h:113-115
         return dh_fail(DH_ERR_RUNTIME, "A factor Ui is exactly singular, so the solution could not be computed");
     return DH_OK;
