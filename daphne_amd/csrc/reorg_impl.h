@@ -10,6 +10,8 @@
 
 #include "common.h"
 
+#include <cmath>
+
 namespace dh_reorg {
 
 // dst[r][c] = src ? src[r][c] : value, for a cols-wide block (cols counted in vectors of VEC)
@@ -186,6 +188,48 @@ __global__ __launch_bounds__(256) void extract_col_kernel(T *res, size_t ld_res,
     res[r * ld_res + k] = arg[r * ld + static_cast<size_t>(c)];
 }
 
+// The same for selections that touch most of a row's 64-byte segments anyway (eight random columns of 64 floats reach
+// 3.6 of the 4): the rows are streamed whole - a wavefront loads 4 KB of consecutive rows with four 16-byte vectors a
+// lane, parks them in a piece of LDS of its own (no barrier: its LDS instructions execute in order) and picks the
+// selected values from there, so that the results of its rows leave as one contiguous run.
+// LPR: lanes (16-byte vectors) per row, a power of two up to 64.
+template <typename T>
+__global__ __launch_bounds__(256) void extract_col_rows_kernel(T *res, size_t ld_res, const T *arg, size_t ld, size_t rows,
+                                                               unsigned cols, const long long *sel, unsigned nsel, size_t ld_sel,
+                                                               unsigned lpr) {
+    constexpr int VEC = 16 / sizeof(T), UN = 4;
+    extern __shared__ __attribute__((aligned(16))) unsigned char extract_lds[];
+    unsigned *selc = reinterpret_cast<unsigned *>(extract_lds);                    // nsel positions, as given or counted from the end
+    T *park = reinterpret_cast<T *>(extract_lds + ((nsel * 4u + 15u) & ~15u));     // 4 waves x UN KB
+    const unsigned tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
+    const unsigned rps = 64 / lpr, rpw = rps * UN;                                 // rows per load, rows per wavefront
+    const size_t row0 = (static_cast<size_t>(blockIdx.x) * 4 + wave) * rpw;
+    T v[UN][VEC];
+#pragma unroll
+    for (int u = 0; u < UN; u++) {
+        size_t r = row0 + u * rps + lane / lpr;
+        r = r < rows ? r : rows - 1; // beyond the end: the last row again, never stored
+        dh_load_vec_stream<T, VEC>(arg + r * ld + (lane % lpr) * VEC, v[u]);
+    }
+    for (unsigned k = tid; k < nsel; k += 256) {
+        long long c = sel[k * ld_sel];
+        selc[k] = static_cast<unsigned>(c < 0 ? c + static_cast<long long>(cols) : c);
+    }
+    T *mine = park + wave * (UN * 64 * VEC);
+#pragma unroll
+    for (int u = 0; u < UN; u++)
+        dh_store_vec<T, VEC>(mine + (u * 64 + lane) * VEC, v[u]); // row u rps + lane / lpr at (that row) * cols: cols = lpr VEC
+    __syncthreads(); // the positions
+    if (row0 >= rows)
+        return;
+    const unsigned live = rows - row0 < rpw ? static_cast<unsigned>(rows - row0) : rpw;
+    const unsigned nout = live * nsel;
+    for (unsigned o = lane; o < nout; o += 64) {
+        const unsigned r = o / nsel, k = o - r * nsel;
+        dh_store_stream(res + (row0 + r) * ld_res + k, mine[r * cols + selc[k]]);
+    }
+}
+
 // ExtractCol<DenseMatrix<VT>,DenseMatrix<VT>,DenseMatrix<int64_t>>::apply
 // (kernels/ExtractCol.h:74-114, kernels/CUDA/ExtractCol.cu:21-56)
 template <typename T>
@@ -220,6 +264,24 @@ dh_status extract_col(dh_ctx *ctx, T *res, size_t ld_res, const T *arg, size_t r
                        "invalid argument '%lld' passed to ExtractCol: out of bounds for dense matrix with column "
                        "boundaries '[0, %zu)'",
                        v, cols);
+    }
+    {
+        // whole rows where a gather would fetch most of them anyway: rows of a power-of-two number of 16-byte vectors
+        // (up to 1 KB), an expected share of at least 60 % of a row's 64-byte segments hit by the selection
+        constexpr size_t V = 16 / sizeof(T);
+        const size_t row_bytes = cols * sizeof(T), lpr = cols / V;
+        const double segments = row_bytes < 64 ? 1.0 : static_cast<double>(row_bytes) / 64.0;
+        const double coverage = 1.0 - pow(1.0 - 1.0 / segments, static_cast<double>(sel_rows));
+        const size_t rpw = lpr ? (64 / lpr) * 4 : 0;
+        if (cols % V == 0 && lpr >= 1 && lpr <= 64 && (lpr & (lpr - 1)) == 0 && ld % V == 0 && dh_aligned(arg, 16) &&
+            sel_rows <= 1024 && coverage >= 0.6 && rows >= 4096 && dh_ceil_div(rows, rpw * 4) < (size_t(1) << 31)) {
+            const size_t lds = ((sel_rows * 4 + 15) & ~size_t(15)) + 4 * 4 * 1024;
+            hipLaunchKernelGGL((extract_col_rows_kernel<T>), dim3(static_cast<unsigned>(dh_ceil_div(rows, rpw * 4))), dim3(256), lds,
+                               ctx->stream, res, ld_res, arg, ld, rows, static_cast<unsigned>(cols), sel,
+                               static_cast<unsigned>(sel_rows), ld_sel, static_cast<unsigned>(lpr));
+            DH_CHECK_LAUNCH();
+            return DH_OK;
+        }
     }
     unsigned tx = 1;
     while (tx < 256 && tx < sel_rows)

@@ -67,7 +67,11 @@ def test_col_bind_views_and_errors(ctx, dt):
 
 @pytest.mark.parametrize("dt", DTYPES)
 @pytest.mark.parametrize("rows,cols,sel", [(3, 3, [0, 2]), (3, 3, [2, 0, 1]), (3, 3, [1, 2, 2, 0, 1, 0, 1, 2]), (5, 7, [-1, -7, 3]),
-                                           (100000, 64, [63, 0, 17, 17]), (1, 1, [0]), (40, 300, list(range(299, -1, -3)))])
+                                           (100000, 64, [63, 0, 17, 17]), (1, 1, [0]), (40, 300, list(range(299, -1, -3))),
+                                           # selections that take the kernel which streams whole rows (4096 rows or more,
+                                           # rows of 1, 4, 16, 64 vectors), with a last wavefront that is not full
+                                           (50001, 64, [5, -1, 33, 33, 0, -64, 47, 18]), (8193, 16, [3, -1, 0]),
+                                           (20000, 256, list(range(0, 256, 3))), (5003, 4, [1]), (4100, 64, list(range(63, -1, -1)))])
 def test_extract_col(ctx, dt, rows, cols, sel):
     rng = np.random.default_rng(rows + cols)
     a = rng.standard_normal((rows, cols)).astype(dt)
@@ -91,6 +95,15 @@ def test_extract_col_errors_and_views(ctx, dt):
     two = DenseMatrix.from_numpy(ctx, np.zeros((2, 2), np.int64))
     with pytest.raises(capi.DaphneHipError, match="column matrix"):
         extractCol(None, dA, two, ctx)
+    # the same on views of a matrix with enough rows for the kernel that streams whole rows
+    rngv = np.random.default_rng(18)
+    wide = rngv.standard_normal((6000, 80)).astype(dt)
+    sv = np.asarray([63, 1, -2, 40, 7, 7, 22, 0], dtype=np.int64).reshape(-1, 1)
+    resv = DenseMatrix(ctx, 6000, 12, dt, zero=True)
+    extractCol(resv.slice(0, 6000, 2, 10), DenseMatrix.from_numpy(ctx, wide).slice(0, 6000, 8, 72), DenseMatrix.from_numpy(ctx, sv), ctx)
+    fullv = resv.to_numpy()
+    assert_exact(fullv[:, 2:10], wide[:, 8:72][:, [63, 1, 62, 40, 7, 7, 22, 0]])
+    assert (fullv[:, :2] == 0).all() and (fullv[:, 10:] == 0).all()
     # argument and result views
     rng = np.random.default_rng(8)
     big = rng.standard_normal((30, 20)).astype(dt)
