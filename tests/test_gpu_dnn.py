@@ -272,7 +272,9 @@ def test_batchnorm_inference(ctx, dt, rows, C, HW):
 @pytest.mark.parametrize("dt", DTYPES)
 @pytest.mark.parametrize("rows,cols", [(3, 3), (1, 9), (4096, 10), (7, 1), (33, 1000), (5, 64),
                                        # short rows staged through LDS: a partial last workgroup, a scalar tail, 31 values
-                                       (5000, 10), (1030, 7), (2000, 31), (1500, 1), (1024, 12)])
+                                       (5000, 10), (1030, 7), (2000, 31), (1500, 1), (1024, 12),
+                                       # two rows a thread (2^18 rows or more, up to 10 floats / 5 doubles a row)
+                                       (262444, 10), (300001, 5), (262145, 3)])
 def test_softmax(ctx, dt, rows, cols):
     rng = np.random.default_rng(rows + cols)
     x = (rng.standard_normal((rows, cols)) * 4).astype(dt)
