@@ -249,6 +249,19 @@ def main() -> int:
                  timed(lambda: K.batchNorm2DTrainForward(x, gam, zer, zer, gam, 1e-5, 0.1, ctx)), 2 * el * sz)
             emit("batchNorm2DBackward 64 channels (sums pass + gradient pass)", dt, f"{N}x{64 * 196}",
                  timed(lambda: K.batchNorm2DBackward(res_bn[3], res_bn[4], x, dy, gam, 1e-5, ctx)), 3 * el * sz)
+            # the same where a channel's values fit a workgroup's LDS: 32 images of 512 channels, 14 x 14
+            ns, cs = 32, 512
+            xs = DM.from_torch(ctx, torch.randn(ns, cs * 196, device="cuda", dtype=tdt, generator=gen))
+            dys = DM.from_torch(ctx, torch.randn(ns, cs * 196, device="cuda", dtype=tdt, generator=gen))
+            gs = DM.from_torch(ctx, torch.rand(cs, 1, device="cuda", dtype=tdt, generator=gen) + 0.5)
+            zs = DM.from_torch(ctx, torch.zeros(cs, 1, device="cuda", dtype=tdt))
+            rs = K.batchNorm2DTrainForward(xs, gs, zs, zs, gs, 1e-5, 0.1, ctx)
+            emit("batchNorm2DTrainForward 512 channels, 14x14 (one read where a channel fits LDS)", dt, f"{ns}x{cs * 196}",
+                 timed(lambda: K.batchNorm2DTrainForward(xs, gs, zs, zs, gs, 1e-5, 0.1, ctx)), 2 * ns * cs * 196 * sz)
+            emit("batchNorm2DBackward 512 channels, 14x14 (one read where a channel and its gradient fit LDS)", dt, f"{ns}x{cs * 196}",
+                 timed(lambda: K.batchNorm2DBackward(rs[3], rs[4], xs, dys, gs, 1e-5, ctx)), 3 * ns * cs * 196 * sz)
+            for m_ in (xs, dys, gs, zs, *rs):
+                m_.destroy()
             dpool = DM.from_torch(ctx, torch.randn(N, 64 * 49, device="cuda", dtype=tdt, generator=gen))
             dxp = DM(ctx, N, 64 * 196, ndt)
             emit("maxPoolBackward 2x2/2 on 14x14", dt, f"{N}x{64 * 196}",

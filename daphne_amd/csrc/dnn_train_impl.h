@@ -212,6 +212,108 @@ __global__ __launch_bounds__(THREADS) void chan_apply(T *res, const T *x, const 
     }
 }
 
+// Both passes from ONE read where a channel's values (all images) fit a workgroup's LDS: the workgroup of a channel
+// copies them in, adds up what the channel's statistics need (in double, threads in a fixed order), derives the
+// channel's coefficients in one thread and applies them to the copy. FWD: the sums of chan_stage1 MODE 3 and the
+// arithmetic of chan_stage2 STEP 3 and chan_apply; else MODE 2, STEP 2 and the gradient form, with dy in LDS beside x.
+template <typename T, bool FWD>
+__global__ __launch_bounds__(512) void chan_lds_kernel(T *res, const T *x, const T *dy, unsigned N, unsigned C, unsigned HW, T *mean,
+                                                       T *inv_var, T *new_ema_mean, T *new_ema_var, const T *ema_mean,
+                                                       const T *ema_var, T eps, T mu_, const T *gamma, const T *beta, T *dGamma,
+                                                       T *dBeta) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char chan_lds[];
+    T *sx = reinterpret_cast<T *>(chan_lds);
+    __shared__ double red[3][8];
+    __shared__ T coef[4];
+    const unsigned c = blockIdx.x, tid = threadIdx.x, n_el = N * HW;
+    T *sdy = sx + n_el;
+    for (unsigned idx = tid; idx < n_el; idx += 512) {
+        const unsigned n = idx / HW, j = idx - n * HW;
+        const size_t off = (static_cast<size_t>(n) * C + c) * HW + j;
+        sx[idx] = x[off];
+        if constexpr (!FWD)
+            sdy[idx] = dy[off];
+    }
+    __syncthreads();
+    const double shift = FWD ? static_cast<double>(sx[0]) : static_cast<double>(mean[c]);
+    double a[3] = {0.0, 0.0, 0.0};
+    for (unsigned idx = tid; idx < n_el; idx += 512) {
+        const double d = static_cast<double>(sx[idx]) - shift;
+        if constexpr (FWD) {
+            a[0] += d;
+            a[1] += d * d;
+        } else {
+            const double gr = static_cast<double>(sdy[idx]);
+            a[0] += gr;
+            a[1] += gr * d;
+            a[2] += d;
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < 3; k++) {
+        double v = a[k];
+        dh_butterfly(DH_WAVE, [&](auto peer) { v += peer(v); });
+        if (tid % DH_WAVE == 0)
+            red[k][tid / DH_WAVE] = v;
+    }
+    __syncthreads();
+    if (tid == 0) {
+        double s[3];
+#pragma unroll
+        for (int k = 0; k < 3; k++) {
+            s[k] = 0.0;
+            for (int w = 0; w < 8; w++)
+                s[k] += red[k][w];
+        }
+        const double m = static_cast<double>(n_el);
+        if constexpr (FWD) {
+            // BatchNorm2DTrainForward.h:84-106 from the shifted sums
+            const double d = s[0] / m; // mean - shift
+            const T mn = static_cast<T>(shift + d);
+            const double v = s[1] / m - d * d;
+            const T var = static_cast<T>(v > 0.0 ? v : 0.0);
+            const T sd = sizeof(T) == 4 ? static_cast<T>(sqrtf(static_cast<float>(var + eps))) : static_cast<T>(sqrt(static_cast<double>(var + eps)));
+            mean[c] = mn;
+            inv_var[c] = T(1) / sd;
+            new_ema_mean[c] = (T(1) - mu_) * ema_mean[c] + mu_ * mn;
+            new_ema_var[c] = (T(1) - mu_) * ema_var[c] + mu_ * var;
+            coef[0] = mn;
+            coef[1] = sd;
+        } else {
+            // BatchNorm2DBackward.h:88-118 with the sums taken out of the loops
+            const double iv = static_cast<double>(inv_var[c]), g = static_cast<double>(gamma[c]);
+            dBeta[c] = static_cast<T>(s[0]);
+            dGamma[c] = static_cast<T>(s[1] * iv);
+            const double dVar = -(g * s[1]) * 0.5 * iv * iv * iv;
+            const double c2m = 2.0 / m;
+            const double dMean = -(g * s[0]) * iv + dVar * (-c2m) * s[2];
+            coef[0] = static_cast<T>(dVar * c2m);
+            coef[1] = static_cast<T>(dMean / m);
+        }
+    }
+    __syncthreads();
+    const T g = gamma[c];
+    const T p0 = coef[0], p1 = coef[1];
+    const T mn = FWD ? p0 : mean[c], ivc = FWD ? T(0) : inv_var[c], bt = FWD ? beta[c] : T(0);
+    for (unsigned idx = tid; idx < n_el; idx += 512) {
+        const unsigned n = idx / HW, j = idx - n * HW;
+        const size_t off = (static_cast<size_t>(n) * C + c) * HW + j;
+        const T xv = sx[idx];
+        if constexpr (FWD)
+            res[off] = g * ((xv - mn) / p1) + bt;
+        else
+            res[off] = (sdy[idx] * g) * ivc + p0 * (xv - mn) + p1;
+    }
+}
+
+// Whether a channel's values fit: at most 64 KB of LDS (two workgroups a CU), enough channels to occupy the device or a
+// tensor so small that the launches of the general path would cost more than idle CUs.
+static inline bool chan_fits_lds(const dh_ctx *ctx, size_t N, size_t C, size_t HW, size_t elem, int arrays) {
+    const size_t slice = N * HW * elem * arrays;
+    return slice <= (size_t(64) << 10) && N * HW < (size_t(1) << 31) && C < (size_t(1) << 31) &&
+           (C * 4 >= static_cast<size_t>(ctx->num_cus) || slice * C <= (size_t(8) << 20));
+}
+
 struct ChanPlan {
     size_t S, imgs_per_slice;
 };
@@ -264,6 +366,14 @@ dh_status batchnorm_train_forward(dh_ctx *ctx, T *res, T *new_ema_mean, T *new_e
     if (rows * (cols / C) >= (size_t(1) << 31) * C && rows >= (size_t(1) << 31))
         return dh_fail(DH_ERR_RUNTIME, "BatchNorm2DTrainForward - too many images");
     const size_t HW = cols / C;
+    if (chan_fits_lds(ctx, rows, C, HW, sizeof(T), 1)) {
+        hipLaunchKernelGGL((chan_lds_kernel<T, true>), dim3(static_cast<unsigned>(C)), dim3(512), rows * HW * sizeof(T), ctx->stream, res, in,
+                           static_cast<const T *>(nullptr), static_cast<unsigned>(rows), static_cast<unsigned>(C),
+                           static_cast<unsigned>(HW), mean, inv_var, new_ema_mean, new_ema_var, ema_mean, ema_var, eps, mu, gamma, beta,
+                           static_cast<T *>(nullptr), static_cast<T *>(nullptr));
+        DH_CHECK_LAUNCH();
+        return DH_OK;
+    }
     const ChanPlan p = chan_plan(ctx, rows, C);
     void *wsv = nullptr;
     dh_status st = dh_workspace(ctx, C * p.S * 3 * sizeof(double) + 2 * C * sizeof(T) + 256, &wsv);
@@ -291,6 +401,15 @@ dh_status batchnorm_backward(dh_ctx *ctx, T *dX, T *dGamma, T *dBeta, const T *m
     if (rows == 0 || cols == 0)
         return DH_OK;
     const size_t HW = cols / C;
+    if (chan_fits_lds(ctx, rows, C, HW, sizeof(T), 2)) {
+        hipLaunchKernelGGL((chan_lds_kernel<T, false>), dim3(static_cast<unsigned>(C)), dim3(512), 2 * rows * HW * sizeof(T), ctx->stream, dX,
+                           in, dout, static_cast<unsigned>(rows), static_cast<unsigned>(C), static_cast<unsigned>(HW),
+                           const_cast<T *>(mean), const_cast<T *>(inv_var), static_cast<T *>(nullptr), static_cast<T *>(nullptr),
+                           static_cast<const T *>(nullptr), static_cast<const T *>(nullptr), T(0), T(0), gamma,
+                           static_cast<const T *>(nullptr), dGamma, dBeta);
+        DH_CHECK_LAUNCH();
+        return DH_OK;
+    }
     const ChanPlan p = chan_plan(ctx, rows, C);
     void *wsv = nullptr;
     dh_status st = dh_workspace(ctx, C * p.S * 3 * sizeof(double) + 2 * C * sizeof(T) + 256, &wsv);

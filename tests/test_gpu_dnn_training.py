@@ -22,7 +22,10 @@ def D(ctx, a):
 
 
 @pytest.mark.parametrize("dt", DTYPES)
-@pytest.mark.parametrize("N,C,H,W", [(2, 3, 3, 3), (64, 8, 14, 14), (7, 5, 9, 11), (1, 1, 1, 1), (300, 3, 8, 8), (3, 130, 2, 2)])
+@pytest.mark.parametrize("N,C,H,W", [(2, 3, 3, 3), (64, 8, 14, 14), (7, 5, 9, 11), (1, 1, 1, 1), (300, 3, 8, 8), (3, 130, 2, 2),
+                                     # a channel's values beyond a workgroup's LDS (the general passes), many channels that
+                                     # fit (one read), and a size where the forward fits and the backward in double does not
+                                     (513, 4, 7, 9), (40, 70, 5, 5), (128, 16, 6, 10)])
 def test_batchnorm_train_forward_and_backward(ctx, dt, N, C, H, W):
     rng = np.random.default_rng(N * 7 + C)
     x = (rng.standard_normal((N, C * H * W)) * 2 + 1).astype(dt)
