@@ -227,12 +227,21 @@ __global__ __launch_bounds__(512) void chan_lds_kernel(T *res, const T *x, const
     __shared__ T coef[4];
     const unsigned c = blockIdx.x, tid = threadIdx.x, n_el = N * HW;
     T *sdy = sx + n_el;
-    for (unsigned idx = tid; idx < n_el; idx += 512) {
-        const unsigned n = idx / HW, j = idx - n * HW;
-        const size_t off = (static_cast<size_t>(n) * C + c) * HW + j;
-        sx[idx] = x[off];
-        if constexpr (!FWD)
-            sdy[idx] = dy[off];
+    // a thread's positions, 512 apart, as (image, position in the plane) pairs advanced without divisions
+    const unsigned dn = 512 / HW, dj = 512 % HW;
+    {
+        unsigned n = tid / HW, j = tid % HW;
+        for (unsigned idx = tid; idx < n_el; idx += 512) {
+            const size_t off = (static_cast<size_t>(n) * C + c) * HW + j;
+            sx[idx] = x[off];
+            if constexpr (!FWD)
+                sdy[idx] = dy[off];
+            n += dn;
+            j += dj;
+            const bool wrap = j >= HW;
+            j -= wrap ? HW : 0;
+            n += wrap ? 1 : 0;
+        }
     }
     __syncthreads();
     const double shift = FWD ? static_cast<double>(sx[0]) : static_cast<double>(mean[c]);
@@ -295,14 +304,19 @@ __global__ __launch_bounds__(512) void chan_lds_kernel(T *res, const T *x, const
     const T g = gamma[c];
     const T p0 = coef[0], p1 = coef[1];
     const T mn = FWD ? p0 : mean[c], ivc = FWD ? T(0) : inv_var[c], bt = FWD ? beta[c] : T(0);
+    unsigned n = tid / HW, j = tid % HW;
     for (unsigned idx = tid; idx < n_el; idx += 512) {
-        const unsigned n = idx / HW, j = idx - n * HW;
         const size_t off = (static_cast<size_t>(n) * C + c) * HW + j;
         const T xv = sx[idx];
         if constexpr (FWD)
             res[off] = g * ((xv - mn) / p1) + bt;
         else
             res[off] = (sdy[idx] * g) * ivc + p0 * (xv - mn) + p1;
+        n += dn;
+        j += dj;
+        const bool wrap = j >= HW;
+        j -= wrap ? HW : 0;
+        n += wrap ? 1 : 0;
     }
 }
 
