@@ -397,10 +397,10 @@ struct TsNtArgs {
 // ASSIGN: the product is not stored; it goes on, rounded exactly as the stored one would be, into the distance
 // (C * -2 + row_add[row]) + col_add[col] (three separately rounded operations) and the row's IDXMIN over it: the first
 // position of the strict minimum, NaN never better, position 0 if the first value is NaN or all are.
-// UPDATE (with ASSIGN; float, one step per pair of row blocks with four chunks, i.e. 49..64 columns): the rows, still in
-// the registers they were loaded into - lane group h on row 4 c + h, lane i on vector i, the operand layout of
-// t(P) X - go through the matrix instruction once more against the one-hot of the assignment just found, so that one
-// pass over A gives the assignment, the per-position sums and the counts. The grid is then what the device holds at
+// UPDATE (with ASSIGN; float, one step per pair of row blocks with four chunks, i.e. 49..64 columns): the rows, read
+// back from the wave's staging piece as they were loaded - lane group h on row 4 c + h, lane i on vector i, the
+// operand layout of t(P) X - go through the matrix instruction once more against the one-hot of the assignment just
+// found, so that one pass over A gives the assignment, the per-position sums and the counts. The grid is then what the device holds at
 // once (one partial result per workgroup) and deals the pairs round-robin.
 template <typename T, int NB, bool ASSIGN, int CPG, bool UPDATE = false>
 __global__ __launch_bounds__(256, UPDATE ? (NB == 1 ? 3 : 2) : 1) void ts_nt_kernel(TsNtArgs g) {
@@ -583,7 +583,7 @@ __global__ __launch_bounds__(256, UPDATE ? (NB == 1 ? 3 : 2) : 1) void ts_nt_ker
                 acc_s[a][e] = typename M::acc_t{0, 0, 0, 0};
         }
     }
-    auto finish_pair = [&](AccSet &acc, unsigned pair, const T (&radd)[2][RPL], const Frag &fr) {
+    auto finish_pair = [&](AccSet &acc, unsigned pair, const T (&radd)[2][RPL]) {
         const size_t rbase = (first_pair + static_cast<size_t>(pair) * pair_stride) * 32;
         if constexpr (ASSIGN) {
 #pragma clang fp contract(off)
@@ -730,7 +730,7 @@ __global__ __launch_bounds__(256, UPDATE ? (NB == 1 ? 3 : 2) : 1) void ts_nt_ker
     auto compute_step = [&](const Frag &fr, unsigned pair, unsigned grp) {
         mma_step(accA, fr, grp);
         if (grp + 1 == cg)
-            finish_pair(accA, pair, fr.ra, fr);
+            finish_pair(accA, pair, fr.ra);
     };
     // (pair, grp) of a step and of the one after it, stepped without divisions
     auto advance = [&](unsigned &pair, unsigned &grp) {
@@ -787,22 +787,22 @@ __global__ __launch_bounds__(256, UPDATE ? (NB == 1 ? 3 : 2) : 1) void ts_nt_ker
             load_step(f0, sdone + 1, 0);
             __builtin_amdgcn_sched_barrier(0);
             mma_step(accB, f1, 0);
-            finish_pair(accA, sdone - 1, ra0, f0);
+            finish_pair(accA, sdone - 1, ra0);
             keep(ra1, f1);
             __builtin_amdgcn_sched_barrier(0);
             load_step(f1, sdone + 2 < nsteps ? sdone + 2 : nsteps - 1, 0);
             __builtin_amdgcn_sched_barrier(0);
             mma_step(accA, f0, 0);
-            finish_pair(accB, sdone, ra1, f0);
+            finish_pair(accB, sdone, ra1);
             keep(ra0, f0);
             __builtin_amdgcn_sched_barrier(0);
         }
         if (sdone < nsteps) {
             mma_step(accB, f1, 0);
-            finish_pair(accA, sdone - 1, ra0, f0);
-            finish_pair(accB, sdone, f1.ra, f1);
+            finish_pair(accA, sdone - 1, ra0);
+            finish_pair(accB, sdone, f1.ra);
         } else {
-            finish_pair(accA, sdone - 1, ra0, f0);
+            finish_pair(accA, sdone - 1, ra0);
         }
         return;
     }
