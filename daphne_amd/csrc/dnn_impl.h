@@ -505,7 +505,7 @@ __global__ __launch_bounds__(512) void conv2d_resident_kernel(ConvResidentArgs g
         if (c0 == 0) {
 #pragma unroll
             for (int i = 0; i < KTR; i++)
-                if (tid + i * 512 < g.Kpad)
+                if (static_cast<unsigned>(tid + i * 512) < g.Kpad)
                     ktab[tid + i * 512] = ktreg[i];
             for (unsigned k = tid + KTR * 512; k < g.Kpad; k += 512)
                 ktab[k] = g.ktab[k];

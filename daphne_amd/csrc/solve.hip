@@ -16,8 +16,6 @@ namespace {
 constexpr int SOLVE_THREADS = 1024;
 
 template <typename T> __device__ __forceinline__ T dev_abs(T a) { return a < T(0) ? -a : a; }
-__device__ __forceinline__ float dev_max(float a, float b) { return __builtin_fmaxf(a, b); }
-__device__ __forceinline__ double dev_max(double a, double b) { return __builtin_fmax(a, b); }
 
 template <typename T>
 __global__ __launch_bounds__(SOLVE_THREADS) void lu_solve_kernel(T *lu, T *x, const T *A, size_t lda, const T *b,
