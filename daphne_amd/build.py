@@ -26,8 +26,10 @@ KERNEL_GENERATOR = KERNEL_SRC_DIR / "genHIPKernelInst.py"
 KERNEL_LIB_DIR = CPP_DIR / "lib"
 KERNEL_LIB_PATH = KERNEL_LIB_DIR / "libHIPKernels.so"
 KERNEL_CATALOG_PATH = KERNEL_LIB_DIR / "HIPcatalog.json"
-# host-side C++ of the kernel layer: DAPHNE's include paths, served here by the stand-in headers
-HOST_CXX_FLAGS = ["-std=c++17", "-O1", "-Wall", f"-I{CPP_DIR / 'src'}", f"-I{CPP_DIR / 'standalone'}",
+# host-side C++ of the kernel layer: DAPHNE's include paths, served here by the stand-in headers (two roots: what
+# stands in for DAPHNE's MLIR-dependent context headers, and what stands in for its data structures)
+HOST_CXX_FLAGS = ["-std=c++17", "-O1", "-Wall", f"-I{CPP_DIR}", f"-I{CPP_DIR / 'src'}", f"-I{CPP_DIR / 'standalone' / 'context'}",
+                  f"-I{CPP_DIR / 'standalone' / 'data'}",
                   f"-I{PKG_DIR.parent / 'include'}"]
 
 HIPCC_FLAGS = [

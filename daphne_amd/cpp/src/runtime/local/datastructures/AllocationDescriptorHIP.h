@@ -6,7 +6,9 @@
 // `m->getValues(&alloc_desc)` for a device pointer (the matrix uploads itself on first use and remembers the
 // placement) and to `DataObjectFactory::create<DT>(rows, cols, zero, &alloc_desc)` for a result that exists on the
 // device only. The buffer is shared between the context's registry and every clone of the descriptor that a
-// placement holds; the clone that finds itself the last holder outside the registry unregisters it.
+// placement holds (a view's placements are clones of its parent's, so a view addresses into its parent's buffer);
+// the clone that finds itself the last holder outside the registry unregisters it. The offset forms of the
+// transfers exist in IAllocationDescriptor once patches/0011-dense-matrix-device-views.patch is applied.
 //
 // In DAPHNE this file is src/runtime/local/datastructures/AllocationDescriptorHIP.h.
 #pragma once
@@ -57,6 +59,17 @@ class AllocationDescriptorHIP : public IAllocationDescriptor {
     }
     void transferFrom(std::byte *dst, size_t size) override {
         HIP::check(dh_d2h(HIPContext::get(dctx, device_id)->raw(), dst, data.get(), size));
+    }
+    // the same for a view that starts `offset` bytes into the allocation it shares with its parent
+    void transferToOffset(std::byte *src, size_t size, size_t offset) override {
+        if (!src)
+            throw std::runtime_error("src ptr requested for transfer to device is null");
+        if (size != 0)
+            HIP::check(dh_h2d(HIPContext::get(dctx, device_id)->raw(), data.get() + offset, src, size));
+    }
+    void transferFromOffset(std::byte *dst, size_t size, size_t offset) override {
+        if (size != 0)
+            HIP::check(dh_d2h(HIPContext::get(dctx, device_id)->raw(), dst, data.get() + offset, size));
     }
 
     bool operator==(const IAllocationDescriptor *other) const override {

@@ -79,6 +79,16 @@ template <typename VT> struct VectorizedPipeline<DenseMatrix<VT>> {
         std::vector<DT **> res(numOutputs);
         for (size_t o = 0; o < numOutputs; ++o)
             res[o] = outputs + o;
+        // A view takes over its parent's placements as they are when it is cut (Structure.cpp:24-36), so the device
+        // copies are made current in the whole objects before any task slices them: the row-split inputs are
+        // uploaded once (what cudaPrefetchInputs does, MTWrapper.h:94-114) instead of batch by batch, and a result
+        // the caller brought along is marked as written on the device.
+        for (size_t i = 0; i < numInputs; ++i)
+            if (splits[i] == VectorSplit::ROWS && !isScalar[i] && inputs[i]->getNumRows() > 1)
+                (void)static_cast<const DT *>(inputs[i])->getValues(&alloc_desc);
+        for (size_t o = 0; o < numOutputs; ++o)
+            if (outputs[o] != nullptr && (combines[o] == VectorCombine::ROWS || combines[o] == VectorCombine::COLS))
+                (void)outputs[o]->getValues(&alloc_desc);
 
         const auto &cfg = ctx->getUserConfig();
         const uint64_t shares = std::max<uint64_t>(1, std::min<uint64_t>(cfg.hip_vect_shares, std::max<uint64_t>(len, 1)));

@@ -28,6 +28,15 @@
 #include <string>
 #include <vector>
 
+// Batches are handed to the pipeline body as views, and the body's kernels take their device pointers from
+// getValues(&alloc_desc) on those views. In an unpatched DAPHNE that call returns the base of the parent's device
+// buffer for every view (DenseMatrix.cpp:99-114, 176-182: the cloned placement yields allocation->getData().get()),
+// so every batch after the first would read and write row 0. patches/0011-dense-matrix-device-views.patch makes
+// views address their parent's device buffer at their own offset and announces it with this macro.
+#ifndef DAPHNE_DENSE_MATRIX_DEVICE_VIEWS
+#error "TasksHIP.h needs DenseMatrix views that address device placements at their offset: apply patches/0011-dense-matrix-device-views.patch"
+#endif
+
 template <class DT> class CompiledPipelineTaskHIP : public CompiledPipelineTaskBase<DT> {};
 
 template <typename VT> class CompiledPipelineTaskHIP<DenseMatrix<VT>> : public CompiledPipelineTaskBase<DenseMatrix<VT>> {

@@ -3,7 +3,8 @@
 // the data every task of one pipeline call shares, and how a task cuts its row range out of the inputs.
 #pragma once
 
-#include <DaphneStandalone.h>
+#include <runtime/local/context/DaphneContext.h>
+#include <runtime/local/datastructures/Structure.h>
 
 #include <cstdint>
 #include <functional>

@@ -10,7 +10,7 @@
 #include <string>
 #include <vector>
 
-#include "../../daphne_amd/cpp/daphne_hip_kernels.h"
+#include <daphne_hip_kernels.h>
 
 namespace {
 thread_local std::string g_error;
@@ -86,9 +86,10 @@ size_t th_device_allocations(void *ctx) { return HIPContext::get(static_cast<Dap
     }                                                                                                                   \
     int th_mat_to_host_##SUF(const void *m, T *out) {                                                                   \
         return guarded([&] {                                                                                            \
-            const auto v = static_cast<const DenseMatrix<T> *>(m)->toHost();                                            \
-            if (!v.empty())                                                                                             \
-                std::memcpy(out, v.data(), v.size() * sizeof(T));                                                       \
+            const auto *dm = static_cast<const DenseMatrix<T> *>(m);                                                    \
+            const T *h = dm->getValues();                                                                               \
+            for (size_t r = 0; r < dm->getNumRows(); r++)                                                               \
+                std::memcpy(out + r * dm->getNumCols(), h + r * dm->getRowSkip(), dm->getNumCols() * sizeof(T));        \
         });                                                                                                             \
     }                                                                                                                   \
     void *th_mat_slice_##SUF(const void *m, size_t rl, size_t ru, size_t cl, size_t cu) {                               \

@@ -9,47 +9,14 @@
 #include <stdexcept>
 #include <vector>
 
-#include "../../daphne_amd/cpp/daphne_hip_kernels.h"
+#include <daphne_hip_kernels.h>
 
-static int g_fail = 0, g_checks = 0;
-#define CHECK(cond)                                                                                 \
-    do {                                                                                            \
-        g_checks++;                                                                                 \
-        if (!(cond)) {                                                                              \
-            g_fail++;                                                                               \
-            std::printf("FAILED %s:%d: %s\n", __FILE__, __LINE__, #cond);                           \
-        }                                                                                           \
-    } while (0)
-#define CHECK_THROWS_AS(expr, EX)                                                                   \
-    do {                                                                                            \
-        g_checks++;                                                                                 \
-        bool ok__ = false;                                                                          \
-        try {                                                                                       \
-            expr;                                                                                   \
-        } catch (const EX &) {                                                                      \
-            ok__ = true;                                                                            \
-        } catch (...) {                                                                             \
-        }                                                                                           \
-        if (!ok__) {                                                                                \
-            g_fail++;                                                                               \
-            std::printf("FAILED %s:%d: %s did not throw %s\n", __FILE__, __LINE__, #expr, #EX);     \
-        }                                                                                           \
-    } while (0)
-
-template <class DT> bool equals(const DT *m, const std::vector<typename DT::VT> &exp) { return m->toHost() == exp; }
-template <class DT> bool approx(const DT *m, const std::vector<typename DT::VT> &exp, double eps) {
-    auto v = m->toHost();
-    if (v.size() != exp.size())
-        return false;
-    for (size_t i = 0; i < v.size(); i++)
-        if (!(std::fabs(double(v[i]) - double(exp[i])) <= eps))
-            return false;
-    return true;
-}
+#include "dm_access.h"
+#include "placement_and_tasks.h"
 
 template <typename VT> void run_all(DaphneContext *dctx) {
     using DT = DenseMatrix<VT>;
-    auto G = [&](size_t rows, std::vector<VT> v) { return genGivenVals<DT>(rows, v); };
+    auto G = [&](size_t rows, std::vector<VT> v) { return given<DT>(rows, v); };
 
     // CUDA/MatMulTest.cpp:37-123
     {
@@ -58,7 +25,7 @@ template <typename VT> void run_all(DaphneContext *dctx) {
         auto v2 = G(3, {1, 2, 3});
         DT *res = nullptr;
         HIP::matMul(res, m1, m1, false, false, dctx);
-        CHECK(equals(res, m2v->toHost()));
+        CHECK(equals(res, toHost(m2v)));
         DataObjectFactory::destroy(res);
         res = nullptr;
         HIP::matMul(res, m3, m4, false, false, dctx);
@@ -112,11 +79,11 @@ template <typename VT> void run_all(DaphneContext *dctx) {
         CHECK_THROWS_AS(HIP::ewBinaryMat(static_cast<BinaryOpCode>(999), res, m, m, dctx), std::runtime_error);
         CHECK_THROWS_AS(HIP::ewBinaryMat(BinaryOpCode::ADD, res, m, bad, dctx), std::runtime_error);
         // a view with rowSkip > numCols
-        std::unique_ptr<DT> view(m->slice(0, 2, 1, 3));
+        DT *view = m->slice(0, 2, 1, 3);
         DT *vres = nullptr;
-        HIP::ewBinaryObjSca(BinaryOpCode::MUL, vres, view.get(), VT(2), dctx);
+        HIP::ewBinaryObjSca(BinaryOpCode::MUL, vres, view, VT(2), dctx);
         CHECK(equals(vres, {4, 6, 10, 12}));
-        for (auto *x : {m, rv, cv, bad, res, sca, vres})
+        for (auto *x : {view, m, rv, cv, bad, res, sca, vres})
             DataObjectFactory::destroy(x);
     }
     // EwUnaryMatTest.cpp:148 sqrt domain_error, :62 abs
@@ -223,11 +190,11 @@ template <typename VT> void run_all(DaphneContext *dctx) {
         CHECK(threw);
         auto arg = G(3, {1, 2, 3, 4, 5, 6, 7, 8, 9});
         using DTSel = DenseMatrix<int64_t>;
-        auto sel = genGivenVals<DTSel>(8, {1, 2, 2, 0, 1, 0, 1, 2});
+        auto sel = given<DTSel>(8, {1, 2, 2, 0, 1, 0, 1, 2});
         DT *ex = nullptr;
         HIP::extractCol(ex, arg, sel, dctx);
         CHECK(equals(ex, {2, 3, 3, 1, 2, 1, 2, 3, 5, 6, 6, 4, 5, 4, 5, 6, 8, 9, 9, 7, 8, 7, 8, 9}));
-        auto selbad = genGivenVals<DTSel>(2, {1, 3});
+        auto selbad = given<DTSel>(2, {1, 3});
         threw = false;
         try {
             DT *bad = nullptr;
@@ -251,7 +218,7 @@ template <typename VT> void run_all(DaphneContext *dctx) {
         size_t oh = 0, ow = 0;
         HIP::NN::Pooling::Forward<HIP::NN::Pooling::AVG, DT, DT>::apply(avg, oh, ow, pin, 2, 3, 5, 5, 2, 2, 2, 2, 1, 1, dctx);
         CHECK(oh == 3 && ow == 3);
-        auto av = avg->toHost();
+        auto av = toHost(avg);
         const VT first[9] = {0.25, 1.25, 2.25, 4.25, 10, 12, 9.25, 20, 22};
         bool ok = av.size() == 54;
         for (int i = 0; ok && i < 9; i++)
@@ -261,7 +228,7 @@ template <typename VT> void run_all(DaphneContext *dctx) {
         DT *gv = nullptr, *gm = nullptr;
         HIP::gemv(gv, X, yv, dctx);
         HIP::matMul(gm, X, yv, true, false, dctx);
-        CHECK(equals(gv, gm->toHost()));
+        CHECK(equals(gv, toHost(gm)));
         for (auto *q : {m, mt, m0, m1, cb, arg, ex, in, rl, f, pin, avg, X, yv, gv, gm})
             DataObjectFactory::destroy(q);
         DataObjectFactory::destroy(sel);
@@ -274,7 +241,7 @@ template <typename VT> void run_all(DaphneContext *dctx) {
         HIP::matMul(y, X, w, false, false, dctx);
         HIP::syrk(A, X, true, dctx);
         HIP::matMul(A2, X, X, true, false, dctx);
-        CHECK(equals(A, A2->toHost()));
+        CHECK(equals(A, toHost(A2)));
         HIP::matMul(b, X, y, true, false, dctx);
         HIP::solve(sol, A, b, dctx);
         CHECK(approx(sol, {1, 2, 3}, sizeof(VT) == 4 ? 1e-3 : 1e-6));
@@ -287,7 +254,7 @@ template <typename VT> void run_all(DaphneContext *dctx) {
 // DNNBatchNorm2DBackwardTest.cpp:22-70, DNNBatchNorm2DForwardTest.cpp:51-90)
 template <typename VT> void run_training(DaphneContext *dctx) {
     using DT = DenseMatrix<VT>;
-    auto G = [&](size_t rows, std::vector<VT> v) { return genGivenVals<DT>(rows, v); };
+    auto G = [&](size_t rows, std::vector<VT> v) { return given<DT>(rows, v); };
     {
         auto dy = G(1, {1, 2, 3, 4, 5, 6, 7, 8});
         auto filter = G(2, {1, 0, 0, 2, 2, 0, 0, 3, 3, 0, 0, 4, 5, 0, 0, 6, 6, 0, 0, 7, 7, 0, 0, 8});
@@ -335,7 +302,7 @@ template <typename VT> void run_training(DaphneContext *dctx) {
         HIP::BatchNorm2DBackward<DT, DT>::apply(dX, dG, dB, mean, invVar, in, dout, gamma, VT(1e-5), dctx);
         CHECK(approx(dG, {8.9442, 8.9442, 8.9442}, 1e-3));
         CHECK(approx(dB, {20, 52, 84}, 1e-4));
-        CHECK(std::fabs(double(dX->toHost()[0]) + 1.0733e-05) < 1e-5);
+        CHECK(std::fabs(double(toHost(dX)[0]) + 1.0733e-05) < 1e-5);
         // training forward: statistics of the batch, output normalised per channel
         DT *res = nullptr, *nm = nullptr, *nv = nullptr, *mn = nullptr, *iv2 = nullptr;
         auto zeros = G(3, {0, 0, 0}), ones = G(3, {1, 1, 1});
@@ -343,7 +310,7 @@ template <typename VT> void run_training(DaphneContext *dctx) {
         CHECK(approx(mn, {2.5, 6.5, 10.5}, 1e-5));
         CHECK(approx(nv, {1.25, 1.25, 1.25}, 1e-5));
         CHECK(approx(iv2, {ivv, ivv, ivv}, 1e-5));
-        CHECK(std::fabs(double(res->toHost()[0]) - (1 - 2.5) * double(ivv)) < 1e-5);
+        CHECK(std::fabs(double(toHost(res)[0]) - (1 - 2.5) * double(ivv)) < 1e-5);
         for (auto *m : {in, dout, gamma, mean, invVar, dX, dG, dB, res, nm, nv, mn, iv2, zeros, ones})
             DataObjectFactory::destroy(m);
     }
@@ -353,12 +320,12 @@ template <typename VT> void run_training(DaphneContext *dctx) {
 // int64_t among others): the reference's literals where they are integers, plus integer-only behaviour.
 template <typename VT> void run_integer_elementwise(DaphneContext *dctx) {
     using DT = DenseMatrix<VT>;
-    auto G = [&](size_t rows, std::vector<VT> v) { return genGivenVals<DT>(rows, v); };
+    auto G = [&](size_t rows, std::vector<VT> v) { return given<DT>(rows, v); };
     // EwBinaryMatTest.cpp:69-102 (add), :104-125 (mul), :178-222 (div), :523-557 (max)
     auto m1 = G(2, {1, 2, 0, 0, 1, 3}), m2 = G(2, {0, 9, 0, 0, 3, 4}), m3 = G(2, {1, 11, 0, 0, 4, 7});
     DT *res = nullptr;
     HIP::ewBinaryMat(BinaryOpCode::ADD, res, m1, m2, dctx);
-    CHECK(equals(res, m3->toHost()));
+    CHECK(equals(res, toHost(m3)));
     HIP::ewBinaryMat(BinaryOpCode::MUL, res, m1, m2, dctx);
     CHECK(equals(res, {0, 18, 0, 0, 3, 12}));
     HIP::ewBinaryMat(BinaryOpCode::MAX, res, m1, m2, dctx);
@@ -381,7 +348,7 @@ template <typename VT> void run_integer_elementwise(DaphneContext *dctx) {
 
 static void run_si64(DaphneContext *dctx) {
     using DT = DenseMatrix<int64_t>;
-    auto G = [&](size_t rows, std::vector<int64_t> v) { return genGivenVals<DT>(rows, v); };
+    auto G = [&](size_t rows, std::vector<int64_t> v) { return given<DT>(rows, v); };
     // AggRowTest.cpp / AggColTest.cpp literal, AggAllTest.cpp:62-75
     auto m = G(3, {3, 0, 2, 0, 0, 0, 1, 0, 0, 1, 0, 3});
     CHECK(HIP::aggAll<int64_t>(AggOpCode::SUM, m, dctx) == 10);
@@ -405,248 +372,6 @@ static void run_si64(DaphneContext *dctx) {
     for (auto *x : {m, r, c, t, b, f})
         DataObjectFactory::destroy(x);
     DataObjectFactory::destroy(idx);
-}
-
-// ------------------------------------------------------------------------------------------------
-// Data placement: what DenseMatrix::getValues(&alloc_desc) and AllocationDescriptorHIP do together
-// (DenseMatrix.cpp:126-234, AllocationDescriptorCUDA.h:24-75)
-// ------------------------------------------------------------------------------------------------
-template <class DT> int whereIs(const DT *m) {
-    const MetaDataObject *mdo = m->getMetaDataObject();
-    int where = 0;
-    for (size_t id : mdo->getLatest())
-        where |= mdo->getDataPlacementByID(id)->allocation->getType() == ALLOCATION_TYPE::HOST ? 1 : 2;
-    return where;
-}
-static void run_placement(DaphneContext *dctx) {
-    using DT = DenseMatrix<float>;
-    HIPContext *hc = HIPContext::get(dctx, 0);
-    const size_t allocs0 = hc->numAllocations();
-    const size_t used0 = hc->getMemInUse();
-    auto a = genGivenVals<DT>(2, {1, 2, 3, 4, 5, 6});
-    CHECK(whereIs(a) == 1 && a->getMetaDataObject()->numDataPlacements() == 1); // host only, nothing uploaded yet
-    CHECK(hc->numAllocations() == allocs0);
-    DT *r = nullptr;
-    HIP::ewBinaryObjSca(BinaryOpCode::MUL, r, a, 2.0f, dctx);
-    // the input was uploaded on first use and both copies stay valid; the result exists on the device only
-    CHECK(whereIs(a) == 3 && a->getMetaDataObject()->numDataPlacements() == 2);
-    CHECK(whereIs(r) == 2 && r->getMetaDataObject()->numDataPlacements() == 1);
-    CHECK(hc->numAllocations() == allocs0 + 2);
-    // a second use finds the device copy: no further placement, no further allocation
-    DT *r2 = nullptr;
-    HIP::ewBinaryMat(BinaryOpCode::ADD, r2, a, r, dctx);
-    CHECK(a->getMetaDataObject()->numDataPlacements() == 2 && hc->numAllocations() == allocs0 + 3);
-    // reading the result on the host downloads it once; both copies are then current
-    CHECK(equals(r2, {3, 6, 9, 12, 15, 18}));
-    CHECK(whereIs(r2) == 3);
-    // writing on the host makes the device copy stale; the next kernel uploads again and sees the new value
-    a->set(0, 0, 10.f);
-    CHECK(whereIs(a) == 1);
-    HIP::ewBinaryObjSca(BinaryOpCode::MUL, r, a, 2.0f, dctx); // in place into r
-    CHECK(whereIs(a) == 3 && whereIs(r) == 2);
-    CHECK(equals(r, {20, 4, 6, 8, 10, 12}));
-    // a kernel that writes into a matrix makes its host copy stale
-    HIP::ewBinaryObjSca(BinaryOpCode::ADD, a, a, 1.0f, dctx);
-    CHECK(whereIs(a) == 2);
-    CHECK(equals(a, {11, 3, 4, 5, 6, 7}));
-    // views share their parent's placements: a kernel on a view sees device data without another upload
-    std::unique_ptr<DT> v(a->sliceRow(1, 2));
-    DT *rv = nullptr;
-    HIP::ewBinaryObjSca(BinaryOpCode::SUB, rv, v.get(), 1.0f, dctx);
-    CHECK(equals(rv, {4, 5, 6}));
-    CHECK(a->getMetaDataObject()->numDataPlacements() == 2);
-    v.reset();
-    // destroying the matrices gives the device memory back
-    DataObjectFactory::destroy(a, r, r2, rv);
-    CHECK(hc->numAllocations() == allocs0);
-    CHECK(hc->getMemInUse() == used0);
-}
-
-// ------------------------------------------------------------------------------------------------
-// Vectorized pipeline on the device: tasks over row shares, outputs combined
-// (MultiThreadedKernelTest.cpp:30-154 bodies; TasksCUDA.cpp:21-119; MTWrapper_dense.cpp:339-373)
-// ------------------------------------------------------------------------------------------------
-// bodies as the compiler outlines them: operator by operator, results through *outputs[i], inputs given back
-template <class DT> void funAdd(DT ***outputs, Structure **inputs, DCTX(ctx)) {
-    auto *l = static_cast<DT *>(inputs[0]), *r = static_cast<DT *>(inputs[1]);
-    HIP::ewBinaryMat(BinaryOpCode::ADD, *outputs[0], l, r, ctx);
-    DataObjectFactory::destroy(l, r);
-}
-template <class DT> void funMul(DT ***outputs, Structure **inputs, DCTX(ctx)) {
-    auto *l = static_cast<DT *>(inputs[0]), *r = static_cast<DT *>(inputs[1]);
-    HIP::ewBinaryMat(BinaryOpCode::MUL, *outputs[0], l, r, ctx);
-    DataObjectFactory::destroy(l, r);
-}
-// a body that ignores the offered output and returns a matrix of its own, like the reference's compiled bodies
-template <class DT> void funAddFresh(DT ***outputs, Structure **inputs, DCTX(ctx)) {
-    auto *l = static_cast<DT *>(inputs[0]), *r = static_cast<DT *>(inputs[1]);
-    DT *fresh = nullptr;
-    HIP::ewBinaryMat(BinaryOpCode::ADD, fresh, l, r, ctx);
-    *outputs[0] = fresh;
-    DataObjectFactory::destroy(l, r);
-}
-// outputs: 0 = (x - mu) * (x - mu) by ROWS, 1 = column sums by ADD, 2 = column minima by MIN, 3 = column maxima by MAX
-template <class DT> void funStats(DT ***outputs, Structure **inputs, DCTX(ctx)) {
-    auto *x = static_cast<DT *>(inputs[0]), *mu = static_cast<DT *>(inputs[1]);
-    DT *c = nullptr;
-    HIP::ewBinaryMat(BinaryOpCode::SUB, c, x, mu, ctx);
-    HIP::ewBinaryMat(BinaryOpCode::MUL, *outputs[0], c, c, ctx);
-    HIP::aggCol(AggOpCode::SUM, *outputs[1], x, ctx);
-    HIP::aggCol(AggOpCode::MIN, *outputs[2], x, ctx);
-    HIP::aggCol(AggOpCode::MAX, *outputs[3], x, ctx);
-    DataObjectFactory::destroy(c, x, mu);
-}
-
-template <typename VT> void run_pipeline_tasks(DaphneContext *dctx) {
-    using DT = DenseMatrix<VT>;
-    using Fn = void (*)(DT ***, Structure **, DCTX(ctx));
-    const size_t rows = 1234, cols = 10;
-    std::vector<VT> a(rows * cols), b(rows * cols);
-    uint32_t s = 12345u;
-    auto rnd = [&] { // values in [0, 1), as randMatrix(..., 0.0, 1.0, ...) in the reference's test
-        s = s * 1664525u + 1013904223u;
-        return VT((s >> 8) * (1.0 / 16777216.0));
-    };
-    for (auto &v : a)
-        v = rnd();
-    for (auto &v : b)
-        v = rnd();
-    auto m1 = genGivenVals<DT>(rows, a), m2 = genGivenVals<DT>(rows, b);
-    bool isScalar[] = {false, false};
-    Structure *inputs[] = {m1, m2};
-    int64_t outRows[] = {int64_t(rows)}, outCols[] = {int64_t(cols)};
-    int64_t splits[] = {int64_t(VectorSplit::ROWS), int64_t(VectorSplit::ROWS)};
-    int64_t combines[] = {int64_t(VectorCombine::ROWS)};
-    struct Case {
-        uint64_t shares, batch;
-    };
-    const Case cases[] = {{1, 0}, {2, 0}, {7, 0}, {3, 100}, {1, 1000}};
-    for (Fn fn : {Fn(&funAdd<DT>), Fn(&funMul<DT>), Fn(&funAddFresh<DT>)}) {
-        DT *whole = nullptr; // single call on the whole matrices
-        HIP::ewBinaryMat(fn == Fn(&funMul<DT>) ? BinaryOpCode::MUL : BinaryOpCode::ADD, whole, m1, m2, dctx);
-        const auto expect = whole->toHost();
-        bool host_ok = true;
-        for (size_t i = 0; i < expect.size(); i++)
-            host_ok &= expect[i] == (fn == Fn(&funMul<DT>) ? a[i] * b[i] : a[i] + b[i]);
-        CHECK(host_ok);
-        for (const Case &c : cases) {
-            dctx->config.hip_vect_shares = c.shares;
-            dctx->config.hip_vect_batch_rows = c.batch;
-            DT *out[] = {nullptr};
-            void *fun[] = {reinterpret_cast<void *>(fn)};
-            HIP::vectorizedPipeline<DT>(out, 1, isScalar, inputs, 2, outRows, outCols, splits, combines, 1, fun, dctx);
-            CHECK(out[0] != nullptr && out[0]->getNumRows() == rows && out[0]->getNumCols() == cols);
-            CHECK(whereIs(out[0]) == 2); // combined on the device, not through the host
-            CHECK(out[0]->toHost() == expect); // ROWS: bit for bit the whole-matrix result
-            DataObjectFactory::destroy(out[0]);
-        }
-        DataObjectFactory::destroy(whole);
-    }
-    CHECK(m1->getRefCounter() == 1 && m2->getRefCounter() == 1);
-
-    // ROWS + ADD + MIN + MAX in one pipeline, a broadcast input, op-by-op body
-    {
-        DT *mu = nullptr;
-        HIP::aggCol(AggOpCode::MEAN, mu, m1, dctx);
-        DT *c = nullptr, *sq = nullptr, *sum = nullptr, *mn = nullptr, *mx = nullptr;
-        HIP::ewBinaryMat(BinaryOpCode::SUB, c, m1, mu, dctx);
-        HIP::ewBinaryMat(BinaryOpCode::MUL, sq, c, c, dctx);
-        HIP::aggCol(AggOpCode::SUM, sum, m1, dctx);
-        HIP::aggCol(AggOpCode::MIN, mn, m1, dctx);
-        HIP::aggCol(AggOpCode::MAX, mx, m1, dctx);
-        bool isScalar2[] = {false, false};
-        Structure *inputs2[] = {m1, mu};
-        int64_t outRows2[] = {int64_t(rows), 1, 1, 1}, outCols2[] = {int64_t(cols), int64_t(cols), int64_t(cols), int64_t(cols)};
-        int64_t splits2[] = {int64_t(VectorSplit::ROWS), int64_t(VectorSplit::NONE)};
-        int64_t combines2[] = {int64_t(VectorCombine::ROWS), int64_t(VectorCombine::ADD), int64_t(VectorCombine::MIN),
-                               int64_t(VectorCombine::MAX)};
-        const double tol = std::is_same<VT, float>::value ? 1e-4 : 1e-12; // sums of 1234 values in [0,1) in another order
-        for (const Case &cs : cases) {
-            dctx->config.hip_vect_shares = cs.shares;
-            dctx->config.hip_vect_batch_rows = cs.batch;
-            DT *out[] = {nullptr, nullptr, nullptr, nullptr};
-            void *fun[] = {reinterpret_cast<void *>(Fn(&funStats<DT>))};
-            HIP::vectorizedPipeline<DT>(out, 4, isScalar2, inputs2, 2, outRows2, outCols2, splits2, combines2, 1, fun, dctx);
-            CHECK(out[0]->toHost() == sq->toHost());
-            const auto got = out[1]->toHost(), want = sum->toHost();
-            bool ok = got.size() == want.size();
-            for (size_t i = 0; ok && i < got.size(); i++)
-                ok = std::fabs(double(got[i]) - double(want[i])) <= tol * std::fabs(double(want[i]));
-            CHECK(ok);
-            CHECK(out[2]->toHost() == mn->toHost()); // MIN / MAX do not depend on the order
-            CHECK(out[3]->toHost() == mx->toHost());
-            DataObjectFactory::destroy(out[0], out[1], out[2], out[3]);
-        }
-        CHECK(mu->getRefCounter() == 1);
-        DataObjectFactory::destroy(mu, c, sq, sum, mn, mx);
-    }
-
-    // the same shape of work as ONE kernel per batch: z = (x - mu) / sd by ROWS, r = rowSums(z * z) by ROWS,
-    // count of r > thr by ADD, largest r by MAX
-    {
-        DT *mu = nullptr, *var = nullptr, *sd = nullptr;
-        HIP::aggCol(AggOpCode::MEAN, mu, m1, dctx);
-        HIP::aggCol(AggOpCode::VAR, var, m1, dctx);
-        HIP::ewUnaryMat(UnaryOpCode::SQRT, sd, var, dctx);
-        const VT thr = VT(10);
-        auto I = [](int kind, int op, int domain, int operand, int index, double scalar = 0) {
-            return dh_pipe_instr{kind, op, domain, operand, index, 0, scalar};
-        };
-        HIP::FusedPipelineBody<VT> body;
-        body.program = {I(DH_PIPE_EW_BINARY, int(BinaryOpCode::SUB), 0, DH_OPD_ROWVEC, 0),
-                        I(DH_PIPE_EW_BINARY, int(BinaryOpCode::DIV), 0, DH_OPD_ROWVEC, 1),
-                        I(DH_PIPE_STORE_TILE, 0, 0, 0, 0),
-                        I(DH_PIPE_EW_BINARY, int(BinaryOpCode::MUL), 0, DH_OPD_SELF, 0),
-                        I(DH_PIPE_ROW_AGG, int(AggOpCode::SUM), 0, 0, 0),
-                        I(DH_PIPE_STORE_ROW, 0, 1, 0, 0),
-                        I(DH_PIPE_REDUCE_ALL, int(AggOpCode::MAX), 1, 0, 1),
-                        I(DH_PIPE_EW_BINARY, int(BinaryOpCode::GT), 1, DH_OPD_SCALAR, 0, double(thr)),
-                        I(DH_PIPE_REDUCE_ALL, int(AggOpCode::SUM), 1, 0, 0)};
-        body.inputs = {{HIP::PipeInput::PRIMARY, 0}, {HIP::PipeInput::ROWVEC, 0}, {HIP::PipeInput::ROWVEC, 1}};
-        body.outputs = {{HIP::PipeOutput::TILE, 0}, {HIP::PipeOutput::ROW, 0}, {HIP::PipeOutput::ALL, 0}, {HIP::PipeOutput::ALL, 1}};
-        // op by op on the whole matrix
-        DT *c = nullptr, *z = nullptr, *zz = nullptr, *r = nullptr, *gt = nullptr;
-        HIP::ewBinaryMat(BinaryOpCode::SUB, c, m1, mu, dctx);
-        HIP::ewBinaryMat(BinaryOpCode::DIV, z, c, sd, dctx);
-        HIP::ewBinaryMat(BinaryOpCode::MUL, zz, z, z, dctx);
-        HIP::aggRow(AggOpCode::SUM, r, zz, dctx);
-        HIP::ewBinaryObjSca(BinaryOpCode::GT, gt, r, thr, dctx);
-        const VT count = HIP::aggAll<VT, DT>(AggOpCode::SUM, gt, dctx), rmax = HIP::aggAll<VT, DT>(AggOpCode::MAX, r, dctx);
-        CHECK(count > VT(0) && count < VT(rows)); // the threshold splits the rows
-        bool isScalar3[] = {false, false, false};
-        Structure *inputs3[] = {m1, mu, sd};
-        int64_t outRows3[] = {int64_t(rows), int64_t(rows), 1, 1}, outCols3[] = {int64_t(cols), 1, 1, 1};
-        int64_t splits3[] = {int64_t(VectorSplit::ROWS), int64_t(VectorSplit::NONE), int64_t(VectorSplit::NONE)};
-        VectorCombine combines3[] = {VectorCombine::ROWS, VectorCombine::ROWS, VectorCombine::ADD, VectorCombine::MAX};
-        const double tol = std::is_same<VT, float>::value ? 1e-5 : 1e-13;
-        for (const Case &cs : cases) {
-            dctx->config.hip_vect_shares = cs.shares;
-            dctx->config.hip_vect_batch_rows = cs.batch;
-            DT *out[] = {nullptr, nullptr, nullptr, nullptr};
-            std::vector<std::function<void(DT ***, Structure **, DCTX(ctx))>> funcs{body};
-            HIP::VectorizedPipeline<DT>::apply(out, 4, isScalar3, inputs3, 3, outRows3, outCols3,
-                                               reinterpret_cast<const VectorSplit *>(splits3), combines3, funcs, dctx);
-            CHECK(out[0]->toHost() == z->toHost()); // same IEEE operations per element: bit for bit
-            const auto got = out[1]->toHost(), want = r->toHost();
-            bool ok = got.size() == want.size();
-            for (size_t i = 0; ok && i < got.size(); i++)
-                ok = std::fabs(double(got[i]) - double(want[i])) <= tol * std::fabs(double(want[i]));
-            CHECK(ok);
-            // rows whose r is within rounding of the threshold may fall on either side
-            size_t ambiguous = 0;
-            for (VT v : want)
-                ambiguous += std::fabs(double(v) - double(thr)) <= tol * double(thr);
-            CHECK(std::fabs(double(out[2]->toHost()[0]) - double(count)) <= double(ambiguous));
-            CHECK(std::fabs(double(out[3]->toHost()[0]) - double(rmax)) <= tol * double(rmax));
-            DataObjectFactory::destroy(out[0], out[1], out[2], out[3]);
-        }
-        DataObjectFactory::destroy(mu, var, sd, c, z);
-        DataObjectFactory::destroy(zz, r, gt);
-    }
-    dctx->config.hip_vect_shares = 1;
-    dctx->config.hip_vect_batch_rows = 0;
-    CHECK(m1->getRefCounter() == 1);
-    DataObjectFactory::destroy(m1, m2);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -675,7 +400,7 @@ static void run_generated_wrappers(DaphneContext *dctx, const char *lib_path) {
                                                           "script.daphne", 3, 7);
     const int kSum = dctx->dispatchMapping.registerKernel("HIP_sumAll__double__DenseMatrix_double", "script.daphne", 4, 1);
     const int kSqrt = dctx->dispatchMapping.registerKernel("HIP_ewSqrt__DenseMatrix_double__DenseMatrix_double", "script.daphne", 5, 2);
-    auto a = genGivenVals<DT>(2, {1, 2, 3, 4}), b = genGivenVals<DT>(2, {10, 20, 30, 40}), bad = genGivenVals<DT>(3, {1, 2, 3});
+    auto a = given<DT>(2, {1, 2, 3, 4}), b = given<DT>(2, {10, 20, 30, 40}), bad = given<DT>(3, {1, 2, 3});
     dctx->config.enable_statistics = true;
     DT *res = nullptr;
     ewAdd(&res, a, b, kAdd, dctx);
@@ -696,7 +421,7 @@ static void run_generated_wrappers(DaphneContext *dctx, const char *lib_path) {
     CHECK(what.find("The kernel-function HIP_ewAdd__DenseMatrix_double__DenseMatrix_double__DenseMatrix_double failed during runtime") == 0);
     CHECK(what.find("script.daphne:3:7") != std::string::npos);
     what.clear();
-    auto neg = genGivenVals<DT>(1, {4, -1});
+    auto neg = given<DT>(1, {4, -1});
     try {
         DT *r3 = nullptr;
         ewSqrt(&r3, neg, kSqrt, dctx);
