@@ -1,7 +1,8 @@
 // The whole HIP kernel layer in one include: every kernel header of src/runtime/local/kernels/HIP, the device
 // context, the allocation descriptor and the vectorized-pipeline task. Include paths needed:
 //   <this directory>/src          the files that go into DAPHNE's src/ tree (same relative paths)
-//   <this directory>/standalone   stand-ins for DAPHNE's own headers; leave out when building inside DAPHNE
+//   <this directory>/standalone/context, <this directory>/standalone/data
+//                                 stand-ins for DAPHNE's own headers; leave out when building inside DAPHNE
 //   <repository>/include          daphne_hip.h, the C ABI of libdaphne_hip.so
 #pragma once
 

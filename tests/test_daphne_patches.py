@@ -17,7 +17,7 @@ needs_reference = pytest.mark.skipif(not (REF / "src").is_dir(), reason="the ref
 @needs_reference
 def test_patches_apply_to_the_reference_tree(tmp_path):
     patches = sorted((CPP / "patches").glob("*.patch"))
-    assert len(patches) >= 10
+    assert len(patches) >= 11
     for p in patches:
         for line in p.read_text().splitlines():
             if line.startswith("--- a/"):
