@@ -50,6 +50,35 @@ def measured_traffic(kernel: str):
 
 
 
+def time_stage_via_wrappers(x_ptr: int, rows: int, cols: int, thr: float, steps: int):
+    """ms per run of the fused stage through the generated kernel entry points (tests/cpp/glue_harness.cpp builds the
+    run-time objects those take). None if the harness or the kernel library was not built."""
+    import ctypes as C
+
+    from daphne_amd import build as b
+
+    harness = os.path.join(ROOT, "tests", "cpp", "build", "libglue_harness.so")
+    if not (os.path.exists(harness) and os.path.exists(b.KERNEL_LIB_PATH)):
+        return None
+    h = C.CDLL(harness)
+    h.th_ctx_create.restype = C.c_void_p
+    h.th_last_error.restype = C.c_char_p
+    h.th_ctx_destroy.argtypes = [C.c_void_p]
+    f = h.th_time_zscore_stage_f32
+    f.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_size_t, C.c_size_t, C.c_float, C.c_int, C.c_int] + [C.POINTER(C.c_double)] * 4
+    dctx = h.th_ctx_create()
+    if not dctx:
+        raise RuntimeError(h.th_last_error().decode())
+    out = [C.c_double() for _ in range(4)]
+    try:
+        if f(dctx, str(b.KERNEL_LIB_PATH).encode(), C.c_void_p(x_ptr), rows, cols, thr, 1, steps, *[C.byref(o) for o in out]) != 0:
+            raise RuntimeError(h.th_last_error().decode())
+    finally:
+        h.th_ctx_destroy(dctx)
+    return {"ms_by_operators": out[0].value, "ms_as_one_kernel": out[1].value, "count_by_operators": out[2].value,
+            "count_as_one_kernel": out[3].value, "steps": steps}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -67,6 +96,8 @@ def main() -> int:
     ap.add_argument("--cpu-reps", type=int, default=3, help="repetitions of the CPU baseline (median is reported)")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-contractions", action="store_true", help="skip the MatMul / Syrk measurements after the pipeline")
+    ap.add_argument("--no-wrappers", action="store_true",
+                    help="skip timing the fused stage through the generated HIP_<mnemonic> entry points of libHIPKernels.so")
     ap.add_argument("--contraction-steps", type=int, default=5)
     ap.add_argument("--calib", action="store_true",
                     help="also launch one plain elementwise copy of X (reads |X|, writes |X|): the known-size "
@@ -179,6 +210,16 @@ def main() -> int:
 
     pipeline_mode = int(capi.lib().dh_vectorized_pipeline_last_mode())
 
+    # The same fused stage the way a DAPHNE program compiled with --hip reaches it: through the generated
+    # HIP_<mnemonic> entry points of libHIPKernels.so, as the outlined device body (one entry point per operator) and
+    # as HIP_fusedPipeline with the body's text (lowered to the one kernel at run time).
+    via_wrappers = None
+    if not args.no_wrappers:
+        via_wrappers = time_stage_via_wrappers(int(X_t.data_ptr()), R, Cc, thr, max(1, min(args.steps, 5)))
+        if via_wrappers is not None and via_wrappers["count_by_operators"] != via_wrappers["count_as_one_kernel"]:
+            print(f"bench.py: the two forms of the fused stage disagree: {via_wrappers}", file=sys.stderr)
+            return 4
+
     xh = None
     if not args.no_cpu:
         xh = X_t[:min(args.cpu_rows, R)].cpu().numpy()
@@ -241,6 +282,10 @@ def main() -> int:
                           "fused_pipeline": round(bytes_s3 / t_s3 / 1e6, 1)},
             "count_r_gt_thr": s_val,
             "pipeline_mode": "specialised" if pipeline_mode == 1 else "interpreted",
+            # the fused stage as a patched DAPHNE dispatches it, through libHIPKernels.so: the outlined body (one entry
+            # point per operator, every intermediate in memory) and HIP_fusedPipeline with the body's text (one launch)
+            "ms_fused_stage_op_by_op_via_wrappers": None if via_wrappers is None else round(via_wrappers["ms_by_operators"], 4),
+            "ms_fused_stage_via_fusedPipeline_wrapper": None if via_wrappers is None else round(via_wrappers["ms_as_one_kernel"], 4),
             "contractions": contractions,
             "device": props["name"], "compute_units": props["compute_units"], "clock_khz": props["clock_khz"],
         },

@@ -30,6 +30,7 @@
 #include <runtime/local/kernels/HIP/FusedPipeline.h>
 #include <runtime/local/kernels/HIP/Gemv.h>
 #include <runtime/local/kernels/HIP/MatMul.h>
+#include <runtime/local/kernels/HIP/PipelineProgramBuilder.h>
 #include <runtime/local/kernels/HIP/Pooling.h>
 #include <runtime/local/kernels/HIP/PoolingBackward.h>
 #include <runtime/local/kernels/HIP/Softmax.h>

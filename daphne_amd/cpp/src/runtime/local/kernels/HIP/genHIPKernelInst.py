@@ -255,6 +255,13 @@ def render_cpp(wrappers: list[Wrapper], api: str = "HIP") -> str:
             lines += ["    // " + "-" * 76, "    // " + w.op_name, "    // " + "-" * 76]
             last = w.op_name
         lines.append(w.definition().rstrip("\n"))
+    if any(w.op_name == "fusedPipeline" for w in wrappers):
+        # not kernels (and not in the catalog): how the calling thread's last fusedPipeline call ran
+        lines += ["    // " + "-" * 76,
+                  "    // diagnostics of fusedPipeline: 1 one kernel per batch, 0 operator by operator (and why), -1 none yet",
+                  "    // " + "-" * 76,
+                  f"    int {api}_fusedPipeline_lastMode() {{ return {api}::fusedPipelineLastMode(); }}",
+                  f"    const char *{api}_fusedPipeline_lastReason() {{ return {api}::fusedPipelineLastReason().c_str(); }}"]
     lines += ["}", ""]
     return "\n".join(lines)
 

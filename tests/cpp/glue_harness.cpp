@@ -12,6 +12,8 @@
 
 #include <daphne_hip_kernels.h>
 
+#include "zscore_via_wrappers.h"
+
 namespace {
 thread_local std::string g_error;
 template <class F> int guarded(F &&f) {
@@ -140,5 +142,55 @@ TH_MATRIX(ui32, uint32_t)
 TH_PIPELINE(f32, float)
 TH_PIPELINE(f64, double)
 #undef TH_PIPELINE
+
+// Times the fused stage of the z-score pipeline over x (rows x cols floats in device memory) the two ways a DAPHNE
+// program compiled with --hip can run it, both through the generated entry points of the kernel library at
+// `kernel_lib`: HIP_fusedPipeline without the body's text (the outlined body: one HIP_<mnemonic> call per operator,
+// every intermediate in memory) and with it (one launch). Milliseconds per run from the context's stream stopwatch.
+int th_time_zscore_stage_f32(void *ctx, const char *kernel_lib, const float *x_dev, size_t rows, size_t cols, float thr, int warmup,
+                             int steps, double *ms_by_operators, double *ms_as_one_kernel, double *count_by_operators,
+                             double *count_as_one_kernel) {
+    return guarded([&] {
+        using Z = ZscoreViaWrappers<float>;
+        using DT = DenseMatrix<float>;
+        auto *dctx = static_cast<DaphneContext *>(ctx);
+        void *lib = dlopen(kernel_lib, RTLD_NOW | RTLD_LOCAL);
+        if (!lib)
+            throw std::runtime_error(std::string("cannot load the kernel library: ") + dlerror());
+        if (!Z::load(lib))
+            throw std::runtime_error("the kernel library lacks an entry point of the z-score pipeline");
+        AllocationDescriptorHIP alloc_desc(dctx, 0);
+        dh_ctx *raw = HIPContext::get(dctx, 0)->raw();
+        DT *x = DataObjectFactory::create<DT>(rows, cols, false, &alloc_desc);
+        HIP::check(dh_d2d(raw, x->getValues(&alloc_desc), x_dev, rows * cols * sizeof(float)));
+        DT *mu = nullptr, *var = nullptr, *sd = nullptr;
+        HIP::aggCol(AggOpCode::MEAN, mu, x, dctx);
+        HIP::aggCol(AggOpCode::VAR, var, x, dctx);
+        HIP::ewUnaryMat(UnaryOpCode::SQRT, sd, var, dctx);
+        const int kId = dctx->dispatchMapping.registerKernel("_vect_hip1", "bench", 0, 0);
+        double *ms_out[] = {ms_by_operators, ms_as_one_kernel}, *count_out[] = {count_by_operators, count_as_one_kernel};
+        for (int described = 0; described < 2; described++) {
+            DT *out[] = {nullptr, nullptr};
+            for (int i = 0; i < warmup + steps; i++) {
+                if (i == warmup)
+                    HIP::check(dh_timer_start(raw));
+                if (out[1] != nullptr) { // the count is folded into its result: start it from nothing each run
+                    DataObjectFactory::destroy(out[1]);
+                    out[1] = nullptr;
+                }
+                Z::run(out, x, mu, sd, double(thr), described != 0, kId, dctx);
+            }
+            float ms = 0;
+            HIP::check(dh_timer_stop_ms(raw, &ms));
+            if (Z::entry().lastMode() != described)
+                throw std::runtime_error(std::string("the fused stage did not run the way it was asked to: ") + Z::entry().lastReason());
+            *ms_out[described] = double(ms) / double(steps);
+            *count_out[described] = double(static_cast<const DT *>(out[1])->getValues()[0]);
+            DataObjectFactory::destroy(out[0], out[1]);
+        }
+        DataObjectFactory::destroy(x, mu, var, sd);
+        dlclose(lib);
+    });
+}
 
 } // extern "C"

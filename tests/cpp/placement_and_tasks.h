@@ -11,7 +11,9 @@
 #endif
 
 #include <cmath>
+#include <cstring>
 #include <functional>
+#include <string>
 #include <vector>
 
 // ------------------------------------------------------------------------------------------------
@@ -169,6 +171,36 @@ template <class DT> void funStats(DT ***outputs, Structure **inputs, DCTX(ctx)) 
     DataObjectFactory::destroy(c, x, mu);
 }
 
+// the z-score body as the compiler outlines it for the device: one kernel per operator; inputs x, mu, sd and the
+// threshold as a scalar in the place of a pointer (the bits of a double); outputs r by ROWS, count by ADD
+template <class DT> void funZscoreOpByOp(DT ***outputs, Structure **inputs, DCTX(ctx)) {
+    using VT = typename DT::VT;
+    auto *x = static_cast<DT *>(inputs[0]), *mu = static_cast<DT *>(inputs[1]), *sd = static_cast<DT *>(inputs[2]);
+    const VT thr = HIP::FusedPipelineBody<VT>::scalarOf(inputs[3]);
+    DT *c = nullptr, *z = nullptr, *zz = nullptr, *gt = nullptr;
+    HIP::ewBinaryMat(BinaryOpCode::SUB, c, x, mu, ctx);
+    HIP::ewBinaryMat(BinaryOpCode::DIV, z, c, sd, ctx);
+    HIP::ewBinaryMat(BinaryOpCode::MUL, zz, z, z, ctx);
+    HIP::aggRow(AggOpCode::SUM, *outputs[0], zz, ctx);
+    HIP::ewBinaryObjSca(BinaryOpCode::GT, gt, *outputs[0], thr, ctx);
+    const VT count = HIP::aggAll<VT, DT>(AggOpCode::SUM, gt, ctx);
+    HIP::fill(*outputs[1], count, 1, 1, ctx);
+    DataObjectFactory::destroy(c, z, zz, gt);
+    DataObjectFactory::destroy(x, mu, sd);
+}
+static const char *const kZscoreBody = "%0 = ewSub in0, in1\n%1 = ewDiv %0, in2\n%2 = ewMul %1, %1\n%3 = sumRow %2\n"
+                                       "%4 = ewGt %3, in3\n%5 = sumAll %4\n%6 = cast %5\nreturn %3, %6\n";
+// a body that keeps two tiles alive (x - mu is used again after it was squared): it cannot run as one kernel
+template <class DT> void funTwoTilesOpByOp(DT ***outputs, Structure **inputs, DCTX(ctx)) {
+    auto *x = static_cast<DT *>(inputs[0]), *mu = static_cast<DT *>(inputs[1]);
+    DT *c = nullptr, *sq = nullptr;
+    HIP::ewBinaryMat(BinaryOpCode::SUB, c, x, mu, ctx);
+    HIP::ewBinaryMat(BinaryOpCode::MUL, sq, c, c, ctx);
+    HIP::ewBinaryMat(BinaryOpCode::ADD, *outputs[0], sq, c, ctx);
+    DataObjectFactory::destroy(c, sq, x, mu);
+}
+static const char *const kTwoTilesBody = "%0 = ewSub in0, in1\n%1 = ewMul %0, %0\n%2 = ewAdd %1, %0\nreturn %2\n";
+
 template <typename VT> void run_pipeline_tasks(DaphneContext *dctx) {
     using DT = DenseMatrix<VT>;
     using Fn = void (*)(DT ***, Structure **, DCTX(ctx));
@@ -314,6 +346,81 @@ template <typename VT> void run_pipeline_tasks(DaphneContext *dctx) {
         }
         DataObjectFactory::destroy(mu, var, sd, c, z);
         DataObjectFactory::destroy(zz, r, gt);
+    }
+    // HIP::fusedPipeline: the same pipeline given as the outlined device body AND as the text of its operators. The
+    // text is lowered to the fused kernel's instruction list on the first call: every batch is ONE launch, and what it
+    // stores by ROWS equals, bit for bit, what the body stores when it runs operator by operator.
+    {
+        using Fn4 = void (*)(DT ***, Structure **, DCTX(ctx));
+        DT *mu = nullptr, *var = nullptr, *sd = nullptr;
+        HIP::aggCol(AggOpCode::MEAN, mu, m1, dctx);
+        HIP::aggCol(AggOpCode::VAR, var, m1, dctx);
+        HIP::ewUnaryMat(UnaryOpCode::SQRT, sd, var, dctx);
+        const double thr = 10.0;
+        Structure *thrDisguised;
+        std::memcpy(&thrDisguised, &thr, sizeof(thr));
+        bool isScalar4[] = {false, false, false, true};
+        Structure *inputs4[] = {m1, mu, sd, thrDisguised};
+        int64_t outRows4[] = {int64_t(rows), 1}, outCols4[] = {1, 1};
+        int64_t splits4[] = {int64_t(VectorSplit::ROWS), int64_t(VectorSplit::NONE), int64_t(VectorSplit::NONE), int64_t(VectorSplit::NONE)};
+        int64_t combines4[] = {int64_t(VectorCombine::ROWS), int64_t(VectorCombine::ADD)};
+        void *fun[] = {nullptr, reinterpret_cast<void *>(Fn4(&funZscoreOpByOp<DT>))}; // {host body, device body}
+        // operator by operator, whole matrix at once: the reference result
+        dctx->config.hip_vect_shares = 1;
+        dctx->config.hip_vect_batch_rows = 0;
+        DT *ref[] = {nullptr, nullptr};
+        HIP::fusedPipeline<DT>(ref, 2, isScalar4, inputs4, 4, outRows4, outCols4, splits4, combines4, 2, fun, nullptr, dctx);
+        CHECK(HIP::fusedPipelineLastMode() == 0);
+        const auto r_ref = toHost(ref[0]);
+        const VT count_ref = toHost(ref[1])[0];
+        CHECK(count_ref > VT(0) && count_ref < VT(rows));
+        for (const Case &cs : cases) {
+            dctx->config.hip_vect_shares = cs.shares;
+            dctx->config.hip_vect_batch_rows = cs.batch;
+            DT *out[] = {nullptr, nullptr};
+            HIP::fusedPipeline<DT>(out, 2, isScalar4, inputs4, 4, outRows4, outCols4, splits4, combines4, 2, fun, kZscoreBody, dctx);
+            CHECK(HIP::fusedPipelineLastMode() == 1);
+#ifdef TEST_ON_DEVICE
+            CHECK(dh_vectorized_pipeline_last_mode() == 1); // the specialised kernel: one launch per batch
+#endif
+            CHECK(whereIs(out[0]) == 2);
+            // ten columns: the fused kernel and the row-sum kernel add a row's values in different orders (at the
+            // 64-column shape of the configuration they add them alike: test_glue.cpp checks that one bit for bit)
+            const auto got = toHost(out[0]);
+            const double tol4 = std::is_same<VT, float>::value ? 1e-5 : 1e-13;
+            bool ok = got.size() == r_ref.size();
+            size_t ambiguous = 0;
+            for (size_t i = 0; ok && i < got.size(); i++) {
+                ok = std::fabs(double(got[i]) - double(r_ref[i])) <= tol4 * std::fabs(double(r_ref[i]));
+                ambiguous += std::fabs(double(r_ref[i]) - thr) <= tol4 * thr;
+            }
+            CHECK(ok);
+            CHECK(std::fabs(double(toHost(out[1])[0]) - double(count_ref)) <= double(ambiguous));
+            DataObjectFactory::destroy(out[0], out[1]);
+        }
+        // a body that does not fit runs operator by operator, with the reason on record
+        {
+            bool isScalar2[] = {false, false};
+            Structure *inputs2[] = {m1, mu};
+            int64_t outRows2[] = {int64_t(rows)}, outCols2[] = {int64_t(cols)};
+            int64_t splits2[] = {int64_t(VectorSplit::ROWS), int64_t(VectorSplit::NONE)};
+            int64_t combines2[] = {int64_t(VectorCombine::ROWS)};
+            void *fun2[] = {nullptr, reinterpret_cast<void *>(Fn4(&funTwoTilesOpByOp<DT>))};
+            dctx->config.hip_vect_shares = 3;
+            dctx->config.hip_vect_batch_rows = 100;
+            DT *out[] = {nullptr};
+            HIP::fusedPipeline<DT>(out, 1, isScalar2, inputs2, 2, outRows2, outCols2, splits2, combines2, 2, fun2, kTwoTilesBody, dctx);
+            CHECK(HIP::fusedPipelineLastMode() == 0);
+            CHECK(HIP::fusedPipelineLastReason().find("no longer held") != std::string::npos);
+            DT *c = nullptr, *sq = nullptr, *want = nullptr;
+            HIP::ewBinaryMat(BinaryOpCode::SUB, c, m1, mu, dctx);
+            HIP::ewBinaryMat(BinaryOpCode::MUL, sq, c, c, dctx);
+            HIP::ewBinaryMat(BinaryOpCode::ADD, want, sq, c, dctx);
+            CHECK(toHost(out[0]) == toHost(want));
+            DataObjectFactory::destroy(out[0], c, sq, want);
+        }
+        CHECK(mu->getRefCounter() == 1 && sd->getRefCounter() == 1);
+        DataObjectFactory::destroy(ref[0], ref[1], mu, var, sd);
     }
     dctx->config.hip_vect_shares = 1;
     dctx->config.hip_vect_batch_rows = 0;

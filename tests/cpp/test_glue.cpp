@@ -4,6 +4,8 @@
 // literals are the reference's own test vectors. Built with a plain host compiler.
 #include <cmath>
 #include <cstdio>
+#include <cstring>
+#include <string>
 #include <functional>
 #include <memory>
 #include <stdexcept>
@@ -11,8 +13,10 @@
 
 #include <daphne_hip_kernels.h>
 
+#define TEST_ON_DEVICE 1 // the C ABI under the tests is libdaphne_hip.so on a GPU
 #include "dm_access.h"
 #include "placement_and_tasks.h"
+#include "zscore_via_wrappers.h"
 
 template <typename VT> void run_all(DaphneContext *dctx) {
     using DT = DenseMatrix<VT>;
@@ -374,6 +378,61 @@ static void run_si64(DaphneContext *dctx) {
     DataObjectFactory::destroy(idx);
 }
 
+#include <dlfcn.h>
+template <typename VT> static void run_zscore_via_wrappers(DaphneContext *dctx, void *lib) {
+    using DT = DenseMatrix<VT>;
+    using Z = ZscoreViaWrappers<VT>;
+    CHECK(Z::load(lib));
+    if (!Z::load(lib))
+        return;
+    {
+        {
+            const size_t rows = 5000, cols = 64;
+            std::vector<VT> xv(rows * cols);
+            uint32_t seed = 777u;
+            for (auto &v : xv) {
+                seed = seed * 1664525u + 1013904223u;
+                v = VT(5.0 + 4.0 * ((seed >> 8) * (1.0 / 16777216.0) - 0.5));
+            }
+            auto x = given<DT>(rows, xv);
+            DT *mu = nullptr, *var = nullptr, *sd = nullptr;
+            HIP::aggCol(AggOpCode::MEAN, mu, x, dctx);
+            HIP::aggCol(AggOpCode::VAR, var, x, dctx);
+            HIP::ewUnaryMat(UnaryOpCode::SQRT, sd, var, dctx);
+            const int kPipe = dctx->dispatchMapping.registerKernel("_vect_hip1", "script.daphne", 9, 1);
+            DT *byOps[] = {nullptr, nullptr}, *asOne[] = {nullptr, nullptr};
+            dctx->config.hip_vect_shares = 2;
+            dctx->config.hip_vect_batch_rows = 1000;
+            Z::run(byOps, x, mu, sd, 64.0, false, kPipe, dctx);
+            CHECK(Z::entry().lastMode() == 0);
+            Z::run(asOne, x, mu, sd, 64.0, true, kPipe, dctx);
+            CHECK(Z::entry().lastMode() == 1);
+            if (Z::entry().lastMode() != 1)
+                std::printf("fusedPipeline ran operator by operator: %s\n", Z::entry().lastReason());
+            CHECK(dh_vectorized_pipeline_last_mode() == 1);
+            // r: the same IEEE operations per element, and for float also the same order of additions over a row of
+            // 64 (both kernels give a row to 16 lanes of four values): bit for bit. For double the row-sum kernel takes
+            // 32 lanes of two values where the fused kernel takes 16 lanes of four: equal within rounding.
+            if (std::is_same<VT, float>::value)
+                CHECK(toHost(asOne[0]) == toHost(byOps[0]));
+            else {
+                const auto got = toHost(asOne[0]), want = toHost(byOps[0]);
+                bool ok = got.size() == want.size();
+                for (size_t i = 0; ok && i < got.size(); i++)
+                    ok = std::fabs(double(got[i]) - double(want[i])) <= 1e-14 * std::fabs(double(want[i]));
+                CHECK(ok);
+            }
+            CHECK(toHost(asOne[1]) == toHost(byOps[1]));
+            const double count = double(toHost(asOne[1])[0]);
+            CHECK(count > 0 && count < double(rows));
+            dctx->config.hip_vect_shares = 1;
+            dctx->config.hip_vect_batch_rows = 0;
+            DataObjectFactory::destroy(byOps[0], byOps[1], asOne[0], asOne[1]);
+            DataObjectFactory::destroy(x, mu, var, sd);
+        }
+    }
+}
+
 // ------------------------------------------------------------------------------------------------
 // The generated entry points of libHIPKernels.so, called the way a compiled program calls them
 // (genKernelInst.py:132-154, 236-262; ErrorHandler.cpp:80-90)
@@ -431,8 +490,18 @@ static void run_generated_wrappers(DaphneContext *dctx, const char *lib_path) {
     CHECK(what.find("HIP_ewSqrt__DenseMatrix_double__DenseMatrix_double") != std::string::npos &&
           what.find("script.daphne:5:2") != std::string::npos);
     DataObjectFactory::destroy(a, b, bad, res, neg);
+
+    // The z-score pipeline the way a compiled program runs it with patch 0012: HIP_fusedPipeline gets the outlined
+    // device body - a function that calls the generated HIP_<mnemonic> entry points one after the other - and the
+    // text of the same operators. With the text every batch is ONE launch of the specialised kernel; without it the
+    // outlined body runs. ROWS results are equal bit for bit.
+    {
+        run_zscore_via_wrappers<float>(dctx, lib);
+        run_zscore_via_wrappers<double>(dctx, lib);
+    }
     dlclose(lib);
 }
+
 
 int main(int argc, char **argv) {
     // test/runtime/local/kernels/CUDA_ContextTest.cpp:25-30

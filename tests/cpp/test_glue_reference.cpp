@@ -14,6 +14,7 @@
 #include <runtime/local/kernels/HIP/EwBinaryMat.h>
 #include <runtime/local/kernels/HIP/EwBinaryObjSca.h>
 #include <runtime/local/kernels/HIP/EwUnaryMat.h>
+#include <runtime/local/kernels/HIP/Fill.h>
 #include <runtime/local/kernels/HIP/FusedPipeline.h>
 #include <runtime/local/kernels/HIP/VectorizedPipeline.h>
 #include <runtime/local/vectorized/TasksHIP.h>

@@ -10,6 +10,7 @@ ROOT = Path(__file__).resolve().parent.parent
 OUT = ROOT / "tests" / "cpp" / "build"
 GLUE_BIN = OUT / "test_glue"
 HARNESS_LIB = OUT / "libglue_harness.so"
+BUILDER_BIN = OUT / "test_pipeline_builder"
 
 
 def _link_flags():
@@ -28,3 +29,11 @@ def build_harness() -> Path:
     subprocess.run(["g++", *b.HOST_CXX_FLAGS, "-fPIC", "-shared", "-o", str(HARNESS_LIB),
                     str(ROOT / "tests" / "cpp" / "glue_harness.cpp"), *_link_flags()], check=True)
     return HARNESS_LIB
+
+
+def build_builder_test() -> Path:
+    """Host-only: the pipeline-body lowering needs neither the device library nor a device."""
+    OUT.mkdir(parents=True, exist_ok=True)
+    subprocess.run(["g++", *b.HOST_CXX_FLAGS, "-o", str(BUILDER_BIN), str(ROOT / "tests" / "cpp" / "test_pipeline_builder.cpp")],
+                   check=True)
+    return BUILDER_BIN
