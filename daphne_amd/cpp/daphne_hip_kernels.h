@@ -27,9 +27,11 @@
 #include <runtime/local/kernels/HIP/EwUnaryMat.h>
 #include <runtime/local/kernels/HIP/ExtractCol.h>
 #include <runtime/local/kernels/HIP/Fill.h>
+#include <runtime/local/kernels/HIP/FusedOperators.h>
 #include <runtime/local/kernels/HIP/FusedPipeline.h>
 #include <runtime/local/kernels/HIP/Gemv.h>
 #include <runtime/local/kernels/HIP/MatMul.h>
+#include <runtime/local/kernels/HIP/OperatorChainMatcher.h>
 #include <runtime/local/kernels/HIP/PipelineProgramBuilder.h>
 #include <runtime/local/kernels/HIP/Pooling.h>
 #include <runtime/local/kernels/HIP/PoolingBackward.h>

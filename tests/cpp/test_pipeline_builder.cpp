@@ -1,5 +1,8 @@
-// Host-only tests of HIP::PipelineProgramBuilder: the text form of a device body to the instruction list of the fused
-// pipeline kernel, or the reason why a body does not fit. No device and no device library involved.
+// Host-only tests of the two lowerings that sit between DaphneIR operators and the multi-operator kernels:
+// HIP::PipelineProgramBuilder (the text form of a pipeline's device body to the instruction list of the fused pipeline
+// kernel, or the reason why a body does not fit) and HIP::OperatorChainMatcher (which operator chains one kernel of
+// FusedOperators.h stands for). No device and no device library involved.
+#include <runtime/local/kernels/HIP/OperatorChainMatcher.h>
 #include <runtime/local/kernels/HIP/PipelineProgramBuilder.h>
 
 #include <cstdio>
@@ -26,6 +29,85 @@ static bool buildText(const char *text, const std::vector<PipeInputShape> &in, c
                       std::string &why) {
     PipeBodyDesc d;
     return PipelineProgramBuilder::parse(text, d, &why) && PipelineProgramBuilder::build(d, in, comb, p, &why);
+}
+
+static void run_chain_matcher() {
+    // LeNet's second block and its head, as the DSL builtins produce them (values are numbered as they appear):
+    //   (v20, v21, v22) = Convolution_Forward(x v1, W v2, b v3, N v4, C v5, H v6, W v7, 5 v8, 5 v9, 1 v10, 1 v11, 2 v12, 2 v13)
+    //   v23 = NN_Relu_Forward(v20); (v24, v25, v26) = NN_Max_Forward(v23, v4, v14, v21, v22, 2 v15, 2 v15, 2 v15, 2 v15, 0 v16, 0 v16)
+    //   v27 = NN_Affine_Forward(v24, v17, v18); v28 = NN_Relu_Forward(v27); v29 = NN_Affine_Forward(v28, v19, v30); v31 = Softmax(v29)
+    ChainGraph g;
+    g.ops = {{"Convolution_Forward", {1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13}, {20, 21, 22}},
+             {"NN_Relu_Forward", {20}, {23}},
+             {"NN_Max_Forward", {23, 4, 14, 21, 22, 15, 15, 15, 15, 16, 16}, {24, 25, 26}},
+             {"NN_Affine_Forward", {24, 17, 18}, {27}},
+             {"NN_Relu_Forward", {27}, {28}},
+             {"NN_Affine_Forward", {28, 19, 30}, {29}},
+             {"Softmax", {29}, {31}}};
+    g.constants = {{8, 5}, {9, 5}, {10, 1}, {11, 1}, {12, 2}, {13, 2}, {15, 2}, {16, 0}};
+    g.escaping = {31};
+    auto found = OperatorChainMatcher::match(g);
+    CHECK(found.size() == 2);
+    if (found.size() == 2) {
+        CHECK(found[0].kind == ChainKind::CONV_RELU_POOL && found[0].epilogue == 3 && found[0].ops == (std::vector<size_t>{0, 1, 2}));
+        CHECK(found[0].results == (std::vector<int>{24, 25, 26}) && found[0].args.at("filter") == 2 && found[0].args.at("pad_w") == 13);
+        CHECK(found[1].kind == ChainKind::AFFINE_RELU && found[1].ops == (std::vector<size_t>{3, 4}) && found[1].results == (std::vector<int>{28}));
+    }
+    // the rectified activations are needed elsewhere: only the rectifier folds into the convolution
+    ChainGraph g2 = g;
+    g2.escaping.push_back(23);
+    found = OperatorChainMatcher::match(g2);
+    CHECK(found.size() == 2 && found[0].kind == ChainKind::CONV_RELU_POOL && found[0].epilogue == 1 &&
+          found[0].results == (std::vector<int>{23, 21, 22}));
+    // a 3 x 3 pooling window does not fold; a convolution with nothing behind it is left alone
+    ChainGraph g3 = g;
+    g3.constants[15] = 3;
+    found = OperatorChainMatcher::match(g3);
+    CHECK(found.size() == 2 && found[0].epilogue == 1);
+    ChainGraph g4;
+    g4.ops = {g.ops[0]};
+    g4.escaping = {20};
+    CHECK(OperatorChainMatcher::match(g4).empty());
+
+    // lmDS: A = syrk(X); b = t(X) @ y; both spellings of the transposed product
+    ChainGraph n;
+    n.ops = {{"syrk", {1, 2}, {10}}, {"transpose", {1}, {11}}, {"matMul", {11, 3, 4, 4}, {12}}, {"ewAdd", {10, 5}, {13}}, {"solve", {13, 12}, {14}}};
+    n.constants = {{2, 1}, {4, 0}};
+    n.shapes = {{1, {100000, 100}}, {3, {100000, 1}}};
+    n.escaping = {14};
+    found = OperatorChainMatcher::match(n);
+    CHECK(found.size() == 1 && found[0].kind == ChainKind::NORMAL_EQUATIONS && found[0].ops == (std::vector<size_t>{0, 1, 2}) &&
+          found[0].results == (std::vector<int>{10, 12}) && found[0].args.at("X") == 1 && found[0].args.at("y") == 3);
+    n.ops[2] = {"matMul", {1, 3, 2, 4}, {12}}; // transa = true on X itself; the transpose stays (it has no other use, but is not ours)
+    found = OperatorChainMatcher::match(n);
+    CHECK(found.size() == 1 && found[0].ops == (std::vector<size_t>{0, 2}));
+    n.shapes[3] = {100000, 7}; // a right-hand side of seven columns is a matrix product, not t(X) y
+    CHECK(OperatorChainMatcher::match(n).empty());
+
+    // k-means: D = (X @ t(C)) * -2 + xx + t(cc'); idx = idxminRow(D)
+    ChainGraph k;
+    k.ops = {{"transpose", {2}, {10}}, {"matMul", {1, 10, 5, 5}, {11}}, {"ewMul", {11, 6}, {12}}, {"ewAdd", {12, 3}, {13}},
+             {"ewAdd", {13, 4}, {14}}, {"idxminRow", {14}, {15}}};
+    k.constants = {{5, 0}, {6, -2}};
+    k.shapes = {{1, {2000000, 64}}, {2, {16, 64}}, {3, {2000000, 1}}, {4, {1, 16}}};
+    k.escaping = {15};
+    found = OperatorChainMatcher::match(k);
+    CHECK(found.size() == 1 && found[0].kind == ChainKind::KMEANS_ASSIGN && found[0].ops.size() == 6 && found[0].args.at("C") == 2 &&
+          found[0].args.at("xx") == 3 && found[0].args.at("cc") == 4 && found[0].results == (std::vector<int>{15}));
+    // xx - 2 * (X @ t(C)) + cc rounds the same way; X @ t(C) * 2 + xx + cc does not compute the distances
+    ChainGraph k2 = k;
+    k2.ops[2] = {"ewMul", {7, 11}, {12}};
+    k2.ops[3] = {"ewSub", {3, 12}, {13}};
+    k2.ops[4] = {"ewAdd", {4, 13}, {14}};
+    k2.constants[7] = 2;
+    found = OperatorChainMatcher::match(k2);
+    CHECK(found.size() == 1 && found[0].kind == ChainKind::KMEANS_ASSIGN);
+    ChainGraph k3 = k;
+    k3.constants[6] = 2;
+    CHECK(OperatorChainMatcher::match(k3).empty());
+    ChainGraph k4 = k; // the distances are printed as well: they have to exist
+    k4.escaping.push_back(14);
+    CHECK(OperatorChainMatcher::match(k4).empty());
 }
 
 int main() {
@@ -103,6 +185,7 @@ int main() {
         CHECK(!buildText(text.c_str(), {X}, {VectorCombine::ROWS}, p, why));
         CHECK(why.find("instructions") != std::string::npos);
     }
+    run_chain_matcher();
     std::printf("%s: %d checks, %d failed\n", g_fail ? "FAILED" : "PASSED", g_checks, g_fail);
     return g_fail ? 1 : 0;
 }

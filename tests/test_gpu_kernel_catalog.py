@@ -200,6 +200,90 @@ def test_dnn_forward_kernels(rt, rng, dt):
         m.destroy()
 
 
+@pytest.mark.parametrize("dt", FP)
+def test_operator_chains_as_one_kernel(rt, rng, dt):
+    """The kernels that stand for a chain of operators (kernels/HIP/FusedOperators.h), looked up like any other kernel,
+    against the chain itself run through the catalog: conv -> relu -> max-pool, affine -> relu and the k-means
+    assignment bit for bit; the normal equations and the k-means means within rounding (sums in another order)."""
+    sz = "size_t"
+    # conv2d -> relu -> max_pool2d (2 x 2 / 2), LeNet's second block at a small batch
+    N, Cc, H, W, F, Hf, Wf = 6, 8, 14, 14, 16, 5, 5
+    x = rng.standard_normal((N, Cc * H * W)).astype(dt)
+    w = (rng.standard_normal((F, Cc * Hf * Wf)) * 0.1).astype(dt)
+    bias = rng.standard_normal((F, 1)).astype(dt)
+    X, Wm, Bm = rt.matrix(x), rt.matrix(w), rt.matrix(bias)
+    geo = (N, Cc, H, W, Hf, Wf, 1, 1, 2, 2)
+    conv, rh, rw = by_catalog(rt, "Convolution_Forward", [dm(dt), sz, sz], [dm(dt)] * 3 + [sz] * 10, X, Wm, Bm, *geo)
+    relu = by_catalog(rt, "NN_Relu_Forward", [dm(dt)], [dm(dt)], conv)
+    # (the pooling entry point takes its two extent results by value, as the reference's does: only the matrix comes back)
+    pool = by_catalog(rt, "NN_Max_Forward", [dm(dt), sz, sz], [dm(dt)] + [sz] * 10, relu, N, F, rh, rw, 2, 2, 2, 2, 0, 0)
+    ph, pw = rh // 2, rw // 2
+    for epilogue, want, extents in ((3, pool, (ph, pw)), (1, relu, (rh, rw))):
+        one, oh, ow = by_catalog(rt, "conv2DForwardFused", [dm(dt), sz, sz], [dm(dt)] * 3 + [sz] * 11, X, Wm, Bm, *geo, epilogue)
+        assert (oh, ow) == extents
+        assert_exact(one.to_numpy(), want.to_numpy())
+        one.destroy()
+    # affine -> relu
+    feat = pool.shape[1]
+    wa = (rng.standard_normal((feat, 24)) * 0.1).astype(dt)
+    ba = rng.standard_normal((1, 24)).astype(dt)
+    WA, BA = rt.matrix(wa), rt.matrix(ba)
+    aff = by_catalog(rt, "NN_Affine_Forward", [dm(dt)], [dm(dt)] * 3, pool, WA, BA)
+    arelu = by_catalog(rt, "NN_Relu_Forward", [dm(dt)], [dm(dt)], aff)
+    one = by_catalog(rt, "affineForwardFused", [dm(dt)], [dm(dt)] * 3 + [sz], pool, WA, BA, 1)
+    assert_exact(one.to_numpy(), arelu.to_numpy())
+    for m in (X, Wm, Bm, conv, relu, pool, WA, BA, aff, arelu, one):
+        m.destroy()
+
+    # lmDS: A = syrk(X), b = t(X) @ y from one pass over X (100 columns: the symmetric streaming kernel)
+    xs = rng.random((6000, 100)).astype(dt)
+    ys = (xs @ rng.standard_normal((100, 1)) + 0.01 * rng.standard_normal((6000, 1))).astype(dt)
+    XS, YS = rt.matrix(xs), rt.matrix(ys)
+    a_seq = by_catalog(rt, "syrk", [dm(dt)], [dm(dt), "bool"], XS, True)
+    b_seq = by_catalog(rt, "matMul", [dm(dt)], [dm(dt), dm(dt), "bool", "bool"], XS, YS, True, False)
+    a_one, b_one = by_catalog(rt, "normalEquations", [dm(dt), dm(dt)], [dm(dt), dm(dt), CPP[np.dtype(dt)]], XS, YS, 0.0)
+    assert a_one.shape == (100, 100) and b_one.shape == (100, 1)
+    assert_close(a_one.to_numpy(), a_seq.to_numpy(), elementwise=False)
+    assert_close(b_one.to_numpy(), b_seq.to_numpy(), elementwise=False)
+    assert_close(a_one.to_numpy(), orc.syrk(xs, True)[1], elementwise=False)
+    for m in (XS, YS, a_seq, b_seq, a_one, b_one):
+        m.destroy()
+
+    # k-means: idx = idxminRow(((X @ t(C)) * -2 + xx) + cc); enough rows for the streaming product, whose bits the
+    # assignment kernel reproduces
+    rows, cols, k = 70000, 64, 16
+    centres = (rng.standard_normal((k, cols)) * 5).astype(dt)
+    xk = (centres[rng.integers(0, k, rows)] + rng.standard_normal((rows, cols))).astype(dt)
+    ck = xk[:: rows // k][:k].copy()
+    XK, CK = rt.matrix(xk), rt.matrix(ck)
+    sq = lambda M: by_catalog(rt, "ewMul", [dm(dt)], [dm(dt), dm(dt)], M, M)
+    x2, c2 = sq(XK), sq(CK)
+    xx = by_catalog(rt, "sumRow", [dm(dt)], [dm(dt)], x2)
+    cc_col = by_catalog(rt, "sumRow", [dm(dt)], [dm(dt)], c2)
+    cc = by_catalog(rt, "transpose", [dm(dt)], [dm(dt)], cc_col)
+    prod = by_catalog(rt, "matMul", [dm(dt)], [dm(dt), dm(dt), "bool", "bool"], XK, CK, False, True)
+    d1 = by_catalog(rt, "ewMul", [dm(dt)], [dm(dt), CPP[np.dtype(dt)]], prod, -2.0)
+    d2 = by_catalog(rt, "ewAdd", [dm(dt)], [dm(dt), dm(dt)], d1, xx)
+    d3 = by_catalog(rt, "ewAdd", [dm(dt)], [dm(dt), dm(dt)], d2, cc)
+    idx_seq = by_catalog(rt, "idxminRow", ["DenseMatrix<size_t>"], [dm(dt)], d3)
+    IDX = "DenseMatrix<size_t>"
+    idx_one = by_catalog(rt, "kmeansAssign", [IDX], [dm(dt)] * 4, XK, CK, xx, cc)
+    assert_exact(idx_one.to_numpy(), idx_seq.to_numpy())
+    assert len(np.unique(idx_one.to_numpy())) == k
+    cn, counts = by_catalog(rt, "kmeansUpdate", [dm(dt), dm(dt)], [dm(dt), IDX, sz], XK, idx_one, k)
+    lab = idx_one.to_numpy()[:, 0]
+    want_counts = np.bincount(lab, minlength=k).astype(dt)
+    assert_exact(counts.to_numpy()[0], want_counts)
+    want_means = np.stack([xk[lab == c].astype(np.float64).mean(axis=0) for c in range(k)]).astype(dt)
+    assert_close(cn.to_numpy(), want_means, elementwise=False)
+    idx_s, cn_s, counts_s = by_catalog(rt, "kmeansStep", [IDX, dm(dt), dm(dt)], [dm(dt)] * 4, XK, CK, xx, cc)
+    assert_exact(idx_s.to_numpy(), idx_one.to_numpy())
+    assert_exact(counts_s.to_numpy(), counts.to_numpy())
+    assert_close(cn_s.to_numpy(), cn.to_numpy(), elementwise=False)
+    for m in (XK, CK, x2, c2, xx, cc_col, cc, prod, d1, d2, d3, idx_seq, idx_one, cn, counts, idx_s, cn_s, counts_s):
+        m.destroy()
+
+
 @pytest.mark.parametrize("dt", FP + [np.int64])
 def test_fill_colbind_extractcol_transpose(rt, rng, dt):
     vt = CPP[np.dtype(dt)]
