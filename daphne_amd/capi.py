@@ -71,6 +71,8 @@ def _signatures(lib: C.CDLL) -> None:
     lib.dh_vectorized_pipeline_last_mode.argtypes = []
     lib.dh_vectorized_pipeline_cache_size.argtypes = []
     lib.dh_vectorized_pipeline_cache_size.restype = sz
+    lib.dh_vectorized_pipeline_set_cache_limit.argtypes = [sz]
+    lib.dh_vectorized_pipeline_set_cache_limit.restype = sz
     lib.dh_agg_col_noalloc_f32.argtypes = [ctxp, i32, vp, vp, sz, sz, sz]
     lib.dh_agg_col_noalloc_scratch_bytes.argtypes = []
     lib.dh_agg_col_noalloc_scratch_bytes.restype = sz

@@ -25,6 +25,9 @@ dh_status assign(dh_ctx *ctx, unsigned long long *idx, const T *X, size_t rows, 
     constexpr int V = 16 / sizeof(T), KC = 4 * V;
     if (rows == 0)
         return DH_OK;
+    // the kernel reads and writes all of these unconditionally: a null pointer is an error of the caller, not a fault
+    if (idx == nullptr || X == nullptr || C == nullptr || xx == nullptr || cc == nullptr)
+        return dh_fail(DH_ERR_INVALID_ARG, "kmeans assign: idx, X, C, xx and cc must not be null");
     if (k == 0 || k > 32 || cols == 0 || cols > 512)
         return dh_fail(DH_ERR_INVALID_ARG, "kmeans assign: 1..32 centroids of 1..512 features are supported (got %zu of %zu)", k, cols);
     if (!dh_aligned(X, 16) || !dh_aligned(C, 16) || ldx % V || ldc % V || cols % V || ldx < cols || ldc < cols)
@@ -282,6 +285,8 @@ dh_status update(dh_ctx *ctx, T *Cn, size_t ldc, T *counts, const T *X, size_t r
     DH_REQUIRE_CTX(ctx);
     constexpr int V = 16 / sizeof(T);
     constexpr size_t COLS_PER_BLOCK = 16 * V;
+    if (Cn == nullptr || (rows > 0 && (X == nullptr || idx == nullptr))) // `counts` alone may be null
+        return dh_fail(DH_ERR_INVALID_ARG, "kmeans update: C_new, X and idx must not be null");
     if (k == 0 || k > 32 || cols == 0 || cols > 4 * COLS_PER_BLOCK)
         return dh_fail(DH_ERR_INVALID_ARG, "kmeans update: 1..32 centroids of 1..%zu features are supported (got %zu of %zu)",
                        4 * COLS_PER_BLOCK, k, cols);
@@ -348,6 +353,8 @@ template <typename T>
 dh_status step(dh_ctx *ctx, unsigned long long *idx, T *Cn, size_t ldcn, T *counts, const T *X, size_t rows, size_t cols, size_t ldx,
                const T *C, size_t k, size_t ldc, const T *xx, const T *cc) {
     DH_REQUIRE_CTX(ctx);
+    if (Cn == nullptr || (rows > 0 && (idx == nullptr || X == nullptr || C == nullptr || xx == nullptr || cc == nullptr)))
+        return dh_fail(DH_ERR_INVALID_ARG, "kmeans step: idx, C_new, X, C, xx and cc must not be null");
     if constexpr (sizeof(T) == 4) {
         constexpr int V = 4, KC = 16;
         const size_t kpad = dh_ceil_div(cols, KC) * KC;

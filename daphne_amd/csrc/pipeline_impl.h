@@ -7,6 +7,7 @@
 #include "pipeline_kernel.h"
 
 #include <cstdlib>
+#include <memory>
 #include <string>
 
 namespace dh_pipe {
@@ -14,7 +15,7 @@ namespace dh_pipe {
 // pipeline_jit.hip
 bool jit_enabled();
 bool jit_lookup(int device, const char *tname, int vec, int kv, size_t cols, int G, int S, const dh_pipe_instr *prog, int n,
-                hipFunction_t *fn, std::string *err, bool compile_only);
+                hipFunction_t *fn, std::shared_ptr<const void> *keep, std::string *err, bool compile_only);
 void jit_set_last_mode(int m);
 size_t jit_cache_size();
 
@@ -205,11 +206,12 @@ dh_status run(dh_ctx *ctx, const dh_pipe_instr *prog, int n, const IO_C *cio, si
     // Preferred path: the body specialised at run time (pipeline_jit.hip). The generic interpreter
     // kernel below is the fallback when specialisation is switched off or fails.
     hipFunction_t jit_fn = nullptr;
+    std::shared_ptr<const void> jit_keep; // the module stays loaded at least until the launch below is queued
     std::string jit_err;
     // the context's setting wins over the environment's (dh_ctx_set_pipeline_mode)
     const bool want_jit = n >= 1 && (ctx->pipeline_mode < 0 ? jit_enabled() : ctx->pipeline_mode == 1);
     const bool use_jit = want_jit && jit_lookup(ctx->device, sizeof(T) == 4 ? "float" : "double", vec, KV, cols, G, S, P.ins, n,
-                                                &jit_fn, &jit_err, false);
+                                                &jit_fn, &jit_keep, &jit_err, false);
     if (want_jit && !use_jit) {
         // The body still runs (interpreted, at a fraction of the rate); the reason stays readable through
         // dh_last_error() and dh_vectorized_pipeline_last_mode() says 0. Reported once per process on stderr.

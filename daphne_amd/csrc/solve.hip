@@ -642,15 +642,20 @@ template <typename T> dh_status solve(dh_ctx *ctx, T *x, const T *A, size_t n, s
         return dh_fail(DH_ERR_RUNTIME, "Solve: systems beyond 32767 unknowns are not supported by this kernel");
     const size_t lds_bytes = LdsSolveShape<T>(n).bytes;
     if (n <= 64 * LDS_SOLVE_MAX_SLOTS && lds_bytes <= (size_t(150) << 10)) {
-        auto launch = [&](auto kernel) -> dh_status {
+        // Systems beyond 64 KB of LDS need the limit of the kernel raised, once per kernel instantiation and device
+        // (the three instantiations have the same pointer type, so the bookkeeping is keyed by SLOTS, not by type).
+        auto launch = [&](auto kernel, int slots) -> dh_status {
             if (lds_bytes > (size_t(64) << 10)) {
+                constexpr int MAX_DEVICES = 64;
                 static std::mutex attr_lock;
-                static bool attr_set[16] = {};
+                static bool attr_set[LDS_SOLVE_MAX_SLOTS + 1][MAX_DEVICES] = {};
                 std::lock_guard<std::mutex> guard(attr_lock);
-                if (ctx->device < 16 && !attr_set[ctx->device]) {
+                const bool tracked = ctx->device >= 0 && ctx->device < MAX_DEVICES;
+                if (!tracked || !attr_set[slots][ctx->device]) {
                     DH_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                                      150 << 10));
-                    attr_set[ctx->device] = true;
+                    if (tracked)
+                        attr_set[slots][ctx->device] = true;
                 }
             }
             hipLaunchKernelGGL(kernel, dim3(1), dim3(LDS_SOLVE_THREADS), lds_bytes, ctx->stream, x, A, lda, b,
@@ -659,11 +664,11 @@ template <typename T> dh_status solve(dh_ctx *ctx, T *x, const T *A, size_t n, s
         };
         dh_status lst;
         if (n <= 64)
-            lst = launch(&lu_solve_lds_kernel<T, 1>);
+            lst = launch(&lu_solve_lds_kernel<T, 1>, 1);
         else if (n <= 128)
-            lst = launch(&lu_solve_lds_kernel<T, 2>);
+            lst = launch(&lu_solve_lds_kernel<T, 2>, 2);
         else
-            lst = launch(&lu_solve_lds_kernel<T, 3>);
+            lst = launch(&lu_solve_lds_kernel<T, 3>, 3);
         if (lst != DH_OK)
             return lst;
     } else {

@@ -720,8 +720,11 @@ int dh_ctx_get_pipeline_mode(const dh_ctx *ctx);
 /* Number of specialised bodies this process holds. A body is keyed by its instruction kinds, op codes,
  * operand slots, value type and row width; its immediates are kernel arguments, so a scalar that changes
  * from call to call (a threshold, a learning rate) reuses the compiled kernel. At most 128 bodies stay
- * loaded, the least recently used one is unloaded beyond that. */
+ * loaded by default, the least recently used one is unloaded beyond that. */
 size_t dh_vectorized_pipeline_cache_size(void);
+/* Sets how many specialised bodies stay loaded (at least 1) and returns the previous limit. A body that leaves the
+ * cache is unloaded once no caller is about to launch it and its device has drained. */
+size_t dh_vectorized_pipeline_set_cache_limit(size_t bodies);
 /* Compiles the specialised kernel of a body for rows of `cols` values without loading or running
  * it (no device needed). value_type 0 = float, 1 = double; vectorised != 0: rows are read as
  * 16-byte vectors (cols a multiple of 4 / 2), as the launch does for aligned operands. */

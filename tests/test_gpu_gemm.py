@@ -493,3 +493,25 @@ def test_kmeans_assign_nan_semantics_and_errors(ctx, dt):
     with pytest.raises(capi.DaphneHipError, match="features are supported"):
         wide = DenseMatrix.from_numpy(ctx, np.zeros((4, 600), dt))
         kmeansUpdate(None, wide, DenseMatrix.from_numpy(ctx, np.zeros((4, 1), np.uint64)), 2, ctx)
+    # a null pointer is refused on the host (the kernels read and write all of these unconditionally); only
+    # `counts` may be left out
+    suf = "f32" if dt == np.float32 else "f64"
+    lib = capi.lib()
+    idx_ok = DenseMatrix(ctx, X.rows, 1, np.uint64)
+    cc = DenseMatrix.from_numpy(ctx, cc_h)
+    cn = DenseMatrix(ctx, k, cols, dt)
+    good = dict(idx=idx_ok.ptr, X=X.ptr, C=C.ptr, xx=xx.ptr, cc=cc.ptr)
+    for missing in good:
+        a = dict(good, **{missing: None})
+        st = getattr(lib, f"dh_kmeans_assign_{suf}")(ctx._h, a["idx"], a["X"], X.rows, cols, X.row_skip, a["C"], k, C.row_skip, a["xx"], a["cc"])
+        assert st == 2 and b"must not be null" in lib.dh_last_error(), missing   # DH_ERR_INVALID_ARG
+        st = getattr(lib, f"dh_kmeans_step_{suf}")(ctx._h, a["idx"], cn.ptr, cn.row_skip, None, a["X"], X.rows, cols, X.row_skip, a["C"], k,
+                                                   C.row_skip, a["xx"], a["cc"])
+        assert st == 2 and b"must not be null" in lib.dh_last_error(), missing
+    st = getattr(lib, f"dh_kmeans_step_{suf}")(ctx._h, idx_ok.ptr, None, cols, None, X.ptr, X.rows, cols, X.row_skip, C.ptr, k, C.row_skip,
+                                               xx.ptr, cc.ptr)
+    assert st == 2
+    for a_cn, a_x, a_idx in ((None, X.ptr, idx_ok.ptr), (cn.ptr, None, idx_ok.ptr), (cn.ptr, X.ptr, None)):
+        st = getattr(lib, f"dh_kmeans_update_{suf}")(ctx._h, a_cn, cols, None, a_x, X.rows, cols, X.row_skip, a_idx, k)
+        assert st == 2 and b"must not be null" in lib.dh_last_error()
+    capi.check(getattr(lib, f"dh_kmeans_update_{suf}")(ctx._h, cn.ptr, cn.row_skip, None, X.ptr, X.rows, cols, X.row_skip, idx_ok.ptr, k))

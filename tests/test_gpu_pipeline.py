@@ -270,3 +270,28 @@ def test_changing_immediates_reuse_the_compiled_body(ctx, pipeline_mode):
             want = ((x * np.float32(1.0 + k)) > np.float32(thr)).astype(np.float32)
         assert_exact(out.to_numpy(), want)
     assert len(set(sizes)) == 1, sizes
+
+
+def test_an_evicted_body_is_compiled_again_and_runs(ctx, pipeline_mode):
+    """More distinct bodies than the cache may hold: the least recently used one leaves (and is unloaded once nobody
+    is about to launch it); using it again compiles it again, with the same results."""
+    if pipeline_mode != 1:
+        pytest.skip("only the specialised path compiles anything")
+    rng = np.random.default_rng(11)
+    x = rng.standard_normal((1500, 32)).astype(np.float32)
+    X = DenseMatrix.from_numpy(ctx, x)
+    ops = [BinaryOpCode.ADD, BinaryOpCode.SUB, BinaryOpCode.MUL, BinaryOpCode.MAX]
+    fns = {BinaryOpCode.ADD: np.add, BinaryOpCode.SUB: np.subtract, BinaryOpCode.MUL: np.multiply, BinaryOpCode.MAX: np.maximum}
+    lib = capi.lib()
+    before = lib.dh_vectorized_pipeline_set_cache_limit(2)
+    try:
+        for op in ops + ops[:2]:  # the first two bodies have left the cache by the time they come round again
+            p = VectorizedPipeline(ctx, X)
+            p.ewBinary(op, 0.75).ewUnary(UnaryOpCode.ABS)
+            out = p.storeTile()
+            p.run()
+            assert_ran_as(1)
+            assert lib.dh_vectorized_pipeline_cache_size() <= 2
+            assert_exact(out.to_numpy(), np.abs(fns[op](x, np.float32(0.75))))
+    finally:
+        lib.dh_vectorized_pipeline_set_cache_limit(before)
