@@ -53,13 +53,16 @@ struct ConvArgs {
 template <typename T>
 __global__ __launch_bounds__(256) void conv_prep_kernel(int *tab, T *wpack, const T *filter, unsigned F, unsigned Fpad,
                                                         unsigned K, unsigned Kpad, unsigned HpWp, unsigned Wp,
-                                                        unsigned Hf, unsigned Wf) {
+                                                        unsigned Hf, unsigned Wf, unsigned stage_channels = ~0u,
+                                                        unsigned scale = 1) {
+    // stage_channels: offsets count from the first channel of the LDS stage a channel belongs to (all channels in one
+    // stage by default); scale: 1 for offsets in elements, sizeof(T) for offsets in bytes
     const unsigned t = blockIdx.x * 256 + threadIdx.x, nt = gridDim.x * 256;
     for (unsigned k = t; k < Kpad; k += nt) {
         int off = 0;
         if (k < K) {
             const unsigned c = k / (Hf * Wf), hw = k % (Hf * Wf);
-            off = static_cast<int>(c * HpWp + (hw / Wf) * Wp + hw % Wf);
+            off = static_cast<int>(((c % stage_channels) * HpWp + (hw / Wf) * Wp + hw % Wf) * scale);
         }
         tab[k] = off;
     }
@@ -318,7 +321,7 @@ __global__ __launch_bounds__(64 * WN) void conv2d_kernel(ConvArgs g) {
 struct ConvResidentArgs {
     const void *x;     // N x C x H x W
     const void *wpack; // filter matrix padded with zeros to Fpad x Kpad
-    const int *ktab;   // k -> c*Hp*Wp + hy*Wp + hx (0 beyond K)
+    const int *ktab;   // k -> byte offset of tap (c, hy, hx) from the start of its channel stage in LDS (0 beyond K)
     const void *bias;
     void *res;
     unsigned C, H, W, Hp, Wp, ph, pw, Q, sh, sw, F, Kpad, HpWp, PQ, chunk;
@@ -443,54 +446,75 @@ __global__ __launch_bounds__(512) void conv2d_resident_kernel(ConvResidentArgs g
         acc[j] = typename M::acc_t{0, 0, 0, 0};
 
     const T *wrow = static_cast<const T *>(g.wpack) + static_cast<size_t>(f0 + mf * 16 + li) * g.Kpad + lk * VEC;
-    const int *ktl = ktab + lk * VEC;
-    // The contraction, for a number of pixel blocks fixed at compile time: no branch inside the loop body, so that
-    // LDS reads and matrix instructions of neighbouring blocks interleave. A wave with fewer blocks than NF - 1
-    // computes all NF (the spare ones gather pixel 0 and are never stored).
-    // k_begin .. k_end: this stage's share of K; sub: the table offset of the stage's first channel
-    auto contract = [&](auto nv_tag, unsigned k_begin, unsigned k_end, int sub) {
+    const int *ktl = ktab + lk * VEC; // byte offsets from the start of a channel's stage (conv_prep_kernel)
+    const char *frame_b = reinterpret_cast<const char *>(frame);
+#pragma unroll
+    for (int j = 0; j < NF; j++)
+        pixoff[j] *= static_cast<int>(sizeof(T));
+    // The contraction, for a number of pixel blocks fixed at compile time: no branch inside the loop body. A wave
+    // with fewer blocks than NF - 1 computes all NF (the spare ones gather pixel 0 and are never stored).
+    // Every ordinary vector instruction and every LDS read that a SIMD issues takes about one pass out of its matrix
+    // pipe (a 16x16x4 instruction is 8 passes), so the loop is written to issue as few as it can beside the matrix
+    // instructions: per instruction one gather and one address add. The table holds ready byte offsets; the patch
+    // values alternate between two register sets from step to step and the filter values / table entries between
+    // two sets from block to block (both counts are even), so that nothing is copied from register to register.
+    // One block = 4 * VEC values of k = VEC steps: (a_c, kt_c) are the block's filter values and table entries, those
+    // of the block after it are fetched into (a_n, kt_n).
+    auto kblock = [&](auto nv_tag, T(&a_c)[VEC], int(&kt_c)[VEC], T(&a_n)[VEC], int(&kt_n)[VEC], T(&b_even)[NF], T(&b_odd)[NF],
+                      unsigned kn) {
         constexpr int NV = decltype(nv_tag)::value;
-        T a_cur[VEC], b_cur[NV];
-        int kt[VEC];
-        dh_load_vec<T, VEC>(wrow + k_begin, a_cur);
+        static_assert(VEC % 2 == 0, "the two sets of patch registers alternate from step to step");
+        dh_load_vec<T, VEC>(wrow + kn, a_n);
 #pragma unroll
         for (int s_ = 0; s_ < VEC; s_++)
-            kt[s_] = max(ktl[k_begin + s_] - sub, 0); // the zero entries beyond K stay inside the stage
+            kt_n[s_] = ktl[kn + s_];
+#pragma unroll
+        for (int s_ = 0; s_ < VEC; s_++) {
+            // the patch values of the following step are on their way while this step's matrix instructions run
+            const int kt_after = (s_ + 1 < VEC) ? kt_c[s_ + 1] : kt_n[0];
+            __builtin_amdgcn_sched_barrier(0); // a gather must not sink to its use in the next step
+            if (s_ % 2 == 0) {
+#pragma unroll
+                for (int j = 0; j < NV; j++)
+                    b_odd[j] = *reinterpret_cast<const T *>(frame_b + (pixoff[j] + kt_after));
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int j = 0; j < NV; j++)
+                    acc[j] = M::mma(a_c[s_], b_even[j], acc[j]);
+            } else {
+#pragma unroll
+                for (int j = 0; j < NV; j++)
+                    b_even[j] = *reinterpret_cast<const T *>(frame_b + (pixoff[j] + kt_after));
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int j = 0; j < NV; j++)
+                    acc[j] = M::mma(a_c[s_], b_odd[j], acc[j]);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    // k_begin .. k_end: this stage's share of K; its blocks are taken two to a turn of the loop, a last odd one alone
+    auto contract = [&](auto nv_tag, unsigned k_begin, unsigned k_end) {
+        constexpr int NV = decltype(nv_tag)::value;
+        constexpr unsigned KB = 4 * VEC;
+        T a0[VEC], a1[VEC], b_even[NF], b_odd[NF];
+        int kt0[VEC], kt1[VEC];
+        dh_load_vec<T, VEC>(wrow + k_begin, a0);
+#pragma unroll
+        for (int s_ = 0; s_ < VEC; s_++)
+            kt0[s_] = ktl[k_begin + s_];
 #pragma unroll
         for (int j = 0; j < NV; j++)
-            b_cur[j] = frame[pixoff[j] + kt[0]];
-        for (unsigned k0 = k_begin; k0 < k_end; k0 += 4 * VEC) {
-            // the next block's filter values and table entries, loaded unconditionally (the last block loads itself again)
-            const unsigned kn = (k0 + 4 * VEC < k_end) ? k0 + 4 * VEC : k0;
-            T a_nxt[VEC];
-            int kt_nxt[VEC];
-            dh_load_vec<T, VEC>(wrow + kn, a_nxt);
-#pragma unroll
-            for (int s_ = 0; s_ < VEC; s_++)
-                kt_nxt[s_] = max(ktl[kn + s_] - sub, 0);
-#pragma unroll
-            for (int s_ = 0; s_ < VEC; s_++) {
-                // the patch values of the following step are on their way while this step's matrix instructions run
-                const int kt_after = (s_ + 1 < VEC) ? kt[s_ + 1] : kt_nxt[0];
-                T b_nxt[NV];
-#pragma unroll
-                for (int j = 0; j < NV; j++)
-                    b_nxt[j] = frame[pixoff[j] + kt_after];
-                __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                for (int j = 0; j < NV; j++)
-                    acc[j] = M::mma(a_cur[s_], b_cur[j], acc[j]);
-                __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                for (int j = 0; j < NV; j++)
-                    b_cur[j] = b_nxt[j];
-            }
-#pragma unroll
-            for (int s_ = 0; s_ < VEC; s_++) {
-                a_cur[s_] = a_nxt[s_];
-                kt[s_] = kt_nxt[s_];
-            }
+            b_even[j] = *reinterpret_cast<const T *>(frame_b + (pixoff[j] + kt0[0]));
+        unsigned k0 = k_begin;
+        for (; k0 + 2 * KB <= k_end; k0 += 2 * KB) {
+            // the block after the second one of this turn (the stage's last turn fetches a block of its own again)
+            const unsigned kn = (k0 + 2 * KB < k_end) ? k0 + 2 * KB : k0;
+            kblock(nv_tag, a0, kt0, a1, kt1, b_even, b_odd, k0 + KB);
+            kblock(nv_tag, a1, kt1, a0, kt0, b_even, b_odd, kn);
         }
+        if (k0 < k_end)
+            kblock(nv_tag, a0, kt0, a1, kt1, b_even, b_odd, k0);
     };
     // The image goes through LDS in stages of CG channels (all of them when they fit); the accumulators stay.
     const T *ximg = static_cast<const T *>(g.x) + static_cast<size_t>(img) * g.C * g.H * g.W;
@@ -511,11 +535,10 @@ __global__ __launch_bounds__(512) void conv2d_resident_kernel(ConvResidentArgs g
                 ktab[k] = g.ktab[k];
         }
         __syncthreads();
-        const int sub = static_cast<int>(c0 * g.HpWp);
         if (nfv == NF - 1)
-            contract(std::integral_constant<int, NF - 1>{}, k_begin, k_end, sub);
+            contract(std::integral_constant<int, NF - 1>{}, k_begin, k_end);
         else if (nfv > 0)
-            contract(std::integral_constant<int, NF>{}, k_begin, k_end, sub);
+            contract(std::integral_constant<int, NF>{}, k_begin, k_end);
     }
 
     T *out = static_cast<T *>(g.res) + static_cast<size_t>(img) * g.F * PQout;
@@ -805,7 +828,8 @@ dh_status conv2d_forward(dh_ctx *ctx, T *res, size_t *res_h, size_t *res_w, cons
             hipLaunchKernelGGL((conv_prep_kernel<T>), dim3(static_cast<unsigned>(pg)), dim3(256), 0, ctx->stream, tab, wpack,
                                filter, static_cast<unsigned>(F), static_cast<unsigned>(fpad), static_cast<unsigned>(K),
                                static_cast<unsigned>(kpad), static_cast<unsigned>(Hp * Wp), static_cast<unsigned>(Wp),
-                               static_cast<unsigned>(Hf), static_cast<unsigned>(Wf));
+                               static_cast<unsigned>(Hf), static_cast<unsigned>(Wf), static_cast<unsigned>(cg),
+                               static_cast<unsigned>(sizeof(T)));
             DH_CHECK_LAUNCH();
             ConvResidentArgs r{};
             r.x = data;
