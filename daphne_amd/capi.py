@@ -59,6 +59,8 @@ def _signatures(lib: C.CDLL) -> None:
     lib.dh_ctx_get_stream.argtypes = [ctxp]
     lib.dh_ctx_get_stream.restype = vp
     lib.dh_sync.argtypes = [ctxp]
+    lib.dh_defer_checks.argtypes = [ctxp, i32]
+    lib.dh_check_deferred.argtypes = [ctxp]
     lib.dh_malloc.argtypes = [ctxp, sz, i32, C.POINTER(vp)]
     lib.dh_free.argtypes = [ctxp, vp]
     lib.dh_h2d.argtypes = [ctxp, vp, vp, sz]

@@ -40,6 +40,36 @@ inline void check(dh_status st) {
         throw std::runtime_error(msg);
     }
 }
+
+// While one of these lives, kernels that validate their arguments on the device (integer DIV / MOD, SQRT / LN /
+// ASIN / ACOS, ExtractCol positions) do not wait for their verdict after every call (dh_defer_checks). finish()
+// leaves that mode and throws what the first failing call would have thrown; a scope left without finish() - an
+// exception on its way out - leaves the mode too and drops a pending verdict, so that none outlives its scope.
+class DeferredChecks {
+    dh_ctx *ctx;
+    bool open = false;
+
+  public:
+    explicit DeferredChecks(dh_ctx *c) : ctx(c) {
+        check(dh_defer_checks(ctx, 1));
+        open = true;
+    }
+    DeferredChecks(const DeferredChecks &) = delete;
+    DeferredChecks &operator=(const DeferredChecks &) = delete;
+    void finish() {
+        if (!open)
+            return;
+        open = false;
+        check(dh_defer_checks(ctx, 0));
+        check(dh_check_deferred(ctx));
+    }
+    ~DeferredChecks() {
+        if (open) {
+            (void)dh_defer_checks(ctx, 0);
+            (void)dh_check_deferred(ctx);
+        }
+    }
+};
 } // namespace HIP
 
 class HIPContext final : public IContext {

@@ -13,7 +13,11 @@
 //         folded into a task-local partial with the elementwise kernel in place (res == lhs), and the partial into
 //         the shared result under the result lock when the task ends. The reference's device task knows ADD only;
 //         MIN and MAX follow its CPU task (Tasks.cpp:51-84).
-// Everything stays in device memory; nothing here synchronises with the host.
+// Everything stays in device memory, and no batch waits for the host: kernels of the body that validate their
+// arguments on the device (integer DIV / MOD, SQRT / LN / ASIN / ACOS, ExtractCol) run with deferred verdicts
+// (HIP::DeferredChecks), and execute() throws the first failure of any batch when the task's batches are enqueued -
+// the same exception, from the same call, as a body that checked after every kernel. A task whose body has no such
+// kernel never waits at all.
 //
 // In DAPHNE this file is src/runtime/local/vectorized/TasksHIP.h (header only: no device compiler needed).
 #pragma once
@@ -121,6 +125,7 @@ template <typename VT> class CompiledPipelineTaskHIP<DenseMatrix<VT>> : public C
         const size_t n = _data._numOutputs;
         std::vector<DT *> localAggRes(n, nullptr), localResults(n, nullptr), targets(n, nullptr);
         std::vector<DT **> outputs(n);
+        HIP::DeferredChecks verdicts(HIPContext::get(_data._ctx, 0)->raw());
         for (uint64_t r = _data._rl; r < _data._ru; r += batchSize) {
             const uint64_t r2 = std::min<uint64_t>(r + batchSize, _data._ru);
             auto linputs = this->createFuncInputs(r, r2);
@@ -139,6 +144,14 @@ template <typename VT> class CompiledPipelineTaskHIP<DenseMatrix<VT>> : public C
                 localResults[o] = targets[o] = nullptr;
             }
             // The body owns the references to its inputs (views included) and gives them back itself.
+        }
+        try {
+            verdicts.finish(); // before the task's partial aggregates are folded into the shared results
+        } catch (...) {
+            for (DT *partial : localAggRes)
+                if (partial != nullptr)
+                    DataObjectFactory::destroy(partial);
+            throw;
         }
         for (size_t o = 0; o < n; ++o) {
             if (!isAggregating(_data._combines[o]) || localAggRes[o] == nullptr)

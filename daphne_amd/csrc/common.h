@@ -53,6 +53,11 @@ struct dh_ctx {
     // The host mirror as the device sees it: a kernel that reports through it spares the copy back (the caller still
     // waits for the stream before it reads flag_host). Plain stores only - no atomics on host memory.
     int *flag_host_dev = nullptr;
+    // Deferred verdicts (dh_defer_checks): while deferred_depth > 0 a checked call does not read its flag back; a
+    // one-thread kernel copies a raised flag into the record at flag_dev + DH_DEFERRED_AT (the first one stays) and
+    // dh_check_deferred reads that record. The record's host mirror is flag_host + DH_DEFERRED_AT.
+    int deferred_depth = 0;
+    size_t deferred_enqueued = 0; // checked calls since the last dh_check_deferred (none: nothing to wait for)
 
     hipEvent_t ev_start = nullptr, ev_stop = nullptr;
     int num_cus = 0;
@@ -97,6 +102,21 @@ dh_status dh_fail(dh_status st, const char *fmt, ...) __attribute__((format(prin
             return dh_fail(DH_ERR_HIP, "hipSetDevice(%d): %s", (ctx)->device,                      \
                            hipGetErrorString(e__));                                                \
     } while (0)
+
+// The deferred-verdict record, in ints from flag_dev / flag_host (both are 256 bytes; int 0 is the flag of a checked
+// call and the 8 bytes at byte 64 are the result slot of AggAll):
+//   [0] kind (0: nothing pending)  [1] operator code  [2..3] a 64-bit value  [4..5] a 64-bit bound
+constexpr int DH_DEFERRED_AT = 32, DH_DEFERRED_INTS = 6;
+enum { DH_DEFERRED_NONE = 0, DH_DEFERRED_INT_DIVMOD = 1, DH_DEFERRED_UNARY_DOMAIN = 2, DH_DEFERRED_EXTRACT_COL = 3, DH_DEFERRED_PIPELINE_DOMAIN = 4 };
+// The failures a checked call reports, immediately or from dh_check_deferred (context.hip).
+dh_status dh_fail_int_divmod(int op);
+dh_status dh_fail_unary_domain(int op);
+dh_status dh_fail_extract_col(long long position, size_t cols);
+dh_status dh_fail_pipeline_domain();
+// After the kernels of a checked call on a context that defers its verdicts: enqueues the kernel that keeps the
+// call's flag (at ctx->flag_dev, raised if != ok_value) in the deferred record. sel != nullptr: the flag is the
+// index + 1 of the offending entry of sel (stride ld_sel), whose value is kept along with `bound`.
+dh_status dh_latch_deferred(dh_ctx *ctx, int ok_value, int kind, int op, const long long *sel, size_t ld_sel, long long bound);
 
 // Returns a workspace of at least `bytes` bytes (256-byte aligned). Growing frees the old
 // buffer after a stream synchronise.

@@ -69,6 +69,7 @@ extern "C" dh_status dh_ctx_create(int device, dh_ctx **out) {
               hipHostMalloc(reinterpret_cast<void **>(&ctx->flag_host), 256, hipHostMallocMapped) == hipSuccess &&
               hipHostGetDevicePointer(reinterpret_cast<void **>(&ctx->flag_host_dev), ctx->flag_host, 0) == hipSuccess &&
               hipEventCreate(&ctx->ev_start) == hipSuccess && hipEventCreate(&ctx->ev_stop) == hipSuccess;
+    ok = ok && hipMemset(ctx->flag_dev, 0, 256) == hipSuccess; // no deferred verdict pending
     if (!ok) {
         dh_ctx_destroy(ctx);
         return dh_fail(DH_ERR_HIP, "dh_ctx_create: could not allocate the context's flag words / events");
@@ -143,6 +144,103 @@ extern "C" dh_status dh_sync(dh_ctx *ctx) {
     DH_REQUIRE_CTX(ctx);
     DH_CHECK_HIP(hipStreamSynchronize(ctx->stream));
     return DH_OK;
+}
+
+// ---------------------------------------------------------------------------------------
+// deferred verdicts
+// ---------------------------------------------------------------------------------------
+dh_status dh_fail_int_divmod(int op) {
+    return dh_fail(DH_ERR_DOMAIN, "integer %s: a divisor is zero%s", op == DH_BIN_DIV ? "division" : "remainder",
+                   op == DH_BIN_DIV ? " or the quotient does not fit the value type" : "");
+}
+
+dh_status dh_fail_unary_domain(int op) {
+    const char *dom = op == DH_UN_SQRT   ? "SQRT with domain [-0, inf]"
+                      : op == DH_UN_LN   ? "LN with domain [-0, inf]"
+                      : op == DH_UN_ASIN ? "ASIN with domain [-1, 1]"
+                                         : "ACOS with domain [-1, 1]";
+    return dh_fail(DH_ERR_DOMAIN, "invalid argument passed to unary func %s", dom);
+}
+
+dh_status dh_fail_extract_col(long long position, size_t cols) {
+    return dh_fail(DH_ERR_OUT_OF_RANGE,
+                   "invalid argument '%lld' passed to ExtractCol: out of bounds for dense matrix with column "
+                   "boundaries '[0, %zu)'",
+                   position, cols);
+}
+
+dh_status dh_fail_pipeline_domain() {
+    return dh_fail(DH_ERR_DOMAIN, "invalid argument passed to a unary function inside the pipeline");
+}
+
+// One thread: the record keeps the first failure of the stream's order.
+static __global__ void latch_deferred_kernel(const int *flag, int ok_value, int *rec, int kind, int op, const long long *sel,
+                                             size_t ld_sel, long long bound) {
+    const int f = *flag;
+    if (f == ok_value || rec[0] != DH_DEFERRED_NONE)
+        return;
+    const long long v = sel ? sel[static_cast<size_t>(f - 1) * ld_sel] : 0;
+    rec[1] = op;
+    rec[2] = static_cast<int>(static_cast<unsigned long long>(v) & 0xffffffffull);
+    rec[3] = static_cast<int>(static_cast<unsigned long long>(v) >> 32);
+    rec[4] = static_cast<int>(static_cast<unsigned long long>(bound) & 0xffffffffull);
+    rec[5] = static_cast<int>(static_cast<unsigned long long>(bound) >> 32);
+    rec[0] = kind;
+}
+
+static __global__ void clear_deferred_kernel(int *rec) {
+    if (threadIdx.x < DH_DEFERRED_INTS)
+        rec[threadIdx.x] = 0;
+}
+
+dh_status dh_latch_deferred(dh_ctx *ctx, int ok_value, int kind, int op, const long long *sel, size_t ld_sel, long long bound) {
+    hipLaunchKernelGGL(latch_deferred_kernel, dim3(1), dim3(1), 0, ctx->stream, ctx->flag_dev, ok_value,
+                       ctx->flag_dev + DH_DEFERRED_AT, kind, op, sel, ld_sel, bound);
+    DH_CHECK_LAUNCH();
+    ctx->deferred_enqueued++;
+    return DH_OK;
+}
+
+extern "C" dh_status dh_defer_checks(dh_ctx *ctx, int on) {
+    DH_REQUIRE_CTX(ctx);
+    if (on)
+        ctx->deferred_depth++;
+    else if (ctx->deferred_depth > 0)
+        ctx->deferred_depth--;
+    else
+        return dh_fail(DH_ERR_RUNTIME, "dh_defer_checks: left more often than entered");
+    return DH_OK;
+}
+
+extern "C" dh_status dh_check_deferred(dh_ctx *ctx) {
+    DH_REQUIRE_CTX(ctx);
+    if (ctx->deferred_enqueued == 0)
+        return DH_OK; // no checked call since the last verdict: nothing can be pending
+    ctx->deferred_enqueued = 0;
+    int *rec = ctx->flag_host + DH_DEFERRED_AT;
+    DH_CHECK_HIP(hipMemcpyAsync(rec, ctx->flag_dev + DH_DEFERRED_AT, DH_DEFERRED_INTS * sizeof(int), hipMemcpyDeviceToHost,
+                                ctx->stream));
+    DH_CHECK_HIP(hipStreamSynchronize(ctx->stream));
+    if (rec[0] == DH_DEFERRED_NONE)
+        return DH_OK;
+    // a small kernel, not a memset, so that a caller may capture this stream (memset nodes replay badly)
+    hipLaunchKernelGGL(clear_deferred_kernel, dim3(1), dim3(64), 0, ctx->stream, ctx->flag_dev + DH_DEFERRED_AT);
+    DH_CHECK_LAUNCH();
+    const long long value = static_cast<long long>((static_cast<unsigned long long>(static_cast<unsigned>(rec[3])) << 32) |
+                                                   static_cast<unsigned>(rec[2]));
+    const unsigned long long bound = (static_cast<unsigned long long>(static_cast<unsigned>(rec[5])) << 32) | static_cast<unsigned>(rec[4]);
+    switch (rec[0]) {
+    case DH_DEFERRED_INT_DIVMOD:
+        return dh_fail_int_divmod(rec[1]);
+    case DH_DEFERRED_UNARY_DOMAIN:
+        return dh_fail_unary_domain(rec[1]);
+    case DH_DEFERRED_EXTRACT_COL:
+        return dh_fail_extract_col(value, static_cast<size_t>(bound));
+    case DH_DEFERRED_PIPELINE_DOMAIN:
+        return dh_fail_pipeline_domain();
+    default:
+        return dh_fail(DH_ERR_RUNTIME, "dh_check_deferred: unknown record kind %d", rec[0]);
+    }
 }
 
 // Capacity class of a request: multiples of 512 B below 64 KiB, above that 1/16 of the largest

@@ -257,11 +257,12 @@ static inline dh_status dispatch_binary(dh_ctx *ctx, int op, T *res, size_t ld_r
 #undef DH_CASE
     DH_CHECK_LAUNCH();
     if (checks) {
+        if (ctx->deferred_depth > 0) // the verdict waits for dh_check_deferred
+            return dh_latch_deferred(ctx, 0, DH_DEFERRED_INT_DIVMOD, op, nullptr, 0, 0);
         DH_CHECK_HIP(hipMemcpyAsync(ctx->flag_host, ctx->flag_dev, sizeof(int), hipMemcpyDeviceToHost, ctx->stream));
         DH_CHECK_HIP(hipStreamSynchronize(ctx->stream));
         if (*ctx->flag_host != 0)
-            return dh_fail(DH_ERR_DOMAIN, "integer %s: a divisor is zero%s", op == DH_BIN_DIV ? "division" : "remainder",
-                           op == DH_BIN_DIV ? " or the quotient does not fit the value type" : "");
+            return dh_fail_int_divmod(op);
     }
     return DH_OK;
 }
@@ -357,15 +358,12 @@ dh_status ew_unary(dh_ctx *ctx, int op, T *res, size_t ld_res, const T *arg, siz
 #undef DH_CASE
     DH_CHECK_LAUNCH();
     if (checks) {
+        if (ctx->deferred_depth > 0) // the verdict waits for dh_check_deferred
+            return dh_latch_deferred(ctx, 0, DH_DEFERRED_UNARY_DOMAIN, op, nullptr, 0, 0);
         DH_CHECK_HIP(hipMemcpyAsync(ctx->flag_host, ctx->flag_dev, sizeof(int), hipMemcpyDeviceToHost, ctx->stream));
         DH_CHECK_HIP(hipStreamSynchronize(ctx->stream));
-        if (*ctx->flag_host != 0) {
-            const char *dom = op == DH_UN_SQRT   ? "SQRT with domain [-0, inf]"
-                              : op == DH_UN_LN   ? "LN with domain [-0, inf]"
-                              : op == DH_UN_ASIN ? "ASIN with domain [-1, 1]"
-                                                 : "ACOS with domain [-1, 1]";
-            return dh_fail(DH_ERR_DOMAIN, "invalid argument passed to unary func %s", dom);
-        }
+        if (*ctx->flag_host != 0)
+            return dh_fail_unary_domain(op);
     }
     return DH_OK;
 }

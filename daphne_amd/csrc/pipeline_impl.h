@@ -276,10 +276,12 @@ dh_status run(dh_ctx *ctx, const dh_pipe_instr *prog, int n, const IO_C *cio, si
             DH_CHECK_LAUNCH();
         }
     if (checks) {
+        if (ctx->deferred_depth > 0) // the verdict waits for dh_check_deferred
+            return dh_latch_deferred(ctx, 0, DH_DEFERRED_PIPELINE_DOMAIN, 0, nullptr, 0, 0);
         DH_CHECK_HIP(hipMemcpyAsync(ctx->flag_host, ctx->flag_dev, sizeof(int), hipMemcpyDeviceToHost, ctx->stream));
         DH_CHECK_HIP(hipStreamSynchronize(ctx->stream));
         if (*ctx->flag_host != 0)
-            return dh_fail(DH_ERR_DOMAIN, "invalid argument passed to a unary function inside the pipeline");
+            return dh_fail_pipeline_domain();
     }
     return DH_OK;
 }

@@ -185,6 +185,8 @@ __global__ __launch_bounds__(256) void extract_col_kernel(T *res, size_t ld_res,
     long long c = sel[k * ld_sel];
     if (c < 0)
         c += static_cast<long long>(cols);
+    // a position that is out of range (reported by check_sel_kernel) reads column 0
+    c = (c < 0 || static_cast<unsigned long long>(c) >= cols) ? 0 : c;
     res[r * ld_res + k] = arg[r * ld + static_cast<size_t>(c)];
 }
 
@@ -213,7 +215,9 @@ __global__ __launch_bounds__(256) void extract_col_rows_kernel(T *res, size_t ld
     }
     for (unsigned k = tid; k < nsel; k += 256) {
         long long c = sel[k * ld_sel];
-        selc[k] = static_cast<unsigned>(c < 0 ? c + static_cast<long long>(cols) : c);
+        c = c < 0 ? c + static_cast<long long>(cols) : c;
+        // a position that is out of range (reported by check_sel_kernel) reads column 0
+        selc[k] = (c < 0 || c >= static_cast<long long>(cols)) ? 0u : static_cast<unsigned>(c);
     }
     T *mine = park + wave * (UN * 64 * VEC);
 #pragma unroll
@@ -254,16 +258,21 @@ dh_status extract_col(dh_ctx *ctx, T *res, size_t ld_res, const T *arg, size_t r
     hipLaunchKernelGGL(check_sel_kernel, dim3(static_cast<unsigned>(cg)), dim3(256), 0, ctx->stream, sel, sel_rows, ld_sel,
                        cols, ctx->flag_dev);
     DH_CHECK_LAUNCH();
-    DH_CHECK_HIP(hipMemcpyAsync(ctx->flag_host, ctx->flag_dev, sizeof(int), hipMemcpyDeviceToHost, ctx->stream));
-    DH_CHECK_HIP(hipStreamSynchronize(ctx->stream));
-    if (*ctx->flag_host != 0x7fffffff) {
-        const size_t bad = static_cast<size_t>(*ctx->flag_host) - 1;
-        long long v = 0;
-        DH_CHECK_HIP(hipMemcpy(&v, sel + bad * ld_sel, sizeof(v), hipMemcpyDeviceToHost));
-        return dh_fail(DH_ERR_OUT_OF_RANGE,
-                       "invalid argument '%lld' passed to ExtractCol: out of bounds for dense matrix with column "
-                       "boundaries '[0, %zu)'",
-                       v, cols);
+    if (ctx->deferred_depth > 0) {
+        // the verdict waits for dh_check_deferred; the kernels below keep a bad position inside the row, and what
+        // they then extract is never used
+        if (dh_status st = dh_latch_deferred(ctx, 0x7fffffff, DH_DEFERRED_EXTRACT_COL, 0, sel, ld_sel, static_cast<long long>(cols));
+            st != DH_OK)
+            return st;
+    } else {
+        DH_CHECK_HIP(hipMemcpyAsync(ctx->flag_host, ctx->flag_dev, sizeof(int), hipMemcpyDeviceToHost, ctx->stream));
+        DH_CHECK_HIP(hipStreamSynchronize(ctx->stream));
+        if (*ctx->flag_host != 0x7fffffff) {
+            const size_t bad = static_cast<size_t>(*ctx->flag_host) - 1;
+            long long v = 0;
+            DH_CHECK_HIP(hipMemcpy(&v, sel + bad * ld_sel, sizeof(v), hipMemcpyDeviceToHost));
+            return dh_fail_extract_col(v, cols);
+        }
     }
     {
         // whole rows where a gather would fetch most of them anyway: rows of a power-of-two number of 16-byte vectors

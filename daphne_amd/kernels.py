@@ -83,6 +83,30 @@ class HIPContext:
     def sync(self) -> None:
         capi.check(capi.lib().dh_sync(self._h))
 
+    def deferred_checks(self):
+        """Context manager: inside it, kernels that validate their arguments on the device (integer DIV / MOD,
+        SQRT / LN / ASIN / ACOS, ExtractCol positions) do not wait for their verdict; the first failure is raised
+        when the block ends (or by check_deferred() inside it)."""
+        ctx = self
+
+        class _Deferred:
+            def __enter__(self_inner):
+                capi.check(capi.lib().dh_defer_checks(ctx._h, 1))
+                return ctx
+
+            def __exit__(self_inner, exc_type, exc, tb):
+                capi.check(capi.lib().dh_defer_checks(ctx._h, 0))
+                if exc_type is None:
+                    ctx.check_deferred()
+                else:  # do not let a pending verdict leak into later calls
+                    capi.lib().dh_check_deferred(ctx._h)
+                return False
+
+        return _Deferred()
+
+    def check_deferred(self) -> None:
+        capi.check(capi.lib().dh_check_deferred(self._h))
+
     def set_pipeline_mode(self, mode: int) -> None:
         """1: fused pipeline bodies are specialised at run time, 0: interpreted, -1: as the environment says."""
         capi.check(capi.lib().dh_ctx_set_pipeline_mode(self._h, mode))

@@ -104,6 +104,22 @@ dh_status dh_ctx_set_stream(dh_ctx *ctx, void *hip_stream);
 void *dh_ctx_get_stream(const dh_ctx *ctx);
 /* Blocks until all work enqueued on the context's stream has finished. */
 dh_status dh_sync(dh_ctx *ctx);
+/* Deferred verdicts. Some kernels can only tell on the device whether their arguments were valid: integer DIV and MOD
+ * (a zero divisor, EwBinarySca.h:114-127 through the host's arithmetic), SQRT / LN / ASIN / ACOS (EwUnarySca.h:130-170),
+ * the column positions of ExtractCol (ExtractCol.h:98-108) and checked unary functions inside a fused pipeline body.
+ * By default such a call waits for its kernels and returns the failure itself, as the CPU kernel throws. A caller that
+ * runs many of them back to back - the task of a vectorized pipeline walking its batches,
+ * vectorized/TasksCUDA.cpp:61-100 has no counterpart because the CUDA kernels do not check - enters deferred mode:
+ *   dh_defer_checks(ctx, 1)   from now on these calls return DH_OK without waiting; the first failure in the stream's
+ *                             order is kept on the device (results computed from invalid arguments are unspecified,
+ *                             but every access stays inside its matrix). Calls nest; each needs a matching
+ *   dh_defer_checks(ctx, 0)   which leaves the mode (a pending failure stays pending).
+ *   dh_check_deferred(ctx)    returns DH_OK at once if no such call was made since the last verdict; else waits
+ *                             for the stream and returns DH_OK, or the pending failure with the status and
+ *                             message the immediate form would have given, and clears it. Valid in either mode.
+ * Neither call has a counterpart in the reference. */
+dh_status dh_defer_checks(dh_ctx *ctx, int on);
+dh_status dh_check_deferred(dh_ctx *ctx);
 
 /* CUDAContext::malloc(size, zero, id) / free(id) (CUDAContext.cpp:120-135). The device
  * pointer itself is the registry key. Fails with DH_ERR_OOM past the budget.

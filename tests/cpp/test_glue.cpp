@@ -350,6 +350,103 @@ template <typename VT> void run_integer_elementwise(DaphneContext *dctx) {
         DataObjectFactory::destroy(m);
 }
 
+// A pipeline body with one integer division, the way the compiler outlines it.
+static void funDivSi64(DenseMatrix<int64_t> ***outputs, Structure **inputs, DCTX(ctx)) {
+    auto *a = dynamic_cast<DenseMatrix<int64_t> *>(inputs[0]), *b = dynamic_cast<DenseMatrix<int64_t> *>(inputs[1]);
+    HIP::ewBinaryMat(BinaryOpCode::DIV, *outputs[0], a, b, ctx);
+    DataObjectFactory::destroy(a);
+    DataObjectFactory::destroy(b);
+}
+
+// Kernels that validate their arguments on the device, called batch after batch by a pipeline task: no batch waits
+// for its verdict, and the task's execute() still throws what the failing kernel would have thrown.
+static void run_deferred_verdicts(DaphneContext *dctx) {
+    using DT = DenseMatrix<int64_t>;
+    dh_ctx *raw = HIPContext::get(dctx, 0)->raw();
+    const size_t rows = 700, cols = 4;
+    std::vector<int64_t> num(rows * cols), den(rows * cols);
+    for (size_t i = 0; i < num.size(); i++) {
+        num[i] = int64_t(i) * 7 - 1000;
+        den[i] = int64_t(i % 9) + 1;
+    }
+    auto a = given<DT>(rows, num), good = given<DT>(rows, den);
+    den[250 * cols + 1] = 0; // batch 3 of 7 with 100 rows to a batch
+    auto bad = given<DT>(rows, den);
+    auto result = DataObjectFactory::create<DT>(rows, cols, false);
+    DT **resPtr = &result;
+    bool isScalar[] = {false, false};
+    int64_t outRows[] = {int64_t(rows)}, outCols[] = {int64_t(cols)};
+    const VectorSplit splits[] = {VectorSplit::ROWS, VectorSplit::ROWS};
+    const VectorCombine combines[] = {VectorCombine::ROWS};
+    std::mutex resLock;
+    auto task = [&](DT *divisor) {
+        Structure *inputs[] = {a, divisor};
+        CompiledPipelineTaskData<DT> data{{&funDivSi64}, isScalar, inputs, 2, 1, outRows, outCols, splits, combines, 0, rows, outRows, outCols, 0, dctx};
+        CompiledPipelineTaskHIP<DT> t(data, resLock, &resPtr);
+        t.execute(0, 100);
+    };
+    // result is written on the device by the task: say so, as the pipeline kernel does before it starts its tasks
+    {
+        AllocationDescriptorHIP alloc_desc(dctx, 0);
+        (void)result->getValues(&alloc_desc);
+    }
+    task(good);
+    {
+        const auto got = toHost(result);
+        bool ok = got.size() == num.size();
+        for (size_t i = 0; ok && i < got.size(); i++)
+            ok = got[i] == num[i] / (int64_t(i % 9) + 1);
+        CHECK(ok);
+    }
+    CHECK_THROWS_AS(task(bad), std::domain_error);
+    // the verdict went with the exception: the next task on the context starts clean, and so does a direct call
+    CHECK(dh_check_deferred(raw) == DH_OK);
+    task(good);
+    DT *direct = nullptr;
+    CHECK_THROWS_AS(HIP::ewBinaryMat(BinaryOpCode::MOD, direct, a, bad, dctx), std::domain_error); // immediate outside a task
+    HIP::ewBinaryMat(BinaryOpCode::MOD, direct, a, good, dctx);
+    CHECK(direct != nullptr);
+
+    // the C ABI directly: first failure in stream order wins, its status and message are those of the immediate form
+    {
+        AllocationDescriptorHIP alloc_desc(dctx, 0);
+        const int64_t *pa = a->getValues(&alloc_desc), *pbad = bad->getValues(&alloc_desc);
+        int64_t *pres = result->getValues(&alloc_desc);
+        DenseMatrix<double> *neg = given<DenseMatrix<double>>(1, {4.0, -1.0, 9.0}), *root = DataObjectFactory::create<DenseMatrix<double>>(1, 3, false);
+        const double *pneg = neg->getValues(&alloc_desc);
+        double *proot = root->getValues(&alloc_desc);
+        auto sel = given<DT>(2, {1, 17});
+        const int64_t *psel = sel->getValues(&alloc_desc);
+        auto picked = DataObjectFactory::create<DT>(rows, 2, false);
+        int64_t *ppicked = picked->getValues(&alloc_desc);
+        CHECK(dh_defer_checks(raw, 1) == DH_OK);
+        CHECK(dh_defer_checks(raw, 1) == DH_OK); // nests
+        CHECK(dh_ew_unary_f64(raw, DH_UN_SQRT, proot, 3, pneg, 1, 3, 3) == DH_OK);
+        CHECK(dh_ew_binary_si64(raw, DH_BIN_MOD, pres, cols, pa, rows, cols, cols, pbad, rows, cols, cols) == DH_OK);
+        CHECK(dh_extract_col_si64(raw, ppicked, 2, pa, rows, cols, cols, psel, 2, 1, 1) == DH_OK);
+        CHECK(dh_defer_checks(raw, 0) == DH_OK);
+        CHECK(dh_defer_checks(raw, 0) == DH_OK);
+        CHECK(dh_defer_checks(raw, 0) != DH_OK); // left more often than entered
+        CHECK(dh_check_deferred(raw) == DH_ERR_DOMAIN);
+        CHECK(std::string(dh_last_error()).find("SQRT") != std::string::npos);
+        CHECK(dh_check_deferred(raw) == DH_OK); // cleared
+        // ExtractCol alone: the position and the bounds are in the message, the extraction itself stayed in bounds
+        CHECK(dh_defer_checks(raw, 1) == DH_OK);
+        CHECK(dh_extract_col_si64(raw, ppicked, 2, pa, rows, cols, cols, psel, 2, 1, 1) == DH_OK);
+        CHECK(dh_defer_checks(raw, 0) == DH_OK);
+        CHECK(dh_check_deferred(raw) == DH_ERR_OUT_OF_RANGE);
+        CHECK(std::string(dh_last_error()).find("'17'") != std::string::npos && std::string(dh_last_error()).find("[0, 4)") != std::string::npos);
+        // immediate mode again
+        CHECK(dh_extract_col_si64(raw, ppicked, 2, pa, rows, cols, cols, psel, 2, 1, 1) == DH_ERR_OUT_OF_RANGE);
+        for (auto *m : {sel, picked})
+            DataObjectFactory::destroy(m);
+        DataObjectFactory::destroy(neg);
+        DataObjectFactory::destroy(root);
+    }
+    for (auto *m : {a, good, bad, result, direct})
+        DataObjectFactory::destroy(m);
+}
+
 static void run_si64(DaphneContext *dctx) {
     using DT = DenseMatrix<int64_t>;
     auto G = [&](size_t rows, std::vector<int64_t> v) { return given<DT>(rows, v); };
@@ -526,6 +623,7 @@ int main(int argc, char **argv) {
     run_placement(dctx.get());
     run_pipeline_tasks<float>(dctx.get());
     run_pipeline_tasks<double>(dctx.get());
+    run_deferred_verdicts(dctx.get());
     if (argc > 1) // path of libHIPKernels.so
         run_generated_wrappers(dctx.get(), argv[1]);
     std::printf("%s: %d checks, %d failed\n", g_fail ? "FAILED" : "PASSED", g_checks, g_fail);

@@ -176,3 +176,45 @@ def test_si64_reorganisation(ctx, shape):
         extractCol(None, X, DenseMatrix.from_numpy(ctx, np.array([[shape[1]]], dtype=np.int64)), ctx)
     assert_exact(fill(None, -(2 ** 62) - 3, 7, 9, ctx, dtype=np.int64).to_numpy(), orc.fill(-(2 ** 62) - 3, 7, 9, np.int64)[1])
     assert_exact(fill(None, 2 ** 63 + 5, 33, 2, ctx, dtype=np.uint64).to_numpy(), orc.fill(2 ** 63 + 5, 33, 2, np.uint64)[1])
+
+
+def test_deferred_verdicts_report_the_first_failure_once(ctx):
+    """With verdicts deferred, checked calls return at once (results of valid calls are unchanged) and the first
+    failure in call order is raised when the block ends, with the status and text of the immediate form."""
+    rng = np.random.default_rng(11)
+    a, b = _ints(rng, (700, 4), np.int64), _ints(rng, (700, 4), np.int64)
+    b[b == 0] = 3
+    z = b.copy()
+    z[250, 1] = 0
+    A, B, Z = (DenseMatrix.from_numpy(ctx, m) for m in (a, b, z))
+    sel_bad = DenseMatrix.from_numpy(ctx, np.array([[1], [17]], dtype=np.int64))
+    sel_ok = DenseMatrix.from_numpy(ctx, np.array([[3], [-4]], dtype=np.int64))
+    with ctx.deferred_checks():
+        q = ewBinaryMat(BinaryOpCode.DIV, None, A, B, ctx)
+        r = ewBinaryMat(BinaryOpCode.MOD, None, A, B, ctx)
+        e = extractCol(None, A, sel_ok, ctx)
+    assert_exact(q.to_numpy(), orc.ew_binary(BinaryOpCode.DIV, a, b)[1])
+    assert_exact(r.to_numpy(), orc.ew_binary(BinaryOpCode.MOD, a, b)[1])
+    assert_exact(e.to_numpy(), orc.extract_col(a, np.array([[3], [-4]], dtype=np.int64))[1])
+    # a failure among valid calls: raised at the end of the block, by the call order's first failing call
+    with pytest.raises(capi.DaphneHipOutOfRange, match=r"'17'.*\[0, 4\)"):
+        with ctx.deferred_checks():
+            ewBinaryMat(BinaryOpCode.DIV, None, A, B, ctx)
+            extractCol(None, A, sel_bad, ctx)      # first
+            ewBinaryMat(BinaryOpCode.MOD, None, A, Z, ctx)  # second: not the one reported
+    ctx.check_deferred()  # nothing left pending
+    with pytest.raises(capi.DaphneHipDomainError, match="remainder"):
+        with ctx.deferred_checks():
+            with ctx.deferred_checks():  # nests
+                ewBinaryMat(BinaryOpCode.MOD, None, A, Z, ctx)
+            # the inner block ending reports already: the outer one never gets here
+    # an exception of the caller's own inside the block leaves the mode and drops what was pending
+    with pytest.raises(KeyError):
+        with ctx.deferred_checks():
+            ewBinaryMat(BinaryOpCode.DIV, None, A, Z, ctx)
+            raise KeyError("the caller's own")
+    ctx.check_deferred()
+    # immediate form as before
+    with pytest.raises(capi.DaphneHipDomainError):
+        ewBinaryMat(BinaryOpCode.DIV, None, A, Z, ctx)
+    assert_exact(ewBinaryMat(BinaryOpCode.DIV, None, A, B, ctx).to_numpy(), orc.ew_binary(BinaryOpCode.DIV, a, b)[1])
