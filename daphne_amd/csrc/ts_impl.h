@@ -398,10 +398,13 @@ struct TsNtArgs {
 // (C * -2 + row_add[row]) + col_add[col] (three separately rounded operations) and the row's IDXMIN over it: the first
 // position of the strict minimum, NaN never better, position 0 if the first value is NaN or all are.
 // UPDATE (with ASSIGN; float, one step per pair of row blocks with four chunks, i.e. 49..64 columns): the rows, read
-// back from the wave's staging piece as they were loaded - lane group h on row 4 c + h, lane i on vector i, the
-// operand layout of t(P) X - go through the matrix instruction once more against the one-hot of the assignment just
-// found, so that one pass over A gives the assignment, the per-position sums and the counts. The grid is then what the device holds at
-// once (one partial result per workgroup) and deals the pairs round-robin.
+// back from the wave's staging piece one at a time - lane j on column j -, are added to the sum of the position just
+// found for them. A lane keeps its column's 16 NB sums in registers, and the position, the same for all lanes, picks
+// the register (register-relative moves): four ordinary instructions and an LDS read per row, where the one-hot
+// product t(P) X on the matrix cores costs as many matrix instructions again as the distances - sixteen times the
+// flops of these additions - plus the one-hot itself. One pass over A then gives the assignment, the per-position
+// sums and the counts. The grid is what the device holds at once (one partial result per workgroup) and deals the
+// pairs round-robin.
 template <typename T, int NB, bool ASSIGN, int CPG, bool UPDATE = false>
 __global__ __launch_bounds__(256, UPDATE ? (NB == 1 ? 3 : 2) : 1) void ts_nt_kernel(TsNtArgs g) {
     static_assert(!UPDATE || (ASSIGN && sizeof(T) == 4 && CPG == 4), "the one-pass form exists for float and 49..64 columns");
@@ -570,18 +573,17 @@ __global__ __launch_bounds__(256, UPDATE ? (NB == 1 ? 3 : 2) : 1) void ts_nt_ker
         else
             mma_step_k(acc, fr, grp, std::false_type{});
     };
-    // UPDATE: per-position sums (register v of lane (i, h), instruction e: position 16 a + 4 h + v, column 4 i + e) and counts
-    typename M::acc_t acc_s[UPDATE ? NB : 1][V];
-    T cnt[UPDATE ? NB : 1];
-    __shared__ __attribute__((aligned(16))) unsigned ridx[UPDATE ? 4 * 32 : 4];
+    // UPDATE: lane j holds the sums of column j for the 16 NB positions, the counts are integers in LDS (one set per wave)
+    constexpr unsigned NPOS = NB * 16;
+    typedef T sums_t __attribute__((ext_vector_type(UPDATE ? NB * 16 : 2)));
+    sums_t sums;
+    __shared__ unsigned cnts[UPDATE ? 4 * NPOS : 4];
     if constexpr (UPDATE) {
 #pragma unroll
-        for (int a = 0; a < NB; a++) {
-            cnt[a] = T(0);
-#pragma unroll
-            for (int e = 0; e < V; e++)
-                acc_s[a][e] = typename M::acc_t{0, 0, 0, 0};
-        }
+        for (unsigned p = 0; p < NPOS; p++)
+            sums[p] = T(0);
+        if (lane < NPOS)
+            cnts[wave * NPOS + lane] = 0u; // the wave's own entries: its LDS instructions execute in order
     }
     auto finish_pair = [&](AccSet &acc, unsigned pair, const T (&radd)[2][RPL]) {
         const size_t rbase = (first_pair + static_cast<size_t>(pair) * pair_stride) * 32;
@@ -633,36 +635,27 @@ __global__ __launch_bounds__(256, UPDATE ? (NB == 1 ? 3 : 2) : 1) void ts_nt_ker
                         g.idx[row] = bi[t];
                 }
                 if constexpr (UPDATE) {
-                    // the assignment goes to the lanes that hold the rows as rows: row r of the pair at entry 8 (r % 4) +
-                    // r / 4 of the wave's 32, so that lane group h finds its rows 4 c + h (c = 0 .. 7) side by side
-                    unsigned *mine = ridx + wave * 32;
-                    if (h == 0) {
+                    // after the exchanges every lane group holds the positions of its rows: lane r that of row r
+                    auto add_rows = [&](auto whole_tag) {
+                        constexpr bool WHOLE = decltype(whole_tag)::value; // no row of the pair lies beyond M
 #pragma unroll
                         for (int t = 0; t < 2; t++) {
-                            const unsigned r = t * 16 + i;
-                            mine[8 * (i % 4) + i / 4 + 4 * t] = rbase + r < g.M ? bi[t] : NONE; // rows beyond M belong nowhere
-                        }
-                    }
-                    unsigned of_row[2][4];
-                    dh_load_vec<unsigned, 4>(mine + 8 * h, of_row[0]);
-                    dh_load_vec<unsigned, 4>(mine + 8 * h + 4, of_row[1]);
+                            if (h == 0 && (WHOLE || rbase + t * 16 + i < g.M))
+                                atomicAdd(cnts + wave * NPOS + bi[t], 1u); // integers: the order does not matter
 #pragma unroll
-                    for (int t = 0; t < 2; t++)
-#pragma unroll
-                        for (int c = 0; c < 4; c++) {
-                            // the rows as rows - row 4 c + h, vector i - come back from the staging piece (kept in
-                            // registers since they were loaded, they would cost the kernel a wave per SIMD)
-                            T xr[V];
-                            dh_load_vec<T, V>(stage + (t * 16 + 4 * c + h) * SX + i * V, xr);
-#pragma unroll
-                            for (int a = 0; a < NB; a++) {
-                                const T p = of_row[t][c] == static_cast<unsigned>(a * 16 + i) ? T(1) : T(0);
-                                cnt[a] += p;
-#pragma unroll
-                                for (int e = 0; e < V; e++)
-                                    acc_s[a][e] = M::mma(p, xr[e], acc_s[a][e]);
+                            for (int r = 0; r < 16; r++) {
+                                const unsigned pos = static_cast<unsigned>(__builtin_amdgcn_readlane(static_cast<int>(bi[t]), r));
+                                T x = stage[(t * 16 + r) * SX + lane]; // the row as a row: lane j on column j
+                                if constexpr (!WHOLE)
+                                    x = rbase + t * 16 + r < g.M ? x : T(0); // rows beyond M repeat the last row
+                                sums[pos] += x;
                             }
                         }
+                    };
+                    if (rbase + 32 <= g.M) // the same in all lanes
+                        add_rows(std::true_type{});
+                    else
+                        add_rows(std::false_type{});
                 }
             } else {
                 // register v of lane (i, h) is C[row 4 v + h][column 16 b + i]: a row's values sit in the sixteen lanes of a group
@@ -822,61 +815,27 @@ __global__ __launch_bounds__(256, UPDATE ? (NB == 1 ? 3 : 2) : 1) void ts_nt_ker
         advance(cp, cgp);
     }
     if constexpr (UPDATE) {
-        // counts: the four lane groups of a wave counted different rows; then the four waves, added in wave order
-#pragma unroll
-        for (int a = 0; a < NB; a++) {
-            cnt[a] += dh_peer_swap<16>{}(cnt[a]);
-            cnt[a] += dh_peer_swap<32>{}(cnt[a]);
-        }
-        constexpr int NVAL = NB * V * 4 + NB;
-        static_assert(NVAL * 64 <= 4 * 2 * 16 * (4 * 4 * V + V), "the exchange area must fit the staging pieces");
+        // the workgroup's partial result: the four waves' sums and counts, added in wave order
+        static_assert(4 * NPOS * 64 <= 4 * 2 * 16 * (4 * 4 * V + V), "the exchange area must fit the staging pieces");
         __syncthreads(); // every wave is done with its staging piece: the exchange between the waves takes their place
-        T(*red)[64] = reinterpret_cast<T(*)[64]>(lb + NB * 16 * ldl);
-        for (int w = 1; w < 4; w++) {
-            if (wave == w) {
-                int q = 0;
+        T *red = lb + NB * 16 * ldl; // [wave][position][column]
 #pragma unroll
-                for (int a = 0; a < NB; a++) {
+        for (unsigned p = 0; p < NPOS; p++)
+            red[(wave * NPOS + p) * 64 + lane] = sums[p];
+        __syncthreads();
+        T *slab = static_cast<T *>(g.slabs) + static_cast<size_t>(blockIdx.x) * NPOS * g.K;
+        T *sizes = static_cast<T *>(g.slabs) + static_cast<size_t>(gridDim.x) * NPOS * g.K + static_cast<size_t>(blockIdx.x) * NPOS;
+        for (unsigned e = tid; e < NPOS * 64; e += 256) {
+            const unsigned cen = e / 64, col = e % 64;
+            T t = red[e];
 #pragma unroll
-                    for (int e = 0; e < V; e++)
-#pragma unroll
-                        for (int v = 0; v < 4; v++)
-                            red[q++][lane] = acc_s[a][e][v];
-                    red[q++][lane] = cnt[a];
-                }
-            }
-            __syncthreads();
-            if (wave == 0) {
-                int q = 0;
-#pragma unroll
-                for (int a = 0; a < NB; a++) {
-#pragma unroll
-                    for (int e = 0; e < V; e++)
-#pragma unroll
-                        for (int v = 0; v < 4; v++)
-                            acc_s[a][e][v] += red[q++][lane];
-                    cnt[a] += red[q++][lane];
-                }
-            }
-            __syncthreads();
+            for (unsigned w = 1; w < 4; w++)
+                t += red[w * NPOS * 64 + e];
+            if (col < g.K)
+                slab[static_cast<size_t>(cen) * g.K + col] = t;
         }
-        if (wave != 0)
-            return;
-        T *slab = static_cast<T *>(g.slabs) + static_cast<size_t>(blockIdx.x) * (NB * 16) * g.K;
-        T *sizes = static_cast<T *>(g.slabs) + static_cast<size_t>(gridDim.x) * (NB * 16) * g.K + static_cast<size_t>(blockIdx.x) * (NB * 16);
-#pragma unroll
-        for (int a = 0; a < NB; a++) {
-#pragma unroll
-            for (int v = 0; v < 4; v++) {
-                const unsigned cen = a * 16 + M::row(lane, v);
-#pragma unroll
-                for (int e = 0; e < V; e++)
-                    if (static_cast<unsigned>(V * i + e) < g.K)
-                        slab[static_cast<size_t>(cen) * g.K + V * i + e] = acc_s[a][e][v];
-            }
-            if (h == 0)
-                sizes[a * 16 + i] = cnt[a];
-        }
+        if (tid < NPOS)
+            sizes[tid] = static_cast<T>((cnts[tid] + cnts[NPOS + tid]) + (cnts[2 * NPOS + tid] + cnts[3 * NPOS + tid]));
     }
 }
 
