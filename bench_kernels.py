@@ -137,8 +137,11 @@ def main() -> int:
             CB.destroy()
             sel = DM.from_numpy(ctx, np.array([63, 0, 17, 5, 9, 33, 2, 41], dtype=np.int64).reshape(-1, 1))
             E = DM(ctx, rows, 8, ndt)
-            emit("extractCol 8 of 64 columns (sector traffic: whole rows)", dt, shape, timed(lambda: K.extractCol(E, X, sel, ctx)),
-                 nb + rows * 8 * sz)
+            t_ext = timed(lambda: K.extractCol(E, X, sel, ctx))
+            # two byte conventions for the same launches: what the memory system has to move (every 64-byte segment of
+            # a row holds a selected column, so whole rows), and the selected values alone (read once, written once)
+            emit("extractCol 8 of 64 columns (sector traffic: whole rows)", dt, shape, t_ext, nb + rows * 8 * sz)
+            emit("extractCol 8 of 64 columns (selected values only: 2 x rows x 8)", dt, shape, t_ext, 2 * rows * 8 * sz)
             E.destroy()
             L.destroy()
         # --- tall-and-skinny contractions ----------------------------------------------------------------------

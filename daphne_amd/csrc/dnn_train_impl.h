@@ -906,6 +906,9 @@ template <typename T> static bool conv_backward_data_mfma(dh_ctx *ctx, T *dX, co
 // the padded image into LDS, reads dY rows from global memory (a 16-byte vector of consecutive pixels per lane)
 // and gathers the patch values from LDS at "column offset + pixel offset". Every workgroup leaves one partial
 // F x K slab; a second kernel adds the slabs in order.
+// DB (small planes, two images fit LDS): the next image is copied into a second LDS frame while the current one is
+// contracted - a few channels per pixel block of the contraction, loaded at its start and stored at its end - so
+// that a workgroup that has its CU to itself never waits for an image, and an image costs one barrier, not two.
 // ---------------------------------------------------------------------------------------
 struct ConvFilterResidentArgs {
     const void *x;     // N x C x H x W
@@ -932,7 +935,8 @@ static __global__ __launch_bounds__(256) void conv_filter_tables_kernel(int *kof
         pixtab[i] = i < PQ ? static_cast<int>((i / Q) * sh * Wp + (i % Q) * sw) : 0;
 }
 
-template <typename T, int MFW, int WAVES, int NF>
+constexpr int CONV_FILTER_STAGE_CH = 4; // DB: channels of the next image that one pixel block of the contraction brings in, at most
+template <typename T, int MFW, int WAVES, int NF, bool DB>
 __global__ __launch_bounds__(64 * WAVES) void conv_filter_resident_kernel(ConvFilterResidentArgs g) {
     using M = dh_gemm::Mfma16<T>;
     constexpr int VEC = 16 / sizeof(T), NPARTS = WAVES / MFW, NT = 64 * WAVES;
@@ -942,8 +946,10 @@ __global__ __launch_bounds__(64 * WAVES) void conv_filter_resident_kernel(ConvFi
     T *frame = reinterpret_cast<T *>(conv_lds + g.PQpad * sizeof(int));
     const int tid = threadIdx.x, lane = tid % 64, wave = __builtin_amdgcn_readfirstlane(tid / 64);
     const unsigned f0 = blockIdx.y * (16 * MFW), col0 = blockIdx.z * g.chunk;
+    // both tables as byte offsets into the LDS image: a gather's address is then one addition (every ordinary vector
+    // instruction issued beside the matrix instructions takes a pass out of the matrix pipe)
     for (unsigned i = tid; i < g.PQpad; i += NT)
-        pixtab[i] = g.pixtab[i];
+        pixtab[i] = g.pixtab[i] * static_cast<int>(sizeof(T));
 
     const int mf = wave % MFW, part = wave / MFW;
     const int li = lane % 16, lk = lane / 16;
@@ -953,7 +959,7 @@ __global__ __launch_bounds__(64 * WAVES) void conv_filter_resident_kernel(ConvFi
 #pragma unroll
     for (int j = 0; j < NF; j++) {
         const unsigned first = col0 + (j * NPARTS + part) * 16;
-        koffs[j] = g.koff[first + li];
+        koffs[j] = g.koff[first + li] * static_cast<int>(sizeof(T));
         if (first < g.K)
             nfv = j + 1;
     }
@@ -966,12 +972,33 @@ __global__ __launch_bounds__(64 * WAVES) void conv_filter_resident_kernel(ConvFi
     const bool rowok = frow < g.F;
     const T *dy = static_cast<const T *>(g.dy);
     const int *pixl = pixtab + lk * VEC;
-
-    for (unsigned img = blockIdx.x; img < g.N; img += gridDim.x) {
-        __syncthreads(); // every wave is done with the previous image
-        dh_dnn::conv_stage_frame<T, 32>(frame, static_cast<const T *>(g.x) + static_cast<size_t>(img) * g.C * g.H * g.W, g.C, g.H, g.W,
+    const char *frame_b = reinterpret_cast<const char *>(frame);
+    // DB: this thread's position in the padded plane (planes of at most NT positions), where it lies in the image
+    // (position 0 for the border, which is stored as zero), and the channels a pixel block brings in
+    const unsigned HW = g.H * g.W;
+    const unsigned sy = static_cast<unsigned>(tid) / g.Wp - g.ph, sxx = static_cast<unsigned>(tid) % g.Wp - g.pw; // wrap inside the border
+    const bool s_plane = static_cast<unsigned>(tid) < g.HpWp, s_in = s_plane && sy < g.H && sxx < g.W;
+    const unsigned s_src = s_in ? sy * g.W + sxx : 0;
+    const unsigned cpi = (g.C + g.PQpad / (4 * VEC) - 1) / (g.PQpad / (4 * VEC));
+    unsigned cur = 0;
+    if constexpr (DB) {
+        dh_dnn::conv_stage_frame<T, 32>(frame, static_cast<const T *>(g.x) + static_cast<size_t>(blockIdx.x) * g.C * HW, g.C, g.H, g.W,
                                     g.Wp, g.ph, g.pw, g.HpWp, g.frame, tid, NT);
         __syncthreads();
+    }
+
+    for (unsigned img = blockIdx.x; img < g.N; img += gridDim.x) {
+        if constexpr (!DB) {
+            __syncthreads(); // every wave is done with the previous image
+            dh_dnn::conv_stage_frame<T, 32>(frame, static_cast<const T *>(g.x) + static_cast<size_t>(img) * g.C * HW, g.C, g.H, g.W,
+                                        g.Wp, g.ph, g.pw, g.HpWp, g.frame, tid, NT);
+            __syncthreads();
+        }
+        // DB: the frame being contracted, the frame being filled, and the image that fills it (the last image of
+        // the workgroup brings itself in again; nobody reads that copy)
+        const char *fb = DB ? frame_b + static_cast<size_t>(cur) * g.frame * sizeof(T) : frame_b;
+        T *fill = frame + static_cast<size_t>(cur ^ 1u) * g.frame;
+        const T *xnext = static_cast<const T *>(g.x) + static_cast<size_t>(img + gridDim.x < g.N ? img + gridDim.x : img) * g.C * HW;
         const T *arow = dy + (static_cast<size_t>(img) * g.F + (rowok ? frow : 0)) * g.PQ + lk * VEC;
         // dY values of pixel block q0 for this lane; lanes past the row end (or past F) read the tensor's first
         // vector instead and are zeroed when the values are taken into use
@@ -979,7 +1006,10 @@ __global__ __launch_bounds__(64 * WAVES) void conv_filter_resident_kernel(ConvFi
         auto contract = [&](auto nv_tag) {
             constexpr int NV = decltype(nv_tag)::value;
             // dY comes from HBM: its vectors are asked for two pixel blocks ahead
-            T a_cur[VEC], a_nxt[VEC], b_cur[NV];
+            // the patch values alternate between two register sets from step to step (an even number of steps per
+            // pixel block), so that none is copied
+            static_assert(VEC % 2 == 0, "the two sets of patch registers alternate from step to step");
+            T a_cur[VEC], a_nxt[VEC], b_even[NV], b_odd[NV];
             int pt[VEC];
             const unsigned q1 = (4 * VEC < g.PQpad) ? 4 * VEC : 0;
             bool ok_nxt = a_ok(q1);
@@ -996,8 +1026,17 @@ __global__ __launch_bounds__(64 * WAVES) void conv_filter_resident_kernel(ConvFi
                 pt[s_] = pixl[s_];
 #pragma unroll
             for (int j = 0; j < NV; j++)
-                b_cur[j] = frame[koffs[j] + pt[0]];
+                b_even[j] = *reinterpret_cast<const T *>(fb + (koffs[j] + pt[0]));
+            unsigned c_lo = 0; // DB: first channel this pixel block brings in
             for (unsigned q0 = 0; q0 < g.PQpad; q0 += 4 * VEC) {
+                T sv[CONV_FILTER_STAGE_CH];
+                if constexpr (DB) {
+#pragma unroll
+                    for (int u = 0; u < CONV_FILTER_STAGE_CH; u++) {
+                        const unsigned c = c_lo + u;
+                        sv[u] = xnext[s_src + (c < g.C ? c : 0) * HW];
+                    }
+                }
                 const unsigned qn = (q0 + 4 * VEC < g.PQpad) ? q0 + 4 * VEC : q0;
                 const unsigned qnn = (q0 + 8 * VEC < g.PQpad) ? q0 + 8 * VEC : q0;
                 const bool ok_nn = a_ok(qnn);
@@ -1010,18 +1049,25 @@ __global__ __launch_bounds__(64 * WAVES) void conv_filter_resident_kernel(ConvFi
 #pragma unroll
                 for (int s_ = 0; s_ < VEC; s_++) {
                     const int pt_after = (s_ + 1 < VEC) ? pt[s_ + 1] : pt_nxt[0];
-                    T b_nxt[NV];
+                    __builtin_amdgcn_sched_barrier(0); // a gather must not sink to its use in the next step
+                    if (s_ % 2 == 0) {
 #pragma unroll
-                    for (int j = 0; j < NV; j++)
-                        b_nxt[j] = frame[koffs[j] + pt_after];
+                        for (int j = 0; j < NV; j++)
+                            b_odd[j] = *reinterpret_cast<const T *>(fb + (koffs[j] + pt_after));
+                        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                        for (int j = 0; j < NV; j++)
+                            acc[j] = M::mma(a_cur[s_], b_even[j], acc[j]);
+                    } else {
+#pragma unroll
+                        for (int j = 0; j < NV; j++)
+                            b_even[j] = *reinterpret_cast<const T *>(fb + (koffs[j] + pt_after));
+                        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                        for (int j = 0; j < NV; j++)
+                            acc[j] = M::mma(a_cur[s_], b_odd[j], acc[j]);
+                    }
                     __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                    for (int j = 0; j < NV; j++)
-                        acc[j] = M::mma(a_cur[s_], b_cur[j], acc[j]);
-                    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                    for (int j = 0; j < NV; j++)
-                        b_cur[j] = b_nxt[j];
                 }
 #pragma unroll
                 for (int s_ = 0; s_ < VEC; s_++) {
@@ -1030,12 +1076,31 @@ __global__ __launch_bounds__(64 * WAVES) void conv_filter_resident_kernel(ConvFi
                     pt[s_] = pt_nxt[s_];
                 }
                 ok_nxt = ok_nn;
+                if constexpr (DB) {
+#pragma unroll
+                    for (int u = 0; u < CONV_FILTER_STAGE_CH; u++) {
+                        const unsigned c = c_lo + u;
+                        if (s_plane && static_cast<unsigned>(u) < cpi && c < g.C)
+                            fill[c * g.HpWp + tid] = s_in ? sv[u] : T(0);
+                    }
+                    c_lo += cpi;
+                }
             }
         };
         if (nfv == NF - 1)
             contract(std::integral_constant<int, NF - 1>{});
         else if (nfv > 0)
             contract(std::integral_constant<int, NF>{});
+        if constexpr (DB) {
+            // a wave without column blocks (nfv == 0) has to bring in its share of the next image all the same
+            if (nfv == 0) {
+                for (unsigned c = 0; c < g.C; c++)
+                    if (s_plane)
+                        fill[c * g.HpWp + tid] = s_in ? xnext[s_src + c * HW] : T(0);
+            }
+            __syncthreads(); // the next image is in place, and every wave is done with this one
+            cur ^= 1u;
+        }
     }
 
     T *slab = static_cast<T *>(g.slabs) + static_cast<size_t>(blockIdx.x) * g.F * g.K;
@@ -1069,14 +1134,14 @@ template <typename T> __global__ __launch_bounds__(THREADS) void slab_sum_kernel
     res[i] = sum;
 }
 
-template <typename T, int MFW, int WAVES, int NF>
+template <typename T, int MFW, int WAVES, int NF, bool DB>
 static inline dh_status conv_filter_resident_launch(dh_ctx *ctx, const ConvFilterResidentArgs &g, dim3 grid, size_t lds) {
     // dynamic LDS beyond 64 KiB has to be asked for, per kernel and device (the call is cheap next to the kernel)
     if (lds > 65536) {
-        DH_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&conv_filter_resident_kernel<T, MFW, WAVES, NF>),
+        DH_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&conv_filter_resident_kernel<T, MFW, WAVES, NF, DB>),
                                          hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
     }
-    hipLaunchKernelGGL((conv_filter_resident_kernel<T, MFW, WAVES, NF>), grid, dim3(64 * WAVES), lds, ctx->stream, g);
+    hipLaunchKernelGGL((conv_filter_resident_kernel<T, MFW, WAVES, NF, DB>), grid, dim3(64 * WAVES), lds, ctx->stream, g);
     DH_CHECK_LAUNCH();
     return DH_OK;
 }
@@ -1087,7 +1152,7 @@ template <typename T> static bool conv_backward_filter_resident(dh_ctx *ctx, T *
     const size_t PQ = static_cast<size_t>(g.P) * g.Q, K = static_cast<size_t>(g.C) * g.Hf * g.Wf;
     const size_t Hp = g.H + 2 * g.padh, Wp = g.W + 2 * g.padw, frame = g.C * Hp * Wp;
     const size_t PQpad = dh_ceil_div(PQ, static_cast<size_t>(4 * VEC)) * (4 * VEC);
-    const size_t lds = PQpad * sizeof(int) + frame * sizeof(T);
+    size_t lds = PQpad * sizeof(int) + frame * sizeof(T);
     const int mfw = g.F <= 16 ? 1 : (g.F <= 32 ? 2 : 4);
     const size_t waves = 8;
     const size_t parts = waves / mfw, fgroups = dh_ceil_div(static_cast<size_t>(g.F), static_cast<size_t>(16 * mfw));
@@ -1100,6 +1165,13 @@ template <typename T> static bool conv_backward_filter_resident(dh_ctx *ctx, T *
         return false;
     // up to 7 column blocks per wave take few enough registers for two workgroups per CU, LDS permitting
     const size_t per_cu = (nf <= 7 && lds <= 80 * 1024) ? 2 : 1;
+    // A workgroup alone on its CU has nothing to cover the copy-in of an image with: it brings the next image in
+    // beside the contraction, where a plane has no more positions than the workgroup has threads, a pixel block's
+    // share of the channels is small, and two images fit LDS.
+    const bool db = per_cu == 1 && Hp * Wp <= waves * 64 && dh_ceil_div(static_cast<size_t>(g.C), PQpad / (4 * VEC)) <= CONV_FILTER_STAGE_CH &&
+                    PQpad * sizeof(int) + 2 * frame * sizeof(T) <= 150 * 1024;
+    if (db)
+        lds = PQpad * sizeof(int) + 2 * frame * sizeof(T);
     size_t groups = static_cast<size_t>(ctx->num_cus) * per_cu / (fgroups * chunks);
     if (groups < 1)
         groups = 1;
@@ -1141,9 +1213,11 @@ template <typename T> static bool conv_backward_filter_resident(dh_ctx *ctx, T *
     r.chunk = static_cast<unsigned>(chunk);
     const dim3 grid(static_cast<unsigned>(groups), static_cast<unsigned>(fgroups), static_cast<unsigned>(chunks));
 #define DH_CONV_FILTER_NF(MFW_, WAVES_)                                                                                   \
-    (nf <= 7 ? conv_filter_resident_launch<T, MFW_, WAVES_, 7>(ctx, r, grid, lds)                                         \
-             : (nf <= 10 ? conv_filter_resident_launch<T, MFW_, WAVES_, 10>(ctx, r, grid, lds)                            \
-                         : conv_filter_resident_launch<T, MFW_, WAVES_, 13>(ctx, r, grid, lds)))
+    (nf <= 7 ? conv_filter_resident_launch<T, MFW_, WAVES_, 7, false>(ctx, r, grid, lds)                                  \
+             : (nf <= 10 ? (db ? conv_filter_resident_launch<T, MFW_, WAVES_, 10, true>(ctx, r, grid, lds)                \
+                               : conv_filter_resident_launch<T, MFW_, WAVES_, 10, false>(ctx, r, grid, lds))              \
+                         : (db ? conv_filter_resident_launch<T, MFW_, WAVES_, 13, true>(ctx, r, grid, lds)                \
+                               : conv_filter_resident_launch<T, MFW_, WAVES_, 13, false>(ctx, r, grid, lds))))
 #define DH_CONV_FILTER_RES(MFW_) DH_CONV_FILTER_NF(MFW_, 8)
     *st = mfw == 1 ? DH_CONV_FILTER_RES(1) : (mfw == 2 ? DH_CONV_FILTER_RES(2) : DH_CONV_FILTER_RES(4));
 #undef DH_CONV_FILTER_RES

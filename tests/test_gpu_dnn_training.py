@@ -105,7 +105,10 @@ def test_pooling_backward_all_negative_window_goes_to_the_padding(ctx):
                                   # 20 filters (two filter blocks, 4 column parts); 70 filters (two groups) with stride 2;
                                   # 8 filters (one filter block, 8 column parts)
                                   (24, 32, 14, 14, 64, 5, 5, 1, 1, 2, 2), (32, 16, 12, 12, 20, 3, 3, 1, 1, 1, 1),
-                                  (20, 24, 31, 31, 70, 3, 3, 2, 2, 1, 1), (17, 48, 16, 16, 8, 3, 3, 1, 1, 1, 1)])
+                                  (20, 24, 31, 31, 70, 3, 3, 2, 2, 1, 1), (17, 48, 16, 16, 8, 3, 3, 1, 1, 1, 1),
+                                  # more images than workgroups: the next image is brought into the second LDS frame
+                                  # beside the contraction (two channels per pixel block), some workgroups take two images
+                                  (300, 10, 12, 12, 64, 5, 5, 1, 1, 2, 2)])
 def test_conv_backward(ctx, dt, case):
     N, C, H, W, F, Hf, Wf, sh, sw, ph, pw = case
     rng = np.random.default_rng(sum(case))
