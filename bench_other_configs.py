@@ -255,9 +255,9 @@ def run(args) -> int:
                    "sample": f"one iteration on all {n} rows, {threads} threads: products by numpy's {_blas_name()} sgemm, the other "
                              f"operators by the port's scalar kernels on row pieces ({dt:.2f} s)"}
         step_bytes = n * f * 4 + n * 4 + n * 8  # X, xx, idx
-        step_flops = 2 * 2.0 * n * f * k      # X t(C) and t(P) X
+        step_flops = 2.0 * n * f * k          # X t(C) on the matrix cores; the per-cluster sums are n * f additions on the ordinary ALUs
         roof = {"bound": "hbm", "kernel": "ts_nt_kernel<float,1,true,4,true> + kmeans_finish_kernel (one pass over X: X t(C), distances, "
-                                          "row arg-min, t(one-hot) X and sizes)",
+                                          "row arg-min, per-cluster sums and sizes)",
                 "achieved": round(step_bytes / t_step / 1e6, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(step_bytes / t_step / 1e6 / HBM_PEAK_GBS, 4), "traffic": None,
                 "mfma_tflops": round(step_flops / t_step / 1e9, 1)}
