@@ -107,12 +107,13 @@ dh_status dh_fail(dh_status st, const char *fmt, ...) __attribute__((format(prin
 // call and the 8 bytes at byte 64 are the result slot of AggAll):
 //   [0] kind (0: nothing pending)  [1] operator code  [2..3] a 64-bit value  [4..5] a 64-bit bound
 constexpr int DH_DEFERRED_AT = 32, DH_DEFERRED_INTS = 6;
-enum { DH_DEFERRED_NONE = 0, DH_DEFERRED_INT_DIVMOD = 1, DH_DEFERRED_UNARY_DOMAIN = 2, DH_DEFERRED_EXTRACT_COL = 3, DH_DEFERRED_PIPELINE_DOMAIN = 4 };
+enum { DH_DEFERRED_NONE = 0, DH_DEFERRED_INT_DIVMOD = 1, DH_DEFERRED_UNARY_DOMAIN = 2, DH_DEFERRED_EXTRACT_COL = 3, DH_DEFERRED_PIPELINE_DOMAIN = 4, DH_DEFERRED_SOLVE_SINGULAR = 5 };
 // The failures a checked call reports, immediately or from dh_check_deferred (context.hip).
 dh_status dh_fail_int_divmod(int op);
 dh_status dh_fail_unary_domain(int op);
 dh_status dh_fail_extract_col(long long position, size_t cols);
 dh_status dh_fail_pipeline_domain();
+dh_status dh_fail_solve_singular();
 // After the kernels of a checked call on a context that defers its verdicts: enqueues the kernel that keeps the
 // call's flag (at ctx->flag_dev, raised if != ok_value) in the deferred record. sel != nullptr: the flag is the
 // index + 1 of the offending entry of sel (stride ld_sel), whose value is kept along with `bound`.

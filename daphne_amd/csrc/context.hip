@@ -173,6 +173,11 @@ dh_status dh_fail_pipeline_domain() {
     return dh_fail(DH_ERR_DOMAIN, "invalid argument passed to a unary function inside the pipeline");
 }
 
+dh_status dh_fail_solve_singular() {
+    // Solve.h:113-115
+    return dh_fail(DH_ERR_RUNTIME, "A factor Ui is exactly singular, so the solution could not be computed");
+}
+
 // One thread: the record keeps the first failure of the stream's order.
 static __global__ void latch_deferred_kernel(const int *flag, int ok_value, int *rec, int kind, int op, const long long *sel,
                                              size_t ld_sel, long long bound) {
@@ -238,6 +243,8 @@ extern "C" dh_status dh_check_deferred(dh_ctx *ctx) {
         return dh_fail_extract_col(value, static_cast<size_t>(bound));
     case DH_DEFERRED_PIPELINE_DOMAIN:
         return dh_fail_pipeline_domain();
+    case DH_DEFERRED_SOLVE_SINGULAR:
+        return dh_fail_solve_singular();
     default:
         return dh_fail(DH_ERR_RUNTIME, "dh_check_deferred: unknown record kind %d", rec[0]);
     }

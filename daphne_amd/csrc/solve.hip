@@ -640,6 +640,10 @@ template <typename T> dh_status solve(dh_ctx *ctx, T *x, const T *A, size_t n, s
         return dh_fail(DH_ERR_RUNTIME, "#cols of lhs must match row skip");
     if (n >= (size_t(1) << 15))
         return dh_fail(DH_ERR_RUNTIME, "Solve: systems beyond 32767 unknowns are not supported by this kernel");
+    // where the verdict goes: the pinned host word that the wait below reads, or - with deferred verdicts - the
+    // context's flag on the device, which a one-thread kernel then keeps for dh_check_deferred
+    const bool deferred = ctx->deferred_depth > 0;
+    int *verdict = deferred ? ctx->flag_dev : ctx->flag_host_dev;
     const size_t lds_bytes = LdsSolveShape<T>(n).bytes;
     if (n <= 64 * LDS_SOLVE_MAX_SLOTS && lds_bytes <= (size_t(150) << 10)) {
         // Systems beyond 64 KB of LDS need the limit of the kernel raised, once per kernel instantiation and device
@@ -659,7 +663,7 @@ template <typename T> dh_status solve(dh_ctx *ctx, T *x, const T *A, size_t n, s
                 }
             }
             hipLaunchKernelGGL(kernel, dim3(1), dim3(LDS_SOLVE_THREADS), lds_bytes, ctx->stream, x, A, lda, b,
-                               static_cast<unsigned>(n), ctx->flag_host_dev);
+                               static_cast<unsigned>(n), verdict);
             return DH_OK;
         };
         dh_status lst;
@@ -672,20 +676,21 @@ template <typename T> dh_status solve(dh_ctx *ctx, T *x, const T *A, size_t n, s
         if (lst != DH_OK)
             return lst;
     } else {
-        hipLaunchKernelGGL(clear_flag_kernel, dim3(1), dim3(1), 0, ctx->stream, ctx->flag_host_dev);
+        hipLaunchKernelGGL(clear_flag_kernel, dim3(1), dim3(1), 0, ctx->stream, verdict);
         void *wsv = nullptr;
         dh_status st = dh_workspace(ctx, n * n * sizeof(T), &wsv);
         if (st != DH_OK)
             return st;
         hipLaunchKernelGGL((lu_solve_kernel<T>), dim3(1), dim3(SOLVE_THREADS), 0, ctx->stream, static_cast<T *>(wsv), x,
-                           A, lda, b, static_cast<unsigned>(n), ctx->flag_host_dev);
+                           A, lda, b, static_cast<unsigned>(n), verdict);
     }
     DH_CHECK_LAUNCH();
+    if (deferred)
+        return dh_latch_deferred(ctx, 0, DH_DEFERRED_SOLVE_SINGULAR, 0, nullptr, 0, 0);
     // the kernels write the flag into the pinned host word itself: no copy back, only the wait
     DH_CHECK_HIP(hipStreamSynchronize(ctx->stream));
     if (*static_cast<volatile int *>(ctx->flag_host) != 0)
-        // Solve.h:113-115
-        return dh_fail(DH_ERR_RUNTIME, "A factor Ui is exactly singular, so the solution could not be computed");
+        return dh_fail_solve_singular();
     return DH_OK;
 }
 

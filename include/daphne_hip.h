@@ -106,7 +106,8 @@ void *dh_ctx_get_stream(const dh_ctx *ctx);
 dh_status dh_sync(dh_ctx *ctx);
 /* Deferred verdicts. Some kernels can only tell on the device whether their arguments were valid: integer DIV and MOD
  * (a zero divisor, EwBinarySca.h:114-127 through the host's arithmetic), SQRT / LN / ASIN / ACOS (EwUnarySca.h:130-170),
- * the column positions of ExtractCol (ExtractCol.h:98-108) and checked unary functions inside a fused pipeline body.
+ * the column positions of ExtractCol (ExtractCol.h:98-108), checked unary functions inside a fused pipeline body, and
+ * the singular factor of Solve (Solve.h:113-115).
  * By default such a call waits for its kernels and returns the failure itself, as the CPU kernel throws. A caller that
  * runs many of them back to back - the task of a vectorized pipeline walking its batches,
  * vectorized/TasksCUDA.cpp:61-100 has no counterpart because the CUDA kernels do not check - enters deferred mode:

@@ -228,6 +228,31 @@ def test_solve_errors(ctx, dt):
 
 
 @pytest.mark.parametrize("dt", DTYPES)
+def test_solve_with_deferred_verdicts(ctx, dt):
+    """Inside a deferred block solves do not wait for their verdict: good systems give the bits of the direct call,
+    and a singular one among them is reported when the block ends, with the direct call's error."""
+    rng = np.random.default_rng(5)
+    systems = []
+    for n in (3, 100, 150):  # LDS-resident (one and two rows a lane) and the global-memory kernel's sizes
+        A = rng.random((n, n)).astype(dt) + np.eye(n, dtype=dt) * dt(n)
+        b = rng.random((n, 1)).astype(dt)
+        systems.append((DenseMatrix.from_numpy(ctx, A), DenseMatrix.from_numpy(ctx, b)))
+    direct = [solve(None, A, b, ctx).to_numpy() for A, b in systems]
+    with ctx.deferred_checks():
+        inside = [solve(None, A, b, ctx) for A, b in systems]
+    for d, i in zip(direct, inside):
+        assert np.array_equal(d, i.to_numpy())
+    Z = DenseMatrix.from_numpy(ctx, np.zeros((3, 3), dt))
+    with pytest.raises(capi.DaphneHipError, match="exactly singular"):
+        with ctx.deferred_checks():
+            solve(None, *systems[1], ctx)
+            solve(None, Z, systems[0][1], ctx)
+            solve(None, *systems[0], ctx)  # a good one after the failure does not clear it
+    ctx.check_deferred()  # reported once
+    assert np.array_equal(solve(None, *systems[1], ctx).to_numpy(), direct[1])
+
+
+@pytest.mark.parametrize("dt", DTYPES)
 @pytest.mark.parametrize("m,k,n", [(1, 9, 2), (64, 100, 10), (300, 3136, 512), (257, 512, 10)])
 def test_affine(ctx, dt, m, k, n):
     """Affine = MatMul then row-vector add (the reference has no CPU affine kernel)."""
