@@ -10,8 +10,9 @@
 // What is a chain is not decided here: every block is written down as a HIP::ChainGraph - mnemonics, value numbers,
 // the constants and shapes that are known - and handed to HIP::OperatorChainMatcher
 // (src/runtime/local/kernels/HIP/OperatorChainMatcher.h), which is plain C++ and tested with the kernel layer. This
-// file only translates: operations marked `hip_device` in, daphne.conv2DForwardFused / affineForwardFused /
-// normalEquations / kmeansAssign out. The new operations carry `hip_device` too, so RewriteToCallKernelOpPass finds
+// file only translates: operations marked `hip_device` in (and, as links of a k-means iteration only, the one-hot
+// encoding of the labels and a cast in front of it, which have no device kernels of their own), daphne.conv2DForwardFused /
+// affineForwardFused / normalEquations / kmeansAssign / kmeansStep out. The new operations carry `hip_device` too, so RewriteToCallKernelOpPass finds
 // their kernels in HIPcatalog.json by mnemonic like any other (HIP_conv2DForwardFused__..., kernels/HIP/FusedOperators.h).
 #ifdef USE_HIP
 #include "ir/daphneir/Daphne.h"
@@ -79,8 +80,8 @@ struct FuseHIPOperatorChainsPass : public PassWrapper<FuseHIPOperatorChainsPass,
                 g.constants[number(op.getResult(0))] = c;
             for (Value r : op.getResults())
                 noteShape(r);
-            const bool isChainOp = llvm::isa<daphne::DaphneDialect>(op.getDialect()) && op.hasAttr(ATTR_HIP_DEVICE) &&
-                                   op.getNumRegions() == 0;
+            const bool isChainOp = llvm::isa<daphne::DaphneDialect>(op.getDialect()) && op.getNumRegions() == 0 &&
+                                   (op.hasAttr(ATTR_HIP_DEVICE) || llvm::isa<daphne::OneHotOp, daphne::CastOp>(op));
             if (isChainOp) {
                 HIP::ChainOp co;
                 co.mnemonic = op.getName().stripDialect().str();
@@ -139,6 +140,9 @@ struct FuseHIPOperatorChainsPass : public PassWrapper<FuseHIPOperatorChainsPass,
         }
         case HIP::ChainKind::KMEANS_ASSIGN:
             fused = builder.create<daphne::KmeansAssignOp>(loc, resultTypes, ValueRange{arg("X"), arg("C"), arg("xx"), arg("cc")});
+            break;
+        case HIP::ChainKind::KMEANS_STEP: // results: the labels, the new centroids, the cluster sizes (the column sums of the encoding)
+            fused = builder.create<daphne::KmeansStepOp>(loc, resultTypes, ValueRange{arg("X"), arg("C"), arg("xx"), arg("cc")});
             break;
         }
         fused->setAttr(ATTR_HIP_DEVICE, builder.getI32IntegerAttr(0));

@@ -16,6 +16,9 @@
 //                      (scripts/algorithms/lmDS_.daph:100-101 after the t(X) @ X -> syrk rewrite)
 //   KMEANS_ASSIGN      idxminRow of (matMul(X, t(C)) * -2 + xx) + cc, written with ewMul / ewAdd / ewSub in any of the
 //                      forms that round the same way (x * -2 + a, a - x * 2, operands of ewAdd / ewMul in either order)
+//   KMEANS_STEP        KMEANS_ASSIGN whose labels go on (possibly through a cast) into oneHot(idx, info) -> P,
+//                      matMul(t(P), X) / t(sumCol(P)) over the same X: a whole Lloyd iteration, labels and new centroids from
+//                      one pass over X. The labels may have other users (the kernel returns them); P may not.
 // An intermediate value must have no other user, or the chain's kernel could not leave it out.
 #pragma once
 
@@ -39,7 +42,7 @@ struct ChainGraph {
     std::vector<int> escaping;                     // values used outside the described operators (returned, stored, ...)
 };
 
-enum class ChainKind { CONV_RELU_POOL, AFFINE_RELU, NORMAL_EQUATIONS, KMEANS_ASSIGN };
+enum class ChainKind { CONV_RELU_POOL, AFFINE_RELU, NORMAL_EQUATIONS, KMEANS_ASSIGN, KMEANS_STEP };
 
 struct ChainMatch {
     ChainKind kind;
@@ -287,6 +290,77 @@ class OperatorChainMatcher {
         return false;
     }
 
+    // m: a KMEANS_ASSIGN match. If the labels are one-hot encoded and the encoding is only used for the cluster means
+    // of the same X - oneHot(idx, info) -> P, matMul(t(P), X) -> S, sumCol(P) -> n, S / t(n) - the match becomes
+    // KMEANS_STEP with the results (idx, C_new, n). The labels come from an arg-min over C's rows, so they are valid
+    // positions of the encoding whenever P is as wide as C has rows - which the shapes must show.
+    bool extendToKmeansStep(ChainMatch &m) const {
+        const int idx = m.results[0], X = m.args.at("X"), C = m.args.at("C");
+        auto iu = users.find(idx);
+        if (iu == users.end() || colsOf(idx) != 1)
+            return false;
+        for (size_t u : iu->second) {
+            std::vector<size_t> chain;
+            size_t oh = u;
+            int labels = idx;
+            size_t next;
+            if (!taken[u] && isOp(u, "cast", 1) && g.ops[u].results.size() == 1 && soleUser(g.ops[u].results[0], next)) {
+                chain.push_back(u);
+                labels = g.ops[u].results[0];
+                oh = next;
+            }
+            if (taken[oh] || !isOp(oh, "oneHot", 2) || g.ops[oh].operands[0] != labels || g.ops[oh].results.size() != 1)
+                continue;
+            const int P = g.ops[oh].results[0];
+            auto pu = users.find(P);
+            if (escapes(P) || pu == users.end() || pu->second.size() != 2 || colsOf(P) < 1 || colsOf(P) != rowsOf(C))
+                continue;
+            bool haveMm = false, haveSc = false;
+            size_t mm = 0, sc = 0;
+            std::vector<size_t> extra;
+            for (size_t q : pu->second) {
+                if (taken[q])
+                    continue;
+                const ChainOp &o = g.ops[q];
+                if (isOp(q, "sumCol", 1) && o.results.size() == 1) {
+                    sc = q;
+                    haveSc = true;
+                } else if (isOp(q, "matMul", 4) && o.results.size() == 1 && o.operands[0] == P && o.operands[1] == X &&
+                           constantIs(o.operands[2], 1) && constantIs(o.operands[3], 0)) {
+                    mm = q;
+                    haveMm = true;
+                } else if (isOp(q, "transpose", 1) && o.results.size() == 1 && soleUser(o.results[0], next) && isOp(next, "matMul", 4) &&
+                           g.ops[next].results.size() == 1 && g.ops[next].operands[0] == o.results[0] && g.ops[next].operands[1] == X &&
+                           constantIs(g.ops[next].operands[2], 0) && constantIs(g.ops[next].operands[3], 0)) {
+                    mm = next;
+                    haveMm = true;
+                    extra.push_back(q);
+                }
+            }
+            if (!haveMm || !haveSc)
+                continue;
+            const int S = g.ops[mm].results[0], n = g.ops[sc].results[0];
+            size_t tn, dv, only;
+            if (!soleUser(n, tn) || !isOp(tn, "transpose", 1) || g.ops[tn].results.size() != 1)
+                continue;
+            const int nT = g.ops[tn].results[0];
+            if (!soleUser(nT, dv) || !isOp(dv, "ewDiv", 2) || g.ops[dv].results.size() != 1 || g.ops[dv].operands[0] != S ||
+                g.ops[dv].operands[1] != nT || !soleUser(S, only) || only != dv)
+                continue;
+            m.kind = ChainKind::KMEANS_STEP;
+            for (size_t o : chain)
+                m.ops.push_back(o);
+            for (size_t o : {oh, sc, mm, tn, dv})
+                m.ops.push_back(o);
+            for (size_t o : extra)
+                m.ops.push_back(o);
+            m.results = {idx, g.ops[dv].results[0], n};
+            sortOps(m);
+            return true;
+        }
+        return false;
+    }
+
   public:
     // Every chain found, each operator in at most one of them.
     static std::vector<ChainMatch> match(const ChainGraph &graph) {
@@ -297,6 +371,8 @@ class OperatorChainMatcher {
                 continue;
             ChainMatch m;
             if (self.matchConv(i, m) || self.matchAffine(i, m) || self.matchNormalEquations(i, m) || self.matchKmeansAssign(i, m)) {
+                if (m.kind == ChainKind::KMEANS_ASSIGN)
+                    self.extendToKmeansStep(m);
                 self.take(m);
                 found.push_back(m);
             }

@@ -108,6 +108,48 @@ static void run_chain_matcher() {
     ChainGraph k4 = k; // the distances are printed as well: they have to exist
     k4.escaping.push_back(14);
     CHECK(OperatorChainMatcher::match(k4).empty());
+
+    // the whole Lloyd iteration: P = oneHot(idx, [16]); C' = (t(P) @ X) / t(sum(P, 1)) - labels and centroids from one pass
+    ChainGraph s = k;
+    s.ops.push_back({"cast", {15}, {16}});
+    s.ops.push_back({"oneHot", {16, 8}, {17}});
+    s.ops.push_back({"matMul", {17, 1, 9, 5}, {18}}); // transa = 1 (value 9), transb = 0 (value 5)
+    s.ops.push_back({"sumCol", {17}, {19}});
+    s.ops.push_back({"transpose", {19}, {20}});
+    s.ops.push_back({"ewDiv", {18, 20}, {21}});
+    s.constants[9] = 1;
+    s.shapes[15] = {2000000, 1};
+    s.shapes[16] = {2000000, 1};
+    s.shapes[17] = {2000000, 16};
+    s.escaping = {21};
+    found = OperatorChainMatcher::match(s);
+    CHECK(found.size() == 1 && found[0].kind == ChainKind::KMEANS_STEP && found[0].ops.size() == 12 &&
+          found[0].results == (std::vector<int>{15, 21, 19}) && found[0].args.at("X") == 1 && found[0].args.at("C") == 2);
+    ChainGraph s2 = s; // the labels are returned as well: still one kernel, it makes them anyway
+    s2.escaping.push_back(15);
+    found = OperatorChainMatcher::match(s2);
+    CHECK(found.size() == 1 && found[0].kind == ChainKind::KMEANS_STEP);
+    ChainGraph s3 = s; // t(P) written out
+    s3.ops[8] = {"transpose", {17}, {22}};
+    s3.ops.insert(s3.ops.begin() + 9, {"matMul", {22, 1, 5, 5}, {18}});
+    found = OperatorChainMatcher::match(s3);
+    CHECK(found.size() == 1 && found[0].kind == ChainKind::KMEANS_STEP && found[0].ops.size() == 13);
+    ChainGraph s4 = s; // the means of another matrix: the assignment alone is fused
+    s4.ops[8] = {"matMul", {17, 30, 9, 5}, {18}};
+    found = OperatorChainMatcher::match(s4);
+    CHECK(found.size() == 1 && found[0].kind == ChainKind::KMEANS_ASSIGN && found[0].results == (std::vector<int>{15}));
+    ChainGraph s5 = s; // the encoding is printed: it has to exist
+    s5.escaping.push_back(17);
+    found = OperatorChainMatcher::match(s5);
+    CHECK(found.size() == 1 && found[0].kind == ChainKind::KMEANS_ASSIGN);
+    ChainGraph s6 = s; // an encoding wider than C has rows is not an encoding of these labels
+    s6.shapes[17] = {2000000, 20};
+    found = OperatorChainMatcher::match(s6);
+    CHECK(found.size() == 1 && found[0].kind == ChainKind::KMEANS_ASSIGN);
+    ChainGraph s7 = s; // the sums divided by something else than their counts
+    s7.ops[11] = {"ewDiv", {18, 31}, {21}};
+    found = OperatorChainMatcher::match(s7);
+    CHECK(found.size() == 1 && found[0].kind == ChainKind::KMEANS_ASSIGN);
 }
 
 int main() {
