@@ -397,7 +397,7 @@ struct TsNtArgs {
 // ASSIGN: the product is not stored; it goes on, rounded exactly as the stored one would be, into the distance
 // (C * -2 + row_add[row]) + col_add[col] (three separately rounded operations) and the row's IDXMIN over it: the first
 // position of the strict minimum, NaN never better, position 0 if the first value is NaN or all are.
-// UPDATE (with ASSIGN; float, one step per pair of row blocks with four chunks, i.e. 49..64 columns): the rows, read
+// UPDATE (with ASSIGN; float, one step per pair of row blocks, i.e. K of exactly CPG chunks: up to 16, 32 or 64 columns): the rows, read
 // back from the wave's staging piece one at a time - lane j on column j -, are added to the sum of the position just
 // found for them. A lane keeps its column's 16 NB sums in registers, and the position, the same for all lanes, picks
 // the register (register-relative moves): four ordinary instructions and an LDS read per row, where the one-hot
@@ -407,7 +407,7 @@ struct TsNtArgs {
 // pairs round-robin.
 template <typename T, int NB, bool ASSIGN, int CPG, bool UPDATE = false>
 __global__ __launch_bounds__(256, UPDATE ? (NB == 1 ? 3 : 2) : 1) void ts_nt_kernel(TsNtArgs g) {
-    static_assert(!UPDATE || (ASSIGN && sizeof(T) == 4 && CPG == 4), "the one-pass form exists for float and 49..64 columns");
+    static_assert(!UPDATE || (ASSIGN && sizeof(T) == 4), "the one-pass form exists for float, K of CPG whole chunks (a lane per column)");
     using M = Mfma16<T>;
     constexpr int V = 16 / sizeof(T);
     constexpr int KC = 4 * V;     // k values per chunk
@@ -645,7 +645,9 @@ __global__ __launch_bounds__(256, UPDATE ? (NB == 1 ? 3 : 2) : 1) void ts_nt_ker
 #pragma unroll
                             for (int r = 0; r < 16; r++) {
                                 const unsigned pos = static_cast<unsigned>(__builtin_amdgcn_readlane(static_cast<int>(bi[t]), r));
-                                T x = stage[(t * 16 + r) * SX + lane]; // the row as a row: lane j on column j
+                                // the row as a row: lane j on column j (lanes beyond the step's columns repeat column 0;
+                                // their sums are never stored)
+                                T x = stage[(t * 16 + r) * SX + (lane < static_cast<int>(CPG * KC) ? lane : 0)];
                                 if constexpr (!WHOLE)
                                     x = rbase + t * 16 + r < g.M ? x : T(0); // rows beyond M repeat the last row
                                 sums[pos] += x;
@@ -816,8 +818,8 @@ __global__ __launch_bounds__(256, UPDATE ? (NB == 1 ? 3 : 2) : 1) void ts_nt_ker
     }
     if constexpr (UPDATE) {
         // the workgroup's partial result: the four waves' sums and counts, added in wave order
-        static_assert(4 * NPOS * 64 <= 4 * 2 * 16 * (4 * 4 * V + V), "the exchange area must fit the staging pieces");
         __syncthreads(); // every wave is done with its staging piece: the exchange between the waves takes their place
+                         // (the launch sizes the dynamic LDS for the larger of the two)
         T *red = lb + NB * 16 * ldl; // [wave][position][column]
 #pragma unroll
         for (unsigned p = 0; p < NPOS; p++)
@@ -948,10 +950,12 @@ template <typename T> inline size_t ts_nt_lds_bytes(int nb, unsigned kpad, int c
     constexpr size_t V = 16 / sizeof(T), KC = 4 * V;
     return (static_cast<size_t>(nb) * 16 * (kpad + V) + 4 * 16 * (cpg * KC + V)) * sizeof(T);
 }
-// ... of the one-pass form: the staging piece holds both row blocks of a pair
-template <typename T> inline size_t ts_nt_update_lds_bytes(int nb, unsigned kpad) {
+// ... of the one-pass form: the staging piece holds both row blocks of a pair, and at the end the waves exchange their
+// sums (16 nb positions x 64 lanes each) through the same area
+template <typename T> inline size_t ts_nt_update_lds_bytes(int nb, unsigned kpad, int cpg) {
     constexpr size_t V = 16 / sizeof(T), KC = 4 * V;
-    return (static_cast<size_t>(nb) * 16 * (kpad + V) + 4 * 2 * 16 * (4 * KC + V)) * sizeof(T);
+    const size_t stage = 4 * 2 * 16 * (static_cast<size_t>(cpg) * KC + V), exchange = 4 * static_cast<size_t>(nb) * 16 * 64;
+    return (static_cast<size_t>(nb) * 16 * (kpad + V) + (stage > exchange ? stage : exchange)) * sizeof(T);
 }
 // chunks of k per step: the largest of 4, 2, 1 that divides their number
 template <typename T> inline int ts_nt_chunks_per_step(unsigned kpad) {
@@ -974,9 +978,9 @@ inline dh_status ts_nt_launch_cpg(dh_ctx *ctx, const TsNtArgs &g, size_t lds) {
 // The one-pass form (UPDATE): a grid of as many workgroups as the device holds at once; *blocks_out receives their
 // number (that of the partial results in g.slabs, which must hold blocks * (16 NB K + 16 NB) values: ask with
 // g.slabs == nullptr first).
-template <typename T, int NB> inline dh_status ts_nt_update_launch(dh_ctx *ctx, const TsNtArgs &g, size_t *blocks_out) {
-    const void *kernel = reinterpret_cast<const void *>(&ts_nt_kernel<T, NB, true, 4, true>);
-    const size_t lds = ts_nt_update_lds_bytes<T>(NB, g.kpad);
+template <typename T, int NB, int CPG = 4> inline dh_status ts_nt_update_launch(dh_ctx *ctx, const TsNtArgs &g, size_t *blocks_out) {
+    const void *kernel = reinterpret_cast<const void *>(&ts_nt_kernel<T, NB, true, CPG, true>);
+    const size_t lds = ts_nt_update_lds_bytes<T>(NB, g.kpad, CPG);
     // three workgroups per CU (measured 2 .. 4 per CU: 104 .. 110 us at 2M x 64, no trend; a loop that only loads the
     // rows this way and stores the assignment takes 86 us, 74 us without the stores)
     (void)kernel;
@@ -988,7 +992,7 @@ template <typename T, int NB> inline dh_status ts_nt_update_launch(dh_ctx *ctx, 
     *blocks_out = blocks;
     if (g.slabs == nullptr)
         return DH_OK;
-    hipLaunchKernelGGL((ts_nt_kernel<T, NB, true, 4, true>), dim3(static_cast<unsigned>(blocks)), dim3(256), lds, ctx->stream, g);
+    hipLaunchKernelGGL((ts_nt_kernel<T, NB, true, CPG, true>), dim3(static_cast<unsigned>(blocks)), dim3(256), lds, ctx->stream, g);
     return DH_OK;
 }
 

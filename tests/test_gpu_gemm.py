@@ -477,7 +477,7 @@ def test_kmeans_assign_and_update(ctx, dt, rows, cols, k):
             kmeansUpdate(None, X, DenseMatrix.from_numpy(ctx, idx), k, ctx)
         return
     Cn, counts = kmeansUpdate(None, X, DenseMatrix.from_numpy(ctx, idx), k, ctx)
-    # both passes as one call (one pass over X for 49 to 64 float features): the same assignment and sizes bit for bit
+    # both passes as one call (one pass over X for up to 32 or 49 to 64 float features): the same assignment and sizes bit for bit
     idx1, Cn1, counts1 = kmeansStep(None, None, X, C, xx, cc, ctx)
     assert_exact(idx1.to_numpy(), idx)
     assert_exact(counts1.to_numpy(), counts.to_numpy())
