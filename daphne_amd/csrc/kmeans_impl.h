@@ -347,8 +347,7 @@ dh_status update(dh_ctx *ctx, T *Cn, size_t ldc, T *counts, const T *X, size_t r
     return DH_OK;
 }
 
-// assign and update in one pass over X where the one-pass kernel exists (float; up to 16, 17..32 or 49..64 features - K
-// padded to whole chunks of 16 must be 1, 2 or 4 of them -, 16-byte rows), else
+// assign and update in one pass over X where the one-pass kernel exists (float, up to 64 features, 16-byte rows), else
 // one after the other; idx, C_new and counts as those two give them (C_new to rounding: other order of addition)
 template <typename T>
 dh_status step(dh_ctx *ctx, unsigned long long *idx, T *Cn, size_t ldcn, T *counts, const T *X, size_t rows, size_t cols, size_t ldx,
@@ -359,7 +358,7 @@ dh_status step(dh_ctx *ctx, unsigned long long *idx, T *Cn, size_t ldcn, T *coun
     if constexpr (sizeof(T) == 4) {
         constexpr int V = 4, KC = 16;
         const size_t kpad = dh_ceil_div(cols, KC) * KC;
-        if (rows > 0 && k >= 1 && k <= 32 && (kpad == 16 || kpad == 32 || kpad == 64) && dh_aligned(X, 16) && dh_aligned(C, 16) && ldx % V == 0 && ldc % V == 0 &&
+        if (rows > 0 && k >= 1 && k <= 32 && kpad <= 64 && dh_aligned(X, 16) && dh_aligned(C, 16) && ldx % V == 0 && ldc % V == 0 &&
             cols % V == 0 && ldx >= cols && ldc >= cols && ldcn >= cols && ldx * sizeof(T) < (size_t(1) << 24)) {
             const int nb = k <= 16 ? 1 : 2;
             TsNtArgs g{};
@@ -379,6 +378,8 @@ dh_status step(dh_ctx *ctx, unsigned long long *idx, T *Cn, size_t ldcn, T *coun
             auto launch = [&]() -> dh_status {
                 if (kpad == 64)
                     return nb == 1 ? dh_gemm::ts_nt_update_launch<T, 1, 4>(ctx, g, &blocks) : dh_gemm::ts_nt_update_launch<T, 2, 4>(ctx, g, &blocks);
+                if (kpad == 48)
+                    return nb == 1 ? dh_gemm::ts_nt_update_launch<T, 1, 3>(ctx, g, &blocks) : dh_gemm::ts_nt_update_launch<T, 2, 3>(ctx, g, &blocks);
                 if (kpad == 32)
                     return nb == 1 ? dh_gemm::ts_nt_update_launch<T, 1, 2>(ctx, g, &blocks) : dh_gemm::ts_nt_update_launch<T, 2, 2>(ctx, g, &blocks);
                 return nb == 1 ? dh_gemm::ts_nt_update_launch<T, 1, 1>(ctx, g, &blocks) : dh_gemm::ts_nt_update_launch<T, 2, 1>(ctx, g, &blocks);

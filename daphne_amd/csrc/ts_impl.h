@@ -397,7 +397,7 @@ struct TsNtArgs {
 // ASSIGN: the product is not stored; it goes on, rounded exactly as the stored one would be, into the distance
 // (C * -2 + row_add[row]) + col_add[col] (three separately rounded operations) and the row's IDXMIN over it: the first
 // position of the strict minimum, NaN never better, position 0 if the first value is NaN or all are.
-// UPDATE (with ASSIGN; float, one step per pair of row blocks, i.e. K of exactly CPG chunks: up to 16, 32 or 64 columns): the rows, read
+// UPDATE (with ASSIGN; float, one step per pair of row blocks, i.e. K of exactly CPG chunks, CPG = 1 .. 4: up to 64 columns): the rows, read
 // back from the wave's staging piece one at a time - lane j on column j -, are added to the sum of the position just
 // found for them. A lane keeps its column's 16 NB sums in registers, and the position, the same for all lanes, picks
 // the register (register-relative moves): four ordinary instructions and an LDS read per row, where the one-hot
