@@ -67,6 +67,7 @@ def _signatures(lib: C.CDLL) -> None:
     lib.dh_d2h.argtypes = [ctxp, vp, vp, sz]
     lib.dh_d2d.argtypes = [ctxp, vp, vp, sz]
     lib.dh_d2d_2d.argtypes = [ctxp, vp, sz, vp, sz, sz, sz]
+    lib.dh_d2h_2d.argtypes = [ctxp, vp, sz, vp, sz, sz, sz]
     lib.dh_timer_start.argtypes = [ctxp]
     lib.dh_ctx_set_pipeline_mode.argtypes = [ctxp, i32]
     lib.dh_ctx_get_pipeline_mode.argtypes = [ctxp]

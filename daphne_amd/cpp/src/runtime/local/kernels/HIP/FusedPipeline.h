@@ -219,7 +219,11 @@ template <typename VT> struct FusedPipeline<DenseMatrix<VT>> {
         if (built && built->fits) {
             fusedPipelineLastMode() = 1;
             fusedPipelineLastReason().clear();
-            std::vector<std::function<PipelineFunc>> funcs{FusedPipelineBody<VT>(built->program)};
+            // {host body, device body} as the caller has them, with the one kernel in the place of the device body
+            std::vector<std::function<PipelineFunc>> funcs;
+            if (numFuncs > 1 && fun[0] != nullptr)
+                funcs.emplace_back(reinterpret_cast<PipelineFunc *>(fun[0]));
+            funcs.emplace_back(FusedPipelineBody<VT>(built->program));
             VectorizedPipeline<DT>::apply(outputs, numOutputs, isScalar, inputs, numInputs, outRows, outCols,
                                           reinterpret_cast<const VectorSplit *>(splits), reinterpret_cast<const VectorCombine *>(combines),
                                           funcs, ctx);

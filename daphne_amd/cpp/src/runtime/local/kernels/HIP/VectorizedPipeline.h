@@ -1,4 +1,5 @@
-// HIP::VectorizedPipeline: runs a vectorized pipeline entirely on the HIP device.
+// HIP::VectorizedPipeline: runs a vectorized pipeline on the HIP device - all of its rows, or a share of them beside
+// the CPU workers.
 //
 // Same parameters as the reference's kernel (src/runtime/local/kernels/VectorizedPipeline.h:35-69), which hands
 // the pipeline to MTWrapper<DenseMatrix<VT>>::executeQueuePerDeviceType (src/runtime/local/vectorized/
@@ -7,7 +8,9 @@
 // all rows here and takes them in as few launches as possible: the row range is cut into `hip_vect_shares` tasks
 // (default 1) and each task runs in batches of `hip_vect_batch_rows` rows (default 0: the whole task at once).
 // More shares and smaller batches give the same result (that is what the tests check) and are there for results
-// too large for one pass and for callers that combine the device with other workers.
+// too large for one pass. A caller that wants the reference's hybrid execution sets `hip_vect_device_share` below 1:
+// then MTWrapperHIP (runtime/local/vectorized/MTWrapperHIP.h) gives that share of the rows to a device worker and
+// the rest to CPU workers that run the host body, and the results end up in host memory.
 //
 // Outputs are allocated on the device as MTWrapperBase::allocateOutput does on the host
 // (src/runtime/local/vectorized/MTWrapper.h:116-140): ROWS / COLS results uninitialised, aggregating results
@@ -19,6 +22,7 @@
 
 #include <runtime/local/kernels/HIP/Fill.h>
 #include <runtime/local/kernels/HIP/HostUtils.h>
+#include <runtime/local/vectorized/MTWrapperHIP.h>
 #include <runtime/local/vectorized/TasksHIP.h>
 
 #include <functional>
@@ -42,8 +46,12 @@ template <typename VT> struct VectorizedPipeline<DenseMatrix<VT>> {
         if (numFuncs == 0)
             throw std::runtime_error("HIP::vectorizedPipeline: no pipeline body given");
         std::vector<std::function<PipelineFunc>> funcs;
-        for (size_t i = 0; i < numFuncs; ++i)
-            funcs.emplace_back(reinterpret_cast<PipelineFunc *>(fun[i]));
+        for (size_t i = 0; i < numFuncs; ++i) {
+            if (fun[i] != nullptr)
+                funcs.emplace_back(reinterpret_cast<PipelineFunc *>(fun[i]));
+            else
+                funcs.emplace_back(); // no such body: only an error if somebody has to run it
+        }
         apply(outputs, numOutputs, isScalar, inputs, numInputs, outRows, outCols, reinterpret_cast<VectorSplit *>(splits),
               reinterpret_cast<VectorCombine *>(combines), funcs, ctx);
     }
@@ -52,6 +60,13 @@ template <typename VT> struct VectorizedPipeline<DenseMatrix<VT>> {
     static void apply(DT **outputs, size_t numOutputs, const bool *isScalar, Structure **inputs, size_t numInputs,
                       const int64_t *outRows, const int64_t *outCols, const VectorSplit *splits, const VectorCombine *combines,
                       std::vector<std::function<PipelineFunc>> funcs, DCTX(ctx)) {
+        // The reference's division of labour, on request: the device takes hip_vect_device_share of the rows and the
+        // CPU workers run the host body on the others; the results then live in host memory.
+        if (ctx->getUserConfig().hip_vect_device_share < 1.0 && funcs.size() > 1) {
+            MTWrapperHIP<DT>::executeQueuePerDeviceType(std::move(funcs), outputs, numOutputs, isScalar, inputs, numInputs, outRows,
+                                                        outCols, splits, combines, ctx->getUserConfig().hip_vect_device_share, ctx);
+            return;
+        }
         AllocationDescriptorHIP alloc_desc(ctx, detail::deviceID);
         // the number of rows to split: the tallest row-split input (others are broadcast)
         uint64_t len = 0;

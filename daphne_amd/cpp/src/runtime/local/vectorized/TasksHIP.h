@@ -126,16 +126,7 @@ template <typename VT> class CompiledPipelineTaskHIP<DenseMatrix<VT>> : public C
         std::vector<DT *> localAggRes(n, nullptr), localResults(n, nullptr), targets(n, nullptr);
         std::vector<DT **> outputs(n);
         HIP::DeferredChecks verdicts(HIPContext::get(_data._ctx, 0)->raw());
-        for (uint64_t r = _data._rl; r < _data._ru; r += batchSize) {
-            const uint64_t r2 = std::min<uint64_t>(r + batchSize, _data._ru);
-            auto linputs = this->createFuncInputs(r, r2);
-            for (size_t o = 0; o < n; ++o) {
-                targets[o] = targetView(o, r, r2);
-                localResults[o] = targets[o]; // the body may write straight into the result
-                outputs[o] = &localResults[o];
-            }
-            _data._funcs[fid](outputs.data(), linputs.data(), _data._ctx);
-            accumulateOutputs(localResults, localAggRes, targets);
+        auto dropBatch = [&] { // the views into the results and what the body returned for the current batch
             for (size_t o = 0; o < n; ++o) {
                 if (localResults[o] != nullptr && localResults[o] != targets[o])
                     DataObjectFactory::destroy(localResults[o]);
@@ -143,11 +134,25 @@ template <typename VT> class CompiledPipelineTaskHIP<DenseMatrix<VT>> : public C
                     DataObjectFactory::destroy(targets[o]);
                 localResults[o] = targets[o] = nullptr;
             }
-            // The body owns the references to its inputs (views included) and gives them back itself.
-        }
+        };
         try {
+            for (uint64_t r = _data._rl; r < _data._ru; r += batchSize) {
+                const uint64_t r2 = std::min<uint64_t>(r + batchSize, _data._ru);
+                auto linputs = this->createFuncInputs(r, r2);
+                for (size_t o = 0; o < n; ++o) {
+                    targets[o] = targetView(o, r, r2);
+                    localResults[o] = targets[o]; // the body may write straight into the result
+                    outputs[o] = &localResults[o];
+                }
+                _data._funcs[fid](outputs.data(), linputs.data(), _data._ctx);
+                accumulateOutputs(localResults, localAggRes, targets);
+                dropBatch();
+                // The body owns the references to its inputs (views included) and gives them back itself.
+            }
             verdicts.finish(); // before the task's partial aggregates are folded into the shared results
         } catch (...) {
+            // a view holds on to the device buffer it looks into: none may outlive the failure
+            dropBatch();
             for (DT *partial : localAggRes)
                 if (partial != nullptr)
                     DataObjectFactory::destroy(partial);

@@ -36,6 +36,10 @@ struct DaphneUserConfig {
     // (0: all of its rows at once)
     uint64_t hip_vect_shares = 1;
     uint64_t hip_vect_batch_rows = 0;
+    // the share of a pipeline's rows that the device takes; below 1 the CPU workers take the other rows
+    double hip_vect_device_share = 1.0;
+    int numberOfThreads = -1;         // CPU workers of a vectorized pipeline (-1: one per hardware thread)
+    size_t phyBatchSize = 96 * 1024;  // bytes of input and output rows that a CPU worker handles per call of the body
 };
 
 struct KernelDispatchInfo {

@@ -412,6 +412,23 @@ extern "C" dh_status dh_d2d_2d(dh_ctx *ctx, void *dst_dev, size_t dst_pitch, con
     return DH_OK;
 }
 
+extern "C" dh_status dh_d2h_2d(dh_ctx *ctx, void *dst_host, size_t dst_pitch, const void *src_dev, size_t src_pitch,
+                               size_t width_bytes, size_t rows) {
+    DH_REQUIRE_CTX(ctx);
+    if (width_bytes == 0 || rows == 0)
+        return DH_OK;
+    if (dst_pitch < width_bytes || src_pitch < width_bytes)
+        return dh_fail(DH_ERR_INVALID_ARG, "dh_d2h_2d: a pitch (%zu, %zu) is smaller than the row width %zu", dst_pitch,
+                       src_pitch, width_bytes);
+    if (dst_pitch == width_bytes && src_pitch == width_bytes)
+        DH_CHECK_HIP(hipMemcpyAsync(dst_host, src_dev, width_bytes * rows, hipMemcpyDeviceToHost, ctx->stream));
+    else
+        DH_CHECK_HIP(hipMemcpy2DAsync(dst_host, dst_pitch, src_dev, src_pitch, width_bytes, rows, hipMemcpyDeviceToHost,
+                                      ctx->stream));
+    DH_CHECK_HIP(hipStreamSynchronize(ctx->stream));
+    return DH_OK;
+}
+
 extern "C" dh_status dh_timer_start(dh_ctx *ctx) {
     DH_REQUIRE_CTX(ctx);
     DH_CHECK_HIP(hipEventRecord(ctx->ev_start, ctx->stream));

@@ -145,6 +145,12 @@ dh_status dh_d2d(dh_ctx *ctx, void *dst_dev, const void *src_dev, size_t bytes);
  * per share or per row there). */
 dh_status dh_d2d_2d(dh_ctx *ctx, void *dst_dev, size_t dst_pitch, const void *src_dev, size_t src_pitch,
                     size_t width_bytes, size_t rows);
+/* The same from a pitched device buffer into pitched host memory, synchronous like dh_d2h: how the device's share of
+ * a pipeline's result is put into a result in host memory when CPU workers computed the other rows
+ * (MTWrapper<DenseMatrix<VT>>::combineOutputs, runtime/local/vectorized/MTWrapper_dense.cpp:339-373: one cudaMemcpy
+ * for a row share, one per row for a column share). */
+dh_status dh_d2h_2d(dh_ctx *ctx, void *dst_host, size_t dst_pitch, const void *src_dev, size_t src_pitch,
+                    size_t width_bytes, size_t rows);
 
 /* Stream-ordered stopwatch on the context's stream (hipEvent pair). dh_timer_stop_ms
  * synchronises on the stop event and returns the elapsed milliseconds. */

@@ -300,6 +300,14 @@ dh_status dh_d2d_2d(dh_ctx *, void *dst_dev, size_t dst_pitch, const void *src_d
         std::memcpy(static_cast<char *>(dst_dev) + r * dst_pitch, static_cast<const char *>(src_dev) + r * src_pitch, width_bytes);
     return DH_OK;
 }
+dh_status dh_d2h_2d(dh_ctx *ctx, void *dst_host, size_t dst_pitch, const void *src_dev, size_t src_pitch, size_t width_bytes,
+                    size_t rows) {
+    if (rows != 0 && width_bytes != 0 && !inside(ctx, src_dev, (rows - 1) * src_pitch + width_bytes))
+        return fail(DH_ERR_HIP, "dh_d2h_2d: source outside any device allocation");
+    for (size_t r = 0; r < rows; r++)
+        std::memcpy(static_cast<char *>(dst_host) + r * dst_pitch, static_cast<const char *>(src_dev) + r * src_pitch, width_bytes);
+    return DH_OK;
+}
 
 #define MOCK_KERNELS(SUF, T)                                                                                            \
     dh_status dh_ew_binary_##SUF(dh_ctx *, int op, T *res, size_t ld_res, const T *lhs, size_t lr, size_t lc, size_t ld_lhs,      \

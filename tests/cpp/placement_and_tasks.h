@@ -428,3 +428,229 @@ template <typename VT> void run_pipeline_tasks(DaphneContext *dctx) {
     DataObjectFactory::destroy(m1, m2);
 }
 
+
+// ------------------------------------------------------------------------------------------------
+// One pipeline shared between the device and CPU workers
+// (MTWrapper_dense.cpp:203-336 executeQueuePerDeviceType, 339-373 combineOutputs; WorkerGPU.h:22-52)
+// ------------------------------------------------------------------------------------------------
+// the host body of funStats: the same four results by loops in host memory, as fresh matrices
+template <class DT> void hostStats(DT ***outputs, Structure **inputs, DCTX(ctx)) {
+    using VT = typename DT::VT;
+    auto *x = static_cast<DT *>(inputs[0]), *mu = static_cast<DT *>(inputs[1]);
+    const size_t n = x->getNumRows(), c = x->getNumCols();
+    const VT *xv = static_cast<const DT *>(x)->getValues(), *mv = static_cast<const DT *>(mu)->getValues();
+    auto *sq = DataObjectFactory::create<DT>(n, c, false), *sum = DataObjectFactory::create<DT>(1, c, false);
+    auto *mn = DataObjectFactory::create<DT>(1, c, false), *mx = DataObjectFactory::create<DT>(1, c, false);
+    for (size_t j = 0; j < c; j++) {
+        sum->getValues()[j] = VT(0);
+        mn->getValues()[j] = std::numeric_limits<VT>::infinity();
+        mx->getValues()[j] = -std::numeric_limits<VT>::infinity();
+    }
+    for (size_t i = 0; i < n; i++)
+        for (size_t j = 0; j < c; j++) {
+            const VT v = xv[i * x->getRowSkip() + j], d = v - mv[j];
+            sq->getValues()[i * c + j] = d * d;
+            sum->getValues()[j] += v;
+            mn->getValues()[j] = std::min(mn->getValues()[j], v);
+            mx->getValues()[j] = std::max(mx->getValues()[j], v);
+        }
+    *outputs[0] = sq;
+    *outputs[1] = sum;
+    *outputs[2] = mn;
+    *outputs[3] = mx;
+    DataObjectFactory::destroy(x, mu);
+}
+// the host body of the z-score pipeline (funZscoreOpByOp): r by ROWS, the count of r > thr by ADD
+template <class DT> void hostZscore(DT ***outputs, Structure **inputs, DCTX(ctx)) {
+    using VT = typename DT::VT;
+    auto *x = static_cast<DT *>(inputs[0]), *mu = static_cast<DT *>(inputs[1]), *sd = static_cast<DT *>(inputs[2]);
+    const VT thr = HIP::FusedPipelineBody<VT>::scalarOf(inputs[3]);
+    const size_t n = x->getNumRows(), c = x->getNumCols();
+    const VT *xv = static_cast<const DT *>(x)->getValues(), *mv = static_cast<const DT *>(mu)->getValues(),
+             *sv = static_cast<const DT *>(sd)->getValues();
+    auto *r = DataObjectFactory::create<DT>(n, 1, false), *count = DataObjectFactory::create<DT>(1, 1, true);
+    for (size_t i = 0; i < n; i++) {
+        VT acc = VT(0);
+        for (size_t j = 0; j < c; j++) {
+            const VT z = (xv[i * x->getRowSkip() + j] - mv[j]) / sv[j];
+            acc += z * z;
+        }
+        r->getValues()[i] = acc;
+        count->getValues()[0] += acc > thr ? VT(1) : VT(0);
+    }
+    *outputs[0] = r;
+    *outputs[1] = count;
+    DataObjectFactory::destroy(x, mu, sd);
+}
+// a device body that fails after it has given its inputs back
+template <class DT> void funFails(DT ***, Structure **inputs, DCTX(ctx)) {
+    DataObjectFactory::destroy(static_cast<DT *>(inputs[0]), static_cast<DT *>(inputs[1]));
+    throw std::domain_error("the device body failed");
+}
+
+template <typename VT> void run_hybrid_pipeline(DaphneContext *dctx) {
+    using DT = DenseMatrix<VT>;
+    using Fn = void (*)(DT ***, Structure **, DCTX(ctx));
+    HIPContext *hc = HIPContext::get(dctx, 0);
+    const size_t rows = 1234, cols = 10;
+    std::vector<VT> a(rows * cols);
+    uint32_t s = 777u;
+    for (auto &v : a) {
+        s = s * 1664525u + 1013904223u;
+        v = VT((s >> 8) * (1.0 / 16777216.0));
+    }
+    auto m1 = given<DT>(rows, a);
+    // the whole matrix on the device, operator by operator: what every division of the rows has to give
+    DT *mu = nullptr, *c = nullptr, *sq = nullptr, *sum = nullptr, *mn = nullptr, *mx = nullptr;
+    HIP::aggCol(AggOpCode::MEAN, mu, m1, dctx); // lives on the device only: the CPU workers need it brought home
+    HIP::ewBinaryMat(BinaryOpCode::SUB, c, m1, mu, dctx);
+    HIP::ewBinaryMat(BinaryOpCode::MUL, sq, c, c, dctx);
+    HIP::aggCol(AggOpCode::SUM, sum, m1, dctx);
+    HIP::aggCol(AggOpCode::MIN, mn, m1, dctx);
+    HIP::aggCol(AggOpCode::MAX, mx, m1, dctx);
+    const auto sq_want = toHost(sq), sum_want = toHost(sum), mn_want = toHost(mn), mx_want = toHost(mx);
+    const size_t allocs0 = hc->numAllocations();
+
+    bool isScalar[] = {false, false};
+    Structure *inputs[] = {m1, mu};
+    int64_t outRows[] = {int64_t(rows), 1, 1, 1}, outCols[] = {int64_t(cols), int64_t(cols), int64_t(cols), int64_t(cols)};
+    int64_t splits[] = {int64_t(VectorSplit::ROWS), int64_t(VectorSplit::NONE)};
+    int64_t combines[] = {int64_t(VectorCombine::ROWS), int64_t(VectorCombine::ADD), int64_t(VectorCombine::MIN),
+                          int64_t(VectorCombine::MAX)};
+    void *fun[] = {reinterpret_cast<void *>(Fn(&hostStats<DT>)), reinterpret_cast<void *>(Fn(&funStats<DT>))}; // {host, device}
+    const double tol = std::is_same<VT, float>::value ? 1e-4 : 1e-12; // sums of 1234 values in [0,1) in another order
+    struct Case {
+        double share;
+        uint64_t shares, batch;
+        int threads;
+        size_t phyBatch;
+    };
+    // a quarter as the reference fixes it; one row; all but one row; nothing at all for the device
+    const Case cases[] = {{0.25, 1, 0, 3, 96 * 1024}, {0.25, 3, 100, 1, 4096}, {0.5, 2, 0, 8, 1024},
+                          {0.0005, 1, 0, 2, 96 * 1024}, {0.9995, 7, 50, 4, 96 * 1024}, {0.0, 1, 0, 2, 2048}};
+    for (const Case &cs : cases) {
+        dctx->config.hip_vect_device_share = cs.share;
+        dctx->config.hip_vect_shares = cs.shares;
+        dctx->config.hip_vect_batch_rows = cs.batch;
+        dctx->config.numberOfThreads = cs.threads;
+        dctx->config.phyBatchSize = cs.phyBatch;
+        DT *out[] = {nullptr, nullptr, nullptr, nullptr};
+        HIP::vectorizedPipeline<DT>(out, 4, isScalar, inputs, 2, outRows, outCols, splits, combines, 2, fun, dctx);
+        CHECK(out[0] != nullptr && out[0]->getNumRows() == rows && out[0]->getNumCols() == cols);
+        CHECK(whereIs(out[0]) == 1); // combined in host memory
+        CHECK(toHost(out[0]) == sq_want); // ROWS: the same IEEE operations per element on either side
+        const auto got = toHost(out[1]);
+        bool ok = got.size() == sum_want.size();
+        for (size_t i = 0; ok && i < got.size(); i++)
+            ok = std::fabs(double(got[i]) - double(sum_want[i])) <= tol * std::fabs(double(sum_want[i]));
+        CHECK(ok);
+        CHECK(toHost(out[2]) == mn_want);
+        CHECK(toHost(out[3]) == mx_want);
+        DataObjectFactory::destroy(out[0], out[1], out[2], out[3]);
+        CHECK(m1->getRefCounter() == 1 && mu->getRefCounter() == 1);
+    }
+    // a result that the caller brings along, wider than what the pipeline fills: the other columns stay
+    {
+        dctx->config.hip_vect_device_share = 0.3;
+        dctx->config.hip_vect_shares = 2;
+        dctx->config.hip_vect_batch_rows = 0;
+        dctx->config.numberOfThreads = 3;
+        auto *wide = DataObjectFactory::create<DT>(rows, cols + 3, false);
+        std::fill(wide->getValues(), wide->getValues() + rows * (cols + 3), VT(-7));
+        DT *out[] = {wide->sliceCol(0, cols), nullptr, nullptr, nullptr};
+        HIP::vectorizedPipeline<DT>(out, 4, isScalar, inputs, 2, outRows, outCols, splits, combines, 2, fun, dctx);
+        const VT *w = static_cast<const DT *>(wide)->getValues();
+        bool ok = true;
+        for (size_t i = 0; i < rows; i++)
+            for (size_t j = 0; j < cols + 3; j++)
+                ok &= w[i * (cols + 3) + j] == (j < cols ? sq_want[i * cols + j] : VT(-7));
+        CHECK(ok);
+        DataObjectFactory::destroy(out[0], out[1], out[2], out[3], wide);
+    }
+    // the device's share as ONE kernel per batch (the body's operators as text beside the outlined bodies)
+    {
+        DT *var = nullptr, *sd = nullptr;
+        HIP::aggCol(AggOpCode::VAR, var, m1, dctx);
+        HIP::ewUnaryMat(UnaryOpCode::SQRT, sd, var, dctx);
+        const double thr = 10.0;
+        Structure *thrDisguised;
+        std::memcpy(&thrDisguised, &thr, sizeof(thr));
+        bool isScalar4[] = {false, false, false, true};
+        Structure *inputs4[] = {m1, mu, sd, thrDisguised};
+        int64_t outRows4[] = {int64_t(rows), 1}, outCols4[] = {1, 1};
+        int64_t splits4[] = {int64_t(VectorSplit::ROWS), int64_t(VectorSplit::NONE), int64_t(VectorSplit::NONE), int64_t(VectorSplit::NONE)};
+        int64_t combines4[] = {int64_t(VectorCombine::ROWS), int64_t(VectorCombine::ADD)};
+        void *fun4[] = {reinterpret_cast<void *>(Fn(&hostZscore<DT>)), reinterpret_cast<void *>(Fn(&funZscoreOpByOp<DT>))};
+        dctx->config.hip_vect_device_share = 1.0;
+        dctx->config.hip_vect_shares = 1;
+        dctx->config.hip_vect_batch_rows = 0;
+        DT *ref[] = {nullptr, nullptr};
+        HIP::fusedPipeline<DT>(ref, 2, isScalar4, inputs4, 4, outRows4, outCols4, splits4, combines4, 2, fun4, kZscoreBody, dctx);
+        CHECK(HIP::fusedPipelineLastMode() == 1 && whereIs(ref[0]) == 2);
+        const auto r_ref = toHost(ref[0]);
+        const VT count_ref = toHost(ref[1])[0];
+        const double rtol = std::is_same<VT, float>::value ? 1e-5 : 1e-13;
+        size_t ambiguous = 0;
+        for (VT v : r_ref)
+            ambiguous += std::fabs(double(v) - thr) <= rtol * thr;
+        for (double share : {0.25, 0.7}) {
+            dctx->config.hip_vect_device_share = share;
+            dctx->config.hip_vect_shares = 2;
+            dctx->config.hip_vect_batch_rows = 128;
+            dctx->config.numberOfThreads = 4;
+            DT *out[] = {nullptr, nullptr};
+            HIP::fusedPipeline<DT>(out, 2, isScalar4, inputs4, 4, outRows4, outCols4, splits4, combines4, 2, fun4, kZscoreBody, dctx);
+            CHECK(HIP::fusedPipelineLastMode() == 1 && whereIs(out[0]) == 1);
+            const auto got = toHost(out[0]);
+            bool ok = got.size() == r_ref.size();
+            for (size_t i = 0; ok && i < got.size(); i++)
+                ok = std::fabs(double(got[i]) - double(r_ref[i])) <= rtol * std::fabs(double(r_ref[i]));
+            CHECK(ok);
+            CHECK(std::fabs(double(toHost(out[1])[0]) - double(count_ref)) <= double(ambiguous));
+            DataObjectFactory::destroy(out[0], out[1]);
+        }
+        // no host body, and rows left for the CPU: refused before any worker starts
+        {
+            void *none[] = {nullptr, reinterpret_cast<void *>(Fn(&funZscoreOpByOp<DT>))};
+            DT *out[] = {nullptr, nullptr};
+            bool thrown = false;
+            try {
+                HIP::fusedPipeline<DT>(out, 2, isScalar4, inputs4, 4, outRows4, outCols4, splits4, combines4, 2, none, nullptr, dctx);
+            } catch (const std::runtime_error &e) {
+                thrown = std::string(e.what()).find("no host body") != std::string::npos;
+            }
+            CHECK(thrown);
+            for (DT *o : out)
+                if (o != nullptr)
+                    DataObjectFactory::destroy(o);
+        }
+        CHECK(sd->getRefCounter() == 1);
+        DataObjectFactory::destroy(ref[0], ref[1], var, sd);
+    }
+    // a device task that throws: the exception reaches the caller once every worker has finished, nothing is left behind
+    {
+        void *bad[] = {reinterpret_cast<void *>(Fn(&hostStats<DT>)), reinterpret_cast<void *>(Fn(&funFails<DT>))};
+        dctx->config.hip_vect_device_share = 0.25;
+        dctx->config.hip_vect_shares = 3;
+        DT *out[] = {nullptr, nullptr, nullptr, nullptr};
+        bool thrown = false;
+        try {
+            HIP::vectorizedPipeline<DT>(out, 4, isScalar, inputs, 2, outRows, outCols, splits, combines, 2, bad, dctx);
+        } catch (const std::domain_error &e) {
+            thrown = std::string(e.what()) == "the device body failed";
+        }
+        CHECK(thrown);
+        for (DT *o : out)
+            if (o != nullptr)
+                DataObjectFactory::destroy(o);
+        CHECK(m1->getRefCounter() == 1 && mu->getRefCounter() == 1);
+    }
+    CHECK(hc->numAllocations() == allocs0); // the device's views and results are gone
+    dctx->config.hip_vect_device_share = 1.0;
+    dctx->config.hip_vect_shares = 1;
+    dctx->config.hip_vect_batch_rows = 0;
+    dctx->config.numberOfThreads = -1;
+    dctx->config.phyBatchSize = 96 * 1024;
+    DataObjectFactory::destroy(m1, mu, c, sq, sum);
+    DataObjectFactory::destroy(mn, mx);
+}

@@ -360,6 +360,62 @@ static void funDivSi64(DenseMatrix<int64_t> ***outputs, Structure **inputs, DCTX
 
 // Kernels that validate their arguments on the device, called batch after batch by a pipeline task: no batch waits
 // for its verdict, and the task's execute() still throws what the failing kernel would have thrown.
+// COLS on a pipeline shared with the CPU workers: a batch of rows becomes a batch of columns (t(x)); the device's
+// columns come home with one pitched copy (MTWrapper_dense.cpp:355-368 copies them row by row)
+template <class DT> void funTranspose(DT ***outputs, Structure **inputs, DCTX(ctx)) {
+    auto *x = static_cast<DT *>(inputs[0]);
+    HIP::transpose(*outputs[0], x, ctx);
+    DataObjectFactory::destroy(x);
+}
+template <class DT> void hostTranspose(DT ***outputs, Structure **inputs, DCTX(ctx)) {
+    auto *x = static_cast<DT *>(inputs[0]);
+    const size_t n = x->getNumRows(), c = x->getNumCols();
+    const auto *xv = static_cast<const DT *>(x)->getValues();
+    auto *t = DataObjectFactory::create<DT>(c, n, false);
+    for (size_t i = 0; i < n; i++)
+        for (size_t j = 0; j < c; j++)
+            t->getValues()[j * n + i] = xv[i * x->getRowSkip() + j];
+    *outputs[0] = t;
+    DataObjectFactory::destroy(x);
+}
+template <typename VT> void run_hybrid_cols(DaphneContext *dctx) {
+    using DT = DenseMatrix<VT>;
+    using Fn = void (*)(DT ***, Structure **, DCTX(ctx));
+    const size_t rows = 777, cols = 6;
+    std::vector<VT> a(rows * cols);
+    for (size_t i = 0; i < a.size(); i++)
+        a[i] = VT(i % 1000) * VT(0.5);
+    auto *x = given<DT>(rows, a);
+    std::vector<VT> want(rows * cols);
+    for (size_t i = 0; i < rows; i++)
+        for (size_t j = 0; j < cols; j++)
+            want[j * rows + i] = a[i * cols + j];
+    bool isScalar[] = {false};
+    Structure *inputs[] = {x};
+    int64_t outRows[] = {int64_t(cols)}, outCols[] = {int64_t(rows)};
+    int64_t splits[] = {int64_t(VectorSplit::ROWS)}, combines[] = {int64_t(VectorCombine::COLS)};
+    void *fun[] = {reinterpret_cast<void *>(Fn(&hostTranspose<DT>)), reinterpret_cast<void *>(Fn(&funTranspose<DT>))};
+    for (double share : {0.25, 0.6, 1.0}) {
+        dctx->config.hip_vect_device_share = share;
+        dctx->config.hip_vect_shares = 2;
+        dctx->config.hip_vect_batch_rows = 64;
+        dctx->config.numberOfThreads = 3;
+        dctx->config.phyBatchSize = 2048;
+        DT *out[] = {nullptr};
+        HIP::vectorizedPipeline<DT>(out, 1, isScalar, inputs, 1, outRows, outCols, splits, combines, 2, fun, dctx);
+        CHECK(whereIs(out[0]) == (share < 1.0 ? 1 : 2));
+        CHECK(toHost(out[0]) == want);
+        DataObjectFactory::destroy(out[0]);
+    }
+    dctx->config.hip_vect_device_share = 1.0;
+    dctx->config.hip_vect_shares = 1;
+    dctx->config.hip_vect_batch_rows = 0;
+    dctx->config.numberOfThreads = -1;
+    dctx->config.phyBatchSize = 96 * 1024;
+    CHECK(x->getRefCounter() == 1);
+    DataObjectFactory::destroy(x);
+}
+
 static void run_deferred_verdicts(DaphneContext *dctx) {
     using DT = DenseMatrix<int64_t>;
     dh_ctx *raw = HIPContext::get(dctx, 0)->raw();
@@ -623,6 +679,10 @@ int main(int argc, char **argv) {
     run_placement(dctx.get());
     run_pipeline_tasks<float>(dctx.get());
     run_pipeline_tasks<double>(dctx.get());
+    run_hybrid_pipeline<float>(dctx.get());
+    run_hybrid_pipeline<double>(dctx.get());
+    run_hybrid_cols<float>(dctx.get());
+    run_hybrid_cols<double>(dctx.get());
     run_deferred_verdicts(dctx.get());
     if (argc > 1) // path of libHIPKernels.so
         run_generated_wrappers(dctx.get(), argv[1]);

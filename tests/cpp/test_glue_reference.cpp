@@ -32,6 +32,8 @@ int main() {
     run_placement(dctx.get());
     run_pipeline_tasks<float>(dctx.get());
     run_pipeline_tasks<double>(dctx.get());
+    run_hybrid_pipeline<float>(dctx.get());
+    run_hybrid_pipeline<double>(dctx.get());
     std::printf("%s: %d checks, %d failed\n", g_fail ? "FAILED" : "PASSED", g_checks, g_fail);
     return g_fail ? 1 : 0;
 }

@@ -100,3 +100,30 @@ def test_two_host_threads_share_one_context():
     c.sync()
     assert c.memInUse() == 0
     c.destroy()
+
+
+def test_pitched_copies_between_device_and_host():
+    """dh_d2d_2d and dh_d2h_2d move `rows` pieces of `width` bytes between buffers with their own row pitches: a
+    pipeline's row or column share on its way into the whole result (TasksCUDA.cpp:73-100, MTWrapper_dense.cpp:339-373)."""
+    c = HIPContext(0)
+    lib = capi.lib()
+    rows, width, sp, dp, hp = 37, 24, 40, 56, 64
+    src = np.arange(rows * sp, dtype=np.uint8)
+    d_src, d_dst = c.malloc(src.nbytes), c.malloc(rows * dp, zero=True)
+    capi.check(lib.dh_h2d(c._h, d_src, src.ctypes.data, src.nbytes))
+    capi.check(lib.dh_d2d_2d(c._h, d_dst, dp, d_src, sp, width, rows))
+    host = np.full(rows * hp, 255, dtype=np.uint8)
+    capi.check(lib.dh_d2h_2d(c._h, host.ctypes.data, hp, d_dst, dp, width, rows))
+    want = np.full((rows, hp), 255, dtype=np.uint8)
+    want[:, :width] = src.reshape(rows, sp)[:, :width]
+    np.testing.assert_array_equal(host.reshape(rows, hp), want)
+    tight = np.empty(rows * width, dtype=np.uint8)  # both pitches equal to the width: one plain copy
+    packed = c.malloc(rows * width)
+    capi.check(lib.dh_d2d_2d(c._h, packed, width, d_src, sp, width, rows))
+    capi.check(lib.dh_d2h_2d(c._h, tight.ctypes.data, width, packed, width, width, rows))
+    np.testing.assert_array_equal(tight.reshape(rows, width), want[:, :width])
+    with pytest.raises(DaphneHipError):
+        capi.check(lib.dh_d2h_2d(c._h, host.ctypes.data, width - 1, d_dst, dp, width, rows))
+    for p in (d_src, d_dst, packed):
+        c.free(p)
+    c.destroy()
