@@ -54,22 +54,36 @@ template <typename T>
 __global__ __launch_bounds__(256) void conv_prep_kernel(int *tab, T *wpack, const T *filter, unsigned F, unsigned Fpad,
                                                         unsigned K, unsigned Kpad, unsigned HpWp, unsigned Wp,
                                                         unsigned Hf, unsigned Wf, unsigned stage_channels = ~0u,
-                                                        unsigned scale = 1) {
+                                                        unsigned scale = 1, unsigned pixel_stride = 0) {
     // stage_channels: offsets count from the first channel of the LDS stage a channel belongs to (all channels in one
-    // stage by default); scale: 1 for offsets in elements, sizeof(T) for offsets in bytes
+    // stage by default); scale: 1 for offsets in elements, sizeof(T) for offsets in bytes.
+    // pixel_stride != 0: the LDS stage holds its channels interleaved - element (y, x, c) at (y Wp + x) pixel_stride + c -
+    // and k runs through a stage's taps with the stage's channels innermost: k = stage KG + tap stage_channels + c
+    // (the channel count is a multiple of stage_channels), so that consecutive k are consecutive addresses.
     const unsigned t = blockIdx.x * 256 + threadIdx.x, nt = gridDim.x * 256;
+    const unsigned HfWf = Hf * Wf, KG = stage_channels * HfWf; // KG only used with pixel_stride != 0
     for (unsigned k = t; k < Kpad; k += nt) {
         int off = 0;
         if (k < K) {
-            const unsigned c = k / (Hf * Wf), hw = k % (Hf * Wf);
-            off = static_cast<int>(((c % stage_channels) * HpWp + (hw / Wf) * Wp + hw % Wf) * scale);
+            if (pixel_stride != 0) {
+                const unsigned kk = k % KG, tap = kk / stage_channels, c = kk % stage_channels;
+                off = static_cast<int>((((tap / Wf) * Wp + tap % Wf) * pixel_stride + c) * scale);
+            } else {
+                const unsigned c = k / HfWf, hw = k % HfWf;
+                off = static_cast<int>(((c % stage_channels) * HpWp + (hw / Wf) * Wp + hw % Wf) * scale);
+            }
         }
         tab[k] = off;
     }
     const size_t total = static_cast<size_t>(Fpad) * Kpad;
     for (size_t i = t; i < total; i += nt) {
         const unsigned f = static_cast<unsigned>(i / Kpad), k = static_cast<unsigned>(i % Kpad);
-        wpack[i] = (f < F && k < K) ? filter[static_cast<size_t>(f) * K + k] : T(0);
+        unsigned src = k;
+        if (pixel_stride != 0 && k < K) {
+            const unsigned stage = k / KG, kk = k % KG;
+            src = (stage * stage_channels + kk % stage_channels) * HfWf + kk / stage_channels;
+        }
+        wpack[i] = (f < F && k < K) ? filter[static_cast<size_t>(f) * K + src] : T(0);
     }
 }
 
@@ -329,6 +343,7 @@ struct ConvResidentArgs {
     unsigned N, NI;    // images in all, images per workgroup (their pixels form one pixel range)
     unsigned relu;     // 1: max(0, .) after the bias
     unsigned Qo, PQo;  // POOL: width and size of the pooled output plane (PQ, Q stay those of the convolution)
+    unsigned lds_bias; // byte offset of the workgroup's bias values in LDS (behind the image stage)
 };
 
 // Copies one image (C x H x W at x) into LDS as C x Hp x Wp with the zero border of Padding.h:11-22 written out,
@@ -388,22 +403,67 @@ __device__ __forceinline__ void conv_stage_frame(T *frame, const T *x, unsigned 
     }
 }
 
+// The same with the channels interleaved: element (y, x, c) of the padded image at (y Wp + x) PS + c, PS = C + one
+// vector. A thread takes VEC consecutive channels of one position: its loads are coalesced per channel plane
+// (consecutive lanes, consecutive positions) and its one vector store lands PS elements from its neighbour's - with the
+// odd vector of padding in PS, the 16 lanes that LDS serves together reach all banks.
+template <typename T, int UB>
+__device__ __forceinline__ void conv_stage_frame_interleaved(T *frame, const T *x, unsigned C, unsigned H, unsigned W, unsigned Wp,
+                                                             unsigned ph, unsigned pw, unsigned HpWp, unsigned PS, int tid,
+                                                             unsigned nt) {
+    constexpr int VEC = 16 / sizeof(T);
+    const unsigned HW = H * W, total = HpWp * (C / VEC);
+    for (unsigned e0 = tid; e0 < total; e0 += nt * UB) {
+        T v[UB][VEC];
+        unsigned dst[UB];
+        bool in[UB];
+#pragma unroll
+        for (int u = 0; u < UB; u++) {
+            const unsigned e = e0 + u * nt < total ? e0 + u * nt : e0;
+            const unsigned cv = e / HpWp, r = e % HpWp;
+            const unsigned y = r / Wp - ph, xx = r % Wp - pw; // wraps to a huge value inside the border
+            in[u] = y < H && xx < W;
+            const unsigned src = (in[u] ? y * W + xx : 0) + cv * VEC * HW;
+            dst[u] = r * PS + cv * VEC;
+#pragma unroll
+            for (int q = 0; q < VEC; q++)
+                v[u][q] = __builtin_nontemporal_load(x + (src + q * HW));
+        }
+#pragma unroll
+        for (int u = 0; u < UB; u++) {
+            if (e0 + u * nt < total) {
+                if (!in[u]) {
+#pragma unroll
+                    for (int q = 0; q < VEC; q++)
+                        v[u][q] = T(0);
+                }
+                dh_store_vec<T, VEC>(frame + dst[u], v[u]);
+            }
+        }
+    }
+}
+
 // POOL: the result is the 2 x 2 / stride 2 maximum of the (biased, optionally rectified) convolution, as maxPoolForward
 // computes it (running maximum from zero over the window in row order, Pooling.cpp:77-105). The pixel index that
 // workgroups and waves divide among themselves then counts window positions, four to a pooled pixel, so that a
 // window's values end up in four neighbouring lanes.
-template <typename T, int MFW, int NF, bool POOL>
-__global__ __launch_bounds__(512) void conv2d_resident_kernel(ConvResidentArgs g) {
+// CI: the LDS image holds its channels interleaved (conv_stage_frame_interleaved; the stage's channel count is a
+// multiple of 4 VEC, and k runs taps-outer / channels-inner, see conv_prep_kernel): the VEC values of k that a lane
+// feeds into VEC consecutive matrix instructions are consecutive channels at one tap, one 16-byte LDS read.
+template <typename T, int MFW, int NF, bool POOL, bool CI = false>
+__global__ __launch_bounds__(512, (CI && NF <= 7) ? 4 : 1) void conv2d_resident_kernel(ConvResidentArgs g) {
     using M = dh_gemm::Mfma16<T>;
     constexpr int VEC = 16 / sizeof(T), NPARTS = 8 / MFW;
     extern __shared__ __attribute__((aligned(16))) unsigned char conv_lds[];
     int *ktab = reinterpret_cast<int *>(conv_lds);               // Kpad entries: a multiple of 16 bytes
     T *frame = reinterpret_cast<T *>(conv_lds + g.Kpad * sizeof(int));
+    T *bias_l = reinterpret_cast<T *>(conv_lds + g.lds_bias); // the workgroup's 16 MFW bias values, behind the image
     const int tid = threadIdx.x, lane = tid % 64, wave = __builtin_amdgcn_readfirstlane(tid / 64);
     const unsigned img = blockIdx.x * g.NI, f0 = blockIdx.y * (16 * MFW), px0 = blockIdx.z * g.chunk;
     const unsigned nimg = (g.N - img < g.NI) ? g.N - img : g.NI; // images of this workgroup
     const unsigned PQv = POOL ? 4 * g.PQo : g.PQ, PQout = POOL ? g.PQo : g.PQ; // "pixels" and results per image
-    const unsigned npix = nimg * PQv, stage_elems = g.CG * g.HpWp;
+    const unsigned PS = CI ? g.CG + VEC : 1;                     // CI: elements from a position to the next
+    const unsigned npix = nimg * PQv, stage_elems = CI ? g.HpWp * PS : g.CG * g.HpWp;
 
     // the offset table: its first 2048 entries are asked for now and put into LDS after the first image stage has
     // been copied in, so that both sets of loads are on their way together
@@ -435,7 +495,7 @@ __global__ __launch_bounds__(512) void conv2d_resident_kernel(ConvResidentArgs g
             pp = pq / g.Q;
             qq = pq % g.Q;
         }
-        pixoff[j] = static_cast<int>(il * stage_elems + pp * g.sh * g.Wp + qq * g.sw);
+        pixoff[j] = static_cast<int>(il * stage_elems + (pp * g.sh * g.Wp + qq * g.sw) * PS);
         outoff[j] = ok ? static_cast<int>(il * g.F * PQout + po) : -1;
         if (first < npix)
             nfv = j + 1;
@@ -516,6 +576,46 @@ __global__ __launch_bounds__(512) void conv2d_resident_kernel(ConvResidentArgs g
         if (k0 < k_end)
             kblock(nv_tag, a0, kt0, a1, kt1, b_even, b_odd, k0);
     };
+    // CI: a block's patch values are one vector read per pixel block, asked for right after the matrix instructions
+    // that used the previous block's vector in the same registers: per VEC matrix instructions one read and one
+    // address addition (measured on a loop of nothing else: 87 % of the pipe's peak against 78 % with a 4-byte read
+    // and an addition per instruction).
+    typedef T patch_t __attribute__((ext_vector_type(VEC)));
+    auto contract_ci = [&](auto nv_tag, unsigned k_begin, unsigned k_end) {
+        constexpr int NV = decltype(nv_tag)::value;
+        constexpr unsigned KB = 4 * VEC;
+        T a0[VEC], a1[VEC];
+        patch_t b[NF];
+        dh_load_vec<T, VEC>(wrow + k_begin, a0);
+        {
+            const int kt = ktl[k_begin];
+#pragma unroll
+            for (int j = 0; j < NV; j++)
+                b[j] = *reinterpret_cast<const patch_t *>(frame_b + (pixoff[j] + kt));
+        }
+        auto block = [&](T(&a_c)[VEC], T(&a_n)[VEC], unsigned kn) {
+            dh_load_vec<T, VEC>(wrow + kn, a_n);
+            const int kt_n = ktl[kn];
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int j = 0; j < NV; j++) {
+#pragma unroll
+                for (int s_ = 0; s_ < VEC; s_++)
+                    acc[j] = M::mma(a_c[s_], b[j][s_], acc[j]);
+                __builtin_amdgcn_sched_barrier(0);
+                b[j] = *reinterpret_cast<const patch_t *>(frame_b + (pixoff[j] + kt_n));
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        };
+        unsigned k0 = k_begin;
+        for (; k0 + 2 * KB <= k_end; k0 += 2 * KB) {
+            const unsigned kn = (k0 + 2 * KB < k_end) ? k0 + 2 * KB : k0; // the last turn fetches a block of its own again
+            block(a0, a1, k0 + KB);
+            block(a1, a0, kn);
+        }
+        if (k0 < k_end)
+            block(a0, a1, k0);
+    };
     // The image goes through LDS in stages of CG channels (all of them when they fit); the accumulators stay.
     const T *ximg = static_cast<const T *>(g.x) + static_cast<size_t>(img) * g.C * g.H * g.W;
     for (unsigned c0 = 0, k_begin = 0; c0 < g.C; c0 += g.CG, k_begin += g.KG) {
@@ -523,9 +623,13 @@ __global__ __launch_bounds__(512) void conv2d_resident_kernel(ConvResidentArgs g
         const unsigned k_end = (c0 + g.CG < g.C) ? k_begin + g.KG : g.Kpad;
         if (c0)
             __syncthreads(); // every wave is done with the previous stage
-        for (unsigned il = 0; il < nimg; il++)
-            conv_stage_frame<T, 8>(frame + il * stage_elems, ximg + (static_cast<size_t>(il) * g.C + c0) * g.H * g.W, cg, g.H, g.W,
-                                g.Wp, g.ph, g.pw, g.HpWp, cg * g.HpWp, tid, 512);
+        for (unsigned il = 0; il < nimg; il++) {
+            const T *xs = ximg + (static_cast<size_t>(il) * g.C + c0) * g.H * g.W;
+            if constexpr (CI)
+                conv_stage_frame_interleaved<T, 6>(frame + il * stage_elems, xs, cg, g.H, g.W, g.Wp, g.ph, g.pw, g.HpWp, PS, tid, 512);
+            else
+                conv_stage_frame<T, 8>(frame + il * stage_elems, xs, cg, g.H, g.W, g.Wp, g.ph, g.pw, g.HpWp, cg * g.HpWp, tid, 512);
+        }
         if (c0 == 0) {
 #pragma unroll
             for (int i = 0; i < KTR; i++)
@@ -533,22 +637,32 @@ __global__ __launch_bounds__(512) void conv2d_resident_kernel(ConvResidentArgs g
                     ktab[tid + i * 512] = ktreg[i];
             for (unsigned k = tid + KTR * 512; k < g.Kpad; k += 512)
                 ktab[k] = g.ktab[k];
+            // the bias comes in with the image: the epilogue, which a wave reaches with nothing else to do, then waits
+            // for an LDS read instead of a trip to memory
+            if (tid < 16 * MFW) {
+                const T *bias = static_cast<const T *>(g.bias);
+                bias_l[tid] = (bias && f0 + tid < g.F) ? bias[f0 + tid] : T(0);
+            }
         }
         __syncthreads();
-        if (nfv == NF - 1)
-            contract(std::integral_constant<int, NF - 1>{}, k_begin, k_end);
-        else if (nfv > 0)
-            contract(std::integral_constant<int, NF>{}, k_begin, k_end);
+        if constexpr (CI) {
+            if (nfv == NF - 1)
+                contract_ci(std::integral_constant<int, NF - 1>{}, k_begin, k_end);
+            else if (nfv > 0)
+                contract_ci(std::integral_constant<int, NF>{}, k_begin, k_end);
+        } else {
+            if (nfv == NF - 1)
+                contract(std::integral_constant<int, NF - 1>{}, k_begin, k_end);
+            else if (nfv > 0)
+                contract(std::integral_constant<int, NF>{}, k_begin, k_end);
+        }
     }
 
     T *out = static_cast<T *>(g.res) + static_cast<size_t>(img) * g.F * PQout;
-    const T *bias = static_cast<const T *>(g.bias);
     T bv[4];
 #pragma unroll
-    for (int v = 0; v < 4; v++) {
-        const unsigned f = f0 + mf * 16 + M::row(lane, v);
-        bv[v] = (bias && f < g.F) ? bias[f] : T(0);
-    }
+    for (int v = 0; v < 4; v++)
+        bv[v] = bias_l[mf * 16 + M::row(lane, v)];
     if constexpr (POOL) {
 #pragma unroll
         for (int j = 0; j < NF; j++) {
@@ -587,14 +701,14 @@ __global__ __launch_bounds__(512) void conv2d_resident_kernel(ConvResidentArgs g
     }
 }
 
-template <typename T, int MFW, int NF, bool POOL = false>
+template <typename T, int MFW, int NF, bool POOL = false, bool CI = false>
 static inline dh_status conv2d_resident_launch(dh_ctx *ctx, const ConvResidentArgs &g, dim3 grid, size_t lds) {
     // dynamic LDS beyond 64 KiB has to be asked for, per kernel and device (the call is cheap next to the kernel)
     if (lds > 65536) {
-        DH_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&conv2d_resident_kernel<T, MFW, NF, POOL>),
+        DH_CHECK_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&conv2d_resident_kernel<T, MFW, NF, POOL, CI>),
                                          hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
     }
-    hipLaunchKernelGGL((conv2d_resident_kernel<T, MFW, NF, POOL>), grid, dim3(512), lds, ctx->stream, g);
+    hipLaunchKernelGGL((conv2d_resident_kernel<T, MFW, NF, POOL, CI>), grid, dim3(512), lds, ctx->stream, g);
     DH_CHECK_LAUNCH();
     return DH_OK;
 }
@@ -798,12 +912,26 @@ dh_status conv2d_forward(dh_ctx *ctx, T *res, size_t *res_h, size_t *res_w, cons
         while (cg == 0 && ni > 1)
             cg = channels_per_stage(--ni);
         const size_t blocks16 = dh_ceil_div(ni * P * Q, 16);
-        const size_t lds = kpad * sizeof(int) + ni * cg * plane_bytes;
+        size_t lds = kpad * sizeof(int) + ni * cg * plane_bytes;
         const size_t fgroups = dh_ceil_div(F, static_cast<size_t>(16 * mfw));
         const size_t chunks = dh_ceil_div(blocks16, parts * 13);            // at most 13 blocks per wave
         const size_t nf = dh_ceil_div(blocks16, parts * chunks);            // spread evenly over the chunks
         const size_t chunk = parts * nf * 16;
         const size_t igroups = dh_ceil_div(N, ni);
+        // Channels interleaved in LDS (one vector read per VEC matrix instructions): the stage's channels must come in
+        // whole groups of 4 VEC, every stage must have the same number, and the wider image (a vector of padding per
+        // position) must not cost a workgroup per CU.
+        constexpr size_t vec = 16 / sizeof(T);
+        bool ci = cg != 0 && cg % (4 * vec) == 0 && C % cg == 0 && mfw > 1;
+        if (ci) {
+            const size_t lds_ci = kpad * sizeof(int) + ni * Hp * Wp * (cg + vec) * sizeof(T);
+            if (lds_ci > 150 * 1024 || (lds <= 80 * 1024 && lds_ci > 80 * 1024) || (lds <= 52 * 1024 && lds_ci > 53 * 1024))
+                ci = false;
+            else
+                lds = lds_ci;
+        }
+        const size_t lds_bias = lds; // a whole number of elements: the table is whole K blocks of ints
+        lds += 16 * mfw * sizeof(T);
         // One workgroup per CU (more than 80 KiB of LDS) has nothing to cover its loading phase and its LDS
         // latencies with: taken only when a wave has at least six blocks of matrix instructions per step.
         // With K < 32 (one or two K blocks) the output stores dominate, and the tiled kernel below writes longer
@@ -829,7 +957,7 @@ dh_status conv2d_forward(dh_ctx *ctx, T *res, size_t *res_h, size_t *res_w, cons
                                filter, static_cast<unsigned>(F), static_cast<unsigned>(fpad), static_cast<unsigned>(K),
                                static_cast<unsigned>(kpad), static_cast<unsigned>(Hp * Wp), static_cast<unsigned>(Wp),
                                static_cast<unsigned>(Hf), static_cast<unsigned>(Wf), static_cast<unsigned>(cg),
-                               static_cast<unsigned>(sizeof(T)));
+                               static_cast<unsigned>(sizeof(T)), static_cast<unsigned>(ci ? cg + vec : 0));
             DH_CHECK_LAUNCH();
             ConvResidentArgs r{};
             r.x = data;
@@ -857,6 +985,7 @@ dh_status conv2d_forward(dh_ctx *ctx, T *res, size_t *res_h, size_t *res_w, cons
             r.PQ = static_cast<unsigned>(P * Q);
             r.chunk = static_cast<unsigned>(chunk);
             r.relu = relu;
+            r.lds_bias = static_cast<unsigned>(lds_bias);
             r.Qo = static_cast<unsigned>(Qo);
             r.PQo = static_cast<unsigned>(Po * Qo);
             if (pool) {
@@ -871,6 +1000,14 @@ dh_status conv2d_forward(dh_ctx *ctx, T *res, size_t *res_h, size_t *res_w, cons
              : (np <= 7 ? conv2d_resident_launch<T, MFW_, 7, true>(ctx, r, pgrid, lds)             \
                         : (np <= 10 ? conv2d_resident_launch<T, MFW_, 10, true>(ctx, r, pgrid, lds) \
                                     : conv2d_resident_launch<T, MFW_, 13, true>(ctx, r, pgrid, lds))))
+#define DH_CONV_POOL_CI(MFW_)                                                                      \
+    (np <= 4 ? conv2d_resident_launch<T, MFW_, 4, true, true>(ctx, r, pgrid, lds)                  \
+             : (np <= 7 ? conv2d_resident_launch<T, MFW_, 7, true, true>(ctx, r, pgrid, lds)       \
+                        : (np <= 10 ? conv2d_resident_launch<T, MFW_, 10, true, true>(ctx, r, pgrid, lds) \
+                                    : conv2d_resident_launch<T, MFW_, 13, true, true>(ctx, r, pgrid, lds))))
+                if (ci)
+                    return mfw == 2 ? DH_CONV_POOL_CI(2) : DH_CONV_POOL_CI(4);
+#undef DH_CONV_POOL_CI
                 return mfw == 1 ? DH_CONV_POOL(1) : (mfw == 2 ? DH_CONV_POOL(2) : DH_CONV_POOL(4));
 #undef DH_CONV_POOL
             }
@@ -880,6 +1017,14 @@ dh_status conv2d_forward(dh_ctx *ctx, T *res, size_t *res_h, size_t *res_w, cons
              : (nf <= 7 ? conv2d_resident_launch<T, MFW_, 7>(ctx, r, grid, lds)                    \
                         : (nf <= 10 ? conv2d_resident_launch<T, MFW_, 10>(ctx, r, grid, lds)       \
                                     : conv2d_resident_launch<T, MFW_, 13>(ctx, r, grid, lds))))
+#define DH_CONV_RES_CI(MFW_)                                                                       \
+    (nf <= 4 ? conv2d_resident_launch<T, MFW_, 4, false, true>(ctx, r, grid, lds)                  \
+             : (nf <= 7 ? conv2d_resident_launch<T, MFW_, 7, false, true>(ctx, r, grid, lds)       \
+                        : (nf <= 10 ? conv2d_resident_launch<T, MFW_, 10, false, true>(ctx, r, grid, lds) \
+                                    : conv2d_resident_launch<T, MFW_, 13, false, true>(ctx, r, grid, lds))))
+            if (ci)
+                return mfw == 2 ? DH_CONV_RES_CI(2) : DH_CONV_RES_CI(4);
+#undef DH_CONV_RES_CI
             return mfw == 1 ? DH_CONV_RES(1) : (mfw == 2 ? DH_CONV_RES(2) : DH_CONV_RES(4));
 #undef DH_CONV_RES
         }

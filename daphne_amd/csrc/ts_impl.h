@@ -414,7 +414,12 @@ __global__ __launch_bounds__(256, UPDATE ? (NB == 1 ? 3 : 2) : 1) void ts_nt_ker
     // float: the operands of the matrix instruction are exchanged, which transposes the result tile in the
     // registers (row = 4 * (lane / 16) + v becomes the column) and turns four 4-byte stores per lane into one of
     // 16 bytes; the double layout (row = 4 * v + lane / 16) already stores whole 128-byte rows
-    constexpr bool SWAP = sizeof(T) == 4;
+    // ASSIGN in double exchanges them as well: nothing is stored there, and a row whose 16 values sit in four lanes
+    // (column 4 v + h in register v) finds its minimum with two exchanges between lanes where the sixteen lanes of
+    // the plain layout need four - for each of the lane's four rows
+    constexpr bool SWAP = sizeof(T) == 4 || ASSIGN;
+    // the column, within a block of 16, of register v in lane group h of the exchanged layout
+    auto swapped_col = [](int hh, int vv) { return sizeof(T) == 4 ? 4 * hh + vv : 4 * vv + hh; };
     extern __shared__ __attribute__((aligned(16))) unsigned char ts_nt_lds[];
     T *lb = reinterpret_cast<T *>(ts_nt_lds); // [NB*16][kpad + V], zero padded
     const int tid = threadIdx.x, lane = tid % 64;
@@ -432,7 +437,7 @@ __global__ __launch_bounds__(256, UPDATE ? (NB == 1 ? 3 : 2) : 1) void ts_nt_ker
         for (int b = 0; b < NB; b++)
 #pragma unroll
             for (int v = 0; v < CPL; v++) {
-                const unsigned col = SWAP ? b * 16 + 4 * h + v : b * 16 + i;
+                const unsigned col = SWAP ? b * 16 + swapped_col(h, v) : b * 16 + i;
                 col_add[b][v] = col < g.n ? static_cast<const T *>(g.col_add)[col] : dh_inf<T>(); // beyond n: never the minimum
             }
     }
@@ -595,8 +600,9 @@ __global__ __launch_bounds__(256, UPDATE ? (NB == 1 ? 3 : 2) : 1) void ts_nt_ker
                 best = better ? ov : best;
                 bi = better ? oi : bi;
             };
-            if constexpr (SWAP) {
-                // register v of lane (i, h) is C[row i][column 16 b + 4 h + v]: a row's values sit in the four lanes i + 16 h
+            static_assert(SWAP, "the arg-min epilogue reads the exchanged layout");
+            {
+                // register v of lane (i, h) is C[row i][column 16 b + 4 h + v] (double: 4 v + h): a row's values sit in the four lanes i + 16 h
                 T d[2][NB][4];
 #pragma unroll
                 for (int t = 0; t < 2; t++)
@@ -621,7 +627,7 @@ __global__ __launch_bounds__(256, UPDATE ? (NB == 1 ? 3 : 2) : 1) void ts_nt_ker
                         for (int v = 0; v < 4; v++) {
                             const bool lt = d[t][b][v] < best;
                             best = lt ? d[t][b][v] : best;
-                            at = lt ? static_cast<unsigned>(b * 16 + 4 * h + v) : at;
+                            at = lt ? static_cast<unsigned>(b * 16 + swapped_col(h, v)) : at;
                         }
                     take(best, at, dh_peer_swap<16>{}(best), dh_peer_swap<16>{}(at));
                     take(best, at, dh_peer_swap<32>{}(best), dh_peer_swap<32>{}(at));
@@ -659,30 +665,6 @@ __global__ __launch_bounds__(256, UPDATE ? (NB == 1 ? 3 : 2) : 1) void ts_nt_ker
                     else
                         add_rows(std::false_type{});
                 }
-            } else {
-                // register v of lane (i, h) is C[row 4 v + h][column 16 b + i]: a row's values sit in the sixteen lanes of a group
-#pragma unroll
-                for (int t = 0; t < 2; t++)
-#pragma unroll
-                    for (int v = 0; v < 4; v++) {
-                        const size_t row = rbase + static_cast<size_t>(t) * 16 + M::row(lane, v);
-                        const T ra = radd[t][SWAP ? 0 : v];
-                        T best = dh_inf<T>(), first = T(0);
-                        unsigned bi = NONE;
-#pragma unroll
-                        for (int b = 0; b < NB; b++) {
-                            const unsigned col = b * 16 + i;
-                            const T d = (acc[t][b][v] * T(-2) + ra) + col_add[b][0];
-                            if (b == 0)
-                                first = d; // column 0 in the lanes i = 0
-                            const bool lt = d < best; // columns beyond n carry +inf
-                            best = lt ? d : best;
-                            bi = lt ? col : bi;
-                        }
-                        dh_butterfly(16, [&](auto peer) { take(best, bi, peer(best), peer(bi)); });
-                        if (i == 0 && row < g.M)
-                            g.idx[row] = ((first != first) || bi == NONE) ? 0ull : static_cast<unsigned long long>(bi);
-                    }
             }
         } else if constexpr (SWAP) {
             // the tile was computed transposed: register v of lane (i, h) is C[row i][column 4h + v], so a lane
@@ -998,6 +980,13 @@ template <typename T, int NB, int CPG = 4> inline dh_status ts_nt_update_launch(
 
 template <typename T, int NB, bool ASSIGN> inline dh_status ts_nt_launch(dh_ctx *ctx, const TsNtArgs &g) {
     const int cpg = ts_nt_chunks_per_step<T>(g.kpad);
+    // 64 doubles a row, product stored: all eight chunks in one step, which takes the loop that finishes a pair beside
+    // the matrix instructions of the next (10M x 64 by 16: 1240 -> 1090 us, at one wave per SIMD instead of two). The
+    // arg-min form loses by it (1060 -> 1250 us, with or without that loop).
+    if constexpr (sizeof(T) == 8 && NB == 1 && !ASSIGN) {
+        if (g.kpad == 64)
+            return ts_nt_launch_cpg<T, NB, ASSIGN, 8>(ctx, g, ts_nt_lds_bytes<T>(NB, g.kpad, 8));
+    }
     const size_t lds = ts_nt_lds_bytes<T>(NB, g.kpad, cpg);
     return cpg == 4 ? ts_nt_launch_cpg<T, NB, ASSIGN, 4>(ctx, g, lds)
                     : (cpg == 2 ? ts_nt_launch_cpg<T, NB, ASSIGN, 2>(ctx, g, lds) : ts_nt_launch_cpg<T, NB, ASSIGN, 1>(ctx, g, lds));
