@@ -44,6 +44,12 @@ CONV_CASES = [  # N, C, H, W, F, Hf, Wf, sh, sw, ph, pw
     (9, 16, 7, 7, 32, 3, 3, 1, 1, 1, 1),
     (20, 8, 4, 4, 64, 3, 3, 1, 1, 1, 1),
     (7, 64, 14, 14, 32, 5, 5, 1, 1, 0, 0),
+    # channels in whole groups of 16 (8 in double): the LDS image with its channels interleaved - strides, a partial
+    # filter block, three stages of 16 channels, 24 channels (interleaved in double only), odd planes
+    (6, 16, 15, 13, 20, 3, 3, 2, 2, 1, 1),
+    (2, 48, 12, 12, 40, 3, 3, 1, 2, 0, 1),
+    (4, 24, 10, 10, 33, 3, 3, 1, 1, 1, 1),
+    (5, 32, 9, 11, 64, 2, 4, 1, 1, 1, 0),
     # fewer than 32 filter taps: 33 filters (a partial filter block) and
     # uneven strides, 17 filters with wide padding, 31 taps in a column, more than 256 pixels per image
     (3, 1, 19, 23, 33, 3, 5, 2, 3, 1, 2),
