@@ -355,10 +355,18 @@ dh_status step(dh_ctx *ctx, unsigned long long *idx, T *Cn, size_t ldcn, T *coun
     DH_REQUIRE_CTX(ctx);
     if (Cn == nullptr || (rows > 0 && (idx == nullptr || X == nullptr || C == nullptr || xx == nullptr || cc == nullptr)))
         return dh_fail(DH_ERR_INVALID_ARG, "kmeans step: idx, C_new, X, C, xx and cc must not be null");
-    if constexpr (sizeof(T) == 4) {
-        constexpr int V = 4, KC = 16;
-        const size_t kpad = dh_ceil_div(cols, KC) * KC;
-        if (rows > 0 && k >= 1 && k <= 32 && kpad <= 64 && dh_aligned(X, 16) && dh_aligned(C, 16) && ldx % V == 0 && ldc % V == 0 &&
+    {
+        // One pass: up to 64 columns (a lane per column when the rows are added up). Float: the columns are one step
+        // of 1 .. 4 chunks of 16. Double: chunks of 8 - up to four of them one step, five to eight two steps of four
+        // (the rows of both stay staged until the pair's assignment is known).
+        constexpr int V = 16 / sizeof(T), KC = 4 * V;
+        size_t kpad = dh_ceil_div(cols, KC) * KC;
+        if (sizeof(T) == 8 && kpad > 4 * KC && kpad <= 64)
+            kpad = 64;
+        const size_t chunks_per_step = kpad / KC <= 4 ? kpad / KC : 4;
+        // (32 sums of doubles per lane do not fit the registers of two waves per SIMD: up to 16 centroids in double)
+        constexpr size_t max_k = sizeof(T) == 4 ? 32 : 16;
+        if (rows > 0 && k >= 1 && k <= max_k && kpad <= 64 && dh_aligned(X, 16) && dh_aligned(C, 16) && ldx % V == 0 && ldc % V == 0 &&
             cols % V == 0 && ldx >= cols && ldc >= cols && ldcn >= cols && ldx * sizeof(T) < (size_t(1) << 24)) {
             const int nb = k <= 16 ? 1 : 2;
             TsNtArgs g{};
@@ -375,14 +383,15 @@ dh_status step(dh_ctx *ctx, unsigned long long *idx, T *Cn, size_t ldcn, T *coun
             g.idx = idx;
             size_t blocks = 0;
             // with g.slabs == nullptr: how many partial results; then the launch
+            constexpr int NB2 = sizeof(T) == 4 ? 2 : 1; // double: nb is always 1
             auto launch = [&]() -> dh_status {
-                if (kpad == 64)
-                    return nb == 1 ? dh_gemm::ts_nt_update_launch<T, 1, 4>(ctx, g, &blocks) : dh_gemm::ts_nt_update_launch<T, 2, 4>(ctx, g, &blocks);
-                if (kpad == 48)
-                    return nb == 1 ? dh_gemm::ts_nt_update_launch<T, 1, 3>(ctx, g, &blocks) : dh_gemm::ts_nt_update_launch<T, 2, 3>(ctx, g, &blocks);
-                if (kpad == 32)
-                    return nb == 1 ? dh_gemm::ts_nt_update_launch<T, 1, 2>(ctx, g, &blocks) : dh_gemm::ts_nt_update_launch<T, 2, 2>(ctx, g, &blocks);
-                return nb == 1 ? dh_gemm::ts_nt_update_launch<T, 1, 1>(ctx, g, &blocks) : dh_gemm::ts_nt_update_launch<T, 2, 1>(ctx, g, &blocks);
+                if (chunks_per_step == 4)
+                    return nb == 1 ? dh_gemm::ts_nt_update_launch<T, 1, 4>(ctx, g, &blocks) : dh_gemm::ts_nt_update_launch<T, NB2, 4>(ctx, g, &blocks);
+                if (chunks_per_step == 3)
+                    return nb == 1 ? dh_gemm::ts_nt_update_launch<T, 1, 3>(ctx, g, &blocks) : dh_gemm::ts_nt_update_launch<T, NB2, 3>(ctx, g, &blocks);
+                if (chunks_per_step == 2)
+                    return nb == 1 ? dh_gemm::ts_nt_update_launch<T, 1, 2>(ctx, g, &blocks) : dh_gemm::ts_nt_update_launch<T, NB2, 2>(ctx, g, &blocks);
+                return nb == 1 ? dh_gemm::ts_nt_update_launch<T, 1, 1>(ctx, g, &blocks) : dh_gemm::ts_nt_update_launch<T, NB2, 1>(ctx, g, &blocks);
             };
             dh_status st = launch();
             if (st != DH_OK)

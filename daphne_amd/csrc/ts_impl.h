@@ -406,8 +406,8 @@ struct TsNtArgs {
 // sums and the counts. The grid is what the device holds at once (one partial result per workgroup) and deals the
 // pairs round-robin.
 template <typename T, int NB, bool ASSIGN, int CPG, bool UPDATE = false>
-__global__ __launch_bounds__(256, UPDATE ? (NB == 1 ? 3 : 2) : 1) void ts_nt_kernel(TsNtArgs g) {
-    static_assert(!UPDATE || (ASSIGN && sizeof(T) == 4), "the one-pass form exists for float, K of CPG whole chunks (a lane per column)");
+__global__ __launch_bounds__(256, UPDATE ? ((NB == 1 && sizeof(T) == 4) ? 3 : 2) : 1) void ts_nt_kernel(TsNtArgs g) {
+    static_assert(!UPDATE || ASSIGN, "the one-pass form goes on from the assignment");
     using M = Mfma16<T>;
     constexpr int V = 16 / sizeof(T);
     constexpr int KC = 4 * V;     // k values per chunk
@@ -453,8 +453,9 @@ __global__ __launch_bounds__(256, UPDATE ? (NB == 1 ? 3 : 2) : 1) void ts_nt_ker
     // against a grid of resident workgroups that deal the pairs round-robin, this is as fast at 2M rows and 7 % faster
     // at 20M).
     const unsigned chunks = g.kpad / KC;
-    // chunk groups per row-block pair (CPG divides chunks); the one-pass form only exists for a single group
-    const unsigned cg = UPDATE ? 1u : chunks / CPG;
+    // chunk groups per row-block pair (CPG divides chunks); the one-pass form keeps the staged rows of all of a pair's
+    // groups (at most 64 columns, a lane per column)
+    const unsigned cg = chunks / CPG;
     const size_t total_pairs = (g.M + 31) / 32;
     const size_t first_pair = (static_cast<size_t>(blockIdx.x) * 4 + wave) * (UPDATE ? 1 : TS_NT_PAIRS);
     const size_t pair_stride = UPDATE ? static_cast<size_t>(gridDim.x) * 4 : 1;
@@ -477,9 +478,9 @@ __global__ __launch_bounds__(256, UPDATE ? (NB == 1 ? 3 : 2) : 1) void ts_nt_ker
     // no barrier, the wave's own LDS instructions execute in order. Row stride SX = CPG KC + V: free of bank conflicts.
     constexpr unsigned VPR = CPG * 4;      // vectors of a row in one step
     constexpr unsigned SX = CPG * KC + V;
-    // one row block at a time; UPDATE: both row blocks of the pair, which stay there until the pair is finished
-    constexpr unsigned STAGE_BLOCKS = UPDATE ? 2 : 1;
-    T *stage = lb + NB * 16 * ldl + wave * (STAGE_BLOCKS * 16 * SX);
+    // one row block at a time; UPDATE: both row blocks of the pair for each of its chunk groups ([group][block][row]),
+    // which stay there until the pair is finished
+    T *stage = lb + NB * 16 * ldl + wave * (UPDATE ? cg * 2 * 16 * SX : 16 * SX);
     // Addresses are a base that is the same for the whole wave - the pair's first row - plus a 32-bit byte offset per
     // lane (32 rows of at most 2^24 bytes): one 24-bit multiplication and an addition per load, rows beyond M cut
     // back to the last row by a minimum on the row number.
@@ -533,7 +534,7 @@ __global__ __launch_bounds__(256, UPDATE ? (NB == 1 ? 3 : 2) : 1) void ts_nt_ker
         T xa[2][CPG][V];
 #pragma unroll
         for (int t = 0; t < 2; t++) {
-            T *st = stage + (UPDATE ? t * 16 * SX : 0);
+            T *st = stage + (UPDATE ? (grp * 2 + t) * 16 * SX : 0);
 #pragma unroll
             for (int c = 0; c < CPG; c++) {
                 // vector 64 c + lane of the block: row (64 c + lane) / VPR; with 16 vectors a row that is row 4 c + h,
@@ -583,6 +584,10 @@ __global__ __launch_bounds__(256, UPDATE ? (NB == 1 ? 3 : 2) : 1) void ts_nt_ker
     typedef T sums_t __attribute__((ext_vector_type(UPDATE ? NB * 16 : 2)));
     sums_t sums;
     __shared__ unsigned cnts[UPDATE ? 4 * NPOS : 4];
+    // UPDATE: where this lane's column lies in a staged row block (lanes beyond the columns repeat column 0; their
+    // sums are never stored)
+    const unsigned ucol = static_cast<unsigned>(lane) < g.kpad ? lane : 0;
+    const unsigned colbase = (ucol / (CPG * KC)) * (2 * 16 * SX) + ucol % (CPG * KC);
     if constexpr (UPDATE) {
 #pragma unroll
         for (unsigned p = 0; p < NPOS; p++)
@@ -651,9 +656,8 @@ __global__ __launch_bounds__(256, UPDATE ? (NB == 1 ? 3 : 2) : 1) void ts_nt_ker
 #pragma unroll
                             for (int r = 0; r < 16; r++) {
                                 const unsigned pos = static_cast<unsigned>(__builtin_amdgcn_readlane(static_cast<int>(bi[t]), r));
-                                // the row as a row: lane j on column j (lanes beyond the step's columns repeat column 0;
-                                // their sums are never stored)
-                                T x = stage[(t * 16 + r) * SX + (lane < static_cast<int>(CPG * KC) ? lane : 0)];
+                                // the row as a row: lane j on column j
+                                T x = stage[(t * 16 + r) * SX + colbase];
                                 if constexpr (!WHOLE)
                                     x = rbase + t * 16 + r < g.M ? x : T(0); // rows beyond M repeat the last row
                                 sums[pos] += x;
@@ -936,7 +940,8 @@ template <typename T> inline size_t ts_nt_lds_bytes(int nb, unsigned kpad, int c
 // sums (16 nb positions x 64 lanes each) through the same area
 template <typename T> inline size_t ts_nt_update_lds_bytes(int nb, unsigned kpad, int cpg) {
     constexpr size_t V = 16 / sizeof(T), KC = 4 * V;
-    const size_t stage = 4 * 2 * 16 * (static_cast<size_t>(cpg) * KC + V), exchange = 4 * static_cast<size_t>(nb) * 16 * 64;
+    const size_t groups = kpad / (static_cast<size_t>(cpg) * KC);
+    const size_t stage = 4 * groups * 2 * 16 * (static_cast<size_t>(cpg) * KC + V), exchange = 4 * static_cast<size_t>(nb) * 16 * 64;
     return (static_cast<size_t>(nb) * 16 * (kpad + V) + (stage > exchange ? stage : exchange)) * sizeof(T);
 }
 // chunks of k per step: the largest of 4, 2, 1 that divides their number
@@ -965,8 +970,9 @@ template <typename T, int NB, int CPG = 4> inline dh_status ts_nt_update_launch(
     const size_t lds = ts_nt_update_lds_bytes<T>(NB, g.kpad, CPG);
     // three workgroups per CU (measured 2 .. 4 per CU: 104 .. 110 us at 2M x 64, no trend; a loop that only loads the
     // rows this way and stores the assignment takes 86 us, 74 us without the stores)
-    (void)kernel;
-    constexpr int per_cu = 3;
+    if (lds > 65536)
+        DH_CHECK_HIP(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
+    constexpr int per_cu = sizeof(T) == 4 ? 3 : 2; // double: two waves per SIMD by registers, two workgroups per CU by LDS
     size_t blocks = static_cast<size_t>(ctx->num_cus) * per_cu;
     const size_t needed = dh_ceil_div(dh_ceil_div(g.M, 32), 4 * 2); // at least two pairs per wavefront
     if (blocks > needed)

@@ -385,7 +385,7 @@ def kmeansUpdate(C_new, X: DenseMatrix, idx: DenseMatrix, k: int, ctx: HIPContex
 def kmeansStep(idx, C_new, X: DenseMatrix, C: DenseMatrix, xx: DenseMatrix, cc: DenseMatrix, ctx: HIPContext,
                counts: Optional[DenseMatrix] = None):
     """kmeansAssign and kmeansUpdate as one call (dh_kmeans_step_*): one pass over X where the library has a kernel for
-    it (float, up to 64 features), the two passes elsewhere. Returns (idx, C_new, counts)."""
+    it (up to 64 features, in double up to 16 centroids), the two passes elsewhere. Returns (idx, C_new, counts)."""
     dt = _same_dtype(X, C, xx, cc)
     k = C.rows
     if C.cols != X.cols or xx.getNumItems() != X.rows or cc.getNumItems() != k:

@@ -71,7 +71,7 @@ class KMeans:
         self.counts = DenseMatrix(ctx, 1, k, dt)
 
     def iterate(self, C: DenseMatrix, C_out: DenseMatrix | None = None, fused=True) -> DenseMatrix:
-        """fused True: kmeansStep (one pass over X for up to 64 float features, two elsewhere); "two_passes":
+        """fused True: kmeansStep (one pass over X for up to 64 features, two elsewhere); "two_passes":
         kmeansAssign then kmeansUpdate; False: one kernel per operator (or fused pipeline of elementwise operators), with
         XC, the one-hot P and t(P) X in memory. self.idx holds the assignment either way."""
         ctx, X, k = self.ctx, self.X, self.k

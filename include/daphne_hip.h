@@ -312,7 +312,7 @@ dh_status dh_kmeans_update_f64(dh_ctx *ctx, double *C_new, size_t ld_new, double
                                const uint64_t *idx, size_t k);
 
 /* dh_kmeans_assign followed by dh_kmeans_update, in one pass over X where the library has a kernel for
- * it (float, up to 64 features: a row, once loaded, serves the distances and then the sums), as the two
+ * it (up to 64 features, in double up to 16 centroids: a row, once loaded, serves the distances and then the sums), as the two
  * calls one after the other elsewhere. idx as dh_kmeans_assign gives it; C_new and counts as
  * dh_kmeans_update gives them (C_new to rounding: the rows are added in another order). Arguments,
  * limits and errors of the two calls. */

@@ -431,6 +431,7 @@ def test_normal_equations_of_other_shapes(ctx, dt, rows, cols):
 KMEANS_SHAPES = [  # rows, cols, k
     (1, 4, 1), (7, 8, 3), (100, 64, 16), (513, 64, 16), (70_000, 64, 16), (66_000, 32, 32), (65_600, 12, 17), (3000, 200, 5),
     (2049, 128, 20), (131_072, 4, 2), (33, 52, 2), (300_001, 60, 30), (1_000_000, 64, 7), (70_001, 40, 9), (65_537, 36, 20),
+    (70_003, 16, 5), (66_001, 24, 12), (67_000, 28, 16),  # two, three and four chunks of doubles in one step
 ]
 
 
@@ -477,7 +478,7 @@ def test_kmeans_assign_and_update(ctx, dt, rows, cols, k):
             kmeansUpdate(None, X, DenseMatrix.from_numpy(ctx, idx), k, ctx)
         return
     Cn, counts = kmeansUpdate(None, X, DenseMatrix.from_numpy(ctx, idx), k, ctx)
-    # both passes as one call (one pass over X for up to 64 float features): the same assignment and sizes bit for bit
+    # both passes as one call (one pass over X for up to 64 features): the same assignment and sizes bit for bit
     idx1, Cn1, counts1 = kmeansStep(None, None, X, C, xx, cc, ctx)
     assert_exact(idx1.to_numpy(), idx)
     assert_exact(counts1.to_numpy(), counts.to_numpy())
