@@ -166,9 +166,8 @@ def main() -> int:
             cnts = DM(ctx, 1, 16, ndt)
             emit("kmeansUpdate (t(one-hot(idx)) X / sizes), 16 centroids", dt, shape, timed(lambda: K.kmeansUpdate(PtX, X, idxv, 16, ctx, cnts)),
                  nb + rows * 8)
-            if dt == "f32":
-                emit("kmeansStep (assignment and update from one pass over X), C 16x64", dt, shape,
-                     timed(lambda: K.kmeansStep(idxv, PtX, X, Cc, xxv, ccv, ctx, cnts)), nb + rows * sz + rows * 8)
+            emit("kmeansStep (assignment and update from one pass over X), C 16x64", dt, shape,
+                 timed(lambda: K.kmeansStep(idxv, PtX, X, Cc, xxv, ccv, ctx, cnts)), nb + rows * sz + rows * 8)
             for m_ in (xxv, ccv, idxv, cnts):
                 m_.destroy()
         for m in (X, R, colv, r1, ri):
