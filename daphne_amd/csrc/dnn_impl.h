@@ -451,7 +451,7 @@ __device__ __forceinline__ void conv_stage_frame_interleaved(T *frame, const T *
 // multiple of 4 VEC, and k runs taps-outer / channels-inner, see conv_prep_kernel): the VEC values of k that a lane
 // feeds into VEC consecutive matrix instructions are consecutive channels at one tap, one 16-byte LDS read.
 template <typename T, int MFW, int NF, bool POOL, bool CI = false>
-__global__ __launch_bounds__(512, (CI && NF <= 7) ? 4 : 1) void conv2d_resident_kernel(ConvResidentArgs g) {
+__global__ __launch_bounds__(512, (CI && NF <= 7 && sizeof(T) == 4) ? 4 : 1) void conv2d_resident_kernel(ConvResidentArgs g) {
     using M = dh_gemm::Mfma16<T>;
     constexpr int VEC = 16 / sizeof(T), NPARTS = 8 / MFW;
     extern __shared__ __attribute__((aligned(16))) unsigned char conv_lds[];
