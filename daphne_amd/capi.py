@@ -80,6 +80,8 @@ def _signatures(lib: C.CDLL) -> None:
     lib.dh_agg_col_noalloc_scratch_bytes.argtypes = []
     lib.dh_agg_col_noalloc_scratch_bytes.restype = sz
     lib.dh_timer_stop_ms.argtypes = [ctxp, C.POINTER(C.c_float)]
+    lib.dh_kernel_timing.argtypes = [ctxp, i32]
+    lib.dh_kernel_timing_read.argtypes = [ctxp, C.POINTER(C.c_double), C.POINTER(sz)]
     for suf, ct in (("f32", C.c_float), ("f64", C.c_double)):
         f = lambda name: getattr(lib, f"{name}_{suf}")
         f("dh_ew_binary").argtypes = [ctxp, i32, vp, sz, vp, sz, sz, sz, vp, sz, sz, sz]

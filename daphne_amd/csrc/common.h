@@ -11,6 +11,8 @@
 #include <map>
 #include <mutex>
 #include <string>
+#include <utility>
+#include <vector>
 
 #include "../../include/daphne_hip.h"
 
@@ -60,6 +62,10 @@ struct dh_ctx {
     size_t deferred_enqueued = 0; // checked calls since the last dh_check_deferred (none: nothing to wait for)
 
     hipEvent_t ev_start = nullptr, ev_stop = nullptr;
+    // dh_kernel_timing: pairs of events around the dominant kernel of each timed call since the last reading
+    bool kernel_timing = false;
+    std::vector<std::pair<hipEvent_t, hipEvent_t>> kernel_events; // created on demand, reused after a reading
+    size_t kernel_events_used = 0;
     int num_cus = 0;
     // How fused pipeline bodies run on this context: -1 as the environment says (DH_PIPELINE_JIT, default:
     // specialised at run time), 0 interpreted, 1 specialised.
@@ -137,5 +143,37 @@ struct PipeShape {
 };
 bool pipe_shape(size_t cols, int vec, PipeShape *sh);
 } // namespace dh_pipe
+
+// Brackets one kernel launch with a pair of events while dh_kernel_timing is on (nothing otherwise): construct right
+// before the launch, let it go out of scope right after.
+struct DhKernelStopwatch {
+    dh_ctx *ctx;
+    hipEvent_t stop = nullptr;
+    explicit DhKernelStopwatch(dh_ctx *c) : ctx(c) {
+        if (!c->kernel_timing || c->kernel_events_used >= 4096)
+            return;
+        if (c->kernel_events_used == c->kernel_events.size()) {
+            hipEvent_t a = nullptr, b = nullptr;
+            if (hipEventCreate(&a) != hipSuccess)
+                return;
+            if (hipEventCreate(&b) != hipSuccess) {
+                (void)hipEventDestroy(a);
+                return;
+            }
+            c->kernel_events.emplace_back(a, b);
+        }
+        auto &pair = c->kernel_events[c->kernel_events_used];
+        if (hipEventRecord(pair.first, c->stream) != hipSuccess)
+            return;
+        c->kernel_events_used++;
+        stop = pair.second;
+    }
+    ~DhKernelStopwatch() {
+        if (stop)
+            (void)hipEventRecord(stop, ctx->stream);
+    }
+    DhKernelStopwatch(const DhKernelStopwatch &) = delete;
+    DhKernelStopwatch &operator=(const DhKernelStopwatch &) = delete;
+};
 
 #include "dev_common.h"

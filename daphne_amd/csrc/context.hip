@@ -104,6 +104,10 @@ extern "C" dh_status dh_ctx_destroy(dh_ctx *ctx) {
         (void)hipEventDestroy(ctx->ev_start);
     if (ctx->ev_stop)
         (void)hipEventDestroy(ctx->ev_stop);
+    for (auto &pair : ctx->kernel_events) {
+        (void)hipEventDestroy(pair.first);
+        (void)hipEventDestroy(pair.second);
+    }
     delete ctx;
     return DH_OK;
 }
@@ -443,6 +447,32 @@ extern "C" dh_status dh_timer_stop_ms(dh_ctx *ctx, float *ms) {
     DH_CHECK_HIP(hipEventElapsedTime(&t, ctx->ev_start, ctx->ev_stop));
     if (ms)
         *ms = t;
+    return DH_OK;
+}
+
+extern "C" dh_status dh_kernel_timing(dh_ctx *ctx, int on) {
+    DH_REQUIRE_CTX(ctx);
+    ctx->kernel_timing = on != 0;
+    ctx->kernel_events_used = 0;
+    return DH_OK;
+}
+
+extern "C" dh_status dh_kernel_timing_read(dh_ctx *ctx, double *total_ms, size_t *launches) {
+    DH_REQUIRE_CTX(ctx);
+    double total = 0.0;
+    const size_t n = ctx->kernel_events_used;
+    if (n > 0)
+        DH_CHECK_HIP(hipEventSynchronize(ctx->kernel_events[n - 1].second));
+    for (size_t i = 0; i < n; i++) {
+        float t = 0.f;
+        DH_CHECK_HIP(hipEventElapsedTime(&t, ctx->kernel_events[i].first, ctx->kernel_events[i].second));
+        total += t;
+    }
+    ctx->kernel_events_used = 0;
+    if (total_ms)
+        *total_ms = total;
+    if (launches)
+        *launches = n;
     return DH_OK;
 }
 

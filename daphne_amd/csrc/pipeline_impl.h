@@ -223,6 +223,8 @@ dh_status run(dh_ctx *ctx, const dh_pipe_instr *prog, int n, const IO_C *cio, si
         }
     }
     const dim3 g(static_cast<unsigned>(grid)), b(THREADS);
+    {
+    DhKernelStopwatch stopwatch(ctx); // around the body kernel alone (dh_kernel_timing)
     if (use_jit) {
         size_t a_rows = rows, a_cols = cols;
         int a_G = G;
@@ -254,6 +256,7 @@ dh_status run(dh_ctx *ctx, const dh_pipe_instr *prog, int n, const IO_C *cio, si
                 DH_LAUNCH(1, 4);
         }
 #undef DH_LAUNCH
+    }
     }
     DH_CHECK_LAUNCH();
     for (int s = 0; s < 2; s++)

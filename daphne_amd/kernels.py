@@ -119,6 +119,17 @@ class HIPContext:
         capi.check(capi.lib().dh_timer_stop_ms(self._h, C.byref(ms)))
         return ms.value
 
+    def kernel_timing(self, on: bool) -> None:
+        """Switches the stopwatch on single kernels on or off (dh_kernel_timing): while it is on, a fused pipeline
+        records the duration of its body kernel alone."""
+        capi.check(capi.lib().dh_kernel_timing(self._h, 1 if on else 0))
+
+    def kernel_timing_read(self):
+        """(sum of the timed kernels' durations in ms, their number) since the stopwatch was switched on or last read."""
+        total, n = C.c_double(), C.c_size_t()
+        capi.check(capi.lib().dh_kernel_timing_read(self._h, C.byref(total), C.byref(n)))
+        return total.value, n.value
+
     def destroy(self) -> None:
         if self._h:
             capi.lib().dh_ctx_destroy(self._h)

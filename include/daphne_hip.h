@@ -156,6 +156,13 @@ dh_status dh_d2h_2d(dh_ctx *ctx, void *dst_host, size_t dst_pitch, const void *s
  * synchronises on the stop event and returns the elapsed milliseconds. */
 dh_status dh_timer_start(dh_ctx *ctx);
 dh_status dh_timer_stop_ms(dh_ctx *ctx, float *ms);
+/* A stopwatch on single kernels (no counterpart in the reference; for measurement). While it is on, a call whose time
+ * is one dominant kernel beside small ones - dh_vectorized_pipeline_*: the body kernel, without the kernels that fold
+ * its partial results - records a pair of events around that kernel alone, on the context's stream, without waiting.
+ * dh_kernel_timing_read waits for the last of them, returns the sum of the kernels' durations and their number since
+ * the stopwatch was switched on or last read, and starts counting again. At most 4096 kernels are kept per reading. */
+dh_status dh_kernel_timing(dh_ctx *ctx, int on);
+dh_status dh_kernel_timing_read(dh_ctx *ctx, double *total_ms, size_t *launches);
 
 /* ------------------------------------------------------------------------------------ */
 /* elementwise                                                                           */

@@ -292,6 +292,14 @@ dh_status dh_d2h(dh_ctx *ctx, void *dst_host, const void *src_dev, size_t bytes)
     return DH_OK;
 }
 // The mock's kernels have nothing to validate on a device: no verdict is ever pending.
+dh_status dh_kernel_timing(dh_ctx *, int) { return DH_OK; }
+dh_status dh_kernel_timing_read(dh_ctx *, double *total_ms, size_t *launches) {
+    if (total_ms)
+        *total_ms = 0.0;
+    if (launches)
+        *launches = 0;
+    return DH_OK;
+}
 dh_status dh_defer_checks(dh_ctx *, int) { return DH_OK; }
 dh_status dh_check_deferred(dh_ctx *) { return DH_OK; }
 dh_status dh_d2d_2d(dh_ctx *, void *dst_dev, size_t dst_pitch, const void *src_dev, size_t src_pitch, size_t width_bytes,

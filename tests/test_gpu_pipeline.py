@@ -295,3 +295,36 @@ def test_an_evicted_body_is_compiled_again_and_runs(ctx, pipeline_mode):
             assert_exact(out.to_numpy(), np.abs(fns[op](x, np.float32(0.75))))
     finally:
         lib.dh_vectorized_pipeline_set_cache_limit(before)
+
+
+def test_kernel_stopwatch_times_the_body_kernel_alone(ctx):
+    """dh_kernel_timing: a pair of events around the fused pipeline's body kernel per run; the reading sums them, counts
+    them and starts again; nothing is recorded while the stopwatch is off."""
+    from daphne_amd.kernels import AggOpCode, BinaryOpCode, DenseMatrix, aggCol
+    from daphne_amd.pipeline import SELF, VectorizedPipeline
+
+    x = (np.random.default_rng(3).standard_normal((200_000, 32)) + 2).astype(np.float32)
+    X = DenseMatrix.from_numpy(ctx, x)
+    mu = aggCol(AggOpCode.MEAN, None, X, ctx)
+    p = VectorizedPipeline(ctx, X)
+    p.ewBinary(BinaryOpCode.SUB, mu).ewBinary(BinaryOpCode.MUL, SELF)
+    p.rowAgg(AggOpCode.SUM)
+    r = p.storeRow()
+    s = p.reduceAll(AggOpCode.SUM)
+    p.run()
+    assert ctx.kernel_timing_read() == (0.0, 0)
+    ctx.kernel_timing(True)
+    for _ in range(5):
+        p.run()
+    total, n = ctx.kernel_timing_read()
+    assert n == 5 and 0.0 < total < 50.0
+    assert ctx.kernel_timing_read() == (0.0, 0)  # read and reset
+    p.run()
+    total1, n1 = ctx.kernel_timing_read()
+    assert n1 == 1 and 0.0 < total1 < 10.0
+    ctx.kernel_timing(False)
+    p.run()
+    assert ctx.kernel_timing_read() == (0.0, 0)
+    want = ((x - x.mean(0, dtype=np.float64).astype(np.float32)) ** 2).sum(1)
+    np.testing.assert_allclose(r.to_numpy()[:, 0], want, rtol=1e-4)
+    assert abs(float(s.to_numpy()[0, 0]) - float(want.astype(np.float64).sum())) <= 1e-3 * float(want.sum())
