@@ -750,7 +750,9 @@ int dh_ctx_get_pipeline_mode(const dh_ctx *ctx);
 /* Number of specialised bodies this process holds. A body is keyed by its instruction kinds, op codes,
  * operand slots, value type and row width; its immediates are kernel arguments, so a scalar that changes
  * from call to call (a threshold, a learning rate) reuses the compiled kernel. At most 128 bodies stay
- * loaded by default, the least recently used one is unloaded beyond that. */
+ * loaded by default, the least recently used one is unloaded beyond that. Compiled code is also kept on disk
+ * between processes ($DH_PIPELINE_JIT_CACHE, "0" / "off": nowhere; else $XDG_CACHE_HOME/daphne_hip, else
+ * $HOME/.cache/daphne_hip), named by and checked against the compiler's version, the options and the source. */
 size_t dh_vectorized_pipeline_cache_size(void);
 /* Sets how many specialised bodies stay loaded (at least 1) and returns the previous limit. A body that leaves the
  * cache is unloaded once no caller is about to launch it and its device has drained. */

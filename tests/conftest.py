@@ -13,6 +13,19 @@ def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
 
 
+@pytest.fixture(scope="session", autouse=True)
+def pipeline_bodies_cached_in_a_temporary_directory(tmp_path_factory):
+    """Pipeline bodies compiled at run time are kept on disk between processes (pipeline_jit.hip). The tests keep theirs
+    in a directory of their own, so that a run neither leaves files in the user's cache nor finds old ones there."""
+    before = os.environ.get("DH_PIPELINE_JIT_CACHE")
+    os.environ["DH_PIPELINE_JIT_CACHE"] = str(tmp_path_factory.mktemp("pipeline_bodies"))
+    yield
+    if before is None:
+        os.environ.pop("DH_PIPELINE_JIT_CACHE", None)
+    else:
+        os.environ["DH_PIPELINE_JIT_CACHE"] = before
+
+
 def _has_gpu() -> bool:
     try:
         import torch

@@ -328,3 +328,43 @@ def test_kernel_stopwatch_times_the_body_kernel_alone(ctx):
     want = ((x - x.mean(0, dtype=np.float64).astype(np.float32)) ** 2).sum(1)
     np.testing.assert_allclose(r.to_numpy()[:, 0], want, rtol=1e-4)
     assert abs(float(s.to_numpy()[0, 0]) - float(want.astype(np.float64).sum())) <= 1e-3 * float(want.sum())
+
+
+def test_a_body_compiled_by_one_process_runs_from_disk_in_the_next(tmp_path):
+    """The on-disk cache of compiled bodies: the second process loads the first one's code object and gets its bits."""
+    import os
+    import subprocess
+    import sys
+    from pathlib import Path
+
+    ROOT = Path(__file__).resolve().parent.parent
+    script = r"""
+import sys
+import numpy as np
+sys.path.insert(0, %r)
+from daphne_amd import capi
+from daphne_amd.kernels import AggOpCode, BinaryOpCode, DenseMatrix, HIPContext, aggCol
+from daphne_amd.pipeline import SELF, VectorizedPipeline
+ctx = HIPContext(0)
+ctx.set_pipeline_mode(1)
+x = (np.random.default_rng(11).standard_normal((50_000, 24)) * 3 + 1).astype(np.float32)
+X = DenseMatrix.from_numpy(ctx, x)
+mu = aggCol(AggOpCode.MEAN, None, X, ctx)
+p = VectorizedPipeline(ctx, X)
+p.ewBinary(BinaryOpCode.SUB, mu).ewBinary(BinaryOpCode.MUL, SELF)
+p.rowAgg(AggOpCode.SUM)
+r = p.storeRow()
+p.run()
+assert capi.lib().dh_vectorized_pipeline_last_mode() == 1
+np.save(sys.argv[1], r.to_numpy())
+""" % str(ROOT)
+    env = dict(os.environ, DH_PIPELINE_JIT_CACHE=str(tmp_path / "bodies"))
+    for name in ("a.npy", "b.npy"):
+        done = subprocess.run([sys.executable, "-c", script, str(tmp_path / name)], env=env, capture_output=True, text=True, timeout=300)
+        assert done.returncode == 0, done.stdout[-2000:] + done.stderr[-2000:]
+        files = sorted((tmp_path / "bodies").glob("*.bin"))
+        assert len(files) == 1
+        if name == "a.npy":
+            stamp = files[0].stat().st_mtime_ns
+    assert files[0].stat().st_mtime_ns == stamp  # the second process read it and wrote nothing
+    assert_exact(np.load(tmp_path / "a.npy"), np.load(tmp_path / "b.npy"))
