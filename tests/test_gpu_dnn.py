@@ -290,3 +290,34 @@ def test_softmax(ctx, dt, rows, cols):
     st, exp = orc.softmax(x)
     got = softmax(None, DenseMatrix.from_numpy(ctx, x), ctx).to_numpy()
     assert_close(got, exp)
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("seed", range(12))
+def test_conv2d_random_shapes_with_whole_channel_groups(ctx, dt, seed):
+    """Seeded random shapes whose channel counts come in whole groups of 16 (8 in double) - the LDS image with its
+    channels interleaved where it fits, the plane layout or the tiled kernel elsewhere - against the oracle, plain and
+    with ReLU and pooling folded in."""
+    rng = np.random.default_rng(1000 + seed)
+    C = int(rng.choice([8, 16, 24, 32, 48, 64]))
+    Hf, Wf = int(rng.integers(1, 6)), int(rng.integers(1, 6))
+    sh, sw = int(rng.integers(1, 3)), int(rng.integers(1, 3))
+    ph, pw = int(rng.integers(0, (Hf + 1) // 2 + 1)), int(rng.integers(0, (Wf + 1) // 2 + 1))
+    H, W = int(rng.integers(max(Hf, 6), 23)), int(rng.integers(max(Wf, 6), 23))
+    F = int(rng.choice([17, 20, 32, 33, 48, 64, 70]))
+    N = int(rng.integers(1, 12))
+    x = (rng.random((N, C * H * W)) - 0.4).astype(dt)
+    w = (rng.standard_normal((F, C * Hf * Wf)) * np.sqrt(2.0 / (C * Hf * Wf))).astype(dt)
+    b = (rng.standard_normal((F, 1)) * 0.1).astype(dt)
+    st, exp, eh, ew_ = orc.conv2d(x, w, b, N, C, H, W, Hf, Wf, sh, sw, ph, pw)
+    assert st == 0
+    X, Wd, B = DenseMatrix.from_numpy(ctx, x), DenseMatrix.from_numpy(ctx, w), DenseMatrix.from_numpy(ctx, b)
+    got, gh, gw = conv2dForward(None, X, Wd, B, N, C, H, W, Hf, Wf, sh, sw, ph, pw, ctx)
+    assert (gh, gw) == (eh, ew_)
+    assert_close(got.to_numpy(), exp, elementwise=False)
+    if eh >= 2 and ew_ >= 2:
+        fused, fh, fw = conv2dForwardFused(None, X, Wd, B, N, C, H, W, Hf, Wf, sh, sw, ph, pw, ctx, relu=True, pool=True)
+        r = np.maximum(got.to_numpy().reshape(N, F, eh, ew_), 0)
+        want = r[:, :, : eh // 2 * 2, : ew_ // 2 * 2].reshape(N, F, eh // 2, 2, ew_ // 2, 2).max(axis=(3, 5))
+        assert (fh, fw) == (eh // 2, ew_ // 2)
+        assert_exact(fused.to_numpy(), want.reshape(N, -1).astype(dt))  # the epilogue on the same sums: bit for bit
