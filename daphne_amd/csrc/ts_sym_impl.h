@@ -42,7 +42,7 @@ struct TsSymArgs {
     const void *X, *y;
     void *slabs;     // [gridDim.x][m * m + m]: the triangle in matrix layout (row <= col), then the m values of t(X) y
     size_t ldx, ldy, K;
-    size_t k_chunk;  // rows per workgroup, a multiple of 16
+    size_t k_chunk;  // rows per workgroup, a multiple of 4 TS_SYM_DEPTH
     unsigned m;
 };
 
@@ -92,11 +92,10 @@ template <typename T, int NV, int NS> struct TsSymShape {
 // The work of wave W: its quarter of the tile pairs over all rows of the workgroup's chunk.
 //
 // A wave issues its instructions in order, and the waves of a SIMD are served oldest first (measured: a second wave on
-// a SIMD gets the matrix core only when the first has nothing for it), so what counts is how few instructions stand
-// between one group of matrix instructions and the next: one wave per SIMD, the row address in scalar registers
-// (advanced by scalar adds), every load addressed as that scalar base plus a lane offset that never changes, and no
-// work at all on the loaded values. Then 7 matrix instructions of 64 cycles each are followed by some 40 cycles of
-// other work, not 250.
+// a SIMD gets the matrix core only when the first has nothing for it), so what counts is how few instructions a wave
+// issues beside its matrix instructions: one wave per SIMD, the row address in scalar registers (advanced by scalar
+// adds), every load addressed as that scalar base plus a lane offset that never changes, and no work at all on the
+// loaded values.
 template <typename T, int NV, int NS, bool WITH_Y, int W> __device__ __forceinline__ void ts_sym_wave(const TsSymArgs g) {
     using M = Mfma16<T>;
     using S = TsSymShape<T, NV, NS>;
@@ -129,7 +128,7 @@ template <typename T, int NV, int NS, bool WITH_Y, int W> __device__ __forceinli
             const unsigned c = NV * 16 * V + s * 16 + i;
             os[s] = (rowoff + (c < g.m ? c : 0)) * static_cast<unsigned>(sizeof(T));
         }
-        const unsigned oy = static_cast<unsigned>(h) * static_cast<unsigned>(g.ldy) * static_cast<unsigned>(sizeof(T));
+        unsigned oy = static_cast<unsigned>(h) * static_cast<unsigned>(g.ldy) * static_cast<unsigned>(sizeof(T));
 
         typename M::acc_t acc[NPW];
 #pragma unroll
@@ -150,8 +149,18 @@ template <typename T, int NV, int NS, bool WITH_Y, int W> __device__ __forceinli
         // the quad whose first row `row` points at into a register set, only the tiles this wave multiplies; `row`
         // is the same in all lanes and lives in scalar registers
         auto load_quad = [&](Frag &fr, const char *row, const char *yrow) {
-            if constexpr (WITH_Y)
+            // (the empty statements keep the widening of a 32-bit lane offset beside its load, where it becomes part
+            // of the load's addressing - scalar base plus 32-bit lane offset - instead of a 64-bit addition)
+            if constexpr (WITH_Y) {
+                asm volatile("" : "+v"(oy));
                 fr.y = *reinterpret_cast<const T *>(yrow + oy);
+            }
+#pragma unroll
+            for (int a = 0; a < NV; a++)
+                asm volatile("" : "+v"(ov[a]));
+#pragma unroll
+            for (int sc = 0; sc < NS; sc++)
+                asm volatile("" : "+v"(os[sc]));
 #pragma unroll
             for (int a = 0; a < NV; a++) {
                 bool all = true;
@@ -191,44 +200,66 @@ template <typename T, int NV, int NS, bool WITH_Y, int W> __device__ __forceinli
             }
         };
 
-        // D register sets: the loads of D - 1 quads are in flight while one is being multiplied. Loads that would
-        // run past the last whole quad of the chunk repeat that quad (their values are not used). The pointer of the
+        // D register sets: the loads of D - 1 quads are in flight while one is being multiplied. The pointer of the
         // next quad to load advances on the scalar unit.
         constexpr int D = TS_SYM_DEPTH;
-        const unsigned nq = static_cast<unsigned>((ke - kb) / 4); // whole quads
+        const unsigned nfull = static_cast<unsigned>((ke - kb) / (4 * D)) * D; // quads in whole groups of D
         Frag fr[D];
-        if (nq > 0) {
-            const unsigned last = nq - 1;
+        if (nfull > 0) {
             const size_t sx = 4 * g.ldx * sizeof(T), sy = 4 * g.ldy * sizeof(T);
             const char *px = X + kb * g.ldx * sizeof(T), *py = WITH_Y ? Y + kb * g.ldy * sizeof(T) : nullptr;
-            unsigned nl = 0; // quad that px points at
             auto advance = [&]() {
-                const bool more = nl < last;
-                px += more ? sx : 0;
-                py += more ? sy : 0;
-                nl += more ? 1 : 0;
+                px += sx;
+                if constexpr (WITH_Y)
+                    py += sy;
+            };
+            // the matrix instructions of a quad with its other instructions dealt out between them
+            auto spread = [&]() {
+#pragma unroll
+                for (int n = 0; n < NPW; n++) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); // one matrix instruction
+                    __builtin_amdgcn_sched_group_barrier(0x020, 1, 0); // one load
+                    __builtin_amdgcn_sched_group_barrier(0x002, 2, 0); // two vector instructions
+                    __builtin_amdgcn_sched_group_barrier(0x004, 3, 0); // three scalar instructions
+                }
+                __builtin_amdgcn_sched_barrier(0); // a quad's loads stay in its own step
             };
 #pragma unroll
             for (int d = 0; d < D - 1; d++) {
                 load_quad(fr[d], px, py);
                 advance();
             }
-            for (unsigned q = 0; q < nq; q += D) {
+            // All groups of D quads but the last: every step loads the quad D - 1 ahead, which exists, so nothing
+            // is clamped or tested. Measured with the wave's clock around this loop (100 000 x 100 doubles, 100 quads
+            // per workgroup): what an instruction of the same wave costs beside the matrix instructions (64 cycles
+            // each) does not depend on where it stands - some 7 cycles each, dealt out between them or all behind
+            // them -, so their number is what matters.
+            for (unsigned q = D; q < nfull; q += D) {
 #pragma unroll
                 for (int d = 0; d < D; d++) {
                     load_quad(fr[(d + D - 1) % D], px, py);
                     advance();
-                    __builtin_amdgcn_sched_barrier(0);
-                    if (q + d < nq)
-                        mma_quad(fr[d]);
-                    __builtin_amdgcn_sched_barrier(0);
+                    mma_quad(fr[d]);
+                    spread();
                 }
             }
+            // the last group: one quad is still to load
+            load_quad(fr[D - 1], px, py);
+#pragma unroll
+            for (int d = 0; d < D; d++) {
+                mma_quad(fr[d]);
+                spread();
+            }
         }
-        // the rows after the last whole quad (fewer than four, at the very end of X): every lane addresses its own
-        // row here; lane groups without a row read the last one and contribute zeros
-        if (kb + 4 * static_cast<size_t>(nq) < ke) {
-            const size_t r = kb + 4 * static_cast<size_t>(nq) + h;
+        // The rows after the last whole group of quads (fewer than 4 D, in the last workgroup only: the other
+        // workgroups' chunks are whole groups), a quad at a time without the pipeline: every lane addresses its own row
+        // here; lane groups without a row read the last one and contribute zeros
+#pragma unroll
+        for (int j = 0; j < D; j++) {
+            const size_t r0 = kb + 4 * static_cast<size_t>(nfull + j);
+            if (r0 >= ke)
+                break;
+            const size_t r = r0 + h;
             const bool ok = r < ke;
             const size_t rl = ok ? r : ke - 1;
             const char *row = X + (rl * g.ldx - rowoff) * sizeof(T); // the lane offsets include h * ldx
