@@ -3,6 +3,7 @@ directory). Each step runs in a process of its own - inside one process a body i
 the z-score body without a device (dh_vectorized_pipeline_compile_check)."""
 import os
 import subprocess
+import tempfile
 import sys
 from pathlib import Path
 
@@ -30,7 +31,9 @@ def compile_in_a_process(env_changes, cols=64):
     env = dict(os.environ)
     env.pop("DH_PIPELINE_JIT_CACHE", None)
     env.update(env_changes)
-    r = subprocess.run([sys.executable, "-c", SCRIPT, str(cols)], env=env, capture_output=True, text=True, timeout=600)
+    # in a directory of its own: with an empty XDG_CACHE_HOME the compiler library keeps a cache below the working directory
+    with tempfile.TemporaryDirectory() as cwd:
+        r = subprocess.run([sys.executable, "-c", SCRIPT, str(cols)], env=env, cwd=cwd, capture_output=True, text=True, timeout=600)
     assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-2000:]
     return float(r.stdout.split("seconds")[1])
 
