@@ -52,10 +52,11 @@ def _hipcc() -> str:
 
 # The interpreting pipeline kernel rounds every operator of a body by itself, like the run-time specialised one.
 EXTRA_FLAGS = {"pipeline_f32.hip": ["-ffp-contract=off"], "pipeline_f64.hip": ["-ffp-contract=off"]}
-# The symmetric streaming kernel keeps its accumulators in ordinary vector registers: with the matrix instructions in
-# their accumulator-register form the compiler carries them through the loop in vector registers all the same and
-# copies all of them over and back in every iteration.
-for _f in ("ts_sym_f32.hip", "ts_sym_f64.hip"):
+# The symmetric streaming kernel and the widest step of the double `A t(B)` kernel keep their accumulators in ordinary
+# vector registers: with the matrix instructions in their accumulator-register form the compiler carries the former's
+# accumulators through the loop in vector registers all the same and copies all of them over and back in every
+# iteration, and parks the latter's loaded rows in accumulator registers.
+for _f in ("ts_sym_f32.hip", "ts_sym_f64.hip", "ts_nt_wide_f64.hip"):
     EXTRA_FLAGS[_f] = ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]
 
 

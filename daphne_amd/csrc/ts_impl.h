@@ -984,6 +984,11 @@ template <typename T, int NB, int CPG = 4> inline dh_status ts_nt_update_launch(
     return DH_OK;
 }
 
+// ts_nt_kernel<double, 1, false, 8>, launched from a translation unit of its own (ts_nt_wide_f64.hip): the kernel
+// needs more registers than a wave has vector registers, and built with the matrix instructions in their
+// accumulator-register form the compiler parks loaded rows in accumulator registers and copies them back in every step.
+dh_status ts_nt_launch_wide_f64(dh_ctx *ctx, const TsNtArgs &g, size_t lds);
+
 template <typename T, int NB, bool ASSIGN> inline dh_status ts_nt_launch(dh_ctx *ctx, const TsNtArgs &g) {
     const int cpg = ts_nt_chunks_per_step<T>(g.kpad);
     // 64 doubles a row, product stored: all eight chunks in one step, which takes the loop that finishes a pair beside
@@ -991,7 +996,7 @@ template <typename T, int NB, bool ASSIGN> inline dh_status ts_nt_launch(dh_ctx 
     // arg-min form loses by it (1060 -> 1250 us, with or without that loop).
     if constexpr (sizeof(T) == 8 && NB == 1 && !ASSIGN) {
         if (g.kpad == 64)
-            return ts_nt_launch_cpg<T, NB, ASSIGN, 8>(ctx, g, ts_nt_lds_bytes<T>(NB, g.kpad, 8));
+            return ts_nt_launch_wide_f64(ctx, g, ts_nt_lds_bytes<T>(NB, g.kpad, 8));
     }
     const size_t lds = ts_nt_lds_bytes<T>(NB, g.kpad, cpg);
     return cpg == 4 ? ts_nt_launch_cpg<T, NB, ASSIGN, 4>(ctx, g, lds)
